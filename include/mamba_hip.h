@@ -1,0 +1,146 @@
+/*
+ * mamba_hip.h -- C ABI of libmamba_hip.so: the MI355X (gfx950) Mamba inference
+ * hot path.  Plain pointers and sizes only; every device pointer is a HIP
+ * device address, `stream` is a hipStream_t passed as void* (NULL = the null
+ * stream).  All entry points are stream-ordered, never allocate, never
+ * synchronise (unless stated) and return 0 on success or a negative MRS_E_*
+ * code, with a message available from mrs_last_error() on the calling thread.
+ *
+ * Each declaration names the reference interface it replaces
+ * (silvermpx/mamba-rs v0.5.3, paths relative to that repository).  The
+ * reference looks its kernels up by name in one NVRTC module and launches them
+ * with positional raw-pointer/int arguments (src/mamba_ssm/gpu/kernels.rs:547-700);
+ * the argument order of those launch sites is kept, with `stream` and `dtype`
+ * put in front.
+ */
+#ifndef MAMBA_HIP_H
+#define MAMBA_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+/* Exported symbol marker: the library is built with hidden visibility. */
+#define MRS_API __attribute__((visibility("default")))
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Activation storage type.  Values follow the declaration order of the
+ * reference's WeightDtype enum (src/mamba_ssm/gpu/dtype.rs:12-28).  Compute is
+ * always f32; SSM state, conv state, a_neg, D, biases stay f32. */
+typedef enum { MRS_F32 = 0, MRS_F16 = 1, MRS_BF16 = 2 } mrs_dtype;
+
+/* Scan route request, mirrors ScanMode (src/config.rs:6-18). */
+typedef enum { MRS_SCAN_SEQUENTIAL = 0, MRS_SCAN_PARALLEL = 1, MRS_SCAN_AUTO = 2 } mrs_scan_mode;
+
+enum {
+    MRS_OK = 0,
+    MRS_E_NULL = -1,        /* a required pointer is NULL */
+    MRS_E_SHAPE = -2,       /* unsupported or inconsistent shape */
+    MRS_E_DTYPE = -3,       /* dtype not one of mrs_dtype */
+    MRS_E_WORKSPACE = -4,   /* workspace missing or too small */
+    MRS_E_ALIGN = -5,       /* a pointer breaks the stated alignment */
+    MRS_E_HIP = -6          /* the HIP runtime reported an error at launch */
+};
+
+/* Flags for mrs_ssm_scan_fwd_ex. */
+enum {
+    MRS_GATE_NONE = 0,
+    MRS_GATE_PREACT = 1u << 0, /* gate holds silu(z) already: y *= gate (kernels/mamba_ssm.cu:220-222) */
+    MRS_GATE_SILU = 1u << 1,   /* gate holds raw z: y *= z*sigmoid(z) (split_gate_silu + elementwise_mul fused) */
+    MRS_A_S4D_REAL = 1u << 2,  /* caller asserts a_neg[d,n] = (n+1)*a_neg[d,0] to 4 ulp; see mrs_a_neg_is_s4d_real */
+    MRS_FORCE_SEQUENTIAL = 1u << 3, /* ignore the T-split route */
+    MRS_FORCE_PARALLEL = 1u << 4    /* use the T-split route even for short T */
+};
+
+/* Library version (major*10000 + minor*100 + patch) and the last error text of
+ * the calling thread ("" if none). */
+MRS_API int mrs_version(void);
+MRS_API const char *mrs_last_error(void);
+
+/* ScanMode::use_parallel (src/config.rs:28-37): 1 if the parallel route is
+ * chosen for (mode, seq_len, d_state).  d_state > 64 always answers 1. */
+MRS_API int mrs_scan_use_parallel(int mode, int64_t seq_len, int64_t d_state);
+
+/* exp_negate kernel (kernels/elementwise.cu:140-146; called from
+ * src/mamba_ssm/gpu/inference.rs:266-282): a_neg[i] = -exp(a_log[i]), n floats. */
+MRS_API int mrs_exp_negate(void *stream, float *a_neg, const float *a_log, int64_t n);
+
+/* Writes 1 to *flag_out (a device int) if |a_neg[d,n] - (n+1)*a_neg[d,0]| <=
+ * 2^-21 |a_neg[d,n]| (4 ulp) for every d,n -- the S4D-real initialisation
+ * a_log = log(1..=d_state) (src/weights.rs:143-148), whose a_neg = -exp(a_log)
+ * is (n+1) to within an ulp or two -- else 0.  No counterpart in the reference;
+ * it licenses MRS_A_S4D_REAL, under which exp(delta*a_neg[d,n]) is formed as
+ * exp(delta*a_neg[d,0])^(n+1) (relative deviation <= |delta*a_neg| * 5e-7). */
+MRS_API int mrs_a_neg_is_s4d_real(void *stream, int *flag_out, const float *a_neg, int d_inner, int d_state);
+
+/* ---- Mamba-1 selective scan, full sequence --------------------------------
+ * Replaces ssm_parallel_scan_fwd_nosave_{f32,bf16,f16}
+ * (kernels/mamba_ssm_parallel.cu:544-765, 969-1145) and
+ * ssm_burnin_forward_nosave_{..} (kernels/mamba_ssm.cu:304-400); launch sites
+ * src/mamba_ssm/gpu/prefill.rs:512-549, 910-956, argument order
+ * h, y, delta, u, B, C, a_neg, D, batch, T, d_inner, d_state.
+ *   h      [batch, d_inner, d_state] f32, read and overwritten with the final state
+ *   y      [batch, T, d_inner]       dtype
+ *   delta,u[batch, T, d_inner]       dtype (delta after softplus)
+ *   B, C   [batch, T, d_state]       dtype
+ *   a_neg  [d_inner, d_state] f32,  D [d_inner] f32
+ * d_state in 1..=256, T >= 1.  Uses no workspace: always the sequential route. */
+MRS_API int mrs_ssm_scan_fwd(void *stream, int dtype, float *h, void *y, const void *delta, const void *u,
+                     const void *B, const void *C, const float *a_neg, const float *D,
+                     int batch, int T, int d_inner, int d_state);
+
+/* Same scan with the fusions the prefill chain allows:
+ *   bc_stride  row stride (elements) of B and C, so both can point into xdbl
+ *              [batch*T, xdbl_dim] (replaces gather_bc_cols, kernels/elementwise.cu:291-313)
+ *   gate,flags optional gate tensor [batch,T,d_inner] (replaces elementwise_mul,
+ *              src/mamba_ssm/gpu/prefill.rs:957-971)
+ *   workspace  mrs_ssm_scan_workspace_bytes() bytes of device memory, 256-byte
+ *              aligned; NULL forces the sequential route. */
+MRS_API size_t mrs_ssm_scan_workspace_bytes(int batch, int T, int d_inner, int d_state);
+MRS_API int mrs_ssm_scan_fwd_ex(void *stream, int dtype, float *h, void *y, const void *delta, const void *u,
+                        const void *B, const void *C, int64_t bc_stride, const float *a_neg,
+                        const float *D, const void *gate, unsigned flags,
+                        void *workspace, size_t workspace_bytes,
+                        int batch, int T, int d_inner, int d_state);
+
+/* ---- Mamba-1 selective scan, one step (decode) ------------------------------
+ * ssm_step_forward_{..} (kernels/mamba_ssm.cu:26-116; src/mamba_ssm/gpu/inference.rs:669-698):
+ * delta,u,y [batch,d_inner]; B,C [batch,d_state]. */
+MRS_API int mrs_ssm_step(void *stream, int dtype, float *h, void *y, const void *delta, const void *u,
+                 const void *B, const void *C, const float *a_neg, const float *D,
+                 int batch, int d_inner, int d_state);
+
+/* ssm_step_forward_gather_gate_{..} (kernels/mamba_ssm.cu:180-227;
+ * src/mamba_ssm/gpu/inference.rs:1182-1215): B and C are read from
+ * xdbl[b*xdbl_stride + b_offset + n] / [.. + c_offset + n]; y *= gate_silu.
+ * gate_silu == NULL gives ssm_step_forward_gather_{..} (kernels/mamba_ssm.cu:126-170). */
+MRS_API int mrs_ssm_step_gather_gate(void *stream, int dtype, float *h, void *y, const void *delta,
+                             const void *u, const void *xdbl, const void *gate_silu,
+                             const float *a_neg, const float *D, int batch, int d_inner, int d_state,
+                             int xdbl_stride, int b_offset, int c_offset);
+
+/* ---- causal depthwise conv1d (+SiLU) ----------------------------------------
+ * conv1d_step_forward_silu_{..} (kernels/conv1d.cu:85-115;
+ * src/mamba_ssm/gpu/inference.rs:1062-1084), order out,state,new_x,weight,bias,batch,d_inner,d_conv.
+ *   state [batch,d_inner,d_conv] f32 window, shifted left and updated in place
+ *   new_x,out [batch,d_inner] dtype; weight [d_inner,d_conv], bias [d_inner] f32
+ * apply_silu = 0 gives conv1d_step_forward_{..} (kernels/conv1d.cu:14-75). d_conv in 1..=8. */
+MRS_API int mrs_conv1d_step(void *stream, int dtype, void *out, float *state, const void *new_x,
+                    const float *weight, const float *bias, int batch, int d_inner, int d_conv,
+                    int apply_silu);
+
+/* conv1d_burnin_forward_nosave_{..} (kernels/conv1d.cu:209-315;
+ * src/mamba_ssm/gpu/prefill.rs:417-439, 780-804), order u_out,state,x_branch,weight,bias,batch,T,d_inner,d_conv.
+ *   x_branch rows of x_stride elements ([batch*T] rows; x_stride = d_inner for the
+ *   reference's split buffer, 2*d_inner to read the x half of in_proj's output in place)
+ *   u_out [batch,T,d_inner] dtype, SiLU applied. */
+MRS_API int mrs_conv1d_seq_silu(void *stream, int dtype, void *u_out, float *state, const void *x_branch,
+                        int64_t x_stride, const float *weight, const float *bias,
+                        int batch, int T, int d_inner, int d_conv);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MAMBA_HIP_H */

@@ -1,0 +1,8 @@
+"""MI355X-native Mamba inference hot path (HIP kernels behind a C ABI).
+
+The compute lives in libmamba_hip.so (csrc/*.hip, built for gfx950); this
+package is the thin host side: ctypes binding, operator wrappers and the
+engine types that mirror the reference's GpuMambaBackbone surface.
+"""
+from ._lib import MambaHipError, load as load_library  # noqa: F401
+from .config import MambaConfig, ScanMode, WeightDtype, PARALLEL_SCAN_THRESHOLD  # noqa: F401

@@ -1,0 +1,65 @@
+// Shared device/host helpers for libmamba_hip (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+#include "../../include/mamba_hip.h"
+
+namespace mrs {
+
+constexpr int kWave = 64;
+constexpr float kLog2e = 1.4426950408889634f;
+
+// ---- storage types ---------------------------------------------------------
+// Activations are stored as f32, IEEE f16 or bf16 and widened to f32 on load;
+// stores round to nearest even (gfx950 has v_cvt_pk_bf16_f32 for bf16).
+using f16_t = _Float16;
+using bf16_t = __bf16;
+
+template <typename T> struct Store;
+template <> struct Store<float> {
+    static constexpr int dtype = MRS_F32;
+    __device__ static __forceinline__ float ld(const float *p) { return *p; }
+    __device__ static __forceinline__ void st(float *p, float v) { *p = v; }
+};
+template <> struct Store<f16_t> {
+    static constexpr int dtype = MRS_F16;
+    __device__ static __forceinline__ float ld(const f16_t *p) { return (float)*p; }
+    __device__ static __forceinline__ void st(f16_t *p, float v) { *p = (f16_t)v; }
+};
+template <> struct Store<bf16_t> {
+    static constexpr int dtype = MRS_BF16;
+    __device__ static __forceinline__ float ld(const bf16_t *p) {
+        return __uint_as_float((uint32_t)(*reinterpret_cast<const uint16_t *>(p)) << 16);
+    }
+    __device__ static __forceinline__ void st(bf16_t *p, float v) { *p = (bf16_t)v; }
+};
+
+// 2^x on the transcendental unit (v_exp_f32).  Arguments here are <= 0 or small,
+// results below the f32 normal range flush to 0, which is what the recurrence wants.
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+
+// x * sigmoid(x) = x / (1 + 2^(-x log2 e)); rcp is 1 ulp.  For x -> -inf the
+// denominator overflows to +inf and the product is -0, the correct limit.
+__device__ __forceinline__ float silu(float x) { return x * fast_rcp(1.0f + fast_exp2(-x * kLog2e)); }
+
+// ---- host-side error plumbing ---------------------------------------------
+void set_error(const char *fmt, ...);
+int fail(int code, const char *fmt, ...);
+int check_launch(const char *what);
+
+inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s); }
+inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+
+}  // namespace mrs
+
+// Dispatch a templated launch on the activation storage type.
+#define MRS_DISPATCH_DTYPE(dtype, T, ...)                                         \
+    switch (dtype) {                                                              \
+        case MRS_F32: { using T = float; __VA_ARGS__; break; }                    \
+        case MRS_F16: { using T = mrs::f16_t; __VA_ARGS__; break; }               \
+        case MRS_BF16: { using T = mrs::bf16_t; __VA_ARGS__; break; }             \
+        default: return mrs::fail(MRS_E_DTYPE, "dtype %d is not f32/f16/bf16", (int)(dtype)); \
+    }

@@ -1,0 +1,161 @@
+// Mamba-1 selective scan, one timestep (decode).
+//
+// Replaces ssm_step_forward_*, ssm_step_forward_gather_* and
+// ssm_step_forward_gather_gate_* (kernels/mamba_ssm.cu:26-227).  The work is a
+// read-modify-write of h [batch, d_inner, d_state] f32 -- 2*4*ds bytes per
+// (b,d) against 3-4 activation elements -- so the kernel is laid out for the
+// state stream: a group of LG = ds/4 lanes owns one (b,d) row and each lane
+// moves one float4 of it, which makes every h access a fully coalesced 1 KiB
+// wave transaction; the partial dot products are combined with lane shuffles.
+#include "common.hpp"
+
+namespace mrs {
+
+// B and C of batch row b are read at xdbl + b*stride + {b_off, c_off}; the plain
+// step passes stride = ds and separate base pointers.
+template <typename T, int LG, bool GATE>
+__global__ __launch_bounds__(256) void ssm_step_kernel(
+    float *__restrict__ h, T *__restrict__ y, const T *__restrict__ delta, const T *__restrict__ u,
+    const T *__restrict__ Bbase, const T *__restrict__ Cbase, int64_t bc_stride,
+    const T *__restrict__ gate, const float *__restrict__ a_neg, const float *__restrict__ Dp,
+    int64_t total, int di, int ds) {
+    // total = batch*d_inner rows; ds == 4*LG here.
+    const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t rowi = gid / LG;
+    const int g = (int)(gid % LG);
+    const bool live = rowi < total;
+    const int64_t r = live ? rowi : total - 1;
+    const int b = (int)(r / di);
+    const int d = (int)(r - (int64_t)b * di);
+    float4 hv = *reinterpret_cast<const float4 *>(h + r * ds + 4 * g);
+    const float4 av = *reinterpret_cast<const float4 *>(a_neg + (int64_t)d * ds + 4 * g);
+    const float dl = Store<T>::ld(delta + r);
+    const float uu = Store<T>::ld(u + r);
+    const float du = dl * uu;
+    const T *Br = Bbase + (int64_t)b * bc_stride + 4 * g;
+    const T *Cr = Cbase + (int64_t)b * bc_stride + 4 * g;
+    const float x = dl * kLog2e;
+    hv.x = fmaf(fast_exp2(x * av.x), hv.x, du * Store<T>::ld(Br + 0));
+    hv.y = fmaf(fast_exp2(x * av.y), hv.y, du * Store<T>::ld(Br + 1));
+    hv.z = fmaf(fast_exp2(x * av.z), hv.z, du * Store<T>::ld(Br + 2));
+    hv.w = fmaf(fast_exp2(x * av.w), hv.w, du * Store<T>::ld(Br + 3));
+    float acc = hv.x * Store<T>::ld(Cr + 0);
+    acc = fmaf(hv.y, Store<T>::ld(Cr + 1), acc);
+    acc = fmaf(hv.z, Store<T>::ld(Cr + 2), acc);
+    acc = fmaf(hv.w, Store<T>::ld(Cr + 3), acc);
+#pragma unroll
+    for (int m = 1; m < LG; m <<= 1) acc += __shfl_xor(acc, m, kWave);
+    if (live) {
+        *reinterpret_cast<float4 *>(h + r * ds + 4 * g) = hv;
+        if (g == 0) {
+            acc = fmaf(Dp[d], uu, acc);
+            if (GATE) acc *= Store<T>::ld(gate + r);
+            Store<T>::st(y + r, acc);
+        }
+    }
+}
+
+// Any d_state (1..=256), one lane per (b,d), states streamed in order.
+template <typename T, bool GATE>
+__global__ __launch_bounds__(256) void ssm_step_generic_kernel(
+    float *__restrict__ h, T *__restrict__ y, const T *__restrict__ delta, const T *__restrict__ u,
+    const T *__restrict__ Bbase, const T *__restrict__ Cbase, int64_t bc_stride,
+    const T *__restrict__ gate, const float *__restrict__ a_neg, const float *__restrict__ Dp,
+    int64_t total, int di, int ds) {
+    const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (r >= total) return;
+    const int b = (int)(r / di);
+    const int d = (int)(r - (int64_t)b * di);
+    const float dl = Store<T>::ld(delta + r);
+    const float uu = Store<T>::ld(u + r);
+    const float du = dl * uu;
+    const float x = dl * kLog2e;
+    float acc = Dp[d] * uu;
+    float *hr = h + r * ds;
+    const float *ar = a_neg + (int64_t)d * ds;
+    const T *Br = Bbase + (int64_t)b * bc_stride;
+    const T *Cr = Cbase + (int64_t)b * bc_stride;
+    for (int n = 0; n < ds; n++) {
+        const float hn = fmaf(fast_exp2(x * ar[n]), hr[n], du * Store<T>::ld(Br + n));
+        hr[n] = hn;
+        acc = fmaf(hn, Store<T>::ld(Cr + n), acc);
+    }
+    if (GATE) acc *= Store<T>::ld(gate + r);
+    Store<T>::st(y + r, acc);
+}
+
+template <typename T>
+static int launch_step(hipStream_t st, float *h, void *y, const void *delta, const void *u,
+                       const void *Bb, const void *Cb, int64_t bc_stride, const void *gate,
+                       const float *a_neg, const float *D, int batch, int di, int ds) {
+    const int64_t total = (int64_t)batch * di;
+#define MRS_ARGS h, (T *)y, (const T *)delta, (const T *)u, (const T *)Bb, (const T *)Cb, bc_stride, \
+                 (const T *)gate, a_neg, D, total, di, ds
+    const bool vec_ok = aligned(h, 16) && aligned(a_neg, 16);
+    int lg = 0;
+    if (vec_ok && (ds == 4 || ds == 8 || ds == 16 || ds == 32 || ds == 64 || ds == 128 || ds == 256)) lg = ds / 4;
+    if (lg) {
+        const int64_t threads = total * lg;
+        const int64_t blocks = (threads + 255) / 256;
+        if (blocks > 0x7fffffffLL) return fail(MRS_E_SHAPE, "ssm step: grid too large");
+        const dim3 grid((unsigned)blocks), block(256);
+#define MRS_LG(L)                                                                                      \
+    case L:                                                                                            \
+        if (gate) hipLaunchKernelGGL((ssm_step_kernel<T, L, true>), grid, block, 0, st, MRS_ARGS);     \
+        else hipLaunchKernelGGL((ssm_step_kernel<T, L, false>), grid, block, 0, st, MRS_ARGS);         \
+        break
+        switch (lg) { MRS_LG(1); MRS_LG(2); MRS_LG(4); MRS_LG(8); MRS_LG(16); MRS_LG(32); MRS_LG(64); }
+#undef MRS_LG
+    } else {
+        const int64_t blocks = (total + 255) / 256;
+        if (blocks > 0x7fffffffLL) return fail(MRS_E_SHAPE, "ssm step: grid too large");
+        const dim3 grid((unsigned)blocks), block(256);
+        if (gate) hipLaunchKernelGGL((ssm_step_generic_kernel<T, true>), grid, block, 0, st, MRS_ARGS);
+        else hipLaunchKernelGGL((ssm_step_generic_kernel<T, false>), grid, block, 0, st, MRS_ARGS);
+    }
+#undef MRS_ARGS
+    return check_launch("ssm_step_kernel");
+}
+
+static int step_check(const char *fn, int dtype, const void *h, const void *y, const void *delta,
+                      const void *u, const void *B, const void *C, const void *a_neg, const void *D,
+                      int batch, int di, int ds) {
+    if (dtype != MRS_F32 && dtype != MRS_F16 && dtype != MRS_BF16)
+        return fail(MRS_E_DTYPE, "%s: dtype %d is not f32/f16/bf16", fn, dtype);
+    if (!h || !y || !delta || !u || !B || !C || !a_neg || !D) return fail(MRS_E_NULL, "%s: null pointer", fn);
+    if (batch < 1 || di < 1) return fail(MRS_E_SHAPE, "%s: batch=%d d_inner=%d must be >= 1", fn, batch, di);
+    if (ds < 1 || ds > 256) return fail(MRS_E_SHAPE, "%s: d_state=%d outside 1..=256", fn, ds);
+    if ((int64_t)batch * di * ds > 0x7fffffffLL) return fail(MRS_E_SHAPE, "%s: batch*d_inner*d_state exceeds i32", fn);
+    return MRS_OK;
+}
+
+}  // namespace mrs
+
+using namespace mrs;
+
+extern "C" int mrs_ssm_step(void *stream, int dtype, float *h, void *y, const void *delta, const void *u,
+                            const void *B, const void *C, const float *a_neg, const float *D,
+                            int batch, int d_inner, int d_state) {
+    int rc = step_check("mrs_ssm_step", dtype, h, y, delta, u, B, C, a_neg, D, batch, d_inner, d_state);
+    if (rc) return rc;
+    hipStream_t st = as_stream(stream);
+    MRS_DISPATCH_DTYPE(dtype, T_, return launch_step<T_>(st, h, y, delta, u, B, C, d_state, nullptr, a_neg, D, batch, d_inner, d_state));
+    return MRS_OK;
+}
+
+extern "C" int mrs_ssm_step_gather_gate(void *stream, int dtype, float *h, void *y, const void *delta,
+                                        const void *u, const void *xdbl, const void *gate_silu,
+                                        const float *a_neg, const float *D, int batch, int d_inner,
+                                        int d_state, int xdbl_stride, int b_offset, int c_offset) {
+    int rc = step_check("mrs_ssm_step_gather_gate", dtype, h, y, delta, u, xdbl, xdbl, a_neg, D, batch, d_inner, d_state);
+    if (rc) return rc;
+    if (b_offset < 0 || c_offset < 0 || b_offset + d_state > xdbl_stride || c_offset + d_state > xdbl_stride)
+        return fail(MRS_E_SHAPE, "mrs_ssm_step_gather_gate: offsets %d/%d + d_state %d exceed xdbl_stride %d",
+                    b_offset, c_offset, d_state, xdbl_stride);
+    const size_t es = (dtype == MRS_F32) ? 4 : 2;
+    const char *xb = static_cast<const char *>(xdbl);
+    hipStream_t st = as_stream(stream);
+    MRS_DISPATCH_DTYPE(dtype, T_, return launch_step<T_>(st, h, y, delta, u, xb + es * b_offset, xb + es * c_offset,
+                                                         xdbl_stride, gate_silu, a_neg, D, batch, d_inner, d_state));
+    return MRS_OK;
+}

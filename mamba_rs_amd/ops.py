@@ -1,0 +1,156 @@
+"""Operator-level host API: one function per kernel family, torch tensors in.
+
+These wrappers only validate what the C ABI cannot see (device, dtype
+agreement, contiguity, shapes), pick up torch's current stream and pass raw
+device pointers to libmamba_hip.  Names and argument order follow the
+reference's launch sites (src/mamba_ssm/gpu/prefill.rs:910-933,
+src/mamba_ssm/gpu/inference.rs:1062-1084, 1182-1215).
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+from .config import WeightDtype
+
+GATE_NONE = 0
+GATE_PREACT = 1 << 0
+GATE_SILU = 1 << 1
+A_S4D_REAL = 1 << 2
+FORCE_SEQUENTIAL = 1 << 3
+FORCE_PARALLEL = 1 << 4
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _p(t: torch.Tensor | None) -> int | None:
+    return None if t is None else t.data_ptr()
+
+
+def _dev(*ts: torch.Tensor) -> None:
+    for t in ts:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise ValueError("mamba_rs_amd ops need device tensors (there is no CPU path)")
+        if not t.is_contiguous():
+            raise ValueError("tensor must be contiguous")
+
+
+def _f32(*ts: torch.Tensor) -> None:
+    for t in ts:
+        if t.dtype != torch.float32:
+            raise ValueError(f"expected an f32 tensor, got {t.dtype}")
+
+
+def _act_dtype(*ts: torch.Tensor) -> WeightDtype:
+    dt = ts[0].dtype
+    for t in ts:
+        if t is not None and t.dtype != dt:
+            raise ValueError(f"activation dtypes differ: {dt} vs {t.dtype}")
+    return WeightDtype.from_torch(dt)
+
+
+def exp_negate(a_log: torch.Tensor) -> torch.Tensor:
+    """a_neg = -exp(a_log) (exp_negate, kernels/elementwise.cu:140-146)."""
+    _dev(a_log); _f32(a_log)
+    out = torch.empty_like(a_log)
+    _lib.call("mrs_exp_negate", _stream(), _p(out), _p(a_log), a_log.numel())
+    return out
+
+
+def a_neg_is_s4d_real(a_neg: torch.Tensor) -> bool:
+    """True iff a_neg[d,n] = (n+1)*a_neg[d,0] to 4 ulp (S4D-real init). Synchronises (weight-load time only)."""
+    _dev(a_neg); _f32(a_neg)
+    di, ds = a_neg.shape
+    flag = torch.zeros(1, dtype=torch.int32, device=a_neg.device)
+    _lib.call("mrs_a_neg_is_s4d_real", _stream(), _p(flag), _p(a_neg), di, ds)
+    return bool(flag.item())
+
+
+def ssm_scan_workspace_bytes(batch: int, T: int, d_inner: int, d_state: int) -> int:
+    return int(_lib.load().mrs_ssm_scan_workspace_bytes(batch, T, d_inner, d_state))
+
+
+def ssm_scan_fwd(h, y, delta, u, B, C, a_neg, D, *, gate=None, flags: int = 0, workspace=None):
+    """Selective scan over a whole sequence; h [B,di,ds] is updated in place, y is written.
+
+    delta,u,y (and gate) are [batch,T,d_inner]; B and C are [batch,T,d_state] or
+    strided views into xdbl [batch,T,xd] (same row stride for both)."""
+    batch, T, di = delta.shape
+    ds = a_neg.shape[1]
+    _dev(h, y, delta, u, a_neg, D, gate, workspace); _f32(h, a_neg, D)
+    dt = _act_dtype(delta, u, y, B, C, *([gate] if gate is not None else []))
+    for t in (B, C):
+        if not t.is_cuda or t.stride(-1) != 1 or t.shape != (batch, T, ds):
+            raise ValueError("B/C must be device tensors [batch,T,d_state] with unit inner stride")
+    bc_stride = B.stride(1)
+    if C.stride(1) != bc_stride or B.stride(0) != T * bc_stride or C.stride(0) != T * bc_stride:
+        raise ValueError("B and C must share one row stride and be row-dense over [batch*T]")
+    if h.shape != (batch, di, ds) or y.shape != delta.shape or u.shape != delta.shape or a_neg.shape != (di, ds) or D.shape != (di,):
+        raise ValueError("shape mismatch")
+    if gate is not None and gate.shape != delta.shape:
+        raise ValueError("gate shape mismatch")
+    ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    _lib.call("mrs_ssm_scan_fwd_ex", _stream(), int(dt), _p(h), _p(y), _p(delta), _p(u), _p(B), _p(C), bc_stride,
+              _p(a_neg), _p(D), _p(gate), flags, _p(workspace), ws_bytes, batch, T, di, ds)
+    return y
+
+
+def ssm_step(h, y, delta, u, B, C, a_neg, D):
+    """One decode step (ssm_step_forward, kernels/mamba_ssm.cu:26-116)."""
+    batch, di = delta.shape
+    ds = a_neg.shape[1]
+    _dev(h, y, delta, u, B, C, a_neg, D); _f32(h, a_neg, D)
+    dt = _act_dtype(delta, u, y, B, C)
+    if h.shape != (batch, di, ds) or B.shape != (batch, ds) or C.shape != (batch, ds) or y.shape != delta.shape:
+        raise ValueError("shape mismatch")
+    _lib.call("mrs_ssm_step", _stream(), int(dt), _p(h), _p(y), _p(delta), _p(u), _p(B), _p(C), _p(a_neg), _p(D),
+              batch, di, ds)
+    return y
+
+
+def ssm_step_gather_gate(h, y, delta, u, xdbl, gate_silu, a_neg, D, b_offset: int, c_offset: int):
+    """Decode step reading B/C out of xdbl and multiplying by gate_silu
+    (ssm_step_forward_gather_gate, kernels/mamba_ssm.cu:180-227). gate_silu may be None."""
+    batch, di = delta.shape
+    ds = a_neg.shape[1]
+    _dev(h, y, delta, u, xdbl, gate_silu, a_neg, D); _f32(h, a_neg, D)
+    dt = _act_dtype(delta, u, y, xdbl, *([gate_silu] if gate_silu is not None else []))
+    if h.shape != (batch, di, ds) or xdbl.shape[0] != batch or y.shape != delta.shape:
+        raise ValueError("shape mismatch")
+    _lib.call("mrs_ssm_step_gather_gate", _stream(), int(dt), _p(h), _p(y), _p(delta), _p(u), _p(xdbl), _p(gate_silu),
+              _p(a_neg), _p(D), batch, di, ds, xdbl.shape[1], b_offset, c_offset)
+    return y
+
+
+def conv1d_step(out, state, new_x, weight, bias, *, silu: bool = True):
+    """Shift-register conv step (+SiLU) (conv1d_step_forward[_silu], kernels/conv1d.cu:14-115)."""
+    batch, di = new_x.shape
+    dc = weight.shape[1]
+    _dev(out, state, new_x, weight, bias); _f32(state, weight, bias)
+    dt = _act_dtype(new_x, out)
+    if state.shape != (batch, di, dc) or weight.shape != (di, dc) or bias.shape != (di,) or out.shape != new_x.shape:
+        raise ValueError("shape mismatch")
+    _lib.call("mrs_conv1d_step", _stream(), int(dt), _p(out), _p(state), _p(new_x), _p(weight), _p(bias), batch, di, dc,
+              1 if silu else 0)
+    return out
+
+
+def conv1d_seq_silu(u_out, state, x_branch, weight, bias):
+    """Full-sequence causal conv + SiLU with state carry
+    (conv1d_burnin_forward_nosave, kernels/conv1d.cu:209-315).
+    x_branch is [batch,T,d_inner], possibly a view into a wider row (e.g. in_proj output)."""
+    batch, T, di = x_branch.shape
+    dc = weight.shape[1]
+    _dev(u_out, state, weight, bias); _f32(state, weight, bias)
+    if not x_branch.is_cuda or x_branch.stride(2) != 1 or x_branch.stride(0) != T * x_branch.stride(1):
+        raise ValueError("x_branch must be row-dense over [batch*T] with unit inner stride")
+    dt = _act_dtype(x_branch, u_out)
+    if state.shape != (batch, di, dc) or weight.shape != (di, dc) or bias.shape != (di,) or u_out.shape != (batch, T, di):
+        raise ValueError("shape mismatch")
+    _lib.call("mrs_conv1d_seq_silu", _stream(), int(dt), _p(u_out), _p(state), _p(x_branch), x_branch.stride(1),
+              _p(weight), _p(bias), batch, T, di, dc)
+    return u_out

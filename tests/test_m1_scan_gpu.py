@@ -1,0 +1,158 @@
+"""GPU parity: Mamba-1 selective scan (prefill route) vs the f64 oracle, through the C ABI."""
+import numpy as np
+import pytest
+import torch
+
+import orc
+from gpu_util import DEV, assert_close, dev, host, quant
+from util import scan_inputs
+
+pytestmark = pytest.mark.gpu
+
+ops = pytest.importorskip("mamba_rs_amd.ops")
+from mamba_rs_amd import MambaHipError, _lib  # noqa: E402
+
+GATE_FLAG = {0: ops.GATE_NONE, 1: ops.GATE_PREACT, 2: ops.GATE_SILU}
+
+
+def run_scan(inp, h0, dtype, gate_mode=0, flags=0, bc_view=None, workspace=None):
+    """Run the HIP scan on quantised inputs; returns (y f32 np, h f32 np)."""
+    delta, u = dev(inp["delta"], dtype), dev(inp["u"], dtype)
+    if bc_view is None:
+        Bm, Cm = dev(inp["B"], dtype), dev(inp["C"], dtype)
+    else:
+        Bm, Cm = bc_view
+    a_neg, D = dev(inp["a_neg"]), dev(inp["D"])
+    h = dev(h0)
+    y = torch.full_like(delta, float("nan"))
+    gate = dev(inp["z"], dtype) if gate_mode else None
+    ops.ssm_scan_fwd(h, y, delta, u, Bm, Cm, a_neg, D, gate=gate, flags=flags | GATE_FLAG[gate_mode], workspace=workspace)
+    torch.cuda.synchronize()
+    return host(y), host(h)
+
+
+def quantised(rng, batch, T, di, ds, dtype, s4d=True):
+    inp = scan_inputs(rng, batch, T, di, ds, s4d=s4d)
+    for k in ("u", "delta", "B", "C", "z"):
+        inp[k] = quant(inp[k], dtype)
+    return inp
+
+
+SHAPES = [
+    # batch, T, d_inner, d_state
+    (2, 33, 64, 16),
+    (1, 300, 200, 16),    # d_inner not a multiple of the 64-channel tile
+    (2, 17, 96, 8),
+    (1, 9, 32, 64),       # 4 lanes per channel
+    (1, 5, 16, 256),      # reference maximum d_state (src/config.rs:147-152)
+    (1, 7, 8, 24),        # d_state not a power of two
+    (3, 1, 40, 16),       # T = 1
+]
+
+
+@pytest.mark.parametrize("dtype", [orc.F32, orc.BF16, orc.F16])
+@pytest.mark.parametrize("shape", SHAPES)
+@pytest.mark.parametrize("s4d", [False, True])
+def test_scan_matches_oracle(shape, dtype, s4d):
+    batch, T, di, ds = shape
+    rng = np.random.default_rng(hash((shape, dtype, s4d)) & 0xFFFF)
+    inp = quantised(rng, batch, T, di, ds, dtype, s4d=s4d)
+    h0 = (rng.standard_normal((batch, di, ds)) * 0.1).astype(np.float32)
+    for gate_mode in (0, 1, 2):
+        print(f"case shape={shape} dtype={dtype} s4d={s4d} gate={gate_mode}", flush=True)
+        y_ref, h_ref = orc.m1_scan_f64(h0, inp["delta"], inp["u"], inp["B"], inp["C"], inp["a_neg"], inp["D"],
+                                       gate=inp["z"] if gate_mode else None, gate_mode=gate_mode)
+        y, h = run_scan(inp, h0, dtype, gate_mode, flags=ops.A_S4D_REAL if s4d else 0)
+        assert_close(y, y_ref, dtype, "y")
+        assert_close(h, h_ref, orc.F32, "h")
+
+
+def test_scan_s4d_flag_from_device_check():
+    rng = np.random.default_rng(1)
+    inp = scan_inputs(rng, 1, 4, 32, 16, s4d=True)
+    assert ops.a_neg_is_s4d_real(dev(inp["a_neg"]))
+    # a_neg as the reference derives it: -exp(log(n+1)) in f32 (src/weights.rs:44-48,143-148)
+    a_log = dev(np.log(np.arange(1, 17, dtype=np.float32))[None].repeat(32, 0))
+    a_neg = ops.exp_negate(a_log)
+    assert np.allclose(host(a_neg), -np.exp(host(a_log).astype(np.float64)), rtol=3e-7)
+    assert ops.a_neg_is_s4d_real(a_neg)
+    inp2 = scan_inputs(rng, 1, 4, 32, 16, s4d=False)
+    assert not ops.a_neg_is_s4d_real(dev(inp2["a_neg"]))
+
+
+def test_scan_state_carry_two_calls_equal_one():
+    rng = np.random.default_rng(2)
+    inp = quantised(rng, 2, 70, 128, 16, orc.BF16)
+    h0 = np.zeros((2, 128, 16), np.float32)
+    y, h = run_scan(inp, h0, orc.BF16, 2)
+    a = {k: (v[:, :41] if v.ndim == 3 and v.shape[1] == 70 else v) for k, v in inp.items()}
+    b = {k: (v[:, 41:] if v.ndim == 3 and v.shape[1] == 70 else v) for k, v in inp.items()}
+    y1, h1 = run_scan(a, h0, orc.BF16, 2)
+    y2, h2 = run_scan(b, h1, orc.BF16, 2)
+    assert np.array_equal(np.concatenate([y1, y2], 1), y) and np.array_equal(h2, h)
+
+
+@pytest.mark.parametrize("dtype", [orc.F32, orc.BF16])
+def test_scan_reads_b_c_in_place_from_xdbl(dtype):
+    # B and C as strided views of xdbl [batch, T, dt_rank + 2*ds] (130m shape: 48 + 32)
+    rng = np.random.default_rng(3)
+    batch, T, di, ds, dr = 2, 20, 64, 16, 48
+    inp = quantised(rng, batch, T, di, ds, dtype)
+    xdbl = quant(rng.standard_normal((batch, T, dr + 2 * ds)).astype(np.float32), dtype)
+    inp["B"], inp["C"] = xdbl[:, :, dr:dr + ds].copy(), xdbl[:, :, dr + ds:].copy()
+    h0 = np.zeros((batch, di, ds), np.float32)
+    xd = dev(xdbl, dtype)
+    y, h = run_scan(inp, h0, dtype, 0, bc_view=(xd[:, :, dr:dr + ds], xd[:, :, dr + ds:]))
+    y_ref, h_ref = orc.m1_scan_f64(h0, inp["delta"], inp["u"], inp["B"], inp["C"], inp["a_neg"], inp["D"])
+    assert_close(y, y_ref, dtype, "y")
+    assert_close(h, h_ref, orc.F32, "h")
+
+
+def test_scan_full_size_channel_subset_and_linearity():
+    """The isolated-scan workload (B=8, T=2048, d_inner=1536, d_state=16, bf16, gated):
+    channels are independent, so the oracle is run on a subset of channels of the
+    full-size launch; plus linearity in u (h0 = 0, f32 state): scan(2u) = 2 scan(u) exactly."""
+    rng = np.random.default_rng(4)
+    batch, T, di, ds = 8, 2048, 1536, 16
+    inp = quantised(rng, batch, T, di, ds, orc.BF16)
+    h0 = np.zeros((batch, di, ds), np.float32)
+    y, h = run_scan(inp, h0, orc.BF16, 2, flags=ops.A_S4D_REAL)
+    sel = np.sort(rng.choice(di, 48, replace=False))
+    sub = dict(delta=inp["delta"][:, :, sel], u=inp["u"][:, :, sel], z=inp["z"][:, :, sel], B=inp["B"], C=inp["C"],
+               a_neg=inp["a_neg"][sel], D=inp["D"][sel])
+    y_ref, h_ref = orc.m1_scan_f64(h0[:, sel], sub["delta"], sub["u"], sub["B"], sub["C"], sub["a_neg"], sub["D"],
+                                   gate=sub["z"], gate_mode=2)
+    assert_close(y[:, :, sel], y_ref, orc.BF16, "y[subset]")
+    assert_close(h[:, sel], h_ref, orc.F32, "h[subset]")
+    inp2 = dict(inp); inp2["u"] = inp["u"] * 2.0          # exact in bf16
+    y2, h2 = run_scan(inp2, h0, orc.BF16, 0, flags=ops.A_S4D_REAL)
+    y1, h1 = run_scan(inp, h0, orc.BF16, 0, flags=ops.A_S4D_REAL)
+    assert np.array_equal(h2, 2.0 * h1) and np.array_equal(y2, 2.0 * y1)
+
+
+def test_scan_rejects_bad_arguments():
+    rng = np.random.default_rng(5)
+    inp = quantised(rng, 1, 4, 16, 16, orc.F32)
+    t = {k: dev(v) for k, v in inp.items()}
+    h = torch.zeros(1, 16, 16, device=DEV)
+    y = torch.empty_like(t["delta"])
+    s = torch.cuda.current_stream().cuda_stream
+    args = [s, 0, h.data_ptr(), y.data_ptr(), t["delta"].data_ptr(), t["u"].data_ptr(), t["B"].data_ptr(),
+            t["C"].data_ptr(), t["a_neg"].data_ptr(), t["D"].data_ptr(), 1, 4, 16, 16]
+
+    def expect(code, **chg):
+        a = list(args)
+        for i, v in chg.items():
+            a[int(i[1:])] = v
+        with pytest.raises(MambaHipError) as e:
+            _lib.call("mrs_ssm_scan_fwd", *a)
+        assert e.value.code == code and e.value.message
+
+    expect(-1, _2=None)          # null h
+    expect(-3, _1=7)             # dtype
+    expect(-2, _13=0)            # d_state 0
+    expect(-2, _13=257)          # d_state above the reference maximum
+    expect(-2, _11=0)            # T = 0 (src/mamba_ssm/gpu/launch.rs:20-47)
+    expect(-2, _10=0)            # batch = 0
+    _lib.call("mrs_ssm_scan_fwd", *args)   # and the unmodified call succeeds
+    torch.cuda.synchronize()
