@@ -15,8 +15,9 @@ from mamba_rs_amd import MambaHipError, _lib  # noqa: E402
 GATE_FLAG = {0: ops.GATE_NONE, 1: ops.GATE_PREACT, 2: ops.GATE_SILU}
 
 
-def run_scan(inp, h0, dtype, gate_mode=0, flags=0, bc_view=None, workspace=None):
-    """Run the HIP scan on quantised inputs; returns (y f32 np, h f32 np)."""
+def run_scan(inp, h0, dtype, gate_mode=0, flags=0, bc_view=None, split=None):
+    """Run the HIP scan on quantised inputs; returns (y f32 np, h f32 np).
+    split: None = no workspace (sequential route), "auto" = workspace given, "force" = T-split forced."""
     delta, u = dev(inp["delta"], dtype), dev(inp["u"], dtype)
     if bc_view is None:
         Bm, Cm = dev(inp["B"], dtype), dev(inp["C"], dtype)
@@ -26,6 +27,12 @@ def run_scan(inp, h0, dtype, gate_mode=0, flags=0, bc_view=None, workspace=None)
     h = dev(h0)
     y = torch.full_like(delta, float("nan"))
     gate = dev(inp["z"], dtype) if gate_mode else None
+    workspace = None
+    if split is not None:
+        batch, T, di = inp["delta"].shape
+        workspace = torch.empty(ops.ssm_scan_workspace_bytes(batch, T, di, inp["a_neg"].shape[1]), dtype=torch.uint8, device=DEV)
+        if split == "force":
+            flags |= ops.FORCE_PARALLEL
     ops.ssm_scan_fwd(h, y, delta, u, Bm, Cm, a_neg, D, gate=gate, flags=flags | GATE_FLAG[gate_mode], workspace=workspace)
     torch.cuda.synchronize()
     return host(y), host(h)
@@ -65,6 +72,45 @@ def test_scan_matches_oracle(shape, dtype, s4d):
         y, h = run_scan(inp, h0, dtype, gate_mode, flags=ops.A_S4D_REAL if s4d else 0)
         assert_close(y, y_ref, dtype, "y")
         assert_close(h, h_ref, orc.F32, "h")
+
+
+SPLIT_SHAPES = [(2, 333, 64, 16), (1, 300, 200, 16), (3, 64, 128, 16), (1, 1025, 72, 16)]
+
+
+@pytest.mark.parametrize("dtype", [orc.F32, orc.BF16, orc.F16])
+@pytest.mark.parametrize("shape", SPLIT_SHAPES)
+@pytest.mark.parametrize("s4d", [False, True])
+def test_scan_t_split_route_matches_oracle(shape, dtype, s4d):
+    """The chunked (T-split) route: chunk summaries + carry fold must equal the serial scan."""
+    batch, T, di, ds = shape
+    rng = np.random.default_rng(hash((shape, dtype, s4d, 1)) & 0xFFFF)
+    inp = quantised(rng, batch, T, di, ds, dtype, s4d=s4d)
+    h0 = (rng.standard_normal((batch, di, ds)) * 0.1).astype(np.float32)
+    for gate_mode in (0, 1, 2):
+        print(f"case split shape={shape} dtype={dtype} s4d={s4d} gate={gate_mode}", flush=True)
+        y_ref, h_ref = orc.m1_scan_f64(h0, inp["delta"], inp["u"], inp["B"], inp["C"], inp["a_neg"], inp["D"],
+                                       gate=inp["z"] if gate_mode else None, gate_mode=gate_mode)
+        y, h = run_scan(inp, h0, dtype, gate_mode, flags=ops.A_S4D_REAL if s4d else 0, split="force")
+        assert_close(y, y_ref, dtype, "y")
+        assert_close(h, h_ref, orc.F32, "h")
+
+
+def test_scan_auto_route_threshold_and_workspace_errors():
+    """T <= 256 stays on the sequential route even with a workspace (src/config.rs:21-37), so it is
+    bitwise equal to the no-workspace call; a short workspace is refused."""
+    rng = np.random.default_rng(9)
+    inp = quantised(rng, 2, 256, 64, 16, orc.BF16)
+    h0 = np.zeros((2, 64, 16), np.float32)
+    y_seq, h_seq = run_scan(inp, h0, orc.BF16)
+    y_auto, h_auto = run_scan(inp, h0, orc.BF16, split="auto")
+    assert np.array_equal(y_seq, y_auto) and np.array_equal(h_seq, h_auto)
+    inp = quantised(rng, 2, 512, 64, 16, orc.BF16)
+    t = {k: dev(v, orc.BF16 if k in ("u", "delta", "B", "C", "z") else orc.F32) for k, v in inp.items()}
+    h = torch.zeros(2, 64, 16, device=DEV); y = torch.empty_like(t["delta"])
+    small = torch.empty(256, dtype=torch.uint8, device=DEV)
+    with pytest.raises(MambaHipError) as e:
+        ops.ssm_scan_fwd(h, y, t["delta"], t["u"], t["B"], t["C"], t["a_neg"], t["D"], workspace=small)
+    assert e.value.code == -4
 
 
 def test_scan_s4d_flag_from_device_check():
@@ -116,7 +162,7 @@ def test_scan_full_size_channel_subset_and_linearity():
     batch, T, di, ds = 8, 2048, 1536, 16
     inp = quantised(rng, batch, T, di, ds, orc.BF16)
     h0 = np.zeros((batch, di, ds), np.float32)
-    y, h = run_scan(inp, h0, orc.BF16, 2, flags=ops.A_S4D_REAL)
+    y, h = run_scan(inp, h0, orc.BF16, 2, flags=ops.A_S4D_REAL, split="auto")
     sel = np.sort(rng.choice(di, 48, replace=False))
     sub = dict(delta=inp["delta"][:, :, sel], u=inp["u"][:, :, sel], z=inp["z"][:, :, sel], B=inp["B"], C=inp["C"],
                a_neg=inp["a_neg"][sel], D=inp["D"][sel])
@@ -125,8 +171,8 @@ def test_scan_full_size_channel_subset_and_linearity():
     assert_close(y[:, :, sel], y_ref, orc.BF16, "y[subset]")
     assert_close(h[:, sel], h_ref, orc.F32, "h[subset]")
     inp2 = dict(inp); inp2["u"] = inp["u"] * 2.0          # exact in bf16
-    y2, h2 = run_scan(inp2, h0, orc.BF16, 0, flags=ops.A_S4D_REAL)
-    y1, h1 = run_scan(inp, h0, orc.BF16, 0, flags=ops.A_S4D_REAL)
+    y2, h2 = run_scan(inp2, h0, orc.BF16, 0, flags=ops.A_S4D_REAL, split="auto")
+    y1, h1 = run_scan(inp, h0, orc.BF16, 0, flags=ops.A_S4D_REAL, split="auto")
     assert np.array_equal(h2, 2.0 * h1) and np.array_equal(y2, 2.0 * y1)
 
 
