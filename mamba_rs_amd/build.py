@@ -18,10 +18,12 @@ CSRC = PKG_DIR / "csrc"
 LIB_PATH = PKG_DIR / "libmamba_hip.so"
 ARCH = "gfx950"
 
-# -packed-fp32-ops: keep the compiler from forming v_pk_*_f32 out of scalar float code.
+# -packed-fp32-ops (a minus sign in front of the feature name): keep the compiler from forming v_pk_*_f32 out of scalar float code.
 DEVICE_FLAGS = [
     f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # MFMA accumulators stay in ordinary VGPRs (no AccVGPR copies around each instruction).
+    "-mllvm", "-amdgpu-mfma-vgpr-form",
     "-Wno-unused-command-line-argument",
 ]
 

@@ -11,6 +11,7 @@
 // segment; the state h[n] of a channel lives in that lane's registers for the
 // whole sequence and is written back once.
 #include "common.hpp"
+#include <stdlib.h>
 
 namespace mrs {
 
@@ -128,7 +129,8 @@ static int launch_seq(hipStream_t st, bool s4d, int gate_mode, float *h, void *y
 // states of a channel in that lane's registers, B_t/C_t rows in scalar registers.
 //   pass A  chunk_state_kernel: chunk-end state S_c reached from a zero entering
 //           state (chunk 0: from the caller's h) and sum_t delta over the chunk,
-//           for chunks 0..C-2; also saves a copy of the caller's h.
+//           for chunks 0..C-2; saves a copy of the caller's h; extra blocks widen
+//           16-bit B/C rows to f32 once so pass B reads them with plain scalar loads.
 //   pass B  chunk_out_kernel: folds the summaries of the chunks before it into its
 //           entering state  h_in(c) = exp(a * sum delta_{c-1}) h_in(c-1) + S_{c-1},
 //           then runs the recurrence over its chunk writing y; the last chunk
@@ -141,56 +143,105 @@ struct SplitPlan {
     int len;     // L
 };
 
+constexpr int kGroup = 4;  // steps per prefetch group; chunk lengths are multiples of 2*kGroup
+
 static SplitPlan make_split_plan(int batch, int Tlen, int di) {
     const int tiles = (di + kWave - 1) / kWave;
     const int64_t base = (int64_t)batch * tiles;
-    int c = (int)((6144 + base - 1) / base);  // ~6 waves per SIMD on 1024 SIMDs
-    if (c > 32) c = 32;                        // the entering-state fold is O(C) per wave
-    if (c > Tlen / 32) c = Tlen / 32;          // chunks of at least 32 steps
+    static const int target = [] { const char *e = getenv("MRS_SCAN_TARGET_WAVES"); return e ? atoi(e) : 3072; }();
+    int c = (int)((target + base - 1) / base);  // ~3 waves per SIMD on 1024 SIMDs
+    if (c > 32) c = 32;                          // the entering-state fold is O(C) per wave
+    if (c > Tlen / 32) c = Tlen / 32;            // chunks of at least 32 steps
     if (c < 1) c = 1;
     int len = (Tlen + c - 1) / c;
-    len = (len + 3) & ~3;
+    len = (len + 2 * kGroup - 1) / (2 * kGroup) * (2 * kGroup);
     c = (Tlen + len - 1) / len;
     return {c, len};
 }
 
-static size_t split_workspace_floats(int batch, int di, int nchunk) {
-    // h0 copy [B][16][di] + S [B][C-1][16][di] + sum delta [B][C-1][di]
-    return (size_t)batch * 16 * di + (size_t)batch * (nchunk - 1) * 17 * di;
+struct SplitWs {
+    float *h0copy;  // [B][16][di]
+    float *S;       // [B][C-1][16][di]
+    float *sumd;    // [B][C-1][di]
+    float *Bt;      // [B*T][4][4] B rows as f32, regrouped: Bt[r][i][q] = B[r][4q+i]
+    float *Cf;      // [B*T][16] widened C rows (16-bit storage only)
+    size_t floats;
+};
+
+static SplitWs carve_workspace(float *base, int batch, int Tlen, int di, int nchunk) {
+    SplitWs w;
+    size_t o = 0;
+    w.h0copy = base + o; o += (size_t)batch * 16 * di;
+    w.S = base + o; o += (size_t)batch * (nchunk - 1) * 16 * di;
+    w.sumd = base + o; o += (size_t)batch * (nchunk - 1) * di;
+    o = (o + 63) & ~(size_t)63;  // 256-byte aligned rows for the scalar loads
+    w.Bt = base + o; o += (size_t)batch * Tlen * 16;
+    w.Cf = base + o; o += (size_t)batch * Tlen * 16;
+    w.floats = o;
+    return w;
 }
 
-// One row of B or C (16 values) as uniform f32.  16-bit rows are read as 8 packed
-// dwords with scalar loads (the address is wave-uniform), so they cost no VALU/LDS.
-template <typename T> struct Row16;
-template <> struct Row16<float> {
-    __device__ static __forceinline__ void ld(const float *r, float (&o)[16]) {
-#pragma unroll
-        for (int j = 0; j < 16; j++) o[j] = r[j];
+// Raw (unconverted) element types, so loads can be issued a group of steps ahead
+// of the arithmetic that widens and uses them.
+template <typename T> struct RawElem { using type = uint16_t; };
+template <> struct RawElem<float> { using type = float; };
+// Per-lane activation access through a buffer resource: address = base (scalar
+// registers) + per-step scalar offset + per-lane 32-bit offset, so the row walk costs
+// no vector ALU work.  num_records bounds the slab; offsets here stay below 2^31.
+template <typename T> struct LaneBuf {
+    __amdgpu_buffer_rsrc_t r;
+    __device__ __forceinline__ LaneBuf(const T *base, int64_t elems) {
+        r = __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(base), 0, (int)(elems * (int64_t)sizeof(T)), 0x00020000);
     }
-};
-template <> struct Row16<bf16_t> {
-    __device__ static __forceinline__ void ld(const bf16_t *r, float (&o)[16]) {
-        const uint32_t *w = reinterpret_cast<const uint32_t *>(r);
-#pragma unroll
-        for (int j = 0; j < 8; j++) {
-            const uint32_t v = w[j];
-            o[2 * j] = __uint_as_float(v << 16);
-            o[2 * j + 1] = __uint_as_float(v & 0xffff0000u);
+    __device__ __forceinline__ typename RawElem<T>::type ld(unsigned voff, unsigned soff) const {
+        if constexpr (sizeof(T) == 4) return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0));
+        else return __builtin_amdgcn_raw_buffer_load_b16(r, voff, soff, 0);
+    }
+    __device__ __forceinline__ void st(float v, unsigned voff, unsigned soff) const {
+        if constexpr (sizeof(T) == 4) {
+            __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), r, voff, soff, 0);
+        } else {
+            const T t = (T)v;
+            __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(uint16_t, t), r, voff, soff, 0);
         }
     }
 };
-template <> struct Row16<f16_t> {
-    __device__ static __forceinline__ void ld(const f16_t *r, float (&o)[16]) {
-        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
-        const h2 *w = reinterpret_cast<const h2 *>(r);
+__device__ __forceinline__ float widen(float v, const float *) { return v; }
+__device__ __forceinline__ float widen(uint16_t v, const bf16_t *) { return __uint_as_float((uint32_t)v << 16); }
+__device__ __forceinline__ float widen(uint16_t v, const f16_t *) { return (float)__builtin_bit_cast(_Float16, v); }
+
+// One row of B or C (16 values).  The address is wave-uniform, so these are scalar
+// loads; 16-bit rows come as 8 packed dwords and are unpacked on the scalar ALU.
+template <typename T> struct RowRaw { uint32_t w[8]; };
+template <> struct RowRaw<float> { float w[16]; };
+
+template <typename T> __device__ __forceinline__ void row_ld(const T *r, RowRaw<T> &o) {
+    const uint32_t *w = reinterpret_cast<const uint32_t *>(r);
 #pragma unroll
-        for (int j = 0; j < 8; j++) {
-            const h2 v = w[j];
-            o[2 * j] = (float)v.x;
-            o[2 * j + 1] = (float)v.y;
-        }
+    for (int j = 0; j < 8; j++) o.w[j] = w[j];
+}
+template <> __device__ __forceinline__ void row_ld<float>(const float *r, RowRaw<float> &o) {
+#pragma unroll
+    for (int j = 0; j < 16; j++) o.w[j] = r[j];
+}
+__device__ __forceinline__ void row_unpack(const RowRaw<float> &r, float (&o)[16], const float *) {
+#pragma unroll
+    for (int j = 0; j < 16; j++) o[j] = r.w[j];
+}
+__device__ __forceinline__ void row_unpack(const RowRaw<bf16_t> &r, float (&o)[16], const bf16_t *) {
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        o[2 * j] = __uint_as_float(r.w[j] << 16);
+        o[2 * j + 1] = __uint_as_float(r.w[j] & 0xffff0000u);
     }
-};
+}
+__device__ __forceinline__ void row_unpack(const RowRaw<f16_t> &r, float (&o)[16], const f16_t *) {
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        o[2 * j] = (float)__builtin_bit_cast(_Float16, (uint16_t)(r.w[j] & 0xffffu));
+        o[2 * j + 1] = (float)__builtin_bit_cast(_Float16, (uint16_t)(r.w[j] >> 16));
+    }
+}
 
 // Decay factors of one step: da[n] = 2^(dl * a2[n]); S4D: a2[n] = (n+1) a2[0] -> powers of one exp.
 template <bool S4D>
@@ -203,6 +254,16 @@ __device__ __forceinline__ void decay16(float dl, const float (&a2)[16], float (
     } else {
 #pragma unroll
         for (int j = 0; j < 16; j++) da[j] = fast_exp2(dl * a2[j]);
+    }
+}
+
+template <bool S4D>
+__device__ __forceinline__ void load_a2(float (&a2)[16], const float *__restrict__ a_neg, int d) {
+#pragma unroll
+    for (int j = 0; j < 16; j++) a2[j] = a_neg[(int64_t)d * 16 + j] * kLog2e;
+    if (S4D) {
+#pragma unroll
+        for (int j = 1; j < 16; j++) a2[j] = a2[0] * (float)(j + 1);
     }
 }
 
@@ -226,84 +287,136 @@ __device__ __forceinline__ void fold_entering_state(float (&hs)[16], const float
 template <typename T, bool S4D>
 __global__ __launch_bounds__(kWave) void chunk_state_kernel(
     const float *__restrict__ h, const T *__restrict__ delta, const T *__restrict__ u,
-    const T *__restrict__ Bm, int64_t bc_stride, const float *__restrict__ a_neg,
-    float *__restrict__ h0copy, float *__restrict__ S, float *__restrict__ sumd,
-    int Tlen, int di, int tiles, int nchunk, int len) {
+    const T *__restrict__ Bm, const T *__restrict__ Cm, int64_t bc_stride,
+    const float *__restrict__ a_neg, float *__restrict__ h0copy, float *__restrict__ S,
+    float *__restrict__ sumd, float *__restrict__ Bt, float *__restrict__ Cf, int batch, int Tlen,
+    int di, int tiles, int nchunk, int len, int n_state_blocks) {
+    using raw_t = typename RawElem<T>::type;
+    if ((int)blockIdx.x >= n_state_blocks) {
+        // 64 rows of B and C as f32: lane = (row % 4, column).  B is regrouped so that the four
+        // values a lane feeds to the outer-product MFMAs of pass B are one 16-byte load.
+        const int64_t rows = (int64_t)batch * Tlen;
+        const int64_t r0 = (int64_t)(blockIdx.x - n_state_blocks) * 64;
+        const int col = threadIdx.x & 15, sub = threadIdx.x >> 4;
+#pragma unroll 4
+        for (int k = 0; k < 16; k++) {
+            const int64_t r = r0 + 4 * k + sub;
+            if (r < rows) {
+                Bt[r * 16 + (col & 3) * 4 + (col >> 2)] = Store<T>::ld(Bm + r * bc_stride + col);
+                if (sizeof(T) != 4) Cf[r * 16 + col] = Store<T>::ld(Cm + r * bc_stride + col);
+            }
+        }
+        return;
+    }
     const int nc1 = nchunk - 1;
     const int tile = blockIdx.x % tiles;
     const int rest = blockIdx.x / tiles;
     const int c = rest % nc1;
     const int b = rest / nc1;
-    const int d = tile * kWave + threadIdx.x;
-    const bool live = d < di;
-    const int dd = live ? d : di - 1;
+    const int d0 = tile * kWave;
+    const bool live = d0 + (int)threadIdx.x < di;
+    const unsigned lx = live ? threadIdx.x : (unsigned)(di - 1 - d0);  // dead lanes shadow the last live channel
+    const int dd = d0 + (int)lx;
+    const unsigned lxb = lx * (unsigned)sizeof(T);
 
     float hs[16], a2[16];
+    load_a2<S4D>(a2, a_neg, dd);
 #pragma unroll
-    for (int j = 0; j < 16; j++) {
-        a2[j] = a_neg[(int64_t)dd * 16 + j] * kLog2e;
-        hs[j] = 0.0f;
-    }
-    if (S4D) {
-#pragma unroll
-        for (int j = 1; j < 16; j++) a2[j] = a2[0] * (float)(j + 1);
-    }
+    for (int j = 0; j < 16; j++) hs[j] = 0.0f;
     if (c == 0) {
 #pragma unroll
         for (int j = 0; j < 16; j++) {
             hs[j] = h[((int64_t)b * di + dd) * 16 + j];
-            if (live) h0copy[((int64_t)b * 16 + j) * di + d] = hs[j];
+            if (live) h0copy[((int64_t)b * 16 + j) * di + dd] = hs[j];
         }
     }
     const int t0 = c * len, t1 = min(Tlen, t0 + len);
-    float sd = 0.0f;
     const int64_t row0 = (int64_t)b * Tlen;
-#pragma unroll 2
-    for (int t = t0; t < t1; t++) {
-        const int64_t row = row0 + t;
-        const float dl = Store<T>::ld(delta + row * di + dd);
-        const float uu = Store<T>::ld(u + row * di + dd);
-        const float du = dl * uu;
-        float Bv[16], da[16];
-        Row16<T>::ld(Bm + row * bc_stride, Bv);
-        decay16<S4D>(dl, a2, da);
-        sd += dl;
+    const int64_t slab = (int64_t)Tlen * di - d0;  // elements from this wave's base to the end of batch row b
+    const LaneBuf<T> dbuf(delta + row0 * di + d0, slab), ubuf(u + row0 * di + d0, slab);
+    const unsigned row_bytes = (unsigned)di * (unsigned)sizeof(T);
+    const T *Bp = Bm + row0 * bc_stride;
+    float sd = 0.0f;
+
+    raw_t rdA[kGroup], ruA[kGroup], rdB[kGroup], ruB[kGroup];
+    auto load_group = [&](raw_t (&rd)[kGroup], raw_t (&ru)[kGroup], int tg) {
 #pragma unroll
-        for (int j = 0; j < 16; j++) {
-            hs[j] *= da[j];
-            hs[j] = fmaf(du, Bv[j], hs[j]);
+        for (int k = 0; k < kGroup; k++) {
+            const unsigned off = (unsigned)min(tg + k, t1 - 1) * row_bytes;
+            rd[k] = dbuf.ld(lxb, off);
+            ru[k] = ubuf.ld(lxb, off);
         }
+    };
+    RowRaw<T> curB;
+    row_ld(Bp + (int64_t)t0 * bc_stride, curB);
+    auto compute_group = [&](const raw_t (&rd)[kGroup], const raw_t (&ru)[kGroup], int tg) {
+#pragma unroll
+        for (int k = 0; k < kGroup; k++) {
+            const int t = tg + k;
+            if (t < t1) {
+                RowRaw<T> nxtB;
+                row_ld(Bp + (int64_t)min(t + 1, t1 - 1) * bc_stride, nxtB);
+                const float dl = widen(rd[k], (const T *)nullptr);
+                const float uu = widen(ru[k], (const T *)nullptr);
+                const float du = dl * uu;
+                float Bv[16], da[16];
+                row_unpack(curB, Bv, (const T *)nullptr);
+                decay16<S4D>(dl, a2, da);
+                sd += dl;
+#pragma unroll
+                for (int j = 0; j < 16; j++) {
+                    hs[j] *= da[j];
+                    hs[j] = fmaf(du, Bv[j], hs[j]);
+                }
+                curB = nxtB;
+            }
+        }
+    };
+    load_group(rdA, ruA, t0);
+    for (int tg = t0; tg < t1; tg += 2 * kGroup) {
+        load_group(rdB, ruB, tg + kGroup);
+        compute_group(rdA, ruA, tg);
+        load_group(rdA, ruA, tg + 2 * kGroup);
+        compute_group(rdB, ruB, tg + kGroup);
     }
     if (live) {
         const int64_t sbase = (int64_t)b * nc1 + c;
 #pragma unroll
-        for (int j = 0; j < 16; j++) S[(sbase * 16 + j) * di + d] = hs[j];
-        sumd[sbase * di + d] = sd;
+        for (int j = 0; j < 16; j++) S[(sbase * 16 + j) * di + dd] = hs[j];
+        sumd[sbase * di + dd] = sd;
     }
 }
 
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+// Bt: regrouped f32 B rows from pass A; Cf: f32 C rows of stride cf_stride (the widened
+// copy, or the caller's rows at f32 storage).
+//
+// The rank-1 update h[n] += (delta*u)[channel] * B[n] of a wave is an outer product
+// (64 channels) x (16 states): four v_mfma_f32_4x4x1 (16 blocks of 4x4, K = 1) do it on
+// the matrix core with the decayed state as the accumulator -- lane l receives, in
+// result register i, A(lane 4*(l/4)+i) * B(lane l) + C: A carries B[4q+i], B carries the
+// lane's own delta*u -- which takes 16 multiply-adds per step off the vector ALU.
 template <typename T, bool S4D, int GATE>
 __global__ __launch_bounds__(kWave) void chunk_out_kernel(
     float *__restrict__ h, T *__restrict__ y, const T *__restrict__ delta, const T *__restrict__ u,
-    const T *__restrict__ Bm, const T *__restrict__ Cm, int64_t bc_stride,
+    const float *__restrict__ Bt, const float *__restrict__ Cf, int64_t cf_stride,
     const float *__restrict__ a_neg, const float *__restrict__ Dp, const T *__restrict__ gate,
     const float *__restrict__ h0copy, const float *__restrict__ S, const float *__restrict__ sumd,
     int Tlen, int di, int tiles, int nchunk, int len) {
+    using raw_t = typename RawElem<T>::type;
     const int tile = blockIdx.x % tiles;
     const int rest = blockIdx.x / tiles;
     const int c = rest % nchunk;
     const int b = rest / nchunk;
-    const int d = tile * kWave + threadIdx.x;
-    const bool live = d < di;
-    const int dd = live ? d : di - 1;
+    const int d0 = tile * kWave;
+    const bool live = d0 + (int)threadIdx.x < di;
+    const unsigned lx = live ? threadIdx.x : (unsigned)(di - 1 - d0);
+    const int dd = d0 + (int)lx;
+    const unsigned lxb = lx * (unsigned)sizeof(T);
 
     float hs[16], a2[16];
-#pragma unroll
-    for (int j = 0; j < 16; j++) a2[j] = a_neg[(int64_t)dd * 16 + j] * kLog2e;
-    if (S4D) {
-#pragma unroll
-        for (int j = 1; j < 16; j++) a2[j] = a2[0] * (float)(j + 1);
-    }
+    load_a2<S4D>(a2, a_neg, dd);
     if (c == 0) {
 #pragma unroll
         for (int j = 0; j < 16; j++) hs[j] = h0copy[((int64_t)b * 16 + j) * di + dd];
@@ -313,35 +426,75 @@ __global__ __launch_bounds__(kWave) void chunk_out_kernel(
     const float Dd = Dp[dd];
     const int t0 = c * len, t1 = min(Tlen, t0 + len);
     const int64_t row0 = (int64_t)b * Tlen;
-#pragma unroll 2
-    for (int t = t0; t < t1; t++) {
-        const int64_t row = row0 + t;
-        const int64_t i = row * di + dd;
-        const float dl = Store<T>::ld(delta + i);
-        const float uu = Store<T>::ld(u + i);
-        float g = 1.0f;
-        if (GATE) g = Store<T>::ld(gate + i);
-        const float du = dl * uu;
-        float Bv[16], Cv[16], da[16];
-        Row16<T>::ld(Bm + row * bc_stride, Bv);
-        Row16<T>::ld(Cm + row * bc_stride, Cv);
-        decay16<S4D>(dl, a2, da);
-        float acc = Dd * uu;
+    const int64_t slab = (int64_t)Tlen * di - d0;
+    const LaneBuf<T> dbuf(delta + row0 * di + d0, slab), ubuf(u + row0 * di + d0, slab);
+    const LaneBuf<T> gbuf(GATE ? gate + row0 * di + d0 : delta, GATE ? slab : 0), ybuf(y + row0 * di + d0, slab);
+    const unsigned row_bytes = (unsigned)di * (unsigned)sizeof(T);
+    const __amdgpu_buffer_rsrc_t btbuf =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(Bt + row0 * 16), 0, (int)((int64_t)Tlen * 64), 0x00020000);
+    const unsigned bt_lane = (threadIdx.x & 3) * 16;  // this lane's 4 floats inside a regrouped row
+    const float *Cp = Cf + row0 * cf_stride;
+
+    raw_t rdA[kGroup], ruA[kGroup], rgA[kGroup], rdB[kGroup], ruB[kGroup], rgB[kGroup];
+    v4f bvA[kGroup], bvB[kGroup];
+    auto load_group = [&](raw_t (&rd)[kGroup], raw_t (&ru)[kGroup], raw_t (&rg)[kGroup], v4f (&bv)[kGroup], int tg) {
 #pragma unroll
-        for (int j = 0; j < 16; j++) {
-            hs[j] *= da[j];
-            hs[j] = fmaf(du, Bv[j], hs[j]);
-            acc = fmaf(hs[j], Cv[j], acc);
+        for (int k = 0; k < kGroup; k++) {
+            const unsigned tt = (unsigned)min(tg + k, t1 - 1);
+            rd[k] = dbuf.ld(lxb, tt * row_bytes);
+            ru[k] = ubuf.ld(lxb, tt * row_bytes);
+            if (GATE) rg[k] = gbuf.ld(lxb, tt * row_bytes);
+            bv[k] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(btbuf, bt_lane, tt * 64u, 0));
         }
-        if (GATE == 1) acc *= g;
-        if (GATE == 2) acc *= silu(g);
-        if (live) Store<T>::st(y + i, acc);
+    };
+    RowRaw<float> curC;
+    row_ld(Cp + (int64_t)t0 * cf_stride, curC);
+    auto compute_group = [&](const raw_t (&rd)[kGroup], const raw_t (&ru)[kGroup], const raw_t (&rg)[kGroup],
+                             const v4f (&bv)[kGroup], int tg) {
+#pragma unroll
+        for (int k = 0; k < kGroup; k++) {
+            const int t = tg + k;
+            if (t < t1) {
+                RowRaw<float> nxtC;
+                row_ld(Cp + (int64_t)min(t + 1, t1 - 1) * cf_stride, nxtC);
+                const float dl = widen(rd[k], (const T *)nullptr);
+                const float uu = widen(ru[k], (const T *)nullptr);
+                const float du = dl * uu;
+                float da[16];
+                decay16<S4D>(dl, a2, da);
+                float acc = Dd * uu;
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    v4f hq = {hs[4 * q] * da[4 * q], hs[4 * q + 1] * da[4 * q + 1], hs[4 * q + 2] * da[4 * q + 2],
+                              hs[4 * q + 3] * da[4 * q + 3]};
+                    hq = __builtin_amdgcn_mfma_f32_4x4x1f32(bv[k][q], du, hq, 0, 0, 0);
+#pragma unroll
+                    for (int i = 0; i < 4; i++) hs[4 * q + i] = hq[i];
+                }
+#pragma unroll
+                for (int j = 0; j < 16; j++) acc = fmaf(hs[j], curC.w[j], acc);
+                if (GATE == 1) acc *= widen(rg[k], (const T *)nullptr);
+                if (GATE == 2) acc *= silu(widen(rg[k], (const T *)nullptr));
+                if (live) ybuf.st(acc, lxb, (unsigned)t * row_bytes);
+                curC = nxtC;
+            }
+        }
+    };
+    load_group(rdA, ruA, rgA, bvA, t0);
+    for (int tg = t0; tg < t1; tg += 2 * kGroup) {
+        load_group(rdB, ruB, rgB, bvB, tg + kGroup);
+        compute_group(rdA, ruA, rgA, bvA, tg);
+        load_group(rdA, ruA, rgA, bvA, tg + 2 * kGroup);
+        compute_group(rdB, ruB, rgB, bvB, tg + kGroup);
     }
     if (c == nchunk - 1 && live) {
 #pragma unroll
-        for (int j = 0; j < 16; j++) h[((int64_t)b * di + d) * 16 + j] = hs[j];
+        for (int j = 0; j < 16; j++) h[((int64_t)b * di + dd) * 16 + j] = hs[j];
     }
 }
+
+template <typename T> struct IsF32 { static constexpr bool value = false; };
+template <> struct IsF32<float> { static constexpr bool value = true; };
 
 template <typename T, bool S4D>
 static int launch_split_s4d(hipStream_t st, int gate_mode, float *h, T *y, const T *delta, const T *u,
@@ -350,18 +503,20 @@ static int launch_split_s4d(hipStream_t st, int gate_mode, float *h, T *y, const
                             int Tlen, int di) {
     const int tiles = (di + kWave - 1) / kWave;
     const int C = plan.nchunk, L = plan.len;
-    float *h0copy = ws;
-    float *S = h0copy + (size_t)batch * 16 * di;
-    float *sumd = S + (size_t)batch * (C - 1) * 16 * di;
+    const SplitWs w = carve_workspace(ws, batch, Tlen, di, C);
+    const int n_state = batch * (C - 1) * tiles;
+    const int n_widen = (int)(((int64_t)batch * Tlen + 63) / 64);
     const dim3 block(kWave);
-    const dim3 gridA((unsigned)(batch * (C - 1) * tiles)), gridB((unsigned)(batch * C * tiles));
-    hipLaunchKernelGGL((chunk_state_kernel<T, S4D>), gridA, block, 0, st, h, delta, u, Bm, bc_stride, a_neg,
-                       h0copy, S, sumd, Tlen, di, tiles, C, L);
+    const dim3 gridA((unsigned)(n_state + n_widen)), gridB((unsigned)(batch * C * tiles));
+    hipLaunchKernelGGL((chunk_state_kernel<T, S4D>), gridA, block, 0, st, h, delta, u, Bm, Cm, bc_stride, a_neg,
+                       w.h0copy, w.S, w.sumd, w.Bt, w.Cf, batch, Tlen, di, tiles, C, L, n_state);
     int rc = check_launch("chunk_state_kernel");
     if (rc) return rc;
+    const float *Cf = IsF32<T>::value ? reinterpret_cast<const float *>(Cm) : w.Cf;
+    const int64_t bcf = IsF32<T>::value ? bc_stride : 16;
 #define MRS_LAUNCH(G)                                                                                   \
-    hipLaunchKernelGGL((chunk_out_kernel<T, S4D, G>), gridB, block, 0, st, h, y, delta, u, Bm, Cm,      \
-                       bc_stride, a_neg, D, gate, h0copy, S, sumd, Tlen, di, tiles, C, L)
+    hipLaunchKernelGGL((chunk_out_kernel<T, S4D, G>), gridB, block, 0, st, h, y, delta, u, w.Bt, Cf, bcf, \
+                       a_neg, D, gate, w.h0copy, w.S, w.sumd, Tlen, di, tiles, C, L)
     if (gate_mode == 0) MRS_LAUNCH(0);
     else if (gate_mode == 1) MRS_LAUNCH(1);
     else MRS_LAUNCH(2);
@@ -379,6 +534,10 @@ static int launch_split(hipStream_t st, bool s4d, int gate_mode, float *h, void 
         a_neg, D, (const T *)gate, ws, plan, batch, Tlen, di
     return s4d ? launch_split_s4d<T, true>(MRS_ARGS) : launch_split_s4d<T, false>(MRS_ARGS);
 #undef MRS_ARGS
+}
+
+static size_t split_workspace_bytes(int batch, int Tlen, int di, int nchunk) {
+    return carve_workspace(nullptr, batch, Tlen, di, nchunk).floats * sizeof(float);
 }
 
 static int scan_check(const char *fn, int dtype, const void *h, const void *y, const void *delta,
@@ -405,7 +564,7 @@ extern "C" size_t mrs_ssm_scan_workspace_bytes(int batch, int T, int d_inner, in
     if (batch < 1 || T < 1 || d_inner < 1 || d_state != 16) return 256;
     const SplitPlan plan = make_split_plan(batch, T, d_inner);
     if (plan.nchunk < 2) return 256;
-    const size_t bytes = split_workspace_floats(batch, d_inner, plan.nchunk) * sizeof(float);
+    const size_t bytes = split_workspace_bytes(batch, T, d_inner, plan.nchunk);
     return (bytes + 255) & ~(size_t)255;
 }
 
@@ -439,7 +598,7 @@ extern "C" int mrs_ssm_scan_fwd_ex(void *stream, int dtype, float *h, void *y, c
     if ((flags & MRS_FORCE_PARALLEL) && !split && d_state == 16 && T >= 64)
         return fail(MRS_E_WORKSPACE, "mrs_ssm_scan_fwd_ex: MRS_FORCE_PARALLEL needs a workspace and 4-byte aligned B/C rows");
     if (split) {
-        const size_t need = split_workspace_floats(batch, d_inner, plan.nchunk) * sizeof(float);
+        const size_t need = split_workspace_bytes(batch, T, d_inner, plan.nchunk);
         if (workspace_bytes < need)
             return fail(MRS_E_WORKSPACE, "mrs_ssm_scan_fwd_ex: workspace %zu bytes < %zu needed", workspace_bytes, need);
         if (!aligned(workspace, 256)) return fail(MRS_E_ALIGN, "mrs_ssm_scan_fwd_ex: workspace must be 256-byte aligned");
