@@ -140,6 +140,54 @@ MRS_API int mrs_conv1d_seq_silu(void *stream, int dtype, void *u_out, float *sta
                         int64_t x_stride, const float *weight, const float *bias,
                         int batch, int T, int d_inner, int d_conv);
 
+/* ---- Mamba-3 SISO trapezoidal scan --------------------------------------------
+ * State of one layer (all f32, mutated in place): ssm_state [batch,nheads,headdim,d_state],
+ * k_state [batch,nheads,d_state] (previous K after bias+RoPE), v_state [batch,nheads,headdim]
+ * (previous x).  d_inner = nheads*headdim.
+ *
+ * m3_step_fwd_{..} (kernels/mamba3_ssd.cu:56-215; src/mamba3_siso/gpu/inference.rs:756-784),
+ * order ssm,k,v,y,x,k_cur,q_cur,alpha,beta,gamma,D,batch,nh,hd,ds:
+ *   x,y [batch,d_inner] dtype; k_cur,q_cur [batch,nheads,d_state] dtype;
+ *   alpha,beta,gamma [batch,nheads] f32; D [nheads] f32.
+ * headdim <= 1024 and d_state <= 256 (the reference stops at headdim 32, d_state 64). */
+MRS_API int mrs_m3_step(void *stream, int dtype, float *ssm_state, float *k_state, float *v_state, void *y,
+                        const void *x, const void *k_cur, const void *q_cur, const float *alpha,
+                        const float *beta, const float *gamma, const float *D, int batch, int nheads,
+                        int headdim, int d_state);
+
+/* m3_burnin_fwd_nosave_{..} (kernels/mamba3_ssd.cu:453-546; src/mamba3_siso/gpu/forward.rs:423-455):
+ * the same recurrence over T steps, state carried in and out.
+ *   x,y [batch,T,d_inner]; k,q [batch,T,nheads,d_state]; alpha,beta,gamma [batch,T,nheads]. */
+MRS_API int mrs_m3_seq_fwd(void *stream, int dtype, float *ssm_state, float *k_state, float *v_state,
+                           void *y, const void *x, const void *k, const void *q, const float *alpha,
+                           const float *beta, const float *gamma, const float *D, int batch, int T,
+                           int nheads, int headdim, int d_state);
+
+/* m3_compute_abg (kernels/mamba3_ops.cu:735-753): alpha = exp(a_val*dt), beta = alpha*dt*(1-trap),
+ * gamma = trap*dt over n = batch*T*nheads f32 elements (trap already sigmoided, a_val <= 0). */
+MRS_API int mrs_m3_compute_abg(void *stream, float *alpha, float *beta, float *gamma, const float *dt,
+                               const float *a_val, const float *trap, int64_t n);
+
+/* Chunked SSD forward: one call for the reference's adt product + m3_preprocess_chunks +
+ * m3_dA_cumsum + m3_chunk_state_fwd + m3_state_passing_fwd + m3_chunk_scan_fwd +
+ * m3_writeback_parallel_states (kernels/mamba3_chunked.cu:57-419, 1050-1242;
+ * src/mamba3_siso/gpu/forward.rs:257-421).
+ *   x,y [batch,T,d_inner] dtype; K,Q [batch,T,nheads,d_state] dtype (after bias+RoPE);
+ *   dt, trap (sigmoided), a_val [batch,T,nheads] f32; D [nheads] f32.
+ * flags = 0 is the reference's stateless window: the entering ssm/k/v state is ignored
+ * (chunk 0 starts from zero, kernels/mamba3_chunked.cu:219-223) and the final state is
+ * written back.  MRS_M3_CARRY_STATE continues from the entering state instead (prefill
+ * after an earlier window, handing over to mrs_m3_step); the reference has no such mode.
+ * chunk_size must be 64; headdim and d_state multiples of 16 with headdim <= 64, d_state <= 64
+ * for the matrix-core path -- other shapes are refused (use mrs_m3_seq_fwd). */
+enum { MRS_M3_CARRY_STATE = 1u << 0 };
+MRS_API size_t mrs_m3_ssd_workspace_bytes(int batch, int T, int nheads, int headdim, int d_state, int chunk_size);
+MRS_API int mrs_m3_ssd_fwd(void *stream, int dtype, float *ssm_state, float *k_state, float *v_state, void *y,
+                           const void *x, const void *K, const void *Q, const float *dt, const float *trap,
+                           const float *a_val, const float *D, void *workspace, size_t workspace_bytes,
+                           unsigned flags, int batch, int T, int nheads, int headdim, int d_state,
+                           int chunk_size);
+
 #ifdef __cplusplus
 }
 #endif

@@ -36,6 +36,12 @@ _SIGNATURES = {
                                          c_int, c_int, c_int]),
     "mrs_conv1d_step": (c_int, [_P, c_int, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int]),
     "mrs_conv1d_seq_silu": (c_int, [_P, c_int, _P, _P, _P, c_int64, _P, _P, c_int, c_int, c_int, c_int]),
+    "mrs_m3_step": (c_int, [_P, c_int, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int]),
+    "mrs_m3_seq_fwd": (c_int, [_P, c_int, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int]),
+    "mrs_m3_compute_abg": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int64]),
+    "mrs_m3_ssd_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int, c_int]),
+    "mrs_m3_ssd_fwd": (c_int, [_P, c_int, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, c_size_t, c_uint,
+                               c_int, c_int, c_int, c_int, c_int, c_int]),
 }
 
 _lib = None

@@ -1,0 +1,384 @@
+// Mamba-3 SISO chunked SSD forward on the matrix cores.
+//
+// Replaces the reference's six-kernel pipeline m3_preprocess_chunks / m3_dA_cumsum /
+// m3_chunk_state_fwd / m3_state_passing_fwd / m3_chunk_scan_fwd /
+// m3_writeback_parallel_states (kernels/mamba3_chunked.cu:57-419) with ONE kernel:
+// a workgroup owns a (batch row, head) and walks its 64-step chunks in order, so the
+// inter-chunk state never leaves registers, K_scaled / qk_dot / dA_cumsum / chunk states
+// are never written to memory, and Q, K, x are read once and y written once.
+//
+// Per chunk (t, s index the 64 steps, n the state, p the head dimension):
+//   G^T[s,t] = sum_n K[s,n] Q[t,n]                                   (MFMA, K = n)
+//   P[t,s]   = G[t,s] scale[s] exp(dA[t]-dA[s])   (s <  t)
+//            = D + gamma[t] G[t,t]                (s == t)  -- the D / qk_dot skip term
+//            = 0                                  (s >  t)
+//   y[t,p]   = exp(dA[t]) sum_n Q[t,n] S[p,n]  +  sum_s P[t,s] x[s,p]   (MFMA, K = n then K = s)
+//   S^T[n,p] = exp(dA_end) S^T[n,p] + sum_t K[t,n] (w[t] x[t,p]),  w[t] = exp(dA_end-dA[t]) scale[t]
+// with gamma = dt trap, scale[t] = gamma[t] + dt[t+1](1-trap[t+1]), dA = cumsum(a dt) in the chunk.
+//
+// Wave w of the workgroup owns the 16 columns p in [16w, 16w+16) of y and of the state.
+// Operand layouts are chosen so that no accumulator is ever transposed: G is produced
+// transposed (A = K rows, B = Q rows) which leaves P directly in A-operand layout, and the
+// state is kept as S^T accumulator tiles, which is B-operand layout for Q S^T.
+// v_mfma_f32_16x16x16 (bf16 or f16 inputs, f32 accumulate): lane l holds A[m=l%16][k=4(l/16)..+3],
+// B[k=4(l/16)..+3][n=l%16], and C/D[m=4(l/16)+i][n=l%16], i = 0..3.
+#include "common.hpp"
+
+namespace mrs {
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef short v4s __attribute__((ext_vector_type(4)));
+typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+
+constexpr int kCS = 64;  // chunk size (the reference's CHUNK_SIZE, src/mamba3_siso/gpu/state.rs:97)
+constexpr int kPad = 8;  // halfword padding of LDS rows (keeps rows 16-byte aligned, staggers banks)
+
+template <typename T> struct Mma;
+template <> struct Mma<bf16_t> {
+    __device__ static __forceinline__ v4f mma(uint2 a, uint2 b, v4f c) {
+        return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(v4s, a), __builtin_bit_cast(v4s, b), c, 0, 0, 0);
+    }
+    __device__ static __forceinline__ uint2 pack(float a, float b, float c, float d) {
+        typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+        b2 lo = {(__bf16)a, (__bf16)b}, hi = {(__bf16)c, (__bf16)d};
+        return make_uint2(__builtin_bit_cast(unsigned, lo), __builtin_bit_cast(unsigned, hi));
+    }
+    __device__ static __forceinline__ void unpack(uint2 v, float (&o)[4]) {
+        o[0] = __uint_as_float(v.x << 16); o[1] = __uint_as_float(v.x & 0xffff0000u);
+        o[2] = __uint_as_float(v.y << 16); o[3] = __uint_as_float(v.y & 0xffff0000u);
+    }
+};
+template <> struct Mma<f16_t> {
+    __device__ static __forceinline__ v4f mma(uint2 a, uint2 b, v4f c) {
+        return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(v4h, a), __builtin_bit_cast(v4h, b), c, 0, 0, 0);
+    }
+    __device__ static __forceinline__ uint2 pack(float a, float b, float c, float d) {
+        v4h v = {(_Float16)a, (_Float16)b, (_Float16)c, (_Float16)d};
+        return __builtin_bit_cast(uint2, v);
+    }
+    __device__ static __forceinline__ void unpack(uint2 v, float (&o)[4]) {
+        const v4h h = __builtin_bit_cast(v4h, v);
+        o[0] = (float)h.x; o[1] = (float)h.y; o[2] = (float)h.z; o[3] = (float)h.w;
+    }
+};
+
+template <int HD, int DS> struct alignas(16) SsdSmem {
+    static constexpr int NW = HD / 16;
+    alignas(16) uint16_t Qs[kCS][DS + kPad];       // Q rows
+    alignas(16) uint16_t Ks[kCS][DS + kPad];       // K rows
+    alignas(16) uint16_t Kt[DS][kCS + kPad];       // K transposed: Kt[n][t]
+    alignas(16) uint16_t Xt[NW][16][kCS + kPad];   // per wave: x slice transposed, Xt[p][t]
+    alignas(16) float sc[NW][5][kCS];              // per wave: dA, scale, gamma, exp(dA), w
+};
+
+template <typename T, int HD, int DS>
+__global__ __launch_bounds__(HD * 4) void m3_ssd_kernel(
+    float *__restrict__ ssm, float *__restrict__ kst, float *__restrict__ vst, T *__restrict__ y,
+    const T *__restrict__ x, const T *__restrict__ K, const T *__restrict__ Q,
+    const float *__restrict__ dt, const float *__restrict__ trap, const float *__restrict__ a_val,
+    const float *__restrict__ Dp, int Tlen, int nh, int carry) {
+    constexpr int NW = HD / 16, NTHR = NW * 64, KN = DS / 16;
+    constexpr int VPR = DS / 8;                    // 16-byte vectors per Q/K row
+    constexpr int NVEC = kCS * VPR;                // vectors per tile
+    constexpr int NV = (NVEC + NTHR - 1) / NTHR;   // vectors per thread per tile
+    __shared__ SsdSmem<HD, DS> sm;
+
+    const int b = blockIdx.x / nh, h = blockIdx.x - b * nh;
+    const int tid = threadIdx.x, w = tid >> 6, l = tid & 63;
+    const int lr = l & 15, lg = l >> 4;            // fragment row/col index and k-group
+    const int di = nh * HD;
+    const int64_t bh = (int64_t)b * nh + h;
+    const float Dh = Dp[h];
+    const int nchunks = (Tlen + kCS - 1) / kCS;
+
+    // ---- running state S^T as accumulator tiles: lane holds S[p=16w+lr][n=16jn+4lg+i] ----
+    v4f St[KN];
+#pragma unroll
+    for (int jn = 0; jn < KN; jn++) St[jn] = (v4f){0.f, 0.f, 0.f, 0.f};
+    if (carry) {
+        const int64_t t0row = (int64_t)b * Tlen * nh + h;
+        const float sgm1 = dt[t0row] * (1.0f - trap[t0row]);
+        const float vin = vst[bh * HD + 16 * w + lr];
+#pragma unroll
+        for (int jn = 0; jn < KN; jn++) {
+            const float4 s = *reinterpret_cast<const float4 *>(ssm + (bh * HD + 16 * w + lr) * DS + 16 * jn + 4 * lg);
+            const float4 kin = *reinterpret_cast<const float4 *>(kst + bh * DS + 16 * jn + 4 * lg);
+            St[jn] = (v4f){fmaf(sgm1 * vin, kin.x, s.x), fmaf(sgm1 * vin, kin.y, s.y), fmaf(sgm1 * vin, kin.z, s.z),
+                           fmaf(sgm1 * vin, kin.w, s.w)};
+        }
+    }
+
+    // ---- global -> register prefetch of one chunk ----
+    uint4 rq[NV], rk[NV], rx[2];
+    float rdt, rtr, ra, ndt0, ntr0;
+    auto prefetch = [&](int c) {
+        const int t0 = c * kCS;
+#pragma unroll
+        for (int v = 0; v < NV; v++) {
+            const int vi = tid + v * NTHR, row = vi / VPR, col = (vi % VPR) * 8;
+            const int t = t0 + row;
+            if (vi < NVEC && t < Tlen) {
+                const int64_t off = (((int64_t)b * Tlen + t) * nh + h) * DS + col;
+                rq[v] = *reinterpret_cast<const uint4 *>(Q + off);
+                rk[v] = *reinterpret_cast<const uint4 *>(K + off);
+            } else {
+                rq[v] = make_uint4(0, 0, 0, 0);
+                rk[v] = make_uint4(0, 0, 0, 0);
+            }
+        }
+        const int t = t0 + l;  // lane = step
+        if (t < Tlen) {
+            const int64_t xo = ((int64_t)b * Tlen + t) * di + h * HD + 16 * w;
+            rx[0] = *reinterpret_cast<const uint4 *>(x + xo);
+            rx[1] = *reinterpret_cast<const uint4 *>(x + xo + 8);
+            const int64_t so = ((int64_t)b * Tlen + t) * nh + h;
+            rdt = dt[so]; rtr = trap[so]; ra = a_val[so];
+        } else {
+            rx[0] = make_uint4(0, 0, 0, 0); rx[1] = make_uint4(0, 0, 0, 0);
+            rdt = 0.f; rtr = 0.f; ra = 0.f;
+        }
+        const int tn = t0 + kCS;  // first step of the next chunk, for the shifted gamma of step 63
+        if (tn < Tlen) {
+            const int64_t so = ((int64_t)b * Tlen + tn) * nh + h;
+            ndt0 = dt[so]; ntr0 = trap[so];
+        } else { ndt0 = 0.f; ntr0 = 1.f; }
+    };
+
+    prefetch(0);
+    for (int c = 0; c < nchunks; c++) {
+        const int t0 = c * kCS;
+        __syncthreads();  // every wave is done reading the previous chunk's tiles
+        // ---- registers -> LDS ----
+#pragma unroll
+        for (int v = 0; v < NV; v++) {
+            const int vi = tid + v * NTHR, row = vi / VPR, col = (vi % VPR) * 8;
+            if (vi >= NVEC) continue;
+            *reinterpret_cast<uint4 *>(&sm.Qs[row][col]) = rq[v];
+            *reinterpret_cast<uint4 *>(&sm.Ks[row][col]) = rk[v];
+            const unsigned kw[4] = {rk[v].x, rk[v].y, rk[v].z, rk[v].w};
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                sm.Kt[col + 2 * j][row] = (uint16_t)(kw[j] & 0xffffu);
+                sm.Kt[col + 2 * j + 1][row] = (uint16_t)(kw[j] >> 16);
+            }
+        }
+        {
+            const unsigned xw[8] = {rx[0].x, rx[0].y, rx[0].z, rx[0].w, rx[1].x, rx[1].y, rx[1].z, rx[1].w};
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                sm.Xt[w][2 * j][l] = (uint16_t)(xw[j] & 0xffffu);
+                sm.Xt[w][2 * j + 1][l] = (uint16_t)(xw[j] >> 16);
+            }
+        }
+        // ---- per-step scalars, lane = step ----
+        float dAend;
+        {
+            float dtn = __shfl_down(rdt, 1, kWave), trn = __shfl_down(rtr, 1, kWave);
+            if (l == 63) { dtn = ndt0; trn = ntr0; }
+            if (t0 + l + 1 >= Tlen) { dtn = 0.f; trn = 1.f; }       // no step after the last one
+            const float gam = rdt * rtr;
+            const float scl = fmaf(dtn, 1.0f - trn, gam);
+            float dA = ra * rdt;
+#pragma unroll
+            for (int m = 1; m < kWave; m <<= 1) {                    // inclusive scan over the 64 steps
+                const float o = __shfl_up(dA, m, kWave);
+                if (l >= m) dA += o;
+            }
+            dAend = __shfl(dA, 63, kWave);
+            sm.sc[w][0][l] = dA;
+            sm.sc[w][1][l] = scl;
+            sm.sc[w][2][l] = gam;
+            sm.sc[w][3][l] = fast_exp2(dA * kLog2e);
+            sm.sc[w][4][l] = fast_exp2((dAend - dA) * kLog2e) * scl;
+        }
+        __syncthreads();  // tiles visible to every wave
+        if (c + 1 < nchunks) prefetch(c + 1);
+
+        // ---- x fragments: lane holds x[t=16kt+4lg+i][p=16w+lr]; also scaled by w[t] for the state update ----
+        uint2 xf[4], xwf[4];
+#pragma unroll
+        for (int kt = 0; kt < 4; kt++) {
+            xf[kt] = *reinterpret_cast<const uint2 *>(&sm.Xt[w][lr][16 * kt + 4 * lg]);
+            const float4 wv = *reinterpret_cast<const float4 *>(&sm.sc[w][4][16 * kt + 4 * lg]);
+            float xv[4];
+            Mma<T>::unpack(xf[kt], xv);
+            xwf[kt] = Mma<T>::pack(xv[0] * wv.x, xv[1] * wv.y, xv[2] * wv.z, xv[3] * wv.w);
+        }
+        // ---- entering state as B-operand fragments (16-bit) ----
+        uint2 Sf[KN];
+#pragma unroll
+        for (int jn = 0; jn < KN; jn++) Sf[jn] = Mma<T>::pack(St[jn][0], St[jn][1], St[jn][2], St[jn][3]);
+
+#pragma unroll
+        for (int it = 0; it < 4; it++) {
+            // Q fragments of this t-tile: lane holds Q[t=16it+lr][n=16kk+4lg..+3]
+            uint2 qf[KN];
+#pragma unroll
+            for (int kk = 0; kk < KN; kk++) qf[kk] = *reinterpret_cast<const uint2 *>(&sm.Qs[16 * it + lr][16 * kk + 4 * lg]);
+            // y_off = exp(dA[t]) * Q S^T     (acc rows t = 16it+4lg+i, cols p = 16w+lr)
+            v4f acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int kk = 0; kk < KN; kk++) acc = Mma<T>::mma(qf[kk], Sf[kk], acc);
+            {
+                const float4 e = *reinterpret_cast<const float4 *>(&sm.sc[w][3][16 * it + 4 * lg]);
+                acc[0] *= e.x; acc[1] *= e.y; acc[2] *= e.z; acc[3] *= e.w;
+            }
+            const float dAt = sm.sc[w][0][16 * it + lr];
+            const float gamt = sm.sc[w][2][16 * it + lr];
+#pragma unroll
+            for (int js = 0; js <= it; js++) {
+                // G^T tile: rows s = 16js+4lg+i, cols t = 16it+lr
+                v4f g = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int kk = 0; kk < KN; kk++) {
+                    const uint2 kf = *reinterpret_cast<const uint2 *>(&sm.Ks[16 * js + lr][16 * kk + 4 * lg]);
+                    g = Mma<T>::mma(kf, qf[kk], g);
+                }
+                const float4 dAs = *reinterpret_cast<const float4 *>(&sm.sc[w][0][16 * js + 4 * lg]);
+                const float4 scs = *reinterpret_cast<const float4 *>(&sm.sc[w][1][16 * js + 4 * lg]);
+                const float das[4] = {dAs.x, dAs.y, dAs.z, dAs.w}, sc4[4] = {scs.x, scs.y, scs.z, scs.w};
+                float pv[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const float dec = fast_exp2((dAt - das[i]) * kLog2e);
+                    pv[i] = g[i] * sc4[i] * dec;
+                    if (js == it) {  // diagonal tile: strict causality, skip term on the diagonal
+                        const int s = 4 * lg + i;
+                        if (s > lr) pv[i] = 0.f;
+                        else if (s == lr) pv[i] = fmaf(gamt, g[i], Dh);
+                    }
+                }
+                const uint2 pf = Mma<T>::pack(pv[0], pv[1], pv[2], pv[3]);  // A operand: P[t=lr][s=4lg+i]
+                acc = Mma<T>::mma(pf, xf[js], acc);
+            }
+            // store y rows t = t0+16it+4lg+i, column p = 16w+lr
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int t = t0 + 16 * it + 4 * lg + i;
+                if (t < Tlen) Store<T>::st(y + ((int64_t)b * Tlen + t) * di + h * HD + 16 * w + lr, acc[i]);
+            }
+        }
+        // ---- state update: S^T[n,p] = exp(dA_end) S^T + K^T (w x) ----
+        const float decay = fast_exp2(dAend * kLog2e);
+#pragma unroll
+        for (int jn = 0; jn < KN; jn++) {
+            v4f s = St[jn] * decay;
+#pragma unroll
+            for (int kt = 0; kt < 4; kt++) {
+                const uint2 ktf = *reinterpret_cast<const uint2 *>(&sm.Kt[16 * jn + lr][16 * kt + 4 * lg]);
+                s = Mma<T>::mma(ktf, xwf[kt], s);
+            }
+            St[jn] = s;
+        }
+    }
+    // ---- write back: ssm <- S, k_state <- K[T-1], v_state <- x[T-1] ----
+#pragma unroll
+    for (int jn = 0; jn < KN; jn++)
+        *reinterpret_cast<float4 *>(ssm + (bh * HD + 16 * w + lr) * DS + 16 * jn + 4 * lg) =
+            make_float4(St[jn][0], St[jn][1], St[jn][2], St[jn][3]);
+    const int64_t last = (int64_t)b * Tlen + (Tlen - 1);
+    for (int n = tid; n < DS; n += NTHR) kst[bh * DS + n] = Store<T>::ld(K + (last * nh + h) * DS + n);
+    for (int p = tid; p < HD; p += NTHR) vst[bh * HD + p] = Store<T>::ld(x + last * di + h * HD + p);
+}
+
+__global__ void m3_abg_kernel(float *__restrict__ alpha, float *__restrict__ beta, float *__restrict__ gamma,
+                              const float *__restrict__ dt, const float *__restrict__ a_val,
+                              const float *__restrict__ trap, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const float d = dt[i], t = trap[i];
+    const float al = fast_exp2(a_val[i] * d * kLog2e);
+    alpha[i] = al;
+    beta[i] = al * d * (1.0f - t);
+    gamma[i] = t * d;
+}
+
+__global__ void zero_kernel(float *__restrict__ p, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0.0f;
+}
+
+template <typename T, int HD, int DS>
+static void launch_ssd_shape(hipStream_t st, float *ssm, float *kst, float *vst, void *y, const void *x,
+                             const void *K, const void *Q, const float *dt, const float *trap,
+                             const float *a_val, const float *D, int batch, int Tlen, int nh, int carry) {
+    hipLaunchKernelGGL((m3_ssd_kernel<T, HD, DS>), dim3((unsigned)(batch * nh)), dim3(HD * 4), 0, st, ssm, kst, vst,
+                       (T *)y, (const T *)x, (const T *)K, (const T *)Q, dt, trap, a_val, D, Tlen, nh, carry);
+}
+
+template <typename T>
+static int launch_ssd(hipStream_t st, float *ssm, float *kst, float *vst, void *y, const void *x, const void *K,
+                      const void *Q, const float *dt, const float *trap, const float *a_val, const float *D,
+                      int batch, int Tlen, int nh, int hd, int ds, int carry) {
+#define MRS_SHAPE(H, S)                                                                                      \
+    if (hd == H && ds == S) {                                                                                \
+        launch_ssd_shape<T, H, S>(st, ssm, kst, vst, y, x, K, Q, dt, trap, a_val, D, batch, Tlen, nh, carry); \
+        return check_launch("m3_ssd_kernel");                                                                \
+    }
+    MRS_SHAPE(64, 64) MRS_SHAPE(64, 32) MRS_SHAPE(64, 16)
+    MRS_SHAPE(32, 64) MRS_SHAPE(32, 32) MRS_SHAPE(32, 16)
+    MRS_SHAPE(16, 64) MRS_SHAPE(16, 32) MRS_SHAPE(16, 16)
+#undef MRS_SHAPE
+    return fail(MRS_E_SHAPE, "mrs_m3_ssd_fwd: headdim=%d d_state=%d not in {16,32,64}x{16,32,64}", hd, ds);
+}
+
+}  // namespace mrs
+
+using namespace mrs;
+
+extern "C" int mrs_m3_compute_abg(void *stream, float *alpha, float *beta, float *gamma, const float *dt,
+                                  const float *a_val, const float *trap, int64_t n) {
+    if (!alpha || !beta || !gamma || !dt || !a_val || !trap) return fail(MRS_E_NULL, "mrs_m3_compute_abg: null pointer");
+    if (n < 1 || n > 0x7fffffffLL * 256) return fail(MRS_E_SHAPE, "mrs_m3_compute_abg: n=%lld", (long long)n);
+    hipLaunchKernelGGL(m3_abg_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, as_stream(stream), alpha, beta, gamma,
+                       dt, a_val, trap, n);
+    return check_launch("m3_abg_kernel");
+}
+
+extern "C" size_t mrs_m3_ssd_workspace_bytes(int batch, int T, int nheads, int headdim, int d_state, int chunk_size) {
+    (void)headdim; (void)d_state; (void)chunk_size;
+    if (batch < 1 || T < 1 || nheads < 1) return 256;
+    // alpha, beta, gamma for the f32-storage route (sequential kernel)
+    const size_t n = (size_t)batch * T * nheads;
+    return ((3 * n * sizeof(float)) + 255) & ~(size_t)255;
+}
+
+extern "C" int mrs_m3_ssd_fwd(void *stream, int dtype, float *ssm_state, float *k_state, float *v_state, void *y,
+                              const void *x, const void *K, const void *Q, const float *dt, const float *trap,
+                              const float *a_val, const float *D, void *workspace, size_t workspace_bytes,
+                              unsigned flags, int batch, int T, int nheads, int headdim, int d_state,
+                              int chunk_size) {
+    const char *fn = "mrs_m3_ssd_fwd";
+    if (dtype != MRS_F32 && dtype != MRS_F16 && dtype != MRS_BF16) return fail(MRS_E_DTYPE, "%s: dtype %d is not f32/f16/bf16", fn, dtype);
+    if (!ssm_state || !k_state || !v_state || !y || !x || !K || !Q || !dt || !trap || !a_val || !D)
+        return fail(MRS_E_NULL, "%s: null pointer", fn);
+    if (batch < 1 || T < 1 || nheads < 1) return fail(MRS_E_SHAPE, "%s: batch=%d T=%d nheads=%d must be >= 1", fn, batch, T, nheads);
+    if (chunk_size != kCS) return fail(MRS_E_SHAPE, "%s: chunk_size=%d, only %d is built", fn, chunk_size, kCS);
+    if (!((headdim == 16 || headdim == 32 || headdim == 64) && (d_state == 16 || d_state == 32 || d_state == 64)))
+        return fail(MRS_E_SHAPE, "%s: headdim=%d d_state=%d not in {16,32,64}x{16,32,64}", fn, headdim, d_state);
+    if ((int64_t)batch * T * nheads * headdim > 0x7fffffffLL) return fail(MRS_E_SHAPE, "%s: batch*T*d_inner exceeds i32", fn);
+    hipStream_t st = as_stream(stream);
+    const int carry = (flags & MRS_M3_CARRY_STATE) ? 1 : 0;
+    if (dtype == MRS_F32) {
+        // f32 storage asks for 1e-4 parity, which 16-bit matrix-core operands cannot give:
+        // run the recurrence itself (alpha/beta/gamma into the workspace, then the sequential kernel).
+        const size_t n = (size_t)batch * T * nheads;
+        if (!workspace || workspace_bytes < 3 * n * sizeof(float))
+            return fail(MRS_E_WORKSPACE, "%s: f32 storage needs a workspace of %zu bytes", fn, 3 * n * sizeof(float));
+        float *al = (float *)workspace, *be = al + n, *ga = be + n;
+        int rc = mrs_m3_compute_abg(stream, al, be, ga, dt, a_val, trap, (int64_t)n);
+        if (rc) return rc;
+        if (!carry) {
+            const int64_t ns = (int64_t)batch * nheads * headdim * d_state, nk = (int64_t)batch * nheads * d_state,
+                          nv = (int64_t)batch * nheads * headdim;
+            hipLaunchKernelGGL(zero_kernel, dim3((unsigned)((ns + 255) / 256)), dim3(256), 0, st, ssm_state, ns);
+            hipLaunchKernelGGL(zero_kernel, dim3((unsigned)((nk + 255) / 256)), dim3(256), 0, st, k_state, nk);
+            hipLaunchKernelGGL(zero_kernel, dim3((unsigned)((nv + 255) / 256)), dim3(256), 0, st, v_state, nv);
+        }
+        return mrs_m3_seq_fwd(stream, dtype, ssm_state, k_state, v_state, y, x, K, Q, al, be, ga, D, batch, T, nheads, headdim, d_state);
+    }
+    if (!aligned(x, 16) || !aligned(K, 16) || !aligned(Q, 16) || !aligned(ssm_state, 16) || !aligned(k_state, 16))
+        return fail(MRS_E_ALIGN, "%s: x, K, Q, ssm_state, k_state must be 16-byte aligned", fn);
+    if (dtype == MRS_BF16) return launch_ssd<bf16_t>(st, ssm_state, k_state, v_state, y, x, K, Q, dt, trap, a_val, D, batch, T, nheads, headdim, d_state, carry);
+    return launch_ssd<f16_t>(st, ssm_state, k_state, v_state, y, x, K, Q, dt, trap, a_val, D, batch, T, nheads, headdim, d_state, carry);
+}

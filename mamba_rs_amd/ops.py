@@ -154,3 +154,64 @@ def conv1d_seq_silu(u_out, state, x_branch, weight, bias):
     _lib.call("mrs_conv1d_seq_silu", _stream(), int(dt), _p(u_out), _p(state), _p(x_branch), x_branch.stride(1),
               _p(weight), _p(bias), batch, T, di, dc)
     return u_out
+
+
+# ----------------------------------------------------------------------------- Mamba-3 SISO
+M3_CARRY_STATE = 1 << 0
+
+
+def m3_compute_abg(dt, a_val, trap):
+    """alpha, beta, gamma from dt, a_val, sigmoided trap (m3_compute_abg, kernels/mamba3_ops.cu:735-753)."""
+    _dev(dt, a_val, trap); _f32(dt, a_val, trap)
+    al, be, ga = torch.empty_like(dt), torch.empty_like(dt), torch.empty_like(dt)
+    _lib.call("mrs_m3_compute_abg", _stream(), _p(al), _p(be), _p(ga), _p(dt), _p(a_val), _p(trap), dt.numel())
+    return al, be, ga
+
+
+def _m3_shapes(ssm, kst, vst, x, k, T_axis: bool):
+    batch, nh, hd, ds = ssm.shape
+    if kst.shape != (batch, nh, ds) or vst.shape != (batch, nh, hd):
+        raise ValueError("state shape mismatch")
+    if T_axis:
+        if x.dim() != 3 or x.shape[0] != batch or x.shape[2] != nh * hd or k.shape != (batch, x.shape[1], nh, ds):
+            raise ValueError("x must be [batch,T,nheads*headdim], k/q [batch,T,nheads,d_state]")
+    else:
+        if x.shape != (batch, nh * hd) or k.shape != (batch, nh, ds):
+            raise ValueError("x must be [batch,nheads*headdim], k/q [batch,nheads,d_state]")
+    return batch, nh, hd, ds
+
+
+def m3_step(ssm, kst, vst, y, x, k_cur, q_cur, alpha, beta, gamma, D):
+    """One decode step of the trapezoidal recurrence (m3_step_fwd, kernels/mamba3_ssd.cu:56-215)."""
+    _dev(ssm, kst, vst, y, x, k_cur, q_cur, alpha, beta, gamma, D); _f32(ssm, kst, vst, alpha, beta, gamma, D)
+    dt = _act_dtype(x, y, k_cur, q_cur)
+    batch, nh, hd, ds = _m3_shapes(ssm, kst, vst, x, k_cur, False)
+    _lib.call("mrs_m3_step", _stream(), int(dt), _p(ssm), _p(kst), _p(vst), _p(y), _p(x), _p(k_cur), _p(q_cur), _p(alpha),
+              _p(beta), _p(gamma), _p(D), batch, nh, hd, ds)
+    return y
+
+
+def m3_seq_fwd(ssm, kst, vst, y, x, k, q, alpha, beta, gamma, D):
+    """T steps, sequential in time, state carried (m3_burnin_fwd_nosave, kernels/mamba3_ssd.cu:453-546)."""
+    _dev(ssm, kst, vst, y, x, k, q, alpha, beta, gamma, D); _f32(ssm, kst, vst, alpha, beta, gamma, D)
+    dt = _act_dtype(x, y, k, q)
+    batch, nh, hd, ds = _m3_shapes(ssm, kst, vst, x, k, True)
+    _lib.call("mrs_m3_seq_fwd", _stream(), int(dt), _p(ssm), _p(kst), _p(vst), _p(y), _p(x), _p(k), _p(q), _p(alpha),
+              _p(beta), _p(gamma), _p(D), batch, x.shape[1], nh, hd, ds)
+    return y
+
+
+def m3_ssd_workspace_bytes(batch, T, nheads, headdim, d_state, chunk_size=64) -> int:
+    return int(_lib.load().mrs_m3_ssd_workspace_bytes(batch, T, nheads, headdim, d_state, chunk_size))
+
+
+def m3_ssd_fwd(ssm, kst, vst, y, x, K, Q, dt, trap, a_val, D, *, carry_state=False, workspace=None, chunk_size=64):
+    """Chunked SSD forward (the six kernels of kernels/mamba3_chunked.cu:57-419 in one call)."""
+    _dev(ssm, kst, vst, y, x, K, Q, dt, trap, a_val, D, workspace); _f32(ssm, kst, vst, dt, trap, a_val, D)
+    adt = _act_dtype(x, y, K, Q)
+    batch, nh, hd, ds = _m3_shapes(ssm, kst, vst, x, K, True)
+    ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    _lib.call("mrs_m3_ssd_fwd", _stream(), int(adt), _p(ssm), _p(kst), _p(vst), _p(y), _p(x), _p(K), _p(Q), _p(dt), _p(trap),
+              _p(a_val), _p(D), _p(workspace), ws_bytes, M3_CARRY_STATE if carry_state else 0, batch, x.shape[1], nh, hd, ds,
+              chunk_size)
+    return y

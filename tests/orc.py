@@ -214,3 +214,117 @@ def m1_zero_state(P: M1Params):
 
 def num_threads():
     return int(lib().orc_num_threads())
+
+
+# ----------------------------------------------------------------------------- Mamba-3
+def m3_abg_f64(dt, a_val, trap):
+    dt = _c(dt); a_val = _c(a_val); trap = _c(trap)
+    al = np.zeros(dt.shape, np.float64); be = np.zeros_like(al); ga = np.zeros_like(al)
+    lib().orc_m3_abg_f64(_p(al), _p(be), _p(ga), _p(dt), _p(a_val), _p(trap), c_int64(dt.size))
+    return al, be, ga
+
+
+def m3_seq_f64(ssm, kst, vst, x, k, q, alpha, beta, gamma, D):
+    """Sequential trapezoid in f64. x [B,T,nh*hd]; k,q [B,T,nh,ds]; alpha.. [B,T,nh] (any float dtype).
+    Returns (y, ssm, kst, vst) as new f64 arrays."""
+    x = _c(x); k = _c(k); q = _c(q); D = _c(D)
+    al = _c(alpha, np.float64); be = _c(beta, np.float64); ga = _c(gamma, np.float64)
+    B, T, nh, ds = k.shape
+    hd = x.shape[2] // nh
+    ssm = np.array(ssm, np.float64, copy=True, order="C"); kst = np.array(kst, np.float64, copy=True, order="C")
+    vst = np.array(vst, np.float64, copy=True, order="C")
+    y = np.zeros(x.shape, np.float64)
+    lib().orc_m3_seq_f64(_p(ssm), _p(kst), _p(vst), _p(y), _p(x), _p(k), _p(q), _p(al), _p(be), _p(ga), _p(D),
+                         c_int64(B), c_int64(T), c_int64(nh), c_int64(hd), c_int64(ds))
+    return y, ssm, kst, vst
+
+
+def m3_seq_gpu(ssm, kst, vst, x, k, q, alpha, beta, gamma, D, dtype=F32):
+    x = _c(x); k = _c(k); q = _c(q); D = _c(D); al = _c(alpha); be = _c(beta); ga = _c(gamma)
+    B, T, nh, ds = k.shape
+    hd = x.shape[2] // nh
+    ssm = np.array(ssm, np.float32, copy=True, order="C"); kst = np.array(kst, np.float32, copy=True, order="C")
+    vst = np.array(vst, np.float32, copy=True, order="C")
+    y = np.zeros(x.shape, np.float32)
+    lib().orc_m3_seq_gpu(_p(ssm), _p(kst), _p(vst), _p(y), _p(x), _p(k), _p(q), _p(al), _p(be), _p(ga), _p(D),
+                         c_int64(B), c_int64(T), c_int64(nh), c_int64(hd), c_int64(ds), c_int(dtype))
+    return y, ssm, kst, vst
+
+
+def m3_chunked_f64(ssm, kst, vst, x, K, Q, dt, trap, a_val, D, chunk, carry=False):
+    x = _c(x); K = _c(K); Q = _c(Q); dt = _c(dt); trap = _c(trap); a_val = _c(a_val); D = _c(D)
+    B, T, nh, ds = K.shape
+    hd = x.shape[2] // nh
+    ssm = np.array(ssm, np.float64, copy=True, order="C"); kst = np.array(kst, np.float64, copy=True, order="C")
+    vst = np.array(vst, np.float64, copy=True, order="C")
+    y = np.zeros(x.shape, np.float64)
+    lib().orc_m3_chunked_f64(_p(ssm), _p(kst), _p(vst), _p(y), _p(x), _p(K), _p(Q), _p(dt), _p(trap), _p(a_val), _p(D),
+                             c_int64(B), c_int64(T), c_int64(nh), c_int64(hd), c_int64(ds), c_int64(chunk),
+                             c_int(1 if carry else 0))
+    return y, ssm, kst, vst
+
+
+class M3Params:
+    """Flat parameter block of Mamba3Weights::init with named views."""
+
+    def __init__(self, dm, ds, expand, hd, ng, n_layers, rope_fraction, input_dim, seed=None, a_floor=1e-4,
+                 outproj_norm=False):
+        self.dm, self.ds, self.expand, self.hd, self.ng, self.n_layers = dm, ds, expand, hd, ng, n_layers
+        self.input_dim, self.a_floor, self.outproj_norm = input_dim, a_floor, outproj_norm
+        self.di = dm * expand
+        self.nh = self.di // hd
+        self.n_rope = int(np.float32(ds) * np.float32(rope_fraction)) // 2
+        self.ip = 2 * self.di + 2 * ng * ds + 3 * self.nh + self.n_rope
+        L = lib()
+        L.orc_m3_param_count.restype = c_int64
+        n = L.orc_m3_param_count(c_int64(dm), c_int64(ds), c_int64(expand), c_int64(hd), c_int64(ng), c_int64(n_layers),
+                                 c_int64(self.n_rope), c_int64(input_dim))
+        flat = np.zeros(n, np.float32)
+        L.orc_m3_weights_init(_p(flat), c_int64(dm), c_int64(ds), c_int64(expand), c_int64(hd), c_int64(ng),
+                              c_int64(n_layers), c_int64(self.n_rope), c_int64(input_dim), c_uint64(seed))
+        self.flat = flat
+        o = 0
+
+        def take(*shape):
+            nonlocal o
+            k = int(np.prod(shape))
+            v = flat[o:o + k].reshape(shape)
+            o += k
+            return v
+
+        di, nh = self.di, self.nh
+        self.input_proj_w = take(input_dim, dm); self.input_proj_b = take(dm)
+        self.layers = []
+        for _ in range(n_layers):
+            self.layers.append(dict(norm_weight=take(dm), in_proj_w=take(dm, self.ip), dt_bias=take(nh), b_norm_weight=take(ds),
+                                    c_norm_weight=take(ds), b_bias=take(nh, ds), c_bias=take(nh, ds), d_param=take(nh),
+                                    norm_gate_weight=take(di), out_proj_w=take(di, dm)))
+        self.norm_f_weight = take(dm)
+        assert o == n
+
+    def zero_state(self):
+        L, nh, hd, ds = self.n_layers, self.nh, self.hd, self.ds
+        return (np.zeros((L, nh, hd, ds), np.float32), np.zeros((L, nh, ds), np.float32), np.zeros((L, nh, hd), np.float32),
+                np.zeros((L, nh, max(self.n_rope, 1)), np.float32))
+
+
+def m3_backbone_step(P: M3Params, x, state, taps=False):
+    """One token through the Mamba-3 backbone (CPU route). state = (ssm, kst, vst, angle), updated in place.
+    With taps=True also returns per-layer dict of the scan-level quantities."""
+    ssm, kst, vst, angle = state
+    x = _c(x)
+    out = np.zeros(P.dm, np.float32)
+    tp = np.zeros((P.n_layers, 6 * P.nh + 2 * P.nh * P.ds), np.float32) if taps else None
+    lib().orc_m3_backbone_step(_p(out), _p(x), _p(P.flat), _p(ssm), _p(kst), _p(vst), _p(angle), _p(tp), c_int64(P.dm),
+                               c_int64(P.ds), c_int64(P.expand), c_int64(P.hd), c_int64(P.ng), c_int64(P.n_layers),
+                               c_int64(P.n_rope), c_float(P.a_floor), c_int(1 if P.outproj_norm else 0), c_int64(P.input_dim))
+    if not taps:
+        return out
+    nh, ds = P.nh, P.ds
+    res = []
+    for l in range(P.n_layers):
+        t = tp[l]
+        res.append(dict(alpha=t[0:nh], beta=t[nh:2 * nh], gamma=t[2 * nh:3 * nh], dt=t[3 * nh:4 * nh], trap=t[4 * nh:5 * nh],
+                        a_val=t[5 * nh:6 * nh], k=t[6 * nh:6 * nh + nh * ds].reshape(nh, ds),
+                        q=t[6 * nh + nh * ds:].reshape(nh, ds)))
+    return out, res
