@@ -94,14 +94,16 @@ MRS_API int mrs_ssm_scan_fwd(void *stream, int dtype, float *h, void *y, const v
 /* Same scan with the fusions the prefill chain allows:
  *   bc_stride  row stride (elements) of B and C, so both can point into xdbl
  *              [batch*T, xdbl_dim] (replaces gather_bc_cols, kernels/elementwise.cu:291-313)
- *   gate,flags optional gate tensor [batch,T,d_inner] (replaces elementwise_mul,
- *              src/mamba_ssm/gpu/prefill.rs:957-971)
+ *   gate,flags optional gate tensor, [batch*T] rows of gate_stride elements (0 = d_inner), the
+ *              first d_inner of each used (replaces elementwise_mul, src/mamba_ssm/gpu/prefill.rs:957-971;
+ *              with MRS_GATE_SILU and gate_stride = 2*d_inner it reads the z half of in_proj's
+ *              output in place, which also replaces split_gate_silu, kernels/elementwise.cu:172-189)
  *   workspace  mrs_ssm_scan_workspace_bytes() bytes of device memory, 256-byte
  *              aligned; NULL forces the sequential route. */
 MRS_API size_t mrs_ssm_scan_workspace_bytes(int batch, int T, int d_inner, int d_state);
 MRS_API int mrs_ssm_scan_fwd_ex(void *stream, int dtype, float *h, void *y, const void *delta, const void *u,
                         const void *B, const void *C, int64_t bc_stride, const float *a_neg,
-                        const float *D, const void *gate, unsigned flags,
+                        const float *D, const void *gate, int64_t gate_stride, unsigned flags,
                         void *workspace, size_t workspace_bytes,
                         int batch, int T, int d_inner, int d_state);
 
@@ -187,6 +189,90 @@ MRS_API int mrs_m3_ssd_fwd(void *stream, int dtype, float *ssm_state, float *k_s
                            const float *a_val, const float *D, void *workspace, size_t workspace_bytes,
                            unsigned flags, int batch, int T, int nheads, int headdim, int d_state,
                            int chunk_size);
+
+/* ---- Mamba-1 backbone engine ----------------------------------------------------
+ * The host surface of GpuMambaBackbone (src/mamba_ssm/gpu/inference.rs:1515-1855): the engine
+ * owns device copies of the weights (projection matrices in `dtype`, the rest f32), the
+ * persistent per-layer conv/SSM state and all scratch; nothing is allocated per step.
+ * Host I/O is always f32.  Batch is fixed at creation.  An engine is not thread-safe
+ * (the reference's is !Sync too, context.rs:16-56); it runs on its own non-blocking stream. */
+typedef struct mrs_backbone mrs_backbone;
+
+typedef struct {            /* MambaConfig, src/config.rs:57-84 */
+    int d_model, d_state, d_conv, expand, n_layers;
+    int scan_mode;          /* mrs_scan_mode */
+    float rms_norm_eps;
+} mrs_m1_config;
+
+typedef struct {            /* MambaLayerWeights, src/weights.rs:7-42: host f32, row-major [n_in, n_out] */
+    const float *norm_weight;   /* [d_model] */
+    const float *in_proj_w;     /* [d_model, 2*d_inner] */
+    const float *conv1d_weight; /* [d_inner, d_conv] */
+    const float *conv1d_bias;   /* [d_inner] */
+    const float *x_proj_w;      /* [d_inner, dt_rank + 2*d_state] */
+    const float *dt_proj_w;     /* [dt_rank, d_inner] */
+    const float *dt_proj_b;     /* [d_inner] */
+    const float *a_log;         /* [d_inner, d_state]; a_neg = -exp(a_log) is derived at load */
+    const float *d_param;       /* [d_inner] */
+    const float *out_proj_w;    /* [d_inner, d_model] */
+} mrs_m1_layer_weights;
+
+typedef struct {            /* MambaWeights, src/weights.rs:51-64 */
+    const float *input_proj_w;  /* [input_dim, d_model], or NULL for the identity (LM) case */
+    const float *input_proj_b;  /* [d_model] or NULL (zeros) */
+    const mrs_m1_layer_weights *layers; /* n_layers entries */
+    const float *norm_f_weight; /* [d_model] */
+} mrs_m1_weights;
+
+/* GpuMambaBackbone::new_with_dtype(gpu_ordinal, &weights, cfg, input_dim, batch, dtype)  (inference.rs:1517-1575).
+ * Validates the config with the reference's bounds (src/config.rs:108-170). */
+MRS_API int mrs_backbone_create(mrs_backbone **out, int gpu_ordinal, const mrs_m1_weights *weights,
+                                const mrs_m1_config *cfg, int input_dim, int batch, int dtype);
+MRS_API void mrs_backbone_destroy(mrs_backbone *bb);
+/* step(&[f32] input [batch*input_dim], &mut [f32] output [batch*d_model])  (inference.rs:1586): H2D, one
+ * token through every layer, D2H, synchronises. */
+MRS_API int mrs_backbone_step(mrs_backbone *bb, const float *input, float *output);
+/* step_gpu_only (inference.rs:1670): input already in mrs_backbone_input_ptr(), output left in temporal_ptr(). */
+MRS_API int mrs_backbone_step_gpu_only(mrs_backbone *bb);
+/* reset (inference.rs:1599): zero conv and SSM state. */
+MRS_API int mrs_backbone_reset(mrs_backbone *bb);
+/* capture_graph (inference.rs:1608-1630): warm step, then capture the step body into a hipGraph that
+ * step()/step_gpu_only() replay afterwards. State is preserved across the call. */
+MRS_API int mrs_backbone_capture_graph(mrs_backbone *bb);
+/* alloc_prefill_scratch / prefill_sequence[_mixed] (inference.rs:1752-1831; src/mamba_ssm/gpu/prefill.rs:676-1049):
+ * input [batch, T, input_dim] f32 on the host; the whole sequence runs through the layers, the state ends
+ * positioned after token T (so step continues), output_last (may be NULL) receives norm_f of the last position
+ * [batch, d_model].  One sequence length per engine (scratch is sized once). T >= 2. */
+MRS_API int mrs_backbone_alloc_prefill_scratch(mrs_backbone *bb, int T);
+MRS_API int mrs_backbone_prefill_sequence(mrs_backbone *bb, const float *input, int T, float *output_last);
+/* Same, input already on the device ([batch,T,input_dim] f32); does not synchronise. */
+MRS_API int mrs_backbone_prefill_device(mrs_backbone *bb, const float *input_dev, int T);
+/* temporal_ptr / input buffer / stream accessors (inference.rs:1717-1737) and state access for tests. */
+MRS_API float *mrs_backbone_temporal_ptr(mrs_backbone *bb);
+MRS_API float *mrs_backbone_input_ptr(mrs_backbone *bb);
+MRS_API float *mrs_backbone_prefill_input_ptr(mrs_backbone *bb);
+MRS_API void *mrs_backbone_stream(mrs_backbone *bb);
+MRS_API int mrs_backbone_sync(mrs_backbone *bb);
+MRS_API int mrs_backbone_state_ptrs(mrs_backbone *bb, int layer, float **conv_state, float **ssm_state);
+MRS_API int mrs_backbone_download_state(mrs_backbone *bb, int layer, float *conv_state, float *ssm_state);
+
+/* ---- greedy LM loop on top of a backbone ------------------------------------------
+ * The decode loop of GpuMambaLM::generate_streaming (src/module/gpu_lm.rs:334-377) with tied
+ * embedding / lm_head (gpu_lm.rs:560-679), temperature 0: next token = last index of the maximum
+ * logit (src/module/sample.rs:250-257).  Unlike the reference the embedding gather and the argmax
+ * run on the device, so a decode step needs no host round trip.
+ *   embed: [vocab, d_model] f32 on the host (rows >= vocab of the 64-padded table are zero). */
+typedef struct mrs_lm mrs_lm;
+MRS_API int mrs_lm_create(mrs_lm **out, mrs_backbone *decode_engine, const float *embed, int vocab);
+MRS_API void mrs_lm_destroy(mrs_lm *lm);
+MRS_API int mrs_lm_set_tokens(mrs_lm *lm, const int *tokens);      /* [batch] current tokens */
+MRS_API int mrs_lm_get_tokens(mrs_lm *lm, int *tokens);            /* synchronises */
+MRS_API int mrs_lm_decode_step(mrs_lm *lm);                        /* tokens <- greedy next tokens */
+MRS_API int mrs_lm_capture_graph(mrs_lm *lm);                      /* capture one decode step */
+MRS_API int mrs_lm_last_logits(mrs_lm *lm, float *logits);         /* [batch, vocab] f32, synchronises */
+/* tokens [prefill_engine.batch, T] -> embeddings -> prefill on `prefill_engine` (which may be the decode
+ * engine itself: then the head + argmax run and the next tokens are left in the token buffer). */
+MRS_API int mrs_lm_prefill(mrs_lm *lm, mrs_backbone *prefill_engine, const int *tokens, int T);
 
 #ifdef __cplusplus
 }

@@ -6,3 +6,5 @@ engine types that mirror the reference's GpuMambaBackbone surface.
 """
 from ._lib import MambaHipError, load as load_library  # noqa: F401
 from .config import MambaConfig, ScanMode, WeightDtype, PARALLEL_SCAN_THRESHOLD  # noqa: F401
+from .weights import MambaWeights, MambaLayerWeights  # noqa: F401
+from .backbone import GpuMambaBackbone, GpuMambaLM  # noqa: F401

@@ -1,0 +1,258 @@
+"""GpuMambaBackbone / GpuMambaLM: host mirror of the reference's engine types
+(src/mamba_ssm/gpu/inference.rs:1515-1855, src/module/gpu_lm.rs:121-516) over the C ABI.
+
+All arithmetic happens in libmamba_hip.so; this module only marshals numpy arrays.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import POINTER, Structure, byref, c_float, c_int, c_void_p
+
+import numpy as np
+
+from . import _lib
+from .config import MambaConfig, WeightDtype
+from .weights import MambaWeights
+
+_FP = POINTER(c_float)
+
+
+class _CConfig(Structure):
+    _fields_ = [("d_model", c_int), ("d_state", c_int), ("d_conv", c_int), ("expand", c_int), ("n_layers", c_int),
+                ("scan_mode", c_int), ("rms_norm_eps", c_float)]
+
+
+class _CLayer(Structure):
+    _fields_ = [(n, _FP) for n in ("norm_weight", "in_proj_w", "conv1d_weight", "conv1d_bias", "x_proj_w", "dt_proj_w",
+                                   "dt_proj_b", "a_log", "d_param", "out_proj_w")]
+
+
+class _CWeights(Structure):
+    _fields_ = [("input_proj_w", _FP), ("input_proj_b", _FP), ("layers", POINTER(_CLayer)), ("norm_f_weight", _FP)]
+
+
+def _fp(a: np.ndarray):
+    return a.ctypes.data_as(_FP)
+
+
+def _bind():
+    lib = _lib.load()
+    if getattr(lib, "_engine_bound", False):
+        return lib
+    P = c_void_p
+    sigs = {
+        "mrs_backbone_create": (c_int, [POINTER(P), c_int, POINTER(_CWeights), POINTER(_CConfig), c_int, c_int, c_int]),
+        "mrs_backbone_destroy": (None, [P]),
+        "mrs_backbone_step": (c_int, [P, _FP, _FP]),
+        "mrs_backbone_step_gpu_only": (c_int, [P]),
+        "mrs_backbone_reset": (c_int, [P]),
+        "mrs_backbone_capture_graph": (c_int, [P]),
+        "mrs_backbone_alloc_prefill_scratch": (c_int, [P, c_int]),
+        "mrs_backbone_prefill_sequence": (c_int, [P, _FP, c_int, _FP]),
+        "mrs_backbone_prefill_device": (c_int, [P, P, c_int]),
+        "mrs_backbone_temporal_ptr": (P, [P]),
+        "mrs_backbone_input_ptr": (P, [P]),
+        "mrs_backbone_prefill_input_ptr": (P, [P]),
+        "mrs_backbone_stream": (P, [P]),
+        "mrs_backbone_sync": (c_int, [P]),
+        "mrs_backbone_state_ptrs": (c_int, [P, c_int, POINTER(P), POINTER(P)]),
+        "mrs_backbone_download_state": (c_int, [P, c_int, _FP, _FP]),
+        "mrs_lm_create": (c_int, [POINTER(P), P, _FP, c_int]),
+        "mrs_lm_destroy": (None, [P]),
+        "mrs_lm_set_tokens": (c_int, [P, POINTER(c_int)]),
+        "mrs_lm_get_tokens": (c_int, [P, POINTER(c_int)]),
+        "mrs_lm_decode_step": (c_int, [P]),
+        "mrs_lm_capture_graph": (c_int, [P]),
+        "mrs_lm_last_logits": (c_int, [P, _FP]),
+        "mrs_lm_prefill": (c_int, [P, P, POINTER(c_int), c_int]),
+    }
+    for name, (res, args) in sigs.items():
+        fn = getattr(lib, name)
+        fn.restype, fn.argtypes = res, args
+    lib._engine_bound = True
+    lib._engine_names = sorted(sigs)
+    return lib
+
+
+def engine_exported_names():
+    return list(_bind()._engine_names)
+
+
+def _call(name, *args):
+    lib = _bind()
+    rc = getattr(lib, name)(*args)
+    if rc != 0:
+        raise _lib.MambaHipError(name, rc, lib.mrs_last_error().decode())
+
+
+class GpuMambaBackbone:
+    """One-GPU Mamba-1 backbone engine with fixed batch; `step` decodes one token per batch row,
+    `prefill_sequence` runs whole sequences and leaves the state positioned for `step`."""
+
+    def __init__(self, gpu_ordinal: int, weights: MambaWeights, cfg: MambaConfig, input_dim: int, batch: int,
+                 dtype: WeightDtype = WeightDtype.F32):
+        cfg.validate()
+        weights.validate(cfg, input_dim)
+        self.cfg, self.input_dim, self.batch, self.dtype = cfg, input_dim, batch, WeightDtype(dtype)
+        keep = []
+
+        def arr(a):
+            a = np.ascontiguousarray(a, dtype=np.float32)
+            keep.append(a)
+            return _fp(a)
+
+        layers = (_CLayer * cfg.n_layers)()
+        for i, lw in enumerate(weights.layers):
+            for n, _ in _CLayer._fields_:
+                setattr(layers[i], n, arr(getattr(lw, n)))
+        cw = _CWeights()
+        identity = weights.input_proj_w.size == 0
+        cw.input_proj_w = None if identity else arr(weights.input_proj_w)
+        cw.input_proj_b = None if identity else arr(weights.input_proj_b)
+        cw.layers = layers
+        cw.norm_f_weight = arr(weights.norm_f_weight)
+        cc = _CConfig(cfg.d_model, cfg.d_state, cfg.d_conv, cfg.expand, cfg.n_layers, int(cfg.scan_mode), cfg.rms_norm_eps)
+        h = c_void_p()
+        _call("mrs_backbone_create", byref(h), gpu_ordinal, byref(cw), byref(cc), input_dim, batch, int(self.dtype))
+        self._h = h
+
+    @classmethod
+    def new(cls, gpu_ordinal, weights, cfg, input_dim, batch):
+        return cls(gpu_ordinal, weights, cfg, input_dim, batch, WeightDtype.F32)
+
+    @classmethod
+    def new_with_dtype(cls, gpu_ordinal, weights, cfg, input_dim, batch, dtype):
+        return cls(gpu_ordinal, weights, cfg, input_dim, batch, dtype)
+
+    def close(self):
+        if getattr(self, "_h", None):
+            _bind().mrs_backbone_destroy(self._h)
+            self._h = None
+
+    __del__ = close
+
+    def step(self, inp: np.ndarray) -> np.ndarray:
+        inp = np.ascontiguousarray(inp, dtype=np.float32)
+        if inp.size != self.batch * self.input_dim:
+            raise ValueError(f"input must hold batch*input_dim = {self.batch * self.input_dim} values")
+        out = np.empty((self.batch, self.cfg.d_model), np.float32)
+        _call("mrs_backbone_step", self._h, _fp(inp), _fp(out))
+        return out
+
+    def step_gpu_only(self):
+        _call("mrs_backbone_step_gpu_only", self._h)
+
+    def reset(self):
+        _call("mrs_backbone_reset", self._h)
+
+    def capture_graph(self):
+        _call("mrs_backbone_capture_graph", self._h)
+
+    def alloc_prefill_scratch(self, T: int):
+        _call("mrs_backbone_alloc_prefill_scratch", self._h, T)
+
+    def prefill_sequence(self, inp: np.ndarray) -> np.ndarray:
+        """inp [batch, T, input_dim] f32 -> norm_f output of the last position [batch, d_model]."""
+        inp = np.ascontiguousarray(inp, dtype=np.float32)
+        if inp.ndim != 3 or inp.shape[0] != self.batch or inp.shape[2] != self.input_dim:
+            raise ValueError("input must be [batch, T, input_dim]")
+        out = np.empty((self.batch, self.cfg.d_model), np.float32)
+        _call("mrs_backbone_prefill_sequence", self._h, _fp(inp), inp.shape[1], _fp(out))
+        return out
+
+    prefill_sequence_mixed = prefill_sequence
+
+    def prefill_device(self, ptr: int, T: int):
+        _call("mrs_backbone_prefill_device", self._h, c_void_p(ptr), T)
+
+    def sync(self):
+        _call("mrs_backbone_sync", self._h)
+
+    def temporal_ptr(self) -> int:
+        return _bind().mrs_backbone_temporal_ptr(self._h)
+
+    def temporal_dtype(self) -> WeightDtype:
+        return WeightDtype.F32
+
+    def input_ptr(self) -> int:
+        return _bind().mrs_backbone_input_ptr(self._h)
+
+    def prefill_input_ptr(self) -> int:
+        return _bind().mrs_backbone_prefill_input_ptr(self._h)
+
+    def stream(self) -> int:
+        return _bind().mrs_backbone_stream(self._h)
+
+    def download_state(self, layer: int):
+        """(conv_state [batch, d_inner, d_conv], ssm_state [batch, d_inner, d_state]) of one layer."""
+        di = self.cfg.d_inner()
+        conv = np.empty((self.batch, di, self.cfg.d_conv), np.float32)
+        ssm = np.empty((self.batch, di, self.cfg.d_state), np.float32)
+        _call("mrs_backbone_download_state", self._h, layer, _fp(conv), _fp(ssm))
+        return conv, ssm
+
+
+class GpuMambaLM:
+    """Greedy LM loop with tied embedding / lm_head on top of a backbone (identity input_proj)."""
+
+    def __init__(self, backbone: GpuMambaBackbone, embed: np.ndarray):
+        self.backbone = backbone
+        embed = np.ascontiguousarray(embed, dtype=np.float32)
+        if embed.ndim != 2 or embed.shape[1] != backbone.cfg.d_model:
+            raise ValueError("embed must be [vocab, d_model]")
+        self.vocab = embed.shape[0]
+        h = c_void_p()
+        _call("mrs_lm_create", byref(h), backbone._h, _fp(embed), self.vocab)
+        self._h = h
+
+    def close(self):
+        if getattr(self, "_h", None):
+            _bind().mrs_lm_destroy(self._h)
+            self._h = None
+
+    __del__ = close
+
+    def set_tokens(self, tokens):
+        t = np.ascontiguousarray(tokens, dtype=np.int32)
+        _call("mrs_lm_set_tokens", self._h, t.ctypes.data_as(POINTER(c_int)))
+
+    def get_tokens(self) -> np.ndarray:
+        t = np.empty(self.backbone.batch, np.int32)
+        _call("mrs_lm_get_tokens", self._h, t.ctypes.data_as(POINTER(c_int)))
+        return t
+
+    def decode_step(self):
+        _call("mrs_lm_decode_step", self._h)
+
+    def capture_graph(self):
+        _call("mrs_lm_capture_graph", self._h)
+
+    def last_logits(self) -> np.ndarray:
+        out = np.empty((self.backbone.batch, self.vocab), np.float32)
+        _call("mrs_lm_last_logits", self._h, _fp(out))
+        return out
+
+    def prefill(self, tokens: np.ndarray, engine: GpuMambaBackbone | None = None):
+        engine = engine or self.backbone
+        t = np.ascontiguousarray(tokens, dtype=np.int32)
+        if t.ndim != 2 or t.shape[0] != engine.batch:
+            raise ValueError("tokens must be [batch, T]")
+        _call("mrs_lm_prefill", self._h, engine._h, t.ctypes.data_as(POINTER(c_int)), t.shape[1])
+
+    def generate(self, prompt, max_tokens: int):
+        """Greedy generation for a batch-1 engine (GpuMambaLM::generate, temperature 0, gpu_lm.rs:323-377):
+        the prompt goes through prefill when it has at least 2 tokens, token by token otherwise."""
+        if self.backbone.batch != 1:
+            raise ValueError("generate() is the batch-1 entry point")
+        prompt = list(prompt)
+        self.backbone.reset()
+        if len(prompt) >= 2:
+            self.prefill(np.asarray([prompt], np.int32))
+        else:
+            self.set_tokens(prompt[:1])
+            self.decode_step()
+        out = [int(self.get_tokens()[0])]
+        for _ in range(max_tokens - 1):
+            self.decode_step()
+            out.append(int(self.get_tokens()[0]))
+        return out

@@ -24,7 +24,7 @@ DEVICE_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     # MFMA accumulators stay in ordinary VGPRs (no AccVGPR copies around each instruction).
     "-mllvm", "-amdgpu-mfma-vgpr-form",
-    "-Wno-unused-command-line-argument",
+    "-Wno-unused-command-line-argument", "-Wno-unused-result", "-Wno-unused-value",
 ]
 
 
@@ -65,7 +65,8 @@ def build_library(verbose: bool = True, jobs: int = 4) -> Path:
     with ThreadPoolExecutor(max_workers=jobs) as ex:
         list(ex.map(compile_one, zip(srcs, objs)))
     tmp = LIB_PATH.with_suffix(".so.tmp")
-    _run([hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(tmp), *map(str, objs)])
+    _run([hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(tmp), *map(str, objs),
+          "-L/opt/rocm/lib", "-lrocblas", "-Wl,-rpath,/opt/rocm/lib"])
     os.replace(tmp, LIB_PATH)
     if verbose:
         print(f"[build] wrote {LIB_PATH}", file=sys.stderr)

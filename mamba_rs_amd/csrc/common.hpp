@@ -50,6 +50,14 @@ void set_error(const char *fmt, ...);
 int fail(int code, const char *fmt, ...);
 int check_launch(const char *what);
 
+// Internal launchers shared with the backbone engine (strides and fusions the public entry points do not expose).
+int launch_ssm_step_fused(hipStream_t st, int dtype, float *h, void *y, const void *delta, const float *dt_bias,
+                          const void *u, const void *Bb, const void *Cb, int64_t bc_stride, const void *gate,
+                          int64_t gate_stride, int gate_mode, const float *a_neg, const float *D, int batch,
+                          int di, int ds);
+int launch_conv1d_step(hipStream_t st, int dtype, void *out, float *state, const void *new_x, int64_t x_stride,
+                       const float *weight, const float *bias, int batch, int d_inner, int d_conv, int apply_silu);
+
 inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s); }
 inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 

@@ -18,18 +18,19 @@ constexpr int kMaxConv = 8;  // reference limit, src/config.rs:154-159
 
 template <typename T, bool SILU>
 __global__ __launch_bounds__(256) void conv1d_step_kernel(
-    T *__restrict__ out, float *__restrict__ state, const T *__restrict__ new_x,
+    T *__restrict__ out, float *__restrict__ state, const T *__restrict__ new_x, int64_t x_stride,
     const float *__restrict__ weight, const float *__restrict__ bias, int64_t total, int di, int dc) {
     const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (r >= total) return;
     const int d = (int)(r % di);
+    const int64_t xi = (r / di) * x_stride + d;  // new_x rows may be wider than d_inner (x half of in_proj's output)
     float *st = state + r * dc;
     const float *w = weight + (int64_t)d * dc;
     float s = bias[d];
     float win[kMaxConv];
 #pragma unroll
     for (int k = 0; k < kMaxConv; k++)
-        if (k < dc) win[k] = (k + 1 < dc) ? st[k + 1] : Store<T>::ld(new_x + r);
+        if (k < dc) win[k] = (k + 1 < dc) ? st[k + 1] : Store<T>::ld(new_x + xi);
 #pragma unroll
     for (int k = 0; k < kMaxConv; k++)
         if (k < dc) { s = fmaf(win[k], w[k], s); st[k] = win[k]; }
@@ -205,6 +206,19 @@ static int conv_check(const char *fn, int dtype, const void *out, const void *st
     return MRS_OK;
 }
 
+int launch_conv1d_step(hipStream_t st, int dtype, void *out, float *state, const void *new_x, int64_t x_stride,
+                       const float *weight, const float *bias, int batch, int d_inner, int d_conv, int apply_silu) {
+    const int64_t total = (int64_t)batch * d_inner;
+    const int64_t blocks = (total + 255) / 256;
+    if (blocks > 0x7fffffffLL) return fail(MRS_E_SHAPE, "conv1d step: grid too large");
+    const dim3 grid((unsigned)blocks), block(256);
+    MRS_DISPATCH_DTYPE(dtype, T_, {
+        if (apply_silu) hipLaunchKernelGGL((conv1d_step_kernel<T_, true>), grid, block, 0, st, (T_ *)out, state, (const T_ *)new_x, x_stride, weight, bias, total, d_inner, d_conv);
+        else hipLaunchKernelGGL((conv1d_step_kernel<T_, false>), grid, block, 0, st, (T_ *)out, state, (const T_ *)new_x, x_stride, weight, bias, total, d_inner, d_conv);
+    });
+    return check_launch("conv1d_step_kernel");
+}
+
 }  // namespace mrs
 
 using namespace mrs;
@@ -214,16 +228,7 @@ extern "C" int mrs_conv1d_step(void *stream, int dtype, void *out, float *state,
                                int d_conv, int apply_silu) {
     int rc = conv_check("mrs_conv1d_step", dtype, out, state, new_x, weight, bias, batch, d_inner, d_conv);
     if (rc) return rc;
-    const int64_t total = (int64_t)batch * d_inner;
-    const int64_t blocks = (total + 255) / 256;
-    if (blocks > 0x7fffffffLL) return fail(MRS_E_SHAPE, "mrs_conv1d_step: grid too large");
-    hipStream_t st = as_stream(stream);
-    const dim3 grid((unsigned)blocks), block(256);
-    MRS_DISPATCH_DTYPE(dtype, T_, {
-        if (apply_silu) hipLaunchKernelGGL((conv1d_step_kernel<T_, true>), grid, block, 0, st, (T_ *)out, state, (const T_ *)new_x, weight, bias, total, d_inner, d_conv);
-        else hipLaunchKernelGGL((conv1d_step_kernel<T_, false>), grid, block, 0, st, (T_ *)out, state, (const T_ *)new_x, weight, bias, total, d_inner, d_conv);
-    });
-    return check_launch("conv1d_step_kernel");
+    return launch_conv1d_step(as_stream(stream), dtype, out, state, new_x, d_inner, weight, bias, batch, d_inner, d_conv, apply_silu);
 }
 
 extern "C" int mrs_conv1d_seq_silu(void *stream, int dtype, void *u_out, float *state, const void *x_branch,

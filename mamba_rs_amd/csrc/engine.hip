@@ -1,0 +1,697 @@
+// Mamba-1 backbone and LM engines: the host-side surface of the reference's
+// GpuMambaBackbone (src/mamba_ssm/gpu/inference.rs:1515-1855) and the greedy loop of
+// GpuMambaLM (src/module/gpu_lm.rs:323-377), driving the kernels of this library.
+//
+// Ownership follows the reference (inference.rs:92-143): the engine owns its weights
+// (bulk projection matrices in the storage dtype, everything else f32), the persistent
+// conv/SSM state and every scratch buffer; step() allocates nothing.  The residual
+// stream, states, a_neg, D, biases and norm weights stay f32 (inference.rs:150-165).
+//
+// Per layer the decode chain is 4 library GEMMs and 3 kernels (the reference launches 10
+// kernels + 4 GEMMs, inference.rs:993-1252): residual-add + RMSNorm, in_proj, conv step +
+// SiLU reading the x half of in_proj's output in place, x_proj, dt_proj, one kernel for
+// dt-bias + softplus + state update + B/C gather + SiLU gate, out_proj.
+#include "common.hpp"
+#include <rocblas/rocblas.h>
+#include <new>
+#include <vector>
+
+namespace mrs {
+
+#define MRS_HIP(expr)                                                                         \
+    do {                                                                                      \
+        hipError_t e_ = (expr);                                                               \
+        if (e_ != hipSuccess) return fail(MRS_E_HIP, "%s: %s", #expr, hipGetErrorString(e_)); \
+    } while (0)
+#define MRS_BLAS(expr)                                                                  \
+    do {                                                                                \
+        rocblas_status s_ = (expr);                                                     \
+        if (s_ != rocblas_status_success) return fail(MRS_E_HIP, "%s: rocblas status %d", #expr, (int)s_); \
+    } while (0)
+#define MRS_TRY(expr)          \
+    do {                       \
+        int rc_ = (expr);      \
+        if (rc_) return rc_;   \
+    } while (0)
+
+static size_t esize(int dtype) { return dtype == MRS_F32 ? 4 : 2; }
+static rocblas_datatype blas_type(int dtype) {
+    return dtype == MRS_F32 ? rocblas_datatype_f32_r : dtype == MRS_F16 ? rocblas_datatype_f16_r : rocblas_datatype_bf16_r;
+}
+
+// ---- glue kernels -------------------------------------------------------------------
+
+// One wave per row: residual (f32) += add (storage dtype, may be null); out = rmsnorm(residual) * w.
+// Reference: residual_add_f32_* + rmsnorm_forward_f32in_* (kernels/elementwise.cu:366-376,
+// kernels/norms.cu:21-171), with its finite guard: rms = 1 if not finite or < 1e-20 (norms.cu:58-61).
+template <typename T, typename TO>
+__global__ __launch_bounds__(256) void add_rmsnorm_kernel(float *__restrict__ residual, const T *__restrict__ add,
+                                                          TO *__restrict__ out, const float *__restrict__ w,
+                                                          float eps, int64_t rows, int dm, int64_t out_stride) {
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int l = threadIdx.x & 63;
+    float *r = residual + row * dm;
+    float ss = 0.0f;
+    for (int i = l; i < dm; i += kWave) {
+        float v = r[i];
+        if (add) { v += Store<T>::ld(add + row * dm + i); r[i] = v; }
+        ss = fmaf(v, v, ss);
+    }
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) ss += __shfl_xor(ss, m, kWave);
+    float rms = sqrtf(ss / (float)dm + eps);
+    if (!isfinite(rms) || rms < 1e-20f) rms = 1.0f;
+    const float inv = 1.0f / rms;
+    for (int i = l; i < dm; i += kWave) Store<TO>::st(out + row * out_stride + i, r[i] * inv * w[i]);
+}
+
+// delta = softplus(raw + bias[d]) in place (dt_proj bias + softplus_forward, kernels/activations.cu:32-52)
+template <typename T>
+__global__ __launch_bounds__(256) void bias_softplus_kernel(T *__restrict__ x, const float *__restrict__ bias, int64_t n, int di) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const float v = Store<T>::ld(x + i) + bias[i % di];
+    Store<T>::st(x + i, v > 20.0f ? v : log1pf(fast_exp2(v * kLog2e)));
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void cast_from_f32_kernel(T *__restrict__ out, const float *__restrict__ in, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) Store<T>::st(out + i, in[i]);
+}
+
+__global__ __launch_bounds__(256) void bias_rows_kernel(float *__restrict__ out, const float *__restrict__ bias, int64_t n, int dm) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = bias[i % dm];
+}
+
+__global__ __launch_bounds__(256) void exp_negate_k(float *__restrict__ a_neg, const float *__restrict__ a_log, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) a_neg[i] = -expf(a_log[i]);
+}
+
+// residual[r, :] = embed[token[r], :] widened to f32 (host-side embed_lookup of the reference, gpu_lm.rs:352-373, moved on device)
+template <typename T>
+__global__ __launch_bounds__(256) void embed_gather_kernel(float *__restrict__ out, const T *__restrict__ embed,
+                                                           const int *__restrict__ tokens, int64_t rows, int dm, int vocab) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= rows * dm) return;
+    const int64_t r = i / dm;
+    int tok = tokens[r];
+    tok = tok < 0 ? 0 : (tok >= vocab ? vocab - 1 : tok);
+    out[i] = Store<T>::ld(embed + (int64_t)tok * dm + (i - r * dm));
+}
+
+// Greedy pick: index of the maximum logit, the LAST one among equals (Iterator::max_by, src/module/sample.rs:250-257).
+__global__ __launch_bounds__(256) void argmax_last_kernel(int *__restrict__ tokens, const float *__restrict__ logits,
+                                                          int vocab, int64_t stride) {
+    __shared__ float sv[256];
+    __shared__ int si[256];
+    const float *row = logits + (int64_t)blockIdx.x * stride;
+    float best = -INFINITY;
+    int bi = 0;
+    for (int i = threadIdx.x; i < vocab; i += 256) {
+        const float v = row[i];
+        if (v >= best) { best = v; bi = i; }   // ascending i per thread: >= keeps the last maximum
+    }
+    sv[threadIdx.x] = best; si[threadIdx.x] = bi;
+    __syncthreads();
+    for (int s = 128; s >= 1; s >>= 1) {
+        if ((int)threadIdx.x < s) {
+            const float ov = sv[threadIdx.x + s];
+            const int oi = si[threadIdx.x + s];
+            if (ov > sv[threadIdx.x] || (ov == sv[threadIdx.x] && oi > si[threadIdx.x])) { sv[threadIdx.x] = ov; si[threadIdx.x] = oi; }
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) tokens[blockIdx.x] = si[0];
+}
+
+}  // namespace mrs
+
+using namespace mrs;
+
+struct LayerDev {
+    float *norm_w, *conv_w, *conv_b, *dt_b, *a_neg, *D;
+    void *in_proj, *x_proj, *dt_w, *out_proj;
+    int s4d;
+};
+
+struct Scratch {  // activations for M rows
+    int64_t rows = 0;
+    void *normed = nullptr, *proj = nullptr, *u = nullptr, *xdbl = nullptr, *delta = nullptr, *y = nullptr, *out = nullptr;
+    float *residual = nullptr;
+    void *scan_ws = nullptr;
+    size_t scan_ws_bytes = 0;
+    int T = 0;
+};
+
+struct mrs_backbone {
+    mrs_m1_config cfg;
+    int input_dim, batch, dtype, di, dr, xd, identity_proj, device;
+    hipStream_t stream;
+    rocblas_handle blas;
+    std::vector<LayerDev> layers;
+    float *input_proj_w, *input_proj_b, *norm_f;
+    std::vector<void *> allocs;
+    float *conv_state, *ssm_state;
+    float *d_input, *temporal;
+    Scratch step_s, prefill_s;
+    float *prefill_in;  // [batch*T, input_dim] f32 staging for host input
+    hipGraph_t graph;
+    hipGraphExec_t graph_exec;
+    int graph_ready;
+};
+
+static int dev_alloc(mrs_backbone *bb, void **p, size_t bytes) {
+    MRS_HIP(hipMalloc(p, bytes ? bytes : 16));
+    bb->allocs.push_back(*p);
+    return MRS_OK;
+}
+
+static int upload_f32(mrs_backbone *bb, float **dst, const float *src, size_t n) {
+    MRS_TRY(dev_alloc(bb, (void **)dst, n * sizeof(float)));
+    MRS_HIP(hipMemcpyAsync(*dst, src, n * sizeof(float), hipMemcpyHostToDevice, bb->stream));
+    return MRS_OK;
+}
+
+// Bulk matrix: upload f32, round to the storage dtype on device (RNE, as the reference's casts, kernels/elementwise.cu:17-38).
+static int upload_bulk(mrs_backbone *bb, void **dst, const float *src, size_t n, float *stage) {
+    MRS_HIP(hipMemcpyAsync(stage, src, n * sizeof(float), hipMemcpyHostToDevice, bb->stream));
+    MRS_TRY(dev_alloc(bb, dst, n * esize(bb->dtype)));
+    const dim3 grid((unsigned)((n + 255) / 256)), block(256);
+    if (bb->dtype == MRS_F32) MRS_HIP(hipMemcpyAsync(*dst, stage, n * 4, hipMemcpyDeviceToDevice, bb->stream));
+    else if (bb->dtype == MRS_BF16) hipLaunchKernelGGL((cast_from_f32_kernel<bf16_t>), grid, block, 0, bb->stream, (bf16_t *)*dst, stage, (int64_t)n);
+    else hipLaunchKernelGGL((cast_from_f32_kernel<f16_t>), grid, block, 0, bb->stream, (f16_t *)*dst, stage, (int64_t)n);
+    MRS_HIP(hipStreamSynchronize(bb->stream));  // stage is reused by the next upload
+    return check_launch("weight cast");
+}
+
+static int alloc_scratch(mrs_backbone *bb, Scratch *s, int64_t rows, int T) {
+    const size_t es = esize(bb->dtype);
+    const int dm = bb->cfg.d_model, di = bb->di, xd = bb->xd;
+    s->rows = rows; s->T = T;
+    MRS_TRY(dev_alloc(bb, (void **)&s->residual, rows * dm * sizeof(float)));
+    MRS_TRY(dev_alloc(bb, &s->normed, rows * dm * es));
+    MRS_TRY(dev_alloc(bb, &s->proj, rows * 2 * di * es));
+    MRS_TRY(dev_alloc(bb, &s->u, rows * di * es));
+    MRS_TRY(dev_alloc(bb, &s->xdbl, rows * xd * es));
+    MRS_TRY(dev_alloc(bb, &s->delta, rows * di * es));
+    MRS_TRY(dev_alloc(bb, &s->y, rows * di * es));
+    MRS_TRY(dev_alloc(bb, &s->out, rows * dm * es));
+    if (T > 1) {
+        s->scan_ws_bytes = mrs_ssm_scan_workspace_bytes(bb->batch, T, di, bb->cfg.d_state);
+        MRS_TRY(dev_alloc(bb, &s->scan_ws, s->scan_ws_bytes));
+    }
+    return MRS_OK;
+}
+
+// C[M,N] = A[M,K] (row stride lda) . W[K,N], all row-major; f32 accumulate.
+static int gemm_rm(mrs_backbone *bb, int dtype, void *C, int ldc, const void *A, int lda, const void *W, int M, int N, int K) {
+    const float one = 1.0f, zero = 0.0f;
+    const rocblas_datatype t = blas_type(dtype);
+    MRS_BLAS(rocblas_gemm_ex(bb->blas, rocblas_operation_none, rocblas_operation_none, N, M, K, &one, W, t, N, A, t, lda,
+                             &zero, C, t, ldc, C, t, ldc, rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0));
+    return MRS_OK;
+}
+
+template <typename T>
+static void launch_add_rmsnorm_t(mrs_backbone *bb, float *residual, const void *add, void *out, bool out_f32,
+                                 const float *w, int64_t rows, int64_t out_stride) {
+    const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
+    if (out_f32)
+        hipLaunchKernelGGL((add_rmsnorm_kernel<T, float>), grid, block, 0, bb->stream, residual, (const T *)add, (float *)out, w,
+                           bb->cfg.rms_norm_eps, rows, bb->cfg.d_model, out_stride);
+    else
+        hipLaunchKernelGGL((add_rmsnorm_kernel<T, T>), grid, block, 0, bb->stream, residual, (const T *)add, (T *)out, w,
+                           bb->cfg.rms_norm_eps, rows, bb->cfg.d_model, out_stride);
+}
+static int launch_add_rmsnorm(mrs_backbone *bb, float *residual, const void *add, void *out, bool out_f32, const float *w,
+                              int64_t rows, int64_t out_stride) {
+    MRS_DISPATCH_DTYPE(bb->dtype, T_, launch_add_rmsnorm_t<T_>(bb, residual, add, out, out_f32, w, rows, out_stride));
+    return check_launch("add_rmsnorm_kernel");
+}
+
+// residual <- input (identity) or input . input_proj_w + b (f32 GEMM)
+static int project_input(mrs_backbone *bb, float *residual, const float *input_dev, int64_t rows) {
+    const int dm = bb->cfg.d_model;
+    if (bb->identity_proj) {
+        MRS_HIP(hipMemcpyAsync(residual, input_dev, rows * dm * sizeof(float), hipMemcpyDeviceToDevice, bb->stream));
+        return MRS_OK;
+    }
+    // bias rows first, then accumulate the GEMM on top (beta = 1)
+    {
+        const int64_t n = rows * dm;
+        hipLaunchKernelGGL(bias_rows_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, bb->stream, residual, bb->input_proj_b, n, dm);
+        MRS_TRY(check_launch("bias_rows_kernel"));
+    }
+    const float one = 1.0f;
+    MRS_BLAS(rocblas_gemm_ex(bb->blas, rocblas_operation_none, rocblas_operation_none, dm, (int)rows, bb->input_dim, &one,
+                             bb->input_proj_w, rocblas_datatype_f32_r, dm, input_dev, rocblas_datatype_f32_r, bb->input_dim,
+                             &one, residual, rocblas_datatype_f32_r, dm, residual, rocblas_datatype_f32_r, dm,
+                             rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0));
+    return MRS_OK;
+}
+
+// The layer stack over `rows` = batch*T rows (T = 1: decode chain, T > 1: prefill chain), leaving the
+// final-norm output of every row (decode) or of the last step of each sequence (prefill) in temporal [batch, dm] f32.
+static int run_layers(mrs_backbone *bb, Scratch *s, int T) {
+    const int dm = bb->cfg.d_model, di = bb->di, ds = bb->cfg.d_state, dc = bb->cfg.d_conv, dr = bb->dr, xd = bb->xd;
+    const int B = bb->batch, dt = bb->dtype;
+    const int64_t rows = (int64_t)B * T;
+    const size_t es = esize(dt);
+    const int L = bb->cfg.n_layers;
+    for (int l = 0; l < L; l++) {
+        const LayerDev &lw = bb->layers[l];
+        float *conv = bb->conv_state + (size_t)l * B * di * dc;
+        float *ssm = bb->ssm_state + (size_t)l * B * di * ds;
+        MRS_TRY(launch_add_rmsnorm(bb, s->residual, l == 0 ? nullptr : s->out, s->normed, false, lw.norm_w, rows, dm));
+        MRS_TRY(gemm_rm(bb, dt, s->proj, 2 * di, s->normed, dm, lw.in_proj, (int)rows, 2 * di, dm));
+        const char *z = (const char *)s->proj + (size_t)di * es;  // gate half of in_proj's output
+        const char *xb = (const char *)s->xdbl;
+        if (T == 1) {
+            MRS_TRY(launch_conv1d_step(bb->stream, dt, s->u, conv, s->proj, 2 * di, lw.conv_w, lw.conv_b, B, di, dc, 1));
+            MRS_TRY(gemm_rm(bb, dt, s->xdbl, xd, s->u, di, lw.x_proj, (int)rows, xd, di));
+            MRS_TRY(gemm_rm(bb, dt, s->delta, di, s->xdbl, xd, lw.dt_w, (int)rows, di, dr));
+            MRS_TRY(launch_ssm_step_fused(bb->stream, dt, ssm, s->y, s->delta, lw.dt_b, s->u, xb + es * dr, xb + es * (dr + ds), xd,
+                                          z, 2 * di, 2, lw.a_neg, lw.D, B, di, ds));
+        } else {
+            MRS_TRY(mrs_conv1d_seq_silu(bb->stream, dt, s->u, conv, s->proj, 2 * di, lw.conv_w, lw.conv_b, B, T, di, dc));
+            MRS_TRY(gemm_rm(bb, dt, s->xdbl, xd, s->u, di, lw.x_proj, (int)rows, xd, di));
+            MRS_TRY(gemm_rm(bb, dt, s->delta, di, s->xdbl, xd, lw.dt_w, (int)rows, di, dr));
+            const int64_t n = rows * di;
+            const dim3 grid((unsigned)((n + 255) / 256)), block(256);
+            MRS_DISPATCH_DTYPE(dt, T_, hipLaunchKernelGGL((bias_softplus_kernel<T_>), grid, block, 0, bb->stream, (T_ *)s->delta, lw.dt_b, n, di));
+            MRS_TRY(check_launch("bias_softplus_kernel"));
+            // ScanMode::use_parallel picks the route (src/mamba_ssm/gpu/prefill.rs:910-956)
+            unsigned flags = MRS_GATE_SILU | (lw.s4d ? MRS_A_S4D_REAL : 0);
+            if (!mrs_scan_use_parallel(bb->cfg.scan_mode, T, ds)) flags |= MRS_FORCE_SEQUENTIAL;
+            else if (bb->cfg.scan_mode == MRS_SCAN_PARALLEL && ds == 16 && T >= 64) flags |= MRS_FORCE_PARALLEL;
+            MRS_TRY(mrs_ssm_scan_fwd_ex(bb->stream, dt, ssm, s->y, s->delta, s->u, xb + es * dr, xb + es * (dr + ds), xd, lw.a_neg,
+                                        lw.D, z, 2 * di, flags, s->scan_ws, s->scan_ws_bytes, B, T, di, ds));
+        }
+        MRS_TRY(gemm_rm(bb, dt, s->out, dm, s->y, di, lw.out_proj, (int)rows, dm, di));
+    }
+    if (T == 1) {
+        MRS_TRY(launch_add_rmsnorm(bb, s->residual, s->out, bb->temporal, true, bb->norm_f, rows, dm));
+    } else {
+        // Only the last step of each sequence is kept (gather_last_timestep,
+        // src/mamba_ssm/gpu/prefill.rs:1030-1046), so the final residual add + norm_f runs on those rows only.
+        for (int b = 0; b < B; b++) {
+            const size_t r = (size_t)b * T + (T - 1);
+            MRS_TRY(launch_add_rmsnorm(bb, s->residual + r * dm, (const char *)s->out + r * dm * es, bb->temporal + (size_t)b * dm, true,
+                                       bb->norm_f, 1, dm));
+        }
+    }
+    return MRS_OK;
+}
+
+extern "C" int mrs_backbone_create(mrs_backbone **out, int gpu_ordinal, const mrs_m1_weights *w,
+                                   const mrs_m1_config *cfg, int input_dim, int batch, int dtype) {
+    if (!out || !w || !cfg || !w->layers || !w->norm_f_weight) return fail(MRS_E_NULL, "mrs_backbone_create: null pointer");
+    if (dtype != MRS_F32 && dtype != MRS_F16 && dtype != MRS_BF16) return fail(MRS_E_DTYPE, "mrs_backbone_create: dtype %d", dtype);
+    // MambaConfig::validate (src/config.rs:108-170)
+    if (cfg->d_model < 1 || cfg->d_state < 1 || cfg->d_conv < 1 || cfg->expand < 1 || cfg->n_layers < 1)
+        return fail(MRS_E_SHAPE, "mrs_backbone_create: d_model, d_state, d_conv, expand, n_layers must be > 0");
+    const int64_t di64 = (int64_t)cfg->expand * cfg->d_model;
+    if (cfg->d_model > (1 << 20) || cfg->n_layers > 4096 || di64 > 65535 || cfg->d_state > 256 || cfg->d_conv > 8 || di64 % 4 != 0)
+        return fail(MRS_E_SHAPE, "mrs_backbone_create: config outside the reference's bounds (d_inner<=65535 and %%4==0, d_state<=256, d_conv<=8)");
+    if (batch < 1 || input_dim < 1) return fail(MRS_E_SHAPE, "mrs_backbone_create: batch=%d input_dim=%d", batch, input_dim);
+    const int identity = (w->input_proj_w == nullptr);
+    if (identity && input_dim != cfg->d_model) return fail(MRS_E_SHAPE, "mrs_backbone_create: identity input_proj needs input_dim == d_model");
+    mrs_backbone *bb = new (std::nothrow) mrs_backbone();
+    if (!bb) return fail(MRS_E_HIP, "mrs_backbone_create: out of host memory");
+    bb->cfg = *cfg; bb->input_dim = input_dim; bb->batch = batch; bb->dtype = dtype; bb->device = gpu_ordinal;
+    bb->di = (int)di64; bb->dr = (cfg->d_model + 15) / 16; bb->xd = bb->dr + 2 * cfg->d_state; bb->identity_proj = identity;
+    bb->graph_ready = 0; bb->graph = nullptr; bb->graph_exec = nullptr; bb->prefill_in = nullptr;
+    bb->input_proj_w = nullptr; bb->input_proj_b = nullptr;
+    *out = nullptr;
+#define MRS_CREATE_TRY(expr) do { int rc_ = (expr); if (rc_) { mrs_backbone_destroy(bb); return rc_; } } while (0)
+    {
+        hipError_t e = hipSetDevice(gpu_ordinal);
+        if (e != hipSuccess) { delete bb; return fail(MRS_E_HIP, "hipSetDevice(%d): %s", gpu_ordinal, hipGetErrorString(e)); }
+        e = hipStreamCreateWithFlags(&bb->stream, hipStreamNonBlocking);
+        if (e != hipSuccess) { delete bb; return fail(MRS_E_HIP, "hipStreamCreate: %s", hipGetErrorString(e)); }
+        if (rocblas_create_handle(&bb->blas) != rocblas_status_success) { hipStreamDestroy(bb->stream); delete bb; return fail(MRS_E_HIP, "rocblas_create_handle failed"); }
+        rocblas_set_stream(bb->blas, bb->stream);
+        rocblas_set_pointer_mode(bb->blas, rocblas_pointer_mode_host);
+    }
+    const int dm = cfg->d_model, di = bb->di, ds = cfg->d_state, dc = cfg->d_conv, dr = bb->dr, xd = bb->xd, L = cfg->n_layers;
+    size_t max_bulk = (size_t)dm * 2 * di;
+    if ((size_t)di * xd > max_bulk) max_bulk = (size_t)di * xd;
+    if ((size_t)di * ds > max_bulk) max_bulk = (size_t)di * ds;
+    float *stage = nullptr;
+    MRS_CREATE_TRY(dev_alloc(bb, (void **)&stage, max_bulk * sizeof(float)));
+    if (!identity) {
+        MRS_CREATE_TRY(upload_f32(bb, &bb->input_proj_w, w->input_proj_w, (size_t)input_dim * dm));
+        if (w->input_proj_b) MRS_CREATE_TRY(upload_f32(bb, &bb->input_proj_b, w->input_proj_b, dm));
+        else { MRS_CREATE_TRY(dev_alloc(bb, (void **)&bb->input_proj_b, dm * 4)); hipMemsetAsync(bb->input_proj_b, 0, dm * 4, bb->stream); }
+    }
+    bb->layers.resize(L);
+    int *flag = nullptr;
+    MRS_CREATE_TRY(dev_alloc(bb, (void **)&flag, sizeof(int)));
+    for (int l = 0; l < L; l++) {
+        const mrs_m1_layer_weights &src = w->layers[l];
+        LayerDev &d = bb->layers[l];
+        if (!src.norm_weight || !src.in_proj_w || !src.conv1d_weight || !src.conv1d_bias || !src.x_proj_w || !src.dt_proj_w ||
+            !src.dt_proj_b || !src.a_log || !src.d_param || !src.out_proj_w) {
+            mrs_backbone_destroy(bb);
+            return fail(MRS_E_NULL, "mrs_backbone_create: layer %d has a null weight", l);
+        }
+        MRS_CREATE_TRY(upload_f32(bb, &d.norm_w, src.norm_weight, dm));
+        MRS_CREATE_TRY(upload_bulk(bb, &d.in_proj, src.in_proj_w, (size_t)dm * 2 * di, stage));
+        MRS_CREATE_TRY(upload_f32(bb, &d.conv_w, src.conv1d_weight, (size_t)di * dc));
+        MRS_CREATE_TRY(upload_f32(bb, &d.conv_b, src.conv1d_bias, di));
+        MRS_CREATE_TRY(upload_bulk(bb, &d.x_proj, src.x_proj_w, (size_t)di * xd, stage));
+        MRS_CREATE_TRY(upload_bulk(bb, &d.dt_w, src.dt_proj_w, (size_t)dr * di, stage));
+        MRS_CREATE_TRY(upload_f32(bb, &d.dt_b, src.dt_proj_b, di));
+        MRS_CREATE_TRY(upload_f32(bb, &d.D, src.d_param, di));
+        MRS_CREATE_TRY(upload_bulk(bb, &d.out_proj, src.out_proj_w, (size_t)di * dm, stage));
+        // a_neg = -exp(a_log) once at load (exp_negate, src/mamba_ssm/gpu/inference.rs:266-282)
+        MRS_CREATE_TRY(dev_alloc(bb, (void **)&d.a_neg, (size_t)di * ds * 4));
+        { hipError_t e = hipMemcpyAsync(stage, src.a_log, (size_t)di * ds * 4, hipMemcpyHostToDevice, bb->stream);
+          if (e != hipSuccess) { mrs_backbone_destroy(bb); return fail(MRS_E_HIP, "a_log upload: %s", hipGetErrorString(e)); } }
+        hipLaunchKernelGGL(exp_negate_k, dim3((unsigned)(((size_t)di * ds + 255) / 256)), dim3(256), 0, bb->stream, d.a_neg, stage, (int64_t)di * ds);
+        MRS_CREATE_TRY(mrs_a_neg_is_s4d_real(bb->stream, flag, d.a_neg, di, ds));
+        int hflag = 0;
+        { hipError_t e = hipMemcpyAsync(&hflag, flag, sizeof(int), hipMemcpyDeviceToHost, bb->stream);
+          if (e == hipSuccess) e = hipStreamSynchronize(bb->stream);
+          if (e != hipSuccess) { mrs_backbone_destroy(bb); return fail(MRS_E_HIP, "s4d flag readback: %s", hipGetErrorString(e)); } }
+        d.s4d = hflag;
+    }
+    MRS_CREATE_TRY(upload_f32(bb, &bb->norm_f, w->norm_f_weight, dm));
+    MRS_CREATE_TRY(dev_alloc(bb, (void **)&bb->conv_state, (size_t)L * batch * di * dc * 4));
+    MRS_CREATE_TRY(dev_alloc(bb, (void **)&bb->ssm_state, (size_t)L * batch * di * ds * 4));
+    MRS_CREATE_TRY(dev_alloc(bb, (void **)&bb->d_input, (size_t)batch * input_dim * 4));
+    MRS_CREATE_TRY(dev_alloc(bb, (void **)&bb->temporal, (size_t)batch * dm * 4));
+    MRS_CREATE_TRY(alloc_scratch(bb, &bb->step_s, batch, 1));
+    MRS_CREATE_TRY(mrs_backbone_reset(bb));
+    { hipError_t e = hipStreamSynchronize(bb->stream);
+      if (e != hipSuccess) { mrs_backbone_destroy(bb); return fail(MRS_E_HIP, "create sync: %s", hipGetErrorString(e)); } }
+#undef MRS_CREATE_TRY
+    *out = bb;
+    return MRS_OK;
+}
+
+extern "C" void mrs_backbone_destroy(mrs_backbone *bb) {
+    if (!bb) return;
+    hipSetDevice(bb->device);
+    if (bb->stream) hipStreamSynchronize(bb->stream);
+    if (bb->graph_exec) hipGraphExecDestroy(bb->graph_exec);
+    if (bb->graph) hipGraphDestroy(bb->graph);
+    for (void *p : bb->allocs) hipFree(p);
+    if (bb->blas) rocblas_destroy_handle(bb->blas);
+    if (bb->stream) hipStreamDestroy(bb->stream);
+    delete bb;
+}
+
+extern "C" int mrs_backbone_reset(mrs_backbone *bb) {
+    if (!bb) return fail(MRS_E_NULL, "mrs_backbone_reset: null engine");
+    const size_t L = bb->cfg.n_layers, B = bb->batch;
+    MRS_HIP(hipMemsetAsync(bb->conv_state, 0, L * B * bb->di * bb->cfg.d_conv * 4, bb->stream));
+    MRS_HIP(hipMemsetAsync(bb->ssm_state, 0, L * B * bb->di * bb->cfg.d_state * 4, bb->stream));
+    return MRS_OK;
+}
+
+static int step_body(mrs_backbone *bb) {
+    MRS_TRY(project_input(bb, bb->step_s.residual, bb->d_input, bb->batch));
+    return run_layers(bb, &bb->step_s, 1);
+}
+
+extern "C" int mrs_backbone_step_gpu_only(mrs_backbone *bb) {
+    if (!bb) return fail(MRS_E_NULL, "mrs_backbone_step_gpu_only: null engine");
+    if (bb->graph_ready) { MRS_HIP(hipGraphLaunch(bb->graph_exec, bb->stream)); return MRS_OK; }
+    return step_body(bb);
+}
+
+extern "C" int mrs_backbone_step(mrs_backbone *bb, const float *input, float *output) {
+    if (!bb || !input || !output) return fail(MRS_E_NULL, "mrs_backbone_step: null pointer");
+    MRS_HIP(hipMemcpyAsync(bb->d_input, input, (size_t)bb->batch * bb->input_dim * 4, hipMemcpyHostToDevice, bb->stream));
+    MRS_TRY(mrs_backbone_step_gpu_only(bb));
+    MRS_HIP(hipMemcpyAsync(output, bb->temporal, (size_t)bb->batch * bb->cfg.d_model * 4, hipMemcpyDeviceToHost, bb->stream));
+    MRS_HIP(hipStreamSynchronize(bb->stream));
+    return MRS_OK;
+}
+
+// One eager warm step (library handles pick their kernels), reset, then capture the step body
+// (src/mamba_ssm/gpu/inference.rs:1608-1630, graph_capture.rs:32-66).  The capture is always ended on error.
+extern "C" int mrs_backbone_capture_graph(mrs_backbone *bb) {
+    if (!bb) return fail(MRS_E_NULL, "mrs_backbone_capture_graph: null engine");
+    if (bb->graph_ready) return MRS_OK;
+    // warm step on a copy of the state: save, run, restore
+    const size_t L = bb->cfg.n_layers, B = bb->batch;
+    const size_t cb = L * B * bb->di * bb->cfg.d_conv * 4, sb = L * B * bb->di * bb->cfg.d_state * 4;
+    void *save = nullptr;
+    MRS_HIP(hipMalloc(&save, cb + sb));
+    hipMemcpyAsync(save, bb->conv_state, cb, hipMemcpyDeviceToDevice, bb->stream);
+    hipMemcpyAsync((char *)save + cb, bb->ssm_state, sb, hipMemcpyDeviceToDevice, bb->stream);
+    int rc = step_body(bb);
+    hipMemcpyAsync(bb->conv_state, save, cb, hipMemcpyDeviceToDevice, bb->stream);
+    hipMemcpyAsync(bb->ssm_state, (char *)save + cb, sb, hipMemcpyDeviceToDevice, bb->stream);
+    hipStreamSynchronize(bb->stream);
+    hipFree(save);
+    if (rc) return rc;
+    MRS_HIP(hipStreamBeginCapture(bb->stream, hipStreamCaptureModeThreadLocal));
+    rc = step_body(bb);
+    hipGraph_t g = nullptr;
+    hipError_t e = hipStreamEndCapture(bb->stream, &g);
+    if (rc) { if (g) hipGraphDestroy(g); return rc; }
+    if (e != hipSuccess) return fail(MRS_E_HIP, "hipStreamEndCapture: %s", hipGetErrorString(e));
+    e = hipGraphInstantiate(&bb->graph_exec, g, nullptr, nullptr, 0);
+    if (e != hipSuccess) { hipGraphDestroy(g); return fail(MRS_E_HIP, "hipGraphInstantiate: %s", hipGetErrorString(e)); }
+    bb->graph = g;
+    bb->graph_ready = 1;
+    return MRS_OK;
+}
+
+extern "C" int mrs_backbone_alloc_prefill_scratch(mrs_backbone *bb, int T) {
+    if (!bb) return fail(MRS_E_NULL, "mrs_backbone_alloc_prefill_scratch: null engine");
+    if (T < 1) return fail(MRS_E_SHAPE, "mrs_backbone_alloc_prefill_scratch: T=%d", T);
+    if (bb->prefill_s.rows && bb->prefill_s.T == T) return MRS_OK;
+    if (bb->prefill_s.rows) return fail(MRS_E_SHAPE, "prefill scratch already sized for T=%d (one sequence length per engine)", bb->prefill_s.T);
+    MRS_TRY(alloc_scratch(bb, &bb->prefill_s, (int64_t)bb->batch * T, T));
+    MRS_TRY(dev_alloc(bb, (void **)&bb->prefill_in, (size_t)bb->batch * T * bb->input_dim * 4));
+    return MRS_OK;
+}
+
+extern "C" int mrs_backbone_prefill_device(mrs_backbone *bb, const float *input_dev, int T) {
+    if (!bb || !input_dev) return fail(MRS_E_NULL, "mrs_backbone_prefill_device: null pointer");
+    MRS_TRY(mrs_backbone_alloc_prefill_scratch(bb, T));
+    if ((int64_t)bb->batch * T * bb->di > 0x7fffffffLL) return fail(MRS_E_SHAPE, "prefill: batch*T*d_inner exceeds i32");
+    if (T == 1) return fail(MRS_E_SHAPE, "prefill needs T >= 2; use step for one token");
+    MRS_TRY(project_input(bb, bb->prefill_s.residual, input_dev, (int64_t)bb->batch * T));
+    return run_layers(bb, &bb->prefill_s, T);
+}
+
+extern "C" int mrs_backbone_prefill_sequence(mrs_backbone *bb, const float *input, int T, float *output_last) {
+    if (!bb || !input) return fail(MRS_E_NULL, "mrs_backbone_prefill_sequence: null pointer");
+    MRS_TRY(mrs_backbone_alloc_prefill_scratch(bb, T));
+    MRS_HIP(hipMemcpyAsync(bb->prefill_in, input, (size_t)bb->batch * T * bb->input_dim * 4, hipMemcpyHostToDevice, bb->stream));
+    MRS_TRY(mrs_backbone_prefill_device(bb, bb->prefill_in, T));
+    if (output_last) MRS_HIP(hipMemcpyAsync(output_last, bb->temporal, (size_t)bb->batch * bb->cfg.d_model * 4, hipMemcpyDeviceToHost, bb->stream));
+    MRS_HIP(hipStreamSynchronize(bb->stream));
+    return MRS_OK;
+}
+
+extern "C" void *mrs_backbone_stream(mrs_backbone *bb) { return bb ? (void *)bb->stream : nullptr; }
+extern "C" float *mrs_backbone_temporal_ptr(mrs_backbone *bb) { return bb ? bb->temporal : nullptr; }
+extern "C" float *mrs_backbone_input_ptr(mrs_backbone *bb) { return bb ? bb->d_input : nullptr; }
+extern "C" float *mrs_backbone_prefill_input_ptr(mrs_backbone *bb) { return bb ? bb->prefill_in : nullptr; }
+extern "C" int mrs_backbone_sync(mrs_backbone *bb) {
+    if (!bb) return fail(MRS_E_NULL, "mrs_backbone_sync: null engine");
+    MRS_HIP(hipStreamSynchronize(bb->stream));
+    return MRS_OK;
+}
+
+extern "C" int mrs_backbone_state_ptrs(mrs_backbone *bb, int layer, float **conv_state, float **ssm_state) {
+    if (!bb) return fail(MRS_E_NULL, "mrs_backbone_state_ptrs: null engine");
+    if (layer < 0 || layer >= bb->cfg.n_layers) return fail(MRS_E_SHAPE, "mrs_backbone_state_ptrs: layer %d", layer);
+    if (conv_state) *conv_state = bb->conv_state + (size_t)layer * bb->batch * bb->di * bb->cfg.d_conv;
+    if (ssm_state) *ssm_state = bb->ssm_state + (size_t)layer * bb->batch * bb->di * bb->cfg.d_state;
+    return MRS_OK;
+}
+
+extern "C" int mrs_backbone_download_state(mrs_backbone *bb, int layer, float *conv_state, float *ssm_state) {
+    float *c, *s;
+    MRS_TRY(mrs_backbone_state_ptrs(bb, layer, &c, &s));
+    if (conv_state) MRS_HIP(hipMemcpyAsync(conv_state, c, (size_t)bb->batch * bb->di * bb->cfg.d_conv * 4, hipMemcpyDeviceToHost, bb->stream));
+    if (ssm_state) MRS_HIP(hipMemcpyAsync(ssm_state, s, (size_t)bb->batch * bb->di * bb->cfg.d_state * 4, hipMemcpyDeviceToHost, bb->stream));
+    MRS_HIP(hipStreamSynchronize(bb->stream));
+    return MRS_OK;
+}
+
+// ---- LM: embedding + tied head + greedy loop, all on device -------------------------------
+struct mrs_lm {
+    mrs_backbone *bb;   // decode engine (not owned)
+    int vocab, vocab_padded, dm, batch, dtype;
+    void *embed;        // [vocab_padded, dm] storage dtype (tied lm_head)
+    float *logits;      // [batch, vocab_padded] f32
+    void *hidden;       // [batch, dm] storage dtype copy of temporal for the head GEMM
+    int *tokens;        // [batch] current token ids on device
+    std::vector<void *> allocs;
+    hipGraph_t graph;
+    hipGraphExec_t graph_exec;
+    int graph_ready;
+};
+
+extern "C" int mrs_lm_create(mrs_lm **out, mrs_backbone *bb, const float *embed, int vocab) {
+    if (!out || !bb || !embed) return fail(MRS_E_NULL, "mrs_lm_create: null pointer");
+    if (!bb->identity_proj) return fail(MRS_E_SHAPE, "mrs_lm_create: the LM feeds embeddings straight into the backbone (identity input_proj)");
+    if (vocab < 1) return fail(MRS_E_SHAPE, "mrs_lm_create: vocab=%d", vocab);
+    mrs_lm *lm = new (std::nothrow) mrs_lm();
+    if (!lm) return fail(MRS_E_HIP, "mrs_lm_create: out of host memory");
+    lm->bb = bb; lm->vocab = vocab; lm->vocab_padded = (vocab + 63) & ~63;  // src/hf/load.rs:59
+    lm->dm = bb->cfg.d_model; lm->batch = bb->batch; lm->dtype = bb->dtype; lm->graph_ready = 0; lm->graph = nullptr; lm->graph_exec = nullptr;
+    *out = nullptr;
+    const size_t es = esize(lm->dtype), ne = (size_t)lm->vocab_padded * lm->dm;
+    float *stage = nullptr;
+    auto cleanup = [&]() { for (void *p : lm->allocs) hipFree(p); if (stage) hipFree(stage); delete lm; };
+#define MRS_LM_HIP(expr) do { hipError_t e_ = (expr); if (e_ != hipSuccess) { cleanup(); return fail(MRS_E_HIP, "%s: %s", #expr, hipGetErrorString(e_)); } } while (0)
+    MRS_LM_HIP(hipMalloc(&lm->embed, ne * es)); lm->allocs.push_back(lm->embed);
+    MRS_LM_HIP(hipMalloc((void **)&lm->logits, (size_t)lm->batch * lm->vocab_padded * 4)); lm->allocs.push_back(lm->logits);
+    MRS_LM_HIP(hipMalloc(&lm->hidden, (size_t)lm->batch * lm->dm * es)); lm->allocs.push_back(lm->hidden);
+    MRS_LM_HIP(hipMalloc((void **)&lm->tokens, (size_t)lm->batch * sizeof(int))); lm->allocs.push_back(lm->tokens);
+    MRS_LM_HIP(hipMalloc((void **)&stage, ne * 4));
+    MRS_LM_HIP(hipMemsetAsync(stage, 0, ne * 4, bb->stream));  // padded rows are zero
+    MRS_LM_HIP(hipMemcpyAsync(stage, embed, (size_t)vocab * lm->dm * 4, hipMemcpyHostToDevice, bb->stream));
+    const dim3 grid((unsigned)((ne + 255) / 256)), block(256);
+    if (lm->dtype == MRS_F32) MRS_LM_HIP(hipMemcpyAsync(lm->embed, stage, ne * 4, hipMemcpyDeviceToDevice, bb->stream));
+    else if (lm->dtype == MRS_BF16) hipLaunchKernelGGL((cast_from_f32_kernel<bf16_t>), grid, block, 0, bb->stream, (bf16_t *)lm->embed, stage, (int64_t)ne);
+    else hipLaunchKernelGGL((cast_from_f32_kernel<f16_t>), grid, block, 0, bb->stream, (f16_t *)lm->embed, stage, (int64_t)ne);
+    MRS_LM_HIP(hipStreamSynchronize(bb->stream));
+#undef MRS_LM_HIP
+    hipFree(stage);
+    *out = lm;
+    return MRS_OK;
+}
+
+extern "C" void mrs_lm_destroy(mrs_lm *lm) {
+    if (!lm) return;
+    hipStreamSynchronize(lm->bb->stream);
+    if (lm->graph_exec) hipGraphExecDestroy(lm->graph_exec);
+    if (lm->graph) hipGraphDestroy(lm->graph);
+    for (void *p : lm->allocs) hipFree(p);
+    delete lm;
+}
+
+// logits = norm_f(hidden) . embed^T  (tied head, OP_T on the row-major [V, dm] table: src/mamba_ssm/gpu/blas.rs:709-740)
+static int lm_logits(mrs_lm *lm) {
+    mrs_backbone *bb = lm->bb;
+    const int dm = lm->dm, V = lm->vocab_padded, B = lm->batch;
+    const float one = 1.0f, zero = 0.0f;
+    const void *hid = bb->temporal;
+    rocblas_datatype ht = rocblas_datatype_f32_r;
+    if (lm->dtype != MRS_F32) {
+        const int64_t n = (int64_t)B * dm;
+        const dim3 grid((unsigned)((n + 255) / 256)), block(256);
+        if (lm->dtype == MRS_BF16) hipLaunchKernelGGL((cast_from_f32_kernel<bf16_t>), grid, block, 0, bb->stream, (bf16_t *)lm->hidden, bb->temporal, n);
+        else hipLaunchKernelGGL((cast_from_f32_kernel<f16_t>), grid, block, 0, bb->stream, (f16_t *)lm->hidden, bb->temporal, n);
+        hid = lm->hidden; ht = blas_type(lm->dtype);
+    }
+    MRS_BLAS(rocblas_gemm_ex(bb->blas, rocblas_operation_transpose, rocblas_operation_none, V, B, dm, &one, lm->embed,
+                             blas_type(lm->dtype), dm, hid, ht, dm, &zero, lm->logits, rocblas_datatype_f32_r, V, lm->logits,
+                             rocblas_datatype_f32_r, V, rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0));
+    return MRS_OK;
+}
+
+static int lm_decode_body(mrs_lm *lm) {
+    mrs_backbone *bb = lm->bb;
+    const int64_t n = (int64_t)lm->batch * lm->dm;
+    const dim3 grid((unsigned)((n + 255) / 256)), block(256);
+    MRS_DISPATCH_DTYPE(lm->dtype, T_, hipLaunchKernelGGL((embed_gather_kernel<T_>), grid, block, 0, bb->stream, bb->d_input,
+                                                         (const T_ *)lm->embed, lm->tokens, (int64_t)lm->batch, lm->dm, lm->vocab));
+    MRS_TRY(step_body(bb));
+    MRS_TRY(lm_logits(lm));
+    hipLaunchKernelGGL(argmax_last_kernel, dim3((unsigned)lm->batch), dim3(256), 0, bb->stream, lm->tokens, lm->logits, lm->vocab,
+                       (int64_t)lm->vocab_padded);
+    return check_launch("argmax_last_kernel");
+}
+
+extern "C" int mrs_lm_set_tokens(mrs_lm *lm, const int *tokens) {
+    if (!lm || !tokens) return fail(MRS_E_NULL, "mrs_lm_set_tokens: null pointer");
+    MRS_HIP(hipMemcpyAsync(lm->tokens, tokens, (size_t)lm->batch * sizeof(int), hipMemcpyHostToDevice, lm->bb->stream));
+    return MRS_OK;
+}
+
+// One greedy decode step for every batch row, entirely on device: gather embedding of the current
+// token, backbone step, tied head, argmax -> next token (left in the device token buffer).
+extern "C" int mrs_lm_decode_step(mrs_lm *lm) {
+    if (!lm) return fail(MRS_E_NULL, "mrs_lm_decode_step: null engine");
+    if (lm->graph_ready) { MRS_HIP(hipGraphLaunch(lm->graph_exec, lm->bb->stream)); return MRS_OK; }
+    return lm_decode_body(lm);
+}
+
+extern "C" int mrs_lm_capture_graph(mrs_lm *lm) {
+    if (!lm) return fail(MRS_E_NULL, "mrs_lm_capture_graph: null engine");
+    if (lm->graph_ready) return MRS_OK;
+    mrs_backbone *bb = lm->bb;
+    const size_t L = bb->cfg.n_layers, B = bb->batch;
+    const size_t cb = L * B * bb->di * bb->cfg.d_conv * 4, sb = L * B * bb->di * bb->cfg.d_state * 4, tb = B * sizeof(int);
+    void *save = nullptr;
+    MRS_HIP(hipMalloc(&save, cb + sb + tb));
+    hipMemcpyAsync(save, bb->conv_state, cb, hipMemcpyDeviceToDevice, bb->stream);
+    hipMemcpyAsync((char *)save + cb, bb->ssm_state, sb, hipMemcpyDeviceToDevice, bb->stream);
+    hipMemcpyAsync((char *)save + cb + sb, lm->tokens, tb, hipMemcpyDeviceToDevice, bb->stream);
+    int rc = lm_decode_body(lm);   // warm, eager
+    hipMemcpyAsync(bb->conv_state, save, cb, hipMemcpyDeviceToDevice, bb->stream);
+    hipMemcpyAsync(bb->ssm_state, (char *)save + cb, sb, hipMemcpyDeviceToDevice, bb->stream);
+    hipMemcpyAsync(lm->tokens, (char *)save + cb + sb, tb, hipMemcpyDeviceToDevice, bb->stream);
+    hipStreamSynchronize(bb->stream);
+    hipFree(save);
+    if (rc) return rc;
+    MRS_HIP(hipStreamBeginCapture(bb->stream, hipStreamCaptureModeThreadLocal));
+    rc = lm_decode_body(lm);
+    hipGraph_t g = nullptr;
+    hipError_t e = hipStreamEndCapture(bb->stream, &g);
+    if (rc) { if (g) hipGraphDestroy(g); return rc; }
+    if (e != hipSuccess) return fail(MRS_E_HIP, "hipStreamEndCapture: %s", hipGetErrorString(e));
+    e = hipGraphInstantiate(&lm->graph_exec, g, nullptr, nullptr, 0);
+    if (e != hipSuccess) { hipGraphDestroy(g); return fail(MRS_E_HIP, "hipGraphInstantiate: %s", hipGetErrorString(e)); }
+    lm->graph = g; lm->graph_ready = 1;
+    return MRS_OK;
+}
+
+extern "C" int mrs_lm_get_tokens(mrs_lm *lm, int *tokens) {
+    if (!lm || !tokens) return fail(MRS_E_NULL, "mrs_lm_get_tokens: null pointer");
+    MRS_HIP(hipMemcpyAsync(tokens, lm->tokens, (size_t)lm->batch * sizeof(int), hipMemcpyDeviceToHost, lm->bb->stream));
+    MRS_HIP(hipStreamSynchronize(lm->bb->stream));
+    return MRS_OK;
+}
+
+extern "C" int mrs_lm_last_logits(mrs_lm *lm, float *logits) {
+    if (!lm || !logits) return fail(MRS_E_NULL, "mrs_lm_last_logits: null pointer");
+    MRS_HIP(hipMemcpy2DAsync(logits, (size_t)lm->vocab * 4, lm->logits, (size_t)lm->vocab_padded * 4, (size_t)lm->vocab * 4, lm->batch,
+                             hipMemcpyDeviceToHost, lm->bb->stream));
+    MRS_HIP(hipStreamSynchronize(lm->bb->stream));
+    return MRS_OK;
+}
+
+// Prefill helper for the LM: token ids [batch, T] (host) -> embeddings on device -> backbone prefill,
+// then the head on the last position; the greedy next token of every row is left in the token buffer.
+extern "C" int mrs_lm_prefill(mrs_lm *lm, mrs_backbone *prefill_bb, const int *tokens, int T) {
+    if (!lm || !prefill_bb || !tokens) return fail(MRS_E_NULL, "mrs_lm_prefill: null pointer");
+    if (prefill_bb->cfg.d_model != lm->dm || prefill_bb->dtype != lm->dtype || !prefill_bb->identity_proj)
+        return fail(MRS_E_SHAPE, "mrs_lm_prefill: prefill engine does not match the LM");
+    MRS_TRY(mrs_backbone_alloc_prefill_scratch(prefill_bb, T));
+    const int64_t rows = (int64_t)prefill_bb->batch * T;
+    int *dtok = nullptr;
+    MRS_HIP(hipMalloc((void **)&dtok, rows * sizeof(int)));
+    hipMemcpyAsync(dtok, tokens, rows * sizeof(int), hipMemcpyHostToDevice, prefill_bb->stream);
+    const int64_t n = rows * lm->dm;
+    const dim3 grid((unsigned)((n + 255) / 256)), block(256);
+    MRS_DISPATCH_DTYPE(lm->dtype, T_, hipLaunchKernelGGL((embed_gather_kernel<T_>), grid, block, 0, prefill_bb->stream, prefill_bb->prefill_in,
+                                                         (const T_ *)lm->embed, dtok, rows, lm->dm, lm->vocab));
+    int rc = mrs_backbone_prefill_device(prefill_bb, prefill_bb->prefill_in, T);
+    if (!rc && prefill_bb == lm->bb) {
+        rc = lm_logits(lm);
+        if (!rc) {
+            hipLaunchKernelGGL(argmax_last_kernel, dim3((unsigned)lm->batch), dim3(256), 0, lm->bb->stream, lm->tokens, lm->logits,
+                               lm->vocab, (int64_t)lm->vocab_padded);
+            rc = check_launch("argmax_last_kernel");
+        }
+    }
+    hipStreamSynchronize(prefill_bb->stream);
+    hipFree(dtok);
+    return rc;
+}

@@ -27,7 +27,7 @@ __global__ __launch_bounds__(kWave) void ssm_scan_seq_kernel(
     float *__restrict__ h, T *__restrict__ y, const T *__restrict__ delta, const T *__restrict__ u,
     const T *__restrict__ Bm, const T *__restrict__ Cm, int64_t bc_stride,
     const float *__restrict__ a_neg, const float *__restrict__ Dp, const T *__restrict__ gate,
-    int Tlen, int di, int ds, int tiles) {
+    int64_t gate_stride, int Tlen, int di, int ds, int tiles) {
     constexpr int CPW = kWave / LPC;
     const int b = blockIdx.x / tiles;
     const int tile = blockIdx.x - b * tiles;
@@ -77,8 +77,8 @@ __global__ __launch_bounds__(kWave) void ssm_scan_seq_kernel(
         }
 #pragma unroll
         for (int m = 1; m < LPC; m <<= 1) acc += __shfl_xor(acc, m, kWave);
-        if (GATE == 1) acc *= Store<T>::ld(gate + i);
-        if (GATE == 2) acc *= silu(Store<T>::ld(gate + i));
+        if (GATE == 1) acc *= Store<T>::ld(gate + row * gate_stride + dd);
+        if (GATE == 2) acc *= silu(Store<T>::ld(gate + row * gate_stride + dd));
         if (live && g == 0) Store<T>::st(y + i, acc);
     }
     if (live) {
@@ -91,13 +91,13 @@ __global__ __launch_bounds__(kWave) void ssm_scan_seq_kernel(
 template <typename T, int LPC, bool S4D>
 static int launch_seq_gate(hipStream_t st, int gate_mode, float *h, T *y, const T *delta, const T *u,
                            const T *Bm, const T *Cm, int64_t bc_stride, const float *a_neg,
-                           const float *D, const T *gate, int batch, int Tlen, int di, int ds) {
+                           const float *D, const T *gate, int64_t gate_stride, int batch, int Tlen, int di, int ds) {
     constexpr int CPW = kWave / LPC;
     const int tiles = (di + CPW - 1) / CPW;
     const dim3 grid((unsigned)(batch * tiles)), block(kWave);
 #define MRS_LAUNCH(G)                                                                              \
     hipLaunchKernelGGL((ssm_scan_seq_kernel<T, LPC, S4D, G>), grid, block, 0, st, h, y, delta, u, Bm, \
-                       Cm, bc_stride, a_neg, D, gate, Tlen, di, ds, tiles)
+                       Cm, bc_stride, a_neg, D, gate, gate_stride, Tlen, di, ds, tiles)
     if (gate_mode == 0) MRS_LAUNCH(0);
     else if (gate_mode == 1) MRS_LAUNCH(1);
     else MRS_LAUNCH(2);
@@ -108,11 +108,11 @@ static int launch_seq_gate(hipStream_t st, int gate_mode, float *h, T *y, const 
 template <typename T>
 static int launch_seq(hipStream_t st, bool s4d, int gate_mode, float *h, void *y, const void *delta,
                       const void *u, const void *Bm, const void *Cm, int64_t bc_stride,
-                      const float *a_neg, const float *D, const void *gate, int batch, int Tlen,
+                      const float *a_neg, const float *D, const void *gate, int64_t gate_stride, int batch, int Tlen,
                       int di, int ds) {
 #define MRS_ARGS                                                                                     \
     st, gate_mode, h, (T *)y, (const T *)delta, (const T *)u, (const T *)Bm, (const T *)Cm, bc_stride, \
-        a_neg, D, (const T *)gate, batch, Tlen, di, ds
+        a_neg, D, (const T *)gate, gate_stride, batch, Tlen, di, ds
 #define MRS_LPC(L) return s4d ? launch_seq_gate<T, L, true>(MRS_ARGS) : launch_seq_gate<T, L, false>(MRS_ARGS)
     if (ds <= 16) { MRS_LPC(1); }
     if (ds <= 32) { MRS_LPC(2); }
@@ -468,7 +468,7 @@ template <typename T, bool S4D, int GATE>
 __global__ __launch_bounds__(kWave) void chunk_out_kernel(
     float *__restrict__ h, T *__restrict__ y, const T *__restrict__ delta, const T *__restrict__ u,
     const float *__restrict__ Bt, const float *__restrict__ Cf, int64_t cf_stride,
-    const float *__restrict__ a_neg, const float *__restrict__ Dp, const T *__restrict__ gate,
+    const float *__restrict__ a_neg, const float *__restrict__ Dp, const T *__restrict__ gate, int64_t gate_stride,
     const float *__restrict__ h0copy, const float *__restrict__ S, const float *__restrict__ sumd,
     int Tlen, int di, int tiles, int nchunk, int len) {
     using raw_t = typename RawElem<T>::type;
@@ -495,8 +495,9 @@ __global__ __launch_bounds__(kWave) void chunk_out_kernel(
     const int64_t row0 = (int64_t)b * Tlen;
     const int64_t slab = (int64_t)Tlen * di - d0;
     const LaneBuf<T> dbuf(delta + row0 * di + d0, slab), ubuf(u + row0 * di + d0, slab);
-    const LaneBuf<T> gbuf(GATE ? gate + row0 * di + d0 : delta, GATE ? slab : 0), ybuf(y + row0 * di + d0, slab);
+    const LaneBuf<T> gbuf(GATE ? gate + row0 * gate_stride + d0 : delta, GATE ? (int64_t)Tlen * gate_stride - d0 : 0), ybuf(y + row0 * di + d0, slab);
     const unsigned row_bytes = (unsigned)di * (unsigned)sizeof(T);
+    const unsigned gate_row_bytes = (unsigned)gate_stride * (unsigned)sizeof(T);
     const __amdgpu_buffer_rsrc_t btbuf =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(Bt + row0 * 16), 0, (int)((int64_t)Tlen * 64), 0x00020000);
     const unsigned bt_lane = (threadIdx.x & 3) * 16;  // this lane's 4 floats inside a regrouped row
@@ -510,7 +511,7 @@ __global__ __launch_bounds__(kWave) void chunk_out_kernel(
             const unsigned tt = (unsigned)min(tg + k, t1 - 1);
             rd[k] = dbuf.ld(lxb, tt * row_bytes);
             ru[k] = ubuf.ld(lxb, tt * row_bytes);
-            if (GATE) rg[k] = gbuf.ld(lxb, tt * row_bytes);
+            if (GATE) rg[k] = gbuf.ld(lxb, tt * gate_row_bytes);
             bv[k] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(btbuf, bt_lane, tt * 64u, 0));
         }
     };
@@ -566,7 +567,7 @@ template <> struct IsF32<float> { static constexpr bool value = true; };
 template <typename T, bool S4D>
 static int launch_split_s4d(hipStream_t st, int gate_mode, float *h, T *y, const T *delta, const T *u,
                             const T *Bm, const T *Cm, int64_t bc_stride, const float *a_neg,
-                            const float *D, const T *gate, float *ws, SplitPlan plan, int batch,
+                            const float *D, const T *gate, int64_t gate_stride, float *ws, SplitPlan plan, int batch,
                             int Tlen, int di) {
     const int tiles = (di + kWave - 1) / kWave;
     const int C = plan.nchunk, L = plan.len;
@@ -583,7 +584,7 @@ static int launch_split_s4d(hipStream_t st, int gate_mode, float *h, T *y, const
     const int64_t bcf = IsF32<T>::value ? bc_stride : 16;
 #define MRS_LAUNCH(G)                                                                                   \
     hipLaunchKernelGGL((chunk_out_kernel<T, S4D, G>), gridB, block, 0, st, h, y, delta, u, w.Bt, Cf, bcf, \
-                       a_neg, D, gate, w.h0copy, w.S, w.sumd, Tlen, di, tiles, C, L)
+                       a_neg, D, gate, gate_stride, w.h0copy, w.S, w.sumd, Tlen, di, tiles, C, L)
     if (gate_mode == 0) MRS_LAUNCH(0);
     else if (gate_mode == 1) MRS_LAUNCH(1);
     else MRS_LAUNCH(2);
@@ -594,11 +595,11 @@ static int launch_split_s4d(hipStream_t st, int gate_mode, float *h, T *y, const
 template <typename T>
 static int launch_split(hipStream_t st, bool s4d, int gate_mode, float *h, void *y, const void *delta,
                         const void *u, const void *Bm, const void *Cm, int64_t bc_stride,
-                        const float *a_neg, const float *D, const void *gate, float *ws, SplitPlan plan,
+                        const float *a_neg, const float *D, const void *gate, int64_t gate_stride, float *ws, SplitPlan plan,
                         int batch, int Tlen, int di) {
 #define MRS_ARGS                                                                                       \
     st, gate_mode, h, (T *)y, (const T *)delta, (const T *)u, (const T *)Bm, (const T *)Cm, bc_stride, \
-        a_neg, D, (const T *)gate, ws, plan, batch, Tlen, di
+        a_neg, D, (const T *)gate, gate_stride, ws, plan, batch, Tlen, di
     return s4d ? launch_split_s4d<T, true>(MRS_ARGS) : launch_split_s4d<T, false>(MRS_ARGS);
 #undef MRS_ARGS
 }
@@ -637,8 +638,8 @@ extern "C" size_t mrs_ssm_scan_workspace_bytes(int batch, int T, int d_inner, in
 
 extern "C" int mrs_ssm_scan_fwd_ex(void *stream, int dtype, float *h, void *y, const void *delta,
                                    const void *u, const void *B, const void *C, int64_t bc_stride,
-                                   const float *a_neg, const float *D, const void *gate, unsigned flags,
-                                   void *workspace, size_t workspace_bytes, int batch, int T,
+                                   const float *a_neg, const float *D, const void *gate, int64_t gate_stride,
+                                   unsigned flags, void *workspace, size_t workspace_bytes, int batch, int T,
                                    int d_inner, int d_state) {
     int rc = scan_check("mrs_ssm_scan_fwd_ex", dtype, h, y, delta, u, B, C, a_neg, D, bc_stride, batch, T, d_inner, d_state);
     if (rc) return rc;
@@ -648,6 +649,8 @@ extern "C" int mrs_ssm_scan_fwd_ex(void *stream, int dtype, float *h, void *y, c
     if (flags & MRS_GATE_PREACT) gate_mode = 1;
     if (flags & MRS_GATE_SILU) gate_mode = 2;
     if (gate_mode && !gate) return fail(MRS_E_NULL, "mrs_ssm_scan_fwd_ex: gate flag set but gate is NULL");
+    if (gate_stride == 0) gate_stride = d_inner;
+    if (gate_mode && gate_stride < d_inner) return fail(MRS_E_SHAPE, "mrs_ssm_scan_fwd_ex: gate_stride=%lld < d_inner=%d", (long long)gate_stride, d_inner);
     const bool s4d = (flags & MRS_A_S4D_REAL) != 0;
     hipStream_t st = as_stream(stream);
     if ((flags & MRS_FORCE_SEQUENTIAL) && (flags & MRS_FORCE_PARALLEL))
@@ -669,16 +672,16 @@ extern "C" int mrs_ssm_scan_fwd_ex(void *stream, int dtype, float *h, void *y, c
         if (workspace_bytes < need)
             return fail(MRS_E_WORKSPACE, "mrs_ssm_scan_fwd_ex: workspace %zu bytes < %zu needed", workspace_bytes, need);
         if (!aligned(workspace, 256)) return fail(MRS_E_ALIGN, "mrs_ssm_scan_fwd_ex: workspace must be 256-byte aligned");
-        MRS_DISPATCH_DTYPE(dtype, T_, return launch_split<T_>(st, s4d, gate_mode, h, y, delta, u, B, C, bc_stride, a_neg, D, gate,
+        MRS_DISPATCH_DTYPE(dtype, T_, return launch_split<T_>(st, s4d, gate_mode, h, y, delta, u, B, C, bc_stride, a_neg, D, gate, gate_stride,
                                                              (float *)workspace, plan, batch, T, d_inner));
     }
-    MRS_DISPATCH_DTYPE(dtype, T_, return launch_seq<T_>(st, s4d, gate_mode, h, y, delta, u, B, C, bc_stride, a_neg, D, gate, batch, T, d_inner, d_state));
+    MRS_DISPATCH_DTYPE(dtype, T_, return launch_seq<T_>(st, s4d, gate_mode, h, y, delta, u, B, C, bc_stride, a_neg, D, gate, gate_stride, batch, T, d_inner, d_state));
     return MRS_OK;
 }
 
 extern "C" int mrs_ssm_scan_fwd(void *stream, int dtype, float *h, void *y, const void *delta,
                                 const void *u, const void *B, const void *C, const float *a_neg,
                                 const float *D, int batch, int T, int d_inner, int d_state) {
-    return mrs_ssm_scan_fwd_ex(stream, dtype, h, y, delta, u, B, C, d_state, a_neg, D, nullptr,
+    return mrs_ssm_scan_fwd_ex(stream, dtype, h, y, delta, u, B, C, d_state, a_neg, D, nullptr, 0,
                                MRS_GATE_NONE, nullptr, 0, batch, T, d_inner, d_state);
 }

@@ -13,12 +13,18 @@ namespace mrs {
 
 // B and C of batch row b are read at xdbl + b*stride + {b_off, c_off}; the plain
 // step passes stride = ds and separate base pointers.
-template <typename T, int LG, bool GATE>
+// softplus with the reference's pass-through above 20 (kernels/activations.cu:39)
+__device__ __forceinline__ float softplus20(float v) { return v > 20.0f ? v : log1pf(fast_exp2(v * kLog2e)); }
+
+// gate_mode: 0 none, 1 y *= gate, 2 y *= silu(gate); gate rows have gate_stride elements.
+// dt_bias != nullptr: delta holds the raw dt_proj output and softplus(delta + dt_bias[d]) is applied here
+// (dt_proj bias add + softplus_forward of the decode chain, src/mamba_ssm/gpu/inference.rs:1129-1158).
+template <typename T, int LG>
 __global__ __launch_bounds__(256) void ssm_step_kernel(
     float *__restrict__ h, T *__restrict__ y, const T *__restrict__ delta, const T *__restrict__ u,
     const T *__restrict__ Bbase, const T *__restrict__ Cbase, int64_t bc_stride,
-    const T *__restrict__ gate, const float *__restrict__ a_neg, const float *__restrict__ Dp,
-    int64_t total, int di, int ds) {
+    const T *__restrict__ gate, int64_t gate_stride, int gate_mode, const float *__restrict__ dt_bias,
+    const float *__restrict__ a_neg, const float *__restrict__ Dp, int64_t total, int di, int ds) {
     // total = batch*d_inner rows; ds == 4*LG here.
     const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int64_t rowi = gid / LG;
@@ -29,7 +35,8 @@ __global__ __launch_bounds__(256) void ssm_step_kernel(
     const int d = (int)(r - (int64_t)b * di);
     float4 hv = *reinterpret_cast<const float4 *>(h + r * ds + 4 * g);
     const float4 av = *reinterpret_cast<const float4 *>(a_neg + (int64_t)d * ds + 4 * g);
-    const float dl = Store<T>::ld(delta + r);
+    float dl = Store<T>::ld(delta + r);
+    if (dt_bias) dl = softplus20(dl + dt_bias[d]);
     const float uu = Store<T>::ld(u + r);
     const float du = dl * uu;
     const T *Br = Bbase + (int64_t)b * bc_stride + 4 * g;
@@ -49,24 +56,26 @@ __global__ __launch_bounds__(256) void ssm_step_kernel(
         *reinterpret_cast<float4 *>(h + r * ds + 4 * g) = hv;
         if (g == 0) {
             acc = fmaf(Dp[d], uu, acc);
-            if (GATE) acc *= Store<T>::ld(gate + r);
+            if (gate_mode == 1) acc *= Store<T>::ld(gate + (int64_t)b * gate_stride + d);
+            if (gate_mode == 2) acc *= silu(Store<T>::ld(gate + (int64_t)b * gate_stride + d));
             Store<T>::st(y + r, acc);
         }
     }
 }
 
 // Any d_state (1..=256), one lane per (b,d), states streamed in order.
-template <typename T, bool GATE>
+template <typename T>
 __global__ __launch_bounds__(256) void ssm_step_generic_kernel(
     float *__restrict__ h, T *__restrict__ y, const T *__restrict__ delta, const T *__restrict__ u,
     const T *__restrict__ Bbase, const T *__restrict__ Cbase, int64_t bc_stride,
-    const T *__restrict__ gate, const float *__restrict__ a_neg, const float *__restrict__ Dp,
-    int64_t total, int di, int ds) {
+    const T *__restrict__ gate, int64_t gate_stride, int gate_mode, const float *__restrict__ dt_bias,
+    const float *__restrict__ a_neg, const float *__restrict__ Dp, int64_t total, int di, int ds) {
     const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (r >= total) return;
     const int b = (int)(r / di);
     const int d = (int)(r - (int64_t)b * di);
-    const float dl = Store<T>::ld(delta + r);
+    float dl = Store<T>::ld(delta + r);
+    if (dt_bias) dl = softplus20(dl + dt_bias[d]);
     const float uu = Store<T>::ld(u + r);
     const float du = dl * uu;
     const float x = dl * kLog2e;
@@ -80,17 +89,20 @@ __global__ __launch_bounds__(256) void ssm_step_generic_kernel(
         hr[n] = hn;
         acc = fmaf(hn, Store<T>::ld(Cr + n), acc);
     }
-    if (GATE) acc *= Store<T>::ld(gate + r);
+    if (gate_mode == 1) acc *= Store<T>::ld(gate + (int64_t)b * gate_stride + d);
+    if (gate_mode == 2) acc *= silu(Store<T>::ld(gate + (int64_t)b * gate_stride + d));
     Store<T>::st(y + r, acc);
 }
 
 template <typename T>
 static int launch_step(hipStream_t st, float *h, void *y, const void *delta, const void *u,
                        const void *Bb, const void *Cb, int64_t bc_stride, const void *gate,
-                       const float *a_neg, const float *D, int batch, int di, int ds) {
+                       int64_t gate_stride, int gate_mode, const float *dt_bias, const float *a_neg,
+                       const float *D, int batch, int di, int ds) {
     const int64_t total = (int64_t)batch * di;
+    if (!gate) gate_mode = 0;
 #define MRS_ARGS h, (T *)y, (const T *)delta, (const T *)u, (const T *)Bb, (const T *)Cb, bc_stride, \
-                 (const T *)gate, a_neg, D, total, di, ds
+                 (const T *)gate, gate_stride, gate_mode, dt_bias, a_neg, D, total, di, ds
     const bool vec_ok = aligned(h, 16) && aligned(a_neg, 16);
     int lg = 0;
     if (vec_ok && (ds == 4 || ds == 8 || ds == 16 || ds == 32 || ds == 64 || ds == 128 || ds == 256)) lg = ds / 4;
@@ -99,22 +111,25 @@ static int launch_step(hipStream_t st, float *h, void *y, const void *delta, con
         const int64_t blocks = (threads + 255) / 256;
         if (blocks > 0x7fffffffLL) return fail(MRS_E_SHAPE, "ssm step: grid too large");
         const dim3 grid((unsigned)blocks), block(256);
-#define MRS_LG(L)                                                                                      \
-    case L:                                                                                            \
-        if (gate) hipLaunchKernelGGL((ssm_step_kernel<T, L, true>), grid, block, 0, st, MRS_ARGS);     \
-        else hipLaunchKernelGGL((ssm_step_kernel<T, L, false>), grid, block, 0, st, MRS_ARGS);         \
-        break
+#define MRS_LG(L) case L: hipLaunchKernelGGL((ssm_step_kernel<T, L>), grid, block, 0, st, MRS_ARGS); break
         switch (lg) { MRS_LG(1); MRS_LG(2); MRS_LG(4); MRS_LG(8); MRS_LG(16); MRS_LG(32); MRS_LG(64); }
 #undef MRS_LG
     } else {
         const int64_t blocks = (total + 255) / 256;
         if (blocks > 0x7fffffffLL) return fail(MRS_E_SHAPE, "ssm step: grid too large");
-        const dim3 grid((unsigned)blocks), block(256);
-        if (gate) hipLaunchKernelGGL((ssm_step_generic_kernel<T, true>), grid, block, 0, st, MRS_ARGS);
-        else hipLaunchKernelGGL((ssm_step_generic_kernel<T, false>), grid, block, 0, st, MRS_ARGS);
+        hipLaunchKernelGGL((ssm_step_generic_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, st, MRS_ARGS);
     }
 #undef MRS_ARGS
     return check_launch("ssm_step_kernel");
+}
+
+int launch_ssm_step_fused(hipStream_t st, int dtype, float *h, void *y, const void *delta, const float *dt_bias,
+                          const void *u, const void *Bb, const void *Cb, int64_t bc_stride, const void *gate,
+                          int64_t gate_stride, int gate_mode, const float *a_neg, const float *D, int batch,
+                          int di, int ds) {
+    MRS_DISPATCH_DTYPE(dtype, T_, return launch_step<T_>(st, h, y, delta, u, Bb, Cb, bc_stride, gate, gate_stride, gate_mode,
+                                                         dt_bias, a_neg, D, batch, di, ds));
+    return MRS_OK;
 }
 
 static int step_check(const char *fn, int dtype, const void *h, const void *y, const void *delta,
@@ -139,7 +154,7 @@ extern "C" int mrs_ssm_step(void *stream, int dtype, float *h, void *y, const vo
     int rc = step_check("mrs_ssm_step", dtype, h, y, delta, u, B, C, a_neg, D, batch, d_inner, d_state);
     if (rc) return rc;
     hipStream_t st = as_stream(stream);
-    MRS_DISPATCH_DTYPE(dtype, T_, return launch_step<T_>(st, h, y, delta, u, B, C, d_state, nullptr, a_neg, D, batch, d_inner, d_state));
+    MRS_DISPATCH_DTYPE(dtype, T_, return launch_step<T_>(st, h, y, delta, u, B, C, d_state, nullptr, 0, 0, nullptr, a_neg, D, batch, d_inner, d_state));
     return MRS_OK;
 }
 
@@ -156,6 +171,6 @@ extern "C" int mrs_ssm_step_gather_gate(void *stream, int dtype, float *h, void 
     const char *xb = static_cast<const char *>(xdbl);
     hipStream_t st = as_stream(stream);
     MRS_DISPATCH_DTYPE(dtype, T_, return launch_step<T_>(st, h, y, delta, u, xb + es * b_offset, xb + es * c_offset,
-                                                         xdbl_stride, gate_silu, a_neg, D, batch, d_inner, d_state));
+                                                         xdbl_stride, gate_silu, d_inner, 1, nullptr, a_neg, D, batch, d_inner, d_state));
     return MRS_OK;
 }

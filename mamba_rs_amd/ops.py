@@ -81,7 +81,7 @@ def ssm_scan_fwd(h, y, delta, u, B, C, a_neg, D, *, gate=None, flags: int = 0, w
     strided views into xdbl [batch,T,xd] (same row stride for both)."""
     batch, T, di = delta.shape
     ds = a_neg.shape[1]
-    _dev(h, y, delta, u, a_neg, D, gate, workspace); _f32(h, a_neg, D)
+    _dev(h, y, delta, u, a_neg, D, workspace); _f32(h, a_neg, D)
     dt = _act_dtype(delta, u, y, B, C, *([gate] if gate is not None else []))
     for t in (B, C):
         if not t.is_cuda or t.stride(-1) != 1 or t.shape != (batch, T, ds):
@@ -91,11 +91,14 @@ def ssm_scan_fwd(h, y, delta, u, B, C, a_neg, D, *, gate=None, flags: int = 0, w
         raise ValueError("B and C must share one row stride and be row-dense over [batch*T]")
     if h.shape != (batch, di, ds) or y.shape != delta.shape or u.shape != delta.shape or a_neg.shape != (di, ds) or D.shape != (di,):
         raise ValueError("shape mismatch")
-    if gate is not None and gate.shape != delta.shape:
-        raise ValueError("gate shape mismatch")
+    gate_stride = 0
+    if gate is not None:
+        if gate.shape != delta.shape or gate.stride(2) != 1 or gate.stride(0) != T * gate.stride(1):
+            raise ValueError("gate must be [batch,T,d_inner], row-dense over [batch*T], unit inner stride")
+        gate_stride = gate.stride(1)
     ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
     _lib.call("mrs_ssm_scan_fwd_ex", _stream(), int(dt), _p(h), _p(y), _p(delta), _p(u), _p(B), _p(C), bc_stride,
-              _p(a_neg), _p(D), _p(gate), flags, _p(workspace), ws_bytes, batch, T, di, ds)
+              _p(a_neg), _p(D), _p(gate), gate_stride, flags, _p(workspace), ws_bytes, batch, T, di, ds)
     return y
 
 
