@@ -19,6 +19,9 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBPS = 8000.0
+# HBM bytes per scan call (both kernels) from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script, each counter
+# scaled by what it reads for a 256 MiB device copy (--copy-calibration): 282.4 MiB read + 63.5 MiB written.
+MEASURED_SCAN_TRAFFIC_BYTES = int((2.0 * (50767 + 92635) + 1.0 * (15056 + 49920)) * 1024)
 
 
 def scan_algorithmic_bytes(batch, T, di, ds, s, gated=True):
@@ -53,6 +56,11 @@ def gpu_leg(args, inp, shape):
     def step():
         ops.ssm_scan_fwd(h, y, delta, u, Bm, Cm, a_neg, D, gate=z, flags=flags, workspace=ws)
 
+    if args.copy_calibration:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        dst.copy_(src)            # 256 MiB read + 256 MiB written
+        torch.cuda.synchronize()
     for _ in range(args.warmup):
         h.zero_()
         step()
@@ -103,12 +111,110 @@ def cpu_leg(inp, shape, nbytes, budget_s=12.0):
                 ms_per_step=best * 1e3)
 
 
+def lm_leg(name, cfg_kw, vocab, prefill_bt, decode_b, decode_steps, seed=42):
+    """Prefill tok/s and greedy-decode us/step of a random-init LM-shaped backbone (bf16 storage):
+    token ids -> device embedding gather -> backbone (-> tied head -> argmax for decode)."""
+    import numpy as np
+    from mamba_rs_amd import GpuMambaBackbone, GpuMambaLM, MambaConfig, MambaWeights, WeightDtype
+    cfg = MambaConfig(**cfg_kw)
+    w = MambaWeights.random_lm(cfg, seed)
+    rng = np.random.default_rng(seed + 1)
+    embed = (rng.standard_normal((vocab, cfg.d_model), dtype=np.float32) * np.float32(0.02))
+    out = {"model": name}
+    pb, pt = prefill_bt
+    pre = GpuMambaBackbone.new_with_dtype(0, w, cfg, cfg.d_model, pb, WeightDtype.BF16)
+    lm_p = GpuMambaLM(pre, embed)
+    toks = rng.integers(0, vocab, (pb, pt)).astype(np.int32)
+    lm_p.prefill(toks); pre.sync()                      # warm-up (library kernel selection, scratch)
+    times = []
+    for _ in range(3):
+        pre.reset(); pre.sync()
+        t0 = time.perf_counter(); lm_p.prefill(toks); pre.sync(); times.append(time.perf_counter() - t0)
+    tp = sorted(times)[1]
+    out["prefill"] = {"batch": pb, "seq_len": pt, "ms": tp * 1e3, "tok_per_s": pb * pt / tp}
+    lm_p.close(); pre.close()
+    dec_out = []
+    for db in (decode_b if isinstance(decode_b, (list, tuple)) else [decode_b]):
+        dec = GpuMambaBackbone.new_with_dtype(0, w, cfg, cfg.d_model, db, WeightDtype.BF16)
+        lm_d = GpuMambaLM(dec, embed)
+        lm_d.set_tokens(rng.integers(0, vocab, db).astype(np.int32))
+        lm_d.capture_graph()
+        for _ in range(8):
+            lm_d.decode_step()
+        dec.sync()
+        t0 = time.perf_counter()
+        for _ in range(decode_steps):
+            lm_d.decode_step()
+        dec.sync()
+        td = (time.perf_counter() - t0) / decode_steps
+        tk = lm_d.get_tokens()
+        assert ((tk >= 0) & (tk < vocab)).all()
+        es = 2
+        di, dm, ds, dc, dr = cfg.d_inner(), cfg.d_model, cfg.d_state, cfg.d_conv, cfg.dt_rank()
+        layer_bytes = es * (dm * 2 * di + di * (dr + 2 * ds) + dr * di + di * dm) + 2 * 4 * db * di * (ds + dc) + 2 * 4 * db * dm
+        step_bytes = cfg.n_layers * layer_bytes + ((vocab + 63) // 64 * 64) * dm * es
+        dec_out.append({"batch": db, "steps": decode_steps, "us_per_step": td * 1e6, "tok_per_s": db / td,
+                        "algorithmic_bytes_per_step": step_bytes, "hbm_frac": step_bytes / td / 1e9 / HBM_PEAK_GBPS})
+        lm_d.close(); dec.close()
+    out["decode"] = dec_out
+    return out
+
+
+def m3_leg():
+    """Mamba-3 SISO scan kernels at the 768-wide shape (24 heads x headdim 64, d_state 64, bf16):
+    chunked SSD over batch 4 x 4096 (one layer) and the batch-1 decode step kernel."""
+    import numpy as np
+    import torch
+    from mamba_rs_amd import ops
+    from test_oracle_m3 import m3_inputs
+    B, T, nh, hd, ds = 4, 4096, 24, 64, 64
+    inp = m3_inputs(np.random.default_rng(3), B, T, nh, hd, ds)
+    dev = "cuda:0"
+    t = {k: torch.from_numpy(v).to(dev) for k, v in inp.items()}
+    x, K, Q = (t[k].to(torch.bfloat16) for k in ("x", "K", "Q"))
+    ssm = torch.zeros(B, nh, hd, ds, device=dev); kst = torch.zeros(B, nh, ds, device=dev); vst = torch.zeros(B, nh, hd, device=dev)
+    y = torch.empty_like(x)
+
+    def timeit(f, n):
+        for _ in range(3):
+            f()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(n):
+            f()
+        b.record(); torch.cuda.synchronize()
+        return a.elapsed_time(b) / n * 1e3
+
+    us = timeit(lambda: ops.m3_ssd_fwd(ssm, kst, vst, y, x, K, Q, t["dt"], t["trap"], t["a_val"], t["D"]), 10)
+    nbytes = 4 * B * T * nh * hd * 2 + 3 * B * T * nh * 4
+    al, be, ga = ops.m3_compute_abg(t["dt"], t["a_val"], t["trap"])
+    x1, K1, Q1 = x[:1, 0].contiguous(), K[:1, 0].contiguous(), Q[:1, 0].contiguous()
+    s1, k1, v1, y1 = ssm[:1].clone(), kst[:1].clone(), vst[:1].clone(), torch.empty_like(x[:1, 0])
+    a1, b1, g1 = al[:1, 0].contiguous(), be[:1, 0].contiguous(), ga[:1, 0].contiguous()
+    g = torch.cuda.CUDAGraph()
+    ops.m3_step(s1, k1, v1, y1, x1, K1, Q1, a1, b1, g1, t["D"])
+    torch.cuda.synchronize()
+    with torch.cuda.graph(g):
+        for _ in range(24):
+            ops.m3_step(s1, k1, v1, y1, x1, K1, Q1, a1, b1, g1, t["D"])
+    us_step = timeit(g.replay, 50) / 24
+    return {"ssd_prefill_layer": {"batch": B, "seq_len": T, "us": us, "algorithmic_bytes": nbytes, "GBps": nbytes / us / 1e3,
+                                  "hbm_frac": nbytes / us / 1e3 / HBM_PEAK_GBPS, "tok_per_s_layer": B * T / us * 1e6,
+                                  "mfma_flop": 4 * 2 * 64 * 64 * 64 * B * (T // 64) * nh},
+            "decode_step_kernel_b1": {"us_per_layer_call_in_graph": us_step}}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extras", action="store_true", help="only the headline scan line (no LM / Mamba-3 legs)")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also launch one 256 MiB device copy (a known-size kernel to scale rocprof FETCH_SIZE/WRITE_SIZE by)")
+    ap.add_argument("--big", action="store_true", help="also run the 2.8b-shape LM leg (several minutes of host-side init)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus must be 1 (no multi-GPU path exists)", file=sys.stderr)
@@ -137,11 +243,21 @@ def main():
                    "tokens_per_step": batch * T, "storage": "bf16"},
         "tokens_per_s": batch * T / (g["ms_per_step"] * 1e-3),
         "roofline": {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": gbps / HBM_PEAK_GBPS, "traffic": None,
+                     "frac": gbps / HBM_PEAK_GBPS, "traffic": MEASURED_SCAN_TRAFFIC_BYTES,
+                     "kernels": ["chunk_state_kernel", "chunk_out_kernel"],
                      "algorithmic_bytes_per_launch": nbytes, "median_launch_ms": g["median_launch_ms"]},
     }
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_leg(inp, shape, nbytes)
+    if not args.no_extras:
+        extras = {}
+        extras["lm_130m_shape_bf16"] = lm_leg("130m-shape", dict(d_model=768, d_state=16, d_conv=4, expand=2, n_layers=24), 50280,
+                                              (8, 2048), 64, 256)
+        extras["mamba3_768_bf16"] = m3_leg()
+        if args.big:
+            extras["lm_2.8b_shape_bf16"] = lm_leg("2.8b-shape", dict(d_model=2560, d_state=16, d_conv=4, expand=2, n_layers=64), 50280,
+                                                  (4, 4096), [1, 16, 128], 128)
+        out["extras"] = extras
     print(json.dumps(out))
 
 
