@@ -52,7 +52,7 @@ int check_launch(const char *what);
 
 // Internal launchers shared with the backbone engine (strides and fusions the public entry points do not expose).
 int launch_ssm_step_fused(hipStream_t st, int dtype, float *h, void *y, const void *delta, const float *dt_bias,
-                          const void *u, const void *Bb, const void *Cb, int64_t bc_stride, const void *gate,
+                          const void *dt_in, const void *dt_w, int dr, const void *u, const void *Bb, const void *Cb, int64_t bc_stride, const void *gate,
                           int64_t gate_stride, int gate_mode, const float *a_neg, const float *D, int batch,
                           int di, int ds);
 int launch_conv1d_step(hipStream_t st, int dtype, void *out, float *state, const void *new_x, int64_t x_stride,

@@ -7,9 +7,9 @@
 // conv/SSM state and every scratch buffer; step() allocates nothing.  The residual
 // stream, states, a_neg, D, biases and norm weights stay f32 (inference.rs:150-165).
 //
-// Per layer the decode chain is 4 library GEMMs and 3 kernels (the reference launches 10
+// Per layer the decode chain is 3 library GEMMs and 3 kernels (the reference launches 10
 // kernels + 4 GEMMs, inference.rs:993-1252): residual-add + RMSNorm, in_proj, conv step +
-// SiLU reading the x half of in_proj's output in place, x_proj, dt_proj, one kernel for
+// SiLU reading the x half of in_proj's output in place, x_proj, one kernel for dt_proj +
 // dt-bias + softplus + state update + B/C gather + SiLU gate, out_proj.
 #include "common.hpp"
 #include <rocblas/rocblas.h>
@@ -41,29 +41,39 @@ static rocblas_datatype blas_type(int dtype) {
 
 // ---- glue kernels -------------------------------------------------------------------
 
-// One wave per row: residual (f32) += add (storage dtype, may be null); out = rmsnorm(residual) * w.
+// One workgroup per row: residual (f32) += add (storage dtype, may be null); out = rmsnorm(residual) * w.
 // Reference: residual_add_f32_* + rmsnorm_forward_f32in_* (kernels/elementwise.cu:366-376,
 // kernels/norms.cu:21-171), with its finite guard: rms = 1 if not finite or < 1e-20 (norms.cu:58-61).
 template <typename T, typename TO>
 __global__ __launch_bounds__(256) void add_rmsnorm_kernel(float *__restrict__ residual, const T *__restrict__ add,
                                                           TO *__restrict__ out, const float *__restrict__ w,
                                                           float eps, int64_t rows, int dm, int64_t out_stride) {
-    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (row >= rows) return;
-    const int l = threadIdx.x & 63;
+    constexpr int kMaxPer = 16;  // elements per thread kept in registers (d_model <= 4096); longer rows re-read
+    __shared__ float part[4];
+    const int64_t row = blockIdx.x;
     float *r = residual + row * dm;
+    float v[kMaxPer];
     float ss = 0.0f;
-    for (int i = l; i < dm; i += kWave) {
-        float v = r[i];
-        if (add) { v += Store<T>::ld(add + row * dm + i); r[i] = v; }
-        ss = fmaf(v, v, ss);
+    int cnt = 0;
+    for (int i = threadIdx.x; i < dm; i += 256, cnt++) {
+        float x = r[i];
+        if (add) { x += Store<T>::ld(add + row * dm + i); r[i] = x; }
+        if (cnt < kMaxPer) v[cnt] = x;
+        ss = fmaf(x, x, ss);
     }
 #pragma unroll
     for (int m = 32; m >= 1; m >>= 1) ss += __shfl_xor(ss, m, kWave);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    ss = part[0] + part[1] + part[2] + part[3];
     float rms = sqrtf(ss / (float)dm + eps);
     if (!isfinite(rms) || rms < 1e-20f) rms = 1.0f;
     const float inv = 1.0f / rms;
-    for (int i = l; i < dm; i += kWave) Store<TO>::st(out + row * out_stride + i, r[i] * inv * w[i]);
+    cnt = 0;
+    for (int i = threadIdx.x; i < dm; i += 256, cnt++) {
+        const float x = cnt < kMaxPer ? v[cnt] : r[i];
+        Store<TO>::st(out + row * out_stride + i, x * inv * w[i]);
+    }
 }
 
 // delta = softplus(raw + bias[d]) in place (dt_proj bias + softplus_forward, kernels/activations.cu:32-52)
@@ -103,18 +113,12 @@ __global__ __launch_bounds__(256) void embed_gather_kernel(float *__restrict__ o
     out[i] = Store<T>::ld(embed + (int64_t)tok * dm + (i - r * dm));
 }
 
-// Greedy pick: index of the maximum logit, the LAST one among equals (Iterator::max_by, src/module/sample.rs:250-257).
-__global__ __launch_bounds__(256) void argmax_last_kernel(int *__restrict__ tokens, const float *__restrict__ logits,
-                                                          int vocab, int64_t stride) {
+// Greedy pick: index of the maximum logit, the LAST one among equals (Iterator::max_by,
+// src/module/sample.rs:250-257).  Stage 1: kArgParts blocks per row reduce a slice each; stage 2 combines.
+constexpr int kArgParts = 32;
+__device__ __forceinline__ void argmax_block_reduce(float &best, int &bi) {
     __shared__ float sv[256];
     __shared__ int si[256];
-    const float *row = logits + (int64_t)blockIdx.x * stride;
-    float best = -INFINITY;
-    int bi = 0;
-    for (int i = threadIdx.x; i < vocab; i += 256) {
-        const float v = row[i];
-        if (v >= best) { best = v; bi = i; }   // ascending i per thread: >= keeps the last maximum
-    }
     sv[threadIdx.x] = best; si[threadIdx.x] = bi;
     __syncthreads();
     for (int s = 128; s >= 1; s >>= 1) {
@@ -125,7 +129,36 @@ __global__ __launch_bounds__(256) void argmax_last_kernel(int *__restrict__ toke
         }
         __syncthreads();
     }
-    if (threadIdx.x == 0) tokens[blockIdx.x] = si[0];
+    best = sv[0]; bi = si[0];
+}
+__global__ __launch_bounds__(256) void argmax_part_kernel(float *__restrict__ pv, int *__restrict__ pi,
+                                                          const float *__restrict__ logits, int vocab, int64_t stride) {
+    const int row = blockIdx.x / kArgParts, part = blockIdx.x % kArgParts;
+    const int per = (vocab + kArgParts - 1) / kArgParts;
+    const int lo = part * per, hi = min(vocab, lo + per);
+    const float *r = logits + (int64_t)row * stride;
+    float best = -INFINITY;
+    int bi = lo < vocab ? lo : vocab - 1;
+    for (int i = lo + threadIdx.x; i < hi; i += 256) {
+        const float v = r[i];
+        if (v >= best) { best = v; bi = i; }   // ascending i per thread: >= keeps the last maximum
+    }
+    argmax_block_reduce(best, bi);
+    if (threadIdx.x == 0) { pv[blockIdx.x] = best; pi[blockIdx.x] = bi; }
+}
+__global__ __launch_bounds__(64) void argmax_final_kernel(int *__restrict__ tokens, const float *__restrict__ pv,
+                                                          const int *__restrict__ pi) {
+    const int row = blockIdx.x;
+    float best = -INFINITY;
+    int bi = 0;
+    if (threadIdx.x < kArgParts) { best = pv[row * kArgParts + threadIdx.x]; bi = pi[row * kArgParts + threadIdx.x]; }
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) {
+        const float ov = __shfl_xor(best, m, kWave);
+        const int oi = __shfl_xor(bi, m, kWave);
+        if (ov > best || (ov == best && oi > bi)) { best = ov; bi = oi; }
+    }
+    if (threadIdx.x == 0) tokens[row] = bi;
 }
 
 }  // namespace mrs
@@ -219,7 +252,7 @@ static int gemm_rm(mrs_backbone *bb, int dtype, void *C, int ldc, const void *A,
 template <typename T>
 static void launch_add_rmsnorm_t(mrs_backbone *bb, float *residual, const void *add, void *out, bool out_f32,
                                  const float *w, int64_t rows, int64_t out_stride) {
-    const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
+    const dim3 grid((unsigned)rows), block(256);
     if (out_f32)
         hipLaunchKernelGGL((add_rmsnorm_kernel<T, float>), grid, block, 0, bb->stream, residual, (const T *)add, (float *)out, w,
                            bb->cfg.rms_norm_eps, rows, bb->cfg.d_model, out_stride);
@@ -273,9 +306,9 @@ static int run_layers(mrs_backbone *bb, Scratch *s, int T) {
         if (T == 1) {
             MRS_TRY(launch_conv1d_step(bb->stream, dt, s->u, conv, s->proj, 2 * di, lw.conv_w, lw.conv_b, B, di, dc, 1));
             MRS_TRY(gemm_rm(bb, dt, s->xdbl, xd, s->u, di, lw.x_proj, (int)rows, xd, di));
-            MRS_TRY(gemm_rm(bb, dt, s->delta, di, s->xdbl, xd, lw.dt_w, (int)rows, di, dr));
-            MRS_TRY(launch_ssm_step_fused(bb->stream, dt, ssm, s->y, s->delta, lw.dt_b, s->u, xb + es * dr, xb + es * (dr + ds), xd,
-                                          z, 2 * di, 2, lw.a_neg, lw.D, B, di, ds));
+            // dt_proj (K = dt_rank) + bias + softplus + state update + B/C gather + SiLU gate: one kernel
+            MRS_TRY(launch_ssm_step_fused(bb->stream, dt, ssm, s->y, s->delta, lw.dt_b, s->xdbl, lw.dt_w, dr, s->u, xb + es * dr,
+                                          xb + es * (dr + ds), xd, z, 2 * di, 2, lw.a_neg, lw.D, B, di, ds));
         } else {
             MRS_TRY(mrs_conv1d_seq_silu(bb->stream, dt, s->u, conv, s->proj, 2 * di, lw.conv_w, lw.conv_b, B, T, di, dc));
             MRS_TRY(gemm_rm(bb, dt, s->xdbl, xd, s->u, di, lw.x_proj, (int)rows, xd, di));
@@ -529,6 +562,8 @@ struct mrs_lm {
     float *logits;      // [batch, vocab_padded] f32
     void *hidden;       // [batch, dm] storage dtype copy of temporal for the head GEMM
     int *tokens;        // [batch] current token ids on device
+    float *arg_v;       // [batch, kArgParts] partial maxima
+    int *arg_i;
     std::vector<void *> allocs;
     hipGraph_t graph;
     hipGraphExec_t graph_exec;
@@ -552,6 +587,8 @@ extern "C" int mrs_lm_create(mrs_lm **out, mrs_backbone *bb, const float *embed,
     MRS_LM_HIP(hipMalloc((void **)&lm->logits, (size_t)lm->batch * lm->vocab_padded * 4)); lm->allocs.push_back(lm->logits);
     MRS_LM_HIP(hipMalloc(&lm->hidden, (size_t)lm->batch * lm->dm * es)); lm->allocs.push_back(lm->hidden);
     MRS_LM_HIP(hipMalloc((void **)&lm->tokens, (size_t)lm->batch * sizeof(int))); lm->allocs.push_back(lm->tokens);
+    MRS_LM_HIP(hipMalloc((void **)&lm->arg_v, (size_t)lm->batch * kArgParts * sizeof(float))); lm->allocs.push_back(lm->arg_v);
+    MRS_LM_HIP(hipMalloc((void **)&lm->arg_i, (size_t)lm->batch * kArgParts * sizeof(int))); lm->allocs.push_back(lm->arg_i);
     MRS_LM_HIP(hipMalloc((void **)&stage, ne * 4));
     MRS_LM_HIP(hipMemsetAsync(stage, 0, ne * 4, bb->stream));  // padded rows are zero
     MRS_LM_HIP(hipMemcpyAsync(stage, embed, (size_t)vocab * lm->dm * 4, hipMemcpyHostToDevice, bb->stream));
@@ -595,6 +632,14 @@ static int lm_logits(mrs_lm *lm) {
     return MRS_OK;
 }
 
+static int lm_argmax(mrs_lm *lm) {
+    hipStream_t st = lm->bb->stream;
+    hipLaunchKernelGGL(argmax_part_kernel, dim3((unsigned)(lm->batch * kArgParts)), dim3(256), 0, st, lm->arg_v, lm->arg_i, lm->logits,
+                       lm->vocab, (int64_t)lm->vocab_padded);
+    hipLaunchKernelGGL(argmax_final_kernel, dim3((unsigned)lm->batch), dim3(64), 0, st, lm->tokens, lm->arg_v, lm->arg_i);
+    return check_launch("argmax kernels");
+}
+
 static int lm_decode_body(mrs_lm *lm) {
     mrs_backbone *bb = lm->bb;
     const int64_t n = (int64_t)lm->batch * lm->dm;
@@ -603,9 +648,7 @@ static int lm_decode_body(mrs_lm *lm) {
                                                          (const T_ *)lm->embed, lm->tokens, (int64_t)lm->batch, lm->dm, lm->vocab));
     MRS_TRY(step_body(bb));
     MRS_TRY(lm_logits(lm));
-    hipLaunchKernelGGL(argmax_last_kernel, dim3((unsigned)lm->batch), dim3(256), 0, bb->stream, lm->tokens, lm->logits, lm->vocab,
-                       (int64_t)lm->vocab_padded);
-    return check_launch("argmax_last_kernel");
+    return lm_argmax(lm);
 }
 
 extern "C" int mrs_lm_set_tokens(mrs_lm *lm, const int *tokens) {
@@ -685,11 +728,7 @@ extern "C" int mrs_lm_prefill(mrs_lm *lm, mrs_backbone *prefill_bb, const int *t
     int rc = mrs_backbone_prefill_device(prefill_bb, prefill_bb->prefill_in, T);
     if (!rc && prefill_bb == lm->bb) {
         rc = lm_logits(lm);
-        if (!rc) {
-            hipLaunchKernelGGL(argmax_last_kernel, dim3((unsigned)lm->batch), dim3(256), 0, lm->bb->stream, lm->tokens, lm->logits,
-                               lm->vocab, (int64_t)lm->vocab_padded);
-            rc = check_launch("argmax_last_kernel");
-        }
+        if (!rc) rc = lm_argmax(lm);
     }
     hipStreamSynchronize(prefill_bb->stream);
     hipFree(dtok);

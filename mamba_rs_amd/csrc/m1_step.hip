@@ -24,6 +24,7 @@ __global__ __launch_bounds__(256) void ssm_step_kernel(
     float *__restrict__ h, T *__restrict__ y, const T *__restrict__ delta, const T *__restrict__ u,
     const T *__restrict__ Bbase, const T *__restrict__ Cbase, int64_t bc_stride,
     const T *__restrict__ gate, int64_t gate_stride, int gate_mode, const float *__restrict__ dt_bias,
+    const T *__restrict__ dt_in, const T *__restrict__ dt_w, int dr,
     const float *__restrict__ a_neg, const float *__restrict__ Dp, int64_t total, int di, int ds) {
     // total = batch*d_inner rows; ds == 4*LG here.
     const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -35,7 +36,19 @@ __global__ __launch_bounds__(256) void ssm_step_kernel(
     const int d = (int)(r - (int64_t)b * di);
     float4 hv = *reinterpret_cast<const float4 *>(h + r * ds + 4 * g);
     const float4 av = *reinterpret_cast<const float4 *>(a_neg + (int64_t)d * ds + 4 * g);
-    float dl = Store<T>::ld(delta + r);
+    float dl;
+    if (dt_w) {
+        // dt_proj folded in: delta_raw[b,d] = sum_r dt_in[b,r] * dt_w[r,d], the dt_rank terms split over the
+        // LG lanes of the row (dt_proj GEMM of the decode chain, src/mamba_ssm/gpu/inference.rs:1129-1146)
+        const T *xr = dt_in + (int64_t)b * bc_stride;
+        float part = 0.0f;
+        for (int k = g; k < dr; k += LG) part = fmaf(Store<T>::ld(xr + k), Store<T>::ld(dt_w + (int64_t)k * di + d), part);
+#pragma unroll
+        for (int m = 1; m < LG; m <<= 1) part += __shfl_xor(part, m, kWave);
+        dl = part;
+    } else {
+        dl = Store<T>::ld(delta + r);
+    }
     if (dt_bias) dl = softplus20(dl + dt_bias[d]);
     const float uu = Store<T>::ld(u + r);
     const float du = dl * uu;
@@ -69,12 +82,19 @@ __global__ __launch_bounds__(256) void ssm_step_generic_kernel(
     float *__restrict__ h, T *__restrict__ y, const T *__restrict__ delta, const T *__restrict__ u,
     const T *__restrict__ Bbase, const T *__restrict__ Cbase, int64_t bc_stride,
     const T *__restrict__ gate, int64_t gate_stride, int gate_mode, const float *__restrict__ dt_bias,
+    const T *__restrict__ dt_in, const T *__restrict__ dt_w, int dr,
     const float *__restrict__ a_neg, const float *__restrict__ Dp, int64_t total, int di, int ds) {
     const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (r >= total) return;
     const int b = (int)(r / di);
     const int d = (int)(r - (int64_t)b * di);
-    float dl = Store<T>::ld(delta + r);
+    float dl;
+    if (dt_w) {
+        dl = 0.0f;
+        for (int k = 0; k < dr; k++) dl = fmaf(Store<T>::ld(dt_in + (int64_t)b * bc_stride + k), Store<T>::ld(dt_w + (int64_t)k * di + d), dl);
+    } else {
+        dl = Store<T>::ld(delta + r);
+    }
     if (dt_bias) dl = softplus20(dl + dt_bias[d]);
     const float uu = Store<T>::ld(u + r);
     const float du = dl * uu;
@@ -97,12 +117,12 @@ __global__ __launch_bounds__(256) void ssm_step_generic_kernel(
 template <typename T>
 static int launch_step(hipStream_t st, float *h, void *y, const void *delta, const void *u,
                        const void *Bb, const void *Cb, int64_t bc_stride, const void *gate,
-                       int64_t gate_stride, int gate_mode, const float *dt_bias, const float *a_neg,
-                       const float *D, int batch, int di, int ds) {
+                       int64_t gate_stride, int gate_mode, const float *dt_bias, const void *dt_in,
+                       const void *dt_w, int dr, const float *a_neg, const float *D, int batch, int di, int ds) {
     const int64_t total = (int64_t)batch * di;
     if (!gate) gate_mode = 0;
 #define MRS_ARGS h, (T *)y, (const T *)delta, (const T *)u, (const T *)Bb, (const T *)Cb, bc_stride, \
-                 (const T *)gate, gate_stride, gate_mode, dt_bias, a_neg, D, total, di, ds
+                 (const T *)gate, gate_stride, gate_mode, dt_bias, (const T *)dt_in, (const T *)dt_w, dr, a_neg, D, total, di, ds
     const bool vec_ok = aligned(h, 16) && aligned(a_neg, 16);
     int lg = 0;
     if (vec_ok && (ds == 4 || ds == 8 || ds == 16 || ds == 32 || ds == 64 || ds == 128 || ds == 256)) lg = ds / 4;
@@ -124,11 +144,12 @@ static int launch_step(hipStream_t st, float *h, void *y, const void *delta, con
 }
 
 int launch_ssm_step_fused(hipStream_t st, int dtype, float *h, void *y, const void *delta, const float *dt_bias,
+                          const void *dt_in, const void *dt_w, int dr,
                           const void *u, const void *Bb, const void *Cb, int64_t bc_stride, const void *gate,
                           int64_t gate_stride, int gate_mode, const float *a_neg, const float *D, int batch,
                           int di, int ds) {
     MRS_DISPATCH_DTYPE(dtype, T_, return launch_step<T_>(st, h, y, delta, u, Bb, Cb, bc_stride, gate, gate_stride, gate_mode,
-                                                         dt_bias, a_neg, D, batch, di, ds));
+                                                         dt_bias, dt_in, dt_w, dr, a_neg, D, batch, di, ds));
     return MRS_OK;
 }
 
@@ -154,7 +175,7 @@ extern "C" int mrs_ssm_step(void *stream, int dtype, float *h, void *y, const vo
     int rc = step_check("mrs_ssm_step", dtype, h, y, delta, u, B, C, a_neg, D, batch, d_inner, d_state);
     if (rc) return rc;
     hipStream_t st = as_stream(stream);
-    MRS_DISPATCH_DTYPE(dtype, T_, return launch_step<T_>(st, h, y, delta, u, B, C, d_state, nullptr, 0, 0, nullptr, a_neg, D, batch, d_inner, d_state));
+    MRS_DISPATCH_DTYPE(dtype, T_, return launch_step<T_>(st, h, y, delta, u, B, C, d_state, nullptr, 0, 0, nullptr, nullptr, nullptr, 0, a_neg, D, batch, d_inner, d_state));
     return MRS_OK;
 }
 
@@ -171,6 +192,6 @@ extern "C" int mrs_ssm_step_gather_gate(void *stream, int dtype, float *h, void 
     const char *xb = static_cast<const char *>(xdbl);
     hipStream_t st = as_stream(stream);
     MRS_DISPATCH_DTYPE(dtype, T_, return launch_step<T_>(st, h, y, delta, u, xb + es * b_offset, xb + es * c_offset,
-                                                         xdbl_stride, gate_silu, d_inner, 1, nullptr, a_neg, D, batch, d_inner, d_state));
+                                                         xdbl_stride, gate_silu, d_inner, 1, nullptr, nullptr, nullptr, 0, a_neg, D, batch, d_inner, d_state));
     return MRS_OK;
 }
