@@ -16,6 +16,12 @@
 //   S^T[n,p] = exp(dA_end) S^T[n,p] + sum_t K[t,n] (w[t] x[t,p]),  w[t] = exp(dA_end-dA[t]) scale[t]
 // with gamma = dt trap, scale[t] = gamma[t] + dt[t+1](1-trap[t+1]), dA = cumsum(a dt) in the chunk.
 //
+// When batch*heads alone cannot fill 256 compute units the sequence is also cut into
+// super-chunks (a run of consecutive chunks): a state-only pass of the same kernel (no Q, no y)
+// leaves each super-chunk's locally accumulated state and total log-decay in a workspace, and the
+// full pass then starts every super-chunk from  sum_k exp(sum_{k<m<sc} dA_m) S_k  -- the same
+// composition law as between chunks -- so all super-chunks of a (row, head) run concurrently.
+//
 // Wave w of the workgroup owns the 16 columns p in [16w, 16w+16) of y and of the state.
 // Operand layouts are chosen so that no accumulator is ever transposed: G is produced
 // transposed (A = K rows, B = Q rows) which leaves P directly in A-operand layout, and the
@@ -23,6 +29,7 @@
 // v_mfma_f32_16x16x16 (bf16 or f16 inputs, f32 accumulate): lane l holds A[m=l%16][k=4(l/16)..+3],
 // B[k=4(l/16)..+3][n=l%16], and C/D[m=4(l/16)+i][n=l%16], i = 0..3.
 #include "common.hpp"
+#include <stdlib.h>
 
 namespace mrs {
 
@@ -69,44 +76,90 @@ template <int HD, int DS> struct alignas(16) SsdSmem {
     alignas(16) uint16_t Kt[DS][kCS + kPad];       // K transposed: Kt[n][t]
     alignas(16) uint16_t Xt[NW][16][kCS + kPad];   // per wave: x slice transposed, Xt[p][t]
     alignas(16) float sc[NW][5][kCS];              // per wave: dA, scale, gamma, exp(dA), w
+    alignas(16) uint2 Ps[10][kWave];               // the 10 causal 16x16 tiles of P as A-operand fragments, by lane
 };
 
-template <typename T, int HD, int DS>
+// Kt rows are XOR-swizzled in units of four steps so that the 16-bit transposing stores of a wave
+// (8 rows x 8 column groups) land in 32 distinct banks; fragment reads take 4 consecutive steps and are unaffected.
+__device__ __forceinline__ int kt_swz(int n) { return ((n >> 3) & 7) << 2; }
+
+// Super-chunk split of one launch: nsc super-chunks of cps chunks each; the three buffers live in
+// the caller's workspace (null when nsc == 1).
+struct SsdSplit {
+    float *Sloc;    // [batch*nh][nsc-1][HD][DS]  state accumulated inside super-chunk k (k = 0 includes the carried-in state)
+    float *dAtot;   // [batch*nh][nsc-1]          sum of a*dt over super-chunk k
+    float *Sinit;   // [batch*nh][HD][DS]         the carried-in state, saved before the last super-chunk overwrites ssm
+    int nsc, cps;
+};
+
+template <typename T, int HD, int DS, bool STATE_ONLY>
 __global__ __launch_bounds__(HD * 4) void m3_ssd_kernel(
     float *__restrict__ ssm, float *__restrict__ kst, float *__restrict__ vst, T *__restrict__ y,
     const T *__restrict__ x, const T *__restrict__ K, const T *__restrict__ Q,
     const float *__restrict__ dt, const float *__restrict__ trap, const float *__restrict__ a_val,
-    const float *__restrict__ Dp, int Tlen, int nh, int carry) {
+    const float *__restrict__ Dp, SsdSplit sp, int Tlen, int nh, int carry) {
     constexpr int NW = HD / 16, NTHR = NW * 64, KN = DS / 16;
     constexpr int VPR = DS / 8;                    // 16-byte vectors per Q/K row
     constexpr int NVEC = kCS * VPR;                // vectors per tile
     constexpr int NV = (NVEC + NTHR - 1) / NTHR;   // vectors per thread per tile
     __shared__ SsdSmem<HD, DS> sm;
 
-    const int b = blockIdx.x / nh, h = blockIdx.x - b * nh;
+    const int nscg = STATE_ONLY ? sp.nsc - 1 : sp.nsc;   // the state-only pass skips the last super-chunk
+    const int bhi = blockIdx.x / nscg, sc = blockIdx.x - bhi * nscg;
+    const int b = bhi / nh, h = bhi - b * nh;
     const int tid = threadIdx.x, w = tid >> 6, l = tid & 63;
     const int lr = l & 15, lg = l >> 4;            // fragment row/col index and k-group
     const int di = nh * HD;
     const int64_t bh = (int64_t)b * nh + h;
     const float Dh = Dp[h];
     const int nchunks = (Tlen + kCS - 1) / kCS;
+    const int c_begin = sc * sp.cps, c_end = min(nchunks, c_begin + sp.cps);
+    const int64_t srow = (bh * HD + 16 * w + lr) * DS + 4 * lg;   // this lane's state elements, + 16 jn
 
     // ---- running state S^T as accumulator tiles: lane holds S[p=16w+lr][n=16jn+4lg+i] ----
     v4f St[KN];
 #pragma unroll
     for (int jn = 0; jn < KN; jn++) St[jn] = (v4f){0.f, 0.f, 0.f, 0.f};
-    if (carry) {
-        const int64_t t0row = (int64_t)b * Tlen * nh + h;
-        const float sgm1 = dt[t0row] * (1.0f - trap[t0row]);
-        const float vin = vst[bh * HD + 16 * w + lr];
+    if (sc == 0) {
+        if (carry && !STATE_ONLY && sp.nsc > 1) {
 #pragma unroll
-        for (int jn = 0; jn < KN; jn++) {
-            const float4 s = *reinterpret_cast<const float4 *>(ssm + (bh * HD + 16 * w + lr) * DS + 16 * jn + 4 * lg);
-            const float4 kin = *reinterpret_cast<const float4 *>(kst + bh * DS + 16 * jn + 4 * lg);
-            St[jn] = (v4f){fmaf(sgm1 * vin, kin.x, s.x), fmaf(sgm1 * vin, kin.y, s.y), fmaf(sgm1 * vin, kin.z, s.z),
-                           fmaf(sgm1 * vin, kin.w, s.w)};
+            for (int jn = 0; jn < KN; jn++) {
+                const float4 s = *reinterpret_cast<const float4 *>(sp.Sinit + srow + 16 * jn);
+                St[jn] = (v4f){s.x, s.y, s.z, s.w};
+            }
+        } else if (carry) {
+            // S_in = ssm + dt_0 (1 - trap_0) v_in (x) k_in : the beta term of step 0, which belongs to the carried state
+            const int64_t t0row = (int64_t)b * Tlen * nh + h;
+            const float sgm1 = dt[t0row] * (1.0f - trap[t0row]);
+            const float vin = vst[bh * HD + 16 * w + lr];
+#pragma unroll
+            for (int jn = 0; jn < KN; jn++) {
+                const float4 s = *reinterpret_cast<const float4 *>(ssm + srow + 16 * jn);
+                const float4 kin = *reinterpret_cast<const float4 *>(kst + bh * DS + 16 * jn + 4 * lg);
+                St[jn] = (v4f){fmaf(sgm1 * vin, kin.x, s.x), fmaf(sgm1 * vin, kin.y, s.y), fmaf(sgm1 * vin, kin.z, s.z),
+                               fmaf(sgm1 * vin, kin.w, s.w)};
+                if (STATE_ONLY)
+                    *reinterpret_cast<float4 *>(sp.Sinit + srow + 16 * jn) = make_float4(St[jn][0], St[jn][1], St[jn][2], St[jn][3]);
+            }
+        }
+    } else if (!STATE_ONLY) {
+        // entering state of super-chunk sc from the local states of the earlier ones (the state-only
+        // pass accumulates every later super-chunk from zero)
+        float run = 0.0f;
+        for (int k = sc - 1; k >= 0; k--) {
+            const int64_t slot = bh * (sp.nsc - 1) + k;
+            const float dec = fast_exp2(run * kLog2e);
+            const float *src = sp.Sloc + slot * (HD * DS) + (16 * w + lr) * DS + 4 * lg;
+#pragma unroll
+            for (int jn = 0; jn < KN; jn++) {
+                const float4 s = *reinterpret_cast<const float4 *>(src + 16 * jn);
+                St[jn] = (v4f){fmaf(dec, s.x, St[jn][0]), fmaf(dec, s.y, St[jn][1]), fmaf(dec, s.z, St[jn][2]),
+                               fmaf(dec, s.w, St[jn][3])};
+            }
+            run += sp.dAtot[slot];
         }
     }
+    float dAsum = 0.0f;
 
     // ---- global -> register prefetch of one chunk ----
     uint4 rq[NV], rk[NV], rx[2];
@@ -119,7 +172,7 @@ __global__ __launch_bounds__(HD * 4) void m3_ssd_kernel(
             const int t = t0 + row;
             if (vi < NVEC && t < Tlen) {
                 const int64_t off = (((int64_t)b * Tlen + t) * nh + h) * DS + col;
-                rq[v] = *reinterpret_cast<const uint4 *>(Q + off);
+                if (!STATE_ONLY) rq[v] = *reinterpret_cast<const uint4 *>(Q + off);
                 rk[v] = *reinterpret_cast<const uint4 *>(K + off);
             } else {
                 rq[v] = make_uint4(0, 0, 0, 0);
@@ -144,8 +197,8 @@ __global__ __launch_bounds__(HD * 4) void m3_ssd_kernel(
         } else { ndt0 = 0.f; ntr0 = 1.f; }
     };
 
-    prefetch(0);
-    for (int c = 0; c < nchunks; c++) {
+    prefetch(c_begin);
+    for (int c = c_begin; c < c_end; c++) {
         const int t0 = c * kCS;
         __syncthreads();  // every wave is done reading the previous chunk's tiles
         // ---- registers -> LDS ----
@@ -153,13 +206,15 @@ __global__ __launch_bounds__(HD * 4) void m3_ssd_kernel(
         for (int v = 0; v < NV; v++) {
             const int vi = tid + v * NTHR, row = vi / VPR, col = (vi % VPR) * 8;
             if (vi >= NVEC) continue;
-            *reinterpret_cast<uint4 *>(&sm.Qs[row][col]) = rq[v];
-            *reinterpret_cast<uint4 *>(&sm.Ks[row][col]) = rk[v];
+            if (!STATE_ONLY) {
+                *reinterpret_cast<uint4 *>(&sm.Qs[row][col]) = rq[v];
+                *reinterpret_cast<uint4 *>(&sm.Ks[row][col]) = rk[v];
+            }
             const unsigned kw[4] = {rk[v].x, rk[v].y, rk[v].z, rk[v].w};
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                sm.Kt[col + 2 * j][row] = (uint16_t)(kw[j] & 0xffffu);
-                sm.Kt[col + 2 * j + 1][row] = (uint16_t)(kw[j] >> 16);
+                sm.Kt[col + 2 * j][row ^ kt_swz(col)] = (uint16_t)(kw[j] & 0xffffu);
+                sm.Kt[col + 2 * j + 1][row ^ kt_swz(col)] = (uint16_t)(kw[j] >> 16);
             }
         }
         {
@@ -192,7 +247,8 @@ __global__ __launch_bounds__(HD * 4) void m3_ssd_kernel(
             sm.sc[w][4][l] = fast_exp2((dAend - dA) * kLog2e) * scl;
         }
         __syncthreads();  // tiles visible to every wave
-        if (c + 1 < nchunks) prefetch(c + 1);
+        if (c + 1 < c_end) prefetch(c + 1);
+        dAsum += dAend;
 
         // ---- x fragments: lane holds x[t=16kt+4lg+i][p=16w+lr]; also scaled by w[t] for the state update ----
         uint2 xf[4], xwf[4];
@@ -209,53 +265,39 @@ __global__ __launch_bounds__(HD * 4) void m3_ssd_kernel(
 #pragma unroll
         for (int jn = 0; jn < KN; jn++) Sf[jn] = Mma<T>::pack(St[jn][0], St[jn][1], St[jn][2], St[jn][3]);
 
+        if (!STATE_ONLY) {
+            // ---- P tiles: P does not depend on p, so the waves split the 10 causal tiles and share them through LDS ----
 #pragma unroll
-        for (int it = 0; it < 4; it++) {
-            // Q fragments of this t-tile: lane holds Q[t=16it+lr][n=16kk+4lg..+3]
-            uint2 qf[KN];
+            for (int it = 0; it < 4; it++) {
 #pragma unroll
-            for (int kk = 0; kk < KN; kk++) qf[kk] = *reinterpret_cast<const uint2 *>(&sm.Qs[16 * it + lr][16 * kk + 4 * lg]);
-            // y_off = exp(dA[t]) * Q S^T     (acc rows t = 16it+4lg+i, cols p = 16w+lr)
-            v4f acc = {0.f, 0.f, 0.f, 0.f};
+                for (int js = 0; js <= it; js++) {
+                    const int tix = it * (it + 1) / 2 + js;
+                    if ((tix % NW) != w) continue;
+                    // G^T tile: rows s = 16js+4lg+i, cols t = 16it+lr
+                    v4f g = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int kk = 0; kk < KN; kk++) acc = Mma<T>::mma(qf[kk], Sf[kk], acc);
-            {
-                const float4 e = *reinterpret_cast<const float4 *>(&sm.sc[w][3][16 * it + 4 * lg]);
-                acc[0] *= e.x; acc[1] *= e.y; acc[2] *= e.z; acc[3] *= e.w;
-            }
-            const float dAt = sm.sc[w][0][16 * it + lr];
-            const float gamt = sm.sc[w][2][16 * it + lr];
-#pragma unroll
-            for (int js = 0; js <= it; js++) {
-                // G^T tile: rows s = 16js+4lg+i, cols t = 16it+lr
-                v4f g = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int kk = 0; kk < KN; kk++) {
-                    const uint2 kf = *reinterpret_cast<const uint2 *>(&sm.Ks[16 * js + lr][16 * kk + 4 * lg]);
-                    g = Mma<T>::mma(kf, qf[kk], g);
-                }
-                const float4 dAs = *reinterpret_cast<const float4 *>(&sm.sc[w][0][16 * js + 4 * lg]);
-                const float4 scs = *reinterpret_cast<const float4 *>(&sm.sc[w][1][16 * js + 4 * lg]);
-                const float das[4] = {dAs.x, dAs.y, dAs.z, dAs.w}, sc4[4] = {scs.x, scs.y, scs.z, scs.w};
-                float pv[4];
-#pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const float dec = fast_exp2((dAt - das[i]) * kLog2e);
-                    pv[i] = g[i] * sc4[i] * dec;
-                    if (js == it) {  // diagonal tile: strict causality, skip term on the diagonal
-                        const int s = 4 * lg + i;
-                        if (s > lr) pv[i] = 0.f;
-                        else if (s == lr) pv[i] = fmaf(gamt, g[i], Dh);
+                    for (int kk = 0; kk < KN; kk++) {
+                        const uint2 kf = *reinterpret_cast<const uint2 *>(&sm.Ks[16 * js + lr][16 * kk + 4 * lg]);
+                        const uint2 qf = *reinterpret_cast<const uint2 *>(&sm.Qs[16 * it + lr][16 * kk + 4 * lg]);
+                        g = Mma<T>::mma(kf, qf, g);
                     }
-                }
-                const uint2 pf = Mma<T>::pack(pv[0], pv[1], pv[2], pv[3]);  // A operand: P[t=lr][s=4lg+i]
-                acc = Mma<T>::mma(pf, xf[js], acc);
-            }
-            // store y rows t = t0+16it+4lg+i, column p = 16w+lr
+                    const float dAt = sm.sc[w][0][16 * it + lr];
+                    const float4 dAs = *reinterpret_cast<const float4 *>(&sm.sc[w][0][16 * js + 4 * lg]);
+                    const float4 scs = *reinterpret_cast<const float4 *>(&sm.sc[w][1][16 * js + 4 * lg]);
+                    const float das[4] = {dAs.x, dAs.y, dAs.z, dAs.w}, sc4[4] = {scs.x, scs.y, scs.z, scs.w};
+                    float pv[4];
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const int t = t0 + 16 * it + 4 * lg + i;
-                if (t < Tlen) Store<T>::st(y + ((int64_t)b * Tlen + t) * di + h * HD + 16 * w + lr, acc[i]);
+                    for (int i = 0; i < 4; i++) {
+                        const float dec = fast_exp2((dAt - das[i]) * kLog2e);
+                        pv[i] = g[i] * sc4[i] * dec;
+                        if (js == it) {  // diagonal tile: strict causality, skip term on the diagonal
+                            const int s = 4 * lg + i;
+                            if (s > lr) pv[i] = 0.f;
+                            else if (s == lr) pv[i] = fmaf(sm.sc[w][2][16 * it + lr], g[i], Dh);
+                        }
+                    }
+                    sm.Ps[tix][l] = Mma<T>::pack(pv[0], pv[1], pv[2], pv[3]);  // A operand: P[t=lr][s=4lg+i]
+                }
             }
         }
         // ---- state update: S^T[n,p] = exp(dA_end) S^T + K^T (w x) ----
@@ -265,17 +307,51 @@ __global__ __launch_bounds__(HD * 4) void m3_ssd_kernel(
             v4f s = St[jn] * decay;
 #pragma unroll
             for (int kt = 0; kt < 4; kt++) {
-                const uint2 ktf = *reinterpret_cast<const uint2 *>(&sm.Kt[16 * jn + lr][16 * kt + 4 * lg]);
+                const uint2 ktf = *reinterpret_cast<const uint2 *>(&sm.Kt[16 * jn + lr][(16 * kt + 4 * lg) ^ kt_swz(16 * jn + lr)]);
                 s = Mma<T>::mma(ktf, xwf[kt], s);
             }
             St[jn] = s;
         }
+        if (!STATE_ONLY) {
+            __syncthreads();  // P tiles visible
+#pragma unroll
+            for (int it = 0; it < 4; it++) {
+                // y_off = exp(dA[t]) * Q S_in^T     (acc rows t = 16it+4lg+i, cols p = 16w+lr)
+                v4f acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int kk = 0; kk < KN; kk++) {
+                    const uint2 qf = *reinterpret_cast<const uint2 *>(&sm.Qs[16 * it + lr][16 * kk + 4 * lg]);
+                    acc = Mma<T>::mma(qf, Sf[kk], acc);
+                }
+                {
+                    const float4 e = *reinterpret_cast<const float4 *>(&sm.sc[w][3][16 * it + 4 * lg]);
+                    acc[0] *= e.x; acc[1] *= e.y; acc[2] *= e.z; acc[3] *= e.w;
+                }
+#pragma unroll
+                for (int js = 0; js <= it; js++) acc = Mma<T>::mma(sm.Ps[it * (it + 1) / 2 + js][l], xf[js], acc);
+                // store y rows t = t0+16it+4lg+i, column p = 16w+lr
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int t = t0 + 16 * it + 4 * lg + i;
+                    if (t < Tlen) Store<T>::st(y + ((int64_t)b * Tlen + t) * di + h * HD + 16 * w + lr, acc[i]);
+                }
+            }
+        }
     }
+    if (STATE_ONLY) {
+        const int64_t slot = bh * (sp.nsc - 1) + sc;
+        float *dst = sp.Sloc + slot * (HD * DS) + (16 * w + lr) * DS + 4 * lg;
+#pragma unroll
+        for (int jn = 0; jn < KN; jn++)
+            *reinterpret_cast<float4 *>(dst + 16 * jn) = make_float4(St[jn][0], St[jn][1], St[jn][2], St[jn][3]);
+        if (tid == 0) sp.dAtot[slot] = dAsum;
+        return;
+    }
+    if (sc != sp.nsc - 1) return;
     // ---- write back: ssm <- S, k_state <- K[T-1], v_state <- x[T-1] ----
 #pragma unroll
     for (int jn = 0; jn < KN; jn++)
-        *reinterpret_cast<float4 *>(ssm + (bh * HD + 16 * w + lr) * DS + 16 * jn + 4 * lg) =
-            make_float4(St[jn][0], St[jn][1], St[jn][2], St[jn][3]);
+        *reinterpret_cast<float4 *>(ssm + srow + 16 * jn) = make_float4(St[jn][0], St[jn][1], St[jn][2], St[jn][3]);
     const int64_t last = (int64_t)b * Tlen + (Tlen - 1);
     for (int n = tid; n < DS; n += NTHR) kst[bh * DS + n] = Store<T>::ld(K + (last * nh + h) * DS + n);
     for (int p = tid; p < HD; p += NTHR) vst[bh * HD + p] = Store<T>::ld(x + last * di + h * HD + p);
@@ -298,21 +374,49 @@ __global__ void zero_kernel(float *__restrict__ p, int64_t n) {
     if (i < n) p[i] = 0.0f;
 }
 
+// Super-chunk plan: enough workgroups to cover the chip about three times over (three workgroups of
+// this kernel fit a compute unit), at least two chunks per super-chunk, at most 32 super-chunks.
+static void ssd_plan(int batch, int Tlen, int nh, int &nsc, int &cps) {
+    const int nchunks = (Tlen + kCS - 1) / kCS;
+    int target = 768;
+    if (const char *e = getenv("MRS_SSD_TARGET_WGS")) { const int v = atoi(e); if (v > 0) target = v; }
+    int64_t want = target / ((int64_t)batch * nh);
+    if (want > 32) want = 32;
+    if (want > nchunks / 2) want = nchunks / 2;
+    if (want <= 1) { nsc = 1; cps = nchunks; return; }
+    cps = (nchunks + (int)want - 1) / (int)want;
+    nsc = (nchunks + cps - 1) / cps;
+}
+
+static size_t ssd_split_bytes(int batch, int nh, int hd, int ds, int nsc, size_t *o_dA, size_t *o_init) {
+    if (nsc <= 1) { if (o_dA) *o_dA = 0; if (o_init) *o_init = 0; return 0; }
+    const size_t bh = (size_t)batch * nh;
+    const size_t sloc = (bh * (nsc - 1) * hd * ds * sizeof(float) + 255) & ~(size_t)255;
+    const size_t dat = (bh * (nsc - 1) * sizeof(float) + 255) & ~(size_t)255;
+    const size_t sin = (bh * hd * ds * sizeof(float) + 255) & ~(size_t)255;
+    if (o_dA) *o_dA = sloc;
+    if (o_init) *o_init = sloc + dat;
+    return sloc + dat + sin;
+}
+
 template <typename T, int HD, int DS>
 static void launch_ssd_shape(hipStream_t st, float *ssm, float *kst, float *vst, void *y, const void *x,
                              const void *K, const void *Q, const float *dt, const float *trap,
-                             const float *a_val, const float *D, int batch, int Tlen, int nh, int carry) {
-    hipLaunchKernelGGL((m3_ssd_kernel<T, HD, DS>), dim3((unsigned)(batch * nh)), dim3(HD * 4), 0, st, ssm, kst, vst,
-                       (T *)y, (const T *)x, (const T *)K, (const T *)Q, dt, trap, a_val, D, Tlen, nh, carry);
+                             const float *a_val, const float *D, SsdSplit sp, int batch, int Tlen, int nh, int carry) {
+    if (sp.nsc > 1)
+        hipLaunchKernelGGL((m3_ssd_kernel<T, HD, DS, true>), dim3((unsigned)(batch * nh * (sp.nsc - 1))), dim3(HD * 4), 0, st,
+                           ssm, kst, vst, (T *)y, (const T *)x, (const T *)K, (const T *)Q, dt, trap, a_val, D, sp, Tlen, nh, carry);
+    hipLaunchKernelGGL((m3_ssd_kernel<T, HD, DS, false>), dim3((unsigned)(batch * nh * sp.nsc)), dim3(HD * 4), 0, st, ssm, kst, vst,
+                       (T *)y, (const T *)x, (const T *)K, (const T *)Q, dt, trap, a_val, D, sp, Tlen, nh, carry);
 }
 
 template <typename T>
 static int launch_ssd(hipStream_t st, float *ssm, float *kst, float *vst, void *y, const void *x, const void *K,
                       const void *Q, const float *dt, const float *trap, const float *a_val, const float *D,
-                      int batch, int Tlen, int nh, int hd, int ds, int carry) {
+                      SsdSplit sp, int batch, int Tlen, int nh, int hd, int ds, int carry) {
 #define MRS_SHAPE(H, S)                                                                                      \
     if (hd == H && ds == S) {                                                                                \
-        launch_ssd_shape<T, H, S>(st, ssm, kst, vst, y, x, K, Q, dt, trap, a_val, D, batch, Tlen, nh, carry); \
+        launch_ssd_shape<T, H, S>(st, ssm, kst, vst, y, x, K, Q, dt, trap, a_val, D, sp, batch, Tlen, nh, carry); \
         return check_launch("m3_ssd_kernel");                                                                \
     }
     MRS_SHAPE(64, 64) MRS_SHAPE(64, 32) MRS_SHAPE(64, 16)
@@ -336,11 +440,16 @@ extern "C" int mrs_m3_compute_abg(void *stream, float *alpha, float *beta, float
 }
 
 extern "C" size_t mrs_m3_ssd_workspace_bytes(int batch, int T, int nheads, int headdim, int d_state, int chunk_size) {
-    (void)headdim; (void)d_state; (void)chunk_size;
-    if (batch < 1 || T < 1 || nheads < 1) return 256;
-    // alpha, beta, gamma for the f32-storage route (sequential kernel)
+    (void)chunk_size;
+    if (batch < 1 || T < 1 || nheads < 1 || headdim < 1 || d_state < 1) return 256;
+    // the larger of: alpha, beta, gamma for the f32-storage route (sequential kernel); the
+    // super-chunk states of the 16-bit route
     const size_t n = (size_t)batch * T * nheads;
-    return ((3 * n * sizeof(float)) + 255) & ~(size_t)255;
+    const size_t f32_route = ((3 * n * sizeof(float)) + 255) & ~(size_t)255;
+    int nsc, cps;
+    ssd_plan(batch, T, nheads, nsc, cps);
+    const size_t split = ssd_split_bytes(batch, nheads, headdim, d_state, nsc, nullptr, nullptr);
+    return f32_route > split ? f32_route : split;
 }
 
 extern "C" int mrs_m3_ssd_fwd(void *stream, int dtype, float *ssm_state, float *k_state, float *v_state, void *y,
@@ -379,6 +488,18 @@ extern "C" int mrs_m3_ssd_fwd(void *stream, int dtype, float *ssm_state, float *
     }
     if (!aligned(x, 16) || !aligned(K, 16) || !aligned(Q, 16) || !aligned(ssm_state, 16) || !aligned(k_state, 16))
         return fail(MRS_E_ALIGN, "%s: x, K, Q, ssm_state, k_state must be 16-byte aligned", fn);
-    if (dtype == MRS_BF16) return launch_ssd<bf16_t>(st, ssm_state, k_state, v_state, y, x, K, Q, dt, trap, a_val, D, batch, T, nheads, headdim, d_state, carry);
-    return launch_ssd<f16_t>(st, ssm_state, k_state, v_state, y, x, K, Q, dt, trap, a_val, D, batch, T, nheads, headdim, d_state, carry);
+    // Super-chunk split when the caller's workspace holds it; otherwise one workgroup walks the whole sequence.
+    SsdSplit sp = {nullptr, nullptr, nullptr, 1, (T + kCS - 1) / kCS};
+    {
+        int nsc, cps;
+        ssd_plan(batch, T, nheads, nsc, cps);
+        size_t o_dA, o_init;
+        const size_t need = ssd_split_bytes(batch, nheads, headdim, d_state, nsc, &o_dA, &o_init);
+        if (nsc > 1 && workspace && workspace_bytes >= need && aligned(workspace, 16)) {
+            char *ws = (char *)workspace;
+            sp = SsdSplit{(float *)ws, (float *)(ws + o_dA), (float *)(ws + o_init), nsc, cps};
+        }
+    }
+    if (dtype == MRS_BF16) return launch_ssd<bf16_t>(st, ssm_state, k_state, v_state, y, x, K, Q, dt, trap, a_val, D, sp, batch, T, nheads, headdim, d_state, carry);
+    return launch_ssd<f16_t>(st, ssm_state, k_state, v_state, y, x, K, Q, dt, trap, a_val, D, sp, batch, T, nheads, headdim, d_state, carry);
 }
