@@ -224,6 +224,17 @@ typedef struct {            /* MambaWeights, src/weights.rs:51-64 */
     const float *norm_f_weight; /* [d_model] */
 } mrs_m1_weights;
 
+/* ---- decode projections --------------------------------------------------------------------
+ * The reference sends the decode chain's projections to cuBLAS (gemm_ex call sites
+ * src/mamba_ssm/gpu/blas.rs:78-96, 721-737; tied head :709-740).  At batch <= 64 this library runs them
+ * on its own matrix-core kernel over a TRANSPOSED weight.
+ *   mrs_gemm_skinny: C[M,N] (row stride ldc; dtype, or f32 when out_f32) = A[M,K] (row stride lda) . Wt[N,K]^T
+ *     dtype f16/bf16 only, 1 <= M <= 64, K % 32 == 0, lda % 8 == 0, A and Wt 16-byte aligned; f32 accumulate.
+ *   mrs_transpose:   Wt[N,K] = W[K,N]^T (any dtype; builds the operand above from the reference's [K,N] layout). */
+MRS_API int mrs_gemm_skinny(void *stream, int dtype, void *C, int out_f32, int64_t ldc, const void *A, int64_t lda,
+                            const void *Wt, int M, int N, int K);
+MRS_API int mrs_transpose(void *stream, int dtype, void *Wt, const void *W, int K, int N);
+
 /* GpuMambaBackbone::new_with_dtype(gpu_ordinal, &weights, cfg, input_dim, batch, dtype)  (inference.rs:1517-1575).
  * Validates the config with the reference's bounds (src/config.rs:108-170). */
 MRS_API int mrs_backbone_create(mrs_backbone **out, int gpu_ordinal, const mrs_m1_weights *weights,

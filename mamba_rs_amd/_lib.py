@@ -36,6 +36,8 @@ _SIGNATURES = {
                                          c_int, c_int, c_int]),
     "mrs_conv1d_step": (c_int, [_P, c_int, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int]),
     "mrs_conv1d_seq_silu": (c_int, [_P, c_int, _P, _P, _P, c_int64, _P, _P, c_int, c_int, c_int, c_int]),
+    "mrs_gemm_skinny": (c_int, [_P, c_int, _P, c_int, c_int64, _P, c_int64, _P, c_int, c_int, c_int]),
+    "mrs_transpose": (c_int, [_P, c_int, _P, _P, c_int, c_int]),
     "mrs_m3_step": (c_int, [_P, c_int, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int]),
     "mrs_m3_seq_fwd": (c_int, [_P, c_int, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int]),
     "mrs_m3_compute_abg": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int64]),

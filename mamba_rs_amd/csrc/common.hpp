@@ -58,6 +58,34 @@ int launch_ssm_step_fused(hipStream_t st, int dtype, float *h, void *y, const vo
 int launch_conv1d_step(hipStream_t st, int dtype, void *out, float *state, const void *new_x, int64_t x_stride,
                        const float *weight, const float *bias, int batch, int d_inner, int d_conv, int apply_silu);
 
+// Skinny (M <= 64) 16-bit GEMM on a transposed weight, with the decode chain's fused prologue / epilogues.
+struct SkinnyEpi {
+    int mode;            // 0: store C
+                         // 1: in_proj  -- conv step + SiLU on columns < di, gate columns stored
+                         // 2: out_proj -- residual[row, col] += round(C); per-row sums of squares of the new
+                         //                residual over this workgroup's 16 columns go to partials[row][column tile]
+    float *conv_state;   // [M][di][dc]                                  (mode 1)
+    const float *conv_w, *conv_b;
+    void *u;             // [M][di], activation type
+    int di, dc;
+    float *residual;     // [M][N] f32, updated in place                 (mode 2)
+    float *partials;     // [M][n_partials] f32: written by mode 2, read when row_scale is set
+    int n_partials;
+    const float *next_norm_w;  // mode 2: norm weight of the layer after, or null (last layer)
+    void *prenorm;       // mode 2: [M][N] activation type, round(residual * next_norm_w): the next in_proj's operand
+    // RMSNorm folded around the product: A = round(residual * norm_w) and the sums are scaled by
+    // 1/rms[row], rms from the row's partials (row_scale != 0)
+    int row_scale;
+    float eps;
+};
+bool skinny_gemm_ok(int dtype, int M, int N, int K, int64_t lda, const void *A, const void *Wt);
+int launch_skinny_gemm(hipStream_t st, int dtype, void *C, int out_f32, int64_t ldc, const void *A, int64_t lda, const void *Wt,
+                       int M, int N, int K, const SkinnyEpi &ep);
+int launch_transpose(hipStream_t st, int dtype, void *Wt, const void *W, int K, int N);
+// partials[row][0] = sum_k x[row][k]^2, partials[row][1..n_partials) = 0; prenorm[row][k] = round(x[row][k] * w[k])
+int launch_prenorm_rows(hipStream_t st, int dtype, float *partials, int n_partials, void *prenorm, const float *x, const float *w,
+                        int M, int K);
+
 inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s); }
 inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 

@@ -13,6 +13,7 @@
 // dt-bias + softplus + state update + B/C gather + SiLU gate, out_proj.
 #include "common.hpp"
 #include <rocblas/rocblas.h>
+#include <stdlib.h>
 #include <new>
 #include <vector>
 
@@ -168,6 +169,7 @@ using namespace mrs;
 struct LayerDev {
     float *norm_w, *conv_w, *conv_b, *dt_b, *a_neg, *D;
     void *in_proj, *x_proj, *dt_w, *out_proj;
+    void *in_proj_t, *x_proj_t, *out_proj_t;  // [N][K] copies for the decode chain's own GEMM (null: library GEMM)
     int s4d;
 };
 
@@ -175,6 +177,7 @@ struct Scratch {  // activations for M rows
     int64_t rows = 0;
     void *normed = nullptr, *proj = nullptr, *u = nullptr, *xdbl = nullptr, *delta = nullptr, *y = nullptr, *out = nullptr;
     float *residual = nullptr;
+    float *partials = nullptr;  // [rows][d_model/16] row sums of squares, decode chain only
     void *scan_ws = nullptr;
     size_t scan_ws_bytes = 0;
     int T = 0;
@@ -183,6 +186,7 @@ struct Scratch {  // activations for M rows
 struct mrs_backbone {
     mrs_m1_config cfg;
     int input_dim, batch, dtype, di, dr, xd, identity_proj, device;
+    int skinny;  // decode projections on the library's own matrix-core GEMM (16-bit storage, batch <= 64, K % 32 == 0)
     hipStream_t stream;
     rocblas_handle blas;
     std::vector<LayerDev> layers;
@@ -233,6 +237,7 @@ static int alloc_scratch(mrs_backbone *bb, Scratch *s, int64_t rows, int T) {
     MRS_TRY(dev_alloc(bb, &s->delta, rows * di * es));
     MRS_TRY(dev_alloc(bb, &s->y, rows * di * es));
     MRS_TRY(dev_alloc(bb, &s->out, rows * dm * es));
+    if (T == 1) MRS_TRY(dev_alloc(bb, (void **)&s->partials, rows * (size_t)((dm + 15) / 16) * sizeof(float)));
     if (T > 1) {
         s->scan_ws_bytes = mrs_ssm_scan_workspace_bytes(bb->batch, T, di, bb->cfg.d_state);
         MRS_TRY(dev_alloc(bb, &s->scan_ws, s->scan_ws_bytes));
@@ -299,10 +304,34 @@ static int run_layers(mrs_backbone *bb, Scratch *s, int T) {
         const LayerDev &lw = bb->layers[l];
         float *conv = bb->conv_state + (size_t)l * B * di * dc;
         float *ssm = bb->ssm_state + (size_t)l * B * di * ds;
-        MRS_TRY(launch_add_rmsnorm(bb, s->residual, l == 0 ? nullptr : s->out, s->normed, false, lw.norm_w, rows, dm));
-        MRS_TRY(gemm_rm(bb, dt, s->proj, 2 * di, s->normed, dm, lw.in_proj, (int)rows, 2 * di, dm));
         const char *z = (const char *)s->proj + (size_t)di * es;  // gate half of in_proj's output
         const char *xb = (const char *)s->xdbl;
+        if (T == 1 && bb->skinny) {
+            // Decode chain on the library's own GEMM, four kernels per layer:
+            //   in_proj  on round(residual * norm_w) with the 1/rms row scale and the conv step + SiLU in its
+            //            epilogue (only u and the gate half are written),
+            //   x_proj,
+            //   dt_proj + softplus + scan step + gate,
+            //   out_proj with the residual add as its epilogue, which also leaves each row's sum of squares
+            //            (per 16-column tile) and round(residual * next norm_w) for the next layer's in_proj.
+            const int P = dm / 16;
+            if (l == 0) MRS_TRY(launch_prenorm_rows(bb->stream, dt, s->partials, P, s->normed, s->residual, lw.norm_w, B, dm));
+            SkinnyEpi inp = {};
+            inp.mode = 1; inp.conv_state = conv; inp.conv_w = lw.conv_w; inp.conv_b = lw.conv_b; inp.u = s->u; inp.di = di; inp.dc = dc;
+            inp.row_scale = 1; inp.partials = s->partials; inp.n_partials = P; inp.eps = bb->cfg.rms_norm_eps;
+            MRS_TRY(launch_skinny_gemm(bb->stream, dt, s->proj, 0, 2 * di, s->normed, dm, lw.in_proj_t, B, 2 * di, dm, inp));
+            const SkinnyEpi none = {};
+            MRS_TRY(launch_skinny_gemm(bb->stream, dt, s->xdbl, 0, xd, s->u, di, lw.x_proj_t, B, xd, di, none));
+            MRS_TRY(launch_ssm_step_fused(bb->stream, dt, ssm, s->y, s->delta, lw.dt_b, s->xdbl, lw.dt_w, dr, s->u, xb + es * dr,
+                                          xb + es * (dr + ds), xd, z, 2 * di, 2, lw.a_neg, lw.D, B, di, ds));
+            SkinnyEpi outp = {};
+            outp.mode = 2; outp.residual = s->residual; outp.partials = s->partials; outp.n_partials = P;
+            outp.next_norm_w = l + 1 < L ? bb->layers[l + 1].norm_w : nullptr; outp.prenorm = s->normed;
+            MRS_TRY(launch_skinny_gemm(bb->stream, dt, s->out, 0, dm, s->y, di, lw.out_proj_t, B, dm, di, outp));
+            continue;
+        }
+        MRS_TRY(launch_add_rmsnorm(bb, s->residual, l == 0 ? nullptr : s->out, s->normed, false, lw.norm_w, rows, dm));
+        MRS_TRY(gemm_rm(bb, dt, s->proj, 2 * di, s->normed, dm, lw.in_proj, (int)rows, 2 * di, dm));
         if (T == 1) {
             MRS_TRY(launch_conv1d_step(bb->stream, dt, s->u, conv, s->proj, 2 * di, lw.conv_w, lw.conv_b, B, di, dc, 1));
             MRS_TRY(gemm_rm(bb, dt, s->xdbl, xd, s->u, di, lw.x_proj, (int)rows, xd, di));
@@ -327,7 +356,8 @@ static int run_layers(mrs_backbone *bb, Scratch *s, int T) {
         MRS_TRY(gemm_rm(bb, dt, s->out, dm, s->y, di, lw.out_proj, (int)rows, dm, di));
     }
     if (T == 1) {
-        MRS_TRY(launch_add_rmsnorm(bb, s->residual, s->out, bb->temporal, true, bb->norm_f, rows, dm));
+        // (the out_proj epilogue of the own-GEMM chain has already added the last layer's output)
+        MRS_TRY(launch_add_rmsnorm(bb, s->residual, bb->skinny ? nullptr : s->out, bb->temporal, true, bb->norm_f, rows, dm));
     } else {
         // Only the last step of each sequence is kept (gather_last_timestep,
         // src/mamba_ssm/gpu/prefill.rs:1030-1046), so the final residual add + norm_f runs on those rows only.
@@ -382,6 +412,10 @@ extern "C" int mrs_backbone_create(mrs_backbone **out, int gpu_ordinal, const mr
         else { MRS_CREATE_TRY(dev_alloc(bb, (void **)&bb->input_proj_b, dm * 4)); hipMemsetAsync(bb->input_proj_b, 0, dm * 4, bb->stream); }
     }
     bb->layers.resize(L);
+    {
+        static const bool off = [] { const char *e = getenv("MRS_DECODE_LIBRARY_GEMM"); return e && atoi(e) != 0; }();
+        bb->skinny = !off && (dtype == MRS_BF16 || dtype == MRS_F16) && batch <= 64 && dm % 32 == 0 && di % 32 == 0;
+    }
     int *flag = nullptr;
     MRS_CREATE_TRY(dev_alloc(bb, (void **)&flag, sizeof(int)));
     for (int l = 0; l < L; l++) {
@@ -401,6 +435,17 @@ extern "C" int mrs_backbone_create(mrs_backbone **out, int gpu_ordinal, const mr
         MRS_CREATE_TRY(upload_f32(bb, &d.dt_b, src.dt_proj_b, di));
         MRS_CREATE_TRY(upload_f32(bb, &d.D, src.d_param, di));
         MRS_CREATE_TRY(upload_bulk(bb, &d.out_proj, src.out_proj_w, (size_t)di * dm, stage));
+        d.in_proj_t = d.x_proj_t = d.out_proj_t = nullptr;
+        if (bb->skinny) {
+            // transposed copies for the decode chain (one more copy of the bulk weights in HBM)
+            const size_t es_ = esize(bb->dtype);
+            MRS_CREATE_TRY(dev_alloc(bb, &d.in_proj_t, (size_t)dm * 2 * di * es_));
+            MRS_CREATE_TRY(dev_alloc(bb, &d.x_proj_t, (size_t)di * xd * es_));
+            MRS_CREATE_TRY(dev_alloc(bb, &d.out_proj_t, (size_t)di * dm * es_));
+            MRS_CREATE_TRY(launch_transpose(bb->stream, bb->dtype, d.in_proj_t, d.in_proj, dm, 2 * di));
+            MRS_CREATE_TRY(launch_transpose(bb->stream, bb->dtype, d.x_proj_t, d.x_proj, di, xd));
+            MRS_CREATE_TRY(launch_transpose(bb->stream, bb->dtype, d.out_proj_t, d.out_proj, di, dm));
+        }
         // a_neg = -exp(a_log) once at load (exp_negate, src/mamba_ssm/gpu/inference.rs:266-282)
         MRS_CREATE_TRY(dev_alloc(bb, (void **)&d.a_neg, (size_t)di * ds * 4));
         { hipError_t e = hipMemcpyAsync(stage, src.a_log, (size_t)di * ds * 4, hipMemcpyHostToDevice, bb->stream);

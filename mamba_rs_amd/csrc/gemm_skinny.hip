@@ -1,0 +1,255 @@
+// Skinny GEMM for the decode chain: C[M,N] = A[M,K] . Wt[N,K]^T with M <= 64 rows (the batch),
+// 16-bit operands, f32 accumulate on the matrix cores.
+//
+// The reference sends every decode projection to the vendor GEMM (cuBLAS call sites
+// src/mamba_ssm/gpu/blas.rs:78-96, 721-737).  At M <= 64 those calls are latency-bound: the work is a
+// single pass over the weights (4.7 MB for in_proj at d_model 768), and what matters is that all of it is
+// in flight at once and that the kernel ends as soon as the last byte has arrived.  Here:
+//   * the weight is kept transposed, Wt[N][K], so that both MFMA operands are 16-byte row reads:
+//     v_mfma_f32_16x16x32 takes A[m = l%16][k = 8(l/16)..+7] and B[k = 8(l/16)..+7][n = l%16], i.e. 8
+//     consecutive k of activation row m and of weight row n (the k order inside the instruction is the
+//     same for both operands, which is all a dot product needs);
+//   * a workgroup owns a 16x16 output tile; its 8 waves split K (interleaved 32-wide steps), so a
+//     K = 768 product is 3 steps per wave with every load independent; the partial tiles meet in LDS;
+//   * the epilogue is fused: plain store (16-bit or f32), or in_proj's -- the x half of the row goes
+//     straight through the depthwise conv step + SiLU (conv1d_step_forward_silu, kernels/conv1d.cu:85-115)
+//     and only u and the gate half are written.
+#include "common.hpp"
+
+namespace mrs {
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+
+template <typename T> struct Mma32;
+template <> struct Mma32<bf16_t> {
+    __device__ static __forceinline__ v4f mma(uint4 a, uint4 b, v4f c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, b), c, 0, 0, 0);
+    }
+};
+template <> struct Mma32<f16_t> {
+    __device__ static __forceinline__ v4f mma(uint4 a, uint4 b, v4f c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, b), c, 0, 0, 0);
+    }
+};
+
+constexpr int kGemmWaves = 8;
+constexpr int kMaxConvTaps = 8;
+
+template <typename TO> __device__ __forceinline__ void store_out(TO *p, float v) { Store<TO>::st(p, v); }
+
+// EPI 0: C[row, col] = sum (TO = T or float)
+// EPI 1: in_proj of a Mamba-1 layer: columns < di are conv inputs (conv state [M][di][dc] f32 shifted in
+//        place, u[row, col] = silu(conv)), columns >= di (the gate) are stored to C.
+// Grid: x = 16-column tile, y = 16-row tile.  A workgroup pulls 16 rows of A and 16 rows of Wt through
+// its L1 (49 KB each at K = 1536); measured, the time of this kernel is set by the bytes ONE workgroup has
+// to pull (wider or taller tiles per workgroup were slower: 6.4 -> 7.5 us at 32 columns, 3.3 -> 6.4 us at
+// 64 rows, K = 768), so tiles are kept minimal and the re-reads of Wt by the row tiles are left to L2.
+constexpr int kStepsPerBatch = 6;  // k-steps whose loads are issued together (covers K <= 1536 in one round trip)
+
+// PRO 1 (RMSNorm folded around the product): A holds round_T(residual[row,k] * norm_w[k]) -- the row scale
+// 1/rms[row] commutes with the product, so it is applied to the f32 sums in the epilogue:
+//   rmsnorm(x) . W = (1/rms) * ((x * w) . W)
+// (rmsnorm_forward_f32in, kernels/norms.cu:21-171, with its guard rms = 1 when not finite or < 1e-20).
+// rms comes from the row's partial sums of squares, which the out_proj epilogue before it (or
+// prenorm_rows_kernel for the first layer) left behind together with A.  Against the reference's order the
+// rounding to the storage type happens before the row scale instead of after it: same relative error.
+template <typename T, typename TO, int EPI, int PRO>
+__global__ __launch_bounds__(kGemmWaves * 64) void skinny_gemm_kernel(
+    TO *__restrict__ C, int64_t ldc, const T *__restrict__ A, int64_t lda, const T *__restrict__ Wt, int M, int N, int K,
+    SkinnyEpi ep) {
+    __shared__ v4f red[kGemmWaves / 2][kWave];
+    const int n0 = blockIdx.x * 16, m0 = blockIdx.y * 16;
+    const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, lr = l & 15, lg = l >> 4;
+    const int nk = K >> 5;
+    v4f acc = {0.f, 0.f, 0.f, 0.f};
+    // Rows past M / columns past N are clamped to the last valid one: their products land in
+    // accumulator elements that are never stored.
+    const T *wrow = Wt + (int64_t)min(n0 + lr, N - 1) * K + 8 * lg;
+    const T *arow = A + (int64_t)min(m0 + lr, M - 1) * lda + 8 * lg;
+    float inv = 1.0f;
+    if (PRO == 1 && tid < 256) {
+        // epilogue thread (row tid/16, column tid%16): the 16 lanes of a row share the sum over the partials
+        const float *pp = ep.partials + (int64_t)min(m0 + (tid >> 4), M - 1) * ep.n_partials;
+        float ss = 0.0f;
+        for (int p = tid & 15; p < ep.n_partials; p += 16) ss += pp[p];
+#pragma unroll
+        for (int m = 8; m >= 1; m >>= 1) ss += __shfl_xor(ss, m, kWave);
+        float rms = sqrtf(ss / (float)K + ep.eps);
+        if (!isfinite(rms) || rms < 1e-20f) rms = 1.0f;
+        inv = 1.0f / rms;
+    }
+    for (int base = w; base < nk; base += kGemmWaves * kStepsPerBatch) {
+        uint4 bf[kStepsPerBatch], af[kStepsPerBatch];
+#pragma unroll
+        for (int s = 0; s < kStepsPerBatch; s++) {
+            const int ks = base + s * kGemmWaves;
+            if (ks < nk) {
+                bf[s] = *reinterpret_cast<const uint4 *>(wrow + 32 * ks);
+                af[s] = *reinterpret_cast<const uint4 *>(arow + 32 * ks);
+            }
+        }
+#pragma unroll
+        for (int s = 0; s < kStepsPerBatch; s++)
+            if (base + s * kGemmWaves < nk) acc = Mma32<T>::mma(af[s], bf[s], acc);
+    }
+    // K-split reduction: upper half of the waves parks its tile in LDS, lower half adds and parks the sums
+    if (w >= kGemmWaves / 2) red[w - kGemmWaves / 2][l] = acc;
+    __syncthreads();
+    if (w < kGemmWaves / 2) red[w][l] += acc;
+    __syncthreads();
+    // element e of the 16x16 tile: row ml = e / 16, column nl = e % 16 lives in lane 16 (ml / 4) + nl, register ml % 4
+    if (tid < 256) {
+        const int ml = tid >> 4, nl = tid & 15;
+        const int lane = (ml >> 2) * 16 + nl, i = ml & 3;
+        float s = 0.0f;
+#pragma unroll
+        for (int ww = 0; ww < kGemmWaves / 2; ww++) s += red[ww][lane][i];
+        s *= inv;
+        const int row = m0 + ml, col = n0 + nl;
+        const bool valid = row < M && col < N;
+        if (EPI == 2) {
+            // out_proj: residual += out (rounded to the storage type as the stored projection would be); the
+            // row's sum of squares over these 16 columns and the pre-scaled operand for the next layer's in_proj
+            float sq = 0.0f;
+            if (valid) {
+                const T orr = (T)s;
+                float *rp = ep.residual + (int64_t)row * N + col;
+                const float rn = *rp + Store<T>::ld(&orr);
+                *rp = rn;
+                sq = rn * rn;
+                if (ep.next_norm_w) Store<T>::st(reinterpret_cast<T *>(ep.prenorm) + (int64_t)row * N + col, rn * ep.next_norm_w[col]);
+            }
+#pragma unroll
+            for (int m = 8; m >= 1; m >>= 1) sq += __shfl_xor(sq, m, kWave);
+            if (nl == 0 && row < M) ep.partials[(int64_t)row * ep.n_partials + blockIdx.x] = sq;
+        } else if (!valid) {
+        } else if (EPI == 1 && col < ep.di) {
+            // conv step on the value as in_proj would have stored it (rounded to the storage type)
+            const T xr = (T)s;
+            const float xnew = Store<T>::ld(&xr);
+            float *st = ep.conv_state + ((int64_t)row * ep.di + col) * ep.dc;
+            const float *cw = ep.conv_w + (int64_t)col * ep.dc;
+            float o = ep.conv_b[col];
+            float win[kMaxConvTaps];
+#pragma unroll
+            for (int k = 0; k < kMaxConvTaps; k++)
+                if (k < ep.dc) win[k] = (k + 1 < ep.dc) ? st[k + 1] : xnew;
+#pragma unroll
+            for (int k = 0; k < kMaxConvTaps; k++)
+                if (k < ep.dc) { o = fmaf(win[k], cw[k], o); st[k] = win[k]; }
+            Store<T>::st(reinterpret_cast<T *>(ep.u) + (int64_t)row * ep.di + col, silu(o));
+        } else {
+            store_out<TO>(C + (int64_t)row * ldc + col, s);
+        }
+    }
+}
+
+// First layer's share of the folded norm: partials[row][0] = sum_k x[row][k]^2 (other slots zero) and
+// prenorm[row][k] = round_T(x[row][k] * w[k]), for a residual stream no out_proj epilogue has produced yet.
+template <typename T>
+__global__ __launch_bounds__(256) void prenorm_rows_kernel(float *__restrict__ partials, int n_partials, T *__restrict__ prenorm,
+                                                           const float *__restrict__ x, const float *__restrict__ w, int K) {
+    __shared__ float part[4];
+    const int64_t row = blockIdx.x;
+    float ss = 0.0f;
+    for (int i = threadIdx.x; i < K; i += 256) {
+        const float v = x[row * K + i];
+        ss = fmaf(v, v, ss);
+        Store<T>::st(prenorm + row * K + i, v * w[i]);
+    }
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) ss += __shfl_xor(ss, m, kWave);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    for (int p = threadIdx.x; p < n_partials; p += 256) partials[row * n_partials + p] = p == 0 ? part[0] + part[1] + part[2] + part[3] : 0.0f;
+}
+
+// Wt[n][k] = W[k][n]: 32x32 tiles through LDS so both sides are coalesced.
+template <typename T>
+__global__ __launch_bounds__(256) void transpose_kernel(T *__restrict__ Wt, const T *__restrict__ W, int K, int N) {
+    __shared__ T tile[32][33];
+    const int k0 = blockIdx.y * 32, n0 = blockIdx.x * 32;
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+    for (int r = ty; r < 32; r += 8)
+        if (k0 + r < K && n0 + tx < N) tile[r][tx] = W[(int64_t)(k0 + r) * N + n0 + tx];
+    __syncthreads();
+    for (int r = ty; r < 32; r += 8)
+        if (n0 + r < N && k0 + tx < K) Wt[(int64_t)(n0 + r) * K + k0 + tx] = tile[tx][r];
+}
+
+template <typename T, typename TO>
+static int launch_skinny_t(hipStream_t st, TO *C, int64_t ldc, const T *A, int64_t lda, const T *Wt, int M, int N, int K,
+                           const SkinnyEpi &ep) {
+    const dim3 grid((unsigned)((N + 15) / 16), (unsigned)((M + 15) / 16)), block(kGemmWaves * 64);
+#define MRS_SG(EPI_, PRO_) hipLaunchKernelGGL((skinny_gemm_kernel<T, TO, EPI_, PRO_>), grid, block, 0, st, C, ldc, A, lda, Wt, M, N, K, ep)
+    const bool pro = ep.row_scale != 0;
+    if (ep.mode != 0 && sizeof(TO) != sizeof(T)) return fail(MRS_E_DTYPE, "skinny gemm: fused epilogues store the activation type");
+    if constexpr (sizeof(TO) == sizeof(T)) {
+        if (ep.mode == 1) { if (pro) MRS_SG(1, 1); else MRS_SG(1, 0); return check_launch("skinny_gemm_kernel"); }
+        if (ep.mode == 2) { if (pro) MRS_SG(2, 1); else MRS_SG(2, 0); return check_launch("skinny_gemm_kernel"); }
+    }
+    if (pro) MRS_SG(0, 1); else MRS_SG(0, 0);
+#undef MRS_SG
+    return check_launch("skinny_gemm_kernel");
+}
+
+bool skinny_gemm_ok(int dtype, int M, int N, int K, int64_t lda, const void *A, const void *Wt) {
+    return (dtype == MRS_BF16 || dtype == MRS_F16) && M >= 1 && M <= 64 && N >= 1 && K >= 32 && K % 32 == 0 && lda % 8 == 0 &&
+           aligned(A, 16) && aligned(Wt, 16);
+}
+
+int launch_skinny_gemm(hipStream_t st, int dtype, void *C, int out_f32, int64_t ldc, const void *A, int64_t lda, const void *Wt,
+                       int M, int N, int K, const SkinnyEpi &ep) {
+    if (!skinny_gemm_ok(dtype, M, N, K, lda, A, Wt))
+        return fail(MRS_E_SHAPE, "skinny gemm: needs 16-bit storage, 1 <= M <= 64, K %% 32 == 0, lda %% 8 == 0, 16-byte aligned A and Wt "
+                                 "(got dtype=%d M=%d N=%d K=%d lda=%lld)", dtype, M, N, K, (long long)lda);
+    if (ep.mode == 1 && (ep.dc < 1 || ep.dc > kMaxConvTaps || ep.di < 1 || ep.di > N || !ep.conv_state || !ep.conv_w || !ep.conv_b || !ep.u))
+        return fail(MRS_E_SHAPE, "skinny gemm: bad in_proj epilogue (di=%d dc=%d)", ep.di, ep.dc);
+    if (ep.mode == 2 && (!ep.residual || !ep.partials || ep.n_partials != (N + 15) / 16 || (ep.next_norm_w && !ep.prenorm)))
+        return fail(MRS_E_SHAPE, "skinny gemm: bad out_proj epilogue (n_partials=%d, column tiles=%d)", ep.n_partials, (N + 15) / 16);
+    if (ep.row_scale && (!ep.partials || ep.n_partials < 1))
+        return fail(MRS_E_SHAPE, "skinny gemm: row scale without partial sums");
+    if (dtype == MRS_BF16) {
+        if (out_f32) return launch_skinny_t<bf16_t, float>(st, (float *)C, ldc, (const bf16_t *)A, lda, (const bf16_t *)Wt, M, N, K, ep);
+        return launch_skinny_t<bf16_t, bf16_t>(st, (bf16_t *)C, ldc, (const bf16_t *)A, lda, (const bf16_t *)Wt, M, N, K, ep);
+    }
+    if (out_f32) return launch_skinny_t<f16_t, float>(st, (float *)C, ldc, (const f16_t *)A, lda, (const f16_t *)Wt, M, N, K, ep);
+    return launch_skinny_t<f16_t, f16_t>(st, (f16_t *)C, ldc, (const f16_t *)A, lda, (const f16_t *)Wt, M, N, K, ep);
+}
+
+int launch_prenorm_rows(hipStream_t st, int dtype, float *partials, int n_partials, void *prenorm, const float *x, const float *w,
+                        int M, int K) {
+    if (dtype == MRS_BF16) hipLaunchKernelGGL((prenorm_rows_kernel<bf16_t>), dim3((unsigned)M), dim3(256), 0, st, partials, n_partials, (bf16_t *)prenorm, x, w, K);
+    else if (dtype == MRS_F16) hipLaunchKernelGGL((prenorm_rows_kernel<f16_t>), dim3((unsigned)M), dim3(256), 0, st, partials, n_partials, (f16_t *)prenorm, x, w, K);
+    else return fail(MRS_E_DTYPE, "prenorm rows: 16-bit storage only");
+    return check_launch("prenorm_rows_kernel");
+}
+
+int launch_transpose(hipStream_t st, int dtype, void *Wt, const void *W, int K, int N) {
+    const dim3 grid((unsigned)((N + 31) / 32), (unsigned)((K + 31) / 32)), block(256);
+    if (dtype == MRS_F32) hipLaunchKernelGGL((transpose_kernel<float>), grid, block, 0, st, (float *)Wt, (const float *)W, K, N);
+    else hipLaunchKernelGGL((transpose_kernel<uint16_t>), grid, block, 0, st, (uint16_t *)Wt, (const uint16_t *)W, K, N);
+    return check_launch("transpose_kernel");
+}
+
+}  // namespace mrs
+
+using namespace mrs;
+
+extern "C" int mrs_gemm_skinny(void *stream, int dtype, void *C, int out_f32, int64_t ldc, const void *A, int64_t lda,
+                               const void *Wt, int M, int N, int K) {
+    if (!C || !A || !Wt) return fail(MRS_E_NULL, "mrs_gemm_skinny: null pointer");
+    if (ldc < N) return fail(MRS_E_SHAPE, "mrs_gemm_skinny: ldc=%lld < N=%d", (long long)ldc, N);
+    if (lda < K) return fail(MRS_E_SHAPE, "mrs_gemm_skinny: lda=%lld < K=%d", (long long)lda, K);
+    SkinnyEpi ep = {};
+    return launch_skinny_gemm(as_stream(stream), dtype, C, out_f32, ldc, A, lda, Wt, M, N, K, ep);
+}
+
+extern "C" int mrs_transpose(void *stream, int dtype, void *Wt, const void *W, int K, int N) {
+    if (!Wt || !W) return fail(MRS_E_NULL, "mrs_transpose: null pointer");
+    if (dtype != MRS_F32 && dtype != MRS_F16 && dtype != MRS_BF16) return fail(MRS_E_DTYPE, "mrs_transpose: dtype %d", dtype);
+    if (K < 1 || N < 1) return fail(MRS_E_SHAPE, "mrs_transpose: K=%d N=%d", K, N);
+    return launch_transpose(as_stream(stream), dtype, Wt, W, K, N);
+}

@@ -41,8 +41,24 @@ __global__ __launch_bounds__(256) void ssm_step_kernel(
         // dt_proj folded in: delta_raw[b,d] = sum_r dt_in[b,r] * dt_w[r,d], the dt_rank terms split over the
         // LG lanes of the row (dt_proj GEMM of the decode chain, src/mamba_ssm/gpu/inference.rs:1129-1146)
         const T *xr = dt_in + (int64_t)b * bc_stride;
+        const T *wc = dt_w + d;
         float part = 0.0f;
-        for (int k = g; k < dr; k += LG) part = fmaf(Store<T>::ld(xr + k), Store<T>::ld(dt_w + (int64_t)k * di + d), part);
+        // batches of 12 terms per lane with every load of a batch issued before the first multiply-add:
+        // the loop is a latency chain otherwise (dt_rank 48 over 4 lanes = one batch)
+        constexpr int kBatch = 12;
+        for (int k0 = g; k0 < dr; k0 += kBatch * LG) {
+            float xv[kBatch], wv[kBatch];
+#pragma unroll
+            for (int j = 0; j < kBatch; j++) {
+                const int k = k0 + j * LG;
+                const int kc = k < dr ? k : g;   // in-range address for the masked-off terms
+                xv[j] = Store<T>::ld(xr + kc);
+                wv[j] = Store<T>::ld(wc + (int64_t)kc * di);
+                if (k >= dr) xv[j] = 0.0f;
+            }
+#pragma unroll
+            for (int j = 0; j < kBatch; j++) part = fmaf(xv[j], wv[j], part);
+        }
 #pragma unroll
         for (int m = 1; m < LG; m <<= 1) part += __shfl_xor(part, m, kWave);
         dl = part;

@@ -142,6 +142,33 @@ def conv1d_step(out, state, new_x, weight, bias, *, silu: bool = True):
     return out
 
 
+def transpose(w):
+    """Wt[N,K] = W[K,N]^T on the device: the operand layout of gemm_skinny."""
+    if w.dim() != 2 or not w.is_contiguous():
+        raise ValueError("w must be a contiguous [K,N] matrix")
+    _dev(w)
+    K, N = w.shape
+    wt = torch.empty(N, K, device=w.device, dtype=w.dtype)
+    _lib.call("mrs_transpose", _stream(), int(_act_dtype(w)), _p(wt), _p(w), K, N)
+    return wt
+
+
+def gemm_skinny(a, wt, *, out_f32: bool = False):
+    """C[M,N] = A[M,K] . Wt[N,K]^T for the decode chain (M <= 64, 16-bit operands, f32 accumulate): the
+    projections the reference sends to cuBLAS (src/mamba_ssm/gpu/blas.rs:78-96)."""
+    _dev(wt)
+    if not a.is_cuda:
+        raise ValueError("mamba_rs_amd ops need device tensors (there is no CPU path)")
+    if a.dim() != 2 or wt.dim() != 2 or a.shape[1] != wt.shape[1] or a.stride(1) != 1:
+        raise ValueError("a [M,K] (unit inner stride) and wt [N,K] (contiguous) must share K")
+    M, K = a.shape
+    N = wt.shape[0]
+    dt = _act_dtype(a, wt)
+    c = torch.empty(M, N, device=a.device, dtype=torch.float32 if out_f32 else a.dtype)
+    _lib.call("mrs_gemm_skinny", _stream(), int(dt), _p(c), 1 if out_f32 else 0, N, _p(a), a.stride(0), _p(wt), M, N, K)
+    return c
+
+
 def conv1d_seq_silu(u_out, state, x_branch, weight, bias):
     """Full-sequence causal conv + SiLU with state carry
     (conv1d_burnin_forward_nosave, kernels/conv1d.cu:209-315).

@@ -1,0 +1,61 @@
+"""GPU parity: the decode chain's skinny matrix-core GEMM (and the weight transpose that feeds it) against a
+float64 matmul of the same 16-bit operands, through the C ABI."""
+import numpy as np
+import pytest
+import torch
+
+import orc
+from gpu_util import DEV, assert_close, dev, host, quant
+
+pytestmark = pytest.mark.gpu
+
+ops = pytest.importorskip("mamba_rs_amd.ops")
+
+# (M, N, K): the 130m decode projections at batch 64 and 1, ragged M / N, the smallest K
+SHAPES = [(64, 3072, 768), (64, 80, 1536), (64, 768, 1536), (1, 3072, 768), (1, 80, 1536), (5, 33, 32), (17, 100, 96),
+          (48, 16, 2560), (33, 1000, 64), (64, 50, 1024)]
+
+
+@pytest.mark.parametrize("dtype", [orc.BF16, orc.F16])
+@pytest.mark.parametrize("shape", SHAPES)
+@pytest.mark.parametrize("out_f32", [False, True])
+def test_gemm_skinny_matches_f64_matmul(shape, dtype, out_f32):
+    M, N, K = shape
+    rng = np.random.default_rng(hash((shape, dtype)) & 0xFFFF)
+    a = quant(rng.standard_normal((M, K)).astype(np.float32), dtype)
+    w = quant((rng.standard_normal((K, N)) / np.sqrt(K)).astype(np.float32), dtype)   # the reference's [K, N] layout
+    print(f"case gemm_skinny shape={shape} dtype={dtype} out_f32={out_f32}", flush=True)
+    wt = ops.transpose(dev(w, dtype))
+    assert np.array_equal(host(wt), w.T)
+    c = ops.gemm_skinny(dev(a, dtype), wt, out_f32=out_f32)
+    ref = a.astype(np.float64) @ w.astype(np.float64)
+    # f32 accumulation of exact 16-bit products: 1e-4 of the row scale when the result stays f32
+    assert_close(host(c), ref, orc.F32 if out_f32 else dtype, "C")
+
+
+def test_gemm_skinny_strided_rows_and_f32_transpose():
+    """A may be a view into wider rows (e.g. a slice of a projection); transpose also serves f32 tables."""
+    rng = np.random.default_rng(3)
+    M, N, K = 12, 40, 64
+    wide = quant(rng.standard_normal((M, 3 * K)).astype(np.float32), orc.BF16)
+    w = quant(rng.standard_normal((K, N)).astype(np.float32), orc.BF16)
+    a = dev(wide, orc.BF16)[:, K:2 * K]
+    c = ops.gemm_skinny(a, ops.transpose(dev(w, orc.BF16)), out_f32=True)
+    assert_close(host(c), wide[:, K:2 * K].astype(np.float64) @ w.astype(np.float64), orc.F32, "C (strided A)")
+    f = rng.standard_normal((37, 53)).astype(np.float32)
+    assert np.array_equal(host(ops.transpose(dev(f))), f.T)
+
+
+def test_gemm_skinny_rejects_bad_arguments():
+    from mamba_rs_amd import MambaHipError
+    a = torch.zeros(65, 64, device=DEV, dtype=torch.bfloat16)
+    wt = torch.zeros(16, 64, device=DEV, dtype=torch.bfloat16)
+    with pytest.raises(MambaHipError) as e:   # M > 64
+        ops.gemm_skinny(a, wt)
+    assert e.value.code == -2
+    with pytest.raises(MambaHipError) as e:   # K not a multiple of 32
+        ops.gemm_skinny(torch.zeros(4, 48, device=DEV, dtype=torch.bfloat16), torch.zeros(16, 48, device=DEV, dtype=torch.bfloat16))
+    assert e.value.code == -2
+    with pytest.raises(MambaHipError) as e:   # f32 storage goes to the library GEMM, not here
+        ops.gemm_skinny(torch.zeros(4, 64, device=DEV), torch.zeros(16, 64, device=DEV))
+    assert e.value.code == -2
