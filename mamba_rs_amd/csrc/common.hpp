@@ -52,7 +52,7 @@ int check_launch(const char *what);
 
 // Internal launchers shared with the backbone engine (strides and fusions the public entry points do not expose).
 int launch_ssm_step_fused(hipStream_t st, int dtype, float *h, void *y, const void *delta, const float *dt_bias,
-                          const void *dt_in, const void *dt_w, int dr, const void *u, const void *Bb, const void *Cb, int64_t bc_stride, const void *gate,
+                          const void *dt_in, const void *dt_w, int dr, int dt_transposed, const void *u, const void *Bb, const void *Cb, int64_t bc_stride, const void *gate,
                           int64_t gate_stride, int gate_mode, const float *a_neg, const float *D, int batch,
                           int di, int ds);
 int launch_conv1d_step(hipStream_t st, int dtype, void *out, float *state, const void *new_x, int64_t x_stride,
@@ -83,8 +83,8 @@ int launch_skinny_gemm(hipStream_t st, int dtype, void *C, int out_f32, int64_t 
                        int M, int N, int K, const SkinnyEpi &ep);
 int launch_transpose(hipStream_t st, int dtype, void *Wt, const void *W, int K, int N);
 // partials[row][0] = sum_k x[row][k]^2, partials[row][1..n_partials) = 0; prenorm[row][k] = round(x[row][k] * w[k])
-int launch_prenorm_rows(hipStream_t st, int dtype, float *partials, int n_partials, void *prenorm, const float *x, const float *w,
-                        int M, int K);
+int launch_prenorm_rows(hipStream_t st, int dtype, float *partials, int n_partials, void *prenorm, const float *x, float *copy_to,
+                        const float *w, int M, int K);
 
 inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s); }
 inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }

@@ -45,9 +45,10 @@ static rocblas_datatype blas_type(int dtype) {
 // One workgroup per row: residual (f32) += add (storage dtype, may be null); out = rmsnorm(residual) * w.
 // Reference: residual_add_f32_* + rmsnorm_forward_f32in_* (kernels/elementwise.cu:366-376,
 // kernels/norms.cu:21-171), with its finite guard: rms = 1 if not finite or < 1e-20 (norms.cu:58-61).
+// out2 (may be null): the same result once more in the storage type (the LM head's operand).
 template <typename T, typename TO>
 __global__ __launch_bounds__(256) void add_rmsnorm_kernel(float *__restrict__ residual, const T *__restrict__ add,
-                                                          TO *__restrict__ out, const float *__restrict__ w,
+                                                          TO *__restrict__ out, T *__restrict__ out2, const float *__restrict__ w,
                                                           float eps, int64_t rows, int dm, int64_t out_stride) {
     constexpr int kMaxPer = 16;  // elements per thread kept in registers (d_model <= 4096); longer rows re-read
     __shared__ float part[4];
@@ -73,7 +74,9 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(float *__restrict__ re
     cnt = 0;
     for (int i = threadIdx.x; i < dm; i += 256, cnt++) {
         const float x = cnt < kMaxPer ? v[cnt] : r[i];
-        Store<TO>::st(out + row * out_stride + i, x * inv * w[i]);
+        const float o = x * inv * w[i];
+        Store<TO>::st(out + row * out_stride + i, o);
+        if (out2) Store<T>::st(out2 + row * out_stride + i, o);
     }
 }
 
@@ -169,6 +172,7 @@ using namespace mrs;
 struct LayerDev {
     float *norm_w, *conv_w, *conv_b, *dt_b, *a_neg, *D;
     void *in_proj, *x_proj, *dt_w, *out_proj;
+    void *dt_w_t;  // [d_inner][dt_rank] copy for the fused decode step (null: the [dt_rank][d_inner] one is read)
     void *in_proj_t, *x_proj_t, *out_proj_t;  // [N][K] copies for the decode chain's own GEMM (null: library GEMM)
     int s4d;
 };
@@ -186,6 +190,7 @@ struct Scratch {  // activations for M rows
 struct mrs_backbone {
     mrs_m1_config cfg;
     int input_dim, batch, dtype, di, dr, xd, identity_proj, device;
+    const float *step_src;  // decode step: where layer 0 reads its input rows (null: the residual buffer itself)
     int skinny;  // decode projections on the library's own matrix-core GEMM (16-bit storage, batch <= 64, K % 32 == 0)
     hipStream_t stream;
     rocblas_handle blas;
@@ -194,6 +199,7 @@ struct mrs_backbone {
     std::vector<void *> allocs;
     float *conv_state, *ssm_state;
     float *d_input, *temporal;
+    void *temporal_t;  // decode: temporal once more in the storage type (16-bit engines), the LM head's operand
     Scratch step_s, prefill_s;
     float *prefill_in;  // [batch*T, input_dim] f32 staging for host input
     hipGraph_t graph;
@@ -256,18 +262,18 @@ static int gemm_rm(mrs_backbone *bb, int dtype, void *C, int ldc, const void *A,
 
 template <typename T>
 static void launch_add_rmsnorm_t(mrs_backbone *bb, float *residual, const void *add, void *out, bool out_f32,
-                                 const float *w, int64_t rows, int64_t out_stride) {
+                                 const float *w, int64_t rows, int64_t out_stride, void *out2) {
     const dim3 grid((unsigned)rows), block(256);
     if (out_f32)
-        hipLaunchKernelGGL((add_rmsnorm_kernel<T, float>), grid, block, 0, bb->stream, residual, (const T *)add, (float *)out, w,
+        hipLaunchKernelGGL((add_rmsnorm_kernel<T, float>), grid, block, 0, bb->stream, residual, (const T *)add, (float *)out, (T *)out2, w,
                            bb->cfg.rms_norm_eps, rows, bb->cfg.d_model, out_stride);
     else
-        hipLaunchKernelGGL((add_rmsnorm_kernel<T, T>), grid, block, 0, bb->stream, residual, (const T *)add, (T *)out, w,
+        hipLaunchKernelGGL((add_rmsnorm_kernel<T, T>), grid, block, 0, bb->stream, residual, (const T *)add, (T *)out, (T *)out2, w,
                            bb->cfg.rms_norm_eps, rows, bb->cfg.d_model, out_stride);
 }
 static int launch_add_rmsnorm(mrs_backbone *bb, float *residual, const void *add, void *out, bool out_f32, const float *w,
-                              int64_t rows, int64_t out_stride) {
-    MRS_DISPATCH_DTYPE(bb->dtype, T_, launch_add_rmsnorm_t<T_>(bb, residual, add, out, out_f32, w, rows, out_stride));
+                              int64_t rows, int64_t out_stride, void *out2 = nullptr) {
+    MRS_DISPATCH_DTYPE(bb->dtype, T_, launch_add_rmsnorm_t<T_>(bb, residual, add, out, out_f32, w, rows, out_stride, out2));
     return check_launch("add_rmsnorm_kernel");
 }
 
@@ -315,14 +321,17 @@ static int run_layers(mrs_backbone *bb, Scratch *s, int T) {
             //   out_proj with the residual add as its epilogue, which also leaves each row's sum of squares
             //            (per 16-column tile) and round(residual * next norm_w) for the next layer's in_proj.
             const int P = dm / 16;
-            if (l == 0) MRS_TRY(launch_prenorm_rows(bb->stream, dt, s->partials, P, s->normed, s->residual, lw.norm_w, B, dm));
+            if (l == 0)
+                MRS_TRY(launch_prenorm_rows(bb->stream, dt, s->partials, P, s->normed, bb->step_src ? bb->step_src : s->residual,
+                                            bb->step_src ? s->residual : nullptr, lw.norm_w, B, dm));
             SkinnyEpi inp = {};
             inp.mode = 1; inp.conv_state = conv; inp.conv_w = lw.conv_w; inp.conv_b = lw.conv_b; inp.u = s->u; inp.di = di; inp.dc = dc;
             inp.row_scale = 1; inp.partials = s->partials; inp.n_partials = P; inp.eps = bb->cfg.rms_norm_eps;
             MRS_TRY(launch_skinny_gemm(bb->stream, dt, s->proj, 0, 2 * di, s->normed, dm, lw.in_proj_t, B, 2 * di, dm, inp));
             const SkinnyEpi none = {};
             MRS_TRY(launch_skinny_gemm(bb->stream, dt, s->xdbl, 0, xd, s->u, di, lw.x_proj_t, B, xd, di, none));
-            MRS_TRY(launch_ssm_step_fused(bb->stream, dt, ssm, s->y, s->delta, lw.dt_b, s->xdbl, lw.dt_w, dr, s->u, xb + es * dr,
+            MRS_TRY(launch_ssm_step_fused(bb->stream, dt, ssm, s->y, s->delta, lw.dt_b, s->xdbl, lw.dt_w_t ? lw.dt_w_t : lw.dt_w, dr,
+                                          lw.dt_w_t != nullptr, s->u, xb + es * dr,
                                           xb + es * (dr + ds), xd, z, 2 * di, 2, lw.a_neg, lw.D, B, di, ds));
             SkinnyEpi outp = {};
             outp.mode = 2; outp.residual = s->residual; outp.partials = s->partials; outp.n_partials = P;
@@ -336,7 +345,8 @@ static int run_layers(mrs_backbone *bb, Scratch *s, int T) {
             MRS_TRY(launch_conv1d_step(bb->stream, dt, s->u, conv, s->proj, 2 * di, lw.conv_w, lw.conv_b, B, di, dc, 1));
             MRS_TRY(gemm_rm(bb, dt, s->xdbl, xd, s->u, di, lw.x_proj, (int)rows, xd, di));
             // dt_proj (K = dt_rank) + bias + softplus + state update + B/C gather + SiLU gate: one kernel
-            MRS_TRY(launch_ssm_step_fused(bb->stream, dt, ssm, s->y, s->delta, lw.dt_b, s->xdbl, lw.dt_w, dr, s->u, xb + es * dr,
+            MRS_TRY(launch_ssm_step_fused(bb->stream, dt, ssm, s->y, s->delta, lw.dt_b, s->xdbl, lw.dt_w_t ? lw.dt_w_t : lw.dt_w, dr,
+                                          lw.dt_w_t != nullptr, s->u, xb + es * dr,
                                           xb + es * (dr + ds), xd, z, 2 * di, 2, lw.a_neg, lw.D, B, di, ds));
         } else {
             MRS_TRY(mrs_conv1d_seq_silu(bb->stream, dt, s->u, conv, s->proj, 2 * di, lw.conv_w, lw.conv_b, B, T, di, dc));
@@ -357,14 +367,15 @@ static int run_layers(mrs_backbone *bb, Scratch *s, int T) {
     }
     if (T == 1) {
         // (the out_proj epilogue of the own-GEMM chain has already added the last layer's output)
-        MRS_TRY(launch_add_rmsnorm(bb, s->residual, bb->skinny ? nullptr : s->out, bb->temporal, true, bb->norm_f, rows, dm));
+        MRS_TRY(launch_add_rmsnorm(bb, s->residual, bb->skinny ? nullptr : s->out, bb->temporal, true, bb->norm_f, rows, dm,
+                                   bb->dtype != MRS_F32 ? bb->temporal_t : nullptr));
     } else {
         // Only the last step of each sequence is kept (gather_last_timestep,
         // src/mamba_ssm/gpu/prefill.rs:1030-1046), so the final residual add + norm_f runs on those rows only.
         for (int b = 0; b < B; b++) {
             const size_t r = (size_t)b * T + (T - 1);
             MRS_TRY(launch_add_rmsnorm(bb, s->residual + r * dm, (const char *)s->out + r * dm * es, bb->temporal + (size_t)b * dm, true,
-                                       bb->norm_f, 1, dm));
+                                       bb->norm_f, 1, dm, bb->dtype != MRS_F32 ? (char *)bb->temporal_t + (size_t)b * dm * es : nullptr));
         }
     }
     return MRS_OK;
@@ -435,7 +446,11 @@ extern "C" int mrs_backbone_create(mrs_backbone **out, int gpu_ordinal, const mr
         MRS_CREATE_TRY(upload_f32(bb, &d.dt_b, src.dt_proj_b, di));
         MRS_CREATE_TRY(upload_f32(bb, &d.D, src.d_param, di));
         MRS_CREATE_TRY(upload_bulk(bb, &d.out_proj, src.out_proj_w, (size_t)di * dm, stage));
-        d.in_proj_t = d.x_proj_t = d.out_proj_t = nullptr;
+        d.in_proj_t = d.x_proj_t = d.out_proj_t = d.dt_w_t = nullptr;
+        if ((ds == 4 || ds == 8 || ds == 16 || ds == 32 || ds == 64 || ds == 128 || ds == 256) && dr % ds == 0 && xd % 4 == 0) {
+            MRS_CREATE_TRY(dev_alloc(bb, &d.dt_w_t, (size_t)dr * di * esize(bb->dtype)));
+            MRS_CREATE_TRY(launch_transpose(bb->stream, bb->dtype, d.dt_w_t, d.dt_w, dr, di));
+        }
         if (bb->skinny) {
             // transposed copies for the decode chain (one more copy of the bulk weights in HBM)
             const size_t es_ = esize(bb->dtype);
@@ -463,6 +478,7 @@ extern "C" int mrs_backbone_create(mrs_backbone **out, int gpu_ordinal, const mr
     MRS_CREATE_TRY(dev_alloc(bb, (void **)&bb->ssm_state, (size_t)L * batch * di * ds * 4));
     MRS_CREATE_TRY(dev_alloc(bb, (void **)&bb->d_input, (size_t)batch * input_dim * 4));
     MRS_CREATE_TRY(dev_alloc(bb, (void **)&bb->temporal, (size_t)batch * dm * 4));
+    MRS_CREATE_TRY(dev_alloc(bb, &bb->temporal_t, (size_t)batch * dm * esize(dtype)));
     MRS_CREATE_TRY(alloc_scratch(bb, &bb->step_s, batch, 1));
     MRS_CREATE_TRY(mrs_backbone_reset(bb));
     { hipError_t e = hipStreamSynchronize(bb->stream);
@@ -493,7 +509,10 @@ extern "C" int mrs_backbone_reset(mrs_backbone *bb) {
 }
 
 static int step_body(mrs_backbone *bb) {
-    MRS_TRY(project_input(bb, bb->step_s.residual, bb->d_input, bb->batch));
+    // identity projection on the own-GEMM chain: the first layer's prenorm kernel reads the input and writes the
+    // residual stream itself, so no copy is needed
+    bb->step_src = (bb->identity_proj && bb->skinny) ? bb->d_input : nullptr;
+    if (!bb->step_src) MRS_TRY(project_input(bb, bb->step_s.residual, bb->d_input, bb->batch));
     return run_layers(bb, &bb->step_s, 1);
 }
 
@@ -605,7 +624,6 @@ struct mrs_lm {
     int vocab, vocab_padded, dm, batch, dtype;
     void *embed;        // [vocab_padded, dm] storage dtype (tied lm_head)
     float *logits;      // [batch, vocab_padded] f32
-    void *hidden;       // [batch, dm] storage dtype copy of temporal for the head GEMM
     int *tokens;        // [batch] current token ids on device
     float *arg_v;       // [batch, kArgParts] partial maxima
     int *arg_i;
@@ -630,7 +648,6 @@ extern "C" int mrs_lm_create(mrs_lm **out, mrs_backbone *bb, const float *embed,
 #define MRS_LM_HIP(expr) do { hipError_t e_ = (expr); if (e_ != hipSuccess) { cleanup(); return fail(MRS_E_HIP, "%s: %s", #expr, hipGetErrorString(e_)); } } while (0)
     MRS_LM_HIP(hipMalloc(&lm->embed, ne * es)); lm->allocs.push_back(lm->embed);
     MRS_LM_HIP(hipMalloc((void **)&lm->logits, (size_t)lm->batch * lm->vocab_padded * 4)); lm->allocs.push_back(lm->logits);
-    MRS_LM_HIP(hipMalloc(&lm->hidden, (size_t)lm->batch * lm->dm * es)); lm->allocs.push_back(lm->hidden);
     MRS_LM_HIP(hipMalloc((void **)&lm->tokens, (size_t)lm->batch * sizeof(int))); lm->allocs.push_back(lm->tokens);
     MRS_LM_HIP(hipMalloc((void **)&lm->arg_v, (size_t)lm->batch * kArgParts * sizeof(float))); lm->allocs.push_back(lm->arg_v);
     MRS_LM_HIP(hipMalloc((void **)&lm->arg_i, (size_t)lm->batch * kArgParts * sizeof(int))); lm->allocs.push_back(lm->arg_i);
@@ -662,15 +679,9 @@ static int lm_logits(mrs_lm *lm) {
     mrs_backbone *bb = lm->bb;
     const int dm = lm->dm, V = lm->vocab_padded, B = lm->batch;
     const float one = 1.0f, zero = 0.0f;
-    const void *hid = bb->temporal;
-    rocblas_datatype ht = rocblas_datatype_f32_r;
-    if (lm->dtype != MRS_F32) {
-        const int64_t n = (int64_t)B * dm;
-        const dim3 grid((unsigned)((n + 255) / 256)), block(256);
-        if (lm->dtype == MRS_BF16) hipLaunchKernelGGL((cast_from_f32_kernel<bf16_t>), grid, block, 0, bb->stream, (bf16_t *)lm->hidden, bb->temporal, n);
-        else hipLaunchKernelGGL((cast_from_f32_kernel<f16_t>), grid, block, 0, bb->stream, (f16_t *)lm->hidden, bb->temporal, n);
-        hid = lm->hidden; ht = blas_type(lm->dtype);
-    }
+    // the final norm leaves its result in the storage type as well (temporal_t), which is the head's operand
+    const void *hid = lm->dtype != MRS_F32 ? bb->temporal_t : (const void *)bb->temporal;
+    const rocblas_datatype ht = lm->dtype != MRS_F32 ? blas_type(lm->dtype) : rocblas_datatype_f32_r;
     MRS_BLAS(rocblas_gemm_ex(bb->blas, rocblas_operation_transpose, rocblas_operation_none, V, B, dm, &one, lm->embed,
                              blas_type(lm->dtype), dm, hid, ht, dm, &zero, lm->logits, rocblas_datatype_f32_r, V, lm->logits,
                              rocblas_datatype_f32_r, V, rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0));

@@ -80,6 +80,37 @@ __global__ __launch_bounds__(kGemmWaves * 64) void skinny_gemm_kernel(
         if (!isfinite(rms) || rms < 1e-20f) rms = 1.0f;
         inv = 1.0f / rms;
     }
+    // Epilogue operands that do not depend on the product -- the conv window / taps / bias (mode 1), the
+    // residual element and next norm weight (mode 2) -- can be requested before the operands stream.
+    const int e_row = m0 + (tid >> 4), e_col = n0 + (tid & 15);
+    const bool e_valid = tid < 256 && e_row < M && e_col < N;
+    float win[kMaxConvTaps], cwv[kMaxConvTaps], cbias = 0.0f, res_old = 0.0f, nw = 0.0f;
+    auto prefetch_epilogue = [&]() {
+        if (EPI == 1 && e_valid && e_col < ep.di) {
+            const float *st = ep.conv_state + ((int64_t)e_row * ep.di + e_col) * ep.dc;
+            const float *cw = ep.conv_w + (int64_t)e_col * ep.dc;
+            if (ep.dc == 4) {   // the usual case: window and taps are one aligned 16-byte vector each
+                const float4 s4 = *reinterpret_cast<const float4 *>(st), c4 = *reinterpret_cast<const float4 *>(cw);
+                win[0] = s4.y; win[1] = s4.z; win[2] = s4.w;
+                cwv[0] = c4.x; cwv[1] = c4.y; cwv[2] = c4.z; cwv[3] = c4.w;
+            } else {
+#pragma unroll
+                for (int k = 0; k < kMaxConvTaps; k++) {
+                    win[k] = (k + 1 < ep.dc) ? st[k + 1] : 0.0f;
+                    cwv[k] = (k < ep.dc) ? cw[k] : 0.0f;
+                }
+            }
+            cbias = ep.conv_b[e_col];
+        }
+        if (EPI == 2 && e_valid) {
+            res_old = ep.residual[(int64_t)e_row * N + e_col];
+            if (ep.next_norm_w) nw = ep.next_norm_w[e_col];
+        }
+    };
+    // Early for the residual epilogue and for a single row tile; with several row tiles the conv windows are a
+    // megabyte-scale read that would queue ahead of the operands, so there they are fetched after the product.
+    const bool early = EPI == 2 || (EPI == 1 && gridDim.y == 1);
+    if (early) prefetch_epilogue();
     for (int base = w; base < nk; base += kGemmWaves * kStepsPerBatch) {
         uint4 bf[kStepsPerBatch], af[kStepsPerBatch];
 #pragma unroll
@@ -101,6 +132,7 @@ __global__ __launch_bounds__(kGemmWaves * 64) void skinny_gemm_kernel(
     __syncthreads();
     // element e of the 16x16 tile: row ml = e / 16, column nl = e % 16 lives in lane 16 (ml / 4) + nl, register ml % 4
     if (tid < 256) {
+        if (EPI != 0 && !early) prefetch_epilogue();
         const int ml = tid >> 4, nl = tid & 15;
         const int lane = (ml >> 2) * 16 + nl, i = ml & 3;
         float s = 0.0f;
@@ -115,11 +147,10 @@ __global__ __launch_bounds__(kGemmWaves * 64) void skinny_gemm_kernel(
             float sq = 0.0f;
             if (valid) {
                 const T orr = (T)s;
-                float *rp = ep.residual + (int64_t)row * N + col;
-                const float rn = *rp + Store<T>::ld(&orr);
-                *rp = rn;
+                const float rn = res_old + Store<T>::ld(&orr);
+                ep.residual[(int64_t)row * N + col] = rn;
                 sq = rn * rn;
-                if (ep.next_norm_w) Store<T>::st(reinterpret_cast<T *>(ep.prenorm) + (int64_t)row * N + col, rn * ep.next_norm_w[col]);
+                if (ep.next_norm_w) Store<T>::st(reinterpret_cast<T *>(ep.prenorm) + (int64_t)row * N + col, rn * nw);
             }
 #pragma unroll
             for (int m = 8; m >= 1; m >>= 1) sq += __shfl_xor(sq, m, kWave);
@@ -130,15 +161,19 @@ __global__ __launch_bounds__(kGemmWaves * 64) void skinny_gemm_kernel(
             const T xr = (T)s;
             const float xnew = Store<T>::ld(&xr);
             float *st = ep.conv_state + ((int64_t)row * ep.di + col) * ep.dc;
-            const float *cw = ep.conv_w + (int64_t)col * ep.dc;
-            float o = ep.conv_b[col];
-            float win[kMaxConvTaps];
+            float o = cbias;
+            if (ep.dc == 4) {
+                o = fmaf(win[0], cwv[0], o); o = fmaf(win[1], cwv[1], o); o = fmaf(win[2], cwv[2], o); o = fmaf(xnew, cwv[3], o);
+                *reinterpret_cast<float4 *>(st) = make_float4(win[0], win[1], win[2], xnew);
+            } else {
 #pragma unroll
-            for (int k = 0; k < kMaxConvTaps; k++)
-                if (k < ep.dc) win[k] = (k + 1 < ep.dc) ? st[k + 1] : xnew;
-#pragma unroll
-            for (int k = 0; k < kMaxConvTaps; k++)
-                if (k < ep.dc) { o = fmaf(win[k], cw[k], o); st[k] = win[k]; }
+                for (int k = 0; k < kMaxConvTaps; k++)
+                    if (k < ep.dc) {
+                        const float wk = (k + 1 < ep.dc) ? win[k] : xnew;
+                        o = fmaf(wk, cwv[k], o);
+                        st[k] = wk;
+                    }
+            }
             Store<T>::st(reinterpret_cast<T *>(ep.u) + (int64_t)row * ep.di + col, silu(o));
         } else {
             store_out<TO>(C + (int64_t)row * ldc + col, s);
@@ -147,16 +182,19 @@ __global__ __launch_bounds__(kGemmWaves * 64) void skinny_gemm_kernel(
 }
 
 // First layer's share of the folded norm: partials[row][0] = sum_k x[row][k]^2 (other slots zero) and
-// prenorm[row][k] = round_T(x[row][k] * w[k]), for a residual stream no out_proj epilogue has produced yet.
+// prenorm[row][k] = round_T(x[row][k] * w[k]), for a residual stream no out_proj epilogue has produced yet;
+// copy_to (may be null) also receives x, so the step's input buffer can feed the residual stream directly.
 template <typename T>
 __global__ __launch_bounds__(256) void prenorm_rows_kernel(float *__restrict__ partials, int n_partials, T *__restrict__ prenorm,
-                                                           const float *__restrict__ x, const float *__restrict__ w, int K) {
+                                                           const float *__restrict__ x, float *__restrict__ copy_to,
+                                                           const float *__restrict__ w, int K) {
     __shared__ float part[4];
     const int64_t row = blockIdx.x;
     float ss = 0.0f;
     for (int i = threadIdx.x; i < K; i += 256) {
         const float v = x[row * K + i];
         ss = fmaf(v, v, ss);
+        if (copy_to) copy_to[row * K + i] = v;   // the residual stream, when x is the step's input buffer
         Store<T>::st(prenorm + row * K + i, v * w[i]);
     }
 #pragma unroll
@@ -219,10 +257,10 @@ int launch_skinny_gemm(hipStream_t st, int dtype, void *C, int out_f32, int64_t 
     return launch_skinny_t<f16_t, f16_t>(st, (f16_t *)C, ldc, (const f16_t *)A, lda, (const f16_t *)Wt, M, N, K, ep);
 }
 
-int launch_prenorm_rows(hipStream_t st, int dtype, float *partials, int n_partials, void *prenorm, const float *x, const float *w,
-                        int M, int K) {
-    if (dtype == MRS_BF16) hipLaunchKernelGGL((prenorm_rows_kernel<bf16_t>), dim3((unsigned)M), dim3(256), 0, st, partials, n_partials, (bf16_t *)prenorm, x, w, K);
-    else if (dtype == MRS_F16) hipLaunchKernelGGL((prenorm_rows_kernel<f16_t>), dim3((unsigned)M), dim3(256), 0, st, partials, n_partials, (f16_t *)prenorm, x, w, K);
+int launch_prenorm_rows(hipStream_t st, int dtype, float *partials, int n_partials, void *prenorm, const float *x, float *copy_to,
+                        const float *w, int M, int K) {
+    if (dtype == MRS_BF16) hipLaunchKernelGGL((prenorm_rows_kernel<bf16_t>), dim3((unsigned)M), dim3(256), 0, st, partials, n_partials, (bf16_t *)prenorm, x, copy_to, w, K);
+    else if (dtype == MRS_F16) hipLaunchKernelGGL((prenorm_rows_kernel<f16_t>), dim3((unsigned)M), dim3(256), 0, st, partials, n_partials, (f16_t *)prenorm, x, copy_to, w, K);
     else return fail(MRS_E_DTYPE, "prenorm rows: 16-bit storage only");
     return check_launch("prenorm_rows_kernel");
 }

@@ -19,12 +19,31 @@ __device__ __forceinline__ float softplus20(float v) { return v > 20.0f ? v : lo
 // gate_mode: 0 none, 1 y *= gate, 2 y *= silu(gate); gate rows have gate_stride elements.
 // dt_bias != nullptr: delta holds the raw dt_proj output and softplus(delta + dt_bias[d]) is applied here
 // (dt_proj bias add + softplus_forward of the decode chain, src/mamba_ssm/gpu/inference.rs:1129-1158).
+// Four consecutive elements as f32: one 8-byte (16-bit storage) or 16-byte (f32) load when the
+// address is aligned for it (vec), four scalar loads otherwise.
+template <typename T> __device__ __forceinline__ void ld4(const T *p, float (&o)[4], bool vec) {
+    if (vec) {
+        struct alignas(4 * sizeof(T)) V { T v[4]; };
+        const V t = *reinterpret_cast<const V *>(p);
+#pragma unroll
+        for (int i = 0; i < 4; i++) o[i] = Store<T>::ld(&t.v[i]);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; i++) o[i] = Store<T>::ld(p + i);
+    }
+}
+
+// flags: bit 0 = B/C rows may be read as aligned 4-element vectors; bit 1 = dt_w is transposed
+// ([d_inner][dt_rank]) and dt_rank / LG is a multiple of 4, so lane g takes the contiguous terms
+// [g dt_rank/LG, (g+1) dt_rank/LG) of both operands as 4-element vectors.
+constexpr int kStepVecBC = 1, kStepDtT = 2;
+
 template <typename T, int LG>
 __global__ __launch_bounds__(256) void ssm_step_kernel(
     float *__restrict__ h, T *__restrict__ y, const T *__restrict__ delta, const T *__restrict__ u,
     const T *__restrict__ Bbase, const T *__restrict__ Cbase, int64_t bc_stride,
     const T *__restrict__ gate, int64_t gate_stride, int gate_mode, const float *__restrict__ dt_bias,
-    const T *__restrict__ dt_in, const T *__restrict__ dt_w, int dr,
+    const T *__restrict__ dt_in, const T *__restrict__ dt_w, int dr, int flags,
     const float *__restrict__ a_neg, const float *__restrict__ Dp, int64_t total, int di, int ds) {
     // total = batch*d_inner rows; ds == 4*LG here.
     const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -41,8 +60,27 @@ __global__ __launch_bounds__(256) void ssm_step_kernel(
         // dt_proj folded in: delta_raw[b,d] = sum_r dt_in[b,r] * dt_w[r,d], the dt_rank terms split over the
         // LG lanes of the row (dt_proj GEMM of the decode chain, src/mamba_ssm/gpu/inference.rs:1129-1146)
         const T *xr = dt_in + (int64_t)b * bc_stride;
-        const T *wc = dt_w + d;
         float part = 0.0f;
+        if (flags & kStepDtT) {
+            const int kpl = dr / LG;
+            const T *xp = xr + g * kpl, *wp = dt_w + (int64_t)d * dr + g * kpl;
+            for (int c0 = 0; c0 < kpl; c0 += 16) {
+                float xv[4][4], wv[4][4];
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const int kk = c0 + 4 * j;
+                    const int kc = kk < kpl ? kk : 0;   // in-range address for the masked-off chunks
+                    ld4<T>(xp + kc, xv[j], true);
+                    ld4<T>(wp + kc, wv[j], true);
+                    if (kk >= kpl) { xv[j][0] = 0.f; xv[j][1] = 0.f; xv[j][2] = 0.f; xv[j][3] = 0.f; }
+                }
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+#pragma unroll
+                    for (int i = 0; i < 4; i++) part = fmaf(xv[j][i], wv[j][i], part);
+            }
+        } else {
+        const T *wc = dt_w + d;
         // batches of 12 terms per lane with every load of a batch issued before the first multiply-add:
         // the loop is a latency chain otherwise (dt_rank 48 over 4 lanes = one batch)
         constexpr int kBatch = 12;
@@ -59,6 +97,7 @@ __global__ __launch_bounds__(256) void ssm_step_kernel(
 #pragma unroll
             for (int j = 0; j < kBatch; j++) part = fmaf(xv[j], wv[j], part);
         }
+        }
 #pragma unroll
         for (int m = 1; m < LG; m <<= 1) part += __shfl_xor(part, m, kWave);
         dl = part;
@@ -71,14 +110,17 @@ __global__ __launch_bounds__(256) void ssm_step_kernel(
     const T *Br = Bbase + (int64_t)b * bc_stride + 4 * g;
     const T *Cr = Cbase + (int64_t)b * bc_stride + 4 * g;
     const float x = dl * kLog2e;
-    hv.x = fmaf(fast_exp2(x * av.x), hv.x, du * Store<T>::ld(Br + 0));
-    hv.y = fmaf(fast_exp2(x * av.y), hv.y, du * Store<T>::ld(Br + 1));
-    hv.z = fmaf(fast_exp2(x * av.z), hv.z, du * Store<T>::ld(Br + 2));
-    hv.w = fmaf(fast_exp2(x * av.w), hv.w, du * Store<T>::ld(Br + 3));
-    float acc = hv.x * Store<T>::ld(Cr + 0);
-    acc = fmaf(hv.y, Store<T>::ld(Cr + 1), acc);
-    acc = fmaf(hv.z, Store<T>::ld(Cr + 2), acc);
-    acc = fmaf(hv.w, Store<T>::ld(Cr + 3), acc);
+    float Bv[4], Cv[4];
+    ld4<T>(Br, Bv, (flags & kStepVecBC) != 0);
+    ld4<T>(Cr, Cv, (flags & kStepVecBC) != 0);
+    hv.x = fmaf(fast_exp2(x * av.x), hv.x, du * Bv[0]);
+    hv.y = fmaf(fast_exp2(x * av.y), hv.y, du * Bv[1]);
+    hv.z = fmaf(fast_exp2(x * av.z), hv.z, du * Bv[2]);
+    hv.w = fmaf(fast_exp2(x * av.w), hv.w, du * Bv[3]);
+    float acc = hv.x * Cv[0];
+    acc = fmaf(hv.y, Cv[1], acc);
+    acc = fmaf(hv.z, Cv[2], acc);
+    acc = fmaf(hv.w, Cv[3], acc);
 #pragma unroll
     for (int m = 1; m < LG; m <<= 1) acc += __shfl_xor(acc, m, kWave);
     if (live) {
@@ -98,7 +140,7 @@ __global__ __launch_bounds__(256) void ssm_step_generic_kernel(
     float *__restrict__ h, T *__restrict__ y, const T *__restrict__ delta, const T *__restrict__ u,
     const T *__restrict__ Bbase, const T *__restrict__ Cbase, int64_t bc_stride,
     const T *__restrict__ gate, int64_t gate_stride, int gate_mode, const float *__restrict__ dt_bias,
-    const T *__restrict__ dt_in, const T *__restrict__ dt_w, int dr,
+    const T *__restrict__ dt_in, const T *__restrict__ dt_w, int dr, int /*flags*/,
     const float *__restrict__ a_neg, const float *__restrict__ Dp, int64_t total, int di, int ds) {
     const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (r >= total) return;
@@ -134,14 +176,22 @@ template <typename T>
 static int launch_step(hipStream_t st, float *h, void *y, const void *delta, const void *u,
                        const void *Bb, const void *Cb, int64_t bc_stride, const void *gate,
                        int64_t gate_stride, int gate_mode, const float *dt_bias, const void *dt_in,
-                       const void *dt_w, int dr, const float *a_neg, const float *D, int batch, int di, int ds) {
+                       const void *dt_w, int dr, int dt_transposed, const float *a_neg, const float *D, int batch, int di, int ds) {
     const int64_t total = (int64_t)batch * di;
     if (!gate) gate_mode = 0;
+    int flags = 0;
 #define MRS_ARGS h, (T *)y, (const T *)delta, (const T *)u, (const T *)Bb, (const T *)Cb, bc_stride, \
-                 (const T *)gate, gate_stride, gate_mode, dt_bias, (const T *)dt_in, (const T *)dt_w, dr, a_neg, D, total, di, ds
+                 (const T *)gate, gate_stride, gate_mode, dt_bias, (const T *)dt_in, (const T *)dt_w, dr, flags, a_neg, D, total, di, ds
     const bool vec_ok = aligned(h, 16) && aligned(a_neg, 16);
     int lg = 0;
     if (vec_ok && (ds == 4 || ds == 8 || ds == 16 || ds == 32 || ds == 64 || ds == 128 || ds == 256)) lg = ds / 4;
+    const size_t v4 = 4 * sizeof(T);
+    if (bc_stride % 4 == 0 && aligned(Bb, v4) && aligned(Cb, v4)) flags |= kStepVecBC;
+    if (dt_w && dt_transposed) {
+        if (!(lg && dr % (4 * lg) == 0 && bc_stride % 4 == 0 && aligned(dt_in, v4) && aligned(dt_w, v4)))
+            return fail(MRS_E_SHAPE, "ssm step: transposed dt_w needs d_state a power of two in 4..256, dt_rank %% d_state == 0 and 4-element aligned rows");
+        flags |= kStepDtT;
+    }
     if (lg) {
         const int64_t threads = total * lg;
         const int64_t blocks = (threads + 255) / 256;
@@ -160,12 +210,12 @@ static int launch_step(hipStream_t st, float *h, void *y, const void *delta, con
 }
 
 int launch_ssm_step_fused(hipStream_t st, int dtype, float *h, void *y, const void *delta, const float *dt_bias,
-                          const void *dt_in, const void *dt_w, int dr,
+                          const void *dt_in, const void *dt_w, int dr, int dt_transposed,
                           const void *u, const void *Bb, const void *Cb, int64_t bc_stride, const void *gate,
                           int64_t gate_stride, int gate_mode, const float *a_neg, const float *D, int batch,
                           int di, int ds) {
     MRS_DISPATCH_DTYPE(dtype, T_, return launch_step<T_>(st, h, y, delta, u, Bb, Cb, bc_stride, gate, gate_stride, gate_mode,
-                                                         dt_bias, dt_in, dt_w, dr, a_neg, D, batch, di, ds));
+                                                         dt_bias, dt_in, dt_w, dr, dt_transposed, a_neg, D, batch, di, ds));
     return MRS_OK;
 }
 
@@ -191,7 +241,7 @@ extern "C" int mrs_ssm_step(void *stream, int dtype, float *h, void *y, const vo
     int rc = step_check("mrs_ssm_step", dtype, h, y, delta, u, B, C, a_neg, D, batch, d_inner, d_state);
     if (rc) return rc;
     hipStream_t st = as_stream(stream);
-    MRS_DISPATCH_DTYPE(dtype, T_, return launch_step<T_>(st, h, y, delta, u, B, C, d_state, nullptr, 0, 0, nullptr, nullptr, nullptr, 0, a_neg, D, batch, d_inner, d_state));
+    MRS_DISPATCH_DTYPE(dtype, T_, return launch_step<T_>(st, h, y, delta, u, B, C, d_state, nullptr, 0, 0, nullptr, nullptr, nullptr, 0, 0, a_neg, D, batch, d_inner, d_state));
     return MRS_OK;
 }
 
@@ -208,6 +258,6 @@ extern "C" int mrs_ssm_step_gather_gate(void *stream, int dtype, float *h, void 
     const char *xb = static_cast<const char *>(xdbl);
     hipStream_t st = as_stream(stream);
     MRS_DISPATCH_DTYPE(dtype, T_, return launch_step<T_>(st, h, y, delta, u, xb + es * b_offset, xb + es * c_offset,
-                                                         xdbl_stride, gate_silu, d_inner, 1, nullptr, nullptr, nullptr, 0, a_neg, D, batch, d_inner, d_state));
+                                                         xdbl_stride, gate_silu, d_inner, 1, nullptr, nullptr, nullptr, 0, 0, a_neg, D, batch, d_inner, d_state));
     return MRS_OK;
 }
