@@ -45,6 +45,17 @@ __device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcp
 // denominator overflows to +inf and the product is -0, the correct limit.
 __device__ __forceinline__ float silu(float x) { return x * fast_rcp(1.0f + fast_exp2(-x * kLog2e)); }
 
+// softplus with the reference's pass-through above 20 (kernels/activations.cu:39): log(1 + e^v) on the
+// transcendental unit.  Below e = 0.03 the sum 1 + e would drop e's low bits, so log1p's series takes over
+// (next term e^6/6 < 1.3e-10); above it the rounding of 1 + e is at most 2e-6 of the result.
+__device__ __forceinline__ float softplus20(float v) {
+    if (v > 20.0f) return v;
+    const float e = fast_exp2(v * kLog2e);
+    const float series = e * fmaf(e, fmaf(e, fmaf(e, fmaf(e, 0.2f, -0.25f), 0.33333334f), -0.5f), 1.0f);
+    const float vialog = __builtin_amdgcn_logf(1.0f + e) * 0.6931471805599453f;
+    return e < 0.03f ? series : vialog;
+}
+
 // ---- host-side error plumbing ---------------------------------------------
 void set_error(const char *fmt, ...);
 int fail(int code, const char *fmt, ...);

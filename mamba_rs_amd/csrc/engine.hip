@@ -80,13 +80,92 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(float *__restrict__ re
     }
 }
 
-// delta = softplus(raw + bias[d]) in place (dt_proj bias + softplus_forward, kernels/activations.cu:32-52)
-template <typename T>
+// delta = softplus(raw + bias[d]) in place (dt_proj bias + softplus_forward, kernels/activations.cu:32-52).
+// VEC elements per thread as one 16-byte access (VEC = 16 / sizeof(T), d_inner % VEC == 0), or one by one.
+template <typename T, int VEC>
 __global__ __launch_bounds__(256) void bias_softplus_kernel(T *__restrict__ x, const float *__restrict__ bias, int64_t n, int di) {
-    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * VEC;
     if (i >= n) return;
-    const float v = Store<T>::ld(x + i) + bias[i % di];
-    Store<T>::st(x + i, v > 20.0f ? v : log1pf(fast_exp2(v * kLog2e)));
+    const int d0 = (int)(i % di);
+    struct alignas(VEC * sizeof(T)) V { T v[VEC]; };
+    V t = *reinterpret_cast<const V *>(x + i);
+    float bv[VEC];
+    if (VEC % 4 == 0) {   // d0 is a multiple of VEC: the bias values are aligned 16-byte vectors too
+#pragma unroll
+        for (int j = 0; j < VEC; j += 4) {
+            const float4 b4 = *reinterpret_cast<const float4 *>(bias + d0 + j);
+            bv[j] = b4.x; bv[j + 1] = b4.y; bv[j + 2] = b4.z; bv[j + 3] = b4.w;
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < VEC; j++) bv[j] = bias[d0 + j];
+    }
+#pragma unroll
+    for (int j = 0; j < VEC; j++) Store<T>::st(&t.v[j], softplus20(Store<T>::ld(&t.v[j]) + bv[j]));
+    *reinterpret_cast<V *>(x + i) = t;
+}
+
+// Prefill-sized rows: one wave per row, 4 elements per lane and trip (16-byte residual accesses), the row
+// kept in registers between the sum of squares and the scaling.  Same arithmetic as add_rmsnorm_kernel.
+template <typename T, typename TO>
+__global__ __launch_bounds__(256) void add_rmsnorm_rows_kernel(float *__restrict__ residual, const T *__restrict__ add,
+                                                               TO *__restrict__ out, const float *__restrict__ w,
+                                                               float eps, int64_t rows, int dm) {
+    constexpr int kMaxTrips = 16;  // d_model <= 4096 stays in registers; longer rows re-read
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int lane = threadIdx.x & 63;
+    const int nv = dm >> 2;
+    float4 *r4 = reinterpret_cast<float4 *>(residual + row * dm);
+    struct alignas(4 * sizeof(T)) V4 { T v[4]; };
+    struct alignas(4 * sizeof(TO)) O4 { TO v[4]; };
+    const V4 *a4 = reinterpret_cast<const V4 *>(add ? add + row * dm : nullptr);
+    float4 v[kMaxTrips];
+    float ss = 0.0f;
+    int cnt = 0;
+    for (int c0 = lane; c0 < nv; c0 += 4 * 64) {
+        // four trips at a time, every load issued before the first use
+        float4 x[4];
+        V4 a[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int c = c0 + 64 * j;
+            if (c < nv) {
+                x[j] = r4[c];
+                if (add) a[j] = a4[c];
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int c = c0 + 64 * j;
+            if (c < nv) {
+                if (add) {
+                    x[j].x += Store<T>::ld(&a[j].v[0]); x[j].y += Store<T>::ld(&a[j].v[1]);
+                    x[j].z += Store<T>::ld(&a[j].v[2]); x[j].w += Store<T>::ld(&a[j].v[3]);
+                    r4[c] = x[j];
+                }
+                if (cnt < kMaxTrips) v[cnt] = x[j];
+                cnt++;
+                ss = fmaf(x[j].x, x[j].x, ss); ss = fmaf(x[j].y, x[j].y, ss); ss = fmaf(x[j].z, x[j].z, ss); ss = fmaf(x[j].w, x[j].w, ss);
+            }
+        }
+    }
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) ss += __shfl_xor(ss, m, kWave);
+    float rms = sqrtf(ss / (float)dm + eps);
+    if (!isfinite(rms) || rms < 1e-20f) rms = 1.0f;
+    const float inv = 1.0f / rms;
+    O4 *o4 = reinterpret_cast<O4 *>(out + row * dm);
+    const float4 *w4 = reinterpret_cast<const float4 *>(w);
+    cnt = 0;
+    for (int c = lane; c < nv; c += 64, cnt++) {
+        const float4 x = cnt < kMaxTrips ? v[cnt] : r4[c];
+        const float4 ww = w4[c];
+        O4 o;
+        Store<TO>::st(&o.v[0], x.x * inv * ww.x); Store<TO>::st(&o.v[1], x.y * inv * ww.y);
+        Store<TO>::st(&o.v[2], x.z * inv * ww.z); Store<TO>::st(&o.v[3], x.w * inv * ww.w);
+        o4[c] = o;
+    }
 }
 
 template <typename T>
@@ -264,6 +343,11 @@ template <typename T>
 static void launch_add_rmsnorm_t(mrs_backbone *bb, float *residual, const void *add, void *out, bool out_f32,
                                  const float *w, int64_t rows, int64_t out_stride, void *out2) {
     const dim3 grid((unsigned)rows), block(256);
+    if (rows >= 256 && bb->cfg.d_model % 4 == 0 && out_stride == bb->cfg.d_model && !out2 && !out_f32) {
+        hipLaunchKernelGGL((add_rmsnorm_rows_kernel<T, T>), dim3((unsigned)((rows + 3) / 4)), block, 0, bb->stream, residual, (const T *)add,
+                           (T *)out, w, bb->cfg.rms_norm_eps, rows, bb->cfg.d_model);
+        return;
+    }
     if (out_f32)
         hipLaunchKernelGGL((add_rmsnorm_kernel<T, float>), grid, block, 0, bb->stream, residual, (const T *)add, (float *)out, (T *)out2, w,
                            bb->cfg.rms_norm_eps, rows, bb->cfg.d_model, out_stride);
@@ -353,8 +437,13 @@ static int run_layers(mrs_backbone *bb, Scratch *s, int T) {
             MRS_TRY(gemm_rm(bb, dt, s->xdbl, xd, s->u, di, lw.x_proj, (int)rows, xd, di));
             MRS_TRY(gemm_rm(bb, dt, s->delta, di, s->xdbl, xd, lw.dt_w, (int)rows, di, dr));
             const int64_t n = rows * di;
-            const dim3 grid((unsigned)((n + 255) / 256)), block(256);
-            MRS_DISPATCH_DTYPE(dt, T_, hipLaunchKernelGGL((bias_softplus_kernel<T_>), grid, block, 0, bb->stream, (T_ *)s->delta, lw.dt_b, n, di));
+            MRS_DISPATCH_DTYPE(dt, T_, {
+                constexpr int VEC = 16 / (int)sizeof(T_);
+                if (di % VEC == 0)
+                    hipLaunchKernelGGL((bias_softplus_kernel<T_, VEC>), dim3((unsigned)((n / VEC + 255) / 256)), dim3(256), 0, bb->stream, (T_ *)s->delta, lw.dt_b, n, di);
+                else
+                    hipLaunchKernelGGL((bias_softplus_kernel<T_, 1>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, bb->stream, (T_ *)s->delta, lw.dt_b, n, di);
+            });
             MRS_TRY(check_launch("bias_softplus_kernel"));
             // ScanMode::use_parallel picks the route (src/mamba_ssm/gpu/prefill.rs:910-956)
             unsigned flags = MRS_GATE_SILU | (lw.s4d ? MRS_A_S4D_REAL : 0);

@@ -13,8 +13,6 @@ namespace mrs {
 
 // B and C of batch row b are read at xdbl + b*stride + {b_off, c_off}; the plain
 // step passes stride = ds and separate base pointers.
-// softplus with the reference's pass-through above 20 (kernels/activations.cu:39)
-__device__ __forceinline__ float softplus20(float v) { return v > 20.0f ? v : log1pf(fast_exp2(v * kLog2e)); }
 
 // gate_mode: 0 none, 1 y *= gate, 2 y *= silu(gate); gate rows have gate_stride elements.
 // dt_bias != nullptr: delta holds the raw dt_proj output and softplus(delta + dt_bias[d]) is applied here
