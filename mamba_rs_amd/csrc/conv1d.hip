@@ -37,6 +37,8 @@ __global__ __launch_bounds__(256) void conv1d_step_kernel(
     Store<T>::st(out + r, SILU ? silu(s) : s);
 }
 
+constexpr int kConvGroup = 8;  // timesteps whose rows a lane requests together
+
 template <typename T> struct alignas(16) Vec16 {
     static constexpr int N = 16 / sizeof(T);
     T v[N];
@@ -83,45 +85,70 @@ __global__ __launch_bounds__(256) void conv1d_seq_silu_kernel(
             for (int c = 0; c < VEC; c++) win[k][c] = state[((int64_t)b * di + d0 + c) * DC + s];
         }
     }
-    for (int t = t0; t < t1; t++) {
-        const Vec16<T> xv = *reinterpret_cast<const Vec16<T> *>(x + ((int64_t)b * Tlen + t) * x_stride + d0);
-        Vec16<T> ov;
+    // New window state = the last DC inputs of (old window ++ x[0..T)).  The chunk-0 lane of a channel vector is
+    // the only reader of that channel's old state (chunks are longer than the window), so it is the one that
+    // writes the new one, after its own read above and from x alone (old slots only when T < DC).
+    if (chunk == 0) {
+        float nw[VEC][DC];
 #pragma unroll
-        for (int c = 0; c < VEC; c++) {
+        for (int k = 0; k < DC; k++) {
+            const int tt = Tlen - DC + k;  // time of slot k after the call
+            if (tt >= 0) {
+                const Vec16<T> xv = *reinterpret_cast<const Vec16<T> *>(x + ((int64_t)b * Tlen + tt) * x_stride + d0);
 #pragma unroll
-            for (int k = 0; k + 1 < DC; k++) win[k][c] = win[k + 1][c];
-            win[DC - 1][c] = Store<T>::ld(&xv.v[c]);
-            float s = bs[c];
+                for (int c = 0; c < VEC; c++) nw[c][k] = Store<T>::ld(&xv.v[c]);
+            } else {
+                // old slot tt + DC = Tlen + k, in 1..DC-1: it is win[Tlen + k] of the window loaded above
 #pragma unroll
-            for (int k = 0; k < DC; k++) s = fmaf(win[k][c], w[k][c], s);
-            Store<T>::st(&ov.v[c], silu(s));
+                for (int c = 0; c < VEC; c++) {
+                    float v = 0.0f;
+#pragma unroll
+                    for (int kk = 1; kk < DC; kk++)
+                        if (kk == Tlen + k) v = win[kk][c];
+                    nw[c][k] = v;
+                }
+            }
         }
-        *reinterpret_cast<Vec16<T> *>(u_out + ((int64_t)b * Tlen + t) * di + d0) = ov;
-    }
-}
-
-// New window state = last DC inputs of (old window ++ x[0..T)).  Launched after the
-// sequence kernel on the same stream, so every chunk has already read the old state.
-template <typename T>
-__global__ __launch_bounds__(256) void conv1d_state_update_kernel(
-    float *__restrict__ state, const T *__restrict__ x, int64_t x_stride, int64_t total, int Tlen,
-    int di, int dc) {
-    const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (r >= total) return;
-    const int b = (int)(r / di);
-    const int d = (int)(r - (int64_t)b * di);
-    float *st = state + r * dc;
-    float nw[kMaxConv];
+        float *sp = state + ((int64_t)b * di + d0) * DC;
 #pragma unroll
-    for (int k = 0; k < kMaxConv; k++) {
-        if (k < dc) {
-            const int tt = Tlen - dc + k;  // time of slot k after the call
-            nw[k] = (tt >= 0) ? Store<T>::ld(x + ((int64_t)b * Tlen + tt) * x_stride + d) : st[tt + dc];
+        for (int c = 0; c < VEC; c++)
+#pragma unroll
+            for (int k = 0; k < DC; k++) sp[c * DC + k] = nw[c][k];
+    }
+    // Groups of kConvGroup steps: the rows of the next group are requested before the current one is
+    // computed, so a lane always has kConvGroup 16-byte loads in flight.
+    Vec16<T> cur[kConvGroup], nxt[kConvGroup];
+    auto load_group = [&](Vec16<T> (&g)[kConvGroup], int tg) {
+#pragma unroll
+        for (int j = 0; j < kConvGroup; j++) {
+            const int t = min(tg + j, t1 - 1);
+            g[j] = *reinterpret_cast<const Vec16<T> *>(x + ((int64_t)b * Tlen + t) * x_stride + d0);
         }
-    }
+    };
+    if (t0 < t1) load_group(cur, t0);
+    for (int tg = t0; tg < t1; tg += kConvGroup) {
+        if (tg + kConvGroup < t1) load_group(nxt, tg + kConvGroup);
 #pragma unroll
-    for (int k = 0; k < kMaxConv; k++)
-        if (k < dc) st[k] = nw[k];
+        for (int j = 0; j < kConvGroup; j++) {
+            const int t = tg + j;
+            if (t < t1) {
+                Vec16<T> ov;
+#pragma unroll
+                for (int c = 0; c < VEC; c++) {
+#pragma unroll
+                    for (int k = 0; k + 1 < DC; k++) win[k][c] = win[k + 1][c];
+                    win[DC - 1][c] = Store<T>::ld(&cur[j].v[c]);
+                    float s = bs[c];
+#pragma unroll
+                    for (int k = 0; k < DC; k++) s = fmaf(win[k][c], w[k][c], s);
+                    Store<T>::st(&ov.v[c], silu(s));
+                }
+                *reinterpret_cast<Vec16<T> *>(u_out + ((int64_t)b * Tlen + t) * di + d0) = ov;
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < kConvGroup; j++) cur[j] = nxt[j];
+    }
 }
 
 // Fallback for shapes the vector kernel does not take (d_inner % VEC != 0 or
@@ -175,7 +202,7 @@ static int launch_conv_seq(hipStream_t st, void *u_out, float *state, const void
     const int nvec = di / VEC;
     // timesteps per lane: enough lanes to fill the chip, long enough to amortise the window reload
     int tpl = 32;
-    while (tpl > 8 && (int64_t)batch * nvec * ((Tlen + tpl - 1) / tpl) < 4 * 256 * 256) tpl >>= 1;
+    while (tpl > 16 && (int64_t)batch * nvec * ((Tlen + tpl - 1) / tpl) < 2 * 256 * 256) tpl >>= 1;
     const int nchunk = (Tlen + tpl - 1) / tpl;
     const int64_t threads = (int64_t)batch * nchunk * nvec;
     const int64_t blocks = (threads + 255) / 256;
@@ -188,12 +215,7 @@ static int launch_conv_seq(hipStream_t st, void *u_out, float *state, const void
         break
     switch (dc) { MRS_DC(2); MRS_DC(3); MRS_DC(4); }
 #undef MRS_DC
-    int rc = check_launch("conv1d_seq_silu_kernel");
-    if (rc) return rc;
-    const int64_t ublocks = (total + 255) / 256;
-    hipLaunchKernelGGL((conv1d_state_update_kernel<T>), dim3((unsigned)ublocks), dim3(256), 0, st, state,
-                       (const T *)x, x_stride, total, Tlen, di, dc);
-    return check_launch("conv1d_state_update_kernel");
+    return check_launch("conv1d_seq_silu_kernel");
 }
 
 static int conv_check(const char *fn, int dtype, const void *out, const void *state, const void *x,
