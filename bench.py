@@ -160,6 +160,51 @@ def lm_leg(name, cfg_kw, vocab, prefill_bt, decode_b, decode_steps, seed=42):
     return out
 
 
+def m1_kernels_leg():
+    """The other Mamba-1 kernels of the path at the 130m shape (bf16 storage), each against its HBM roofline:
+    causal conv1d + SiLU over batch 8 x T 2048 reading the x half of in_proj's rows in place, and the decode
+    scan step (B/C gathered from the x_proj row, SiLU gate fused) at batch 64."""
+    import torch
+    from mamba_rs_amd import ops
+    dev, bf = "cuda:0", torch.bfloat16
+    B, T, di, ds, dc, dr = 8, 2048, 1536, 16, 4, 48
+    g = torch.Generator(device=dev); g.manual_seed(5)
+
+    def timeit(f, n):
+        for _ in range(3):
+            f()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(n):
+            f()
+        b.record(); torch.cuda.synchronize()
+        return a.elapsed_time(b) / n * 1e3
+
+    proj = torch.randn(B, T, 2 * di, device=dev, generator=g).to(bf)
+    w = torch.randn(di, dc, device=dev, generator=g); bias = torch.randn(di, device=dev, generator=g)
+    st = torch.zeros(B, di, dc, device=dev); u = torch.empty(B, T, di, device=dev, dtype=bf)
+    us_conv = timeit(lambda: ops.conv1d_seq_silu(u, st, proj[:, :, :di], w, bias), 30)
+    conv_bytes = 2 * B * T * di * 2 + 2 * 4 * B * di * dc + 4 * di * (dc + 1)
+    Bd = 64
+    h = torch.zeros(Bd, di, ds, device=dev); y = torch.empty(Bd, di, device=dev, dtype=bf)
+    delta = torch.rand(Bd, di, device=dev, generator=g).mul(0.1).to(bf); uu = torch.randn(Bd, di, device=dev, generator=g).to(bf)
+    xdbl = torch.randn(Bd, dr + 2 * ds, device=dev, generator=g).to(bf); gate = torch.randn(Bd, di, device=dev, generator=g).to(bf)
+    a_neg = -torch.arange(1, ds + 1, device=dev, dtype=torch.float32).repeat(di, 1).contiguous(); D = torch.ones(di, device=dev)
+    ops.ssm_step_gather_gate(h, y, delta, uu, xdbl, gate, a_neg, D, dr, dr + ds)
+    torch.cuda.synchronize()
+    gr = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(gr):
+        for _ in range(24):
+            ops.ssm_step_gather_gate(h, y, delta, uu, xdbl, gate, a_neg, D, dr, dr + ds)
+    us_step = timeit(gr.replay, 30) / 24
+    step_bytes = 2 * 4 * Bd * di * ds + 4 * Bd * di * 2 + 4 * di * ds
+    return {"conv1d_seq_silu": {"batch": B, "seq_len": T, "us": us_conv, "algorithmic_bytes": conv_bytes,
+                                "GBps": conv_bytes / us_conv / 1e3, "hbm_frac": conv_bytes / us_conv / 1e3 / HBM_PEAK_GBPS},
+            "ssm_step_gather_gate_b64": {"us_per_call_in_graph": us_step, "algorithmic_bytes": step_bytes,
+                                         "GBps": step_bytes / us_step / 1e3, "hbm_frac": step_bytes / us_step / 1e3 / HBM_PEAK_GBPS}}
+
+
 def m3_leg():
     """Mamba-3 SISO scan kernels at the 768-wide shape (24 heads x headdim 64, d_state 64, bf16):
     chunked SSD over batch 4 x 4096 (one layer) and the batch-1 decode step kernel."""
@@ -186,7 +231,8 @@ def m3_leg():
         b.record(); torch.cuda.synchronize()
         return a.elapsed_time(b) / n * 1e3
 
-    us = timeit(lambda: ops.m3_ssd_fwd(ssm, kst, vst, y, x, K, Q, t["dt"], t["trap"], t["a_val"], t["D"]), 10)
+    ws = torch.empty(ops.m3_ssd_workspace_bytes(B, T, nh, hd, ds), dtype=torch.uint8, device=dev)
+    us = timeit(lambda: ops.m3_ssd_fwd(ssm, kst, vst, y, x, K, Q, t["dt"], t["trap"], t["a_val"], t["D"], workspace=ws), 10)
     nbytes = 4 * B * T * nh * hd * 2 + 3 * B * T * nh * 4
     al, be, ga = ops.m3_compute_abg(t["dt"], t["a_val"], t["trap"])
     x1, K1, Q1 = x[:1, 0].contiguous(), K[:1, 0].contiguous(), Q[:1, 0].contiguous()
@@ -252,7 +298,8 @@ def main():
     if not args.no_extras:
         extras = {}
         extras["lm_130m_shape_bf16"] = lm_leg("130m-shape", dict(d_model=768, d_state=16, d_conv=4, expand=2, n_layers=24), 50280,
-                                              (8, 2048), 64, 256)
+                                              (8, 2048), [64, 1], 256)
+        extras["m1_kernels_130m_shape_bf16"] = m1_kernels_leg()
         extras["mamba3_768_bf16"] = m3_leg()
         if args.big:
             extras["lm_2.8b_shape_bf16"] = lm_leg("2.8b-shape", dict(d_model=2560, d_state=16, d_conv=4, expand=2, n_layers=64), 50280,
