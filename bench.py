@@ -251,6 +251,38 @@ def m3_leg():
             "decode_step_kernel_b1": {"us_per_layer_call_in_graph": us_step}}
 
 
+def m3_engine_leg(steps=512, batches=(1, 16)):
+    """Mamba-3 backbone decode at the 768-wide shape (24 layers, d_inner 1536, 24 heads x 64, d_state 64, 16 rope
+    angles, bf16 storage): us/step of the three-kernel layer chain in a hipGraph; the host writes nothing per step
+    (the input rows stay in the device input buffer)."""
+    import numpy as np
+    from mamba_rs_amd import GpuMamba3Backbone, Mamba3Config, Mamba3Weights, WeightDtype
+    cfg = Mamba3Config(d_model=768, d_state=64, expand=2, headdim=64, ngroups=1, n_layers=24, rope_fraction=0.5)
+    rng = np.random.default_rng(7)
+    w = Mamba3Weights.init(cfg, 768, 42)
+    w.input_proj_w = np.zeros(0, np.float32)   # identity projection, as an LM backbone
+    out = []
+    dm, di, nh, hd, ds, ip = cfg.d_model, cfg.d_inner(), cfg.nheads(), cfg.headdim, cfg.d_state, cfg.in_proj_out_dim()
+    for B in batches:
+        eng = GpuMamba3Backbone.new_with_dtype(0, w, cfg, 768, B, WeightDtype.BF16)
+        eng.step((rng.standard_normal((B, 768)) * 0.5).astype(np.float32))
+        eng.capture_graph()
+        for _ in range(8):
+            eng.step_gpu_only()
+        eng.sync()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            eng.step_gpu_only()
+        eng.sync()
+        td = (time.perf_counter() - t0) / steps
+        layer_bytes = 2 * (dm * ip + di * dm) + 2 * 4 * B * nh * (hd * ds + ds + hd) + 2 * 4 * B * dm
+        step_bytes = cfg.n_layers * layer_bytes
+        out.append({"batch": B, "steps": steps, "us_per_step": td * 1e6, "algorithmic_bytes_per_step": step_bytes,
+                    "hbm_frac": step_bytes / td / 1e9 / HBM_PEAK_GBPS})
+        eng.close()
+    return {"decode": out}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -301,6 +333,7 @@ def main():
                                               (8, 2048), [64, 1], 256)
         extras["m1_kernels_130m_shape_bf16"] = m1_kernels_leg()
         extras["mamba3_768_bf16"] = m3_leg()
+        extras["mamba3_768_bf16"]["backbone"] = m3_engine_leg()
         if args.big:
             extras["lm_2.8b_shape_bf16"] = lm_leg("2.8b-shape", dict(d_model=2560, d_state=16, d_conv=4, expand=2, n_layers=64), 50280,
                                                   (4, 4096), [1, 16, 128], 128)

@@ -285,6 +285,56 @@ MRS_API int mrs_lm_last_logits(mrs_lm *lm, float *logits);         /* [batch, vo
  * engine itself: then the head + argmax run and the next tokens are left in the token buffer). */
 MRS_API int mrs_lm_prefill(mrs_lm *lm, mrs_backbone *prefill_engine, const int *tokens, int T);
 
+/* ---- Mamba-3 SISO backbone engine (decode step) -------------------------------------------------
+ * GpuMamba3Backbone (src/mamba3_siso/gpu/inference.rs:1487-1671): weights, per-layer state
+ * (ssm [batch,nh,hd,ds], k [batch,nh,ds], v [batch,nh,hd], angle [batch,nh,n_rope], all f32) and scratch owned by
+ * the engine; host I/O is f32.  One step per call for every batch row; the ten-phase layer of
+ * step_layer_kernels (inference.rs:506-1000) is three kernels here.  Matrices are row-major [n_in, n_out]. */
+typedef struct mrs_m3_backbone mrs_m3_backbone;
+
+typedef struct {            /* Mamba3Config, src/mamba3_siso/config.rs:7-58 */
+    int d_model, d_state, expand, headdim, ngroups, n_layers;
+    int n_rope_angles;      /* num_rope_angles() = floor(d_state * rope_fraction) / 2 */
+    float a_floor;          /* A <= -a_floor */
+    int is_outproj_norm;    /* RMSNormGated before out_proj */
+    float rms_norm_eps;     /* 1e-5 in the reference (ops/fast_math.rs:17) */
+} mrs_m3_config;
+
+typedef struct {            /* Mamba3LayerWeights, src/mamba3_siso/weights.rs:14-48 */
+    const float *norm_weight;       /* [d_model] */
+    const float *in_proj_w;         /* [d_model, in_proj_out_dim]: z | x | B | C | dd_dt | dd_A | trap | angles */
+    const float *dt_bias;           /* [nheads] */
+    const float *b_norm_weight;     /* [d_state] */
+    const float *c_norm_weight;     /* [d_state] */
+    const float *b_bias;            /* [nheads, d_state] */
+    const float *c_bias;            /* [nheads, d_state] */
+    const float *d_param;           /* [nheads] */
+    const float *norm_gate_weight;  /* [d_inner] */
+    const float *out_proj_w;        /* [d_inner, d_model] */
+} mrs_m3_layer_weights;
+
+typedef struct {            /* Mamba3Weights */
+    const float *input_proj_w;  /* [input_dim, d_model], or NULL for the identity */
+    const float *input_proj_b;  /* [d_model] or NULL (zeros) */
+    const mrs_m3_layer_weights *layers;
+    const float *norm_f_weight; /* [d_model] */
+} mrs_m3_weights;
+
+/* headdim * d_state / 4 <= 1024 and d_state = 4 x a power of two <= 256 (the reference stops at headdim 32). */
+MRS_API int mrs_m3_backbone_create(mrs_m3_backbone **out, int gpu_ordinal, const mrs_m3_weights *weights,
+                                   const mrs_m3_config *cfg, int input_dim, int batch, int dtype);
+MRS_API void mrs_m3_backbone_destroy(mrs_m3_backbone *bb);
+/* step(&mut self, input: &[f32], output: &mut [f32]): input [batch, input_dim] -> norm_f output [batch, d_model] */
+MRS_API int mrs_m3_backbone_step(mrs_m3_backbone *bb, const float *input, float *output);
+MRS_API int mrs_m3_backbone_step_gpu_only(mrs_m3_backbone *bb);   /* input already in input_ptr(), output left in temporal_ptr() */
+MRS_API int mrs_m3_backbone_reset(mrs_m3_backbone *bb);
+MRS_API int mrs_m3_backbone_capture_graph(mrs_m3_backbone *bb);
+MRS_API float *mrs_m3_backbone_temporal_ptr(mrs_m3_backbone *bb);
+MRS_API float *mrs_m3_backbone_input_ptr(mrs_m3_backbone *bb);
+MRS_API void *mrs_m3_backbone_stream(mrs_m3_backbone *bb);
+MRS_API int mrs_m3_backbone_sync(mrs_m3_backbone *bb);
+MRS_API int mrs_m3_backbone_download_state(mrs_m3_backbone *bb, int layer, float *ssm, float *k, float *v, float *angle);
+
 #ifdef __cplusplus
 }
 #endif

@@ -8,3 +8,4 @@ from ._lib import MambaHipError, load as load_library  # noqa: F401
 from .config import MambaConfig, ScanMode, WeightDtype, PARALLEL_SCAN_THRESHOLD  # noqa: F401
 from .weights import MambaWeights, MambaLayerWeights  # noqa: F401
 from .backbone import GpuMambaBackbone, GpuMambaLM  # noqa: F401
+from .mamba3 import Mamba3Config, Mamba3Weights, Mamba3LayerWeights, GpuMamba3Backbone  # noqa: F401

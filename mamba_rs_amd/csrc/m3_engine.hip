@@ -1,0 +1,514 @@
+// Mamba-3 SISO backbone, decode step (GpuMamba3Backbone::step, src/mamba3_siso/gpu/inference.rs:1487-1671).
+//
+// The reference's T = 1 layer is ten phases / fourteen launches (step_layer_kernels, inference.rs:506-1000:
+// residual copy, RMSNorm, in_proj SGEMM, m3_split, bcnorm x2, bc_bias_add x2, angle_dt, rope, compute_abg,
+// m3_step, gate, out_proj SGEMM, residual add).  Every one of them is launch-bound at decode batch sizes, so
+// here a layer is THREE kernels:
+//   1. in_proj on round(residual * norm_w) with the 1/rms row scale in the epilogue (skinny GEMM, f32 output:
+//      dt, A, trap and the angles stay in f32 whatever the storage type);
+//   2. m3_layer_step_kernel, one workgroup per (batch row, head): the 8-way split is just offsets into the
+//      projection row; B/C RMSNorm + bias, softplus / heavy-tail / sigmoid, the angle accumulation (f64, wrapped
+//      to [0, 2 pi)) and rotation, alpha/beta/gamma, the trapezoidal state update with the state row in
+//      registers, y = H q + D x, and the SiLU gate (optionally RMSNormGated over the head) -- the formulas of
+//      mamba3_layer_step (src/mamba3_siso/cpu/inference.rs:68-258) and kernels/mamba3_ops.cu;
+//   3. out_proj with the residual add, the next layer's pre-scaled operand and row sums of squares as epilogue.
+// f32 storage (or shapes the skinny GEMM does not take) runs RMSNorm + rocBLAS GEMMs around the same step kernel.
+#include "common.hpp"
+#include <rocblas/rocblas.h>
+#include <new>
+#include <vector>
+
+namespace mrs {
+
+constexpr float kPi = 3.14159265358979323846f;
+constexpr int kMaxDs = 256;
+
+__device__ __forceinline__ float heavy_tail(float x) { return x >= 0.0f ? 1.0f + x : 1.0f / (1.0f - x); }
+__device__ __forceinline__ float sigmoidf_fast(float x) { return fast_rcp(1.0f + fast_exp2(-x * kLog2e)); }
+
+// One workgroup per (batch row, head); blockDim.x = hd * LG, LG = ds / 4 lanes per state row.
+// proj: [batch, ip] f32 = [z:di | x:di | B:ng*ds | C:ng*ds | dd_dt:nh | dd_A:nh | trap:nh | angles:nr]
+// gated: [batch, di] activation type (out_proj's operand).
+template <typename T, int LG>
+__global__ __launch_bounds__(1024) void m3_layer_step_kernel(
+    float *__restrict__ ssm, float *__restrict__ kst, float *__restrict__ vst, float *__restrict__ angle,
+    T *__restrict__ gated, const float *__restrict__ proj, int64_t ip, const float *__restrict__ dt_bias,
+    const float *__restrict__ bnw, const float *__restrict__ cnw, const float *__restrict__ b_bias,
+    const float *__restrict__ c_bias, const float *__restrict__ Dp, const float *__restrict__ ngw, int nh, int hd, int ng,
+    int nr, float a_floor, float eps, int outproj_norm) {
+    constexpr int ds = 4 * LG;
+    __shared__ float kl[ds], ql[ds], red[16], scal[4];
+    const int b = blockIdx.x / nh, h = blockIdx.x - b * nh;
+    const int tid = threadIdx.x, nthr = blockDim.x;
+    const int p = tid / LG, g = tid % LG;
+    const int di = nh * hd;
+    const int grp = h / (nh / ng);
+    const int64_t bh = (int64_t)b * nh + h;
+    const float *row = proj + (int64_t)b * ip;
+    const float *zr = row, *xr = row + di, *braw = row + 2 * di + (int64_t)grp * ds, *craw = row + 2 * di + (int64_t)(ng + grp) * ds;
+    const float *sc = row + 2 * di + 2 * (int64_t)ng * ds;   // dd_dt | dd_A | trap | angles
+    // state loads first: they are the long-latency part and do not depend on the prologue
+    float *Hrow = ssm + (bh * hd + p) * ds + 4 * g;
+    float4 H = *reinterpret_cast<const float4 *>(Hrow);
+    const float4 kp = *reinterpret_cast<const float4 *>(kst + bh * ds + 4 * g);
+    const float vp = vst[bh * hd + p];
+    const float xv = xr[h * hd + p];
+
+    // ---- B/C RMSNorm over d_state (bcnorm_fwd, ops/norms.rs:50-80) + per-head bias ----
+    float ssb = 0.0f, ssc = 0.0f;
+    for (int n = tid; n < ds; n += nthr) { const float bv = braw[n], cv = craw[n]; ssb = fmaf(bv, bv, ssb); ssc = fmaf(cv, cv, ssc); }
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) { ssb += __shfl_xor(ssb, m, kWave); ssc += __shfl_xor(ssc, m, kWave); }
+    // only the first ceil(ds / 64) waves hold non-zero partial sums; every wave writes its own (zero) slot
+    const int wv = tid >> 6, nw = (nthr + 63) >> 6;
+    if ((tid & 63) == 0 && wv < 8) { red[wv] = ssb; red[8 + wv] = ssc; }
+    __syncthreads();
+    if (tid == 0) {
+        float sb = 0.0f, scc = 0.0f;
+        for (int i = 0; i < min(nw, 8); i++) { sb += red[i]; scc += red[8 + i]; }
+        scal[0] = 1.0f / sqrtf(sb / (float)ds + eps);
+        scal[1] = 1.0f / sqrtf(scc / (float)ds + eps);
+        // per-head scalars (m3_split + compute_abg, kernels/mamba3_ops.cu:72-160, 735-753)
+        scal[2] = softplus20(sc[h] + dt_bias[h]);                                 // dt
+    }
+    __syncthreads();
+    const float invb = scal[0], invc = scal[1], dtv = scal[2];
+    for (int n = tid; n < ds; n += nthr) {
+        kl[n] = braw[n] * invb * bnw[n] + b_bias[(int64_t)h * ds + n];
+        ql[n] = craw[n] * invc * cnw[n] + c_bias[(int64_t)h * ds + n];
+    }
+    __syncthreads();
+    // ---- angle accumulation + rotation of the first 2*nr coordinates (angle_dt_fwd_batch + rope_fwd) ----
+    for (int a = tid; a < nr; a += nthr) {
+        const float delta = tanhf(sc[3 * nh + a]) * kPi * dtv;
+        const double two_pi = 6.283185307179586;
+        double acc = (double)angle[bh * nr + a] + (double)delta;
+        acc -= two_pi * floor(acc / two_pi);
+        const float an = (float)acc;
+        angle[bh * nr + a] = an;
+        float sn, cs;
+        sincosf(an, &sn, &cs);
+        const float b0 = kl[2 * a], b1 = kl[2 * a + 1], c0 = ql[2 * a], c1 = ql[2 * a + 1];
+        kl[2 * a] = cs * b0 - sn * b1; kl[2 * a + 1] = sn * b0 + cs * b1;
+        ql[2 * a] = cs * c0 - sn * c1; ql[2 * a + 1] = sn * c0 + cs * c1;
+    }
+    __syncthreads();
+    // ---- alpha / beta / gamma ----
+    const float a_val = fminf(-heavy_tail(sc[nh + h]), -a_floor);
+    const float trap = sigmoidf_fast(sc[2 * nh + h]);
+    const float al = fast_exp2(a_val * dtv * kLog2e);
+    const float be = al * dtv * (1.0f - trap), ga = trap * dtv;
+    // ---- trapezoidal update of this lane's four states, y = H q + D x ----
+    const float4 kc = *reinterpret_cast<const float4 *>(&kl[4 * g]);
+    const float4 qc = *reinterpret_cast<const float4 *>(&ql[4 * g]);
+    const float bv = be * vp, gx = ga * xv;
+    H.x = fmaf(al, H.x, fmaf(bv, kp.x, gx * kc.x));
+    H.y = fmaf(al, H.y, fmaf(bv, kp.y, gx * kc.y));
+    H.z = fmaf(al, H.z, fmaf(bv, kp.z, gx * kc.z));
+    H.w = fmaf(al, H.w, fmaf(bv, kp.w, gx * kc.w));
+    float acc = H.x * qc.x;
+    acc = fmaf(H.y, qc.y, acc);
+    acc = fmaf(H.z, qc.z, acc);
+    acc = fmaf(H.w, qc.w, acc);
+#pragma unroll
+    for (int m = 1; m < LG; m <<= 1) acc += __shfl_xor(acc, m, kWave);
+    const float yv = fmaf(Dp[h], xv, acc);
+    *reinterpret_cast<float4 *>(Hrow) = H;
+    // ---- gate: y * silu(z), or RMSNormGated over the head first (rmsnorm_gated_forward, ops/norms.rs:84-114) ----
+    float inv_y = 1.0f;
+    if (outproj_norm) {
+        float sq = (g == 0) ? yv * yv : 0.0f;
+#pragma unroll
+        for (int m = 32; m >= 1; m >>= 1) sq += __shfl_xor(sq, m, kWave);
+        __syncthreads();   // red is reused
+        if ((tid & 63) == 0) red[wv & 15] = sq;
+        __syncthreads();
+        float tot = 0.0f;
+        for (int i = 0; i < min(nw, 16); i++) tot += red[i];
+        inv_y = 1.0f / sqrtf(tot / (float)hd + eps);
+    }
+    if (g == 0) {
+        const float zi = zr[h * hd + p];
+        const float o = outproj_norm ? yv * inv_y * ngw[h * hd + p] * silu(zi) : yv * silu(zi);
+        Store<T>::st(gated + (int64_t)b * di + h * hd + p, o);
+        vst[bh * hd + p] = xv;
+    }
+    // every lane has read the previous k_state (kp) at the top; the barriers above order those reads before this write
+    if (p == 0) *reinterpret_cast<float4 *>(kst + bh * ds + 4 * g) = kc;
+}
+
+}  // namespace mrs
+
+using namespace mrs;
+
+#define MRS_HIP(expr)                                                                        \
+    do { hipError_t e_ = (expr); if (e_ != hipSuccess) return fail(MRS_E_HIP, "%s: %s", #expr, hipGetErrorString(e_)); } while (0)
+#define MRS_TRY(expr) do { int rc_ = (expr); if (rc_) return rc_; } while (0)
+#define MRS_BLAS(expr)                                                                        \
+    do { rocblas_status s_ = (expr); if (s_ != rocblas_status_success) return fail(MRS_E_HIP, "%s: rocblas status %d", #expr, (int)s_); } while (0)
+
+namespace {
+
+inline size_t esize3(int dtype) { return dtype == MRS_F32 ? 4 : 2; }
+inline rocblas_datatype blas_type3(int dtype) {
+    return dtype == MRS_F32 ? rocblas_datatype_f32_r : dtype == MRS_F16 ? rocblas_datatype_f16_r : rocblas_datatype_bf16_r;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void cast3_kernel(T *__restrict__ out, const float *__restrict__ in, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) Store<T>::st(out + i, in[i]);
+}
+
+// One workgroup per row: residual (f32) += add (may be null); out = rmsnorm(residual) * w in the activation type or f32.
+template <typename T, typename TO>
+__global__ __launch_bounds__(256) void add_rmsnorm3_kernel(float *__restrict__ residual, const T *__restrict__ add, TO *__restrict__ out,
+                                                           const float *__restrict__ w, float eps, int dm) {
+    __shared__ float part[4];
+    const int64_t row = blockIdx.x;
+    float *r = residual + row * dm;
+    float ss = 0.0f;
+    for (int i = threadIdx.x; i < dm; i += 256) {
+        float x = r[i];
+        if (add) { x += Store<T>::ld(add + row * dm + i); r[i] = x; }
+        ss = fmaf(x, x, ss);
+    }
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) ss += __shfl_xor(ss, m, kWave);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    ss = part[0] + part[1] + part[2] + part[3];
+    float rms = sqrtf(ss / (float)dm + eps);
+    if (!isfinite(rms) || rms < 1e-20f) rms = 1.0f;
+    const float inv = 1.0f / rms;
+    for (int i = threadIdx.x; i < dm; i += 256) Store<TO>::st(out + row * dm + i, r[i] * inv * w[i]);
+}
+
+__global__ void bias_rows3_kernel(float *__restrict__ out, const float *__restrict__ bias, int64_t n, int dm) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = bias ? bias[i % dm] : 0.0f;
+}
+
+struct Layer3 {
+    float *norm_w, *dt_bias, *bnw, *cnw, *b_bias, *c_bias, *D, *ngw;
+    void *in_proj, *out_proj;      // [K][N] storage type (library GEMM)
+    void *in_proj_t, *out_proj_t;  // [N][K] copies for the skinny GEMM (null: library chain)
+};
+
+}  // namespace
+
+struct mrs_m3_backbone {
+    mrs_m3_config cfg;
+    int input_dim, batch, dtype, di, nh, ip, nr, identity_proj, device, skinny;
+    hipStream_t stream;
+    rocblas_handle blas;
+    std::vector<Layer3> layers;
+    std::vector<void *> allocs;
+    float *input_proj_w, *input_proj_b, *norm_f;
+    float *ssm, *kst, *vst, *angle;          // [L][batch]...
+    float *d_input, *temporal, *residual, *proj, *partials;
+    void *normed, *gated, *out;
+    hipGraph_t graph;
+    hipGraphExec_t graph_exec;
+    int graph_ready;
+};
+
+namespace {
+
+int dev_alloc3(mrs_m3_backbone *bb, void **p, size_t bytes) {
+    MRS_HIP(hipMalloc(p, bytes ? bytes : 16));
+    bb->allocs.push_back(*p);
+    return MRS_OK;
+}
+int upload_f32_3(mrs_m3_backbone *bb, float **dst, const float *src, size_t n) {
+    MRS_TRY(dev_alloc3(bb, (void **)dst, n * sizeof(float)));
+    MRS_HIP(hipMemcpyAsync(*dst, src, n * sizeof(float), hipMemcpyHostToDevice, bb->stream));
+    return MRS_OK;
+}
+// bulk matrix: upload f32, round to the storage type on device (RNE)
+int upload_bulk3(mrs_m3_backbone *bb, void **dst, const float *src, size_t n, float *stage) {
+    MRS_HIP(hipMemcpyAsync(stage, src, n * sizeof(float), hipMemcpyHostToDevice, bb->stream));
+    MRS_TRY(dev_alloc3(bb, dst, n * esize3(bb->dtype)));
+    const dim3 grid((unsigned)((n + 255) / 256)), block(256);
+    if (bb->dtype == MRS_F32) MRS_HIP(hipMemcpyAsync(*dst, stage, n * 4, hipMemcpyDeviceToDevice, bb->stream));
+    else if (bb->dtype == MRS_BF16) hipLaunchKernelGGL((cast3_kernel<bf16_t>), grid, block, 0, bb->stream, (bf16_t *)*dst, stage, (int64_t)n);
+    else hipLaunchKernelGGL((cast3_kernel<f16_t>), grid, block, 0, bb->stream, (f16_t *)*dst, stage, (int64_t)n);
+    MRS_HIP(hipStreamSynchronize(bb->stream));
+    return check_launch("weight cast");
+}
+
+// C[M,N] (f32 or storage type) = A[M,K] . W[K,N], row-major, f32 accumulate (library GEMM)
+int gemm3(mrs_m3_backbone *bb, void *C, bool c_f32, const void *A, const void *W, int M, int N, int K) {
+    const float one = 1.0f, zero = 0.0f;
+    const rocblas_datatype t = blas_type3(bb->dtype), ct = c_f32 ? rocblas_datatype_f32_r : t;
+    MRS_BLAS(rocblas_gemm_ex(bb->blas, rocblas_operation_none, rocblas_operation_none, N, M, K, &one, W, t, N, A, t, K, &zero, C, ct, N, C,
+                             ct, N, rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0));
+    return MRS_OK;
+}
+
+template <typename T>
+int launch_layer_step_t(mrs_m3_backbone *bb, int l) {
+    const mrs_m3_config &c = bb->cfg;
+    const Layer3 &lw = bb->layers[l];
+    const int B = bb->batch, nh = bb->nh, hd = c.headdim, ds = c.d_state, lg = ds / 4;
+    float *ssm = bb->ssm + (size_t)l * B * nh * hd * ds, *kst = bb->kst + (size_t)l * B * nh * ds;
+    float *vst = bb->vst + (size_t)l * B * nh * hd, *ang = bb->angle + (size_t)l * B * nh * (bb->nr > 0 ? bb->nr : 1);
+    const dim3 grid((unsigned)(B * nh)), block((unsigned)(hd * lg));
+#define MRS_LG(L)                                                                                                                 \
+    case L:                                                                                                                       \
+        hipLaunchKernelGGL((m3_layer_step_kernel<T, L>), grid, block, 0, bb->stream, ssm, kst, vst, ang, (T *)bb->gated, bb->proj,  \
+                           (int64_t)bb->ip, lw.dt_bias, lw.bnw, lw.cnw, lw.b_bias, lw.c_bias, lw.D, lw.ngw, nh, hd, c.ngroups,     \
+                           bb->nr, c.a_floor, c.rms_norm_eps, c.is_outproj_norm);                                                   \
+        break
+    switch (lg) { MRS_LG(1); MRS_LG(2); MRS_LG(4); MRS_LG(8); MRS_LG(16); MRS_LG(32); MRS_LG(64); default: return fail(MRS_E_SHAPE, "m3 layer step: d_state %d", ds); }
+#undef MRS_LG
+    return check_launch("m3_layer_step_kernel");
+}
+
+int step_body3(mrs_m3_backbone *bb) {
+    const mrs_m3_config &c = bb->cfg;
+    const int dm = c.d_model, di = bb->di, B = bb->batch, dt = bb->dtype, L = c.n_layers, ip = bb->ip;
+    const int P = (dm + 15) / 16;
+    // residual <- input (identity) or input . W + b
+    const float *src = nullptr;
+    if (bb->identity_proj) {
+        if (bb->skinny) src = bb->d_input;   // the first prenorm kernel reads the input and writes the residual stream
+        else MRS_HIP(hipMemcpyAsync(bb->residual, bb->d_input, (size_t)B * dm * 4, hipMemcpyDeviceToDevice, bb->stream));
+    } else {
+        const int64_t n = (int64_t)B * dm;
+        hipLaunchKernelGGL(bias_rows3_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, bb->stream, bb->residual, bb->input_proj_b, n, dm);
+        const float one = 1.0f;
+        MRS_BLAS(rocblas_gemm_ex(bb->blas, rocblas_operation_none, rocblas_operation_none, dm, B, bb->input_dim, &one, bb->input_proj_w,
+                                 rocblas_datatype_f32_r, dm, bb->d_input, rocblas_datatype_f32_r, bb->input_dim, &one, bb->residual,
+                                 rocblas_datatype_f32_r, dm, bb->residual, rocblas_datatype_f32_r, dm, rocblas_datatype_f32_r,
+                                 rocblas_gemm_algo_standard, 0, 0));
+    }
+    for (int l = 0; l < L; l++) {
+        const Layer3 &lw = bb->layers[l];
+        if (bb->skinny) {
+            if (l == 0)
+                MRS_TRY(launch_prenorm_rows(bb->stream, dt, bb->partials, P, bb->normed, src ? src : bb->residual, src ? bb->residual : nullptr,
+                                            lw.norm_w, B, dm));
+            SkinnyEpi inp = {};
+            inp.row_scale = 1; inp.partials = bb->partials; inp.n_partials = P; inp.eps = c.rms_norm_eps;
+            MRS_TRY(launch_skinny_gemm(bb->stream, dt, bb->proj, 1, ip, bb->normed, dm, lw.in_proj_t, B, ip, dm, inp));
+        } else {
+            if (dt == MRS_F32) hipLaunchKernelGGL((add_rmsnorm3_kernel<float, float>), dim3((unsigned)B), dim3(256), 0, bb->stream, bb->residual, l == 0 ? nullptr : (const float *)bb->out, (float *)bb->normed, lw.norm_w, c.rms_norm_eps, dm);
+            else if (dt == MRS_BF16) hipLaunchKernelGGL((add_rmsnorm3_kernel<bf16_t, bf16_t>), dim3((unsigned)B), dim3(256), 0, bb->stream, bb->residual, l == 0 ? nullptr : (const bf16_t *)bb->out, (bf16_t *)bb->normed, lw.norm_w, c.rms_norm_eps, dm);
+            else hipLaunchKernelGGL((add_rmsnorm3_kernel<f16_t, f16_t>), dim3((unsigned)B), dim3(256), 0, bb->stream, bb->residual, l == 0 ? nullptr : (const f16_t *)bb->out, (f16_t *)bb->normed, lw.norm_w, c.rms_norm_eps, dm);
+            MRS_TRY(check_launch("add_rmsnorm3_kernel"));
+            MRS_TRY(gemm3(bb, bb->proj, true, bb->normed, lw.in_proj, B, ip, dm));
+        }
+        MRS_DISPATCH_DTYPE(dt, T_, MRS_TRY(launch_layer_step_t<T_>(bb, l)));
+        if (bb->skinny) {
+            SkinnyEpi outp = {};
+            outp.mode = 2; outp.residual = bb->residual; outp.partials = bb->partials; outp.n_partials = P;
+            outp.next_norm_w = l + 1 < L ? bb->layers[l + 1].norm_w : nullptr; outp.prenorm = bb->normed;
+            MRS_TRY(launch_skinny_gemm(bb->stream, dt, bb->out, 0, dm, bb->gated, di, lw.out_proj_t, B, dm, di, outp));
+        } else {
+            MRS_TRY(gemm3(bb, bb->out, false, bb->gated, lw.out_proj, B, dm, di));
+        }
+    }
+    // final residual add (library chain) + norm_f -> temporal (f32)
+    const void *add = bb->skinny ? nullptr : bb->out;
+    if (dt == MRS_F32) hipLaunchKernelGGL((add_rmsnorm3_kernel<float, float>), dim3((unsigned)B), dim3(256), 0, bb->stream, bb->residual, (const float *)add, bb->temporal, bb->norm_f, c.rms_norm_eps, dm);
+    else if (dt == MRS_BF16) hipLaunchKernelGGL((add_rmsnorm3_kernel<bf16_t, float>), dim3((unsigned)B), dim3(256), 0, bb->stream, bb->residual, (const bf16_t *)add, bb->temporal, bb->norm_f, c.rms_norm_eps, dm);
+    else hipLaunchKernelGGL((add_rmsnorm3_kernel<f16_t, float>), dim3((unsigned)B), dim3(256), 0, bb->stream, bb->residual, (const f16_t *)add, bb->temporal, bb->norm_f, c.rms_norm_eps, dm);
+    return check_launch("add_rmsnorm3_kernel");
+}
+
+}  // namespace
+
+extern "C" int mrs_m3_backbone_reset(mrs_m3_backbone *bb) {
+    if (!bb) return fail(MRS_E_NULL, "mrs_m3_backbone_reset: null engine");
+    const size_t L = bb->cfg.n_layers, B = bb->batch, nh = bb->nh, hd = bb->cfg.headdim, ds = bb->cfg.d_state, na = bb->nr > 0 ? bb->nr : 1;
+    MRS_HIP(hipMemsetAsync(bb->ssm, 0, L * B * nh * hd * ds * 4, bb->stream));
+    MRS_HIP(hipMemsetAsync(bb->kst, 0, L * B * nh * ds * 4, bb->stream));
+    MRS_HIP(hipMemsetAsync(bb->vst, 0, L * B * nh * hd * 4, bb->stream));
+    MRS_HIP(hipMemsetAsync(bb->angle, 0, L * B * nh * na * 4, bb->stream));
+    return MRS_OK;
+}
+
+extern "C" void mrs_m3_backbone_destroy(mrs_m3_backbone *bb) {
+    if (!bb) return;
+    hipSetDevice(bb->device);
+    if (bb->stream) hipStreamSynchronize(bb->stream);
+    if (bb->graph_exec) hipGraphExecDestroy(bb->graph_exec);
+    if (bb->graph) hipGraphDestroy(bb->graph);
+    for (void *p : bb->allocs) hipFree(p);
+    if (bb->blas) rocblas_destroy_handle(bb->blas);
+    if (bb->stream) hipStreamDestroy(bb->stream);
+    delete bb;
+}
+
+extern "C" int mrs_m3_backbone_create(mrs_m3_backbone **out, int gpu_ordinal, const mrs_m3_weights *w, const mrs_m3_config *cfg,
+                                      int input_dim, int batch, int dtype) {
+    const char *fn = "mrs_m3_backbone_create";
+    if (!out || !w || !cfg || !w->layers || !w->norm_f_weight) return fail(MRS_E_NULL, "%s: null pointer", fn);
+    if (dtype != MRS_F32 && dtype != MRS_F16 && dtype != MRS_BF16) return fail(MRS_E_DTYPE, "%s: dtype %d", fn, dtype);
+    // Mamba3Config::validate (src/mamba3_siso/config.rs:60-131), with this library's wider headdim / d_state limits
+    if (cfg->d_model < 1 || cfg->d_state < 1 || cfg->expand < 1 || cfg->headdim < 1 || cfg->ngroups < 1 || cfg->n_layers < 1)
+        return fail(MRS_E_SHAPE, "%s: d_model, d_state, expand, headdim, ngroups, n_layers must be > 0", fn);
+    const int64_t di64 = (int64_t)cfg->d_model * cfg->expand;
+    if (di64 % cfg->headdim != 0) return fail(MRS_E_SHAPE, "%s: d_inner %lld is not a multiple of headdim %d", fn, (long long)di64, cfg->headdim);
+    const int nh = (int)(di64 / cfg->headdim);
+    if (nh % cfg->ngroups != 0) return fail(MRS_E_SHAPE, "%s: nheads %d is not a multiple of ngroups %d", fn, nh, cfg->ngroups);
+    const int ds = cfg->d_state, lg = ds / 4;
+    if (ds % 4 != 0 || (lg & (lg - 1)) != 0 || lg > 64 || (int64_t)cfg->headdim * lg > 1024)
+        return fail(MRS_E_SHAPE, "%s: d_state must be 4 x a power of two <= 256 and headdim * d_state / 4 <= 1024 (got %d, %d)", fn, ds, cfg->headdim);
+    if (cfg->n_rope_angles < 0 || 2 * cfg->n_rope_angles > ds) return fail(MRS_E_SHAPE, "%s: n_rope_angles %d outside 0..d_state/2", fn, cfg->n_rope_angles);
+    if (!(cfg->a_floor > 0.0f)) return fail(MRS_E_SHAPE, "%s: a_floor must be > 0", fn);
+    if (batch < 1 || input_dim < 1 || di64 > 65535 || cfg->n_layers > 4096) return fail(MRS_E_SHAPE, "%s: batch=%d input_dim=%d d_inner=%lld", fn, batch, input_dim, (long long)di64);
+    const int identity = (w->input_proj_w == nullptr);
+    if (identity && input_dim != cfg->d_model) return fail(MRS_E_SHAPE, "%s: identity input_proj needs input_dim == d_model", fn);
+    mrs_m3_backbone *bb = new (std::nothrow) mrs_m3_backbone();
+    if (!bb) return fail(MRS_E_HIP, "%s: out of host memory", fn);
+    bb->cfg = *cfg; bb->input_dim = input_dim; bb->batch = batch; bb->dtype = dtype; bb->device = gpu_ordinal;
+    bb->di = (int)di64; bb->nh = nh; bb->nr = cfg->n_rope_angles; bb->identity_proj = identity;
+    bb->ip = 2 * bb->di + 2 * cfg->ngroups * ds + 3 * nh + bb->nr;
+    bb->graph_ready = 0; bb->graph = nullptr; bb->graph_exec = nullptr; bb->input_proj_w = nullptr; bb->input_proj_b = nullptr;
+    *out = nullptr;
+#define MRS_CREATE_TRY(expr) do { int rc_ = (expr); if (rc_) { mrs_m3_backbone_destroy(bb); return rc_; } } while (0)
+    {
+        hipError_t e = hipSetDevice(gpu_ordinal);
+        if (e != hipSuccess) { delete bb; return fail(MRS_E_HIP, "hipSetDevice(%d): %s", gpu_ordinal, hipGetErrorString(e)); }
+        e = hipStreamCreateWithFlags(&bb->stream, hipStreamNonBlocking);
+        if (e != hipSuccess) { delete bb; return fail(MRS_E_HIP, "hipStreamCreate: %s", hipGetErrorString(e)); }
+        if (rocblas_create_handle(&bb->blas) != rocblas_status_success) { hipStreamDestroy(bb->stream); delete bb; return fail(MRS_E_HIP, "rocblas_create_handle failed"); }
+        rocblas_set_stream(bb->blas, bb->stream);
+        rocblas_set_pointer_mode(bb->blas, rocblas_pointer_mode_host);
+    }
+    const int dm = cfg->d_model, di = bb->di, ip = bb->ip, L = cfg->n_layers;
+    bb->skinny = (dtype == MRS_BF16 || dtype == MRS_F16) && batch <= 64 && dm % 32 == 0 && di % 32 == 0;
+    float *stage = nullptr;
+    {
+        size_t big = (size_t)dm * ip;
+        if ((size_t)di * dm > big) big = (size_t)di * dm;
+        MRS_CREATE_TRY(dev_alloc3(bb, (void **)&stage, big * sizeof(float)));
+    }
+    if (!identity) {
+        MRS_CREATE_TRY(upload_f32_3(bb, &bb->input_proj_w, w->input_proj_w, (size_t)input_dim * dm));
+        if (w->input_proj_b) MRS_CREATE_TRY(upload_f32_3(bb, &bb->input_proj_b, w->input_proj_b, dm));
+    }
+    bb->layers.resize(L);
+    for (int l = 0; l < L; l++) {
+        const mrs_m3_layer_weights &s = w->layers[l];
+        Layer3 &d = bb->layers[l];
+        if (!s.norm_weight || !s.in_proj_w || !s.dt_bias || !s.b_norm_weight || !s.c_norm_weight || !s.b_bias || !s.c_bias || !s.d_param ||
+            !s.norm_gate_weight || !s.out_proj_w) {
+            mrs_m3_backbone_destroy(bb);
+            return fail(MRS_E_NULL, "%s: layer %d has a null weight", fn, l);
+        }
+        MRS_CREATE_TRY(upload_f32_3(bb, &d.norm_w, s.norm_weight, dm));
+        MRS_CREATE_TRY(upload_bulk3(bb, &d.in_proj, s.in_proj_w, (size_t)dm * ip, stage));
+        MRS_CREATE_TRY(upload_f32_3(bb, &d.dt_bias, s.dt_bias, nh));
+        MRS_CREATE_TRY(upload_f32_3(bb, &d.bnw, s.b_norm_weight, ds));
+        MRS_CREATE_TRY(upload_f32_3(bb, &d.cnw, s.c_norm_weight, ds));
+        MRS_CREATE_TRY(upload_f32_3(bb, &d.b_bias, s.b_bias, (size_t)nh * ds));
+        MRS_CREATE_TRY(upload_f32_3(bb, &d.c_bias, s.c_bias, (size_t)nh * ds));
+        MRS_CREATE_TRY(upload_f32_3(bb, &d.D, s.d_param, nh));
+        MRS_CREATE_TRY(upload_f32_3(bb, &d.ngw, s.norm_gate_weight, di));
+        MRS_CREATE_TRY(upload_bulk3(bb, &d.out_proj, s.out_proj_w, (size_t)di * dm, stage));
+        d.in_proj_t = d.out_proj_t = nullptr;
+        if (bb->skinny) {
+            const size_t es = esize3(dtype);
+            MRS_CREATE_TRY(dev_alloc3(bb, &d.in_proj_t, (size_t)dm * ip * es));
+            MRS_CREATE_TRY(dev_alloc3(bb, &d.out_proj_t, (size_t)di * dm * es));
+            MRS_CREATE_TRY(launch_transpose(bb->stream, dtype, d.in_proj_t, d.in_proj, dm, ip));
+            MRS_CREATE_TRY(launch_transpose(bb->stream, dtype, d.out_proj_t, d.out_proj, di, dm));
+        }
+    }
+    MRS_CREATE_TRY(upload_f32_3(bb, &bb->norm_f, w->norm_f_weight, dm));
+    const size_t B = batch, hd = cfg->headdim, na = bb->nr > 0 ? bb->nr : 1, es = esize3(dtype);
+    MRS_CREATE_TRY(dev_alloc3(bb, (void **)&bb->ssm, (size_t)L * B * nh * hd * ds * 4));
+    MRS_CREATE_TRY(dev_alloc3(bb, (void **)&bb->kst, (size_t)L * B * nh * ds * 4));
+    MRS_CREATE_TRY(dev_alloc3(bb, (void **)&bb->vst, (size_t)L * B * nh * hd * 4));
+    MRS_CREATE_TRY(dev_alloc3(bb, (void **)&bb->angle, (size_t)L * B * nh * na * 4));
+    MRS_CREATE_TRY(dev_alloc3(bb, (void **)&bb->d_input, B * input_dim * 4));
+    MRS_CREATE_TRY(dev_alloc3(bb, (void **)&bb->temporal, B * dm * 4));
+    MRS_CREATE_TRY(dev_alloc3(bb, (void **)&bb->residual, B * dm * 4));
+    MRS_CREATE_TRY(dev_alloc3(bb, (void **)&bb->proj, B * ip * 4));
+    MRS_CREATE_TRY(dev_alloc3(bb, (void **)&bb->partials, B * ((dm + 15) / 16) * 4));
+    MRS_CREATE_TRY(dev_alloc3(bb, &bb->normed, B * dm * es));
+    MRS_CREATE_TRY(dev_alloc3(bb, &bb->gated, B * di * es));
+    MRS_CREATE_TRY(dev_alloc3(bb, &bb->out, B * dm * es));
+    MRS_CREATE_TRY(mrs_m3_backbone_reset(bb));
+    { hipError_t e = hipStreamSynchronize(bb->stream);
+      if (e != hipSuccess) { mrs_m3_backbone_destroy(bb); return fail(MRS_E_HIP, "create sync: %s", hipGetErrorString(e)); } }
+#undef MRS_CREATE_TRY
+    *out = bb;
+    return MRS_OK;
+}
+
+extern "C" int mrs_m3_backbone_step_gpu_only(mrs_m3_backbone *bb) {
+    if (!bb) return fail(MRS_E_NULL, "mrs_m3_backbone_step_gpu_only: null engine");
+    if (bb->graph_ready) { MRS_HIP(hipGraphLaunch(bb->graph_exec, bb->stream)); return MRS_OK; }
+    return step_body3(bb);
+}
+
+extern "C" int mrs_m3_backbone_step(mrs_m3_backbone *bb, const float *input, float *output) {
+    if (!bb || !input || !output) return fail(MRS_E_NULL, "mrs_m3_backbone_step: null pointer");
+    MRS_HIP(hipMemcpyAsync(bb->d_input, input, (size_t)bb->batch * bb->input_dim * 4, hipMemcpyHostToDevice, bb->stream));
+    MRS_TRY(mrs_m3_backbone_step_gpu_only(bb));
+    MRS_HIP(hipMemcpyAsync(output, bb->temporal, (size_t)bb->batch * bb->cfg.d_model * 4, hipMemcpyDeviceToHost, bb->stream));
+    MRS_HIP(hipStreamSynchronize(bb->stream));
+    return MRS_OK;
+}
+
+// One eager warm step on a saved copy of the state (library handles pick their kernels), then capture the step body
+// (capture_graph, src/mamba3_siso/gpu/inference.rs:1560-1600).  The capture is always ended on error.
+extern "C" int mrs_m3_backbone_capture_graph(mrs_m3_backbone *bb) {
+    if (!bb) return fail(MRS_E_NULL, "mrs_m3_backbone_capture_graph: null engine");
+    if (bb->graph_ready) return MRS_OK;
+    const size_t L = bb->cfg.n_layers, B = bb->batch, nh = bb->nh, hd = bb->cfg.headdim, ds = bb->cfg.d_state, na = bb->nr > 0 ? bb->nr : 1;
+    const size_t n0 = L * B * nh * hd * ds * 4, n1 = L * B * nh * ds * 4, n2 = L * B * nh * hd * 4, n3 = L * B * nh * na * 4;
+    char *save = nullptr;
+    MRS_HIP(hipMalloc((void **)&save, n0 + n1 + n2 + n3));
+    hipMemcpyAsync(save, bb->ssm, n0, hipMemcpyDeviceToDevice, bb->stream);
+    hipMemcpyAsync(save + n0, bb->kst, n1, hipMemcpyDeviceToDevice, bb->stream);
+    hipMemcpyAsync(save + n0 + n1, bb->vst, n2, hipMemcpyDeviceToDevice, bb->stream);
+    hipMemcpyAsync(save + n0 + n1 + n2, bb->angle, n3, hipMemcpyDeviceToDevice, bb->stream);
+    int rc = step_body3(bb);
+    hipMemcpyAsync(bb->ssm, save, n0, hipMemcpyDeviceToDevice, bb->stream);
+    hipMemcpyAsync(bb->kst, save + n0, n1, hipMemcpyDeviceToDevice, bb->stream);
+    hipMemcpyAsync(bb->vst, save + n0 + n1, n2, hipMemcpyDeviceToDevice, bb->stream);
+    hipMemcpyAsync(bb->angle, save + n0 + n1 + n2, n3, hipMemcpyDeviceToDevice, bb->stream);
+    hipError_t e = hipStreamSynchronize(bb->stream);
+    hipFree(save);
+    if (rc) return rc;
+    if (e != hipSuccess) return fail(MRS_E_HIP, "capture warm-up: %s", hipGetErrorString(e));
+    MRS_HIP(hipStreamBeginCapture(bb->stream, hipStreamCaptureModeThreadLocal));
+    rc = step_body3(bb);
+    hipGraph_t g = nullptr;
+    e = hipStreamEndCapture(bb->stream, &g);
+    if (rc) { if (g) hipGraphDestroy(g); return rc; }
+    if (e != hipSuccess) return fail(MRS_E_HIP, "hipStreamEndCapture: %s", hipGetErrorString(e));
+    hipGraphExec_t ge = nullptr;
+    e = hipGraphInstantiate(&ge, g, nullptr, nullptr, 0);
+    if (e != hipSuccess) { hipGraphDestroy(g); return fail(MRS_E_HIP, "hipGraphInstantiate: %s", hipGetErrorString(e)); }
+    bb->graph = g; bb->graph_exec = ge; bb->graph_ready = 1;
+    return MRS_OK;
+}
+
+extern "C" float *mrs_m3_backbone_temporal_ptr(mrs_m3_backbone *bb) { return bb ? bb->temporal : nullptr; }
+extern "C" float *mrs_m3_backbone_input_ptr(mrs_m3_backbone *bb) { return bb ? bb->d_input : nullptr; }
+extern "C" void *mrs_m3_backbone_stream(mrs_m3_backbone *bb) { return bb ? (void *)bb->stream : nullptr; }
+extern "C" int mrs_m3_backbone_sync(mrs_m3_backbone *bb) {
+    if (!bb) return fail(MRS_E_NULL, "mrs_m3_backbone_sync: null engine");
+    MRS_HIP(hipStreamSynchronize(bb->stream));
+    return MRS_OK;
+}
+
+// Copies layer `layer`'s state to host buffers (any may be null): ssm [batch,nh,hd,ds], k [batch,nh,ds], v [batch,nh,hd],
+// angle [batch,nh,max(n_rope,1)].
+extern "C" int mrs_m3_backbone_download_state(mrs_m3_backbone *bb, int layer, float *ssm, float *k, float *v, float *angle) {
+    if (!bb) return fail(MRS_E_NULL, "mrs_m3_backbone_download_state: null engine");
+    if (layer < 0 || layer >= bb->cfg.n_layers) return fail(MRS_E_SHAPE, "mrs_m3_backbone_download_state: layer %d", layer);
+    const size_t B = bb->batch, nh = bb->nh, hd = bb->cfg.headdim, ds = bb->cfg.d_state, na = bb->nr > 0 ? bb->nr : 1, l = layer;
+    if (ssm) MRS_HIP(hipMemcpyAsync(ssm, bb->ssm + l * B * nh * hd * ds, B * nh * hd * ds * 4, hipMemcpyDeviceToHost, bb->stream));
+    if (k) MRS_HIP(hipMemcpyAsync(k, bb->kst + l * B * nh * ds, B * nh * ds * 4, hipMemcpyDeviceToHost, bb->stream));
+    if (v) MRS_HIP(hipMemcpyAsync(v, bb->vst + l * B * nh * hd, B * nh * hd * 4, hipMemcpyDeviceToHost, bb->stream));
+    if (angle) MRS_HIP(hipMemcpyAsync(angle, bb->angle + l * B * nh * na, B * nh * na * 4, hipMemcpyDeviceToHost, bb->stream));
+    MRS_HIP(hipStreamSynchronize(bb->stream));
+    return MRS_OK;
+}

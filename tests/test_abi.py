@@ -27,7 +27,8 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, n), f"{n} declared in include/ but not exported"
     # and the Python binding table covers exactly the header
     from mamba_rs_amd.backbone import engine_exported_names
-    assert sorted(_lib.exported_names() + engine_exported_names()) == names
+    from mamba_rs_amd.mamba3 import m3_engine_exported_names
+    assert sorted(_lib.exported_names() + engine_exported_names() + m3_engine_exported_names()) == names
 
 
 def test_version_and_error_string_and_dispatch_predicate():

@@ -1,0 +1,133 @@
+"""GPU parity: the Mamba-3 SISO backbone engine (decode step) vs the oracle's restatement of the reference's CPU
+layer (mamba3_layer_step, src/mamba3_siso/cpu/inference.rs:68-298), through the C ABI.
+
+The bodies follow the reference's engine tests (tests/gpu_mamba3_lm_test.rs, tests/m3_cpu_gpu_train_parity.rs:
+CPU route vs GPU route on the same weights, step by step, state compared at the end)."""
+import numpy as np
+import pytest
+
+import orc
+from util import cosine, scaled_err
+
+pytestmark = pytest.mark.gpu
+
+from mamba_rs_amd import GpuMamba3Backbone, Mamba3Config, Mamba3Weights, WeightDtype  # noqa: E402
+
+
+def oracle_params(w: Mamba3Weights, cfg: Mamba3Config, input_dim: int, round_to=None) -> orc.M3Params:
+    """Copy product-side weights into the oracle's flat block (bulk matrices optionally rounded to a storage type)."""
+    P = orc.M3Params(cfg.d_model, cfg.d_state, cfg.expand, cfg.headdim, cfg.ngroups, cfg.n_layers, cfg.rope_fraction, input_dim,
+                     seed=1, a_floor=cfg.a_floor, outproj_norm=cfg.is_outproj_norm)
+    rq = (lambda a: orc.round_to(a, round_to)) if round_to is not None else (lambda a: a)
+    P.input_proj_w[:] = w.input_proj_w; P.input_proj_b[:] = w.input_proj_b
+    for l, lw in enumerate(w.layers):
+        d = P.layers[l]
+        for n in ("norm_weight", "dt_bias", "b_norm_weight", "c_norm_weight", "b_bias", "c_bias", "d_param", "norm_gate_weight"):
+            d[n][:] = getattr(lw, n)
+        d["in_proj_w"][:] = rq(lw.in_proj_w); d["out_proj_w"][:] = rq(lw.out_proj_w)
+    P.norm_f_weight[:] = w.norm_f_weight
+    return P
+
+
+def perturbed(cfg, input_dim, seed):
+    """init() leaves norms, biases and D at one; perturb them so that a dropped or swapped weight shows."""
+    w = Mamba3Weights.init(cfg, input_dim, seed)
+    rng = np.random.default_rng(seed + 7)
+    for lw in w.layers:
+        for n in ("norm_weight", "b_norm_weight", "c_norm_weight", "b_bias", "c_bias", "d_param", "norm_gate_weight"):
+            a = getattr(lw, n)
+            a += (rng.standard_normal(a.shape) * 0.2).astype(np.float32)
+    w.norm_f_weight += (rng.standard_normal(w.norm_f_weight.shape) * 0.2).astype(np.float32)
+    w.input_proj_b += (rng.standard_normal(w.input_proj_b.shape) * 0.1).astype(np.float32)
+    return w
+
+
+CONFIGS = [
+    Mamba3Config(d_model=64, d_state=16, expand=2, headdim=16, ngroups=1, n_layers=2, rope_fraction=0.5),
+    Mamba3Config(d_model=64, d_state=32, expand=2, headdim=32, ngroups=2, n_layers=2, rope_fraction=1.0, is_outproj_norm=True),
+    Mamba3Config(d_model=64, d_state=64, expand=2, headdim=64, ngroups=1, n_layers=3, rope_fraction=0.5, a_floor=0.05),
+]
+
+
+@pytest.mark.parametrize("ci", range(len(CONFIGS)))
+def test_f32_engine_steps_match_cpu_reference_path(ci):
+    cfg = CONFIGS[ci]
+    idim = 24
+    w = perturbed(cfg, idim, 42 + ci)
+    P = oracle_params(w, cfg, idim)
+    eng = GpuMamba3Backbone.new(0, w, cfg, idim, 1)
+    st = P.zero_state()
+    rng = np.random.default_rng(ci)
+    x = rng.standard_normal((96, idim)).astype(np.float32)
+    print(f"case m3 engine f32 config={ci}", flush=True)
+    worst = 0.0
+    for t in range(96):
+        got = eng.step(x[t])
+        want = orc.m3_backbone_step(P, x[t], st)
+        worst = max(worst, scaled_err(got[0], want))
+    assert worst < 2e-4, worst
+    L = cfg.n_layers - 1
+    ssm, k, v, ang = eng.download_state(L)
+    assert scaled_err(ssm[0], st[0][L]) < 2e-4 and scaled_err(k[0], st[1][L]) < 2e-4 and scaled_err(v[0], st[2][L]) < 2e-4
+    if cfg.num_rope_angles():
+        # angles live on a circle: compare through sin/cos
+        assert np.max(np.abs(np.sin(ang[0]) - np.sin(st[3][L]))) < 1e-3 and np.max(np.abs(np.cos(ang[0]) - np.cos(st[3][L]))) < 1e-3
+    eng.close()
+
+
+def test_batch_rows_are_independent_and_graph_equals_eager():
+    cfg = CONFIGS[0]
+    w = perturbed(cfg, 64, 5)
+    w.input_proj_w = np.zeros(0, np.float32)   # identity projection (the LM case)
+    rng = np.random.default_rng(9)
+    x = rng.standard_normal((20, 3, 64)).astype(np.float32)
+    for dtype in (WeightDtype.F32, WeightDtype.BF16):
+        print(f"case m3 engine batch/graph dtype={dtype}", flush=True)
+        eng = GpuMamba3Backbone.new_with_dtype(0, w, cfg, 64, 3, dtype)
+        outs = np.stack([eng.step(x[t]) for t in range(20)])
+        for b in range(3):
+            solo = GpuMamba3Backbone.new_with_dtype(0, w, cfg, 64, 1, dtype)
+            o1 = np.stack([solo.step(x[t, b]) for t in range(20)])
+            assert np.allclose(o1[:, 0], outs[:, b], rtol=1e-5, atol=1e-5)
+            solo.close()
+        eng.reset()
+        eng.capture_graph()
+        outs_g = np.stack([eng.step(x[t]) for t in range(20)])
+        assert np.array_equal(outs_g, outs)
+        eng.close()
+
+
+@pytest.mark.parametrize("dtype", [WeightDtype.BF16, WeightDtype.F16])
+@pytest.mark.parametrize("ci", [0, 1])
+def test_16bit_engine_tracks_cpu_path_on_rounded_weights(dtype, ci):
+    """bf16/f16 storage (own-GEMM decode chain: folded RMSNorm, residual epilogue) vs the CPU route on weights
+    rounded to the storage type: cosine >= 0.999 per step, the reference's mixed-precision bar."""
+    cfg = CONFIGS[ci]
+    w = perturbed(cfg, 64, 11 + ci)
+    w.input_proj_w = np.zeros(0, np.float32)
+    code = orc.BF16 if dtype == WeightDtype.BF16 else orc.F16
+    wi = Mamba3Weights(np.eye(64, dtype=np.float32), np.zeros(64, np.float32), w.layers, w.norm_f_weight)
+    P = oracle_params(wi, cfg, 64, round_to=code)
+    eng = GpuMamba3Backbone.new_with_dtype(0, w, cfg, 64, 2, dtype)
+    st = [P.zero_state() for _ in range(2)]
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((48, 2, 64)).astype(np.float32)
+    print(f"case m3 engine 16-bit dtype={dtype} config={ci}", flush=True)
+    for t in range(48):
+        got = eng.step(x[t])
+        for b in range(2):
+            want = orc.m3_backbone_step(P, x[t, b], st[b])
+            assert cosine(got[b], want) >= 0.999, (t, b)
+    eng.close()
+
+
+def test_create_rejects_bad_configs():
+    from mamba_rs_amd import MambaHipError
+    cfg = CONFIGS[0]
+    w = Mamba3Weights.init(cfg, 16, 1)
+    with pytest.raises(MambaHipError) as e:   # identity projection needs input_dim == d_model
+        w2 = Mamba3Weights(np.zeros(0, np.float32), w.input_proj_b, w.layers, w.norm_f_weight)
+        GpuMamba3Backbone.new(0, w2, cfg, 16, 1)
+    assert e.value.code == -2
+    with pytest.raises(ValueError):           # d_state 24 is not 4 x a power of two
+        Mamba3Config(d_model=64, d_state=24, headdim=16).validate()

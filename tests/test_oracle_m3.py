@@ -272,3 +272,18 @@ def test_m3_step_determinism_reset_and_rotation_norm():
     k_unrot = Braw / np.sqrt(np.mean(Braw ** 2) + 1e-5) + 1.0
     assert np.allclose(np.linalg.norm(k, axis=1), np.linalg.norm(k_unrot), rtol=1e-5)
     assert np.allclose(k[:, 2 * P0.n_rope:], k_unrot[2 * P0.n_rope:], rtol=1e-5, atol=1e-6)   # indices >= 2*n_rope pass through
+
+
+def test_python_mamba3_weights_init_equals_the_oracle_restatement():
+    """Mamba3Weights.init (numpy, the host mirror) against the oracle's C restatement of weights.rs:120-147: the
+    xorshift64 draws and Kaiming scaling bit for bit, dt_bias (exp/log round trip) to 1 ulp."""
+    from mamba_rs_amd import Mamba3Config, Mamba3Weights
+    cfg = Mamba3Config(d_model=32, d_state=16, expand=2, headdim=16, ngroups=1, n_layers=2, rope_fraction=0.5)
+    w = Mamba3Weights.init(cfg, 24, 42)
+    P = orc.M3Params(32, 16, 2, 16, 1, 2, 0.5, 24, seed=42)
+    assert np.array_equal(w.input_proj_w, P.input_proj_w) and np.array_equal(w.norm_f_weight, P.norm_f_weight)
+    for lw, pl in zip(w.layers, P.layers):
+        for n in ("norm_weight", "in_proj_w", "b_norm_weight", "c_norm_weight", "b_bias", "c_bias", "d_param", "norm_gate_weight", "out_proj_w"):
+            assert np.array_equal(getattr(lw, n), pl[n]), n
+        assert np.allclose(lw.dt_bias, pl["dt_bias"], rtol=3e-7, atol=0)
+    assert cfg.in_proj_out_dim() == P.ip and cfg.num_rope_angles() == P.n_rope
