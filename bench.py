@@ -251,10 +251,10 @@ def m3_leg():
             "decode_step_kernel_b1": {"us_per_layer_call_in_graph": us_step}}
 
 
-def m3_engine_leg(steps=512, batches=(1, 16)):
-    """Mamba-3 backbone decode at the 768-wide shape (24 layers, d_inner 1536, 24 heads x 64, d_state 64, 16 rope
-    angles, bf16 storage): us/step of the three-kernel layer chain in a hipGraph; the host writes nothing per step
-    (the input rows stay in the device input buffer)."""
+def m3_engine_leg(steps=512, batches=(1, 16), prefill_bt=(4, 4096)):
+    """Mamba-3 backbone at the 768-wide shape (24 layers, d_inner 1536, 24 heads x 64, d_state 64, 16 rope angles,
+    bf16 storage): prefill tok/s over batch 4 x 4096 (inputs resident in the device input buffer) and decode us/step
+    of the three-kernel layer chain in a hipGraph (the host writes nothing per step)."""
     import numpy as np
     from mamba_rs_amd import GpuMamba3Backbone, Mamba3Config, Mamba3Weights, WeightDtype
     cfg = Mamba3Config(d_model=768, d_state=64, expand=2, headdim=64, ngroups=1, n_layers=24, rope_fraction=0.5)
@@ -263,6 +263,16 @@ def m3_engine_leg(steps=512, batches=(1, 16)):
     w.input_proj_w = np.zeros(0, np.float32)   # identity projection, as an LM backbone
     out = []
     dm, di, nh, hd, ds, ip = cfg.d_model, cfg.d_inner(), cfg.nheads(), cfg.headdim, cfg.d_state, cfg.in_proj_out_dim()
+    pb, pt = prefill_bt
+    pre = GpuMamba3Backbone.new_with_dtype(0, w, cfg, 768, pb, WeightDtype.BF16)
+    pre.prefill_sequence((rng.standard_normal((pb, pt, 768)) * 0.5).astype(np.float32))   # warm-up; leaves the input on the device
+    times = []
+    for _ in range(3):
+        pre.reset(); pre.sync()
+        t0 = time.perf_counter(); pre.prefill_device(pt); pre.sync(); times.append(time.perf_counter() - t0)
+    tp = sorted(times)[1]
+    prefill = {"batch": pb, "seq_len": pt, "ms": tp * 1e3, "tok_per_s": pb * pt / tp}
+    pre.close()
     for B in batches:
         eng = GpuMamba3Backbone.new_with_dtype(0, w, cfg, 768, B, WeightDtype.BF16)
         eng.step((rng.standard_normal((B, 768)) * 0.5).astype(np.float32))
@@ -280,7 +290,7 @@ def m3_engine_leg(steps=512, batches=(1, 16)):
         out.append({"batch": B, "steps": steps, "us_per_step": td * 1e6, "algorithmic_bytes_per_step": step_bytes,
                     "hbm_frac": step_bytes / td / 1e9 / HBM_PEAK_GBPS})
         eng.close()
-    return {"decode": out}
+    return {"prefill": prefill, "decode": out}
 
 
 def main():

@@ -334,6 +334,15 @@ MRS_API float *mrs_m3_backbone_input_ptr(mrs_m3_backbone *bb);
 MRS_API void *mrs_m3_backbone_stream(mrs_m3_backbone *bb);
 MRS_API int mrs_m3_backbone_sync(mrs_m3_backbone *bb);
 MRS_API int mrs_m3_backbone_download_state(mrs_m3_backbone *bb, int layer, float *ssm, float *k, float *v, float *angle);
+/* Prefill: whole sequences [batch, T, input_dim] through the chunked SSD route (in_proj GEMM, angle prefix sums, the
+ * split/bcnorm/bias/rope glue of kernels/mamba3_ops.cu in one kernel, mrs_m3_ssd_fwd with carried state, gate, out_proj),
+ * continuing from the engine's state and leaving it positioned for step().  The reference's GPU forward of a layer over T
+ * is gpu_forward_mamba3_layer (src/mamba3_siso/gpu/forward.rs:27); its CPU prefill mamba3_siso/cpu/prefill.rs:151-572.
+ * One sequence length per engine (scratch is allocated on first use or by alloc_prefill_scratch). */
+MRS_API int mrs_m3_backbone_alloc_prefill_scratch(mrs_m3_backbone *bb, int T);
+MRS_API int mrs_m3_backbone_prefill_sequence(mrs_m3_backbone *bb, const float *input, int T, float *out_last);
+MRS_API int mrs_m3_backbone_prefill_device(mrs_m3_backbone *bb, int T);
+MRS_API float *mrs_m3_backbone_prefill_input_ptr(mrs_m3_backbone *bb);
 
 #ifdef __cplusplus
 }

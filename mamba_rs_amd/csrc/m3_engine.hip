@@ -137,6 +137,183 @@ __global__ __launch_bounds__(1024) void m3_layer_step_kernel(
     if (p == 0) *reinterpret_cast<float4 *>(kst + bh * ds + 4 * g) = kc;
 }
 
+// ---- prefill glue ---------------------------------------------------------------------------------
+// Three kernels in front of the chunked scan (the reference's m3_split, bcnorm_fwd x2, bc_bias_add x2, angle_dt_fwd,
+// rope_fwd, kernels/mamba3_ops.cu:72-650):
+//   m3_scalars_kernel     row-parallel: dt = softplus(dd_dt + bias), a = min(-heavy_tail(dd_A), -a_floor),
+//                         trap = sigmoid(raw), and tanh(angle_raw) * pi per rope pair;
+//   m3_angle_scan_kernel  the rotation angle of (head, pair) at step t is the initial angle plus the running sum over
+//                         time of (tanh * pi) * dt_h (angle_dt_fwd is sequential over T per thread): here a workgroup
+//                         per (batch row, head) splits T into segments -- per-segment sums, an exclusive prefix over
+//                         the segments, then the running sums inside each segment -- in f64, wrapped to [0, 2 pi);
+//   m3_kq_kernel          row-parallel: B/C RMSNorm + per-head bias + rotation -> K, Q; x -> activation type.
+__device__ __forceinline__ double wrap_2pi(double a) {
+    const double two_pi = 6.283185307179586;
+    return a - two_pi * floor(a / two_pi);
+}
+
+// one thread per (row, j): j < nh -> the head scalars, j >= nh -> rope pair j - nh
+__global__ __launch_bounds__(256) void m3_scalars_kernel(float *__restrict__ dt_out, float *__restrict__ a_out, float *__restrict__ trap_out,
+                                                         float *__restrict__ tanhpi_out, const float *__restrict__ proj, int64_t ip,
+                                                         const float *__restrict__ dt_bias, int64_t rows, int nh, int nr, int sc_off,
+                                                         float a_floor) {
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int per = nh + nr;
+    if (idx >= rows * per) return;
+    const int64_t r = idx / per;
+    const int j = (int)(idx - r * per);
+    const float *sc = proj + r * ip + sc_off;
+    if (j < nh) {
+        dt_out[r * nh + j] = softplus20(sc[j] + dt_bias[j]);
+        a_out[r * nh + j] = fminf(-heavy_tail(sc[nh + j]), -a_floor);
+        trap_out[r * nh + j] = sigmoidf_fast(sc[2 * nh + j]);
+    } else {
+        tanhpi_out[r * nr + (j - nh)] = tanhf(sc[3 * nh + (j - nh)]) * kPi;
+    }
+}
+
+// grid = batch * nh, 1024 threads = nr_pad rope pairs (fast) x nsegs segments; angle_out [rows][nh][nr] f32
+__global__ __launch_bounds__(1024) void m3_angle_scan_kernel(float *__restrict__ angle_out, float *__restrict__ angle_state,
+                                                             const float *__restrict__ dt, const float *__restrict__ tanhpi, int Tlen,
+                                                             int nh, int nr, int nr_pad) {
+    __shared__ double part[1024];
+    const int b = blockIdx.x / nh, h = blockIdx.x - b * nh;
+    const int a = threadIdx.x % nr_pad, seg = threadIdx.x / nr_pad;
+    const int nsegs = 1024 / nr_pad;
+    const int seglen = (Tlen + nsegs - 1) / nsegs;
+    const int t0 = min(Tlen, seg * seglen), t1 = min(Tlen, t0 + seglen);
+    const bool live = a < nr;
+    const float *dp = dt + (int64_t)b * Tlen * nh + h;
+    const float *tp = tanhpi + (int64_t)b * Tlen * nr + a;
+    double sum = 0.0;
+    if (live)
+        for (int t = t0; t < t1; t++) sum += (double)(tp[(int64_t)t * nr] * dp[(int64_t)t * nh]);
+    part[seg * nr_pad + a] = sum;
+    __syncthreads();
+    if (seg == 0 && live) {
+        float *stp = angle_state + ((int64_t)b * nh + h) * nr + a;
+        double acc = (double)*stp;
+        for (int s2 = 0; s2 < nsegs; s2++) {
+            const double add = part[s2 * nr_pad + a];
+            part[s2 * nr_pad + a] = acc;
+            acc = wrap_2pi(acc + add);
+        }
+        *stp = (float)acc;
+    }
+    __syncthreads();
+    if (live) {
+        double acc = part[seg * nr_pad + a];
+        for (int t = t0; t < t1; t++) {
+            acc = wrap_2pi(acc + (double)(tp[(int64_t)t * nr] * dp[(int64_t)t * nh]));
+            angle_out[(((int64_t)b * Tlen + t) * nh + h) * nr + a] = (float)acc;
+        }
+    }
+}
+
+// one workgroup (256 threads) per row
+template <typename T>
+__global__ __launch_bounds__(256) void m3_kq_kernel(
+    T *__restrict__ Kout, T *__restrict__ Qout, T *__restrict__ xout, const float *__restrict__ proj, int64_t ip,
+    const float *__restrict__ angle, const float *__restrict__ bnw, const float *__restrict__ cnw,
+    const float *__restrict__ b_bias, const float *__restrict__ c_bias, int nh, int hd, int ng, int ds, int nr, float eps) {
+    extern __shared__ float smem[];
+    const int di = nh * hd, ngds = ng * ds;
+    float *bn = smem, *cn = bn + ngds, *inv = cn + ngds;
+    const int64_t r = blockIdx.x;
+    const float *row = proj + r * ip;
+    const int tid = threadIdx.x;
+    for (int i = tid; i < ngds; i += 256) { bn[i] = row[2 * di + i]; cn[i] = row[2 * di + ngds + i]; }
+    __syncthreads();
+    // one wave-sized slice per (B or C, group): 2*ng reductions of ds values
+    {
+        const int w = tid >> 6, l = tid & 63;
+        for (int q = w; q < 2 * ng; q += 4) {
+            const float *v = (q < ng ? bn : cn) + (q % ng) * ds;
+            float ss = 0.0f;
+            for (int n = l; n < ds; n += 64) ss = fmaf(v[n], v[n], ss);
+#pragma unroll
+            for (int m = 32; m >= 1; m >>= 1) ss += __shfl_xor(ss, m, kWave);
+            if (l == 0) inv[q] = 1.0f / sqrtf(ss / (float)ds + eps);
+        }
+    }
+    __syncthreads();
+    // four consecutive state coordinates (two rotation pairs) per thread and trip: 16-byte reads, 8-byte stores
+    const int hpg = nh / ng, quarter = ds / 4;
+    struct alignas(4 * sizeof(T)) V4 { T v[4]; };
+    for (int i = tid; i < nh * quarter; i += 256) {
+        const int h = i / quarter, j4 = i - h * quarter, g = h / hpg, n = 4 * j4;
+        const float4 bw = *reinterpret_cast<const float4 *>(bnw + n), cw = *reinterpret_cast<const float4 *>(cnw + n);
+        const float4 bb4 = *reinterpret_cast<const float4 *>(b_bias + h * ds + n), cb4 = *reinterpret_cast<const float4 *>(c_bias + h * ds + n);
+        const float ib = inv[g], ic = inv[ng + g];
+        float k[4] = {bn[g * ds + n] * ib * bw.x + bb4.x, bn[g * ds + n + 1] * ib * bw.y + bb4.y, bn[g * ds + n + 2] * ib * bw.z + bb4.z,
+                      bn[g * ds + n + 3] * ib * bw.w + bb4.w};
+        float q[4] = {cn[g * ds + n] * ic * cw.x + cb4.x, cn[g * ds + n + 1] * ic * cw.y + cb4.y, cn[g * ds + n + 2] * ic * cw.z + cb4.z,
+                      cn[g * ds + n + 3] * ic * cw.w + cb4.w};
+#pragma unroll
+        for (int pr = 0; pr < 2; pr++) {
+            const int j = 2 * j4 + pr;
+            if (j < nr) {
+                float s_, c_;
+                sincosf(angle[(r * nh + h) * nr + j], &s_, &c_);
+                const float k0 = k[2 * pr], k1 = k[2 * pr + 1], q0 = q[2 * pr], q1 = q[2 * pr + 1];
+                k[2 * pr] = c_ * k0 - s_ * k1; k[2 * pr + 1] = s_ * k0 + c_ * k1;
+                q[2 * pr] = c_ * q0 - s_ * q1; q[2 * pr + 1] = s_ * q0 + c_ * q1;
+            }
+        }
+        V4 kv, qv;
+#pragma unroll
+        for (int e = 0; e < 4; e++) { Store<T>::st(&kv.v[e], k[e]); Store<T>::st(&qv.v[e], q[e]); }
+        *reinterpret_cast<V4 *>(Kout + (r * nh + h) * ds + n) = kv;
+        *reinterpret_cast<V4 *>(Qout + (r * nh + h) * ds + n) = qv;
+    }
+    if ((di & 3) == 0 && (ip & 3) == 0) {
+        for (int i = tid; i < di / 4; i += 256) {
+            const float4 xv = *reinterpret_cast<const float4 *>(row + di + 4 * i);
+            V4 o;
+            Store<T>::st(&o.v[0], xv.x); Store<T>::st(&o.v[1], xv.y); Store<T>::st(&o.v[2], xv.z); Store<T>::st(&o.v[3], xv.w);
+            *reinterpret_cast<V4 *>(xout + r * di + 4 * i) = o;
+        }
+    } else {
+        for (int i = tid; i < di; i += 256) Store<T>::st(xout + r * di + i, row[di + i]);
+    }
+}
+
+// gated[row, i] = y * silu(z), or RMSNormGated over each head first; one workgroup (256 threads) per row, a wave per head at a time
+template <typename T>
+__global__ __launch_bounds__(256) void m3_gate_kernel(T *__restrict__ gated, const T *__restrict__ y, const float *__restrict__ proj,
+                                                      int64_t ip, const float *__restrict__ ngw, int nh, int hd, float eps, int outproj_norm) {
+    const int64_t r = blockIdx.x;
+    const int di = nh * hd;
+    const float *z = proj + r * ip;
+    if (!outproj_norm) {
+        if ((di & 3) == 0 && (ip & 3) == 0) {
+            struct alignas(4 * sizeof(T)) V4 { T v[4]; };
+            for (int i = threadIdx.x; i < di / 4; i += 256) {
+                const float4 zv = *reinterpret_cast<const float4 *>(z + 4 * i);
+                V4 yv = *reinterpret_cast<const V4 *>(y + r * di + 4 * i);
+                Store<T>::st(&yv.v[0], Store<T>::ld(&yv.v[0]) * silu(zv.x)); Store<T>::st(&yv.v[1], Store<T>::ld(&yv.v[1]) * silu(zv.y));
+                Store<T>::st(&yv.v[2], Store<T>::ld(&yv.v[2]) * silu(zv.z)); Store<T>::st(&yv.v[3], Store<T>::ld(&yv.v[3]) * silu(zv.w));
+                *reinterpret_cast<V4 *>(gated + r * di + 4 * i) = yv;
+            }
+        } else {
+            for (int i = threadIdx.x; i < di; i += 256) Store<T>::st(gated + r * di + i, Store<T>::ld(y + r * di + i) * silu(z[i]));
+        }
+        return;
+    }
+    const int w = threadIdx.x >> 6, l = threadIdx.x & 63;
+    for (int h = w; h < nh; h += 4) {
+        float ss = 0.0f;
+        for (int p = l; p < hd; p += 64) { const float v = Store<T>::ld(y + r * di + h * hd + p); ss = fmaf(v, v, ss); }
+#pragma unroll
+        for (int m = 32; m >= 1; m >>= 1) ss += __shfl_xor(ss, m, kWave);
+        const float inv = 1.0f / sqrtf(ss / (float)hd + eps);
+        for (int p = l; p < hd; p += 64) {
+            const int i = h * hd + p;
+            Store<T>::st(gated + r * di + i, Store<T>::ld(y + r * di + i) * inv * ngw[i] * silu(z[i]));
+        }
+    }
+}
+
 }  // namespace mrs
 
 using namespace mrs;
@@ -211,6 +388,11 @@ struct mrs_m3_backbone {
     hipGraph_t graph;
     hipGraphExec_t graph_exec;
     int graph_ready;
+    // prefill scratch for sequences of pf_T steps (0: not allocated)
+    int pf_T;
+    float *pf_in, *pf_residual, *pf_proj, *pf_dt, *pf_a, *pf_trap, *pf_tanhpi, *pf_angle;
+    void *pf_normed, *pf_x, *pf_K, *pf_Q, *pf_y, *pf_gated, *pf_out, *pf_ws;
+    size_t pf_ws_bytes;
 };
 
 namespace {
@@ -367,6 +549,7 @@ extern "C" int mrs_m3_backbone_create(mrs_m3_backbone **out, int gpu_ordinal, co
     bb->di = (int)di64; bb->nh = nh; bb->nr = cfg->n_rope_angles; bb->identity_proj = identity;
     bb->ip = 2 * bb->di + 2 * cfg->ngroups * ds + 3 * nh + bb->nr;
     bb->graph_ready = 0; bb->graph = nullptr; bb->graph_exec = nullptr; bb->input_proj_w = nullptr; bb->input_proj_b = nullptr;
+    bb->pf_T = 0;
     *out = nullptr;
 #define MRS_CREATE_TRY(expr) do { int rc_ = (expr); if (rc_) { mrs_m3_backbone_destroy(bb); return rc_; } } while (0)
     {
@@ -489,6 +672,166 @@ extern "C" int mrs_m3_backbone_capture_graph(mrs_m3_backbone *bb) {
     bb->graph = g; bb->graph_exec = ge; bb->graph_ready = 1;
     return MRS_OK;
 }
+
+// ---- prefill -----------------------------------------------------------------------------------------
+extern "C" int mrs_m3_backbone_alloc_prefill_scratch(mrs_m3_backbone *bb, int T) {
+    const char *fn = "mrs_m3_backbone_alloc_prefill_scratch";
+    if (!bb) return fail(MRS_E_NULL, "%s: null engine", fn);
+    if (T < 1) return fail(MRS_E_SHAPE, "%s: T=%d", fn, T);
+    if (bb->pf_T == T) return MRS_OK;
+    if (bb->pf_T) return fail(MRS_E_SHAPE, "%s: scratch already allocated for T=%d (one sequence length per engine)", fn, bb->pf_T);
+    const mrs_m3_config &c = bb->cfg;
+    const size_t rows = (size_t)bb->batch * T, es = esize3(bb->dtype), dm = c.d_model, di = bb->di, nh = bb->nh, ds = c.d_state, ip = bb->ip;
+    if ((int64_t)rows * ip > 0x7fffffffLL) return fail(MRS_E_SHAPE, "%s: batch*T*in_proj_dim exceeds i32", fn);
+    if (bb->nr > 1024) return fail(MRS_E_SHAPE, "%s: more than 1024 rope pairs", fn);
+    const size_t nrz = bb->nr > 0 ? bb->nr : 1;
+    MRS_TRY(dev_alloc3(bb, (void **)&bb->pf_in, rows * bb->input_dim * 4));
+    MRS_TRY(dev_alloc3(bb, (void **)&bb->pf_residual, rows * dm * 4));
+    MRS_TRY(dev_alloc3(bb, (void **)&bb->pf_proj, rows * ip * 4));
+    MRS_TRY(dev_alloc3(bb, (void **)&bb->pf_dt, rows * nh * 4));
+    MRS_TRY(dev_alloc3(bb, (void **)&bb->pf_a, rows * nh * 4));
+    MRS_TRY(dev_alloc3(bb, (void **)&bb->pf_trap, rows * nh * 4));
+    MRS_TRY(dev_alloc3(bb, (void **)&bb->pf_tanhpi, rows * nrz * 4));
+    MRS_TRY(dev_alloc3(bb, (void **)&bb->pf_angle, rows * nh * nrz * 4));
+    MRS_TRY(dev_alloc3(bb, &bb->pf_normed, rows * dm * es));
+    MRS_TRY(dev_alloc3(bb, &bb->pf_x, rows * di * es));
+    MRS_TRY(dev_alloc3(bb, &bb->pf_K, rows * nh * ds * es));
+    MRS_TRY(dev_alloc3(bb, &bb->pf_Q, rows * nh * ds * es));
+    MRS_TRY(dev_alloc3(bb, &bb->pf_y, rows * di * es));
+    MRS_TRY(dev_alloc3(bb, &bb->pf_gated, rows * di * es));
+    MRS_TRY(dev_alloc3(bb, &bb->pf_out, rows * dm * es));
+    size_t wsb = mrs_m3_ssd_workspace_bytes(bb->batch, T, (int)nh, c.headdim, c.d_state, 64);
+    const size_t abg = 3 * rows * nh * 4;   // alpha, beta, gamma for shapes the chunked kernel does not take
+    if (abg > wsb) wsb = abg;
+    bb->pf_ws_bytes = wsb;
+    MRS_TRY(dev_alloc3(bb, &bb->pf_ws, wsb));
+    bb->pf_T = T;
+    return MRS_OK;
+}
+
+namespace {
+
+template <typename T>
+int launch_kq_t(mrs_m3_backbone *bb, const Layer3 &lw, int64_t rows) {
+    const mrs_m3_config &c = bb->cfg;
+    const int ng = c.ngroups, ds = c.d_state;
+    const size_t lds = (size_t)(2 * ng * ds + 2 * ng) * sizeof(float);
+    if (lds > 60000) return fail(MRS_E_SHAPE, "m3 K/Q kernel: ngroups * d_state too large for LDS (%zu bytes)", lds);
+    hipLaunchKernelGGL((m3_kq_kernel<T>), dim3((unsigned)rows), dim3(256), lds, bb->stream, (T *)bb->pf_K, (T *)bb->pf_Q, (T *)bb->pf_x,
+                       bb->pf_proj, (int64_t)bb->ip, bb->pf_angle, lw.bnw, lw.cnw, lw.b_bias, lw.c_bias, bb->nh, c.headdim, ng, ds, bb->nr,
+                       c.rms_norm_eps);
+    return check_launch("m3_kq_kernel");
+}
+
+template <typename T>
+int launch_gate_t(mrs_m3_backbone *bb, const Layer3 &lw, int64_t rows) {
+    const mrs_m3_config &c = bb->cfg;
+    hipLaunchKernelGGL((m3_gate_kernel<T>), dim3((unsigned)rows), dim3(256), 0, bb->stream, (T *)bb->pf_gated, (const T *)bb->pf_y, bb->pf_proj,
+                       (int64_t)bb->ip, lw.ngw, bb->nh, c.headdim, c.rms_norm_eps, c.is_outproj_norm);
+    return check_launch("m3_gate_kernel");
+}
+
+int launch_add_rmsnorm3(mrs_m3_backbone *bb, float *residual, const void *add, void *out, bool out_f32, const float *w, int64_t rows) {
+    const int dm = bb->cfg.d_model;
+    const float eps = bb->cfg.rms_norm_eps;
+    const dim3 grid((unsigned)rows), block(256);
+    const int dt = bb->dtype;
+    if (dt == MRS_F32) hipLaunchKernelGGL((add_rmsnorm3_kernel<float, float>), grid, block, 0, bb->stream, residual, (const float *)add, (float *)out, w, eps, dm);
+    else if (dt == MRS_BF16 && out_f32) hipLaunchKernelGGL((add_rmsnorm3_kernel<bf16_t, float>), grid, block, 0, bb->stream, residual, (const bf16_t *)add, (float *)out, w, eps, dm);
+    else if (dt == MRS_BF16) hipLaunchKernelGGL((add_rmsnorm3_kernel<bf16_t, bf16_t>), grid, block, 0, bb->stream, residual, (const bf16_t *)add, (bf16_t *)out, w, eps, dm);
+    else if (out_f32) hipLaunchKernelGGL((add_rmsnorm3_kernel<f16_t, float>), grid, block, 0, bb->stream, residual, (const f16_t *)add, (float *)out, w, eps, dm);
+    else hipLaunchKernelGGL((add_rmsnorm3_kernel<f16_t, f16_t>), grid, block, 0, bb->stream, residual, (const f16_t *)add, (f16_t *)out, w, eps, dm);
+    return check_launch("add_rmsnorm3_kernel");
+}
+
+int prefill_body3(mrs_m3_backbone *bb, int T) {
+    const mrs_m3_config &c = bb->cfg;
+    const int dm = c.d_model, di = bb->di, B = bb->batch, dt = bb->dtype, L = c.n_layers, ip = bb->ip, nh = bb->nh, hd = c.headdim, ds = c.d_state;
+    const int64_t rows = (int64_t)B * T;
+    const size_t es = esize3(dt);
+    const int nr = bb->nr;
+    if (bb->identity_proj) {
+        MRS_HIP(hipMemcpyAsync(bb->pf_residual, bb->pf_in, (size_t)rows * dm * 4, hipMemcpyDeviceToDevice, bb->stream));
+    } else {
+        const int64_t n = rows * dm;
+        hipLaunchKernelGGL(bias_rows3_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, bb->stream, bb->pf_residual, bb->input_proj_b, n, dm);
+        const float one = 1.0f;
+        MRS_BLAS(rocblas_gemm_ex(bb->blas, rocblas_operation_none, rocblas_operation_none, dm, (int)rows, bb->input_dim, &one, bb->input_proj_w,
+                                 rocblas_datatype_f32_r, dm, bb->pf_in, rocblas_datatype_f32_r, bb->input_dim, &one, bb->pf_residual,
+                                 rocblas_datatype_f32_r, dm, bb->pf_residual, rocblas_datatype_f32_r, dm, rocblas_datatype_f32_r,
+                                 rocblas_gemm_algo_standard, 0, 0));
+    }
+    const bool chunked_ok = (hd == 16 || hd == 32 || hd == 64) && (ds == 16 || ds == 32 || ds == 64);
+    for (int l = 0; l < L; l++) {
+        const Layer3 &lw = bb->layers[l];
+        float *ssm = bb->ssm + (size_t)l * B * nh * hd * ds, *kst = bb->kst + (size_t)l * B * nh * ds;
+        float *vst = bb->vst + (size_t)l * B * nh * hd, *ang = bb->angle + (size_t)l * B * nh * (nr > 0 ? nr : 1);
+        MRS_TRY(launch_add_rmsnorm3(bb, bb->pf_residual, l == 0 ? nullptr : bb->pf_out, bb->pf_normed, false, lw.norm_w, rows));
+        // in_proj with an f32 result: dt, A, trap and the angle inputs keep full precision whatever the storage type
+        {
+            const float one = 1.0f, zero = 0.0f;
+            const rocblas_datatype t = blas_type3(dt);
+            MRS_BLAS(rocblas_gemm_ex(bb->blas, rocblas_operation_none, rocblas_operation_none, ip, (int)rows, dm, &one, lw.in_proj, t, ip,
+                                     bb->pf_normed, t, dm, &zero, bb->pf_proj, rocblas_datatype_f32_r, ip, bb->pf_proj, rocblas_datatype_f32_r,
+                                     ip, rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0));
+        }
+        {
+            const int64_t n = rows * (nh + nr);
+            hipLaunchKernelGGL(m3_scalars_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, bb->stream, bb->pf_dt, bb->pf_a, bb->pf_trap,
+                               bb->pf_tanhpi, bb->pf_proj, (int64_t)ip, lw.dt_bias, rows, nh, nr, 2 * di + 2 * c.ngroups * ds, c.a_floor);
+            MRS_TRY(check_launch("m3_scalars_kernel"));
+        }
+        if (nr > 0) {
+            int nr_pad = 1;
+            while (nr_pad < nr) nr_pad <<= 1;
+            hipLaunchKernelGGL(m3_angle_scan_kernel, dim3((unsigned)(B * nh)), dim3(1024), 0, bb->stream, bb->pf_angle, ang, bb->pf_dt,
+                               bb->pf_tanhpi, T, nh, nr, nr_pad);
+            MRS_TRY(check_launch("m3_angle_scan_kernel"));
+        }
+        MRS_DISPATCH_DTYPE(dt, T_, MRS_TRY(launch_kq_t<T_>(bb, lw, rows)));
+        if (chunked_ok) {
+            MRS_TRY(mrs_m3_ssd_fwd(bb->stream, dt, ssm, kst, vst, bb->pf_y, bb->pf_x, bb->pf_K, bb->pf_Q, bb->pf_dt, bb->pf_trap, bb->pf_a, lw.D,
+                                   bb->pf_ws, bb->pf_ws_bytes, MRS_M3_CARRY_STATE, B, T, nh, hd, ds, 64));
+        } else {
+            float *al = (float *)bb->pf_ws, *be = al + rows * nh, *ga = be + rows * nh;
+            MRS_TRY(mrs_m3_compute_abg(bb->stream, al, be, ga, bb->pf_dt, bb->pf_a, bb->pf_trap, rows * nh));
+            MRS_TRY(mrs_m3_seq_fwd(bb->stream, dt, ssm, kst, vst, bb->pf_y, bb->pf_x, bb->pf_K, bb->pf_Q, al, be, ga, lw.D, B, T, nh, hd, ds));
+        }
+        MRS_DISPATCH_DTYPE(dt, T_, MRS_TRY(launch_gate_t<T_>(bb, lw, rows)));
+        MRS_TRY(gemm3(bb, bb->pf_out, false, bb->pf_gated, lw.out_proj, (int)rows, dm, di));
+    }
+    // only the last position of each sequence is kept: final residual add + norm_f on those rows
+    for (int b = 0; b < B; b++) {
+        const size_t r = (size_t)b * T + (T - 1);
+        MRS_TRY(launch_add_rmsnorm3(bb, bb->pf_residual + r * dm, (const char *)bb->pf_out + r * dm * es, bb->temporal + (size_t)b * dm, true,
+                                    bb->norm_f, 1));
+    }
+    return MRS_OK;
+}
+
+}  // namespace
+
+// Runs the sequences already in prefill_input_ptr() ([batch, T, input_dim] f32), continuing from the engine's state and
+// leaving it positioned for step(); norm_f output of the last position in temporal_ptr().
+extern "C" int mrs_m3_backbone_prefill_device(mrs_m3_backbone *bb, int T) {
+    if (!bb) return fail(MRS_E_NULL, "mrs_m3_backbone_prefill_device: null engine");
+    if (T < 1) return fail(MRS_E_SHAPE, "mrs_m3_backbone_prefill_device: T=%d", T);
+    MRS_TRY(mrs_m3_backbone_alloc_prefill_scratch(bb, T));
+    return prefill_body3(bb, T);
+}
+
+extern "C" int mrs_m3_backbone_prefill_sequence(mrs_m3_backbone *bb, const float *input, int T, float *out_last) {
+    if (!bb || !input) return fail(MRS_E_NULL, "mrs_m3_backbone_prefill_sequence: null pointer");
+    if (T < 1) return fail(MRS_E_SHAPE, "mrs_m3_backbone_prefill_sequence: T=%d", T);
+    MRS_TRY(mrs_m3_backbone_alloc_prefill_scratch(bb, T));
+    MRS_HIP(hipMemcpyAsync(bb->pf_in, input, (size_t)bb->batch * T * bb->input_dim * 4, hipMemcpyHostToDevice, bb->stream));
+    MRS_TRY(prefill_body3(bb, T));
+    if (out_last) MRS_HIP(hipMemcpyAsync(out_last, bb->temporal, (size_t)bb->batch * bb->cfg.d_model * 4, hipMemcpyDeviceToHost, bb->stream));
+    MRS_HIP(hipStreamSynchronize(bb->stream));
+    return MRS_OK;
+}
+
+extern "C" float *mrs_m3_backbone_prefill_input_ptr(mrs_m3_backbone *bb) { return bb ? bb->pf_in : nullptr; }
 
 extern "C" float *mrs_m3_backbone_temporal_ptr(mrs_m3_backbone *bb) { return bb ? bb->temporal : nullptr; }
 extern "C" float *mrs_m3_backbone_input_ptr(mrs_m3_backbone *bb) { return bb ? bb->d_input : nullptr; }

@@ -183,6 +183,10 @@ def _bind():
         "mrs_m3_backbone_stream": (P, [P]),
         "mrs_m3_backbone_sync": (c_int, [P]),
         "mrs_m3_backbone_download_state": (c_int, [P, c_int, _FP, _FP, _FP, _FP]),
+        "mrs_m3_backbone_alloc_prefill_scratch": (c_int, [P, c_int]),
+        "mrs_m3_backbone_prefill_sequence": (c_int, [P, _FP, c_int, _FP]),
+        "mrs_m3_backbone_prefill_device": (c_int, [P, c_int]),
+        "mrs_m3_backbone_prefill_input_ptr": (P, [P]),
     }
     for name, (res, args) in sigs.items():
         fn = getattr(lib, name)
@@ -259,6 +263,25 @@ class GpuMamba3Backbone:
 
     def step_gpu_only(self):
         _call("mrs_m3_backbone_step_gpu_only", self._h)
+
+    def alloc_prefill_scratch(self, T: int):
+        _call("mrs_m3_backbone_alloc_prefill_scratch", self._h, T)
+
+    def prefill_sequence(self, inp: np.ndarray) -> np.ndarray:
+        """inp [batch, T, input_dim] f32 -> norm_f output of the last position [batch, d_model]; the state is left
+        positioned for step()."""
+        inp = np.ascontiguousarray(inp, dtype=np.float32)
+        if inp.ndim != 3 or inp.shape[0] != self.batch or inp.shape[2] != self.input_dim:
+            raise ValueError("input must be [batch, T, input_dim]")
+        out = np.empty((self.batch, self.cfg.d_model), np.float32)
+        _call("mrs_m3_backbone_prefill_sequence", self._h, _fp(inp), inp.shape[1], _fp(out))
+        return out
+
+    def prefill_device(self, T: int):
+        _call("mrs_m3_backbone_prefill_device", self._h, T)
+
+    def prefill_input_ptr(self) -> int:
+        return _bind().mrs_m3_backbone_prefill_input_ptr(self._h)
 
     def reset(self):
         _call("mrs_m3_backbone_reset", self._h)

@@ -131,3 +131,78 @@ def test_create_rejects_bad_configs():
     assert e.value.code == -2
     with pytest.raises(ValueError):           # d_state 24 is not 4 x a power of two
         Mamba3Config(d_model=64, d_state=24, headdim=16).validate()
+
+
+# ---- prefill ------------------------------------------------------------------------------------------
+
+PREFILL_CASES = [(0, 150, WeightDtype.F32), (1, 97, WeightDtype.F32), (2, 130, WeightDtype.F32),
+                 (0, 200, WeightDtype.BF16), (2, 200, WeightDtype.BF16), (1, 70, WeightDtype.F16)]
+
+
+@pytest.mark.parametrize("ci,T,dtype", PREFILL_CASES)
+def test_prefill_equals_T_steps_of_the_cpu_path_and_hands_off_to_step(ci, T, dtype):
+    """Whole-sequence prefill (GEMMs over all rows, angle prefix sums, chunked SSD with carried state) against T
+    single steps of the CPU layer: last-position output, final state of every kind, and the steps that follow
+    (the handoff the reference tests in tests/prefill.rs:173-232 for Mamba-1)."""
+    cfg = CONFIGS[ci]
+    w = perturbed(cfg, 64, 21 + ci)
+    w.input_proj_w = np.zeros(0, np.float32)
+    wi = Mamba3Weights(np.eye(64, dtype=np.float32), np.zeros(64, np.float32), w.layers, w.norm_f_weight)
+    code = {WeightDtype.F32: None, WeightDtype.BF16: orc.BF16, WeightDtype.F16: orc.F16}[dtype]
+    P = oracle_params(wi, cfg, 64, round_to=code)
+    B = 2
+    rng = np.random.default_rng(31 + ci)
+    xs = rng.standard_normal((B, T + 6, 64)).astype(np.float32)
+    print(f"case m3 prefill config={ci} T={T} dtype={dtype}", flush=True)
+    eng = GpuMamba3Backbone.new_with_dtype(0, w, cfg, 64, B, dtype)
+    last = eng.prefill_sequence(xs[:, :T])
+    st = [P.zero_state() for _ in range(B)]
+    want_last = np.zeros((B, 64), np.float32)
+    for b in range(B):
+        for t in range(T):
+            want_last[b] = orc.m3_backbone_step(P, xs[b, t], st[b])
+    exact = dtype == WeightDtype.F32
+    for b in range(B):
+        if exact:
+            assert scaled_err(last[b], want_last[b]) < 5e-4, (b, scaled_err(last[b], want_last[b]))
+        else:
+            assert cosine(last[b], want_last[b]) >= 0.999, (b, cosine(last[b], want_last[b]))
+    L = cfg.n_layers - 1
+    ssm, k, v, ang = eng.download_state(L)
+    for b in range(B):
+        tol_cos = 0.9999 if exact else 0.995
+        assert cosine(ssm[b], st[b][0][L]) >= tol_cos and cosine(k[b], st[b][1][L]) >= tol_cos and cosine(v[b], st[b][2][L]) >= tol_cos
+        if cfg.num_rope_angles():
+            lim = 2e-3 if exact else 0.1
+            assert np.max(np.abs(np.sin(ang[b]) - np.sin(st[b][3][L]))) < lim and np.max(np.abs(np.cos(ang[b]) - np.cos(st[b][3][L]))) < lim
+    # handoff: the steps after the prefill continue the same trajectory
+    for t in range(T, T + 6):
+        got = eng.step(xs[:, t])
+        for b in range(B):
+            want = orc.m3_backbone_step(P, xs[b, t], st[b])
+            if exact:
+                assert scaled_err(got[b], want) < 5e-4, (t, b)
+            else:
+                assert cosine(got[b], want) >= 0.999, (t, b)
+    eng.close()
+
+
+def test_prefill_twice_continues_the_state_and_unsupported_chunk_shape_takes_the_sequential_route():
+    """Two prefills of T steps == the CPU path over 2T steps (carried ssm/k/v/angle state); d_state 128 is outside the
+    chunked kernel's shapes, so the engine forms alpha/beta/gamma and runs the recurrence kernel."""
+    cfg = Mamba3Config(d_model=64, d_state=128, expand=2, headdim=16, ngroups=1, n_layers=2, rope_fraction=0.5)
+    w = perturbed(cfg, 64, 77)
+    w.input_proj_w = np.zeros(0, np.float32)
+    wi = Mamba3Weights(np.eye(64, dtype=np.float32), np.zeros(64, np.float32), w.layers, w.norm_f_weight)
+    P = oracle_params(wi, cfg, 64)
+    T = 45
+    rng = np.random.default_rng(5)
+    xs = rng.standard_normal((1, 2 * T, 64)).astype(np.float32)
+    eng = GpuMamba3Backbone.new(0, w, cfg, 64, 1)
+    eng.prefill_sequence(xs[:, :T])
+    last = eng.prefill_sequence(xs[:, T:])
+    st = P.zero_state()
+    for t in range(2 * T):
+        want = orc.m3_backbone_step(P, xs[0, t], st)
+    assert scaled_err(last[0], want) < 5e-4
+    eng.close()
