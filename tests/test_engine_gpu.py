@@ -213,3 +213,23 @@ def test_engine_rejects_bad_config():
     with pytest.raises(MambaHipError):
         eng.alloc_prefill_scratch(32)                     # one sequence length per engine
     eng.close()
+
+
+def test_16bit_engine_batch_above_64_takes_the_library_gemm_chain():
+    """The own skinny GEMM serves batch <= 64; a batch of 65 runs add+RMSNorm, vendor GEMMs, conv step and the fused
+    scan step instead.  Same bar as the small-batch chain: cosine >= 0.999 per step against the CPU route on rounded
+    weights, and rows 0 and 64 (first row of the fifth 16-row tile, were it tiled) behave alike."""
+    w = MambaWeights.init(TINY, 128, 43)
+    P = oracle_params(w, TINY, 128, round_to=orc.BF16)
+    B = 65
+    eng = GpuMambaBackbone.new_with_dtype(0, w, TINY, 128, B, WeightDtype.BF16)
+    rng = np.random.default_rng(8)
+    x = rng.standard_normal((12, B, 128)).astype(np.float32)
+    rows = (0, 31, 64)
+    st = {b: orc.m1_zero_state(P) for b in rows}
+    for t in range(12):
+        got = eng.step(x[t])
+        for b in rows:
+            want = orc.m1_backbone_step(P, x[t, b], *st[b])
+            assert cosine(got[b], want) >= 0.999, (t, b)
+    eng.close()
