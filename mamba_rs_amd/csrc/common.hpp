@@ -93,6 +93,10 @@ bool skinny_gemm_ok(int dtype, int M, int N, int K, int64_t lda, const void *A, 
 int launch_skinny_gemm(hipStream_t st, int dtype, void *C, int out_f32, int64_t ldc, const void *A, int64_t lda, const void *Wt,
                        int M, int N, int K, const SkinnyEpi &ep);
 int launch_transpose(hipStream_t st, int dtype, void *Wt, const void *W, int K, int N);
+// delta[r, d] = softplus(round(dt_in[r, :] . wt[d, :]) + bias[d]) for 16-bit storage; wt is the transposed [d_inner][dt_rank] weight
+bool dt_proj_softplus_ok(int dtype, int di, int dr, int64_t xs, const void *delta, const void *dt_in, const void *wt);
+int launch_dt_proj_softplus(hipStream_t st, int dtype, void *delta, const void *dt_in, int64_t xs, const void *wt, const float *bias,
+                            int64_t rows, int di, int dr);
 // partials[row][0] = sum_k x[row][k]^2, partials[row][1..n_partials) = 0; prenorm[row][k] = round(x[row][k] * w[k])
 int launch_prenorm_rows(hipStream_t st, int dtype, float *partials, int n_partials, void *prenorm, const float *x, float *copy_to,
                         const float *w, int M, int K);

@@ -251,7 +251,8 @@ using namespace mrs;
 struct LayerDev {
     float *norm_w, *conv_w, *conv_b, *dt_b, *a_neg, *D;
     void *in_proj, *x_proj, *dt_w, *out_proj;
-    void *dt_w_t;  // [d_inner][dt_rank] copy for the fused decode step (null: the [dt_rank][d_inner] one is read)
+    void *dt_w_t;  // [d_inner][dt_rank] copy: the fused decode step (when dt_t_step) and the prefill dt_proj+softplus kernel read it
+    int dt_t_step;
     void *in_proj_t, *x_proj_t, *out_proj_t;  // [N][K] copies for the decode chain's own GEMM (null: library GEMM)
     int s4d;
 };
@@ -414,8 +415,8 @@ static int run_layers(mrs_backbone *bb, Scratch *s, int T) {
             MRS_TRY(launch_skinny_gemm(bb->stream, dt, s->proj, 0, 2 * di, s->normed, dm, lw.in_proj_t, B, 2 * di, dm, inp));
             const SkinnyEpi none = {};
             MRS_TRY(launch_skinny_gemm(bb->stream, dt, s->xdbl, 0, xd, s->u, di, lw.x_proj_t, B, xd, di, none));
-            MRS_TRY(launch_ssm_step_fused(bb->stream, dt, ssm, s->y, s->delta, lw.dt_b, s->xdbl, lw.dt_w_t ? lw.dt_w_t : lw.dt_w, dr,
-                                          lw.dt_w_t != nullptr, s->u, xb + es * dr,
+            MRS_TRY(launch_ssm_step_fused(bb->stream, dt, ssm, s->y, s->delta, lw.dt_b, s->xdbl, lw.dt_t_step ? lw.dt_w_t : lw.dt_w, dr,
+                                          lw.dt_t_step, s->u, xb + es * dr,
                                           xb + es * (dr + ds), xd, z, 2 * di, 2, lw.a_neg, lw.D, B, di, ds));
             SkinnyEpi outp = {};
             outp.mode = 2; outp.residual = s->residual; outp.partials = s->partials; outp.n_partials = P;
@@ -429,12 +430,16 @@ static int run_layers(mrs_backbone *bb, Scratch *s, int T) {
             MRS_TRY(launch_conv1d_step(bb->stream, dt, s->u, conv, s->proj, 2 * di, lw.conv_w, lw.conv_b, B, di, dc, 1));
             MRS_TRY(gemm_rm(bb, dt, s->xdbl, xd, s->u, di, lw.x_proj, (int)rows, xd, di));
             // dt_proj (K = dt_rank) + bias + softplus + state update + B/C gather + SiLU gate: one kernel
-            MRS_TRY(launch_ssm_step_fused(bb->stream, dt, ssm, s->y, s->delta, lw.dt_b, s->xdbl, lw.dt_w_t ? lw.dt_w_t : lw.dt_w, dr,
-                                          lw.dt_w_t != nullptr, s->u, xb + es * dr,
+            MRS_TRY(launch_ssm_step_fused(bb->stream, dt, ssm, s->y, s->delta, lw.dt_b, s->xdbl, lw.dt_t_step ? lw.dt_w_t : lw.dt_w, dr,
+                                          lw.dt_t_step, s->u, xb + es * dr,
                                           xb + es * (dr + ds), xd, z, 2 * di, 2, lw.a_neg, lw.D, B, di, ds));
         } else {
             MRS_TRY(mrs_conv1d_seq_silu(bb->stream, dt, s->u, conv, s->proj, 2 * di, lw.conv_w, lw.conv_b, B, T, di, dc));
             MRS_TRY(gemm_rm(bb, dt, s->xdbl, xd, s->u, di, lw.x_proj, (int)rows, xd, di));
+            if (lw.dt_w_t && dt_proj_softplus_ok(dt, di, dr, xd, s->delta, s->xdbl, lw.dt_w_t)) {
+                // dt_proj + bias + softplus in one matrix-core kernel (K = dt_rank is tiny: the op is one write of delta)
+                MRS_TRY(launch_dt_proj_softplus(bb->stream, dt, s->delta, s->xdbl, xd, lw.dt_w_t, lw.dt_b, rows, di, dr));
+            } else {
             MRS_TRY(gemm_rm(bb, dt, s->delta, di, s->xdbl, xd, lw.dt_w, (int)rows, di, dr));
             const int64_t n = rows * di;
             MRS_DISPATCH_DTYPE(dt, T_, {
@@ -445,6 +450,7 @@ static int run_layers(mrs_backbone *bb, Scratch *s, int T) {
                     hipLaunchKernelGGL((bias_softplus_kernel<T_, 1>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, bb->stream, (T_ *)s->delta, lw.dt_b, n, di);
             });
             MRS_TRY(check_launch("bias_softplus_kernel"));
+            }
             // ScanMode::use_parallel picks the route (src/mamba_ssm/gpu/prefill.rs:910-956)
             unsigned flags = MRS_GATE_SILU | (lw.s4d ? MRS_A_S4D_REAL : 0);
             if (!mrs_scan_use_parallel(bb->cfg.scan_mode, T, ds)) flags |= MRS_FORCE_SEQUENTIAL;
@@ -536,7 +542,8 @@ extern "C" int mrs_backbone_create(mrs_backbone **out, int gpu_ordinal, const mr
         MRS_CREATE_TRY(upload_f32(bb, &d.D, src.d_param, di));
         MRS_CREATE_TRY(upload_bulk(bb, &d.out_proj, src.out_proj_w, (size_t)di * dm, stage));
         d.in_proj_t = d.x_proj_t = d.out_proj_t = d.dt_w_t = nullptr;
-        if ((ds == 4 || ds == 8 || ds == 16 || ds == 32 || ds == 64 || ds == 128 || ds == 256) && dr % ds == 0 && xd % 4 == 0) {
+        d.dt_t_step = (ds == 4 || ds == 8 || ds == 16 || ds == 32 || ds == 64 || ds == 128 || ds == 256) && dr % ds == 0 && xd % 4 == 0;
+        if (d.dt_t_step || (bb->dtype != MRS_F32 && dr % 8 == 0)) {
             MRS_CREATE_TRY(dev_alloc(bb, &d.dt_w_t, (size_t)dr * di * esize(bb->dtype)));
             MRS_CREATE_TRY(launch_transpose(bb->stream, bb->dtype, d.dt_w_t, d.dt_w, dr, di));
         }

@@ -204,6 +204,57 @@ __global__ __launch_bounds__(256) void prenorm_rows_kernel(float *__restrict__ p
     for (int p = threadIdx.x; p < n_partials; p += 256) partials[row * n_partials + p] = p == 0 ? part[0] + part[1] + part[2] + part[3] : 0.0f;
 }
 
+
+// Prefill dt_proj with its bias and softplus fused: delta[r, d] = softplus(round_T(sum_k dt_in[r, k] dt_w[k, d]) + bias[d]).
+// The reference runs a GEMM with K = dt_rank, then bias add and softplus_forward (src/mamba_ssm/gpu/prefill.rs:846-905,
+// kernels/activations.cu:32-52).  K is tiny (48 at d_model 768), so the op is one write of delta (50 MB per layer at the
+// 130m prefill shape) and nothing else: a workgroup forms a 64 x 64 tile with two v_mfma_f32_16x16x32 steps per 16 x 16 block
+// (K zero-padded to a multiple of 32), applies the epilogue on the accumulators, and transposes through LDS so that the
+// rows leave as 16-byte stores.  dt_in rows have stride xs (they are the head of the x_proj row); wt is [d_inner][dt_rank].
+template <typename T>
+__global__ __launch_bounds__(256) void dt_proj_softplus_kernel(T *__restrict__ delta, const T *__restrict__ dt_in, int64_t xs,
+                                                               const T *__restrict__ wt, const float *__restrict__ bias, int64_t rows,
+                                                               int di, int dr) {
+    __shared__ alignas(16) T tile[4][16][64 + 8];
+    const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, lr = l & 15, lg = l >> 4;
+    const int64_t m0 = (int64_t)blockIdx.y * 64 + 16 * w;
+    const int n0 = blockIdx.x * 64;
+    v4f acc[4];
+#pragma unroll
+    for (int nt = 0; nt < 4; nt++) acc[nt] = (v4f){0.f, 0.f, 0.f, 0.f};
+    const int64_t arow = min(m0 + lr, rows - 1);
+    for (int k0 = 0; k0 < dr; k0 += 32) {
+        const int k = k0 + 8 * lg;
+        const bool kin = k < dr;   // dt_rank % 8 == 0: a lane's 8 values are all inside or all outside
+        uint4 af = make_uint4(0, 0, 0, 0);
+        if (kin) af = *reinterpret_cast<const uint4 *>(dt_in + arow * xs + k);
+#pragma unroll
+        for (int nt = 0; nt < 4; nt++) {
+            const int col = min(n0 + 16 * nt + lr, di - 1);
+            uint4 bf = make_uint4(0, 0, 0, 0);
+            if (kin) bf = *reinterpret_cast<const uint4 *>(wt + (int64_t)col * dr + k);
+            acc[nt] = Mma32<T>::mma(af, bf, acc[nt]);
+        }
+    }
+#pragma unroll
+    for (int nt = 0; nt < 4; nt++) {
+        const int col = min(n0 + 16 * nt + lr, di - 1);
+        const float bv = bias[col];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const T raw = (T)acc[nt][i];   // the projection as the reference stores it, before bias and softplus
+            Store<T>::st(&tile[w][4 * lg + i][16 * nt + lr], softplus20(Store<T>::ld(&raw) + bv));
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        const int idx = l + 64 * j, r = idx >> 3, seg = idx & 7;
+        if (m0 + r < rows && n0 + seg * 8 < di)
+            *reinterpret_cast<uint4 *>(delta + (m0 + r) * di + n0 + seg * 8) = *reinterpret_cast<const uint4 *>(&tile[w][r][seg * 8]);
+    }
+}
+
 // Wt[n][k] = W[k][n]: 32x32 tiles through LDS so both sides are coalesced.
 template <typename T>
 __global__ __launch_bounds__(256) void transpose_kernel(T *__restrict__ Wt, const T *__restrict__ W, int K, int N) {
@@ -263,6 +314,23 @@ int launch_prenorm_rows(hipStream_t st, int dtype, float *partials, int n_partia
     else if (dtype == MRS_F16) hipLaunchKernelGGL((prenorm_rows_kernel<f16_t>), dim3((unsigned)M), dim3(256), 0, st, partials, n_partials, (f16_t *)prenorm, x, copy_to, w, K);
     else return fail(MRS_E_DTYPE, "prenorm rows: 16-bit storage only");
     return check_launch("prenorm_rows_kernel");
+}
+
+bool dt_proj_softplus_ok(int dtype, int di, int dr, int64_t xs, const void *delta, const void *dt_in, const void *wt) {
+    return (dtype == MRS_BF16 || dtype == MRS_F16) && di % 8 == 0 && dr >= 8 && dr % 8 == 0 && xs % 8 == 0 && aligned(delta, 16) &&
+           aligned(dt_in, 16) && aligned(wt, 16);
+}
+
+int launch_dt_proj_softplus(hipStream_t st, int dtype, void *delta, const void *dt_in, int64_t xs, const void *wt, const float *bias,
+                            int64_t rows, int di, int dr) {
+    if (!dt_proj_softplus_ok(dtype, di, dr, xs, delta, dt_in, wt))
+        return fail(MRS_E_SHAPE, "dt_proj+softplus: needs 16-bit storage, d_inner, dt_rank and the row stride multiples of 8, 16-byte aligned operands");
+    const int64_t gy = (rows + 63) / 64;
+    if (rows < 1 || gy > 65535) return fail(MRS_E_SHAPE, "dt_proj+softplus: rows=%lld", (long long)rows);
+    const dim3 grid((unsigned)((di + 63) / 64), (unsigned)gy), block(256);
+    if (dtype == MRS_BF16) hipLaunchKernelGGL((dt_proj_softplus_kernel<bf16_t>), grid, block, 0, st, (bf16_t *)delta, (const bf16_t *)dt_in, xs, (const bf16_t *)wt, bias, rows, di, dr);
+    else hipLaunchKernelGGL((dt_proj_softplus_kernel<f16_t>), grid, block, 0, st, (f16_t *)delta, (const f16_t *)dt_in, xs, (const f16_t *)wt, bias, rows, di, dr);
+    return check_launch("dt_proj_softplus_kernel");
 }
 
 int launch_transpose(hipStream_t st, int dtype, void *Wt, const void *W, int K, int N) {
