@@ -259,8 +259,7 @@ def m3_engine_leg(steps=512, batches=(1, 16), prefill_bt=(4, 4096)):
     from mamba_rs_amd import GpuMamba3Backbone, Mamba3Config, Mamba3Weights, WeightDtype
     cfg = Mamba3Config(d_model=768, d_state=64, expand=2, headdim=64, ngroups=1, n_layers=24, rope_fraction=0.5)
     rng = np.random.default_rng(7)
-    w = Mamba3Weights.init(cfg, 768, 42)
-    w.input_proj_w = np.zeros(0, np.float32)   # identity projection, as an LM backbone
+    w = Mamba3Weights.random_lm(cfg, 42)       # identity projection, as an LM backbone
     out = []
     dm, di, nh, hd, ds, ip = cfg.d_model, cfg.d_inner(), cfg.nheads(), cfg.headdim, cfg.d_state, cfg.in_proj_out_dim()
     pb, pt = prefill_bt

@@ -248,6 +248,8 @@ __global__ __launch_bounds__(64) void argmax_final_kernel(int *__restrict__ toke
 
 using namespace mrs;
 
+constexpr int64_t kFuseDtProjLimit = 4096;  // batch * dt_rank up to which dt_proj is folded into the decode step kernel
+
 struct LayerDev {
     float *norm_w, *conv_w, *conv_b, *dt_b, *a_neg, *D;
     void *in_proj, *x_proj, *dt_w, *out_proj;
@@ -415,9 +417,16 @@ static int run_layers(mrs_backbone *bb, Scratch *s, int T) {
             MRS_TRY(launch_skinny_gemm(bb->stream, dt, s->proj, 0, 2 * di, s->normed, dm, lw.in_proj_t, B, 2 * di, dm, inp));
             const SkinnyEpi none = {};
             MRS_TRY(launch_skinny_gemm(bb->stream, dt, s->xdbl, 0, xd, s->u, di, lw.x_proj_t, B, xd, di, none));
-            MRS_TRY(launch_ssm_step_fused(bb->stream, dt, ssm, s->y, s->delta, lw.dt_b, s->xdbl, lw.dt_t_step ? lw.dt_w_t : lw.dt_w, dr,
-                                          lw.dt_t_step, s->u, xb + es * dr,
-                                          xb + es * (dr + ds), xd, z, 2 * di, 2, lw.a_neg, lw.D, B, di, ds));
+            if ((int64_t)B * dr > kFuseDtProjLimit && lw.dt_w_t && skinny_gemm_ok(dt, B, di, dr, xd, s->xdbl, lw.dt_w_t)) {
+                // wide dt_rank at a large batch: dt_proj as a GEMM of its own, bias + softplus in the step kernel
+                MRS_TRY(launch_skinny_gemm(bb->stream, dt, s->delta, 0, di, s->xdbl, xd, lw.dt_w_t, B, di, dr, none));
+                MRS_TRY(launch_ssm_step_fused(bb->stream, dt, ssm, s->y, s->delta, lw.dt_b, nullptr, nullptr, 0, 0, s->u, xb + es * dr,
+                                              xb + es * (dr + ds), xd, z, 2 * di, 2, lw.a_neg, lw.D, B, di, ds));
+            } else {
+                MRS_TRY(launch_ssm_step_fused(bb->stream, dt, ssm, s->y, s->delta, lw.dt_b, s->xdbl, lw.dt_t_step ? lw.dt_w_t : lw.dt_w, dr,
+                                              lw.dt_t_step, s->u, xb + es * dr,
+                                              xb + es * (dr + ds), xd, z, 2 * di, 2, lw.a_neg, lw.D, B, di, ds));
+            }
             SkinnyEpi outp = {};
             outp.mode = 2; outp.residual = s->residual; outp.partials = s->partials; outp.n_partials = P;
             outp.next_norm_w = l + 1 < L ? bb->layers[l + 1].norm_w : nullptr; outp.prenorm = s->normed;
@@ -429,10 +438,18 @@ static int run_layers(mrs_backbone *bb, Scratch *s, int T) {
         if (T == 1) {
             MRS_TRY(launch_conv1d_step(bb->stream, dt, s->u, conv, s->proj, 2 * di, lw.conv_w, lw.conv_b, B, di, dc, 1));
             MRS_TRY(gemm_rm(bb, dt, s->xdbl, xd, s->u, di, lw.x_proj, (int)rows, xd, di));
-            // dt_proj (K = dt_rank) + bias + softplus + state update + B/C gather + SiLU gate: one kernel
-            MRS_TRY(launch_ssm_step_fused(bb->stream, dt, ssm, s->y, s->delta, lw.dt_b, s->xdbl, lw.dt_t_step ? lw.dt_w_t : lw.dt_w, dr,
-                                          lw.dt_t_step, s->u, xb + es * dr,
-                                          xb + es * (dr + ds), xd, z, 2 * di, 2, lw.a_neg, lw.D, B, di, ds));
+            if ((int64_t)B * dr <= kFuseDtProjLimit) {
+                // dt_proj (K = dt_rank) + bias + softplus + state update + B/C gather + SiLU gate: one kernel
+                MRS_TRY(launch_ssm_step_fused(bb->stream, dt, ssm, s->y, s->delta, lw.dt_b, s->xdbl, lw.dt_t_step ? lw.dt_w_t : lw.dt_w, dr,
+                                              lw.dt_t_step, s->u, xb + es * dr,
+                                              xb + es * (dr + ds), xd, z, 2 * di, 2, lw.a_neg, lw.D, B, di, ds));
+            } else {
+                // large batch x dt_rank: every batch row would re-read the whole dt_proj weight inside the step kernel
+                // (83 us at batch 128, d_inner 5120, dt_rank 160), so the projection goes to the library GEMM
+                MRS_TRY(gemm_rm(bb, dt, s->delta, di, s->xdbl, xd, lw.dt_w, (int)rows, di, dr));
+                MRS_TRY(launch_ssm_step_fused(bb->stream, dt, ssm, s->y, s->delta, lw.dt_b, nullptr, nullptr, 0, 0, s->u, xb + es * dr,
+                                              xb + es * (dr + ds), xd, z, 2 * di, 2, lw.a_neg, lw.D, B, di, ds));
+            }
         } else {
             MRS_TRY(mrs_conv1d_seq_silu(bb->stream, dt, s->u, conv, s->proj, 2 * di, lw.conv_w, lw.conv_b, B, T, di, dc));
             MRS_TRY(gemm_rm(bb, dt, s->xdbl, xd, s->u, di, lw.x_proj, (int)rows, xd, di));

@@ -133,6 +133,23 @@ class Mamba3Weights:
                                              np.ones(di, np.float32), outw))
         return cls(ipw, np.zeros(dm, np.float32), layers, np.ones(dm, np.float32))
 
+    @classmethod
+    def random_lm(cls, cfg: Mamba3Config, seed: int, std: float = 0.02) -> "Mamba3Weights":
+        """Random-init weights of an LM-shaped backbone (identity input_proj) drawn with numpy's generator -- for
+        benchmarks at sizes where the reference's sequential xorshift initialiser (`init`) would take minutes in
+        Python: projections N(0, std), dt bias inv_softplus(log-uniform[1e-3, 1e-1]), the rest ones as in `init`."""
+        cfg.validate()
+        rng = np.random.default_rng(seed)
+        dm, ds, di, nh, ip = cfg.d_model, cfg.d_state, cfg.d_inner(), cfg.nheads(), cfg.in_proj_out_dim()
+        n = lambda *s: (rng.standard_normal(s, dtype=np.float32) * np.float32(std))
+        layers = []
+        for _ in range(cfg.n_layers):
+            dt = np.exp(rng.uniform(np.log(1e-3), np.log(1e-1), nh))
+            layers.append(Mamba3LayerWeights(np.ones(dm, np.float32), n(dm, ip), np.log(np.expm1(dt)).astype(np.float32),
+                                             np.ones(ds, np.float32), np.ones(ds, np.float32), np.ones((nh, ds), np.float32),
+                                             np.ones((nh, ds), np.float32), np.ones(nh, np.float32), np.ones(di, np.float32), n(di, dm)))
+        return cls(np.zeros(0, np.float32), np.zeros(dm, np.float32), layers, np.ones(dm, np.float32))
+
     def validate(self, cfg: Mamba3Config, input_dim: int) -> None:
         dm, ds, di, nh, ip = cfg.d_model, cfg.d_state, cfg.d_inner(), cfg.nheads(), cfg.in_proj_out_dim()
         if self.input_proj_w.size not in (0, input_dim * dm):
