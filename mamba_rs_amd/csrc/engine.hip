@@ -7,10 +7,14 @@
 // conv/SSM state and every scratch buffer; step() allocates nothing.  The residual
 // stream, states, a_neg, D, biases and norm weights stay f32 (inference.rs:150-165).
 //
-// Per layer the decode chain is 3 library GEMMs and 3 kernels (the reference launches 10
-// kernels + 4 GEMMs, inference.rs:993-1252): residual-add + RMSNorm, in_proj, conv step +
-// SiLU reading the x half of in_proj's output in place, x_proj, one kernel for dt_proj +
-// dt-bias + softplus + state update + B/C gather + SiLU gate, out_proj.
+// Decode, per layer (the reference launches 10 kernels + 4 GEMMs, inference.rs:993-1252):
+//   16-bit storage, batch <= 64: four kernels on the library's own skinny GEMM (gemm_skinny.hip) -- in_proj with the
+//     RMSNorm folded around it and the conv step + SiLU as epilogue, x_proj, one kernel for dt_proj + dt-bias + softplus
+//     + state update + B/C gather + SiLU gate, out_proj with the residual add as epilogue;
+//   otherwise: residual-add + RMSNorm, in_proj (vendor GEMM), conv step + SiLU reading the x half of in_proj's output
+//     in place, x_proj, the fused step kernel, out_proj.
+// Prefill: add + RMSNorm, in_proj, conv over T, x_proj, dt_proj + bias + softplus (one matrix-core kernel for 16-bit
+// storage), the selective scan reading B/C and the raw gate in place, out_proj.
 #include "common.hpp"
 #include <rocblas/rocblas.h>
 #include <stdlib.h>

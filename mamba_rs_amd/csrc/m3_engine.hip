@@ -21,7 +21,6 @@
 namespace mrs {
 
 constexpr float kPi = 3.14159265358979323846f;
-constexpr int kMaxDs = 256;
 
 __device__ __forceinline__ float heavy_tail(float x) { return x >= 0.0f ? 1.0f + x : 1.0f / (1.0f - x); }
 __device__ __forceinline__ float sigmoidf_fast(float x) { return fast_rcp(1.0f + fast_exp2(-x * kLog2e)); }
