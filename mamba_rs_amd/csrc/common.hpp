@@ -101,6 +101,12 @@ int launch_dt_proj_softplus(hipStream_t st, int dtype, void *delta, const void *
 int launch_prenorm_rows(hipStream_t st, int dtype, float *partials, int n_partials, void *prenorm, const float *x, float *copy_to,
                         const float *w, int M, int K);
 
+// mrs_m3_ssd_fwd with x read in place out of wider rows (x_stride elements apart, 0 = dense; 16-bit storage only).
+int m3_ssd_fwd_ex(void *stream, int dtype, float *ssm_state, float *k_state, float *v_state, void *y, const void *x,
+                  int64_t x_stride, const void *K, const void *Q, const float *dt, const float *trap, const float *a_val,
+                  const float *D, void *workspace, size_t workspace_bytes, unsigned flags, int batch, int T, int nheads,
+                  int headdim, int d_state, int chunk_size);
+
 inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s); }
 inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 

@@ -209,19 +209,20 @@ __global__ __launch_bounds__(1024) void m3_angle_scan_kernel(float *__restrict__
     }
 }
 
-// one workgroup (256 threads) per row
+// one workgroup (256 threads) per row.  bulk: rows of ldb elements [z:di | x:di | B:ng*ds | C:ng*ds | ...] in the
+// activation type; xout may be null (x is then read in place by the scan).
 template <typename T>
 __global__ __launch_bounds__(256) void m3_kq_kernel(
-    T *__restrict__ Kout, T *__restrict__ Qout, T *__restrict__ xout, const float *__restrict__ proj, int64_t ip,
+    T *__restrict__ Kout, T *__restrict__ Qout, T *__restrict__ xout, const T *__restrict__ bulk, int64_t ldb,
     const float *__restrict__ angle, const float *__restrict__ bnw, const float *__restrict__ cnw,
     const float *__restrict__ b_bias, const float *__restrict__ c_bias, int nh, int hd, int ng, int ds, int nr, float eps) {
     extern __shared__ float smem[];
     const int di = nh * hd, ngds = ng * ds;
     float *bn = smem, *cn = bn + ngds, *inv = cn + ngds;
     const int64_t r = blockIdx.x;
-    const float *row = proj + r * ip;
+    const T *row = bulk + r * ldb;
     const int tid = threadIdx.x;
-    for (int i = tid; i < ngds; i += 256) { bn[i] = row[2 * di + i]; cn[i] = row[2 * di + ngds + i]; }
+    for (int i = tid; i < ngds; i += 256) { bn[i] = Store<T>::ld(row + 2 * di + i); cn[i] = Store<T>::ld(row + 2 * di + ngds + i); }
     __syncthreads();
     // one wave-sized slice per (B or C, group): 2*ng reductions of ds values
     {
@@ -265,37 +266,30 @@ __global__ __launch_bounds__(256) void m3_kq_kernel(
         *reinterpret_cast<V4 *>(Kout + (r * nh + h) * ds + n) = kv;
         *reinterpret_cast<V4 *>(Qout + (r * nh + h) * ds + n) = qv;
     }
-    if ((di & 3) == 0 && (ip & 3) == 0) {
-        for (int i = tid; i < di / 4; i += 256) {
-            const float4 xv = *reinterpret_cast<const float4 *>(row + di + 4 * i);
-            V4 o;
-            Store<T>::st(&o.v[0], xv.x); Store<T>::st(&o.v[1], xv.y); Store<T>::st(&o.v[2], xv.z); Store<T>::st(&o.v[3], xv.w);
-            *reinterpret_cast<V4 *>(xout + r * di + 4 * i) = o;
-        }
-    } else {
-        for (int i = tid; i < di; i += 256) Store<T>::st(xout + r * di + i, row[di + i]);
-    }
+    if (xout)   // a dense copy of x for scan routes that cannot read it in place
+        for (int i = tid; i < di; i += 256) xout[r * di + i] = row[di + i];
 }
 
-// gated[row, i] = y * silu(z), or RMSNormGated over each head first; one workgroup (256 threads) per row, a wave per head at a time
+// gated[row, i] = y * silu(z), or RMSNormGated over each head first; z = the first d_inner elements of the bulk row.
+// One workgroup (256 threads) per row, a wave per head at a time for the normalised form.
 template <typename T>
-__global__ __launch_bounds__(256) void m3_gate_kernel(T *__restrict__ gated, const T *__restrict__ y, const float *__restrict__ proj,
-                                                      int64_t ip, const float *__restrict__ ngw, int nh, int hd, float eps, int outproj_norm) {
+__global__ __launch_bounds__(256) void m3_gate_kernel(T *__restrict__ gated, const T *__restrict__ y, const T *__restrict__ bulk,
+                                                      int64_t ldb, const float *__restrict__ ngw, int nh, int hd, float eps, int outproj_norm) {
     const int64_t r = blockIdx.x;
     const int di = nh * hd;
-    const float *z = proj + r * ip;
+    const T *z = bulk + r * ldb;
     if (!outproj_norm) {
-        if ((di & 3) == 0 && (ip & 3) == 0) {
+        if ((di & 3) == 0 && (ldb & 3) == 0) {   // four elements per thread and trip
             struct alignas(4 * sizeof(T)) V4 { T v[4]; };
             for (int i = threadIdx.x; i < di / 4; i += 256) {
-                const float4 zv = *reinterpret_cast<const float4 *>(z + 4 * i);
+                const V4 zv = *reinterpret_cast<const V4 *>(z + 4 * i);
                 V4 yv = *reinterpret_cast<const V4 *>(y + r * di + 4 * i);
-                Store<T>::st(&yv.v[0], Store<T>::ld(&yv.v[0]) * silu(zv.x)); Store<T>::st(&yv.v[1], Store<T>::ld(&yv.v[1]) * silu(zv.y));
-                Store<T>::st(&yv.v[2], Store<T>::ld(&yv.v[2]) * silu(zv.z)); Store<T>::st(&yv.v[3], Store<T>::ld(&yv.v[3]) * silu(zv.w));
+#pragma unroll
+                for (int e = 0; e < 4; e++) Store<T>::st(&yv.v[e], Store<T>::ld(&yv.v[e]) * silu(Store<T>::ld(&zv.v[e])));
                 *reinterpret_cast<V4 *>(gated + r * di + 4 * i) = yv;
             }
         } else {
-            for (int i = threadIdx.x; i < di; i += 256) Store<T>::st(gated + r * di + i, Store<T>::ld(y + r * di + i) * silu(z[i]));
+            for (int i = threadIdx.x; i < di; i += 256) Store<T>::st(gated + r * di + i, Store<T>::ld(y + r * di + i) * silu(Store<T>::ld(z + i)));
         }
         return;
     }
@@ -308,7 +302,7 @@ __global__ __launch_bounds__(256) void m3_gate_kernel(T *__restrict__ gated, con
         const float inv = 1.0f / sqrtf(ss / (float)hd + eps);
         for (int p = l; p < hd; p += 64) {
             const int i = h * hd + p;
-            Store<T>::st(gated + r * di + i, Store<T>::ld(y + r * di + i) * inv * ngw[i] * silu(z[i]));
+            Store<T>::st(gated + r * di + i, Store<T>::ld(y + r * di + i) * inv * ngw[i] * silu(Store<T>::ld(z + i)));
         }
     }
 }
@@ -390,7 +384,7 @@ struct mrs_m3_backbone {
     // prefill scratch for sequences of pf_T steps (0: not allocated)
     int pf_T;
     float *pf_in, *pf_residual, *pf_proj, *pf_dt, *pf_a, *pf_trap, *pf_tanhpi, *pf_angle;
-    void *pf_normed, *pf_x, *pf_K, *pf_Q, *pf_y, *pf_gated, *pf_out, *pf_ws;
+    void *pf_normed, *pf_bulk, *pf_x, *pf_K, *pf_Q, *pf_y, *pf_gated, *pf_out, *pf_ws;
     size_t pf_ws_bytes;
 };
 
@@ -686,7 +680,10 @@ extern "C" int mrs_m3_backbone_alloc_prefill_scratch(mrs_m3_backbone *bb, int T)
     const size_t nrz = bb->nr > 0 ? bb->nr : 1;
     MRS_TRY(dev_alloc3(bb, (void **)&bb->pf_in, rows * bb->input_dim * 4));
     MRS_TRY(dev_alloc3(bb, (void **)&bb->pf_residual, rows * dm * 4));
-    MRS_TRY(dev_alloc3(bb, (void **)&bb->pf_proj, rows * ip * 4));
+    // f32 storage: the whole in_proj result; 16-bit: its f32 scalar columns only, the bulk columns live in pf_bulk
+    const size_t nbulk = 2 * di + 2 * (size_t)c.ngroups * ds;
+    MRS_TRY(dev_alloc3(bb, (void **)&bb->pf_proj, rows * (bb->dtype == MRS_F32 ? ip : ip - nbulk) * 4));
+    MRS_TRY(dev_alloc3(bb, &bb->pf_bulk, bb->dtype == MRS_F32 ? 16 : rows * nbulk * es));
     MRS_TRY(dev_alloc3(bb, (void **)&bb->pf_dt, rows * nh * 4));
     MRS_TRY(dev_alloc3(bb, (void **)&bb->pf_a, rows * nh * 4));
     MRS_TRY(dev_alloc3(bb, (void **)&bb->pf_trap, rows * nh * 4));
@@ -711,22 +708,22 @@ extern "C" int mrs_m3_backbone_alloc_prefill_scratch(mrs_m3_backbone *bb, int T)
 namespace {
 
 template <typename T>
-int launch_kq_t(mrs_m3_backbone *bb, const Layer3 &lw, int64_t rows) {
+int launch_kq_t(mrs_m3_backbone *bb, const Layer3 &lw, int64_t rows, const void *bulk, int64_t ldb, bool copy_x) {
     const mrs_m3_config &c = bb->cfg;
     const int ng = c.ngroups, ds = c.d_state;
     const size_t lds = (size_t)(2 * ng * ds + 2 * ng) * sizeof(float);
     if (lds > 60000) return fail(MRS_E_SHAPE, "m3 K/Q kernel: ngroups * d_state too large for LDS (%zu bytes)", lds);
-    hipLaunchKernelGGL((m3_kq_kernel<T>), dim3((unsigned)rows), dim3(256), lds, bb->stream, (T *)bb->pf_K, (T *)bb->pf_Q, (T *)bb->pf_x,
-                       bb->pf_proj, (int64_t)bb->ip, bb->pf_angle, lw.bnw, lw.cnw, lw.b_bias, lw.c_bias, bb->nh, c.headdim, ng, ds, bb->nr,
-                       c.rms_norm_eps);
+    hipLaunchKernelGGL((m3_kq_kernel<T>), dim3((unsigned)rows), dim3(256), lds, bb->stream, (T *)bb->pf_K, (T *)bb->pf_Q,
+                       copy_x ? (T *)bb->pf_x : nullptr, (const T *)bulk, ldb, bb->pf_angle, lw.bnw, lw.cnw, lw.b_bias, lw.c_bias, bb->nh,
+                       c.headdim, ng, ds, bb->nr, c.rms_norm_eps);
     return check_launch("m3_kq_kernel");
 }
 
 template <typename T>
-int launch_gate_t(mrs_m3_backbone *bb, const Layer3 &lw, int64_t rows) {
+int launch_gate_t(mrs_m3_backbone *bb, const Layer3 &lw, int64_t rows, const void *bulk, int64_t ldb) {
     const mrs_m3_config &c = bb->cfg;
-    hipLaunchKernelGGL((m3_gate_kernel<T>), dim3((unsigned)rows), dim3(256), 0, bb->stream, (T *)bb->pf_gated, (const T *)bb->pf_y, bb->pf_proj,
-                       (int64_t)bb->ip, lw.ngw, bb->nh, c.headdim, c.rms_norm_eps, c.is_outproj_norm);
+    hipLaunchKernelGGL((m3_gate_kernel<T>), dim3((unsigned)rows), dim3(256), 0, bb->stream, (T *)bb->pf_gated, (const T *)bb->pf_y,
+                       (const T *)bulk, ldb, lw.ngw, bb->nh, c.headdim, c.rms_norm_eps, c.is_outproj_norm);
     return check_launch("m3_gate_kernel");
 }
 
@@ -766,18 +763,34 @@ int prefill_body3(mrs_m3_backbone *bb, int T) {
         float *ssm = bb->ssm + (size_t)l * B * nh * hd * ds, *kst = bb->kst + (size_t)l * B * nh * ds;
         float *vst = bb->vst + (size_t)l * B * nh * hd, *ang = bb->angle + (size_t)l * B * nh * (nr > 0 ? nr : 1);
         MRS_TRY(launch_add_rmsnorm3(bb, bb->pf_residual, l == 0 ? nullptr : bb->pf_out, bb->pf_normed, false, lw.norm_w, rows));
-        // in_proj with an f32 result: dt, A, trap and the angle inputs keep full precision whatever the storage type
+        // in_proj.  The bulk columns (z, x, B, C) come out in the storage type; the head scalars and angle inputs
+        // (dd_dt, dd_A, trap, angles: the last 3 nh + nr columns) in f32 whatever the storage type -- two GEMMs over
+        // column slices of the same weight for 16-bit storage, one for f32.
+        const int nb = 2 * di + 2 * c.ngroups * ds, ns = ip - nb;
+        const void *bulk; int64_t ldb; const float *scp; int64_t lds_;
         {
             const float one = 1.0f, zero = 0.0f;
             const rocblas_datatype t = blas_type3(dt);
-            MRS_BLAS(rocblas_gemm_ex(bb->blas, rocblas_operation_none, rocblas_operation_none, ip, (int)rows, dm, &one, lw.in_proj, t, ip,
-                                     bb->pf_normed, t, dm, &zero, bb->pf_proj, rocblas_datatype_f32_r, ip, bb->pf_proj, rocblas_datatype_f32_r,
-                                     ip, rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0));
+            if (dt == MRS_F32) {
+                MRS_BLAS(rocblas_gemm_ex(bb->blas, rocblas_operation_none, rocblas_operation_none, ip, (int)rows, dm, &one, lw.in_proj, t, ip,
+                                         bb->pf_normed, t, dm, &zero, bb->pf_proj, t, ip, bb->pf_proj, t, ip, rocblas_datatype_f32_r,
+                                         rocblas_gemm_algo_standard, 0, 0));
+                bulk = bb->pf_proj; ldb = ip; scp = bb->pf_proj + nb; lds_ = ip;
+            } else {
+                MRS_BLAS(rocblas_gemm_ex(bb->blas, rocblas_operation_none, rocblas_operation_none, nb, (int)rows, dm, &one, lw.in_proj, t, ip,
+                                         bb->pf_normed, t, dm, &zero, bb->pf_bulk, t, nb, bb->pf_bulk, t, nb, rocblas_datatype_f32_r,
+                                         rocblas_gemm_algo_standard, 0, 0));
+                MRS_BLAS(rocblas_gemm_ex(bb->blas, rocblas_operation_none, rocblas_operation_none, ns, (int)rows, dm, &one,
+                                         (const char *)lw.in_proj + (size_t)nb * es, t, ip, bb->pf_normed, t, dm, &zero, bb->pf_proj,
+                                         rocblas_datatype_f32_r, ns, bb->pf_proj, rocblas_datatype_f32_r, ns, rocblas_datatype_f32_r,
+                                         rocblas_gemm_algo_standard, 0, 0));
+                bulk = bb->pf_bulk; ldb = nb; scp = bb->pf_proj; lds_ = ns;
+            }
         }
         {
             const int64_t n = rows * (nh + nr);
             hipLaunchKernelGGL(m3_scalars_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, bb->stream, bb->pf_dt, bb->pf_a, bb->pf_trap,
-                               bb->pf_tanhpi, bb->pf_proj, (int64_t)ip, lw.dt_bias, rows, nh, nr, 2 * di + 2 * c.ngroups * ds, c.a_floor);
+                               bb->pf_tanhpi, scp, lds_, lw.dt_bias, rows, nh, nr, 0, c.a_floor);
             MRS_TRY(check_launch("m3_scalars_kernel"));
         }
         if (nr > 0) {
@@ -787,8 +800,16 @@ int prefill_body3(mrs_m3_backbone *bb, int T) {
                                bb->pf_tanhpi, T, nh, nr, nr_pad);
             MRS_TRY(check_launch("m3_angle_scan_kernel"));
         }
-        MRS_DISPATCH_DTYPE(dt, T_, MRS_TRY(launch_kq_t<T_>(bb, lw, rows)));
-        if (chunked_ok) {
+        // the chunked kernel reads x in place out of the bulk rows.  (Folding the SiLU gate into its y store was
+        // measured and dropped: the scattered z reads cost the latency-bound kernel 54 us against 28 us for the
+        // separate gate pass.)
+        const bool in_place = chunked_ok && dt != MRS_F32 && ldb % 8 == 0 && di % 8 == 0;
+        MRS_DISPATCH_DTYPE(dt, T_, MRS_TRY(launch_kq_t<T_>(bb, lw, rows, bulk, ldb, !in_place)));
+        if (in_place) {
+            const char *xb = (const char *)bulk + (size_t)di * es;
+            MRS_TRY(m3_ssd_fwd_ex(bb->stream, dt, ssm, kst, vst, bb->pf_y, xb, ldb, bb->pf_K, bb->pf_Q, bb->pf_dt, bb->pf_trap, bb->pf_a, lw.D,
+                                  bb->pf_ws, bb->pf_ws_bytes, MRS_M3_CARRY_STATE, B, T, nh, hd, ds, 64));
+        } else if (chunked_ok) {
             MRS_TRY(mrs_m3_ssd_fwd(bb->stream, dt, ssm, kst, vst, bb->pf_y, bb->pf_x, bb->pf_K, bb->pf_Q, bb->pf_dt, bb->pf_trap, bb->pf_a, lw.D,
                                    bb->pf_ws, bb->pf_ws_bytes, MRS_M3_CARRY_STATE, B, T, nh, hd, ds, 64));
         } else {
@@ -796,7 +817,7 @@ int prefill_body3(mrs_m3_backbone *bb, int T) {
             MRS_TRY(mrs_m3_compute_abg(bb->stream, al, be, ga, bb->pf_dt, bb->pf_a, bb->pf_trap, rows * nh));
             MRS_TRY(mrs_m3_seq_fwd(bb->stream, dt, ssm, kst, vst, bb->pf_y, bb->pf_x, bb->pf_K, bb->pf_Q, al, be, ga, lw.D, B, T, nh, hd, ds));
         }
-        MRS_DISPATCH_DTYPE(dt, T_, MRS_TRY(launch_gate_t<T_>(bb, lw, rows)));
+        MRS_DISPATCH_DTYPE(dt, T_, MRS_TRY(launch_gate_t<T_>(bb, lw, rows, bulk, ldb)));
         MRS_TRY(gemm3(bb, bb->pf_out, false, bb->pf_gated, lw.out_proj, (int)rows, dm, di));
     }
     // only the last position of each sequence is kept: final residual add + norm_f on those rows

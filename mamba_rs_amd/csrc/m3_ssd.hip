@@ -90,6 +90,8 @@ struct SsdSplit {
     float *dAtot;   // [batch*nh][nsc-1]          sum of a*dt over super-chunk k
     float *Sinit;   // [batch*nh][HD][DS]         the carried-in state, saved before the last super-chunk overwrites ssm
     int nsc, cps;
+    // engine-only extra: x rows may sit inside wider rows (read in place from a projection)
+    int64_t x_stride;     // elements between consecutive rows of x (d_inner for a dense x)
 };
 
 template <typename T, int HD, int DS, bool STATE_ONLY>
@@ -181,7 +183,7 @@ __global__ __launch_bounds__(HD * 4) void m3_ssd_kernel(
         }
         const int t = t0 + l;  // lane = step
         if (t < Tlen) {
-            const int64_t xo = ((int64_t)b * Tlen + t) * di + h * HD + 16 * w;
+            const int64_t xo = ((int64_t)b * Tlen + t) * sp.x_stride + h * HD + 16 * w;
             rx[0] = *reinterpret_cast<const uint4 *>(x + xo);
             rx[1] = *reinterpret_cast<const uint4 *>(x + xo + 8);
             const int64_t so = ((int64_t)b * Tlen + t) * nh + h;
@@ -354,7 +356,7 @@ __global__ __launch_bounds__(HD * 4) void m3_ssd_kernel(
         *reinterpret_cast<float4 *>(ssm + srow + 16 * jn) = make_float4(St[jn][0], St[jn][1], St[jn][2], St[jn][3]);
     const int64_t last = (int64_t)b * Tlen + (Tlen - 1);
     for (int n = tid; n < DS; n += NTHR) kst[bh * DS + n] = Store<T>::ld(K + (last * nh + h) * DS + n);
-    for (int p = tid; p < HD; p += NTHR) vst[bh * HD + p] = Store<T>::ld(x + last * di + h * HD + p);
+    for (int p = tid; p < HD; p += NTHR) vst[bh * HD + p] = Store<T>::ld(x + last * sp.x_stride + h * HD + p);
 }
 
 __global__ void m3_abg_kernel(float *__restrict__ alpha, float *__restrict__ beta, float *__restrict__ gamma,
@@ -457,7 +459,21 @@ extern "C" int mrs_m3_ssd_fwd(void *stream, int dtype, float *ssm_state, float *
                               const float *a_val, const float *D, void *workspace, size_t workspace_bytes,
                               unsigned flags, int batch, int T, int nheads, int headdim, int d_state,
                               int chunk_size) {
+    return mrs::m3_ssd_fwd_ex(stream, dtype, ssm_state, k_state, v_state, y, x, 0, K, Q, dt, trap, a_val, D, workspace,
+                              workspace_bytes, flags, batch, T, nheads, headdim, d_state, chunk_size);
+}
+
+// x_stride = 0 means dense rows (d_inner); a wider stride needs 16-bit storage (the f32 route runs the recurrence kernel).
+int mrs::m3_ssd_fwd_ex(void *stream, int dtype, float *ssm_state, float *k_state, float *v_state, void *y, const void *x,
+                       int64_t x_stride, const void *K, const void *Q, const float *dt,
+                       const float *trap, const float *a_val, const float *D, void *workspace, size_t workspace_bytes,
+                       unsigned flags, int batch, int T, int nheads, int headdim, int d_state, int chunk_size) {
     const char *fn = "mrs_m3_ssd_fwd";
+    const int64_t di_ = (int64_t)nheads * headdim;
+    if (x_stride == 0) x_stride = di_;
+    if (x_stride < di_) return fail(MRS_E_SHAPE, "%s: row stride below d_inner", fn);
+    if (dtype == MRS_F32 && x_stride != di_) return fail(MRS_E_SHAPE, "%s: strided x needs 16-bit storage", fn);
+    if (x_stride % 8 != 0) return fail(MRS_E_ALIGN, "%s: x row stride must be a multiple of 8 elements", fn);
     if (dtype != MRS_F32 && dtype != MRS_F16 && dtype != MRS_BF16) return fail(MRS_E_DTYPE, "%s: dtype %d is not f32/f16/bf16", fn, dtype);
     if (!ssm_state || !k_state || !v_state || !y || !x || !K || !Q || !dt || !trap || !a_val || !D)
         return fail(MRS_E_NULL, "%s: null pointer", fn);
@@ -489,7 +505,7 @@ extern "C" int mrs_m3_ssd_fwd(void *stream, int dtype, float *ssm_state, float *
     if (!aligned(x, 16) || !aligned(K, 16) || !aligned(Q, 16) || !aligned(ssm_state, 16) || !aligned(k_state, 16))
         return fail(MRS_E_ALIGN, "%s: x, K, Q, ssm_state, k_state must be 16-byte aligned", fn);
     // Super-chunk split when the caller's workspace holds it; otherwise one workgroup walks the whole sequence.
-    SsdSplit sp = {nullptr, nullptr, nullptr, 1, (T + kCS - 1) / kCS};
+    SsdSplit sp = {nullptr, nullptr, nullptr, 1, (T + kCS - 1) / kCS, x_stride};
     {
         int nsc, cps;
         ssd_plan(batch, T, nheads, nsc, cps);
@@ -497,7 +513,7 @@ extern "C" int mrs_m3_ssd_fwd(void *stream, int dtype, float *ssm_state, float *
         const size_t need = ssd_split_bytes(batch, nheads, headdim, d_state, nsc, &o_dA, &o_init);
         if (nsc > 1 && workspace && workspace_bytes >= need && aligned(workspace, 16)) {
             char *ws = (char *)workspace;
-            sp = SsdSplit{(float *)ws, (float *)(ws + o_dA), (float *)(ws + o_init), nsc, cps};
+            sp = SsdSplit{(float *)ws, (float *)(ws + o_dA), (float *)(ws + o_init), nsc, cps, x_stride};
         }
     }
     if (dtype == MRS_BF16) return launch_ssd<bf16_t>(st, ssm_state, k_state, v_state, y, x, K, Q, dt, trap, a_val, D, sp, batch, T, nheads, headdim, d_state, carry);
