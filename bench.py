@@ -199,7 +199,22 @@ def m1_kernels_leg():
             ops.ssm_step_gather_gate(h, y, delta, uu, xdbl, gate, a_neg, D, dr, dr + ds)
     us_step = timeit(gr.replay, 30) / 24
     step_bytes = 2 * 4 * Bd * di * ds + 4 * Bd * di * 2 + 4 * di * ds
-    return {"conv1d_seq_silu": {"batch": B, "seq_len": T, "us": us_conv, "algorithmic_bytes": conv_bytes,
+    # the headline scan once more per storage type (the reference ships f32, bf16 and f16 variants of the kernel),
+    # and without the S4D-real shortcut (a general A: 16 exponentials per step instead of one)
+    scan = {}
+    inp = make_inputs(B, T, di, ds)
+    tt = {k: torch.from_numpy(v).to(dev) for k, v in inp.items()}
+    ws = torch.empty(ops.ssm_scan_workspace_bytes(B, T, di, ds), dtype=torch.uint8, device=dev)
+    hs = torch.zeros(B, di, ds, device=dev)
+    for name, tdt, esz, fl in (("f32", torch.float32, 4, ops.A_S4D_REAL), ("f16", torch.float16, 2, ops.A_S4D_REAL),
+                               ("bf16_general_A", bf, 2, 0)):
+        dl, uu_, zz, Bm, Cm = (tt[k].to(tdt) for k in ("delta", "u", "z", "B", "C"))
+        yy = torch.empty_like(dl)
+        us_s = timeit(lambda: ops.ssm_scan_fwd(hs, yy, dl, uu_, Bm, Cm, tt["a_neg"], tt["D"], gate=zz, flags=ops.GATE_SILU | fl, workspace=ws), 20)
+        nb = scan_algorithmic_bytes(B, T, di, ds, esz, gated=True)
+        scan[name] = {"us": us_s, "algorithmic_bytes": nb, "GBps": nb / us_s / 1e3, "hbm_frac": nb / us_s / 1e3 / HBM_PEAK_GBPS}
+    return {"selective_scan_other_storage": scan,
+            "conv1d_seq_silu": {"batch": B, "seq_len": T, "us": us_conv, "algorithmic_bytes": conv_bytes,
                                 "GBps": conv_bytes / us_conv / 1e3, "hbm_frac": conv_bytes / us_conv / 1e3 / HBM_PEAK_GBPS},
             "ssm_step_gather_gate_b64": {"us_per_call_in_graph": us_step, "algorithmic_bytes": step_bytes,
                                          "GBps": step_bytes / us_step / 1e3, "hbm_frac": step_bytes / us_step / 1e3 / HBM_PEAK_GBPS}}
