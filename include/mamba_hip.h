@@ -320,7 +320,7 @@ typedef struct {            /* Mamba3Weights */
     const float *norm_f_weight; /* [d_model] */
 } mrs_m3_weights;
 
-/* headdim * d_state / 4 <= 1024 and d_state = 4 x a power of two <= 256 (the reference stops at headdim 32). */
+/* d_state = 4 x a power of two <= 256 and headdim * d_state / 4 a multiple of 64, <= 1024 (the reference stops at headdim 32). */
 MRS_API int mrs_m3_backbone_create(mrs_m3_backbone **out, int gpu_ordinal, const mrs_m3_weights *weights,
                                    const mrs_m3_config *cfg, int input_dim, int batch, int dtype);
 MRS_API void mrs_m3_backbone_destroy(mrs_m3_backbone *bb);

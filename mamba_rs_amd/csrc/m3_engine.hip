@@ -184,9 +184,22 @@ __global__ __launch_bounds__(1024) void m3_angle_scan_kernel(float *__restrict__
     const bool live = a < nr;
     const float *dp = dt + (int64_t)b * Tlen * nh + h;
     const float *tp = tanhpi + (int64_t)b * Tlen * nr + a;
+    // the per-step increments of this thread's segment, staged in registers in groups of 8 so that the loads of a
+    // group are in flight together (the running sum itself is a dependent chain)
     double sum = 0.0;
-    if (live)
-        for (int t = t0; t < t1; t++) sum += (double)(tp[(int64_t)t * nr] * dp[(int64_t)t * nh]);
+    if (live) {
+        for (int tg = t0; tg < t1; tg += 8) {
+            float d[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const int t = min(tg + j, t1 - 1);
+                d[j] = tp[(int64_t)t * nr] * dp[(int64_t)t * nh];
+            }
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+                if (tg + j < t1) sum += (double)d[j];
+        }
+    }
     part[seg * nr_pad + a] = sum;
     __syncthreads();
     if (seg == 0 && live) {
@@ -202,9 +215,20 @@ __global__ __launch_bounds__(1024) void m3_angle_scan_kernel(float *__restrict__
     __syncthreads();
     if (live) {
         double acc = part[seg * nr_pad + a];
-        for (int t = t0; t < t1; t++) {
-            acc = wrap_2pi(acc + (double)(tp[(int64_t)t * nr] * dp[(int64_t)t * nh]));
-            angle_out[(((int64_t)b * Tlen + t) * nh + h) * nr + a] = (float)acc;
+        for (int tg = t0; tg < t1; tg += 8) {
+            float d[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const int t = min(tg + j, t1 - 1);
+                d[j] = tp[(int64_t)t * nr] * dp[(int64_t)t * nh];
+            }
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                if (tg + j < t1) {
+                    acc = wrap_2pi(acc + (double)d[j]);
+                    angle_out[(((int64_t)b * Tlen + tg + j) * nh + h) * nr + a] = (float)acc;
+                }
+            }
         }
     }
 }
@@ -529,8 +553,9 @@ extern "C" int mrs_m3_backbone_create(mrs_m3_backbone **out, int gpu_ordinal, co
     const int nh = (int)(di64 / cfg->headdim);
     if (nh % cfg->ngroups != 0) return fail(MRS_E_SHAPE, "%s: nheads %d is not a multiple of ngroups %d", fn, nh, cfg->ngroups);
     const int ds = cfg->d_state, lg = ds / 4;
-    if (ds % 4 != 0 || (lg & (lg - 1)) != 0 || lg > 64 || (int64_t)cfg->headdim * lg > 1024)
-        return fail(MRS_E_SHAPE, "%s: d_state must be 4 x a power of two <= 256 and headdim * d_state / 4 <= 1024 (got %d, %d)", fn, ds, cfg->headdim);
+    // one lane per four states of a row: a workgroup of headdim * d_state / 4 lanes, whole waves only
+    if (ds % 4 != 0 || (lg & (lg - 1)) != 0 || lg > 64 || (int64_t)cfg->headdim * lg > 1024 || ((int64_t)cfg->headdim * lg) % 64 != 0)
+        return fail(MRS_E_SHAPE, "%s: d_state must be 4 x a power of two <= 256 and headdim * d_state / 4 a multiple of 64 <= 1024 (got %d, %d)", fn, ds, cfg->headdim);
     if (cfg->n_rope_angles < 0 || 2 * cfg->n_rope_angles > ds) return fail(MRS_E_SHAPE, "%s: n_rope_angles %d outside 0..d_state/2", fn, cfg->n_rope_angles);
     if (!(cfg->a_floor > 0.0f)) return fail(MRS_E_SHAPE, "%s: a_floor must be > 0", fn);
     if (batch < 1 || input_dim < 1 || di64 > 65535 || cfg->n_layers > 4096) return fail(MRS_E_SHAPE, "%s: batch=%d input_dim=%d d_inner=%lld", fn, batch, input_dim, (long long)di64);

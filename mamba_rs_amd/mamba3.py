@@ -55,8 +55,8 @@ class Mamba3Config:
         if self.nheads() % self.ngroups:
             raise ValueError("nheads must be a multiple of ngroups")
         lg = self.d_state // 4
-        if self.d_state % 4 or lg & (lg - 1) or lg > 64 or self.headdim * lg > 1024:
-            raise ValueError("d_state must be 4 x a power of two <= 256 and headdim * d_state / 4 <= 1024")
+        if self.d_state % 4 or lg & (lg - 1) or lg > 64 or self.headdim * lg > 1024 or (self.headdim * lg) % 64:
+            raise ValueError("d_state must be 4 x a power of two <= 256 and headdim * d_state / 4 a multiple of 64 <= 1024")
         if not (self.rope_fraction == 0.5 or self.rope_fraction == 1.0):
             raise ValueError("rope_fraction must be 0.5 or 1.0")
         if not self.a_floor > 0:
