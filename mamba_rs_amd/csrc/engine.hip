@@ -346,6 +346,16 @@ static int gemm_rm(mrs_backbone *bb, int dtype, void *C, int ldc, const void *A,
     return MRS_OK;
 }
 
+// The same product from the transposed copy Wt[N,K] (kept for the decode chain): the vendor kernels for this operand
+// order are faster at the prefill shapes (76 vs 84-92 us for in_proj at 16384 x 3072 x 768).
+static int gemm_rm_t(mrs_backbone *bb, int dtype, void *C, int ldc, const void *A, int lda, const void *Wt, int M, int N, int K) {
+    const float one = 1.0f, zero = 0.0f;
+    const rocblas_datatype t = blas_type(dtype);
+    MRS_BLAS(rocblas_gemm_ex(bb->blas, rocblas_operation_transpose, rocblas_operation_none, N, M, K, &one, Wt, t, K, A, t, lda,
+                             &zero, C, t, ldc, C, t, ldc, rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0));
+    return MRS_OK;
+}
+
 template <typename T>
 static void launch_add_rmsnorm_t(mrs_backbone *bb, float *residual, const void *add, void *out, bool out_f32,
                                  const float *w, int64_t rows, int64_t out_stride, void *out2) {
@@ -438,7 +448,8 @@ static int run_layers(mrs_backbone *bb, Scratch *s, int T) {
             continue;
         }
         MRS_TRY(launch_add_rmsnorm(bb, s->residual, l == 0 ? nullptr : s->out, s->normed, false, lw.norm_w, rows, dm));
-        MRS_TRY(gemm_rm(bb, dt, s->proj, 2 * di, s->normed, dm, lw.in_proj, (int)rows, 2 * di, dm));
+        if (T > 1 && lw.in_proj_t) MRS_TRY(gemm_rm_t(bb, dt, s->proj, 2 * di, s->normed, dm, lw.in_proj_t, (int)rows, 2 * di, dm));
+        else MRS_TRY(gemm_rm(bb, dt, s->proj, 2 * di, s->normed, dm, lw.in_proj, (int)rows, 2 * di, dm));
         if (T == 1) {
             MRS_TRY(launch_conv1d_step(bb->stream, dt, s->u, conv, s->proj, 2 * di, lw.conv_w, lw.conv_b, B, di, dc, 1));
             MRS_TRY(gemm_rm(bb, dt, s->xdbl, xd, s->u, di, lw.x_proj, (int)rows, xd, di));
@@ -479,7 +490,8 @@ static int run_layers(mrs_backbone *bb, Scratch *s, int T) {
             MRS_TRY(mrs_ssm_scan_fwd_ex(bb->stream, dt, ssm, s->y, s->delta, s->u, xb + es * dr, xb + es * (dr + ds), xd, lw.a_neg,
                                         lw.D, z, 2 * di, flags, s->scan_ws, s->scan_ws_bytes, B, T, di, ds));
         }
-        MRS_TRY(gemm_rm(bb, dt, s->out, dm, s->y, di, lw.out_proj, (int)rows, dm, di));
+        if (T > 1 && lw.out_proj_t) MRS_TRY(gemm_rm_t(bb, dt, s->out, dm, s->y, di, lw.out_proj_t, (int)rows, dm, di));
+        else MRS_TRY(gemm_rm(bb, dt, s->out, dm, s->y, di, lw.out_proj, (int)rows, dm, di));
     }
     if (T == 1) {
         // (the out_proj epilogue of the own-GEMM chain has already added the last layer's output)
