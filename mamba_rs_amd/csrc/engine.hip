@@ -16,6 +16,7 @@
 // Prefill: add + RMSNorm, in_proj, conv over T, x_proj, dt_proj + bias + softplus (one matrix-core kernel for 16-bit
 // storage), the selective scan reading B/C and the raw gate in place, out_proj.
 #include "common.hpp"
+#include "glue.hpp"
 #include <rocblas/rocblas.h>
 #include <stdlib.h>
 #include <new>
@@ -46,44 +47,6 @@ static rocblas_datatype blas_type(int dtype) {
 
 // ---- glue kernels -------------------------------------------------------------------
 
-// One workgroup per row: residual (f32) += add (storage dtype, may be null); out = rmsnorm(residual) * w.
-// Reference: residual_add_f32_* + rmsnorm_forward_f32in_* (kernels/elementwise.cu:366-376,
-// kernels/norms.cu:21-171), with its finite guard: rms = 1 if not finite or < 1e-20 (norms.cu:58-61).
-// out2 (may be null): the same result once more in the storage type (the LM head's operand).
-template <typename T, typename TO>
-__global__ __launch_bounds__(256) void add_rmsnorm_kernel(float *__restrict__ residual, const T *__restrict__ add,
-                                                          TO *__restrict__ out, T *__restrict__ out2, const float *__restrict__ w,
-                                                          float eps, int64_t rows, int dm, int64_t out_stride) {
-    constexpr int kMaxPer = 16;  // elements per thread kept in registers (d_model <= 4096); longer rows re-read
-    __shared__ float part[4];
-    const int64_t row = blockIdx.x;
-    float *r = residual + row * dm;
-    float v[kMaxPer];
-    float ss = 0.0f;
-    int cnt = 0;
-    for (int i = threadIdx.x; i < dm; i += 256, cnt++) {
-        float x = r[i];
-        if (add) { x += Store<T>::ld(add + row * dm + i); r[i] = x; }
-        if (cnt < kMaxPer) v[cnt] = x;
-        ss = fmaf(x, x, ss);
-    }
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) ss += __shfl_xor(ss, m, kWave);
-    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
-    __syncthreads();
-    ss = part[0] + part[1] + part[2] + part[3];
-    float rms = sqrtf(ss / (float)dm + eps);
-    if (!isfinite(rms) || rms < 1e-20f) rms = 1.0f;
-    const float inv = 1.0f / rms;
-    cnt = 0;
-    for (int i = threadIdx.x; i < dm; i += 256, cnt++) {
-        const float x = cnt < kMaxPer ? v[cnt] : r[i];
-        const float o = x * inv * w[i];
-        Store<TO>::st(out + row * out_stride + i, o);
-        if (out2) Store<T>::st(out2 + row * out_stride + i, o);
-    }
-}
-
 // delta = softplus(raw + bias[d]) in place (dt_proj bias + softplus_forward, kernels/activations.cu:32-52).
 // VEC elements per thread as one 16-byte access (VEC = 16 / sizeof(T), d_inner % VEC == 0), or one by one.
 template <typename T, int VEC>
@@ -107,80 +70,6 @@ __global__ __launch_bounds__(256) void bias_softplus_kernel(T *__restrict__ x, c
 #pragma unroll
     for (int j = 0; j < VEC; j++) Store<T>::st(&t.v[j], softplus20(Store<T>::ld(&t.v[j]) + bv[j]));
     *reinterpret_cast<V *>(x + i) = t;
-}
-
-// Prefill-sized rows: one wave per row, 4 elements per lane and trip (16-byte residual accesses), the row
-// kept in registers between the sum of squares and the scaling.  Same arithmetic as add_rmsnorm_kernel.
-template <typename T, typename TO>
-__global__ __launch_bounds__(256) void add_rmsnorm_rows_kernel(float *__restrict__ residual, const T *__restrict__ add,
-                                                               TO *__restrict__ out, const float *__restrict__ w,
-                                                               float eps, int64_t rows, int dm) {
-    constexpr int kMaxTrips = 16;  // d_model <= 4096 stays in registers; longer rows re-read
-    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (row >= rows) return;
-    const int lane = threadIdx.x & 63;
-    const int nv = dm >> 2;
-    float4 *r4 = reinterpret_cast<float4 *>(residual + row * dm);
-    struct alignas(4 * sizeof(T)) V4 { T v[4]; };
-    struct alignas(4 * sizeof(TO)) O4 { TO v[4]; };
-    const V4 *a4 = reinterpret_cast<const V4 *>(add ? add + row * dm : nullptr);
-    float4 v[kMaxTrips];
-    float ss = 0.0f;
-    int cnt = 0;
-    for (int c0 = lane; c0 < nv; c0 += 4 * 64) {
-        // four trips at a time, every load issued before the first use
-        float4 x[4];
-        V4 a[4];
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const int c = c0 + 64 * j;
-            if (c < nv) {
-                x[j] = r4[c];
-                if (add) a[j] = a4[c];
-            }
-        }
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const int c = c0 + 64 * j;
-            if (c < nv) {
-                if (add) {
-                    x[j].x += Store<T>::ld(&a[j].v[0]); x[j].y += Store<T>::ld(&a[j].v[1]);
-                    x[j].z += Store<T>::ld(&a[j].v[2]); x[j].w += Store<T>::ld(&a[j].v[3]);
-                    r4[c] = x[j];
-                }
-                if (cnt < kMaxTrips) v[cnt] = x[j];
-                cnt++;
-                ss = fmaf(x[j].x, x[j].x, ss); ss = fmaf(x[j].y, x[j].y, ss); ss = fmaf(x[j].z, x[j].z, ss); ss = fmaf(x[j].w, x[j].w, ss);
-            }
-        }
-    }
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) ss += __shfl_xor(ss, m, kWave);
-    float rms = sqrtf(ss / (float)dm + eps);
-    if (!isfinite(rms) || rms < 1e-20f) rms = 1.0f;
-    const float inv = 1.0f / rms;
-    O4 *o4 = reinterpret_cast<O4 *>(out + row * dm);
-    const float4 *w4 = reinterpret_cast<const float4 *>(w);
-    cnt = 0;
-    for (int c = lane; c < nv; c += 64, cnt++) {
-        const float4 x = cnt < kMaxTrips ? v[cnt] : r4[c];
-        const float4 ww = w4[c];
-        O4 o;
-        Store<TO>::st(&o.v[0], x.x * inv * ww.x); Store<TO>::st(&o.v[1], x.y * inv * ww.y);
-        Store<TO>::st(&o.v[2], x.z * inv * ww.z); Store<TO>::st(&o.v[3], x.w * inv * ww.w);
-        o4[c] = o;
-    }
-}
-
-template <typename T>
-__global__ __launch_bounds__(256) void cast_from_f32_kernel(T *__restrict__ out, const float *__restrict__ in, int64_t n) {
-    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) Store<T>::st(out + i, in[i]);
-}
-
-__global__ __launch_bounds__(256) void bias_rows_kernel(float *__restrict__ out, const float *__restrict__ bias, int64_t n, int dm) {
-    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) out[i] = bias[i % dm];
 }
 
 __global__ __launch_bounds__(256) void exp_negate_k(float *__restrict__ a_neg, const float *__restrict__ a_log, int64_t n) {
@@ -356,26 +245,10 @@ static int gemm_rm_t(mrs_backbone *bb, int dtype, void *C, int ldc, const void *
     return MRS_OK;
 }
 
-template <typename T>
-static void launch_add_rmsnorm_t(mrs_backbone *bb, float *residual, const void *add, void *out, bool out_f32,
-                                 const float *w, int64_t rows, int64_t out_stride, void *out2) {
-    const dim3 grid((unsigned)rows), block(256);
-    if (rows >= 256 && bb->cfg.d_model % 4 == 0 && out_stride == bb->cfg.d_model && !out2 && !out_f32) {
-        hipLaunchKernelGGL((add_rmsnorm_rows_kernel<T, T>), dim3((unsigned)((rows + 3) / 4)), block, 0, bb->stream, residual, (const T *)add,
-                           (T *)out, w, bb->cfg.rms_norm_eps, rows, bb->cfg.d_model);
-        return;
-    }
-    if (out_f32)
-        hipLaunchKernelGGL((add_rmsnorm_kernel<T, float>), grid, block, 0, bb->stream, residual, (const T *)add, (float *)out, (T *)out2, w,
-                           bb->cfg.rms_norm_eps, rows, bb->cfg.d_model, out_stride);
-    else
-        hipLaunchKernelGGL((add_rmsnorm_kernel<T, T>), grid, block, 0, bb->stream, residual, (const T *)add, (T *)out, (T *)out2, w,
-                           bb->cfg.rms_norm_eps, rows, bb->cfg.d_model, out_stride);
-}
 static int launch_add_rmsnorm(mrs_backbone *bb, float *residual, const void *add, void *out, bool out_f32, const float *w,
                               int64_t rows, int64_t out_stride, void *out2 = nullptr) {
-    MRS_DISPATCH_DTYPE(bb->dtype, T_, launch_add_rmsnorm_t<T_>(bb, residual, add, out, out_f32, w, rows, out_stride, out2));
-    return check_launch("add_rmsnorm_kernel");
+    return launch_add_rmsnorm_any(bb->stream, bb->dtype, residual, add, out, out_f32, out2, w, bb->cfg.rms_norm_eps, rows, bb->cfg.d_model,
+                                  out_stride);
 }
 
 // residual <- input (identity) or input . input_proj_w + b (f32 GEMM)

@@ -14,6 +14,7 @@
 //   3. out_proj with the residual add, the next layer's pre-scaled operand and row sums of squares as epilogue.
 // f32 storage (or shapes the skinny GEMM does not take) runs RMSNorm + rocBLAS GEMMs around the same step kernel.
 #include "common.hpp"
+#include "glue.hpp"
 #include <rocblas/rocblas.h>
 #include <new>
 #include <vector>
@@ -348,41 +349,6 @@ inline rocblas_datatype blas_type3(int dtype) {
     return dtype == MRS_F32 ? rocblas_datatype_f32_r : dtype == MRS_F16 ? rocblas_datatype_f16_r : rocblas_datatype_bf16_r;
 }
 
-template <typename T>
-__global__ __launch_bounds__(256) void cast3_kernel(T *__restrict__ out, const float *__restrict__ in, int64_t n) {
-    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) Store<T>::st(out + i, in[i]);
-}
-
-// One workgroup per row: residual (f32) += add (may be null); out = rmsnorm(residual) * w in the activation type or f32.
-template <typename T, typename TO>
-__global__ __launch_bounds__(256) void add_rmsnorm3_kernel(float *__restrict__ residual, const T *__restrict__ add, TO *__restrict__ out,
-                                                           const float *__restrict__ w, float eps, int dm) {
-    __shared__ float part[4];
-    const int64_t row = blockIdx.x;
-    float *r = residual + row * dm;
-    float ss = 0.0f;
-    for (int i = threadIdx.x; i < dm; i += 256) {
-        float x = r[i];
-        if (add) { x += Store<T>::ld(add + row * dm + i); r[i] = x; }
-        ss = fmaf(x, x, ss);
-    }
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) ss += __shfl_xor(ss, m, kWave);
-    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
-    __syncthreads();
-    ss = part[0] + part[1] + part[2] + part[3];
-    float rms = sqrtf(ss / (float)dm + eps);
-    if (!isfinite(rms) || rms < 1e-20f) rms = 1.0f;
-    const float inv = 1.0f / rms;
-    for (int i = threadIdx.x; i < dm; i += 256) Store<TO>::st(out + row * dm + i, r[i] * inv * w[i]);
-}
-
-__global__ void bias_rows3_kernel(float *__restrict__ out, const float *__restrict__ bias, int64_t n, int dm) {
-    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) out[i] = bias ? bias[i % dm] : 0.0f;
-}
-
 struct Layer3 {
     float *norm_w, *dt_bias, *bnw, *cnw, *b_bias, *c_bias, *D, *ngw;
     void *in_proj, *out_proj;      // [K][N] storage type (library GEMM)
@@ -430,8 +396,8 @@ int upload_bulk3(mrs_m3_backbone *bb, void **dst, const float *src, size_t n, fl
     MRS_TRY(dev_alloc3(bb, dst, n * esize3(bb->dtype)));
     const dim3 grid((unsigned)((n + 255) / 256)), block(256);
     if (bb->dtype == MRS_F32) MRS_HIP(hipMemcpyAsync(*dst, stage, n * 4, hipMemcpyDeviceToDevice, bb->stream));
-    else if (bb->dtype == MRS_BF16) hipLaunchKernelGGL((cast3_kernel<bf16_t>), grid, block, 0, bb->stream, (bf16_t *)*dst, stage, (int64_t)n);
-    else hipLaunchKernelGGL((cast3_kernel<f16_t>), grid, block, 0, bb->stream, (f16_t *)*dst, stage, (int64_t)n);
+    else if (bb->dtype == MRS_BF16) hipLaunchKernelGGL((cast_from_f32_kernel<bf16_t>), grid, block, 0, bb->stream, (bf16_t *)*dst, stage, (int64_t)n);
+    else hipLaunchKernelGGL((cast_from_f32_kernel<f16_t>), grid, block, 0, bb->stream, (f16_t *)*dst, stage, (int64_t)n);
     MRS_HIP(hipStreamSynchronize(bb->stream));
     return check_launch("weight cast");
 }
@@ -475,7 +441,7 @@ int step_body3(mrs_m3_backbone *bb) {
         else MRS_HIP(hipMemcpyAsync(bb->residual, bb->d_input, (size_t)B * dm * 4, hipMemcpyDeviceToDevice, bb->stream));
     } else {
         const int64_t n = (int64_t)B * dm;
-        hipLaunchKernelGGL(bias_rows3_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, bb->stream, bb->residual, bb->input_proj_b, n, dm);
+        hipLaunchKernelGGL(bias_rows_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, bb->stream, bb->residual, bb->input_proj_b, n, dm);
         const float one = 1.0f;
         MRS_BLAS(rocblas_gemm_ex(bb->blas, rocblas_operation_none, rocblas_operation_none, dm, B, bb->input_dim, &one, bb->input_proj_w,
                                  rocblas_datatype_f32_r, dm, bb->d_input, rocblas_datatype_f32_r, bb->input_dim, &one, bb->residual,
@@ -492,10 +458,8 @@ int step_body3(mrs_m3_backbone *bb) {
             inp.row_scale = 1; inp.partials = bb->partials; inp.n_partials = P; inp.eps = c.rms_norm_eps;
             MRS_TRY(launch_skinny_gemm(bb->stream, dt, bb->proj, 1, ip, bb->normed, dm, lw.in_proj_t, B, ip, dm, inp));
         } else {
-            if (dt == MRS_F32) hipLaunchKernelGGL((add_rmsnorm3_kernel<float, float>), dim3((unsigned)B), dim3(256), 0, bb->stream, bb->residual, l == 0 ? nullptr : (const float *)bb->out, (float *)bb->normed, lw.norm_w, c.rms_norm_eps, dm);
-            else if (dt == MRS_BF16) hipLaunchKernelGGL((add_rmsnorm3_kernel<bf16_t, bf16_t>), dim3((unsigned)B), dim3(256), 0, bb->stream, bb->residual, l == 0 ? nullptr : (const bf16_t *)bb->out, (bf16_t *)bb->normed, lw.norm_w, c.rms_norm_eps, dm);
-            else hipLaunchKernelGGL((add_rmsnorm3_kernel<f16_t, f16_t>), dim3((unsigned)B), dim3(256), 0, bb->stream, bb->residual, l == 0 ? nullptr : (const f16_t *)bb->out, (f16_t *)bb->normed, lw.norm_w, c.rms_norm_eps, dm);
-            MRS_TRY(check_launch("add_rmsnorm3_kernel"));
+            MRS_TRY(launch_add_rmsnorm_any(bb->stream, dt, bb->residual, l == 0 ? nullptr : bb->out, bb->normed, false, nullptr, lw.norm_w,
+                                           c.rms_norm_eps, B, dm, dm));
             MRS_TRY(gemm3(bb, bb->proj, true, bb->normed, lw.in_proj, B, ip, dm));
         }
         MRS_DISPATCH_DTYPE(dt, T_, MRS_TRY(launch_layer_step_t<T_>(bb, l)));
@@ -509,11 +473,8 @@ int step_body3(mrs_m3_backbone *bb) {
         }
     }
     // final residual add (library chain) + norm_f -> temporal (f32)
-    const void *add = bb->skinny ? nullptr : bb->out;
-    if (dt == MRS_F32) hipLaunchKernelGGL((add_rmsnorm3_kernel<float, float>), dim3((unsigned)B), dim3(256), 0, bb->stream, bb->residual, (const float *)add, bb->temporal, bb->norm_f, c.rms_norm_eps, dm);
-    else if (dt == MRS_BF16) hipLaunchKernelGGL((add_rmsnorm3_kernel<bf16_t, float>), dim3((unsigned)B), dim3(256), 0, bb->stream, bb->residual, (const bf16_t *)add, bb->temporal, bb->norm_f, c.rms_norm_eps, dm);
-    else hipLaunchKernelGGL((add_rmsnorm3_kernel<f16_t, float>), dim3((unsigned)B), dim3(256), 0, bb->stream, bb->residual, (const f16_t *)add, bb->temporal, bb->norm_f, c.rms_norm_eps, dm);
-    return check_launch("add_rmsnorm3_kernel");
+    return launch_add_rmsnorm_any(bb->stream, dt, bb->residual, bb->skinny ? nullptr : bb->out, bb->temporal, true, nullptr, bb->norm_f,
+                                  c.rms_norm_eps, B, dm, dm);
 }
 
 }  // namespace
@@ -753,16 +714,8 @@ int launch_gate_t(mrs_m3_backbone *bb, const Layer3 &lw, int64_t rows, const voi
 }
 
 int launch_add_rmsnorm3(mrs_m3_backbone *bb, float *residual, const void *add, void *out, bool out_f32, const float *w, int64_t rows) {
-    const int dm = bb->cfg.d_model;
-    const float eps = bb->cfg.rms_norm_eps;
-    const dim3 grid((unsigned)rows), block(256);
-    const int dt = bb->dtype;
-    if (dt == MRS_F32) hipLaunchKernelGGL((add_rmsnorm3_kernel<float, float>), grid, block, 0, bb->stream, residual, (const float *)add, (float *)out, w, eps, dm);
-    else if (dt == MRS_BF16 && out_f32) hipLaunchKernelGGL((add_rmsnorm3_kernel<bf16_t, float>), grid, block, 0, bb->stream, residual, (const bf16_t *)add, (float *)out, w, eps, dm);
-    else if (dt == MRS_BF16) hipLaunchKernelGGL((add_rmsnorm3_kernel<bf16_t, bf16_t>), grid, block, 0, bb->stream, residual, (const bf16_t *)add, (bf16_t *)out, w, eps, dm);
-    else if (out_f32) hipLaunchKernelGGL((add_rmsnorm3_kernel<f16_t, float>), grid, block, 0, bb->stream, residual, (const f16_t *)add, (float *)out, w, eps, dm);
-    else hipLaunchKernelGGL((add_rmsnorm3_kernel<f16_t, f16_t>), grid, block, 0, bb->stream, residual, (const f16_t *)add, (f16_t *)out, w, eps, dm);
-    return check_launch("add_rmsnorm3_kernel");
+    return launch_add_rmsnorm_any(bb->stream, bb->dtype, residual, add, out, out_f32, nullptr, w, bb->cfg.rms_norm_eps, rows, bb->cfg.d_model,
+                                  bb->cfg.d_model);
 }
 
 int prefill_body3(mrs_m3_backbone *bb, int T) {
@@ -775,7 +728,7 @@ int prefill_body3(mrs_m3_backbone *bb, int T) {
         MRS_HIP(hipMemcpyAsync(bb->pf_residual, bb->pf_in, (size_t)rows * dm * 4, hipMemcpyDeviceToDevice, bb->stream));
     } else {
         const int64_t n = rows * dm;
-        hipLaunchKernelGGL(bias_rows3_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, bb->stream, bb->pf_residual, bb->input_proj_b, n, dm);
+        hipLaunchKernelGGL(bias_rows_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, bb->stream, bb->pf_residual, bb->input_proj_b, n, dm);
         const float one = 1.0f;
         MRS_BLAS(rocblas_gemm_ex(bb->blas, rocblas_operation_none, rocblas_operation_none, dm, (int)rows, bb->input_dim, &one, bb->input_proj_w,
                                  rocblas_datatype_f32_r, dm, bb->pf_in, rocblas_datatype_f32_r, bb->input_dim, &one, bb->pf_residual,
