@@ -275,6 +275,9 @@ MRS_API int mrs_backbone_download_state(mrs_backbone *bb, int layer, float *conv
  *   embed: [vocab, d_model] f32 on the host (rows >= vocab of the 64-padded table are zero). */
 typedef struct mrs_lm mrs_lm;
 MRS_API int mrs_lm_create(mrs_lm **out, mrs_backbone *decode_engine, const float *embed, int vocab);
+/* A head with weights of its own (tie_word_embeddings = false; src/hf/load.rs:119-141, gpu_lm.rs:182-250):
+ * lm_head is [d_model, vocab] f32 on the host.  Call before mrs_lm_capture_graph. */
+MRS_API int mrs_lm_set_untied_head(mrs_lm *lm, const float *lm_head);
 MRS_API void mrs_lm_destroy(mrs_lm *lm);
 MRS_API int mrs_lm_set_tokens(mrs_lm *lm, const int *tokens);      /* [batch] current tokens */
 MRS_API int mrs_lm_get_tokens(mrs_lm *lm, int *tokens);            /* synchronises */

@@ -58,6 +58,7 @@ def _bind():
         "mrs_backbone_state_ptrs": (c_int, [P, c_int, POINTER(P), POINTER(P)]),
         "mrs_backbone_download_state": (c_int, [P, c_int, _FP, _FP]),
         "mrs_lm_create": (c_int, [POINTER(P), P, _FP, c_int]),
+        "mrs_lm_set_untied_head": (c_int, [P, _FP]),
         "mrs_lm_destroy": (None, [P]),
         "mrs_lm_set_tokens": (c_int, [P, POINTER(c_int)]),
         "mrs_lm_get_tokens": (c_int, [P, POINTER(c_int)]),
@@ -193,9 +194,10 @@ class GpuMambaBackbone:
 
 
 class GpuMambaLM:
-    """Greedy LM loop with tied embedding / lm_head on top of a backbone (identity input_proj)."""
+    """Greedy LM loop on top of a backbone (identity input_proj).  The head is the embedding table (tied)
+    unless `lm_head` [d_model, vocab] is given (GpuMambaLM::new, src/module/gpu_lm.rs:143-262)."""
 
-    def __init__(self, backbone: GpuMambaBackbone, embed: np.ndarray):
+    def __init__(self, backbone: GpuMambaBackbone, embed: np.ndarray, lm_head: np.ndarray | None = None):
         self.backbone = backbone
         embed = np.ascontiguousarray(embed, dtype=np.float32)
         if embed.ndim != 2 or embed.shape[1] != backbone.cfg.d_model:
@@ -204,6 +206,22 @@ class GpuMambaLM:
         h = c_void_p()
         _call("mrs_lm_create", byref(h), backbone._h, _fp(embed), self.vocab)
         self._h = h
+        if lm_head is not None:
+            lm_head = np.ascontiguousarray(lm_head, dtype=np.float32)
+            if lm_head.shape != (backbone.cfg.d_model, self.vocab):
+                raise ValueError("lm_head must be [d_model, vocab]")
+            _call("mrs_lm_set_untied_head", self._h, _fp(lm_head))
+
+    @classmethod
+    def from_hf(cls, directory: str, batch: int = 1, dtype: WeightDtype = WeightDtype.F32, gpu_ordinal: int = 0) -> "GpuMambaLM":
+        """Engine + LM loop from a HuggingFace Mamba-1 checkpoint directory (hf::load_hf then GpuMambaLM::new,
+        src/hf/load.rs:40, src/module/gpu_lm.rs:143)."""
+        from .formats import load_hf
+        m = load_hf(directory)
+        bb = GpuMambaBackbone(gpu_ordinal, m.weights, m.cfg, m.cfg.d_model, batch, dtype)
+        lm = cls(bb, m.embed[:m.vocab_size], m.lm_head)
+        lm.hf = m.hf
+        return lm
 
     def close(self):
         if getattr(self, "_h", None):

@@ -625,6 +625,7 @@ struct mrs_lm {
     mrs_backbone *bb;   // decode engine (not owned)
     int vocab, vocab_padded, dm, batch, dtype;
     void *embed;        // [vocab_padded, dm] storage dtype (tied lm_head)
+    void *head;         // [vocab_padded, dm] storage dtype when the head has weights of its own, else null
     float *logits;      // [batch, vocab_padded] f32
     int *tokens;        // [batch] current token ids on device
     float *arg_v;       // [batch, kArgParts] partial maxima
@@ -643,6 +644,7 @@ extern "C" int mrs_lm_create(mrs_lm **out, mrs_backbone *bb, const float *embed,
     if (!lm) return fail(MRS_E_HIP, "mrs_lm_create: out of host memory");
     lm->bb = bb; lm->vocab = vocab; lm->vocab_padded = (vocab + 63) & ~63;  // src/hf/load.rs:59
     lm->dm = bb->cfg.d_model; lm->batch = bb->batch; lm->dtype = bb->dtype; lm->graph_ready = 0; lm->graph = nullptr; lm->graph_exec = nullptr;
+    lm->head = nullptr;
     *out = nullptr;
     const size_t es = esize(lm->dtype), ne = (size_t)lm->vocab_padded * lm->dm;
     float *stage = nullptr;
@@ -667,6 +669,36 @@ extern "C" int mrs_lm_create(mrs_lm **out, mrs_backbone *bb, const float *embed,
     return MRS_OK;
 }
 
+// A head with weights of its own (tie_word_embeddings = false): `lm_head` is [d_model, vocab] row-major, the
+// layout the reference's loader hands over (src/hf/load.rs:126-141, src/module/gpu_lm.rs:182-250).  It is kept
+// as [vocab_padded, d_model] like the embedding table, so the logits GEMM is the same call on another pointer.
+extern "C" int mrs_lm_set_untied_head(mrs_lm *lm, const float *lm_head) {
+    if (!lm || !lm_head) return fail(MRS_E_NULL, "mrs_lm_set_untied_head: null pointer");
+    if (lm->graph_ready) return fail(MRS_E_SHAPE, "mrs_lm_set_untied_head: set the head before capturing the graph");
+    mrs_backbone *bb = lm->bb;
+    const size_t es = esize(lm->dtype), ne = (size_t)lm->vocab_padded * lm->dm;
+    std::vector<float> host;
+    try { host.assign(ne, 0.0f); } catch (...) { return fail(MRS_E_HIP, "mrs_lm_set_untied_head: out of host memory"); }
+    for (int d = 0; d < lm->dm; ++d)
+        for (int v = 0; v < lm->vocab; ++v) host[(size_t)v * lm->dm + d] = lm_head[(size_t)d * lm->vocab + v];
+    float *stage = nullptr;
+    void *dst = lm->head;
+    if (!dst) { MRS_HIP(hipMalloc(&dst, ne * es)); }
+    hipError_t e = hipMalloc((void **)&stage, ne * 4);
+    if (e == hipSuccess) e = hipMemcpyAsync(stage, host.data(), ne * 4, hipMemcpyHostToDevice, bb->stream);
+    if (e == hipSuccess) {
+        const dim3 grid((unsigned)((ne + 255) / 256)), block(256);
+        if (lm->dtype == MRS_F32) e = hipMemcpyAsync(dst, stage, ne * 4, hipMemcpyDeviceToDevice, bb->stream);
+        else if (lm->dtype == MRS_BF16) hipLaunchKernelGGL((cast_from_f32_kernel<bf16_t>), grid, block, 0, bb->stream, (bf16_t *)dst, stage, (int64_t)ne);
+        else hipLaunchKernelGGL((cast_from_f32_kernel<f16_t>), grid, block, 0, bb->stream, (f16_t *)dst, stage, (int64_t)ne);
+    }
+    if (e == hipSuccess) e = hipStreamSynchronize(bb->stream);
+    if (stage) hipFree(stage);
+    if (e != hipSuccess) { if (!lm->head) hipFree(dst); return fail(MRS_E_HIP, "mrs_lm_set_untied_head: %s", hipGetErrorString(e)); }
+    if (!lm->head) { lm->head = dst; lm->allocs.push_back(dst); }
+    return MRS_OK;
+}
+
 extern "C" void mrs_lm_destroy(mrs_lm *lm) {
     if (!lm) return;
     hipStreamSynchronize(lm->bb->stream);
@@ -676,7 +708,8 @@ extern "C" void mrs_lm_destroy(mrs_lm *lm) {
     delete lm;
 }
 
-// logits = norm_f(hidden) . embed^T  (tied head, OP_T on the row-major [V, dm] table: src/mamba_ssm/gpu/blas.rs:709-740)
+// logits = norm_f(hidden) . table^T, table = the embedding (tied head) or the head's own weights
+// (OP_T on the row-major [V, dm] table: src/mamba_ssm/gpu/blas.rs:709-740)
 static int lm_logits(mrs_lm *lm) {
     mrs_backbone *bb = lm->bb;
     const int dm = lm->dm, V = lm->vocab_padded, B = lm->batch;
@@ -684,8 +717,8 @@ static int lm_logits(mrs_lm *lm) {
     // the final norm leaves its result in the storage type as well (temporal_t), which is the head's operand
     const void *hid = lm->dtype != MRS_F32 ? bb->temporal_t : (const void *)bb->temporal;
     const rocblas_datatype ht = lm->dtype != MRS_F32 ? blas_type(lm->dtype) : rocblas_datatype_f32_r;
-    MRS_BLAS(rocblas_gemm_ex(bb->blas, rocblas_operation_transpose, rocblas_operation_none, V, B, dm, &one, lm->embed,
-                             blas_type(lm->dtype), dm, hid, ht, dm, &zero, lm->logits, rocblas_datatype_f32_r, V, lm->logits,
+    MRS_BLAS(rocblas_gemm_ex(bb->blas, rocblas_operation_transpose, rocblas_operation_none, V, B, dm, &one,
+                             lm->head ? lm->head : lm->embed, blas_type(lm->dtype), dm, hid, ht, dm, &zero, lm->logits, rocblas_datatype_f32_r, V, lm->logits,
                              rocblas_datatype_f32_r, V, rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0));
     return MRS_OK;
 }
