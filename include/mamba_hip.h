@@ -288,6 +288,46 @@ MRS_API int mrs_lm_last_logits(mrs_lm *lm, float *logits);         /* [batch, vo
  * engine itself: then the head + argmax run and the next tokens are left in the token buffer). */
 MRS_API int mrs_lm_prefill(mrs_lm *lm, mrs_backbone *prefill_engine, const int *tokens, int T);
 
+/* ---- sampling and batched generation ------------------------------------------------------
+ * sample_token (src/module/sample.rs:243-265): repetition penalty -> temperature -> top-k -> softmax -> top-p ->
+ * min-p -> weighted draw, with the switches of SampleParams (sample.rs:20-46): temperature <= 0 is greedy (last
+ * index of the maximum, no draw), top_k 0 / top_p outside (0,1) / min_p <= 0 / penalty 1, <= 0 or NaN are off.
+ * The reference samples on the host from downloaded logits; here one launch samples every row on the device. */
+typedef struct { float temperature; int top_k; float top_p; float min_p; float repetition_penalty; } mrs_sampler;
+
+/* Xoshiro256PlusPlus::new (sample.rs:54-66): the four state words for a seed.  Host function. */
+MRS_API void mrs_xoshiro_seed(unsigned long long seed, unsigned long long state[4]);
+
+/* All pointers are device memory.  tokens [rows] <- sampled ids; logits [rows, ld] f32 (read only); work [rows, ld]
+ * f32 scratch; samplers [rows]; seen_counts [rows, vocab] occurrences of each token in the row's seen list, or null
+ * (no penalty); rng_state [rows, 4], advanced by one draw per sampled row; active [rows] or null: rows with 0 are
+ * skipped (token, generator untouched). */
+MRS_API int mrs_sample_tokens(void *stream, int *tokens, const float *logits, float *work, int64_t ld, int rows, int vocab,
+                              const mrs_sampler *samplers, const unsigned *seen_counts, unsigned long long *rng_state,
+                              const int *active);
+
+/* SampleParams (sample.rs:20-46) of one slot; eos_token_ids may be null when n_eos is 0 (at most 16 ids). */
+typedef struct {
+    mrs_sampler sampler;
+    int max_tokens;
+    const int *eos_token_ids;
+    int n_eos;
+    unsigned long long seed;
+} mrs_sample_params;
+
+/* GpuMambaLM::generate_batch (src/module/gpu_lm.rs:389-516): one prompt per batch slot, of any length (an empty
+ * prompt leaves its slot finished); prompts are consumed a token per step, slots whose prompt is done sample from
+ * their own generator and stop at an EOS id or at max_tokens.  The whole loop -- gather, step, head, sampling and
+ * the per-slot bookkeeping -- stays on the device; the host only polls how many slots are still running.
+ *   prompts: all prompts back to back; prompt_lens [batch]; params [batch];
+ *   out_tokens [batch, out_stride] and out_lens [batch] receive the generated ids (prompt excluded);
+ *   out_stride >= every max_tokens.
+ * seen_includes_prompt = 0: the penalty sees the generated tokens only (generate_batch, gpu_lm.rs:470-487);
+ * 1: prompt and generated tokens (generate_streaming, gpu_lm.rs:364-375), and a batch-1 engine takes prompts of 256
+ * tokens or more through prefill (gpu_lm.rs:349). */
+MRS_API int mrs_lm_generate_batch(mrs_lm *lm, const int *prompts, const int *prompt_lens, const mrs_sample_params *params,
+                                  int seen_includes_prompt, int *out_tokens, int out_stride, int *out_lens);
+
 /* ---- Mamba-3 SISO backbone engine (decode step) -------------------------------------------------
  * GpuMamba3Backbone (src/mamba3_siso/gpu/inference.rs:1487-1671): weights, per-layer state
  * (ssm [batch,nh,hd,ds], k [batch,nh,ds], v [batch,nh,hd], angle [batch,nh,n_rope], all f32) and scratch owned by

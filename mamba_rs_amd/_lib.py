@@ -6,7 +6,7 @@ op raises.  Build it with `python -m mamba_rs_amd.build`.
 from __future__ import annotations
 
 import ctypes
-from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_uint, c_void_p
+from ctypes import POINTER, c_char_p, c_float, c_int, c_int64, c_size_t, c_uint, c_uint64, c_void_p
 from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "libmamba_hip.so"
@@ -38,6 +38,8 @@ _SIGNATURES = {
     "mrs_conv1d_seq_silu": (c_int, [_P, c_int, _P, _P, _P, c_int64, _P, _P, c_int, c_int, c_int, c_int]),
     "mrs_gemm_skinny": (c_int, [_P, c_int, _P, c_int, c_int64, _P, c_int64, _P, c_int, c_int, c_int]),
     "mrs_transpose": (c_int, [_P, c_int, _P, _P, c_int, c_int]),
+    "mrs_xoshiro_seed": (None, [c_uint64, POINTER(c_uint64)]),
+    "mrs_sample_tokens": (c_int, [_P, _P, _P, _P, c_int64, c_int, c_int, _P, _P, _P, _P]),
     "mrs_m3_step": (c_int, [_P, c_int, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int]),
     "mrs_m3_seq_fwd": (c_int, [_P, c_int, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int]),
     "mrs_m3_compute_abg": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int64]),

@@ -6,7 +6,8 @@ All arithmetic happens in libmamba_hip.so; this module only marshals numpy array
 from __future__ import annotations
 
 import ctypes
-from ctypes import POINTER, Structure, byref, c_float, c_int, c_void_p
+from dataclasses import dataclass, field
+from ctypes import c_uint64, POINTER, Structure, byref, c_float, c_int, c_void_p
 
 import numpy as np
 
@@ -66,6 +67,8 @@ def _bind():
         "mrs_lm_capture_graph": (c_int, [P]),
         "mrs_lm_last_logits": (c_int, [P, _FP]),
         "mrs_lm_prefill": (c_int, [P, P, POINTER(c_int), c_int]),
+        "mrs_lm_generate_batch": (c_int, [P, POINTER(c_int), POINTER(c_int), POINTER(_CSampleParams), c_int, POINTER(c_int), c_int,
+                                          POINTER(c_int)]),
     }
     for name, (res, args) in sigs.items():
         fn = getattr(lib, name)
@@ -77,6 +80,27 @@ def _bind():
 
 def engine_exported_names():
     return list(_bind()._engine_names)
+
+
+class _CSampler(Structure):
+    _fields_ = [("temperature", c_float), ("top_k", c_int), ("top_p", c_float), ("min_p", c_float), ("repetition_penalty", c_float)]
+
+
+class _CSampleParams(Structure):
+    _fields_ = [("sampler", _CSampler), ("max_tokens", c_int), ("eos_token_ids", POINTER(c_int)), ("n_eos", c_int), ("seed", c_uint64)]
+
+
+@dataclass
+class SampleParams:
+    """SampleParams with the reference's defaults (src/module/sample.rs:20-46)."""
+    temperature: float = 1.0
+    top_k: int = 0
+    top_p: float = 1.0
+    min_p: float = 0.0
+    repetition_penalty: float = 1.0
+    max_tokens: int = 256
+    eos_token_ids: list = field(default_factory=list)
+    seed: int = 42
 
 
 def _call(name, *args):
@@ -257,11 +281,37 @@ class GpuMambaLM:
             raise ValueError("tokens must be [batch, T]")
         _call("mrs_lm_prefill", self._h, engine._h, t.ctypes.data_as(POINTER(c_int)), t.shape[1])
 
-    def generate(self, prompt, max_tokens: int):
-        """Greedy generation for a batch-1 engine (GpuMambaLM::generate, temperature 0, gpu_lm.rs:323-377):
-        the prompt goes through prefill when it has at least 2 tokens, token by token otherwise."""
+    def generate_batch(self, prompts, params, *, seen_includes_prompt: bool = False):
+        """GpuMambaLM::generate_batch (src/module/gpu_lm.rs:389-516): one prompt (any length) and one SampleParams per
+        batch slot -> one list of generated tokens per slot.  The loop runs on the device."""
+        B = self.backbone.batch
+        if len(prompts) != B or len(params) != B:
+            raise ValueError("prompts and params must have one entry per batch slot")
+        lens = np.asarray([len(p) for p in prompts], np.int32)
+        flat = np.ascontiguousarray(np.concatenate([np.asarray(p, np.int32).ravel() for p in prompts] + [np.zeros(0, np.int32)]))
+        cp = (_CSampleParams * B)()
+        keep = []
+        for i, sp in enumerate(params):
+            eos = np.ascontiguousarray(sp.eos_token_ids, dtype=np.int32)
+            keep.append(eos)
+            cp[i].sampler = _CSampler(sp.temperature, sp.top_k, sp.top_p, sp.min_p, sp.repetition_penalty)
+            cp[i].max_tokens, cp[i].n_eos, cp[i].seed = sp.max_tokens, eos.size, sp.seed & 0xFFFFFFFFFFFFFFFF
+            cp[i].eos_token_ids = eos.ctypes.data_as(POINTER(c_int)) if eos.size else None
+        stride = max(1, max(sp.max_tokens for sp in params))
+        out = np.zeros((B, stride), np.int32)
+        out_lens = np.zeros(B, np.int32)
+        _call("mrs_lm_generate_batch", self._h, flat.ctypes.data_as(POINTER(c_int)), lens.ctypes.data_as(POINTER(c_int)), cp,
+              1 if seen_includes_prompt else 0, out.ctypes.data_as(POINTER(c_int)), stride, out_lens.ctypes.data_as(POINTER(c_int)))
+        return [[int(t) for t in out[i, :out_lens[i]]] for i in range(B)]
+
+    def generate(self, prompt, max_tokens: int | None = None, params: SampleParams | None = None):
+        """GpuMambaLM::generate for a batch-1 engine (gpu_lm.rs:323-377).  With `params` the reference's sampled loop
+        (penalty over prompt + generated tokens, EOS, seed); with `max_tokens` alone the greedy loop, where the prompt
+        goes through prefill when it has at least 2 tokens, token by token otherwise."""
         if self.backbone.batch != 1:
             raise ValueError("generate() is the batch-1 entry point")
+        if params is not None:
+            return self.generate_batch([list(prompt)], [params], seen_includes_prompt=True)[0]
         prompt = list(prompt)
         self.backbone.reset()
         if len(prompt) >= 2:

@@ -107,6 +107,10 @@ int m3_ssd_fwd_ex(void *stream, int dtype, float *ssm_state, float *k_state, flo
                   const float *D, void *workspace, size_t workspace_bytes, unsigned flags, int batch, int T, int nheads,
                   int headdim, int d_state, int chunk_size);
 
+// sample_token for every active row (sampling.hip); all pointers device memory
+int launch_sample_rows(hipStream_t st, int *tokens, const float *logits, float *work, int64_t ld, int rows, int vocab,
+                       const mrs_sampler *samplers, const unsigned *seen, unsigned long long *rng, const int *active);
+
 inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s); }
 inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 

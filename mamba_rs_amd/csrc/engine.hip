@@ -21,6 +21,7 @@
 #include <stdlib.h>
 #include <new>
 #include <vector>
+#include <algorithm>
 
 namespace mrs {
 
@@ -78,12 +79,15 @@ __global__ __launch_bounds__(256) void exp_negate_k(float *__restrict__ a_neg, c
 }
 
 // residual[r, :] = embed[token[r], :] widened to f32 (host-side embed_lookup of the reference, gpu_lm.rs:352-373, moved on device)
+// rows with finished[r] != 0 get a zero vector (generate_batch feeds finished slots zeros, gpu_lm.rs:436-441)
 template <typename T>
 __global__ __launch_bounds__(256) void embed_gather_kernel(float *__restrict__ out, const T *__restrict__ embed,
-                                                           const int *__restrict__ tokens, int64_t rows, int dm, int vocab) {
+                                                           const int *__restrict__ tokens, int64_t rows, int dm, int vocab,
+                                                           const int *__restrict__ finished = nullptr) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= rows * dm) return;
     const int64_t r = i / dm;
+    if (finished && finished[r]) { out[i] = 0.0f; return; }
     int tok = tokens[r];
     tok = tok < 0 ? 0 : (tok >= vocab ? vocab - 1 : tok);
     out[i] = Store<T>::ld(embed + (int64_t)tok * dm + (i - r * dm));
@@ -135,6 +139,65 @@ __global__ __launch_bounds__(64) void argmax_final_kernel(int *__restrict__ toke
         if (ov > best || (ov == best && oi > bi)) { best = ov; bi = oi; }
     }
     if (threadIdx.x == 0) tokens[row] = bi;
+}
+
+// ---- generate_batch bookkeeping on the device (src/module/gpu_lm.rs:404-513) ------------------------------
+constexpr int kMaxEos = 16;
+struct GenSlots {            // per-slot arrays, [batch] each unless noted
+    int *prompt_off, *prompt_len, *prompt_pos, *finished, *active, *max_tokens, *n_eos, *eos /*[batch, kMaxEos]*/, *out_len, *sampled;
+    unsigned *seen;          // [batch, vocab] occurrences in the slot's seen list
+    int *n_running;          // [1] slots not finished after the latest step
+};
+struct GenDyn {              // buffers that grow between calls; read through device memory so a captured step stays valid
+    const int *prompts;
+    int *out;
+    int out_stride;
+};
+
+// Seen list of generate_streaming starts as the prompt (gpu_lm.rs:364).
+__global__ __launch_bounds__(256) void gen_seen_prompt_kernel(GenSlots g, const GenDyn *__restrict__ dyn, int batch, int vocab) {
+    const int slot = blockIdx.y;
+    const int n = g.prompt_len[slot];
+    const int *p = dyn->prompts + g.prompt_off[slot];
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) {
+        const int t = p[i];
+        if (t >= 0 && t < vocab) atomicAdd(&g.seen[(int64_t)slot * vocab + t], 1u);
+    }
+}
+
+// After a step: slots still inside their prompt take the next prompt token; slots past it take the sampled token,
+// unless it is an EOS id or max_tokens are out already -- then the slot is finished (gpu_lm.rs:494-511).  Also
+// marks which slots sample after the next step (prompt consumed, not finished) and counts the running ones.
+__global__ __launch_bounds__(1024) void gen_advance_kernel(GenSlots g, const GenDyn *__restrict__ dyn, int *__restrict__ last_token,
+                                                           int batch, int vocab) {
+    __shared__ int running;
+    if (threadIdx.x == 0) running = 0;
+    __syncthreads();
+    for (int i = threadIdx.x; i < batch; i += blockDim.x) {
+        if (!g.finished[i]) {
+            if (g.prompt_pos[i] < g.prompt_len[i]) {
+                last_token[i] = dyn->prompts[g.prompt_off[i] + g.prompt_pos[i]];
+                g.prompt_pos[i] += 1;
+            } else {
+                const int next = g.sampled[i];
+                bool stop = g.out_len[i] >= g.max_tokens[i];
+                for (int e = 0; e < g.n_eos[i]; e++) stop = stop || g.eos[i * kMaxEos + e] == next;
+                if (stop) {
+                    g.finished[i] = 1;
+                } else {
+                    dyn->out[(int64_t)i * dyn->out_stride + g.out_len[i]] = next;
+                    g.out_len[i] += 1;
+                    last_token[i] = next;
+                    if (next >= 0 && next < vocab) g.seen[(int64_t)i * vocab + next] += 1u;
+                }
+            }
+        }
+        const int fin = g.finished[i];
+        g.active[i] = !fin && g.prompt_pos[i] >= g.prompt_len[i];
+        if (!fin) atomicAdd(&running, 1);
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) *g.n_running = running;
 }
 
 }  // namespace mrs
@@ -626,6 +689,18 @@ struct mrs_lm {
     int vocab, vocab_padded, dm, batch, dtype;
     void *embed;        // [vocab_padded, dm] storage dtype (tied lm_head)
     void *head;         // [vocab_padded, dm] storage dtype when the head has weights of its own, else null
+    // generate_batch state (allocated on first use)
+    GenSlots gen;
+    GenDyn *gen_dyn;            // device copy
+    GenDyn gen_dyn_host;
+    int *gen_ints;              // one allocation behind the int arrays of `gen`
+    mrs_sampler *gen_samplers;  // [batch]
+    unsigned long long *gen_rng;  // [batch, 4]
+    float *gen_work;            // [batch, vocab_padded] penalised / scaled logits
+    int gen_prompt_cap, gen_out_cap;
+    hipGraph_t gen_graph;
+    hipGraphExec_t gen_graph_exec;
+    int gen_ready, gen_graph_ready;
     float *logits;      // [batch, vocab_padded] f32
     int *tokens;        // [batch] current token ids on device
     float *arg_v;       // [batch, kArgParts] partial maxima
@@ -645,6 +720,8 @@ extern "C" int mrs_lm_create(mrs_lm **out, mrs_backbone *bb, const float *embed,
     lm->bb = bb; lm->vocab = vocab; lm->vocab_padded = (vocab + 63) & ~63;  // src/hf/load.rs:59
     lm->dm = bb->cfg.d_model; lm->batch = bb->batch; lm->dtype = bb->dtype; lm->graph_ready = 0; lm->graph = nullptr; lm->graph_exec = nullptr;
     lm->head = nullptr;
+    lm->gen_ready = 0; lm->gen_graph_ready = 0; lm->gen_graph = nullptr; lm->gen_graph_exec = nullptr;
+    lm->gen_prompt_cap = 0; lm->gen_out_cap = 0; lm->gen_dyn = nullptr; lm->gen_dyn_host = GenDyn{nullptr, nullptr, 0};
     *out = nullptr;
     const size_t es = esize(lm->dtype), ne = (size_t)lm->vocab_padded * lm->dm;
     float *stage = nullptr;
@@ -704,6 +781,10 @@ extern "C" void mrs_lm_destroy(mrs_lm *lm) {
     hipStreamSynchronize(lm->bb->stream);
     if (lm->graph_exec) hipGraphExecDestroy(lm->graph_exec);
     if (lm->graph) hipGraphDestroy(lm->graph);
+    if (lm->gen_graph_exec) hipGraphExecDestroy(lm->gen_graph_exec);
+    if (lm->gen_graph) hipGraphDestroy(lm->gen_graph);
+    if (lm->gen_dyn_host.prompts) hipFree((void *)lm->gen_dyn_host.prompts);
+    if (lm->gen_dyn_host.out) hipFree(lm->gen_dyn_host.out);
     for (void *p : lm->allocs) hipFree(p);
     delete lm;
 }
@@ -824,4 +905,158 @@ extern "C" int mrs_lm_prefill(mrs_lm *lm, mrs_backbone *prefill_bb, const int *t
     hipStreamSynchronize(prefill_bb->stream);
     hipFree(dtok);
     return rc;
+}
+
+// ---- batched generation ------------------------------------------------------------------------------------
+
+static int gen_alloc(mrs_lm *lm) {
+    if (lm->gen_ready) return MRS_OK;
+    const size_t B = lm->batch;
+    const size_t n_int = B * (10 + kMaxEos) + 1;
+    MRS_HIP(hipMalloc((void **)&lm->gen_ints, n_int * sizeof(int))); lm->allocs.push_back(lm->gen_ints);
+    int *p = lm->gen_ints;
+    GenSlots &g = lm->gen;
+    g.prompt_off = p; p += B; g.prompt_len = p; p += B; g.prompt_pos = p; p += B; g.finished = p; p += B; g.active = p; p += B;
+    g.max_tokens = p; p += B; g.n_eos = p; p += B; g.out_len = p; p += B; g.sampled = p; p += B; p += B /* spare */;
+    g.eos = p; p += B * kMaxEos; g.n_running = p;
+    MRS_HIP(hipMalloc((void **)&g.seen, B * lm->vocab * sizeof(unsigned))); lm->allocs.push_back(g.seen);
+    MRS_HIP(hipMalloc((void **)&lm->gen_samplers, B * sizeof(mrs_sampler))); lm->allocs.push_back(lm->gen_samplers);
+    MRS_HIP(hipMalloc((void **)&lm->gen_rng, B * 4 * sizeof(unsigned long long))); lm->allocs.push_back(lm->gen_rng);
+    MRS_HIP(hipMalloc((void **)&lm->gen_work, B * lm->vocab_padded * sizeof(float))); lm->allocs.push_back(lm->gen_work);
+    MRS_HIP(hipMalloc((void **)&lm->gen_dyn, sizeof(GenDyn))); lm->allocs.push_back(lm->gen_dyn);
+    lm->gen_ready = 1;
+    return MRS_OK;
+}
+
+// sample the active slots from the current logits, then advance every slot
+static int gen_pick(mrs_lm *lm) {
+    hipStream_t st = lm->bb->stream;
+    MRS_TRY(launch_sample_rows(st, lm->gen.sampled, lm->logits, lm->gen_work, lm->vocab_padded, lm->batch, lm->vocab, lm->gen_samplers,
+                               lm->gen.seen, lm->gen_rng, lm->gen.active));
+    hipLaunchKernelGGL(gen_advance_kernel, dim3(1), dim3(1024), 0, st, lm->gen, lm->gen_dyn, lm->tokens, lm->batch, lm->vocab);
+    return check_launch("gen_advance_kernel");
+}
+
+// gather the slots' current tokens (zeros for finished slots), one backbone step, head
+static int gen_forward(mrs_lm *lm) {
+    mrs_backbone *bb = lm->bb;
+    const int64_t n = (int64_t)lm->batch * lm->dm;
+    const dim3 grid((unsigned)((n + 255) / 256)), block(256);
+    MRS_DISPATCH_DTYPE(lm->dtype, T_, hipLaunchKernelGGL((embed_gather_kernel<T_>), grid, block, 0, bb->stream, bb->d_input,
+                                                         (const T_ *)lm->embed, lm->tokens, (int64_t)lm->batch, lm->dm, lm->vocab,
+                                                         (const int *)lm->gen.finished));
+    MRS_TRY(step_body(bb));
+    return lm_logits(lm);
+}
+
+extern "C" int mrs_lm_generate_batch(mrs_lm *lm, const int *prompts, const int *prompt_lens, const mrs_sample_params *params,
+                                     int seen_includes_prompt, int *out_tokens, int out_stride, int *out_lens) {
+    if (!lm || !prompt_lens || !params || !out_tokens || !out_lens) return fail(MRS_E_NULL, "mrs_lm_generate_batch: null pointer");
+    mrs_backbone *bb = lm->bb;
+    hipStream_t st = bb->stream;
+    const int B = lm->batch;
+    int64_t total = 0;
+    int max_prompt = 0, max_tokens = 0;
+    for (int i = 0; i < B; i++) {
+        if (prompt_lens[i] < 0 || params[i].max_tokens < 0 || params[i].n_eos < 0 || params[i].n_eos > kMaxEos ||
+            (params[i].n_eos > 0 && !params[i].eos_token_ids))
+            return fail(MRS_E_SHAPE, "mrs_lm_generate_batch: slot %d: prompt_len=%d max_tokens=%d n_eos=%d (at most %d)", i, prompt_lens[i],
+                        params[i].max_tokens, params[i].n_eos, kMaxEos);
+        if (params[i].max_tokens > out_stride)
+            return fail(MRS_E_SHAPE, "mrs_lm_generate_batch: slot %d: max_tokens=%d exceeds out_stride=%d", i, params[i].max_tokens, out_stride);
+        total += prompt_lens[i];
+        max_prompt = std::max(max_prompt, prompt_lens[i]);
+        max_tokens = std::max(max_tokens, params[i].max_tokens);
+    }
+    if (total > 0 && !prompts) return fail(MRS_E_NULL, "mrs_lm_generate_batch: null prompts");
+    if (total > (int64_t)1 << 30) return fail(MRS_E_SHAPE, "mrs_lm_generate_batch: %lld prompt tokens", (long long)total);
+    MRS_TRY(gen_alloc(lm));
+    // buffers that follow the call's sizes
+    if (total > lm->gen_prompt_cap) {
+        if (lm->gen_dyn_host.prompts) hipFree((void *)lm->gen_dyn_host.prompts);
+        lm->gen_dyn_host.prompts = nullptr; lm->gen_prompt_cap = 0;
+        int *p = nullptr;
+        MRS_HIP(hipMalloc((void **)&p, (size_t)total * sizeof(int)));
+        lm->gen_dyn_host.prompts = p; lm->gen_prompt_cap = (int)total;
+    }
+    const int64_t out_need = (int64_t)B * std::max(max_tokens, 1);
+    if (out_need > lm->gen_out_cap) {
+        if (lm->gen_dyn_host.out) hipFree(lm->gen_dyn_host.out);
+        lm->gen_dyn_host.out = nullptr; lm->gen_out_cap = 0;
+        MRS_HIP(hipMalloc((void **)&lm->gen_dyn_host.out, (size_t)out_need * sizeof(int)));
+        lm->gen_out_cap = (int)out_need;
+    }
+    lm->gen_dyn_host.out_stride = std::max(max_tokens, 1);
+    // host-side initial state (gpu_lm.rs:404-430): the first prompt token is the first input; empty prompts are finished
+    std::vector<int> h((size_t)B * (10 + kMaxEos) + 1, 0);
+    int *off = h.data(), *len = off + B, *pos = len + B, *fin = pos + B, *act = fin + B, *mx = act + B, *neos = mx + B, *olen = neos + B,
+        *eos = olen + 3 * B, *nrun = eos + (size_t)B * kMaxEos;
+    std::vector<int> first(B, 0);
+    std::vector<mrs_sampler> samplers(B);
+    std::vector<unsigned long long> rng((size_t)B * 4);
+    const bool prefill_route = seen_includes_prompt && B == 1 && prompt_lens[0] >= 256;   // PREFILL_PARALLEL_THRESHOLD, gpu_lm.rs:48
+    int64_t o = 0;
+    int running = 0;
+    for (int i = 0; i < B; i++) {
+        off[i] = (int)o; len[i] = prompt_lens[i]; o += prompt_lens[i];
+        fin[i] = prompt_lens[i] == 0;
+        pos[i] = fin[i] ? 0 : (prefill_route ? len[i] : 1);
+        act[i] = !fin[i] && pos[i] >= len[i];
+        first[i] = fin[i] ? 0 : prompts[off[i]];
+        mx[i] = params[i].max_tokens; neos[i] = params[i].n_eos;
+        for (int e = 0; e < params[i].n_eos; e++) eos[(size_t)i * kMaxEos + e] = params[i].eos_token_ids[e];
+        samplers[i] = params[i].sampler;
+        mrs_xoshiro_seed(params[i].seed, &rng[(size_t)i * 4]);
+        running += !fin[i];
+    }
+    *nrun = running;
+    MRS_HIP(hipMemcpyAsync(lm->gen_ints, h.data(), h.size() * sizeof(int), hipMemcpyHostToDevice, st));
+    MRS_HIP(hipMemcpyAsync(lm->gen_samplers, samplers.data(), samplers.size() * sizeof(mrs_sampler), hipMemcpyHostToDevice, st));
+    MRS_HIP(hipMemcpyAsync(lm->gen_rng, rng.data(), rng.size() * sizeof(unsigned long long), hipMemcpyHostToDevice, st));
+    MRS_HIP(hipMemcpyAsync(lm->gen_dyn, &lm->gen_dyn_host, sizeof(GenDyn), hipMemcpyHostToDevice, st));
+    if (total > 0) MRS_HIP(hipMemcpyAsync((void *)lm->gen_dyn_host.prompts, prompts, (size_t)total * sizeof(int), hipMemcpyHostToDevice, st));
+    MRS_HIP(hipMemcpyAsync(lm->tokens, first.data(), (size_t)B * sizeof(int), hipMemcpyHostToDevice, st));
+    MRS_HIP(hipMemsetAsync(lm->gen.seen, 0, (size_t)B * lm->vocab * sizeof(unsigned), st));
+    MRS_HIP(hipStreamSynchronize(st));   // the staging vectors above go out of use here
+    if (seen_includes_prompt && max_prompt > 0)
+        hipLaunchKernelGGL(gen_seen_prompt_kernel, dim3((unsigned)std::min(64, (max_prompt + 255) / 256), (unsigned)B), dim3(256), 0, st, lm->gen,
+                           lm->gen_dyn, B, lm->vocab);
+    MRS_TRY(mrs_backbone_reset(bb));
+    int steps = max_prompt + max_tokens;   // gpu_lm.rs:432
+    if (prefill_route && running) {
+        MRS_TRY(mrs_lm_prefill(lm, bb, prompts, prompt_lens[0]));   // state after the prompt, logits of its last position
+        MRS_TRY(gen_pick(lm));
+        steps = max_tokens;
+    }
+    int done = 0;
+    for (int s = 0; s < steps && running > 0; s++) {
+        if (lm->gen_graph_ready) {
+            MRS_HIP(hipGraphLaunch(lm->gen_graph_exec, st));
+        } else if (s == 1) {
+            // the first step ran eagerly (the GEMM library settles its choices); capture the step now and replay it from here on
+            MRS_HIP(hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal));
+            int rc = gen_forward(lm);
+            if (!rc) rc = gen_pick(lm);
+            hipGraph_t gph = nullptr;
+            hipError_t e = hipStreamEndCapture(st, &gph);
+            if (rc) { if (gph) hipGraphDestroy(gph); return rc; }
+            if (e != hipSuccess) return fail(MRS_E_HIP, "hipStreamEndCapture: %s", hipGetErrorString(e));
+            e = hipGraphInstantiate(&lm->gen_graph_exec, gph, nullptr, nullptr, 0);
+            if (e != hipSuccess) { hipGraphDestroy(gph); return fail(MRS_E_HIP, "hipGraphInstantiate: %s", hipGetErrorString(e)); }
+            lm->gen_graph = gph; lm->gen_graph_ready = 1;
+            MRS_HIP(hipGraphLaunch(lm->gen_graph_exec, st));
+        } else {
+            MRS_TRY(gen_forward(lm));
+            MRS_TRY(gen_pick(lm));
+        }
+        if (++done % 16 == 0 || s + 1 == steps) {   // the only host round trip of the loop: is anyone still running?
+            MRS_HIP(hipMemcpyAsync(&running, lm->gen.n_running, sizeof(int), hipMemcpyDeviceToHost, st));
+            MRS_HIP(hipStreamSynchronize(st));
+        }
+    }
+    MRS_HIP(hipMemcpyAsync(out_lens, lm->gen.out_len, (size_t)B * sizeof(int), hipMemcpyDeviceToHost, st));
+    MRS_HIP(hipMemcpy2DAsync(out_tokens, (size_t)out_stride * sizeof(int), lm->gen_dyn_host.out, (size_t)lm->gen_dyn_host.out_stride * sizeof(int),
+                             (size_t)std::min(out_stride, lm->gen_dyn_host.out_stride) * sizeof(int), B, hipMemcpyDeviceToHost, st));
+    MRS_HIP(hipStreamSynchronize(st));
+    return MRS_OK;
 }

@@ -245,3 +245,38 @@ def m3_ssd_fwd(ssm, kst, vst, y, x, K, Q, dt, trap, a_val, D, *, carry_state=Fal
               _p(a_val), _p(D), _p(workspace), ws_bytes, M3_CARRY_STATE if carry_state else 0, batch, x.shape[1], nh, hd, ds,
               chunk_size)
     return y
+
+
+def xoshiro_seed(seed: int) -> list[int]:
+    """Xoshiro256PlusPlus::new (src/module/sample.rs:54-66): the generator's four state words for a seed."""
+    import ctypes
+    st = (ctypes.c_uint64 * 4)()
+    _lib.load().mrs_xoshiro_seed(ctypes.c_uint64(seed & 0xFFFFFFFFFFFFFFFF), st)
+    return [int(v) for v in st]
+
+
+def sample_tokens(logits, samplers, rng_state, *, seen_counts=None, active=None):
+    """sample_token (src/module/sample.rs:243-265) for every row of logits [rows, vocab] f32 on the device.
+    samplers: float32 tensor [rows, 5] = (temperature, top_k, top_p, min_p, repetition_penalty) per row (top_k is
+    converted to the ABI's int field here); rng_state: int64 tensor [rows, 4] holding the xoshiro256++ words, advanced
+    in place; seen_counts: int32 [rows, vocab] or None; active: int32 [rows] or None.  Returns int32 tokens [rows]
+    (rows with active == 0 keep -1)."""
+    _dev(logits, rng_state); _f32(logits)
+    if logits.dim() != 2 or rng_state.shape != (logits.shape[0], 4) or rng_state.dtype != torch.int64:
+        raise ValueError("logits [rows, vocab] f32 and rng_state [rows, 4] int64 expected")
+    rows, vocab = logits.shape
+    sp = torch.as_tensor(samplers, dtype=torch.float32).reshape(rows, 5).cpu()
+    packed = torch.empty(rows, 5, dtype=torch.int32)
+    packed[:, 0] = sp[:, 0].view(torch.int32); packed[:, 1] = sp[:, 1].to(torch.int32)
+    packed[:, 2:] = sp[:, 2:].contiguous().view(torch.int32)
+    packed = packed.to(logits.device)
+    for t, name in ((seen_counts, "seen_counts"), (active, "active")):
+        if t is not None and (not t.is_cuda or t.dtype != torch.int32 or not t.is_contiguous()):
+            raise ValueError(f"{name} must be a contiguous int32 device tensor")
+    if seen_counts is not None and seen_counts.shape != (rows, vocab):
+        raise ValueError("seen_counts must be [rows, vocab]")
+    tokens = torch.full((rows,), -1, device=logits.device, dtype=torch.int32)
+    work = torch.empty_like(logits)
+    _lib.call("mrs_sample_tokens", _stream(), _p(tokens), _p(logits), _p(work), vocab, rows, vocab, _p(packed), _p(seen_counts),
+              _p(rng_state), _p(active))
+    return tokens

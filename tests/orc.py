@@ -328,3 +328,75 @@ def m3_backbone_step(P: M3Params, x, state, taps=False):
                         a_val=t[5 * nh:6 * nh], k=t[6 * nh:6 * nh + nh * ds].reshape(nh, ds),
                         q=t[6 * nh + nh * ds:].reshape(nh, ds)))
     return out, res
+
+
+# ---- sampling (oracle/sample_oracle.c) -----------------------------------------------------------------
+
+class Xoshiro:
+    """Xoshiro256PlusPlus of src/module/sample.rs:48-86."""
+
+    def __init__(self, seed=None, state=None):
+        self.s = (c_uint64 * 4)()
+        if state is not None:
+            for i, v in enumerate(state):
+                self.s[i] = v
+        else:
+            lib().orc_xoshiro_seed(c_uint64(seed), self.s)
+
+    def state(self):
+        return [int(v) for v in self.s]
+
+    def next_u64(self):
+        lib().orc_xoshiro_next_u64.restype = c_uint64
+        return int(lib().orc_xoshiro_next_u64(self.s))
+
+    def next_f32(self):
+        lib().orc_xoshiro_next_f32.restype = c_float
+        return float(lib().orc_xoshiro_next_f32(self.s))
+
+
+def _filter(name, x, *args):
+    x = np.array(x, dtype=np.float32, copy=True, order="C")
+    getattr(lib(), name)(_p(x), c_int64(x.size), *args)
+    return x
+
+
+def apply_repetition_penalty(logits, seen, penalty):
+    seen = np.ascontiguousarray(seen, dtype=np.uint32)
+    return _filter("orc_apply_repetition_penalty", logits, _p(seen), c_int64(seen.size), c_float(penalty))
+
+
+def apply_temperature(logits, t):
+    return _filter("orc_apply_temperature", logits, c_float(t))
+
+
+def apply_top_k(logits, k):
+    return _filter("orc_apply_top_k", logits, c_int64(k))
+
+
+def softmax(logits):
+    return _filter("orc_softmax_inplace", logits)
+
+
+def apply_top_p(probs, p):
+    return _filter("orc_apply_top_p", probs, c_float(p))
+
+
+def apply_min_p(probs, p):
+    return _filter("orc_apply_min_p", probs, c_float(p))
+
+
+def weighted_sample(probs, r):
+    probs = _c(probs)
+    lib().orc_weighted_sample.restype = ctypes.c_uint32
+    return int(lib().orc_weighted_sample(_p(probs), c_int64(probs.size), c_float(r)))
+
+
+def sample_token(logits, rng: Xoshiro, temperature=1.0, top_k=0, top_p=1.0, min_p=0.0, repetition_penalty=1.0, seen=()):
+    """sample_token (src/module/sample.rs:243-265) -> (token, the logits buffer as the call leaves it)."""
+    x = np.array(logits, dtype=np.float32, copy=True, order="C")
+    seen = np.ascontiguousarray(seen, dtype=np.uint32)
+    lib().orc_sample_token.restype = ctypes.c_uint32
+    tok = lib().orc_sample_token(_p(x), c_int64(x.size), c_float(temperature), c_int64(top_k), c_float(top_p), c_float(min_p),
+                                 c_float(repetition_penalty), _p(seen), c_int64(seen.size), rng.s)
+    return int(tok), x
