@@ -153,8 +153,18 @@ def lm_leg(name, cfg_kw, vocab, prefill_bt, decode_b, decode_steps, seed=42):
         di, dm, ds, dc, dr = cfg.d_inner(), cfg.d_model, cfg.d_state, cfg.d_conv, cfg.dt_rank()
         layer_bytes = es * (dm * 2 * di + di * (dr + 2 * ds) + dr * di + di * dm) + 2 * 4 * db * di * (ds + dc) + 2 * 4 * db * dm
         step_bytes = cfg.n_layers * layer_bytes + ((vocab + 63) // 64 * 64) * dm * es
-        dec_out.append({"batch": db, "steps": decode_steps, "us_per_step": td * 1e6, "tok_per_s": db / td,
-                        "algorithmic_bytes_per_step": step_bytes, "hbm_frac": step_bytes / td / 1e9 / HBM_PEAK_GBPS})
+        entry = {"batch": db, "steps": decode_steps, "us_per_step": td * 1e6, "tok_per_s": db / td,
+                 "algorithmic_bytes_per_step": step_bytes, "hbm_frac": step_bytes / td / 1e9 / HBM_PEAK_GBPS}
+        # batched generation with the sampler in the loop: ragged prompts of 8..12 tokens, 128 new tokens per slot
+        from mamba_rs_amd import SampleParams
+        prompts = [[int(t) for t in rng.integers(0, vocab, 8 + (i % 5))] for i in range(db)]
+        params = [SampleParams(temperature=0.8, top_k=50, top_p=0.9, max_tokens=128, seed=i) for i in range(db)]
+        lm_d.generate_batch(prompts, params)                       # warm-up (captures the step)
+        t0 = time.perf_counter(); gen = lm_d.generate_batch(prompts, params); tg = time.perf_counter() - t0
+        n_gen = sum(len(g) for g in gen)
+        entry["generate_batch"] = {"sampler": "temperature 0.8, top_k 50, top_p 0.9", "new_tokens": n_gen, "ms": tg * 1e3,
+                                   "us_per_step": tg / (12 + 128) * 1e6, "gen_tok_per_s": n_gen / tg}
+        dec_out.append(entry)
         lm_d.close(); dec.close()
     out["decode"] = dec_out
     return out

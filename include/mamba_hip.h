@@ -299,7 +299,7 @@ typedef struct { float temperature; int top_k; float top_p; float min_p; float r
 MRS_API void mrs_xoshiro_seed(unsigned long long seed, unsigned long long state[4]);
 
 /* All pointers are device memory.  tokens [rows] <- sampled ids; logits [rows, ld] f32 (read only); work [rows, ld]
- * f32 scratch; samplers [rows]; seen_counts [rows, vocab] occurrences of each token in the row's seen list, or null
+ * f32 scratch for the penalised rows (may be null when seen_counts is); samplers [rows]; seen_counts [rows, vocab] occurrences of each token in the row's seen list, or null
  * (no penalty); rng_state [rows, 4], advanced by one draw per sampled row; active [rows] or null: rows with 0 are
  * skipped (token, generator untouched). */
 MRS_API int mrs_sample_tokens(void *stream, int *tokens, const float *logits, float *work, int64_t ld, int rows, int vocab,
@@ -324,7 +324,8 @@ typedef struct {
  *   out_stride >= every max_tokens.
  * seen_includes_prompt = 0: the penalty sees the generated tokens only (generate_batch, gpu_lm.rs:470-487);
  * 1: prompt and generated tokens (generate_streaming, gpu_lm.rs:364-375), and a batch-1 engine takes prompts of 256
- * tokens or more through prefill (gpu_lm.rs:349). */
+ * tokens or more through prefill (gpu_lm.rs:349).  Resets the engine state, allocates its buffers on first use (and when
+ * a call needs larger ones) and synchronises the engine's stream before it returns. */
 MRS_API int mrs_lm_generate_batch(mrs_lm *lm, const int *prompts, const int *prompt_lens, const mrs_sample_params *params,
                                   int seen_includes_prompt, int *out_tokens, int out_stride, int *out_lens);
 

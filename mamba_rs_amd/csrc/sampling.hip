@@ -20,6 +20,7 @@ constexpr int kSampWaves = kSampThreads / kWave;
 constexpr int kListCap = 8192;   // bracket entries gathered into LDS
 constexpr int kMaxBlocks = 1024; // block totals of the index-ordered walk
 constexpr int kBinCopies = 32;   // copies of each histogram bin, one per lane modulo 32
+constexpr int kFinish = 512;     // a bracket this small is resolved by ranking its entries against each other
 
 struct SampShared {
     double d_slots[kSampWaves][16];
@@ -33,6 +34,8 @@ struct SampShared {
     uint32_t list[kListCap];
     unsigned long long bins[16 * kBinCopies];
     unsigned long long hist[16];
+    unsigned long long res_ge, res_gt;
+    uint32_t res_key;
 };
 
 template <typename T> __device__ __forceinline__ T wave_sum(T v) {
@@ -104,19 +107,25 @@ struct Row {
     const float *x;
     int vocab;
     bool vec;
+    float scale;   // 1 / temperature, applied on the way in (1 when the stored row already carries it)
+    __device__ __forceinline__ float at(int i) const { return x[i] * scale; }
+    __device__ __forceinline__ float4 at4(int i0) const {
+        float4 v = *reinterpret_cast<const float4 *>(x + i0);
+        v.x *= scale; v.y *= scale; v.z *= scale; v.w *= scale;
+        return v;
+    }
     template <typename F> __device__ __forceinline__ void each(F f) const {
         if (vec) {
-            const float4 *p = reinterpret_cast<const float4 *>(x);
             const int n4 = vocab >> 2;
 #pragma unroll 4
             for (int q = threadIdx.x; q < n4; q += kSampThreads) {
-                const float4 v = p[q];
+                const float4 v = at4(4 * q);
                 f(4 * q, v.x); f(4 * q + 1, v.y); f(4 * q + 2, v.z); f(4 * q + 3, v.w);
             }
-            for (int i = (n4 << 2) + threadIdx.x; i < vocab; i += kSampThreads) f(i, x[i]);
+            for (int i = (n4 << 2) + threadIdx.x; i < vocab; i += kSampThreads) f(i, at(i));
         } else {
 #pragma unroll 4
-            for (int i = threadIdx.x; i < vocab; i += kSampThreads) f(i, x[i]);
+            for (int i = threadIdx.x; i < vocab; i += kSampThreads) f(i, at(i));
         }
     }
 };
@@ -193,7 +202,7 @@ template <bool MASS, typename Get> __device__ SearchOut search_key(const Row &ro
             for (int i0 = 0; i0 < vocab; i0 += kSampThreads) {   // same trip count for all lanes: the ballots see whole waves
                 const int i = i0 + (int)threadIdx.x;
                 uint32_t key = 0;
-                const bool in = i < vocab && get(i, row.x[i], key) && key >= lo_now && key - lo_now < nspan;
+                const bool in = i < vocab && get(i, row.at(i), key) && key >= lo_now && key - lo_now < nspan;
                 const unsigned long long m = __ballot(in);
                 if (m) {
                     const int leader = (int)__ffsll((long long)m) - 1;
@@ -207,6 +216,28 @@ template <bool MASS, typename Get> __device__ SearchOut search_key(const Row &ro
             __syncthreads();
             n_list = sh.n_list;
             listed = n_list <= kListCap;
+            if (n_list <= kFinish) {
+                // few enough to finish at once: every listed key totals what lies above it and what equals it; the key
+                // whose "at or above" total reaches the goal while its "above" total does not is the answer
+                if (threadIdx.x == 0) { sh.res_key = lo; sh.res_ge = ge; sh.res_gt = above; }
+                __syncthreads();
+                if ((int)threadIdx.x < n_list) {
+                    const uint32_t mine = sh.list[threadIdx.x];
+                    unsigned long long g = above, e = 0;
+                    for (int u = 0; u < n_list; u++) {
+                        const uint32_t ku = sh.list[u];
+                        const unsigned long long c = MASS ? fixed_weight(ku) : 1ull;
+                        g += ku > mine ? c : 0ull;
+                        e += ku == mine ? c : 0ull;
+                    }
+                    const bool at = MASS ? g + e > thr : g + e >= thr, over = MASS ? g > thr : g >= thr;
+                    if (at && !over) { sh.res_key = mine; sh.res_ge = g + e; sh.res_gt = g; }   // equal keys write equal values
+                }
+                __syncthreads();
+                const SearchOut r{sh.res_key, sh.res_ge, sh.res_gt, thr};
+                __syncthreads();
+                return r;
+            }
         }
     }
     return SearchOut{lo, ge, gt, thr};
@@ -224,11 +255,11 @@ template <typename W> __device__ int ordered_find(const Row &row, W w, double ta
     const int nb = (vocab + bs - 1) / bs;
     auto load4 = [&](int i0, float (&v)[4]) {   // weights of entries i0 .. i0+3 (0 past the end)
         if (row.vec && i0 + 3 < vocab) {
-            const float4 q = *reinterpret_cast<const float4 *>(row.x + i0);
+            const float4 q = row.at4(i0);
             v[0] = w(i0, q.x); v[1] = w(i0 + 1, q.y); v[2] = w(i0 + 2, q.z); v[3] = w(i0 + 3, q.w);
         } else {
 #pragma unroll
-            for (int c = 0; c < 4; c++) v[c] = i0 + c < vocab ? w(i0 + c, row.x[i0 + c]) : 0.0f;
+            for (int c = 0; c < 4; c++) v[c] = i0 + c < vocab ? w(i0 + c, row.at(i0 + c)) : 0.0f;
         }
     };
 #pragma unroll 2
@@ -315,8 +346,7 @@ template <typename W> __device__ int ordered_find(const Row &row, W w, double ta
 
 __device__ __forceinline__ uint64_t rotl64(uint64_t x, int k) { return (x << k) | (x >> (64 - k)); }
 
-// logits [rows, ld] f32 are read only; `work` [rows, ld] receives the penalised / scaled logits of rows that need
-// them.  seen [rows, vocab] counts how often a token sits in the row's seen list (the penalty is applied once per
+// logits [rows, ld] f32 are read only; `work` [rows, ld] receives the penalised logits of rows with a penalty.  seen [rows, vocab] counts how often a token sits in the row's seen list (the penalty is applied once per
 // occurrence, sample.rs:100-109).  rng [rows, 4] advances by one draw per sampled row (none on the greedy branch).
 // Rows with active[row] == 0 are left alone.
 __global__ __launch_bounds__(kSampThreads) void sample_rows_kernel(int *__restrict__ tokens, const float *__restrict__ logits,
@@ -338,16 +368,14 @@ __global__ __launch_bounds__(kSampThreads) void sample_rows_kernel(int *__restri
     const bool vec = (ld % 4 == 0) && (reinterpret_cast<uintptr_t>(logits) % 16 == 0) && (reinterpret_cast<uintptr_t>(work) % 16 == 0);
 
     // pass 1: penalty and temperature; maximum (and, for the greedy branch, the last index holding it)
-    Row row{lrow, vocab, vec};
+    Row row{lrow, vocab, vec, 1.0f};
     float best = -INFINITY;
     int bi = 0;
-    if (pen_on || scale_on) {
+    if (pen_on) {   // the penalised (and scaled) row goes to `work`; later passes read it from there
         float *wrow = work + (int64_t)rowi * ld;
-        const unsigned *srow = pen_on ? seen + (int64_t)rowi * vocab : nullptr;
+        const unsigned *srow = seen + (int64_t)rowi * vocab;
         row.each([&](int i, float x) {
-            if (pen_on) {
-                for (unsigned c = srow[i]; c > 0; c--) x = x > 0.0f ? x / pen : x * pen;
-            }
+            for (unsigned c = srow[i]; c > 0; c--) x = x > 0.0f ? x / pen : x * pen;
             x *= inv_t;
             wrow[i] = x;
             if (x >= best) { best = x; bi = i; }   // a thread meets its entries in ascending index order
@@ -355,6 +383,7 @@ __global__ __launch_bounds__(kSampThreads) void sample_rows_kernel(int *__restri
         row.x = wrow;
         __syncthreads();   // the row is read back by other threads below (same workgroup, global memory)
     } else {
+        row.scale = inv_t;   // temperature alone is applied on every read
         row.each([&](int i, float x) {
             if (x >= best) { best = x; bi = i; }
         });
@@ -474,6 +503,6 @@ extern "C" int mrs_sample_tokens(void *stream, int *tokens, const float *logits,
                                  const int *active) {
     using namespace mrs;
     if (!tokens || !logits || !samplers || !rng_state) return fail(MRS_E_NULL, "mrs_sample_tokens: null pointer");
-    if (!work) return fail(MRS_E_NULL, "mrs_sample_tokens: the work buffer [rows, ld] is needed for rows with a penalty or a temperature");
+    if (seen_counts && !work) return fail(MRS_E_NULL, "mrs_sample_tokens: rows with a repetition penalty need the work buffer [rows, ld]");
     return launch_sample_rows(as_stream(stream), tokens, logits, work, ld, rows, vocab, samplers, seen_counts, rng_state, active);
 }
