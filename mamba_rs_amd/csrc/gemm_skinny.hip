@@ -15,6 +15,7 @@
 //     straight through the depthwise conv step + SiLU (conv1d_step_forward_silu, kernels/conv1d.cu:85-115)
 //     and only u and the gate half are written.
 #include "common.hpp"
+#include <stdlib.h>
 
 namespace mrs {
 
@@ -37,6 +38,25 @@ template <> struct Mma32<f16_t> {
 constexpr int kGemmWaves = 8;
 constexpr int kMaxConvTaps = 8;
 
+// 8 products of a 16-byte pair of operand chunks, f32 accumulate (v_dot2_f32_bf16 / v_dot2_f32_f16)
+typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+template <typename T> struct Dot2;
+template <> struct Dot2<bf16_t> {
+    __device__ static __forceinline__ float f(uint32_t a, uint32_t b, float c) {
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(v2bf, a), __builtin_bit_cast(v2bf, b), c, false);
+    }
+};
+template <> struct Dot2<f16_t> {
+    __device__ static __forceinline__ float f(uint32_t a, uint32_t b, float c) {
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(v2h, a), __builtin_bit_cast(v2h, b), c, false);
+    }
+};
+template <typename T> __device__ __forceinline__ float dot8(uint4 a, uint4 b, float c) {
+    c = Dot2<T>::f(a.x, b.x, c); c = Dot2<T>::f(a.y, b.y, c); c = Dot2<T>::f(a.z, b.z, c);
+    return Dot2<T>::f(a.w, b.w, c);
+}
+
 template <typename TO> __device__ __forceinline__ void store_out(TO *p, float v) { Store<TO>::st(p, v); }
 
 // EPI 0: C[row, col] = sum (TO = T or float)
@@ -55,11 +75,18 @@ constexpr int kStepsPerBatch = 6;  // k-steps whose loads are issued together (c
 // rms comes from the row's partial sums of squares, which the out_proj epilogue before it (or
 // prenorm_rows_kernel for the first layer) left behind together with A.  Against the reference's order the
 // rounding to the storage type happens before the row scale instead of after it: same relative error.
-template <typename T, typename TO, int EPI, int PRO>
-__global__ __launch_bounds__(kGemmWaves * 64) void skinny_gemm_kernel(
+//
+// LPR != 0 (M <= 4, one row tile): no matrix cores.  At one to four rows the product is a pass over the weight and
+// nothing else, so the layout follows the memory system: LPR lanes (64 or 32) walk one weight row in consecutive
+// 16-byte pieces -- whole kilobytes of one row per load instruction instead of 64-byte pieces of 16 rows -- each wave
+// owns two of the workgroup's 16 columns, all of its loads are in flight at once (in groups of JB per column), and
+// the products are v_dot2 with f32 accumulate.  The epilogues are the same code.  MR = rows computed (1 or 4).
+template <typename T, typename TO, int EPI, int PRO, int LPR = 0, int MR = 1>
+__global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu(6))) void skinny_gemm_kernel(
     TO *__restrict__ C, int64_t ldc, const T *__restrict__ A, int64_t lda, const T *__restrict__ Wt, int M, int N, int K,
     SkinnyEpi ep) {
-    __shared__ v4f red[kGemmWaves / 2][kWave];
+    __shared__ v4f red[LPR ? 1 : kGemmWaves / 2][kWave];
+    __shared__ float gv[4][16];   // LPR != 0: the [row][column] sums of the workgroup
     const int n0 = blockIdx.x * 16, m0 = blockIdx.y * 16;
     const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, lr = l & 15, lg = l >> 4;
     const int nk = K >> 5;
@@ -111,6 +138,52 @@ __global__ __launch_bounds__(kGemmWaves * 64) void skinny_gemm_kernel(
     // megabyte-scale read that would queue ahead of the operands, so there they are fetched after the product.
     const bool early = EPI == 2 || (EPI == 1 && gridDim.y == 1);
     if (early) prefetch_epilogue();
+    if constexpr (LPR != 0) {
+        constexpr int NC = LPR == 64 ? 2 : 1;           // columns a lane works on (with 32 lanes per row each half-wave has its own)
+        constexpr int JB = MR > 1 ? 2 : 4;              // pieces per column requested together
+        const int ll = l & (LPR - 1), half = LPR == 64 ? 0 : (l >> 5);
+        const int per = (K >> 3) / LPR;                 // 16-byte pieces of a row per lane
+        const T *wp[NC];
+#pragma unroll
+        for (int t = 0; t < NC; t++) wp[t] = Wt + (int64_t)min(n0 + 2 * w + (LPR == 64 ? t : half), N - 1) * K + 8 * ll;
+        float sum[NC][MR];
+#pragma unroll
+        for (int t = 0; t < NC; t++)
+#pragma unroll
+            for (int m = 0; m < MR; m++) sum[t][m] = 0.0f;
+        for (int jb = 0; jb < per; jb += JB) {
+            uint4 wv[NC][JB], av[MR][JB];
+#pragma unroll
+            for (int j = 0; j < JB; j++) {
+                if (jb + j < per) {
+                    const int off = 8 * LPR * (jb + j);
+#pragma unroll
+                    for (int t = 0; t < NC; t++) wv[t][j] = *reinterpret_cast<const uint4 *>(wp[t] + off);
+#pragma unroll
+                    for (int m = 0; m < MR; m++) av[m][j] = *reinterpret_cast<const uint4 *>(A + (int64_t)min(m, M - 1) * lda + 8 * ll + off);
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < JB; j++) {
+                if (jb + j < per) {
+#pragma unroll
+                    for (int t = 0; t < NC; t++)
+#pragma unroll
+                        for (int m = 0; m < MR; m++) sum[t][m] = dot8<T>(av[m][j], wv[t][j], sum[t][m]);
+                }
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < NC; t++)
+#pragma unroll
+            for (int m = 0; m < MR; m++) {
+                float v = sum[t][m];
+#pragma unroll
+                for (int x = LPR / 2; x >= 1; x >>= 1) v += __shfl_xor(v, x, kWave);
+                if (ll == 0) gv[m][2 * w + (LPR == 64 ? t : half)] = v;
+            }
+        __syncthreads();
+    } else {
     for (int base = w; base < nk; base += kGemmWaves * kStepsPerBatch) {
         uint4 bf[kStepsPerBatch], af[kStepsPerBatch];
 #pragma unroll
@@ -130,14 +203,19 @@ __global__ __launch_bounds__(kGemmWaves * 64) void skinny_gemm_kernel(
     __syncthreads();
     if (w < kGemmWaves / 2) red[w][l] += acc;
     __syncthreads();
+    }
     // element e of the 16x16 tile: row ml = e / 16, column nl = e % 16 lives in lane 16 (ml / 4) + nl, register ml % 4
     if (tid < 256) {
         if (EPI != 0 && !early) prefetch_epilogue();
         const int ml = tid >> 4, nl = tid & 15;
         const int lane = (ml >> 2) * 16 + nl, i = ml & 3;
         float s = 0.0f;
+        if constexpr (LPR != 0) {
+            s = ml < MR ? gv[ml & 3][nl] : 0.0f;
+        } else {
 #pragma unroll
-        for (int ww = 0; ww < kGemmWaves / 2; ww++) s += red[ww][lane][i];
+            for (int ww = 0; ww < kGemmWaves / 2; ww++) s += red[ww][lane][i];
+        }
         s *= inv;
         const int row = m0 + ml, col = n0 + nl;
         const bool valid = row < M && col < N;
@@ -272,7 +350,17 @@ template <typename T, typename TO>
 static int launch_skinny_t(hipStream_t st, TO *C, int64_t ldc, const T *A, int64_t lda, const T *Wt, int M, int N, int K,
                            const SkinnyEpi &ep) {
     const dim3 grid((unsigned)((N + 15) / 16), (unsigned)((M + 15) / 16)), block(kGemmWaves * 64);
-#define MRS_SG(EPI_, PRO_) hipLaunchKernelGGL((skinny_gemm_kernel<T, TO, EPI_, PRO_>), grid, block, 0, st, C, ldc, A, lda, Wt, M, N, K, ep)
+    // one to four rows: the lanes-along-the-row route (64 lanes per weight row when a row is a multiple of 1 KB, else 32)
+    static const bool no_rowwise = getenv("MRS_DECODE_NO_ROWWISE") != nullptr;
+    const int lpr = (M > 4 || no_rowwise) ? 0 : (K % 512 == 0 ? 64 : (K % 256 == 0 ? 32 : 0));
+#define MRS_SG(EPI_, PRO_)                                                                                                               \
+    do {                                                                                                                                 \
+        if (lpr == 64 && M == 1) hipLaunchKernelGGL((skinny_gemm_kernel<T, TO, EPI_, PRO_, 64, 1>), grid, block, 0, st, C, ldc, A, lda, Wt, M, N, K, ep); \
+        else if (lpr == 64) hipLaunchKernelGGL((skinny_gemm_kernel<T, TO, EPI_, PRO_, 64, 4>), grid, block, 0, st, C, ldc, A, lda, Wt, M, N, K, ep);     \
+        else if (lpr == 32 && M == 1) hipLaunchKernelGGL((skinny_gemm_kernel<T, TO, EPI_, PRO_, 32, 1>), grid, block, 0, st, C, ldc, A, lda, Wt, M, N, K, ep); \
+        else if (lpr == 32) hipLaunchKernelGGL((skinny_gemm_kernel<T, TO, EPI_, PRO_, 32, 4>), grid, block, 0, st, C, ldc, A, lda, Wt, M, N, K, ep);     \
+        else hipLaunchKernelGGL((skinny_gemm_kernel<T, TO, EPI_, PRO_>), grid, block, 0, st, C, ldc, A, lda, Wt, M, N, K, ep);           \
+    } while (0)
     const bool pro = ep.row_scale != 0;
     if (ep.mode != 0 && sizeof(TO) != sizeof(T)) return fail(MRS_E_DTYPE, "skinny gemm: fused epilogues store the activation type");
     if constexpr (sizeof(TO) == sizeof(T)) {

@@ -13,7 +13,9 @@ ops = pytest.importorskip("mamba_rs_amd.ops")
 
 # (M, N, K): the 130m decode projections at batch 64 and 1, ragged M / N, the smallest K
 SHAPES = [(64, 3072, 768), (64, 80, 1536), (64, 768, 1536), (1, 3072, 768), (1, 80, 1536), (5, 33, 32), (17, 100, 96),
-          (48, 16, 2560), (33, 1000, 64), (64, 50, 1024)]
+          (48, 16, 2560), (33, 1000, 64), (64, 50, 1024),
+          # one to four rows: lanes-along-the-row route (64 lanes per weight row at K % 512 == 0, 32 at K % 256 == 0)
+          (1, 10240, 2560), (1, 192, 5120), (2, 2560, 5120), (3, 100, 512), (4, 33, 768), (1, 7, 256), (4, 3072, 768), (2, 50, 1280)]
 
 
 @pytest.mark.parametrize("dtype", [orc.BF16, orc.F16])
