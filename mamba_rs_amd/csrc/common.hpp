@@ -62,10 +62,13 @@ int fail(int code, const char *fmt, ...);
 int check_launch(const char *what);
 
 // Internal launchers shared with the backbone engine (strides and fusions the public entry points do not expose).
+// StepFold: the step kernel forms the x_proj row itself from per-tile shares [n_tiles][rows][xd] f32 (summed in tile
+// order, rounded to the storage type); dt input at element 0, B at b_off, C at c_off of the row.
+struct StepFold { const float *xpart; int n_tiles, rows, xd, b_off, c_off; };
 int launch_ssm_step_fused(hipStream_t st, int dtype, float *h, void *y, const void *delta, const float *dt_bias,
                           const void *dt_in, const void *dt_w, int dr, int dt_transposed, const void *u, const void *Bb, const void *Cb, int64_t bc_stride, const void *gate,
                           int64_t gate_stride, int gate_mode, const float *a_neg, const float *D, int batch,
-                          int di, int ds);
+                          int di, int ds, const StepFold *fold = nullptr);
 int launch_conv1d_step(hipStream_t st, int dtype, void *out, float *state, const void *new_x, int64_t x_stride,
                        const float *weight, const float *bias, int batch, int d_inner, int d_conv, int apply_silu);
 
@@ -88,6 +91,11 @@ struct SkinnyEpi {
     // 1/rms[row], rms from the row's partials (row_scale != 0)
     int row_scale;
     float eps;
+    // mode 1, optional: x_proj's products ride in the same launch (a few rows only).  Every x-half workgroup leaves its
+    // 16 columns' share u[row, 16 cols] . xw[16 rows, xd] in xpart[tile][row][xd]; the step kernel sums the tiles.
+    const void *xw;      // [di][xd] activation type (row-major, not transposed), or null
+    int xd;
+    float *xpart;        // [di / 16][M][xd] f32
 };
 bool skinny_gemm_ok(int dtype, int M, int N, int K, int64_t lda, const void *A, const void *Wt);
 int launch_skinny_gemm(hipStream_t st, int dtype, void *C, int out_f32, int64_t ldc, const void *A, int64_t lda, const void *Wt,

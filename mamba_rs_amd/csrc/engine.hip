@@ -215,11 +215,14 @@ struct LayerDev {
     int s4d;
 };
 
+constexpr int kFoldXprojFloats = 32768;   // largest [d_inner/16][rows][xdbl] block of shares the folded x_proj may use
+
 struct Scratch {  // activations for M rows
     int64_t rows = 0;
     void *normed = nullptr, *proj = nullptr, *u = nullptr, *xdbl = nullptr, *delta = nullptr, *y = nullptr, *out = nullptr;
     float *residual = nullptr;
     float *partials = nullptr;  // [rows][d_model/16] row sums of squares, decode chain only
+    float *xpart = nullptr;     // decode chain, a few rows: per-tile shares of the folded x_proj
     void *scan_ws = nullptr;
     size_t scan_ws_bytes = 0;
     int T = 0;
@@ -282,6 +285,12 @@ static int alloc_scratch(mrs_backbone *bb, Scratch *s, int64_t rows, int T) {
     MRS_TRY(dev_alloc(bb, &s->y, rows * di * es));
     MRS_TRY(dev_alloc(bb, &s->out, rows * dm * es));
     if (T == 1) MRS_TRY(dev_alloc(bb, (void **)&s->partials, rows * (size_t)((dm + 15) / 16) * sizeof(float)));
+    if (T == 1 && bb->skinny && rows <= 4) {
+        static const bool no_fold = getenv("MRS_DECODE_NO_FOLDED_XPROJ") != nullptr;
+        if (!no_fold) {
+            MRS_TRY(dev_alloc(bb, (void **)&s->xpart, (size_t)kFoldXprojFloats * sizeof(float)));
+        }
+    }
     if (T > 1) {
         s->scan_ws_bytes = mrs_ssm_scan_workspace_bytes(bb->batch, T, di, bb->cfg.d_state);
         MRS_TRY(dev_alloc(bb, &s->scan_ws, s->scan_ws_bytes));
@@ -364,9 +373,14 @@ static int run_layers(mrs_backbone *bb, Scratch *s, int T) {
             SkinnyEpi inp = {};
             inp.mode = 1; inp.conv_state = conv; inp.conv_w = lw.conv_w; inp.conv_b = lw.conv_b; inp.u = s->u; inp.di = di; inp.dc = dc;
             inp.row_scale = 1; inp.partials = s->partials; inp.n_partials = P; inp.eps = bb->cfg.rms_norm_eps;
+            // a few rows: x_proj rides in the same launch (its 16-column shares are summed by the last workgroup to finish)
+            const bool fold_x = s->xpart && B <= 4 && xd <= 256 && (int64_t)(di / 16) * B * xd <= kFoldXprojFloats && lw.dt_t_step &&
+                                di % (1024 / ds) == 0 && dr % 4 == 0 && (int64_t)B * dr <= kFuseDtProjLimit;
+            if (fold_x) { inp.xw = lw.x_proj; inp.xd = xd; inp.xpart = s->xpart; }
+            const StepFold fold = {s->xpart, di / 16, B, xd, dr, dr + ds};
             MRS_TRY(launch_skinny_gemm(bb->stream, dt, s->proj, 0, 2 * di, s->normed, dm, lw.in_proj_t, B, 2 * di, dm, inp));
             const SkinnyEpi none = {};
-            MRS_TRY(launch_skinny_gemm(bb->stream, dt, s->xdbl, 0, xd, s->u, di, lw.x_proj_t, B, xd, di, none));
+            if (!fold_x) MRS_TRY(launch_skinny_gemm(bb->stream, dt, s->xdbl, 0, xd, s->u, di, lw.x_proj_t, B, xd, di, none));
             if ((int64_t)B * dr > kFuseDtProjLimit && lw.dt_w_t && skinny_gemm_ok(dt, B, di, dr, xd, s->xdbl, lw.dt_w_t)) {
                 // wide dt_rank at a large batch: dt_proj as a GEMM of its own, bias + softplus in the step kernel
                 MRS_TRY(launch_skinny_gemm(bb->stream, dt, s->delta, 0, di, s->xdbl, xd, lw.dt_w_t, B, di, dr, none));
@@ -375,7 +389,7 @@ static int run_layers(mrs_backbone *bb, Scratch *s, int T) {
             } else {
                 MRS_TRY(launch_ssm_step_fused(bb->stream, dt, ssm, s->y, s->delta, lw.dt_b, s->xdbl, lw.dt_t_step ? lw.dt_w_t : lw.dt_w, dr,
                                               lw.dt_t_step, s->u, xb + es * dr,
-                                              xb + es * (dr + ds), xd, z, 2 * di, 2, lw.a_neg, lw.D, B, di, ds));
+                                              xb + es * (dr + ds), xd, z, 2 * di, 2, lw.a_neg, lw.D, B, di, ds, fold_x ? &fold : nullptr));
             }
             SkinnyEpi outp = {};
             outp.mode = 2; outp.residual = s->residual; outp.partials = s->partials; outp.n_partials = P;

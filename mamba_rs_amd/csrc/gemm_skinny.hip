@@ -80,7 +80,7 @@ constexpr int kStepsPerBatch = 6;  // k-steps whose loads are issued together (c
 // nothing else, so the layout follows the memory system: LPR lanes (64 or 32) walk one weight row in consecutive
 // 16-byte pieces -- whole kilobytes of one row per load instruction instead of 64-byte pieces of 16 rows -- each wave
 // owns two of the workgroup's 16 columns, all of its loads are in flight at once (in groups of JB per column), and
-// the products are v_dot2 with f32 accumulate.  The epilogues are the same code.  MR = rows computed (1 or 4).
+// the products are v_dot2 with f32 accumulate.  The epilogues are the same code.  MR = rows computed (1, 2 or 4; at 8 rows the route was slower than the matrix-core tiles: 642 vs 435 us per 130m-shape step).
 template <typename T, typename TO, int EPI, int PRO, int LPR = 0, int MR = 1>
 __global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu(6))) void skinny_gemm_kernel(
     TO *__restrict__ C, int64_t ldc, const T *__restrict__ A, int64_t lda, const T *__restrict__ Wt, int M, int N, int K,
@@ -140,7 +140,7 @@ __global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu
     if (early) prefetch_epilogue();
     if constexpr (LPR != 0) {
         constexpr int NC = LPR == 64 ? 2 : 1;           // columns a lane works on (with 32 lanes per row each half-wave has its own)
-        constexpr int JB = MR > 1 ? 2 : 4;              // pieces per column requested together
+        constexpr int JB = LPR == 64 ? 2 : 4;             // pieces per column requested together
         const int ll = l & (LPR - 1), half = LPR == 64 ? 0 : (l >> 5);
         const int per = (K >> 3) / LPR;                 // 16-byte pieces of a row per lane
         const T *wp[NC];
@@ -151,27 +151,70 @@ __global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu
         for (int t = 0; t < NC; t++)
 #pragma unroll
             for (int m = 0; m < MR; m++) sum[t][m] = 0.0f;
+        if constexpr (MR == 1) {
+            // one row: each lane reads its own pieces of it next to the weight pieces (the row is 1/2 of a wave's bytes)
+            constexpr int J1 = 4;
+            for (int jb = 0; jb < per; jb += J1) {
+                uint4 wv[NC][J1], av[J1];
+#pragma unroll
+                for (int j = 0; j < J1; j++) {
+                    if (jb + j < per) {
+                        const int off = 8 * LPR * (jb + j);
+#pragma unroll
+                        for (int t = 0; t < NC; t++) wv[t][j] = *reinterpret_cast<const uint4 *>(wp[t] + off);
+                        av[j] = *reinterpret_cast<const uint4 *>(A + 8 * ll + off);
+                    }
+                }
+#pragma unroll
+                for (int j = 0; j < J1; j++) {
+                    if (jb + j < per) {
+#pragma unroll
+                        for (int t = 0; t < NC; t++) sum[t][0] = dot8<T>(av[j], wv[t][j], sum[t][0]);
+                    }
+                }
+            }
+        } else {
+        // two to four rows go through LDS once per workgroup: read per wave from memory they would add M/2 times the
+        // weight bytes to what the workgroup pulls through its L1, which is what bounds this kernel
+        extern __shared__ uint4 a_lds[];                // [MR][K / 8]
+        const int kq = K >> 3;
+        for (int i = tid; i < MR * kq; i += kGemmWaves * 64) {
+            const int m = i / kq, q = i - m * kq;
+            a_lds[i] = *reinterpret_cast<const uint4 *>(A + (int64_t)min(m, M - 1) * lda + 8 * q);
+        }
+        // the first round of weight loads is issued before the barrier that publishes the rows
+        uint4 wv[NC][JB];
+#pragma unroll
+        for (int j = 0; j < JB; j++)
+            if (j < per) {
+#pragma unroll
+                for (int t = 0; t < NC; t++) wv[t][j] = *reinterpret_cast<const uint4 *>(wp[t] + 8 * LPR * j);
+            }
+        __syncthreads();
         for (int jb = 0; jb < per; jb += JB) {
-            uint4 wv[NC][JB], av[MR][JB];
+            uint4 nx[NC][JB];
 #pragma unroll
-            for (int j = 0; j < JB; j++) {
-                if (jb + j < per) {
-                    const int off = 8 * LPR * (jb + j);
+            for (int j = 0; j < JB; j++)
+                if (jb + JB + j < per) {
 #pragma unroll
-                    for (int t = 0; t < NC; t++) wv[t][j] = *reinterpret_cast<const uint4 *>(wp[t] + off);
-#pragma unroll
-                    for (int m = 0; m < MR; m++) av[m][j] = *reinterpret_cast<const uint4 *>(A + (int64_t)min(m, M - 1) * lda + 8 * ll + off);
+                    for (int t = 0; t < NC; t++) nx[t][j] = *reinterpret_cast<const uint4 *>(wp[t] + 8 * LPR * (jb + JB + j));
                 }
-            }
 #pragma unroll
             for (int j = 0; j < JB; j++) {
                 if (jb + j < per) {
 #pragma unroll
-                    for (int t = 0; t < NC; t++)
+                    for (int m = 0; m < MR; m++) {
+                        const uint4 av = a_lds[m * kq + ll + LPR * (jb + j)];
 #pragma unroll
-                        for (int m = 0; m < MR; m++) sum[t][m] = dot8<T>(av[m][j], wv[t][j], sum[t][m]);
+                        for (int t = 0; t < NC; t++) sum[t][m] = dot8<T>(av, wv[t][j], sum[t][m]);
+                    }
                 }
             }
+#pragma unroll
+            for (int j = 0; j < JB; j++)
+#pragma unroll
+                for (int t = 0; t < NC; t++) wv[t][j] = nx[t][j];
+        }
         }
 #pragma unroll
         for (int t = 0; t < NC; t++)
@@ -205,6 +248,7 @@ __global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu
     __syncthreads();
     }
     // element e of the 16x16 tile: row ml = e / 16, column nl = e % 16 lives in lane 16 (ml / 4) + nl, register ml % 4
+    float u_out = 0.0f;   // mode 1: this thread's u as stored (0 for gate columns / rows past M)
     if (tid < 256) {
         if (EPI != 0 && !early) prefetch_epilogue();
         const int ml = tid >> 4, nl = tid & 15;
@@ -252,9 +296,27 @@ __global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu
                         st[k] = wk;
                     }
             }
-            Store<T>::st(reinterpret_cast<T *>(ep.u) + (int64_t)row * ep.di + col, silu(o));
+            const T ur = (T)silu(o);
+            reinterpret_cast<T *>(ep.u)[(int64_t)row * ep.di + col] = ur;
+            u_out = Store<T>::ld(&ur);
         } else {
             store_out<TO>(C + (int64_t)row * ldc + col, s);
+        }
+    }
+    if constexpr (EPI == 1) {
+        if (ep.xw != nullptr && n0 < ep.di) {   // the same for the whole workgroup
+            __shared__ float ush[4][16];
+            if (tid < 64) ush[tid >> 4][tid & 15] = u_out;
+            __syncthreads();
+            const int xd = ep.xd, P = M * xd;   // P <= 512 (checked by the launcher)
+            const T *xw = reinterpret_cast<const T *>(ep.xw);
+            if (tid < P) {
+                const int m = tid / xd, j = tid - m * xd;
+                float a = 0.0f;
+#pragma unroll
+                for (int c = 0; c < 16; c++) a = fmaf(ush[m][c], Store<T>::ld(xw + (int64_t)min(n0 + c, ep.di - 1) * xd + j), a);
+                ep.xpart[(int64_t)blockIdx.x * P + tid] = a;
+            }
         }
     }
 }
@@ -352,13 +414,15 @@ static int launch_skinny_t(hipStream_t st, TO *C, int64_t ldc, const T *A, int64
     const dim3 grid((unsigned)((N + 15) / 16), (unsigned)((M + 15) / 16)), block(kGemmWaves * 64);
     // one to four rows: the lanes-along-the-row route (64 lanes per weight row when a row is a multiple of 1 KB, else 32)
     static const bool no_rowwise = getenv("MRS_DECODE_NO_ROWWISE") != nullptr;
-    const int lpr = (M > 4 || no_rowwise) ? 0 : (K % 512 == 0 ? 64 : (K % 256 == 0 ? 32 : 0));
+    const int lpr = (M > 4 || no_rowwise || (int64_t)K * 8 > 48 * 1024) ? 0 : (K % 512 == 0 ? 64 : (K % 256 == 0 ? 32 : 0));   // rows fit in LDS
 #define MRS_SG(EPI_, PRO_)                                                                                                               \
     do {                                                                                                                                 \
         if (lpr == 64 && M == 1) hipLaunchKernelGGL((skinny_gemm_kernel<T, TO, EPI_, PRO_, 64, 1>), grid, block, 0, st, C, ldc, A, lda, Wt, M, N, K, ep); \
-        else if (lpr == 64) hipLaunchKernelGGL((skinny_gemm_kernel<T, TO, EPI_, PRO_, 64, 4>), grid, block, 0, st, C, ldc, A, lda, Wt, M, N, K, ep);     \
+        else if (lpr == 64 && M == 2) hipLaunchKernelGGL((skinny_gemm_kernel<T, TO, EPI_, PRO_, 64, 2>), grid, block, (size_t)K * 4, st, C, ldc, A, lda, Wt, M, N, K, ep); \
+        else if (lpr == 32 && M == 2) hipLaunchKernelGGL((skinny_gemm_kernel<T, TO, EPI_, PRO_, 32, 2>), grid, block, (size_t)K * 4, st, C, ldc, A, lda, Wt, M, N, K, ep); \
+        else if (lpr == 64) hipLaunchKernelGGL((skinny_gemm_kernel<T, TO, EPI_, PRO_, 64, 4>), grid, block, (size_t)K * 8, st, C, ldc, A, lda, Wt, M, N, K, ep);     \
         else if (lpr == 32 && M == 1) hipLaunchKernelGGL((skinny_gemm_kernel<T, TO, EPI_, PRO_, 32, 1>), grid, block, 0, st, C, ldc, A, lda, Wt, M, N, K, ep); \
-        else if (lpr == 32) hipLaunchKernelGGL((skinny_gemm_kernel<T, TO, EPI_, PRO_, 32, 4>), grid, block, 0, st, C, ldc, A, lda, Wt, M, N, K, ep);     \
+        else if (lpr == 32) hipLaunchKernelGGL((skinny_gemm_kernel<T, TO, EPI_, PRO_, 32, 4>), grid, block, (size_t)K * 8, st, C, ldc, A, lda, Wt, M, N, K, ep);     \
         else hipLaunchKernelGGL((skinny_gemm_kernel<T, TO, EPI_, PRO_>), grid, block, 0, st, C, ldc, A, lda, Wt, M, N, K, ep);           \
     } while (0)
     const bool pro = ep.row_scale != 0;
@@ -384,6 +448,8 @@ int launch_skinny_gemm(hipStream_t st, int dtype, void *C, int out_f32, int64_t 
                                  "(got dtype=%d M=%d N=%d K=%d lda=%lld)", dtype, M, N, K, (long long)lda);
     if (ep.mode == 1 && (ep.dc < 1 || ep.dc > kMaxConvTaps || ep.di < 1 || ep.di > N || !ep.conv_state || !ep.conv_w || !ep.conv_b || !ep.u))
         return fail(MRS_E_SHAPE, "skinny gemm: bad in_proj epilogue (di=%d dc=%d)", ep.di, ep.dc);
+    if (ep.mode == 1 && ep.xw && (M > 4 || ep.xd < 1 || M * ep.xd > kGemmWaves * 64 || ep.di % 16 != 0 || !ep.xpart))
+        return fail(MRS_E_SHAPE, "skinny gemm: bad folded x_proj (M=%d xd=%d di=%d)", M, ep.xd, ep.di);
     if (ep.mode == 2 && (!ep.residual || !ep.partials || ep.n_partials != (N + 15) / 16 || (ep.next_norm_w && !ep.prenorm)))
         return fail(MRS_E_SHAPE, "skinny gemm: bad out_proj epilogue (n_partials=%d, column tiles=%d)", ep.n_partials, (N + 15) / 16);
     if (ep.row_scale && (!ep.partials || ep.n_partials < 1))

@@ -35,14 +35,21 @@ template <typename T> __device__ __forceinline__ void ld4(const T *p, float (&o)
 // ([d_inner][dt_rank]) and dt_rank / LG is a multiple of 4, so lane g takes the contiguous terms
 // [g dt_rank/LG, (g+1) dt_rank/LG) of both operands as 4-element vectors.
 constexpr int kStepVecBC = 1, kStepDtT = 2;
+constexpr int kFoldMaxXd = 256;
 
-template <typename T, int LG>
+// FOLD: the x_proj row (dt input, B, C) has not been formed yet -- the in_proj launch before left its 16-column
+// shares in fold.xpart [tile][row][xd] -- so each workgroup first sums the shares of its batch row, in tile order,
+// rounds them to the storage type as the stored projection would be, and keeps the row in LDS.  A workgroup's 256 / LG
+// channels lie in one batch row (d_inner is a multiple of that).
+template <typename T, int LG, bool FOLD = false>
 __global__ __launch_bounds__(256) void ssm_step_kernel(
     float *__restrict__ h, T *__restrict__ y, const T *__restrict__ delta, const T *__restrict__ u,
     const T *__restrict__ Bbase, const T *__restrict__ Cbase, int64_t bc_stride,
     const T *__restrict__ gate, int64_t gate_stride, int gate_mode, const float *__restrict__ dt_bias,
     const T *__restrict__ dt_in, const T *__restrict__ dt_w, int dr, int flags,
-    const float *__restrict__ a_neg, const float *__restrict__ Dp, int64_t total, int di, int ds) {
+    const float *__restrict__ a_neg, const float *__restrict__ Dp, int64_t total, int di, int ds, StepFold fold) {
+    __shared__ alignas(16) T xs_l[FOLD ? kFoldMaxXd : 4];
+    __shared__ alignas(16) float comb[FOLD ? 1024 : 4];
     // total = batch*d_inner rows; ds == 4*LG here.
     const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int64_t rowi = gid / LG;
@@ -53,11 +60,33 @@ __global__ __launch_bounds__(256) void ssm_step_kernel(
     const int d = (int)(r - (int64_t)b * di);
     float4 hv = *reinterpret_cast<const float4 *>(h + r * ds + 4 * g);
     const float4 av = *reinterpret_cast<const float4 *>(a_neg + (int64_t)d * ds + 4 * g);
+    if constexpr (FOLD) {
+        // thread (group tg, quad jq): 4 consecutive entries of the row over tiles tg, tg + G, ...: one round of 16-byte loads
+        const int xd = fold.xd, xq = xd >> 2, G = 256 / xq, tg = (int)threadIdx.x / xq, jq = (int)threadIdx.x - tg * xq;
+        float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (tg < G) {
+            const float *src = fold.xpart + (int64_t)b * xd + 4 * jq;
+            const int64_t tstride = (int64_t)fold.rows * xd;
+#pragma unroll 8
+            for (int t = tg; t < fold.n_tiles; t += G) {
+                const float4 v = *reinterpret_cast<const float4 *>(src + t * tstride);
+                a.x += v.x; a.y += v.y; a.z += v.z; a.w += v.w;
+            }
+            *reinterpret_cast<float4 *>(&comb[tg * xd + 4 * jq]) = a;
+        }
+        __syncthreads();
+        if ((int)threadIdx.x < xd) {
+            float sum = 0.0f;
+            for (int gg = 0; gg < G; gg++) sum += comb[gg * xd + threadIdx.x];   // fixed order
+            Store<T>::st(&xs_l[threadIdx.x], sum);
+        }
+        __syncthreads();
+    }
     float dl;
     if (dt_w) {
         // dt_proj folded in: delta_raw[b,d] = sum_r dt_in[b,r] * dt_w[r,d], the dt_rank terms split over the
         // LG lanes of the row (dt_proj GEMM of the decode chain, src/mamba_ssm/gpu/inference.rs:1129-1146)
-        const T *xr = dt_in + (int64_t)b * bc_stride;
+        const T *xr = FOLD ? xs_l : dt_in + (int64_t)b * bc_stride;
         float part = 0.0f;
         if (flags & kStepDtT) {
             const int kpl = dr / LG;
@@ -105,8 +134,8 @@ __global__ __launch_bounds__(256) void ssm_step_kernel(
     if (dt_bias) dl = softplus20(dl + dt_bias[d]);
     const float uu = Store<T>::ld(u + r);
     const float du = dl * uu;
-    const T *Br = Bbase + (int64_t)b * bc_stride + 4 * g;
-    const T *Cr = Cbase + (int64_t)b * bc_stride + 4 * g;
+    const T *Br = FOLD ? xs_l + fold.b_off + 4 * g : Bbase + (int64_t)b * bc_stride + 4 * g;
+    const T *Cr = FOLD ? xs_l + fold.c_off + 4 * g : Cbase + (int64_t)b * bc_stride + 4 * g;
     const float x = dl * kLog2e;
     float Bv[4], Cv[4];
     ld4<T>(Br, Bv, (flags & kStepVecBC) != 0);
@@ -174,7 +203,8 @@ template <typename T>
 static int launch_step(hipStream_t st, float *h, void *y, const void *delta, const void *u,
                        const void *Bb, const void *Cb, int64_t bc_stride, const void *gate,
                        int64_t gate_stride, int gate_mode, const float *dt_bias, const void *dt_in,
-                       const void *dt_w, int dr, int dt_transposed, const float *a_neg, const float *D, int batch, int di, int ds) {
+                       const void *dt_w, int dr, int dt_transposed, const float *a_neg, const float *D, int batch, int di, int ds,
+                       const StepFold *fold = nullptr) {
     const int64_t total = (int64_t)batch * di;
     if (!gate) gate_mode = 0;
     int flags = 0;
@@ -195,10 +225,23 @@ static int launch_step(hipStream_t st, float *h, void *y, const void *delta, con
         const int64_t blocks = (threads + 255) / 256;
         if (blocks > 0x7fffffffLL) return fail(MRS_E_SHAPE, "ssm step: grid too large");
         const dim3 grid((unsigned)blocks), block(256);
-#define MRS_LG(L) case L: hipLaunchKernelGGL((ssm_step_kernel<T, L>), grid, block, 0, st, MRS_ARGS); break
+        if (fold) {
+            // the row sits in LDS: offsets must suit the vector reads, every workgroup must lie inside one batch row
+            if (!(fold->xpart && fold->xd >= 4 && fold->xd % 4 == 0 && fold->xd <= kFoldMaxXd && fold->rows == batch && di % (256 / lg) == 0 && dt_w &&
+                  fold->b_off % 4 == 0 && fold->c_off % 4 == 0 && fold->b_off + ds <= fold->xd && fold->c_off + ds <= fold->xd && dr <= fold->xd))
+                return fail(MRS_E_SHAPE, "ssm step: folded x_proj needs xd <= %d, d_inner %% %d == 0, 4-aligned B/C offsets", kFoldMaxXd, 256 / lg);
+            flags |= kStepVecBC;
+#define MRS_LGF(L) case L: hipLaunchKernelGGL((ssm_step_kernel<T, L, true>), grid, block, 0, st, MRS_ARGS, *fold); break
+            switch (lg) { MRS_LGF(1); MRS_LGF(2); MRS_LGF(4); MRS_LGF(8); MRS_LGF(16); MRS_LGF(32); MRS_LGF(64); }
+#undef MRS_LGF
+            return check_launch("ssm_step_kernel");
+        }
+        const StepFold nofold = {};
+#define MRS_LG(L) case L: hipLaunchKernelGGL((ssm_step_kernel<T, L>), grid, block, 0, st, MRS_ARGS, nofold); break
         switch (lg) { MRS_LG(1); MRS_LG(2); MRS_LG(4); MRS_LG(8); MRS_LG(16); MRS_LG(32); MRS_LG(64); }
 #undef MRS_LG
     } else {
+        if (fold) return fail(MRS_E_SHAPE, "ssm step: folded x_proj needs d_state a power of two in 4..256");
         const int64_t blocks = (total + 255) / 256;
         if (blocks > 0x7fffffffLL) return fail(MRS_E_SHAPE, "ssm step: grid too large");
         hipLaunchKernelGGL((ssm_step_generic_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, st, MRS_ARGS);
@@ -211,9 +254,9 @@ int launch_ssm_step_fused(hipStream_t st, int dtype, float *h, void *y, const vo
                           const void *dt_in, const void *dt_w, int dr, int dt_transposed,
                           const void *u, const void *Bb, const void *Cb, int64_t bc_stride, const void *gate,
                           int64_t gate_stride, int gate_mode, const float *a_neg, const float *D, int batch,
-                          int di, int ds) {
+                          int di, int ds, const StepFold *fold) {
     MRS_DISPATCH_DTYPE(dtype, T_, return launch_step<T_>(st, h, y, delta, u, Bb, Cb, bc_stride, gate, gate_stride, gate_mode,
-                                                         dt_bias, dt_in, dt_w, dr, dt_transposed, a_neg, D, batch, di, ds));
+                                                         dt_bias, dt_in, dt_w, dr, dt_transposed, a_neg, D, batch, di, ds, fold));
     return MRS_OK;
 }
 
