@@ -311,8 +311,21 @@ def m3_engine_leg(steps=512, batches=(1, 16), prefill_bt=(4, 4096)):
         td = (time.perf_counter() - t0) / steps
         layer_bytes = 2 * (dm * ip + di * dm) + 2 * 4 * B * nh * (hd * ds + ds + hd) + 2 * 4 * B * dm
         step_bytes = cfg.n_layers * layer_bytes
-        out.append({"batch": B, "steps": steps, "us_per_step": td * 1e6, "algorithmic_bytes_per_step": step_bytes,
-                    "hbm_frac": step_bytes / td / 1e9 / HBM_PEAK_GBPS})
+        entry = {"batch": B, "steps": steps, "us_per_step": td * 1e6, "algorithmic_bytes_per_step": step_bytes,
+                 "hbm_frac": step_bytes / td / 1e9 / HBM_PEAK_GBPS}
+        if B == 1:
+            # the LM loop on top (tied 50280-entry head): 100 greedy tokens from a short prompt, as the reference's
+            # synthetic Mamba-3 LM figure (docs/mamba3-benchmarks.md:28)
+            from mamba_rs_amd import GpuMamba3LM, SampleParams
+            vocab = 50280
+            lm = GpuMamba3LM(eng, (rng.standard_normal((vocab, dm), dtype=np.float32) * np.float32(0.02)))
+            prompt = [int(t) for t in rng.integers(0, vocab, 8)]
+            sp = SampleParams(temperature=0.0, max_tokens=100)
+            lm.generate(prompt, params=sp)
+            t0 = time.perf_counter(); toks = lm.generate(prompt, params=sp); tg = time.perf_counter() - t0
+            entry["lm_greedy_100_tokens"] = {"ms": tg * 1e3, "tok_per_s": len(toks) / tg}
+            lm.close()
+        out.append(entry)
         eng.close()
     return {"prefill": prefill, "decode": out}
 

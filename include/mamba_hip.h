@@ -285,7 +285,7 @@ MRS_API int mrs_lm_decode_step(mrs_lm *lm);                        /* tokens <- 
 MRS_API int mrs_lm_capture_graph(mrs_lm *lm);                      /* capture one decode step */
 MRS_API int mrs_lm_last_logits(mrs_lm *lm, float *logits);         /* [batch, vocab] f32, synchronises */
 /* tokens [prefill_engine.batch, T] -> embeddings -> prefill on `prefill_engine` (which may be the decode
- * engine itself: then the head + argmax run and the next tokens are left in the token buffer). */
+ * engine itself, or null for it: then the head + argmax run and the next tokens are left in the token buffer). */
 MRS_API int mrs_lm_prefill(mrs_lm *lm, mrs_backbone *prefill_engine, const int *tokens, int T);
 
 /* ---- sampling and batched generation ------------------------------------------------------
@@ -387,6 +387,11 @@ MRS_API int mrs_m3_backbone_alloc_prefill_scratch(mrs_m3_backbone *bb, int T);
 MRS_API int mrs_m3_backbone_prefill_sequence(mrs_m3_backbone *bb, const float *input, int T, float *out_last);
 MRS_API int mrs_m3_backbone_prefill_device(mrs_m3_backbone *bb, int T);
 MRS_API float *mrs_m3_backbone_prefill_input_ptr(mrs_m3_backbone *bb);
+
+/* GpuMamba3LM (src/module/gpu_lm3.rs:54-400): the LM loop over a Mamba-3 backbone (identity input_proj).  The handle is
+ * an mrs_lm: every mrs_lm_* entry point above works on it (mrs_lm_prefill with a null prefill engine); the engine is
+ * not owned.  embed: [vocab, d_model] f32 on the host. */
+MRS_API int mrs_lm3_create(mrs_lm **out, mrs_m3_backbone *decode_engine, const float *embed, int vocab);
 
 #ifdef __cplusplus
 }

@@ -59,6 +59,7 @@ def _bind():
         "mrs_backbone_state_ptrs": (c_int, [P, c_int, POINTER(P), POINTER(P)]),
         "mrs_backbone_download_state": (c_int, [P, c_int, _FP, _FP]),
         "mrs_lm_create": (c_int, [POINTER(P), P, _FP, c_int]),
+        "mrs_lm3_create": (c_int, [POINTER(P), P, _FP, c_int]),
         "mrs_lm_set_untied_head": (c_int, [P, _FP]),
         "mrs_lm_destroy": (None, [P]),
         "mrs_lm_set_tokens": (c_int, [P, POINTER(c_int)]),
@@ -218,17 +219,19 @@ class GpuMambaBackbone:
 
 
 class GpuMambaLM:
-    """Greedy LM loop on top of a backbone (identity input_proj).  The head is the embedding table (tied)
-    unless `lm_head` [d_model, vocab] is given (GpuMambaLM::new, src/module/gpu_lm.rs:143-262)."""
+    """LM loop on top of a backbone (identity input_proj): GpuMambaLM (src/module/gpu_lm.rs:121-516) over a
+    GpuMambaBackbone, GpuMamba3LM (src/module/gpu_lm3.rs:54-400) over a GpuMamba3Backbone.  The head is the embedding
+    table (tied) unless `lm_head` [d_model, vocab] is given (GpuMambaLM::new, gpu_lm.rs:143-262)."""
 
-    def __init__(self, backbone: GpuMambaBackbone, embed: np.ndarray, lm_head: np.ndarray | None = None):
+    def __init__(self, backbone, embed: np.ndarray, lm_head: np.ndarray | None = None):
         self.backbone = backbone
         embed = np.ascontiguousarray(embed, dtype=np.float32)
         if embed.ndim != 2 or embed.shape[1] != backbone.cfg.d_model:
             raise ValueError("embed must be [vocab, d_model]")
         self.vocab = embed.shape[0]
         h = c_void_p()
-        _call("mrs_lm_create", byref(h), backbone._h, _fp(embed), self.vocab)
+        self._m1 = isinstance(backbone, GpuMambaBackbone)
+        _call("mrs_lm_create" if self._m1 else "mrs_lm3_create", byref(h), backbone._h, _fp(embed), self.vocab)
         self._h = h
         if lm_head is not None:
             lm_head = np.ascontiguousarray(lm_head, dtype=np.float32)
@@ -275,11 +278,11 @@ class GpuMambaLM:
         return out
 
     def prefill(self, tokens: np.ndarray, engine: GpuMambaBackbone | None = None):
-        engine = engine or self.backbone
+        """tokens [batch, T] through the backbone's prefill; `engine`: another Mamba-1 engine to run it on (its batch)."""
         t = np.ascontiguousarray(tokens, dtype=np.int32)
-        if t.ndim != 2 or t.shape[0] != engine.batch:
+        if t.ndim != 2 or t.shape[0] != (engine or self.backbone).batch:
             raise ValueError("tokens must be [batch, T]")
-        _call("mrs_lm_prefill", self._h, engine._h, t.ctypes.data_as(POINTER(c_int)), t.shape[1])
+        _call("mrs_lm_prefill", self._h, engine._h if engine is not None else None, t.ctypes.data_as(POINTER(c_int)), t.shape[1])
 
     def generate_batch(self, prompts, params, *, seen_includes_prompt: bool = False):
         """GpuMambaLM::generate_batch (src/module/gpu_lm.rs:389-516): one prompt (any length) and one SampleParams per

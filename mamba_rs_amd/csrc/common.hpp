@@ -115,6 +115,25 @@ int m3_ssd_fwd_ex(void *stream, int dtype, float *ssm_state, float *k_state, flo
                   const float *D, void *workspace, size_t workspace_bytes, unsigned flags, int batch, int T, int nheads,
                   int headdim, int d_state, int chunk_size);
 
+// What the LM loop (embedding gather, head, argmax / sampling, generation bookkeeping) needs from a backbone engine;
+// the Mamba-1 and the Mamba-3 engine each fill one in.  All functions are stream-ordered on `stream`.
+struct LmHooks {
+    void *self;
+    int batch, d_model, dtype, identity_proj;
+    hipStream_t stream;
+    void *blas;               // rocblas_handle of the engine
+    float *d_input;           // [batch, d_model] f32: the rows a step reads
+    float *temporal;          // [batch, d_model] f32: final-norm output of the last step / prefill
+    void *temporal_t;         // the same in the storage type, or null when the engine keeps no such copy
+    int (*step)(void *self);                         // one decode step (capturable: launches only)
+    int (*reset)(void *self);
+    size_t (*state_bytes)(void *self);               // recurrent state, for save / restore around a warm-up run
+    int (*state_copy)(void *self, void *buf, int restore);
+    int (*prefill)(void *self, const int *dev_tokens, const void *embed, int vocab, int T);   // tokens [batch, T] on device
+};
+// gathers rows of the embedding table (storage type) as f32: out[r, :] = embed[clamp(tokens[r]), :] (engine prefill staging)
+int launch_embed_gather(hipStream_t st, int dtype, float *out, const void *embed, const int *tokens, int64_t rows, int dm, int vocab);
+
 // sample_token for every active row (sampling.hip); all pointers device memory
 int launch_sample_rows(hipStream_t st, int *tokens, const float *logits, float *work, int64_t ld, int rows, int vocab,
                        const mrs_sampler *samplers, const unsigned *seen, unsigned long long *rng, const int *active);
@@ -123,6 +142,9 @@ inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s);
 inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 
 }  // namespace mrs
+
+// The LM loop over any engine that fills in the hooks (engine.hip); `fn` names the caller in error messages.
+int mrs_lm_create_from_hooks(mrs_lm **out, const mrs::LmHooks &eng, const float *embed, int vocab, const char *fn);
 
 // Dispatch a templated launch on the activation storage type.
 #define MRS_DISPATCH_DTYPE(dtype, T, ...)                                         \

@@ -699,7 +699,9 @@ extern "C" int mrs_backbone_download_state(mrs_backbone *bb, int layer, float *c
 
 // ---- LM: embedding + tied head + greedy loop, all on device -------------------------------
 struct mrs_lm {
-    mrs_backbone *bb;   // decode engine (not owned)
+    LmHooks eng;        // decode engine (not owned)
+    mrs_backbone *bb;   // the same engine when it is a Mamba-1 backbone, else null
+    void *hid_t;        // head operand in the storage type when the engine keeps none
     int vocab, vocab_padded, dm, batch, dtype;
     void *embed;        // [vocab_padded, dm] storage dtype (tied lm_head)
     void *head;         // [vocab_padded, dm] storage dtype when the head has weights of its own, else null
@@ -725,14 +727,23 @@ struct mrs_lm {
     int graph_ready;
 };
 
-extern "C" int mrs_lm_create(mrs_lm **out, mrs_backbone *bb, const float *embed, int vocab) {
-    if (!out || !bb || !embed) return fail(MRS_E_NULL, "mrs_lm_create: null pointer");
-    if (!bb->identity_proj) return fail(MRS_E_SHAPE, "mrs_lm_create: the LM feeds embeddings straight into the backbone (identity input_proj)");
-    if (vocab < 1) return fail(MRS_E_SHAPE, "mrs_lm_create: vocab=%d", vocab);
+int mrs::launch_embed_gather(hipStream_t st, int dtype, float *out, const void *embed, const int *tokens, int64_t rows, int dm, int vocab) {
+    const int64_t n = rows * dm;
+    const dim3 grid((unsigned)((n + 255) / 256)), block(256);
+    MRS_DISPATCH_DTYPE(dtype, T_, hipLaunchKernelGGL((embed_gather_kernel<T_>), grid, block, 0, st, out, (const T_ *)embed, tokens, rows, dm, vocab,
+                                                     (const int *)nullptr));
+    return check_launch("embed_gather_kernel");
+}
+
+int mrs_lm_create_from_hooks(mrs_lm **out, const LmHooks &eng, const float *embed, int vocab, const char *fn) {
+    if (!out || !eng.self || !embed) return fail(MRS_E_NULL, "%s: null pointer", fn);
+    if (!eng.identity_proj) return fail(MRS_E_SHAPE, "%s: the LM feeds embeddings straight into the backbone (identity input_proj)", fn);
+    if (vocab < 1) return fail(MRS_E_SHAPE, "%s: vocab=%d", fn, vocab);
     mrs_lm *lm = new (std::nothrow) mrs_lm();
-    if (!lm) return fail(MRS_E_HIP, "mrs_lm_create: out of host memory");
-    lm->bb = bb; lm->vocab = vocab; lm->vocab_padded = (vocab + 63) & ~63;  // src/hf/load.rs:59
-    lm->dm = bb->cfg.d_model; lm->batch = bb->batch; lm->dtype = bb->dtype; lm->graph_ready = 0; lm->graph = nullptr; lm->graph_exec = nullptr;
+    if (!lm) return fail(MRS_E_HIP, "%s: out of host memory", fn);
+    lm->eng = eng; lm->bb = nullptr; lm->hid_t = nullptr;
+    lm->vocab = vocab; lm->vocab_padded = (vocab + 63) & ~63;  // src/hf/load.rs:59
+    lm->dm = eng.d_model; lm->batch = eng.batch; lm->dtype = eng.dtype; lm->graph_ready = 0; lm->graph = nullptr; lm->graph_exec = nullptr;
     lm->head = nullptr;
     lm->gen_ready = 0; lm->gen_graph_ready = 0; lm->gen_graph = nullptr; lm->gen_graph_exec = nullptr;
     lm->gen_prompt_cap = 0; lm->gen_out_cap = 0; lm->gen_dyn = nullptr; lm->gen_dyn_host = GenDyn{nullptr, nullptr, 0};
@@ -746,17 +757,61 @@ extern "C" int mrs_lm_create(mrs_lm **out, mrs_backbone *bb, const float *embed,
     MRS_LM_HIP(hipMalloc((void **)&lm->tokens, (size_t)lm->batch * sizeof(int))); lm->allocs.push_back(lm->tokens);
     MRS_LM_HIP(hipMalloc((void **)&lm->arg_v, (size_t)lm->batch * kArgParts * sizeof(float))); lm->allocs.push_back(lm->arg_v);
     MRS_LM_HIP(hipMalloc((void **)&lm->arg_i, (size_t)lm->batch * kArgParts * sizeof(int))); lm->allocs.push_back(lm->arg_i);
+    if (!eng.temporal_t && lm->dtype != MRS_F32) { MRS_LM_HIP(hipMalloc(&lm->hid_t, (size_t)lm->batch * lm->dm * es)); lm->allocs.push_back(lm->hid_t); }
     MRS_LM_HIP(hipMalloc((void **)&stage, ne * 4));
-    MRS_LM_HIP(hipMemsetAsync(stage, 0, ne * 4, bb->stream));  // padded rows are zero
-    MRS_LM_HIP(hipMemcpyAsync(stage, embed, (size_t)vocab * lm->dm * 4, hipMemcpyHostToDevice, bb->stream));
+    MRS_LM_HIP(hipMemsetAsync(stage, 0, ne * 4, eng.stream));  // padded rows are zero
+    MRS_LM_HIP(hipMemcpyAsync(stage, embed, (size_t)vocab * lm->dm * 4, hipMemcpyHostToDevice, eng.stream));
     const dim3 grid((unsigned)((ne + 255) / 256)), block(256);
-    if (lm->dtype == MRS_F32) MRS_LM_HIP(hipMemcpyAsync(lm->embed, stage, ne * 4, hipMemcpyDeviceToDevice, bb->stream));
-    else if (lm->dtype == MRS_BF16) hipLaunchKernelGGL((cast_from_f32_kernel<bf16_t>), grid, block, 0, bb->stream, (bf16_t *)lm->embed, stage, (int64_t)ne);
-    else hipLaunchKernelGGL((cast_from_f32_kernel<f16_t>), grid, block, 0, bb->stream, (f16_t *)lm->embed, stage, (int64_t)ne);
-    MRS_LM_HIP(hipStreamSynchronize(bb->stream));
+    if (lm->dtype == MRS_F32) MRS_LM_HIP(hipMemcpyAsync(lm->embed, stage, ne * 4, hipMemcpyDeviceToDevice, eng.stream));
+    else if (lm->dtype == MRS_BF16) hipLaunchKernelGGL((cast_from_f32_kernel<bf16_t>), grid, block, 0, eng.stream, (bf16_t *)lm->embed, stage, (int64_t)ne);
+    else hipLaunchKernelGGL((cast_from_f32_kernel<f16_t>), grid, block, 0, eng.stream, (f16_t *)lm->embed, stage, (int64_t)ne);
+    MRS_LM_HIP(hipStreamSynchronize(eng.stream));
 #undef MRS_LM_HIP
     hipFree(stage);
     *out = lm;
+    return MRS_OK;
+}
+
+// ---- the Mamba-1 engine behind the LM loop ----
+static int m1_hook_step(void *self) { return step_body((mrs_backbone *)self); }
+static int m1_hook_reset(void *self) { return mrs_backbone_reset((mrs_backbone *)self); }
+static size_t m1_hook_state_bytes(void *self) {
+    mrs_backbone *bb = (mrs_backbone *)self;
+    const size_t L = bb->cfg.n_layers, B = bb->batch;
+    return L * B * bb->di * (size_t)(bb->cfg.d_conv + bb->cfg.d_state) * 4;
+}
+static int m1_hook_state_copy(void *self, void *buf, int restore) {
+    mrs_backbone *bb = (mrs_backbone *)self;
+    const size_t L = bb->cfg.n_layers, B = bb->batch;
+    const size_t cb = L * B * bb->di * bb->cfg.d_conv * 4, sb = L * B * bb->di * bb->cfg.d_state * 4;
+    if (restore) {
+        MRS_HIP(hipMemcpyAsync(bb->conv_state, buf, cb, hipMemcpyDeviceToDevice, bb->stream));
+        MRS_HIP(hipMemcpyAsync(bb->ssm_state, (char *)buf + cb, sb, hipMemcpyDeviceToDevice, bb->stream));
+    } else {
+        MRS_HIP(hipMemcpyAsync(buf, bb->conv_state, cb, hipMemcpyDeviceToDevice, bb->stream));
+        MRS_HIP(hipMemcpyAsync((char *)buf + cb, bb->ssm_state, sb, hipMemcpyDeviceToDevice, bb->stream));
+    }
+    return MRS_OK;
+}
+static int m1_hook_prefill(void *self, const int *dev_tokens, const void *embed, int vocab, int T) {
+    mrs_backbone *bb = (mrs_backbone *)self;
+    MRS_TRY(mrs_backbone_alloc_prefill_scratch(bb, T));
+    MRS_TRY(launch_embed_gather(bb->stream, bb->dtype, bb->prefill_in, embed, dev_tokens, (int64_t)bb->batch * T, bb->cfg.d_model, vocab));
+    return mrs_backbone_prefill_device(bb, bb->prefill_in, T);
+}
+static LmHooks m1_hooks(mrs_backbone *bb) {
+    LmHooks h = {};
+    h.self = bb; h.batch = bb->batch; h.d_model = bb->cfg.d_model; h.dtype = bb->dtype; h.identity_proj = bb->identity_proj;
+    h.stream = bb->stream; h.blas = bb->blas; h.d_input = bb->d_input; h.temporal = bb->temporal;
+    h.temporal_t = bb->dtype != MRS_F32 ? bb->temporal_t : nullptr;
+    h.step = m1_hook_step; h.reset = m1_hook_reset; h.state_bytes = m1_hook_state_bytes; h.state_copy = m1_hook_state_copy; h.prefill = m1_hook_prefill;
+    return h;
+}
+
+extern "C" int mrs_lm_create(mrs_lm **out, mrs_backbone *bb, const float *embed, int vocab) {
+    if (!out || !bb || !embed) return fail(MRS_E_NULL, "mrs_lm_create: null pointer");
+    MRS_TRY(mrs_lm_create_from_hooks(out, m1_hooks(bb), embed, vocab, "mrs_lm_create"));
+    (*out)->bb = bb;
     return MRS_OK;
 }
 
@@ -766,7 +821,7 @@ extern "C" int mrs_lm_create(mrs_lm **out, mrs_backbone *bb, const float *embed,
 extern "C" int mrs_lm_set_untied_head(mrs_lm *lm, const float *lm_head) {
     if (!lm || !lm_head) return fail(MRS_E_NULL, "mrs_lm_set_untied_head: null pointer");
     if (lm->graph_ready) return fail(MRS_E_SHAPE, "mrs_lm_set_untied_head: set the head before capturing the graph");
-    mrs_backbone *bb = lm->bb;
+    const LmHooks *bb = &lm->eng;
     const size_t es = esize(lm->dtype), ne = (size_t)lm->vocab_padded * lm->dm;
     std::vector<float> host;
     try { host.assign(ne, 0.0f); } catch (...) { return fail(MRS_E_HIP, "mrs_lm_set_untied_head: out of host memory"); }
@@ -792,7 +847,7 @@ extern "C" int mrs_lm_set_untied_head(mrs_lm *lm, const float *lm_head) {
 
 extern "C" void mrs_lm_destroy(mrs_lm *lm) {
     if (!lm) return;
-    hipStreamSynchronize(lm->bb->stream);
+    hipStreamSynchronize(lm->eng.stream);
     if (lm->graph_exec) hipGraphExecDestroy(lm->graph_exec);
     if (lm->graph) hipGraphDestroy(lm->graph);
     if (lm->gen_graph_exec) hipGraphExecDestroy(lm->gen_graph_exec);
@@ -806,20 +861,30 @@ extern "C" void mrs_lm_destroy(mrs_lm *lm) {
 // logits = norm_f(hidden) . table^T, table = the embedding (tied head) or the head's own weights
 // (OP_T on the row-major [V, dm] table: src/mamba_ssm/gpu/blas.rs:709-740)
 static int lm_logits(mrs_lm *lm) {
-    mrs_backbone *bb = lm->bb;
+    const LmHooks *bb = &lm->eng;
     const int dm = lm->dm, V = lm->vocab_padded, B = lm->batch;
     const float one = 1.0f, zero = 0.0f;
-    // the final norm leaves its result in the storage type as well (temporal_t), which is the head's operand
-    const void *hid = lm->dtype != MRS_F32 ? bb->temporal_t : (const void *)bb->temporal;
+    // the head's operand is the final norm's result in the storage type: the engine's own copy (temporal_t), or a cast
+    const void *hid = bb->temporal;
+    if (lm->dtype != MRS_F32) {
+        hid = bb->temporal_t;
+        if (!hid) {
+            const int64_t n = (int64_t)B * dm;
+            const dim3 grid((unsigned)((n + 255) / 256)), block(256);
+            if (lm->dtype == MRS_BF16) hipLaunchKernelGGL((cast_from_f32_kernel<bf16_t>), grid, block, 0, bb->stream, (bf16_t *)lm->hid_t, bb->temporal, n);
+            else hipLaunchKernelGGL((cast_from_f32_kernel<f16_t>), grid, block, 0, bb->stream, (f16_t *)lm->hid_t, bb->temporal, n);
+            hid = lm->hid_t;
+        }
+    }
     const rocblas_datatype ht = lm->dtype != MRS_F32 ? blas_type(lm->dtype) : rocblas_datatype_f32_r;
-    MRS_BLAS(rocblas_gemm_ex(bb->blas, rocblas_operation_transpose, rocblas_operation_none, V, B, dm, &one,
+    MRS_BLAS(rocblas_gemm_ex((rocblas_handle)bb->blas, rocblas_operation_transpose, rocblas_operation_none, V, B, dm, &one,
                              lm->head ? lm->head : lm->embed, blas_type(lm->dtype), dm, hid, ht, dm, &zero, lm->logits, rocblas_datatype_f32_r, V, lm->logits,
                              rocblas_datatype_f32_r, V, rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0));
     return MRS_OK;
 }
 
 static int lm_argmax(mrs_lm *lm) {
-    hipStream_t st = lm->bb->stream;
+    hipStream_t st = lm->eng.stream;
     hipLaunchKernelGGL(argmax_part_kernel, dim3((unsigned)(lm->batch * kArgParts)), dim3(256), 0, st, lm->arg_v, lm->arg_i, lm->logits,
                        lm->vocab, (int64_t)lm->vocab_padded);
     hipLaunchKernelGGL(argmax_final_kernel, dim3((unsigned)lm->batch), dim3(64), 0, st, lm->tokens, lm->arg_v, lm->arg_i);
@@ -827,19 +892,19 @@ static int lm_argmax(mrs_lm *lm) {
 }
 
 static int lm_decode_body(mrs_lm *lm) {
-    mrs_backbone *bb = lm->bb;
+    const LmHooks *bb = &lm->eng;
     const int64_t n = (int64_t)lm->batch * lm->dm;
     const dim3 grid((unsigned)((n + 255) / 256)), block(256);
     MRS_DISPATCH_DTYPE(lm->dtype, T_, hipLaunchKernelGGL((embed_gather_kernel<T_>), grid, block, 0, bb->stream, bb->d_input,
                                                          (const T_ *)lm->embed, lm->tokens, (int64_t)lm->batch, lm->dm, lm->vocab));
-    MRS_TRY(step_body(bb));
+    MRS_TRY(bb->step(bb->self));
     MRS_TRY(lm_logits(lm));
     return lm_argmax(lm);
 }
 
 extern "C" int mrs_lm_set_tokens(mrs_lm *lm, const int *tokens) {
     if (!lm || !tokens) return fail(MRS_E_NULL, "mrs_lm_set_tokens: null pointer");
-    MRS_HIP(hipMemcpyAsync(lm->tokens, tokens, (size_t)lm->batch * sizeof(int), hipMemcpyHostToDevice, lm->bb->stream));
+    MRS_HIP(hipMemcpyAsync(lm->tokens, tokens, (size_t)lm->batch * sizeof(int), hipMemcpyHostToDevice, lm->eng.stream));
     return MRS_OK;
 }
 
@@ -847,25 +912,23 @@ extern "C" int mrs_lm_set_tokens(mrs_lm *lm, const int *tokens) {
 // token, backbone step, tied head, argmax -> next token (left in the device token buffer).
 extern "C" int mrs_lm_decode_step(mrs_lm *lm) {
     if (!lm) return fail(MRS_E_NULL, "mrs_lm_decode_step: null engine");
-    if (lm->graph_ready) { MRS_HIP(hipGraphLaunch(lm->graph_exec, lm->bb->stream)); return MRS_OK; }
+    if (lm->graph_ready) { MRS_HIP(hipGraphLaunch(lm->graph_exec, lm->eng.stream)); return MRS_OK; }
     return lm_decode_body(lm);
 }
 
 extern "C" int mrs_lm_capture_graph(mrs_lm *lm) {
     if (!lm) return fail(MRS_E_NULL, "mrs_lm_capture_graph: null engine");
     if (lm->graph_ready) return MRS_OK;
-    mrs_backbone *bb = lm->bb;
-    const size_t L = bb->cfg.n_layers, B = bb->batch;
-    const size_t cb = L * B * bb->di * bb->cfg.d_conv * 4, sb = L * B * bb->di * bb->cfg.d_state * 4, tb = B * sizeof(int);
+    const LmHooks *bb = &lm->eng;
+    // a warm, eager step (the GEMM library settles its choices), with the recurrent state and the tokens put back after it
+    const size_t sbytes = bb->state_bytes(bb->self), tb = (size_t)lm->batch * sizeof(int);
     void *save = nullptr;
-    MRS_HIP(hipMalloc(&save, cb + sb + tb));
-    hipMemcpyAsync(save, bb->conv_state, cb, hipMemcpyDeviceToDevice, bb->stream);
-    hipMemcpyAsync((char *)save + cb, bb->ssm_state, sb, hipMemcpyDeviceToDevice, bb->stream);
-    hipMemcpyAsync((char *)save + cb + sb, lm->tokens, tb, hipMemcpyDeviceToDevice, bb->stream);
-    int rc = lm_decode_body(lm);   // warm, eager
-    hipMemcpyAsync(bb->conv_state, save, cb, hipMemcpyDeviceToDevice, bb->stream);
-    hipMemcpyAsync(bb->ssm_state, (char *)save + cb, sb, hipMemcpyDeviceToDevice, bb->stream);
-    hipMemcpyAsync(lm->tokens, (char *)save + cb + sb, tb, hipMemcpyDeviceToDevice, bb->stream);
+    MRS_HIP(hipMalloc(&save, sbytes + tb));
+    int rc = bb->state_copy(bb->self, save, 0);
+    hipMemcpyAsync((char *)save + sbytes, lm->tokens, tb, hipMemcpyDeviceToDevice, bb->stream);
+    if (!rc) rc = lm_decode_body(lm);
+    if (!rc) rc = bb->state_copy(bb->self, save, 1);
+    hipMemcpyAsync(lm->tokens, (char *)save + sbytes, tb, hipMemcpyDeviceToDevice, bb->stream);
     hipStreamSynchronize(bb->stream);
     hipFree(save);
     if (rc) return rc;
@@ -883,40 +946,43 @@ extern "C" int mrs_lm_capture_graph(mrs_lm *lm) {
 
 extern "C" int mrs_lm_get_tokens(mrs_lm *lm, int *tokens) {
     if (!lm || !tokens) return fail(MRS_E_NULL, "mrs_lm_get_tokens: null pointer");
-    MRS_HIP(hipMemcpyAsync(tokens, lm->tokens, (size_t)lm->batch * sizeof(int), hipMemcpyDeviceToHost, lm->bb->stream));
-    MRS_HIP(hipStreamSynchronize(lm->bb->stream));
+    MRS_HIP(hipMemcpyAsync(tokens, lm->tokens, (size_t)lm->batch * sizeof(int), hipMemcpyDeviceToHost, lm->eng.stream));
+    MRS_HIP(hipStreamSynchronize(lm->eng.stream));
     return MRS_OK;
 }
 
 extern "C" int mrs_lm_last_logits(mrs_lm *lm, float *logits) {
     if (!lm || !logits) return fail(MRS_E_NULL, "mrs_lm_last_logits: null pointer");
     MRS_HIP(hipMemcpy2DAsync(logits, (size_t)lm->vocab * 4, lm->logits, (size_t)lm->vocab_padded * 4, (size_t)lm->vocab * 4, lm->batch,
-                             hipMemcpyDeviceToHost, lm->bb->stream));
-    MRS_HIP(hipStreamSynchronize(lm->bb->stream));
+                             hipMemcpyDeviceToHost, lm->eng.stream));
+    MRS_HIP(hipStreamSynchronize(lm->eng.stream));
     return MRS_OK;
 }
 
 // Prefill helper for the LM: token ids [batch, T] (host) -> embeddings on device -> backbone prefill,
 // then the head on the last position; the greedy next token of every row is left in the token buffer.
+// prefill_bb: a Mamba-1 engine (the LM's own or another one with the prefill batch), or null = the LM's own engine.
 extern "C" int mrs_lm_prefill(mrs_lm *lm, mrs_backbone *prefill_bb, const int *tokens, int T) {
-    if (!lm || !prefill_bb || !tokens) return fail(MRS_E_NULL, "mrs_lm_prefill: null pointer");
-    if (prefill_bb->cfg.d_model != lm->dm || prefill_bb->dtype != lm->dtype || !prefill_bb->identity_proj)
-        return fail(MRS_E_SHAPE, "mrs_lm_prefill: prefill engine does not match the LM");
-    MRS_TRY(mrs_backbone_alloc_prefill_scratch(prefill_bb, T));
-    const int64_t rows = (int64_t)prefill_bb->batch * T;
+    if (!lm || !tokens) return fail(MRS_E_NULL, "mrs_lm_prefill: null pointer");
+    if (T < 1) return fail(MRS_E_SHAPE, "mrs_lm_prefill: T=%d", T);
+    const bool own = !prefill_bb || prefill_bb == lm->bb;
+    LmHooks other = {};
+    if (!own) {
+        if (prefill_bb->cfg.d_model != lm->dm || prefill_bb->dtype != lm->dtype || !prefill_bb->identity_proj)
+            return fail(MRS_E_SHAPE, "mrs_lm_prefill: prefill engine does not match the LM");
+        other = m1_hooks(prefill_bb);
+    }
+    const LmHooks *eng = own ? &lm->eng : &other;
+    const int64_t rows = (int64_t)eng->batch * T;
     int *dtok = nullptr;
     MRS_HIP(hipMalloc((void **)&dtok, rows * sizeof(int)));
-    hipMemcpyAsync(dtok, tokens, rows * sizeof(int), hipMemcpyHostToDevice, prefill_bb->stream);
-    const int64_t n = rows * lm->dm;
-    const dim3 grid((unsigned)((n + 255) / 256)), block(256);
-    MRS_DISPATCH_DTYPE(lm->dtype, T_, hipLaunchKernelGGL((embed_gather_kernel<T_>), grid, block, 0, prefill_bb->stream, prefill_bb->prefill_in,
-                                                         (const T_ *)lm->embed, dtok, rows, lm->dm, lm->vocab));
-    int rc = mrs_backbone_prefill_device(prefill_bb, prefill_bb->prefill_in, T);
-    if (!rc && prefill_bb == lm->bb) {
+    hipMemcpyAsync(dtok, tokens, rows * sizeof(int), hipMemcpyHostToDevice, eng->stream);
+    int rc = eng->prefill(eng->self, dtok, lm->embed, lm->vocab, T);
+    if (!rc && own) {
         rc = lm_logits(lm);
         if (!rc) rc = lm_argmax(lm);
     }
-    hipStreamSynchronize(prefill_bb->stream);
+    hipStreamSynchronize(eng->stream);
     hipFree(dtok);
     return rc;
 }
@@ -944,7 +1010,7 @@ static int gen_alloc(mrs_lm *lm) {
 
 // sample the active slots from the current logits, then advance every slot
 static int gen_pick(mrs_lm *lm) {
-    hipStream_t st = lm->bb->stream;
+    hipStream_t st = lm->eng.stream;
     MRS_TRY(launch_sample_rows(st, lm->gen.sampled, lm->logits, lm->gen_work, lm->vocab_padded, lm->batch, lm->vocab, lm->gen_samplers,
                                lm->gen.seen, lm->gen_rng, lm->gen.active));
     hipLaunchKernelGGL(gen_advance_kernel, dim3(1), dim3(1024), 0, st, lm->gen, lm->gen_dyn, lm->tokens, lm->batch, lm->vocab);
@@ -953,20 +1019,20 @@ static int gen_pick(mrs_lm *lm) {
 
 // gather the slots' current tokens (zeros for finished slots), one backbone step, head
 static int gen_forward(mrs_lm *lm) {
-    mrs_backbone *bb = lm->bb;
+    const LmHooks *bb = &lm->eng;
     const int64_t n = (int64_t)lm->batch * lm->dm;
     const dim3 grid((unsigned)((n + 255) / 256)), block(256);
     MRS_DISPATCH_DTYPE(lm->dtype, T_, hipLaunchKernelGGL((embed_gather_kernel<T_>), grid, block, 0, bb->stream, bb->d_input,
                                                          (const T_ *)lm->embed, lm->tokens, (int64_t)lm->batch, lm->dm, lm->vocab,
                                                          (const int *)lm->gen.finished));
-    MRS_TRY(step_body(bb));
+    MRS_TRY(bb->step(bb->self));
     return lm_logits(lm);
 }
 
 extern "C" int mrs_lm_generate_batch(mrs_lm *lm, const int *prompts, const int *prompt_lens, const mrs_sample_params *params,
                                      int seen_includes_prompt, int *out_tokens, int out_stride, int *out_lens) {
     if (!lm || !prompt_lens || !params || !out_tokens || !out_lens) return fail(MRS_E_NULL, "mrs_lm_generate_batch: null pointer");
-    mrs_backbone *bb = lm->bb;
+    const LmHooks *bb = &lm->eng;
     hipStream_t st = bb->stream;
     const int B = lm->batch;
     int64_t total = 0;
@@ -1035,10 +1101,10 @@ extern "C" int mrs_lm_generate_batch(mrs_lm *lm, const int *prompts, const int *
     if (seen_includes_prompt && max_prompt > 0)
         hipLaunchKernelGGL(gen_seen_prompt_kernel, dim3((unsigned)std::min(64, (max_prompt + 255) / 256), (unsigned)B), dim3(256), 0, st, lm->gen,
                            lm->gen_dyn, B, lm->vocab);
-    MRS_TRY(mrs_backbone_reset(bb));
+    MRS_TRY(bb->reset(bb->self));
     int steps = max_prompt + max_tokens;   // gpu_lm.rs:432
     if (prefill_route && running) {
-        MRS_TRY(mrs_lm_prefill(lm, bb, prompts, prompt_lens[0]));   // state after the prompt, logits of its last position
+        MRS_TRY(mrs_lm_prefill(lm, nullptr, prompts, prompt_lens[0]));   // state after the prompt, logits of its last position
         MRS_TRY(gen_pick(lm));
         steps = max_tokens;
     }

@@ -853,3 +853,49 @@ extern "C" int mrs_m3_backbone_download_state(mrs_m3_backbone *bb, int layer, fl
     MRS_HIP(hipStreamSynchronize(bb->stream));
     return MRS_OK;
 }
+
+// ---- the Mamba-3 engine behind the LM loop (GpuMamba3LM, src/module/gpu_lm3.rs:54-400) ---------------------------
+namespace {
+void m3_state_sizes(mrs_m3_backbone *bb, size_t (&n)[4]) {
+    const size_t L = bb->cfg.n_layers, B = bb->batch, nh = bb->nh, hd = bb->cfg.headdim, ds = bb->cfg.d_state, na = bb->nr > 0 ? bb->nr : 1;
+    n[0] = L * B * nh * hd * ds * 4; n[1] = L * B * nh * ds * 4; n[2] = L * B * nh * hd * 4; n[3] = L * B * nh * na * 4;
+}
+int m3_hook_step(void *self) { return step_body3((mrs_m3_backbone *)self); }
+int m3_hook_reset(void *self) { return mrs_m3_backbone_reset((mrs_m3_backbone *)self); }
+size_t m3_hook_state_bytes(void *self) {
+    size_t n[4];
+    m3_state_sizes((mrs_m3_backbone *)self, n);
+    return n[0] + n[1] + n[2] + n[3];
+}
+int m3_hook_state_copy(void *self, void *buf, int restore) {
+    mrs_m3_backbone *bb = (mrs_m3_backbone *)self;
+    size_t n[4];
+    m3_state_sizes(bb, n);
+    float *parts[4] = {bb->ssm, bb->kst, bb->vst, bb->angle};
+    char *p = (char *)buf;
+    for (int i = 0; i < 4; i++) {
+        if (restore) MRS_HIP(hipMemcpyAsync(parts[i], p, n[i], hipMemcpyDeviceToDevice, bb->stream));
+        else MRS_HIP(hipMemcpyAsync(p, parts[i], n[i], hipMemcpyDeviceToDevice, bb->stream));
+        p += n[i];
+    }
+    return MRS_OK;
+}
+int m3_hook_prefill(void *self, const int *dev_tokens, const void *embed, int vocab, int T) {
+    mrs_m3_backbone *bb = (mrs_m3_backbone *)self;
+    MRS_TRY(mrs_m3_backbone_alloc_prefill_scratch(bb, T));
+    MRS_TRY(launch_embed_gather(bb->stream, bb->dtype, bb->pf_in, embed, dev_tokens, (int64_t)bb->batch * T, bb->cfg.d_model, vocab));
+    return prefill_body3(bb, T);
+}
+}  // namespace
+
+// LM loop (embedding gather, head, greedy pick or sampling, generate / generate_batch) over a Mamba-3 backbone: every
+// mrs_lm_* entry point then works on the returned handle.  embed: [vocab, d_model] f32 on the host.
+extern "C" int mrs_lm3_create(mrs_lm **out, mrs_m3_backbone *bb, const float *embed, int vocab) {
+    if (!out || !bb || !embed) return fail(MRS_E_NULL, "mrs_lm3_create: null pointer");
+    LmHooks h = {};
+    h.self = bb; h.batch = bb->batch; h.d_model = bb->cfg.d_model; h.dtype = bb->dtype; h.identity_proj = bb->identity_proj;
+    h.stream = bb->stream; h.blas = bb->blas; h.d_input = bb->d_input; h.temporal = bb->temporal; h.temporal_t = nullptr;
+    h.step = m3_hook_step; h.reset = m3_hook_reset; h.state_bytes = m3_hook_state_bytes; h.state_copy = m3_hook_state_copy;
+    h.prefill = m3_hook_prefill;
+    return mrs_lm_create_from_hooks(out, h, embed, vocab, "mrs_lm3_create");
+}
