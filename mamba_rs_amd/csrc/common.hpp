@@ -56,6 +56,11 @@ __device__ __forceinline__ float softplus20(float v) {
     return e < 0.03f ? series : vialog;
 }
 
+// Workgroup barrier that publishes LDS writes only: global loads issued before it stay in flight across it (the
+// ordinary barrier's fence waits for every outstanding memory operation of the wave).  Not for data that travels
+// through global memory.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 // ---- host-side error plumbing ---------------------------------------------
 void set_error(const char *fmt, ...);
 int fail(int code, const char *fmt, ...);

@@ -190,7 +190,7 @@ __global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu
 #pragma unroll
                 for (int t = 0; t < NC; t++) wv[t][j] = *reinterpret_cast<const uint4 *>(wp[t] + 8 * LPR * j);
             }
-        __syncthreads();
+        lds_barrier();   // the rows are in LDS; the weight loads above stay in flight
         for (int jb = 0; jb < per; jb += JB) {
             uint4 nx[NC][JB];
 #pragma unroll
@@ -225,7 +225,7 @@ __global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu
                 for (int x = LPR / 2; x >= 1; x >>= 1) v += __shfl_xor(v, x, kWave);
                 if (ll == 0) gv[m][2 * w + (LPR == 64 ? t : half)] = v;
             }
-        __syncthreads();
+        lds_barrier();
     } else {
     for (int base = w; base < nk; base += kGemmWaves * kStepsPerBatch) {
         uint4 bf[kStepsPerBatch], af[kStepsPerBatch];
@@ -243,9 +243,9 @@ __global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu
     }
     // K-split reduction: upper half of the waves parks its tile in LDS, lower half adds and parks the sums
     if (w >= kGemmWaves / 2) red[w - kGemmWaves / 2][l] = acc;
-    __syncthreads();
+    lds_barrier();   // LDS exchanges only: the epilogue's prefetched operands stay in flight
     if (w < kGemmWaves / 2) red[w][l] += acc;
-    __syncthreads();
+    lds_barrier();
     }
     // element e of the 16x16 tile: row ml = e / 16, column nl = e % 16 lives in lane 16 (ml / 4) + nl, register ml % 4
     float u_out = 0.0f;   // mode 1: this thread's u as stored (0 for gate columns / rows past M)
@@ -307,7 +307,7 @@ __global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu
         if (ep.xw != nullptr && n0 < ep.di) {   // the same for the whole workgroup
             __shared__ float ush[4][16];
             if (tid < 64) ush[tid >> 4][tid & 15] = u_out;
-            __syncthreads();
+            lds_barrier();
             const int xd = ep.xd, P = M * xd;   // P <= 512 (checked by the launcher)
             const T *xw = reinterpret_cast<const T *>(ep.xw);
             if (tid < P) {

@@ -19,8 +19,8 @@ namespace mrs {
 // (dt_proj bias add + softplus_forward of the decode chain, src/mamba_ssm/gpu/inference.rs:1129-1158).
 // Four consecutive elements as f32: one 8-byte (16-bit storage) or 16-byte (f32) load when the
 // address is aligned for it (vec), four scalar loads otherwise.
-template <typename T> __device__ __forceinline__ void ld4(const T *p, float (&o)[4], bool vec) {
-    if (vec) {
+template <typename T, bool VEC> __device__ __forceinline__ void ld4(const T *p, float (&o)[4]) {
+    if constexpr (VEC) {
         struct alignas(4 * sizeof(T)) V { T v[4]; };
         const V t = *reinterpret_cast<const V *>(p);
 #pragma unroll
@@ -31,22 +31,25 @@ template <typename T> __device__ __forceinline__ void ld4(const T *p, float (&o)
     }
 }
 
-// flags: bit 0 = B/C rows may be read as aligned 4-element vectors; bit 1 = dt_w is transposed
-// ([d_inner][dt_rank]) and dt_rank / LG is a multiple of 4, so lane g takes the contiguous terms
-// [g dt_rank/LG, (g+1) dt_rank/LG) of both operands as 4-element vectors.
-constexpr int kStepVecBC = 1, kStepDtT = 2;
 constexpr int kFoldMaxXd = 256;
 
+// DT: where delta comes from -- 0: `delta` holds it; 1: dt_proj folded in, dt_w [dt_rank][d_inner]; 2: dt_proj folded
+// in, dt_w transposed ([d_inner][dt_rank]) with dt_rank / LG a multiple of 4, so lane g takes the contiguous terms
+// [g dt_rank/LG, (g+1) dt_rank/LG) of both operands as 4-element vectors.  VECBC: B/C rows may be read as aligned
+// 4-element vectors.  Both are template parameters so that the body is straight-line code: with them as run-time flags
+// the compiler fenced every group of loads with its own wait and the kernel was a chain of eight memory round trips
+// (8.4 us at batch 64 against 4.2 us for the same state traffic without the folded dt_proj).
+//
 // FOLD: the x_proj row (dt input, B, C) has not been formed yet -- the in_proj launch before left its 16-column
 // shares in fold.xpart [tile][row][xd] -- so each workgroup first sums the shares of its batch row, in tile order,
 // rounds them to the storage type as the stored projection would be, and keeps the row in LDS.  A workgroup's 256 / LG
 // channels lie in one batch row (d_inner is a multiple of that).
-template <typename T, int LG, bool FOLD = false>
+template <typename T, int LG, int DT, bool VECBC, bool FOLD = false>
 __global__ __launch_bounds__(256) void ssm_step_kernel(
     float *__restrict__ h, T *__restrict__ y, const T *__restrict__ delta, const T *__restrict__ u,
     const T *__restrict__ Bbase, const T *__restrict__ Cbase, int64_t bc_stride,
     const T *__restrict__ gate, int64_t gate_stride, int gate_mode, const float *__restrict__ dt_bias,
-    const T *__restrict__ dt_in, const T *__restrict__ dt_w, int dr, int flags,
+    const T *__restrict__ dt_in, const T *__restrict__ dt_w, int dr,
     const float *__restrict__ a_neg, const float *__restrict__ Dp, int64_t total, int di, int ds, StepFold fold) {
     __shared__ alignas(16) T xs_l[FOLD ? kFoldMaxXd : 4];
     __shared__ alignas(16) float comb[FOLD ? 1024 : 4];
@@ -58,48 +61,89 @@ __global__ __launch_bounds__(256) void ssm_step_kernel(
     const int64_t r = live ? rowi : total - 1;
     const int b = (int)(r / di);
     const int d = (int)(r - (int64_t)b * di);
-    float4 hv = *reinterpret_cast<const float4 *>(h + r * ds + 4 * g);
-    const float4 av = *reinterpret_cast<const float4 *>(a_neg + (int64_t)d * ds + 4 * g);
+    // ---- every load that does not wait for another one, up front; the shares of the x_proj row first, since the
+    // first thing computed is their sum ----
+    float4 share[FOLD ? 8 : 1];
+    int fold_G = 1, fold_tg = 0, fold_jq = 0;
     if constexpr (FOLD) {
         // thread (group tg, quad jq): 4 consecutive entries of the row over tiles tg, tg + G, ...: one round of 16-byte loads
-        const int xd = fold.xd, xq = xd >> 2, G = 256 / xq, tg = (int)threadIdx.x / xq, jq = (int)threadIdx.x - tg * xq;
-        float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (tg < G) {
-            const float *src = fold.xpart + (int64_t)b * xd + 4 * jq;
+        const int xq = fold.xd >> 2;
+        fold_G = 256 / xq; fold_tg = (int)threadIdx.x / xq; fold_jq = (int)threadIdx.x - fold_tg * xq;
+        const float *src = fold.xpart + (int64_t)b * fold.xd + 4 * fold_jq;
+        const int64_t tstride = (int64_t)fold.rows * fold.xd;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const int t = fold_tg + i * fold_G;
+            share[i] = (fold_tg < fold_G && t < fold.n_tiles) ? *reinterpret_cast<const float4 *>(src + t * tstride) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    }
+    float4 hv = *reinterpret_cast<const float4 *>(h + r * ds + 4 * g);
+    const float4 av = *reinterpret_cast<const float4 *>(a_neg + (int64_t)d * ds + 4 * g);
+    const float uu = Store<T>::ld(u + r);
+    const float Dd = Dp[d];
+    float bias = 0.0f, gz = 0.0f, dl = 0.0f;
+    if (dt_bias) bias = dt_bias[d];
+    if (gate_mode != 0) gz = Store<T>::ld(gate + (int64_t)b * gate_stride + d);
+    if constexpr (DT == 0) dl = Store<T>::ld(delta + r);
+    float Bv[4], Cv[4];
+    if constexpr (!FOLD) {
+        ld4<T, VECBC>(Bbase + (int64_t)b * bc_stride + 4 * g, Bv);
+        ld4<T, VECBC>(Cbase + (int64_t)b * bc_stride + 4 * g, Cv);
+    }
+    const int kpl = DT == 2 ? dr / LG : 0;
+    float wv0[4][4];   // DT 2: the first 16 terms of this lane's share of the weight row
+    if constexpr (DT == 2) {
+        const T *wp = dt_w + (int64_t)d * dr + g * kpl;
+#pragma unroll
+        for (int j = 0; j < 4; j++) ld4<T, true>(wp + (4 * j < kpl ? 4 * j : 0), wv0[j]);
+    }
+    if constexpr (FOLD) {
+        const int xd = fold.xd;
+        if (fold_tg < fold_G) {
+            float4 a = share[0];
+#pragma unroll
+            for (int i = 1; i < 8; i++) { a.x += share[i].x; a.y += share[i].y; a.z += share[i].z; a.w += share[i].w; }
+            // more than 8 tiles per group (wide models): the rest in a second round
+            const float *src = fold.xpart + (int64_t)b * xd + 4 * fold_jq;
             const int64_t tstride = (int64_t)fold.rows * xd;
-#pragma unroll 8
-            for (int t = tg; t < fold.n_tiles; t += G) {
+            for (int t = fold_tg + 8 * fold_G; t < fold.n_tiles; t += fold_G) {
                 const float4 v = *reinterpret_cast<const float4 *>(src + t * tstride);
                 a.x += v.x; a.y += v.y; a.z += v.z; a.w += v.w;
             }
-            *reinterpret_cast<float4 *>(&comb[tg * xd + 4 * jq]) = a;
+            *reinterpret_cast<float4 *>(&comb[fold_tg * xd + 4 * fold_jq]) = a;
         }
-        __syncthreads();
+        lds_barrier();
         if ((int)threadIdx.x < xd) {
             float sum = 0.0f;
-            for (int gg = 0; gg < G; gg++) sum += comb[gg * xd + threadIdx.x];   // fixed order
+            for (int gg = 0; gg < fold_G; gg++) sum += comb[gg * xd + threadIdx.x];   // fixed order
             Store<T>::st(&xs_l[threadIdx.x], sum);
         }
-        __syncthreads();
+        lds_barrier();
+        ld4<T, true>(xs_l + fold.b_off + 4 * g, Bv);
+        ld4<T, true>(xs_l + fold.c_off + 4 * g, Cv);
     }
-    float dl;
-    if (dt_w) {
+    if constexpr (DT != 0) {
         // dt_proj folded in: delta_raw[b,d] = sum_r dt_in[b,r] * dt_w[r,d], the dt_rank terms split over the
         // LG lanes of the row (dt_proj GEMM of the decode chain, src/mamba_ssm/gpu/inference.rs:1129-1146)
         const T *xr = FOLD ? xs_l : dt_in + (int64_t)b * bc_stride;
         float part = 0.0f;
-        if (flags & kStepDtT) {
-            const int kpl = dr / LG;
+        if constexpr (DT == 2) {
             const T *xp = xr + g * kpl, *wp = dt_w + (int64_t)d * dr + g * kpl;
             for (int c0 = 0; c0 < kpl; c0 += 16) {
                 float xv[4][4], wv[4][4];
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
                     const int kk = c0 + 4 * j;
-                    const int kc = kk < kpl ? kk : 0;   // in-range address for the masked-off chunks
-                    ld4<T>(xp + kc, xv[j], true);
-                    ld4<T>(wp + kc, wv[j], true);
-                    if (kk >= kpl) { xv[j][0] = 0.f; xv[j][1] = 0.f; xv[j][2] = 0.f; xv[j][3] = 0.f; }
+                    const bool in = kk < kpl;
+                    ld4<T, true>(xp + (in ? kk : 0), xv[j]);      // masked-off chunks read an in-range address
+                    if (c0 == 0) {
+#pragma unroll
+                        for (int i = 0; i < 4; i++) wv[j][i] = wv0[j][i];
+                    } else {
+                        ld4<T, true>(wp + (in ? kk : 0), wv[j]);
+                    }
+#pragma unroll
+                    for (int i = 0; i < 4; i++) xv[j][i] = in ? xv[j][i] : 0.0f;
                 }
 #pragma unroll
                 for (int j = 0; j < 4; j++)
@@ -107,39 +151,31 @@ __global__ __launch_bounds__(256) void ssm_step_kernel(
                     for (int i = 0; i < 4; i++) part = fmaf(xv[j][i], wv[j][i], part);
             }
         } else {
-        const T *wc = dt_w + d;
-        // batches of 12 terms per lane with every load of a batch issued before the first multiply-add:
-        // the loop is a latency chain otherwise (dt_rank 48 over 4 lanes = one batch)
-        constexpr int kBatch = 12;
-        for (int k0 = g; k0 < dr; k0 += kBatch * LG) {
-            float xv[kBatch], wv[kBatch];
+            const T *wc = dt_w + d;
+            // batches of 12 terms per lane with every load of a batch issued before the first multiply-add:
+            // the loop is a latency chain otherwise (dt_rank 48 over 4 lanes = one batch)
+            constexpr int kBatch = 12;
+            for (int k0 = g; k0 < dr; k0 += kBatch * LG) {
+                float xv[kBatch], wv[kBatch];
 #pragma unroll
-            for (int j = 0; j < kBatch; j++) {
-                const int k = k0 + j * LG;
-                const int kc = k < dr ? k : g;   // in-range address for the masked-off terms
-                xv[j] = Store<T>::ld(xr + kc);
-                wv[j] = Store<T>::ld(wc + (int64_t)kc * di);
-                if (k >= dr) xv[j] = 0.0f;
+                for (int j = 0; j < kBatch; j++) {
+                    const int k = k0 + j * LG;
+                    const int kc = k < dr ? k : g;   // in-range address for the masked-off terms
+                    xv[j] = Store<T>::ld(xr + kc);
+                    wv[j] = Store<T>::ld(wc + (int64_t)kc * di);
+                    xv[j] = k < dr ? xv[j] : 0.0f;
+                }
+#pragma unroll
+                for (int j = 0; j < kBatch; j++) part = fmaf(xv[j], wv[j], part);
             }
-#pragma unroll
-            for (int j = 0; j < kBatch; j++) part = fmaf(xv[j], wv[j], part);
-        }
         }
 #pragma unroll
         for (int m = 1; m < LG; m <<= 1) part += __shfl_xor(part, m, kWave);
         dl = part;
-    } else {
-        dl = Store<T>::ld(delta + r);
     }
-    if (dt_bias) dl = softplus20(dl + dt_bias[d]);
-    const float uu = Store<T>::ld(u + r);
+    if (dt_bias) dl = softplus20(dl + bias);
     const float du = dl * uu;
-    const T *Br = FOLD ? xs_l + fold.b_off + 4 * g : Bbase + (int64_t)b * bc_stride + 4 * g;
-    const T *Cr = FOLD ? xs_l + fold.c_off + 4 * g : Cbase + (int64_t)b * bc_stride + 4 * g;
     const float x = dl * kLog2e;
-    float Bv[4], Cv[4];
-    ld4<T>(Br, Bv, (flags & kStepVecBC) != 0);
-    ld4<T>(Cr, Cv, (flags & kStepVecBC) != 0);
     hv.x = fmaf(fast_exp2(x * av.x), hv.x, du * Bv[0]);
     hv.y = fmaf(fast_exp2(x * av.y), hv.y, du * Bv[1]);
     hv.z = fmaf(fast_exp2(x * av.z), hv.z, du * Bv[2]);
@@ -153,9 +189,9 @@ __global__ __launch_bounds__(256) void ssm_step_kernel(
     if (live) {
         *reinterpret_cast<float4 *>(h + r * ds + 4 * g) = hv;
         if (g == 0) {
-            acc = fmaf(Dp[d], uu, acc);
-            if (gate_mode == 1) acc *= Store<T>::ld(gate + (int64_t)b * gate_stride + d);
-            if (gate_mode == 2) acc *= silu(Store<T>::ld(gate + (int64_t)b * gate_stride + d));
+            acc = fmaf(Dd, uu, acc);
+            if (gate_mode == 1) acc *= gz;
+            if (gate_mode == 2) acc *= silu(gz);
             Store<T>::st(y + r, acc);
         }
     }
@@ -167,7 +203,7 @@ __global__ __launch_bounds__(256) void ssm_step_generic_kernel(
     float *__restrict__ h, T *__restrict__ y, const T *__restrict__ delta, const T *__restrict__ u,
     const T *__restrict__ Bbase, const T *__restrict__ Cbase, int64_t bc_stride,
     const T *__restrict__ gate, int64_t gate_stride, int gate_mode, const float *__restrict__ dt_bias,
-    const T *__restrict__ dt_in, const T *__restrict__ dt_w, int dr, int /*flags*/,
+    const T *__restrict__ dt_in, const T *__restrict__ dt_w, int dr,
     const float *__restrict__ a_neg, const float *__restrict__ Dp, int64_t total, int di, int ds) {
     const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (r >= total) return;
@@ -207,18 +243,18 @@ static int launch_step(hipStream_t st, float *h, void *y, const void *delta, con
                        const StepFold *fold = nullptr) {
     const int64_t total = (int64_t)batch * di;
     if (!gate) gate_mode = 0;
-    int flags = 0;
 #define MRS_ARGS h, (T *)y, (const T *)delta, (const T *)u, (const T *)Bb, (const T *)Cb, bc_stride, \
-                 (const T *)gate, gate_stride, gate_mode, dt_bias, (const T *)dt_in, (const T *)dt_w, dr, flags, a_neg, D, total, di, ds
+                 (const T *)gate, gate_stride, gate_mode, dt_bias, (const T *)dt_in, (const T *)dt_w, dr, a_neg, D, total, di, ds
     const bool vec_ok = aligned(h, 16) && aligned(a_neg, 16);
     int lg = 0;
     if (vec_ok && (ds == 4 || ds == 8 || ds == 16 || ds == 32 || ds == 64 || ds == 128 || ds == 256)) lg = ds / 4;
     const size_t v4 = 4 * sizeof(T);
-    if (bc_stride % 4 == 0 && aligned(Bb, v4) && aligned(Cb, v4)) flags |= kStepVecBC;
+    const bool vec_bc = bc_stride % 4 == 0 && aligned(Bb, v4) && aligned(Cb, v4);
+    int dt_mode = dt_w ? 1 : 0;
     if (dt_w && dt_transposed) {
         if (!(lg && dr % (4 * lg) == 0 && bc_stride % 4 == 0 && aligned(dt_in, v4) && aligned(dt_w, v4)))
             return fail(MRS_E_SHAPE, "ssm step: transposed dt_w needs d_state a power of two in 4..256, dt_rank %% d_state == 0 and 4-element aligned rows");
-        flags |= kStepDtT;
+        dt_mode = 2;
     }
     if (lg) {
         const int64_t threads = total * lg;
@@ -227,19 +263,33 @@ static int launch_step(hipStream_t st, float *h, void *y, const void *delta, con
         const dim3 grid((unsigned)blocks), block(256);
         if (fold) {
             // the row sits in LDS: offsets must suit the vector reads, every workgroup must lie inside one batch row
-            if (!(fold->xpart && fold->xd >= 4 && fold->xd % 4 == 0 && fold->xd <= kFoldMaxXd && fold->rows == batch && di % (256 / lg) == 0 && dt_w &&
-                  fold->b_off % 4 == 0 && fold->c_off % 4 == 0 && fold->b_off + ds <= fold->xd && fold->c_off + ds <= fold->xd && dr <= fold->xd))
-                return fail(MRS_E_SHAPE, "ssm step: folded x_proj needs xd <= %d, d_inner %% %d == 0, 4-aligned B/C offsets", kFoldMaxXd, 256 / lg);
-            flags |= kStepVecBC;
-#define MRS_LGF(L) case L: hipLaunchKernelGGL((ssm_step_kernel<T, L, true>), grid, block, 0, st, MRS_ARGS, *fold); break
+            if (!(fold->xpart && fold->xd >= 4 && fold->xd % 4 == 0 && fold->xd <= kFoldMaxXd && fold->rows == batch && di % (256 / lg) == 0 &&
+                  dt_mode == 2 && fold->b_off % 4 == 0 && fold->c_off % 4 == 0 && fold->b_off + ds <= fold->xd && fold->c_off + ds <= fold->xd &&
+                  dr <= fold->xd))
+                return fail(MRS_E_SHAPE, "ssm step: folded x_proj needs xd <= %d, d_inner %% %d == 0, 4-aligned B/C offsets, transposed dt_w",
+                            kFoldMaxXd, 256 / lg);
+#define MRS_LGF(L) case L: hipLaunchKernelGGL((ssm_step_kernel<T, L, 2, true, true>), grid, block, 0, st, MRS_ARGS, *fold); break
             switch (lg) { MRS_LGF(1); MRS_LGF(2); MRS_LGF(4); MRS_LGF(8); MRS_LGF(16); MRS_LGF(32); MRS_LGF(64); }
 #undef MRS_LGF
             return check_launch("ssm_step_kernel");
         }
         const StepFold nofold = {};
-#define MRS_LG(L) case L: hipLaunchKernelGGL((ssm_step_kernel<T, L>), grid, block, 0, st, MRS_ARGS, nofold); break
+        // (delta source, vector B/C): the transposed dt_w route implies vector rows (checked above)
+        const int variant = dt_mode == 2 ? 4 : dt_mode * 2 + (vec_bc ? 1 : 0);
+#define MRS_LGV(L, DT_, V_) hipLaunchKernelGGL((ssm_step_kernel<T, L, DT_, V_>), grid, block, 0, st, MRS_ARGS, nofold)
+#define MRS_LG(L)                                   \
+    case L:                                         \
+        switch (variant) {                          \
+            case 0: MRS_LGV(L, 0, false); break;    \
+            case 1: MRS_LGV(L, 0, true); break;     \
+            case 2: MRS_LGV(L, 1, false); break;    \
+            case 3: MRS_LGV(L, 1, true); break;     \
+            default: MRS_LGV(L, 2, true); break;    \
+        }                                           \
+        break
         switch (lg) { MRS_LG(1); MRS_LG(2); MRS_LG(4); MRS_LG(8); MRS_LG(16); MRS_LG(32); MRS_LG(64); }
 #undef MRS_LG
+#undef MRS_LGV
     } else {
         if (fold) return fail(MRS_E_SHAPE, "ssm step: folded x_proj needs d_state a power of two in 4..256");
         const int64_t blocks = (total + 255) / 256;
