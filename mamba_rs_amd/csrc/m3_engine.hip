@@ -37,7 +37,7 @@ __global__ __launch_bounds__(1024) void m3_layer_step_kernel(
     const float *__restrict__ c_bias, const float *__restrict__ Dp, const float *__restrict__ ngw, int nh, int hd, int ng,
     int nr, float a_floor, float eps, int outproj_norm) {
     constexpr int ds = 4 * LG;
-    __shared__ float kl[ds], ql[ds], red[16], scal[4];
+    __shared__ float kl[ds], ql[ds], red[16];
     const int b = blockIdx.x / nh, h = blockIdx.x - b * nh;
     const int tid = threadIdx.x, nthr = blockDim.x;
     const int p = tid / LG, g = tid % LG;
@@ -47,42 +47,49 @@ __global__ __launch_bounds__(1024) void m3_layer_step_kernel(
     const float *row = proj + (int64_t)b * ip;
     const float *zr = row, *xr = row + di, *braw = row + 2 * di + (int64_t)grp * ds, *craw = row + 2 * di + (int64_t)(ng + grp) * ds;
     const float *sc = row + 2 * di + 2 * (int64_t)ng * ds;   // dd_dt | dd_A | trap | angles
-    // state loads first: they are the long-latency part and do not depend on the prologue
+    // Every global load of the kernel up front -- none depends on another -- so that the body below costs one memory
+    // round trip, not one per phase; the barriers between the phases publish LDS only (lds_barrier) and leave loads in flight.
     float *Hrow = ssm + (bh * hd + p) * ds + 4 * g;
     float4 H = *reinterpret_cast<const float4 *>(Hrow);
     const float4 kp = *reinterpret_cast<const float4 *>(kst + bh * ds + 4 * g);
     const float vp = vst[bh * hd + p];
     const float xv = xr[h * hd + p];
+    const float zi = zr[h * hd + p];
+    const float ngv = outproj_norm ? ngw[h * hd + p] : 1.0f;
+    const float Dh = Dp[h];
+    const float s_dt = sc[h], s_dtb = dt_bias[h], s_A = sc[nh + h], s_tr = sc[2 * nh + h];
+    const bool own_n = tid < ds, own_a = tid < nr;   // blockDim.x >= d_state (headdim >= 4)
+    float bv_raw = 0.0f, cv_raw = 0.0f, bn = 0.0f, cn = 0.0f, bb_ = 0.0f, cb_ = 0.0f, ang_old = 0.0f, ang_in = 0.0f;
+    if (own_n) {
+        bv_raw = braw[tid]; cv_raw = craw[tid]; bn = bnw[tid]; cn = cnw[tid];
+        bb_ = b_bias[(int64_t)h * ds + tid]; cb_ = c_bias[(int64_t)h * ds + tid];
+    }
+    if (own_a) { ang_old = angle[bh * nr + tid]; ang_in = sc[3 * nh + tid]; }
 
     // ---- B/C RMSNorm over d_state (bcnorm_fwd, ops/norms.rs:50-80) + per-head bias ----
-    float ssb = 0.0f, ssc = 0.0f;
-    for (int n = tid; n < ds; n += nthr) { const float bv = braw[n], cv = craw[n]; ssb = fmaf(bv, bv, ssb); ssc = fmaf(cv, cv, ssc); }
+    float ssb = bv_raw * bv_raw, ssc = cv_raw * cv_raw;
 #pragma unroll
     for (int m = 32; m >= 1; m >>= 1) { ssb += __shfl_xor(ssb, m, kWave); ssc += __shfl_xor(ssc, m, kWave); }
     // only the first ceil(ds / 64) waves hold non-zero partial sums; every wave writes its own (zero) slot
     const int wv = tid >> 6, nw = (nthr + 63) >> 6;
     if ((tid & 63) == 0 && wv < 8) { red[wv] = ssb; red[8 + wv] = ssc; }
-    __syncthreads();
-    if (tid == 0) {
-        float sb = 0.0f, scc = 0.0f;
-        for (int i = 0; i < min(nw, 8); i++) { sb += red[i]; scc += red[8 + i]; }
-        scal[0] = 1.0f / sqrtf(sb / (float)ds + eps);
-        scal[1] = 1.0f / sqrtf(scc / (float)ds + eps);
-        // per-head scalars (m3_split + compute_abg, kernels/mamba3_ops.cu:72-160, 735-753)
-        scal[2] = softplus20(sc[h] + dt_bias[h]);                                 // dt
+    lds_barrier();
+    float sb = 0.0f, scc = 0.0f;
+    for (int i = 0; i < min(nw, 8); i++) { sb += red[i]; scc += red[8 + i]; }
+    const float invb = 1.0f / sqrtf(sb / (float)ds + eps), invc = 1.0f / sqrtf(scc / (float)ds + eps);
+    // per-head scalars (m3_split + compute_abg, kernels/mamba3_ops.cu:72-160, 735-753)
+    const float dtv = softplus20(s_dt + s_dtb);
+    if (own_n) {
+        kl[tid] = bv_raw * invb * bn + bb_;
+        ql[tid] = cv_raw * invc * cn + cb_;
     }
-    __syncthreads();
-    const float invb = scal[0], invc = scal[1], dtv = scal[2];
-    for (int n = tid; n < ds; n += nthr) {
-        kl[n] = braw[n] * invb * bnw[n] + b_bias[(int64_t)h * ds + n];
-        ql[n] = craw[n] * invc * cnw[n] + c_bias[(int64_t)h * ds + n];
-    }
-    __syncthreads();
+    lds_barrier();
     // ---- angle accumulation + rotation of the first 2*nr coordinates (angle_dt_fwd_batch + rope_fwd) ----
-    for (int a = tid; a < nr; a += nthr) {
-        const float delta = tanhf(sc[3 * nh + a]) * kPi * dtv;
+    if (own_a) {
+        const int a = tid;
+        const float delta = tanhf(ang_in) * kPi * dtv;
         const double two_pi = 6.283185307179586;
-        double acc = (double)angle[bh * nr + a] + (double)delta;
+        double acc = (double)ang_old + (double)delta;
         acc -= two_pi * floor(acc / two_pi);
         const float an = (float)acc;
         angle[bh * nr + a] = an;
@@ -92,10 +99,10 @@ __global__ __launch_bounds__(1024) void m3_layer_step_kernel(
         kl[2 * a] = cs * b0 - sn * b1; kl[2 * a + 1] = sn * b0 + cs * b1;
         ql[2 * a] = cs * c0 - sn * c1; ql[2 * a + 1] = sn * c0 + cs * c1;
     }
-    __syncthreads();
+    __syncthreads();   // a full barrier: every lane's read of the previous k_state has returned before the write at the end
     // ---- alpha / beta / gamma ----
-    const float a_val = fminf(-heavy_tail(sc[nh + h]), -a_floor);
-    const float trap = sigmoidf_fast(sc[2 * nh + h]);
+    const float a_val = fminf(-heavy_tail(s_A), -a_floor);
+    const float trap = sigmoidf_fast(s_tr);
     const float al = fast_exp2(a_val * dtv * kLog2e);
     const float be = al * dtv * (1.0f - trap), ga = trap * dtv;
     // ---- trapezoidal update of this lane's four states, y = H q + D x ----
@@ -112,7 +119,7 @@ __global__ __launch_bounds__(1024) void m3_layer_step_kernel(
     acc = fmaf(H.w, qc.w, acc);
 #pragma unroll
     for (int m = 1; m < LG; m <<= 1) acc += __shfl_xor(acc, m, kWave);
-    const float yv = fmaf(Dp[h], xv, acc);
+    const float yv = fmaf(Dh, xv, acc);
     *reinterpret_cast<float4 *>(Hrow) = H;
     // ---- gate: y * silu(z), or RMSNormGated over the head first (rmsnorm_gated_forward, ops/norms.rs:84-114) ----
     float inv_y = 1.0f;
@@ -120,20 +127,18 @@ __global__ __launch_bounds__(1024) void m3_layer_step_kernel(
         float sq = (g == 0) ? yv * yv : 0.0f;
 #pragma unroll
         for (int m = 32; m >= 1; m >>= 1) sq += __shfl_xor(sq, m, kWave);
-        __syncthreads();   // red is reused
-        if ((tid & 63) == 0) red[wv & 15] = sq;
-        __syncthreads();
+        if ((tid & 63) == 0) red[wv & 15] = sq;   // (every lane read red before the full barrier above)
+        lds_barrier();
         float tot = 0.0f;
         for (int i = 0; i < min(nw, 16); i++) tot += red[i];
         inv_y = 1.0f / sqrtf(tot / (float)hd + eps);
     }
     if (g == 0) {
-        const float zi = zr[h * hd + p];
-        const float o = outproj_norm ? yv * inv_y * ngw[h * hd + p] * silu(zi) : yv * silu(zi);
+        const float o = outproj_norm ? yv * inv_y * ngv * silu(zi) : yv * silu(zi);
         Store<T>::st(gated + (int64_t)b * di + h * hd + p, o);
         vst[bh * hd + p] = xv;
     }
-    // every lane has read the previous k_state (kp) at the top; the barriers above order those reads before this write
+    // every lane has read the previous k_state (kp) at the top; the full barrier after the rotation orders those reads before this write
     if (p == 0) *reinterpret_cast<float4 *>(kst + bh * ds + 4 * g) = kc;
 }
 
@@ -515,7 +520,7 @@ extern "C" int mrs_m3_backbone_create(mrs_m3_backbone **out, int gpu_ordinal, co
     if (nh % cfg->ngroups != 0) return fail(MRS_E_SHAPE, "%s: nheads %d is not a multiple of ngroups %d", fn, nh, cfg->ngroups);
     const int ds = cfg->d_state, lg = ds / 4;
     // one lane per four states of a row: a workgroup of headdim * d_state / 4 lanes, whole waves only
-    if (ds % 4 != 0 || (lg & (lg - 1)) != 0 || lg > 64 || (int64_t)cfg->headdim * lg > 1024 || ((int64_t)cfg->headdim * lg) % 64 != 0)
+    if (ds % 4 != 0 || (lg & (lg - 1)) != 0 || lg > 64 || cfg->headdim < 4 || (int64_t)cfg->headdim * lg > 1024 || ((int64_t)cfg->headdim * lg) % 64 != 0)
         return fail(MRS_E_SHAPE, "%s: d_state must be 4 x a power of two <= 256 and headdim * d_state / 4 a multiple of 64 <= 1024 (got %d, %d)", fn, ds, cfg->headdim);
     if (cfg->n_rope_angles < 0 || 2 * cfg->n_rope_angles > ds) return fail(MRS_E_SHAPE, "%s: n_rope_angles %d outside 0..d_state/2", fn, cfg->n_rope_angles);
     if (!(cfg->a_floor > 0.0f)) return fail(MRS_E_SHAPE, "%s: a_floor must be > 0", fn);
