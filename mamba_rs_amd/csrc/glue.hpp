@@ -16,13 +16,22 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(float *__restrict__ re
     __shared__ float part[4];
     const int64_t row = blockIdx.x;
     float *r = residual + row * dm;
-    float v[kMaxPer];
+    float v[kMaxPer];   // indexed by unrolled loop counters only (a run-time index would put it in scratch memory)
     float ss = 0.0f;
-    int cnt = 0;
-    for (int i = threadIdx.x; i < dm; i += 256, cnt++) {
+#pragma unroll
+    for (int k = 0; k < kMaxPer; k++) {
+        const int i = threadIdx.x + 256 * k;
+        float x = 0.0f;
+        if (i < dm) {
+            x = r[i];
+            if (add) { x += Store<T>::ld(add + row * dm + i); r[i] = x; }
+        }
+        v[k] = x;
+        ss = fmaf(x, x, ss);
+    }
+    for (int i = threadIdx.x + 256 * kMaxPer; i < dm; i += 256) {
         float x = r[i];
         if (add) { x += Store<T>::ld(add + row * dm + i); r[i] = x; }
-        if (cnt < kMaxPer) v[cnt] = x;
         ss = fmaf(x, x, ss);
     }
 #pragma unroll
@@ -33,22 +42,30 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(float *__restrict__ re
     float rms = sqrtf(ss / (float)dm + eps);
     if (!isfinite(rms) || rms < 1e-20f) rms = 1.0f;
     const float inv = 1.0f / rms;
-    cnt = 0;
-    for (int i = threadIdx.x; i < dm; i += 256, cnt++) {
-        const float x = cnt < kMaxPer ? v[cnt] : r[i];
-        const float o = x * inv * w[i];
+#pragma unroll
+    for (int k = 0; k < kMaxPer; k++) {
+        const int i = threadIdx.x + 256 * k;
+        if (i < dm) {
+            const float o = v[k] * inv * w[i];
+            Store<TO>::st(out + row * out_stride + i, o);
+            if (out2) Store<T>::st(out2 + row * out_stride + i, o);
+        }
+    }
+    for (int i = threadIdx.x + 256 * kMaxPer; i < dm; i += 256) {
+        const float o = r[i] * inv * w[i];
         Store<TO>::st(out + row * out_stride + i, o);
         if (out2) Store<T>::st(out2 + row * out_stride + i, o);
     }
 }
 
 // Prefill-sized rows: one wave per row, 4 elements per lane and trip (16-byte residual accesses), the row
-// kept in registers between the sum of squares and the scaling.  Same arithmetic as add_rmsnorm_kernel.
-template <typename T, typename TO>
+// kept in registers between the sum of squares and the scaling.  Same arithmetic as add_rmsnorm_kernel.  TRIPS (the
+// number of 16-byte pieces a lane holds, d_model <= 256 TRIPS) is a template parameter: the register array must be
+// indexed by compile-time constants, or it lands in scratch memory and every element makes a round trip through it.
+template <typename T, typename TO, int TRIPS>
 __global__ __launch_bounds__(256) void add_rmsnorm_rows_kernel(float *__restrict__ residual, const T *__restrict__ add,
                                                                TO *__restrict__ out, const float *__restrict__ w,
                                                                float eps, int64_t rows, int dm) {
-    constexpr int kMaxTrips = 16;  // d_model <= 4096 stays in registers; longer rows re-read
     const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (row >= rows) return;
     const int lane = threadIdx.x & 63;
@@ -57,34 +74,30 @@ __global__ __launch_bounds__(256) void add_rmsnorm_rows_kernel(float *__restrict
     struct alignas(4 * sizeof(T)) V4 { T v[4]; };
     struct alignas(4 * sizeof(TO)) O4 { TO v[4]; };
     const V4 *a4 = reinterpret_cast<const V4 *>(add ? add + row * dm : nullptr);
-    float4 v[kMaxTrips];
-    float ss = 0.0f;
-    int cnt = 0;
-    for (int c0 = lane; c0 < nv; c0 += 4 * 64) {
-        // four trips at a time, every load issued before the first use
-        float4 x[4];
-        V4 a[4];
+    const float4 *w4 = reinterpret_cast<const float4 *>(w);
+    float4 v[TRIPS], ww[TRIPS];
+    V4 a[TRIPS];
+    // every load of the row before the first use
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const int c = c0 + 64 * j;
-            if (c < nv) {
-                x[j] = r4[c];
-                if (add) a[j] = a4[c];
-            }
+    for (int k = 0; k < TRIPS; k++) {
+        const int c = lane + 64 * k;
+        if (c < nv) {
+            v[k] = r4[c];
+            if (add) a[k] = a4[c];
+            ww[k] = w4[c];
         }
+    }
+    float ss = 0.0f;
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const int c = c0 + 64 * j;
-            if (c < nv) {
-                if (add) {
-                    x[j].x += Store<T>::ld(&a[j].v[0]); x[j].y += Store<T>::ld(&a[j].v[1]);
-                    x[j].z += Store<T>::ld(&a[j].v[2]); x[j].w += Store<T>::ld(&a[j].v[3]);
-                    r4[c] = x[j];
-                }
-                if (cnt < kMaxTrips) v[cnt] = x[j];
-                cnt++;
-                ss = fmaf(x[j].x, x[j].x, ss); ss = fmaf(x[j].y, x[j].y, ss); ss = fmaf(x[j].z, x[j].z, ss); ss = fmaf(x[j].w, x[j].w, ss);
+    for (int k = 0; k < TRIPS; k++) {
+        const int c = lane + 64 * k;
+        if (c < nv) {
+            if (add) {
+                v[k].x += Store<T>::ld(&a[k].v[0]); v[k].y += Store<T>::ld(&a[k].v[1]);
+                v[k].z += Store<T>::ld(&a[k].v[2]); v[k].w += Store<T>::ld(&a[k].v[3]);
+                r4[c] = v[k];
             }
+            ss = fmaf(v[k].x, v[k].x, ss); ss = fmaf(v[k].y, v[k].y, ss); ss = fmaf(v[k].z, v[k].z, ss); ss = fmaf(v[k].w, v[k].w, ss);
         }
     }
 #pragma unroll
@@ -93,15 +106,15 @@ __global__ __launch_bounds__(256) void add_rmsnorm_rows_kernel(float *__restrict
     if (!isfinite(rms) || rms < 1e-20f) rms = 1.0f;
     const float inv = 1.0f / rms;
     O4 *o4 = reinterpret_cast<O4 *>(out + row * dm);
-    const float4 *w4 = reinterpret_cast<const float4 *>(w);
-    cnt = 0;
-    for (int c = lane; c < nv; c += 64, cnt++) {
-        const float4 x = cnt < kMaxTrips ? v[cnt] : r4[c];
-        const float4 ww = w4[c];
-        O4 o;
-        Store<TO>::st(&o.v[0], x.x * inv * ww.x); Store<TO>::st(&o.v[1], x.y * inv * ww.y);
-        Store<TO>::st(&o.v[2], x.z * inv * ww.z); Store<TO>::st(&o.v[3], x.w * inv * ww.w);
-        o4[c] = o;
+#pragma unroll
+    for (int k = 0; k < TRIPS; k++) {
+        const int c = lane + 64 * k;
+        if (c < nv) {
+            O4 o;
+            Store<TO>::st(&o.v[0], v[k].x * inv * ww[k].x); Store<TO>::st(&o.v[1], v[k].y * inv * ww[k].y);
+            Store<TO>::st(&o.v[2], v[k].z * inv * ww[k].z); Store<TO>::st(&o.v[3], v[k].w * inv * ww[k].w);
+            o4[c] = o;
+        }
     }
 }
 
@@ -116,7 +129,6 @@ static __global__ __launch_bounds__(256) void bias_rows_kernel(float *__restrict
     if (i < n) out[i] = bias[i % dm];
 }
 
-
 // residual (f32, rows x dm) += add (storage type, may be null); out = rmsnorm(residual) * w as f32 (out_f32) or in the
 // storage type; out2 (may be null): the result once more in the storage type.  Prefill-sized row counts take the
 // wave-per-row kernel.
@@ -124,9 +136,15 @@ template <typename T>
 inline void launch_add_rmsnorm_typed(hipStream_t st, float *residual, const void *add, void *out, bool out_f32, void *out2, const float *w,
                                      float eps, int64_t rows, int dm, int64_t out_stride) {
     const dim3 grid((unsigned)rows), block(256);
-    if (rows >= 256 && dm % 4 == 0 && out_stride == dm && !out2 && !out_f32) {
-        hipLaunchKernelGGL((add_rmsnorm_rows_kernel<T, T>), dim3((unsigned)((rows + 3) / 4)), block, 0, st, residual, (const T *)add, (T *)out, w,
-                           eps, rows, dm);
+    if (rows >= 256 && dm % 4 == 0 && dm <= 4096 && out_stride == dm && !out2 && !out_f32) {
+        const dim3 g4((unsigned)((rows + 3) / 4));
+#define MRS_ROWS(TR) hipLaunchKernelGGL((add_rmsnorm_rows_kernel<T, T, TR>), g4, block, 0, st, residual, (const T *)add, (T *)out, w, eps, rows, dm)
+        const int trips = (dm / 4 + 63) / 64;
+        if (trips <= 2) MRS_ROWS(2);
+        else if (trips <= 4) MRS_ROWS(4);
+        else if (trips <= 8) MRS_ROWS(8);
+        else MRS_ROWS(16);
+#undef MRS_ROWS
         return;
     }
     if (out_f32)

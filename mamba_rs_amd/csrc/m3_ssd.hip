@@ -202,7 +202,7 @@ __global__ __launch_bounds__(HD * 4) void m3_ssd_kernel(
     prefetch(c_begin);
     for (int c = c_begin; c < c_end; c++) {
         const int t0 = c * kCS;
-        __syncthreads();  // every wave is done reading the previous chunk's tiles
+        lds_barrier();  // every wave is done reading the previous chunk's tiles (LDS only: y stores and the prefetch stay in flight)
         // ---- registers -> LDS ----
 #pragma unroll
         for (int v = 0; v < NV; v++) {
@@ -248,7 +248,7 @@ __global__ __launch_bounds__(HD * 4) void m3_ssd_kernel(
             sm.sc[w][3][l] = fast_exp2(dA * kLog2e);
             sm.sc[w][4][l] = fast_exp2((dAend - dA) * kLog2e) * scl;
         }
-        __syncthreads();  // tiles visible to every wave
+        lds_barrier();  // tiles visible to every wave
         if (c + 1 < c_end) prefetch(c + 1);
         dAsum += dAend;
 
@@ -315,7 +315,7 @@ __global__ __launch_bounds__(HD * 4) void m3_ssd_kernel(
             St[jn] = s;
         }
         if (!STATE_ONLY) {
-            __syncthreads();  // P tiles visible
+            lds_barrier();  // P tiles visible; the next chunk's prefetch, issued above, keeps running under the products below
 #pragma unroll
             for (int it = 0; it < 4; it++) {
                 // y_off = exp(dA[t]) * Q S_in^T     (acc rows t = 16it+4lg+i, cols p = 16w+lr)
