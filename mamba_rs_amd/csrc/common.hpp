@@ -61,6 +61,17 @@ __device__ __forceinline__ float softplus20(float v) {
 // through global memory.
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
+// softplus for a result that is stored in 16 bits (8 or 11 significant bits): one branch of arithmetic instead of two.
+// log(1 + e) on the transcendental unit is off by at most 2^-24 / e relative, i.e. below 2^-12 for e >= 2^-12; under
+// that, log1p(e) = e (1 - e/2) to 2^-25.  Half the issue slots of softplus20.
+__device__ __forceinline__ float softplus20_16(float v) {
+    const float e = fast_exp2(fminf(v, 20.0f) * kLog2e);
+    const float small = e * fmaf(e, -0.5f, 1.0f);
+    const float vialog = __builtin_amdgcn_logf(1.0f + e) * 0.6931471805599453f;
+    const float r = e < 0.000244140625f ? small : vialog;
+    return v > 20.0f ? v : r;
+}
+
 // ---- host-side error plumbing ---------------------------------------------
 void set_error(const char *fmt, ...);
 int fail(int code, const char *fmt, ...);

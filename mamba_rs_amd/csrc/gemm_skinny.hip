@@ -16,6 +16,7 @@
 //     and only u and the gate half are written.
 #include "common.hpp"
 #include <stdlib.h>
+#include <algorithm>
 
 namespace mrs {
 
@@ -351,47 +352,72 @@ __global__ __launch_bounds__(256) void prenorm_rows_kernel(float *__restrict__ p
 // 130m prefill shape) and nothing else: a workgroup forms a 64 x 64 tile with two v_mfma_f32_16x16x32 steps per 16 x 16 block
 // (K zero-padded to a multiple of 32), applies the epilogue on the accumulators, and transposes through LDS so that the
 // rows leave as 16-byte stores.  dt_in rows have stride xs (they are the head of the x_proj row); wt is [d_inner][dt_rank].
-template <typename T>
+// KS = 32-wide k-steps held in registers (dt_rank <= 32 KS).  A workgroup owns 64 columns and walks row tiles blockIdx.y,
+// blockIdx.y + gridDim.y, ...: the weight fragments and the bias are loaded once, the next tile's rows are requested
+// while the current tile is in its epilogue, and the transpose through LDS is private to each wave (no workgroup
+// barrier).  Measured at the 130m prefill shape (50 MB of delta per layer): 25.7 us with one tile per workgroup, 22.4 us
+// walking row tiles, 26.5 us walking along the rows instead, 21.2 us with the one-branch softplus20_16.
+template <typename T, int KS>
 __global__ __launch_bounds__(256) void dt_proj_softplus_kernel(T *__restrict__ delta, const T *__restrict__ dt_in, int64_t xs,
                                                                const T *__restrict__ wt, const float *__restrict__ bias, int64_t rows,
                                                                int di, int dr) {
     __shared__ alignas(16) T tile[4][16][64 + 8];
     const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, lr = l & 15, lg = l >> 4;
-    const int64_t m0 = (int64_t)blockIdx.y * 64 + 16 * w;
     const int n0 = blockIdx.x * 64;
-    v4f acc[4];
-#pragma unroll
-    for (int nt = 0; nt < 4; nt++) acc[nt] = (v4f){0.f, 0.f, 0.f, 0.f};
-    const int64_t arow = min(m0 + lr, rows - 1);
-    for (int k0 = 0; k0 < dr; k0 += 32) {
-        const int k = k0 + 8 * lg;
-        const bool kin = k < dr;   // dt_rank % 8 == 0: a lane's 8 values are all inside or all outside
-        uint4 af = make_uint4(0, 0, 0, 0);
-        if (kin) af = *reinterpret_cast<const uint4 *>(dt_in + arow * xs + k);
-#pragma unroll
-        for (int nt = 0; nt < 4; nt++) {
-            const int col = min(n0 + 16 * nt + lr, di - 1);
-            uint4 bf = make_uint4(0, 0, 0, 0);
-            if (kin) bf = *reinterpret_cast<const uint4 *>(wt + (int64_t)col * dr + k);
-            acc[nt] = Mma32<T>::mma(af, bf, acc[nt]);
-        }
-    }
+    const int64_t n_tiles = (rows + 63) / 64;
+    // weight fragments and bias of this workgroup's 64 columns
+    uint4 bf[KS][4];
+    float bv[4];
 #pragma unroll
     for (int nt = 0; nt < 4; nt++) {
         const int col = min(n0 + 16 * nt + lr, di - 1);
-        const float bv = bias[col];
+        bv[nt] = bias[col];
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const T raw = (T)acc[nt][i];   // the projection as the reference stores it, before bias and softplus
-            Store<T>::st(&tile[w][4 * lg + i][16 * nt + lr], softplus20(Store<T>::ld(&raw) + bv));
+        for (int ks = 0; ks < KS; ks++) {
+            const int k = 32 * ks + 8 * lg;   // dt_rank % 8 == 0: a lane's 8 values are all inside or all outside
+            bf[ks][nt] = k < dr ? *reinterpret_cast<const uint4 *>(wt + (int64_t)col * dr + k) : make_uint4(0, 0, 0, 0);
         }
     }
-    __syncthreads();
+    auto load_a = [&](int64_t rt, uint4 (&af)[KS]) {
+        const int64_t arow = min(rt * 64 + 16 * w + lr, rows - 1);
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
-        const int idx = l + 64 * j, r = idx >> 3, seg = idx & 7;
-        if (m0 + r < rows && n0 + seg * 8 < di)
-            *reinterpret_cast<uint4 *>(delta + (m0 + r) * di + n0 + seg * 8) = *reinterpret_cast<const uint4 *>(&tile[w][r][seg * 8]);
+        for (int ks = 0; ks < KS; ks++) {
+            const int k = 32 * ks + 8 * lg;
+            af[ks] = k < dr ? *reinterpret_cast<const uint4 *>(dt_in + arow * xs + k) : make_uint4(0, 0, 0, 0);
+        }
+    };
+    uint4 af[KS], an[KS];
+    int64_t rt = blockIdx.y;
+    if (rt < n_tiles) load_a(rt, af);
+    for (; rt < n_tiles; rt += gridDim.y) {
+        const int64_t nxt = rt + gridDim.y;
+        if (nxt < n_tiles) load_a(nxt, an);
+        v4f acc[4];
+#pragma unroll
+        for (int nt = 0; nt < 4; nt++) {
+            acc[nt] = (v4f){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++) acc[nt] = Mma32<T>::mma(af[ks], bf[ks][nt], acc[nt]);
+        }
+#pragma unroll
+        for (int nt = 0; nt < 4; nt++) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const T raw = (T)acc[nt][i];   // the projection as the reference stores it, before bias and softplus
+                Store<T>::st(&tile[w][4 * lg + i][16 * nt + lr], softplus20_16(Store<T>::ld(&raw) + bv[nt]));
+            }
+        }
+        __builtin_amdgcn_wave_barrier();   // tile[w] belongs to this wave: its LDS accesses execute in program order
+        const int64_t m0 = rt * 64 + 16 * w;
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const int idx = l + 64 * j, r = idx >> 3, seg = idx & 7;
+            if (m0 + r < rows && n0 + seg * 8 < di)
+                *reinterpret_cast<uint4 *>(delta + (m0 + r) * di + n0 + seg * 8) = *reinterpret_cast<const uint4 *>(&tile[w][r][seg * 8]);
+        }
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) af[ks] = an[ks];
     }
 }
 
@@ -471,7 +497,7 @@ int launch_prenorm_rows(hipStream_t st, int dtype, float *partials, int n_partia
 }
 
 bool dt_proj_softplus_ok(int dtype, int di, int dr, int64_t xs, const void *delta, const void *dt_in, const void *wt) {
-    return (dtype == MRS_BF16 || dtype == MRS_F16) && di % 8 == 0 && dr >= 8 && dr % 8 == 0 && xs % 8 == 0 && aligned(delta, 16) &&
+    return (dtype == MRS_BF16 || dtype == MRS_F16) && di % 8 == 0 && dr >= 8 && dr % 8 == 0 && dr <= 256 && xs % 8 == 0 && aligned(delta, 16) &&
            aligned(dt_in, 16) && aligned(wt, 16);
 }
 
@@ -479,11 +505,26 @@ int launch_dt_proj_softplus(hipStream_t st, int dtype, void *delta, const void *
                             int64_t rows, int di, int dr) {
     if (!dt_proj_softplus_ok(dtype, di, dr, xs, delta, dt_in, wt))
         return fail(MRS_E_SHAPE, "dt_proj+softplus: needs 16-bit storage, d_inner, dt_rank and the row stride multiples of 8, 16-byte aligned operands");
-    const int64_t gy = (rows + 63) / 64;
-    if (rows < 1 || gy > 65535) return fail(MRS_E_SHAPE, "dt_proj+softplus: rows=%lld", (long long)rows);
-    const dim3 grid((unsigned)((di + 63) / 64), (unsigned)gy), block(256);
-    if (dtype == MRS_BF16) hipLaunchKernelGGL((dt_proj_softplus_kernel<bf16_t>), grid, block, 0, st, (bf16_t *)delta, (const bf16_t *)dt_in, xs, (const bf16_t *)wt, bias, rows, di, dr);
-    else hipLaunchKernelGGL((dt_proj_softplus_kernel<f16_t>), grid, block, 0, st, (f16_t *)delta, (const f16_t *)dt_in, xs, (const f16_t *)wt, bias, rows, di, dr);
+    if (rows < 1) return fail(MRS_E_SHAPE, "dt_proj+softplus: rows=%lld", (long long)rows);
+    // about eight workgroups per compute unit in flight, each walking several row tiles
+    const int64_t n_tiles = (rows + 63) / 64;
+    const int gx = (di + 63) / 64;
+    const int64_t gy = std::max<int64_t>(1, std::min<int64_t>(n_tiles, (2048 + gx - 1) / gx));
+    const dim3 grid((unsigned)gx, (unsigned)gy), block(256);
+    const int ks = (dr + 31) / 32;
+#define MRS_DTP(T_, KS_) hipLaunchKernelGGL((dt_proj_softplus_kernel<T_, KS_>), grid, block, 0, st, (T_ *)delta, (const T_ *)dt_in, xs, (const T_ *)wt, bias, rows, di, dr)
+#define MRS_DTP_KS(T_)                                      \
+    switch (ks) {                                           \
+        case 1: MRS_DTP(T_, 1); break;                      \
+        case 2: MRS_DTP(T_, 2); break;                      \
+        case 3: MRS_DTP(T_, 3); break;                      \
+        case 4: MRS_DTP(T_, 4); break;                      \
+        case 5: case 6: MRS_DTP(T_, 6); break;              \
+        default: MRS_DTP(T_, 8); break;                     \
+    }
+    if (dtype == MRS_BF16) { MRS_DTP_KS(bf16_t) } else { MRS_DTP_KS(f16_t) }
+#undef MRS_DTP_KS
+#undef MRS_DTP
     return check_launch("dt_proj_softplus_kernel");
 }
 
