@@ -61,6 +61,8 @@ template <typename T> __device__ __forceinline__ float dot8(uint4 a, uint4 b, fl
 template <typename TO> __device__ __forceinline__ void store_out(TO *p, float v) { Store<TO>::st(p, v); }
 
 // EPI 0: C[row, col] = sum (TO = T or float)
+// EPI 3: EPI 1 for any number of conv taps up to kMaxConvTaps (EPI 1 itself: four taps, window and taps one 16-byte
+//        vector each, a third of the registers).
 // EPI 1: in_proj of a Mamba-1 layer: columns < di are conv inputs (conv state [M][di][dc] f32 shifted in
 //        place, u[row, col] = silu(conv)), columns >= di (the gate) are stored to C.
 // Grid: x = 16-column tile, y = 16-row tile.  A workgroup pulls 16 rows of A and 16 rows of Wt through
@@ -97,33 +99,37 @@ __global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu
     const T *wrow = Wt + (int64_t)min(n0 + lr, N - 1) * K + 8 * lg;
     const T *arow = A + (int64_t)min(m0 + lr, M - 1) * lda + 8 * lg;
     float inv = 1.0f;
-    if (PRO == 1 && tid < 256) {
-        // epilogue thread (row tid/16, column tid%16): the 16 lanes of a row share the sum over the partials
-        const float *pp = ep.partials + (int64_t)min(m0 + (tid >> 4), M - 1) * ep.n_partials;
-        float ss = 0.0f;
-        for (int p = tid & 15; p < ep.n_partials; p += 16) ss += pp[p];
+    auto row_scale = [&]() {
+        if (PRO == 1 && tid < 256) {
+            // epilogue thread (row tid/16, column tid%16): the 16 lanes of a row share the sum over the partials
+            const float *pp = ep.partials + (int64_t)min(m0 + (tid >> 4), M - 1) * ep.n_partials;
+            float ss = 0.0f;
+            for (int p = tid & 15; p < ep.n_partials; p += 16) ss += pp[p];
 #pragma unroll
-        for (int m = 8; m >= 1; m >>= 1) ss += __shfl_xor(ss, m, kWave);
-        float rms = sqrtf(ss / (float)K + ep.eps);
-        if (!isfinite(rms) || rms < 1e-20f) rms = 1.0f;
-        inv = 1.0f / rms;
-    }
+            for (int m = 8; m >= 1; m >>= 1) ss += __shfl_xor(ss, m, kWave);
+            float rms = sqrtf(ss / (float)K + ep.eps);
+            if (!isfinite(rms) || rms < 1e-20f) rms = 1.0f;
+            inv = 1.0f / rms;
+        }
+    };
     // Epilogue operands that do not depend on the product -- the conv window / taps / bias (mode 1), the
     // residual element and next norm weight (mode 2) -- can be requested before the operands stream.
     const int e_row = m0 + (tid >> 4), e_col = n0 + (tid & 15);
     const bool e_valid = tid < 256 && e_row < M && e_col < N;
-    float win[kMaxConvTaps], cwv[kMaxConvTaps], cbias = 0.0f, res_old = 0.0f, nw = 0.0f;
+    constexpr bool kConv = EPI == 1 || EPI == 3;
+    constexpr int kTaps = EPI == 3 ? kMaxConvTaps : 4;
+    float win[kTaps], cwv[kTaps], cbias = 0.0f, res_old = 0.0f, nw = 0.0f;
     auto prefetch_epilogue = [&]() {
-        if (EPI == 1 && e_valid && e_col < ep.di) {
+        if (kConv && e_valid && e_col < ep.di) {
             const float *st = ep.conv_state + ((int64_t)e_row * ep.di + e_col) * ep.dc;
             const float *cw = ep.conv_w + (int64_t)e_col * ep.dc;
-            if (ep.dc == 4) {   // the usual case: window and taps are one aligned 16-byte vector each
+            if constexpr (EPI == 1) {   // four taps: window and taps are one aligned 16-byte vector each
                 const float4 s4 = *reinterpret_cast<const float4 *>(st), c4 = *reinterpret_cast<const float4 *>(cw);
                 win[0] = s4.y; win[1] = s4.z; win[2] = s4.w;
                 cwv[0] = c4.x; cwv[1] = c4.y; cwv[2] = c4.z; cwv[3] = c4.w;
             } else {
 #pragma unroll
-                for (int k = 0; k < kMaxConvTaps; k++) {
+                for (int k = 0; k < kTaps; k++) {
                     win[k] = (k + 1 < ep.dc) ? st[k + 1] : 0.0f;
                     cwv[k] = (k < ep.dc) ? cw[k] : 0.0f;
                 }
@@ -135,11 +141,11 @@ __global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu
             if (ep.next_norm_w) nw = ep.next_norm_w[e_col];
         }
     };
-    // Early for the residual epilogue and for a single row tile; with several row tiles the conv windows are a
-    // megabyte-scale read that would queue ahead of the operands, so there they are fetched after the product.
-    const bool early = EPI == 2 || (EPI == 1 && gridDim.y == 1);
-    if (early) prefetch_epilogue();
+    // Requested up front, but on the matrix-core route behind the first round of operand loads: with several row
+    // tiles the conv windows are a megabyte-scale read that would otherwise queue ahead of the operands.
     if constexpr (LPR != 0) {
+        row_scale();
+        prefetch_epilogue();
         constexpr int NC = LPR == 64 ? 2 : 1;           // columns a lane works on (with 32 lanes per row each half-wave has its own)
         constexpr int JB = LPR == 64 ? 2 : 4;             // pieces per column requested together
         const int ll = l & (LPR - 1), half = LPR == 64 ? 0 : (l >> 5);
@@ -228,19 +234,23 @@ __global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu
             }
         lds_barrier();
     } else {
-    for (int base = w; base < nk; base += kGemmWaves * kStepsPerBatch) {
-        uint4 bf[kStepsPerBatch], af[kStepsPerBatch];
+    uint4 bf[kStepsPerBatch], af[kStepsPerBatch];
+    auto request = [&](int base) {
 #pragma unroll
         for (int s = 0; s < kStepsPerBatch; s++) {
             const int ks = base + s * kGemmWaves;
-            if (ks < nk) {
-                bf[s] = *reinterpret_cast<const uint4 *>(wrow + 32 * ks);
-                af[s] = *reinterpret_cast<const uint4 *>(arow + 32 * ks);
-            }
+            // steps past K multiply zeros (every fragment is defined on every path)
+            bf[s] = ks < nk ? *reinterpret_cast<const uint4 *>(wrow + 32 * ks) : make_uint4(0, 0, 0, 0);
+            af[s] = ks < nk ? *reinterpret_cast<const uint4 *>(arow + 32 * ks) : make_uint4(0, 0, 0, 0);
         }
+    };
+    request(w);
+    row_scale();
+    prefetch_epilogue();
+    for (int base = w; base < nk; base += kGemmWaves * kStepsPerBatch) {
+        if (base != w) request(base);
 #pragma unroll
-        for (int s = 0; s < kStepsPerBatch; s++)
-            if (base + s * kGemmWaves < nk) acc = Mma32<T>::mma(af[s], bf[s], acc);
+        for (int s = 0; s < kStepsPerBatch; s++) acc = Mma32<T>::mma(af[s], bf[s], acc);
     }
     // K-split reduction: upper half of the waves parks its tile in LDS, lower half adds and parks the sums
     if (w >= kGemmWaves / 2) red[w - kGemmWaves / 2][l] = acc;
@@ -251,7 +261,6 @@ __global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu
     // element e of the 16x16 tile: row ml = e / 16, column nl = e % 16 lives in lane 16 (ml / 4) + nl, register ml % 4
     float u_out = 0.0f;   // mode 1: this thread's u as stored (0 for gate columns / rows past M)
     if (tid < 256) {
-        if (EPI != 0 && !early) prefetch_epilogue();
         const int ml = tid >> 4, nl = tid & 15;
         const int lane = (ml >> 2) * 16 + nl, i = ml & 3;
         float s = 0.0f;
@@ -279,18 +288,18 @@ __global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu
             for (int m = 8; m >= 1; m >>= 1) sq += __shfl_xor(sq, m, kWave);
             if (nl == 0 && row < M) ep.partials[(int64_t)row * ep.n_partials + blockIdx.x] = sq;
         } else if (!valid) {
-        } else if (EPI == 1 && col < ep.di) {
+        } else if (kConv && col < ep.di) {
             // conv step on the value as in_proj would have stored it (rounded to the storage type)
             const T xr = (T)s;
             const float xnew = Store<T>::ld(&xr);
             float *st = ep.conv_state + ((int64_t)row * ep.di + col) * ep.dc;
             float o = cbias;
-            if (ep.dc == 4) {
+            if constexpr (EPI == 1) {
                 o = fmaf(win[0], cwv[0], o); o = fmaf(win[1], cwv[1], o); o = fmaf(win[2], cwv[2], o); o = fmaf(xnew, cwv[3], o);
                 *reinterpret_cast<float4 *>(st) = make_float4(win[0], win[1], win[2], xnew);
             } else {
 #pragma unroll
-                for (int k = 0; k < kMaxConvTaps; k++)
+                for (int k = 0; k < kTaps; k++)
                     if (k < ep.dc) {
                         const float wk = (k + 1 < ep.dc) ? win[k] : xnew;
                         o = fmaf(wk, cwv[k], o);
@@ -304,7 +313,7 @@ __global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu
             store_out<TO>(C + (int64_t)row * ldc + col, s);
         }
     }
-    if constexpr (EPI == 1) {
+    if constexpr (kConv) {
         if (ep.xw != nullptr && n0 < ep.di) {   // the same for the whole workgroup
             __shared__ float ush[4][16];
             if (tid < 64) ush[tid >> 4][tid & 15] = u_out;
@@ -454,7 +463,8 @@ static int launch_skinny_t(hipStream_t st, TO *C, int64_t ldc, const T *A, int64
     const bool pro = ep.row_scale != 0;
     if (ep.mode != 0 && sizeof(TO) != sizeof(T)) return fail(MRS_E_DTYPE, "skinny gemm: fused epilogues store the activation type");
     if constexpr (sizeof(TO) == sizeof(T)) {
-        if (ep.mode == 1) { if (pro) MRS_SG(1, 1); else MRS_SG(1, 0); return check_launch("skinny_gemm_kernel"); }
+        if (ep.mode == 1 && ep.dc == 4) { if (pro) MRS_SG(1, 1); else MRS_SG(1, 0); return check_launch("skinny_gemm_kernel"); }
+        if (ep.mode == 1) { if (pro) MRS_SG(3, 1); else MRS_SG(3, 0); return check_launch("skinny_gemm_kernel"); }
         if (ep.mode == 2) { if (pro) MRS_SG(2, 1); else MRS_SG(2, 0); return check_launch("skinny_gemm_kernel"); }
     }
     if (pro) MRS_SG(0, 1); else MRS_SG(0, 0);
