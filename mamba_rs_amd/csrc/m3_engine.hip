@@ -760,9 +760,15 @@ int prefill_body3(mrs_m3_backbone *bb, int T) {
                                          rocblas_gemm_algo_standard, 0, 0));
                 bulk = bb->pf_proj; ldb = ip; scp = bb->pf_proj + nb; lds_ = ip;
             } else {
-                MRS_BLAS(rocblas_gemm_ex(bb->blas, rocblas_operation_none, rocblas_operation_none, nb, (int)rows, dm, &one, lw.in_proj, t, ip,
-                                         bb->pf_normed, t, dm, &zero, bb->pf_bulk, t, nb, bb->pf_bulk, t, nb, rocblas_datatype_f32_r,
-                                         rocblas_gemm_algo_standard, 0, 0));
+                if (lw.in_proj_t) {   // the vendor kernels for the transposed operand are faster at these shapes (its first nb rows)
+                    MRS_BLAS(rocblas_gemm_ex(bb->blas, rocblas_operation_transpose, rocblas_operation_none, nb, (int)rows, dm, &one, lw.in_proj_t,
+                                             t, dm, bb->pf_normed, t, dm, &zero, bb->pf_bulk, t, nb, bb->pf_bulk, t, nb, rocblas_datatype_f32_r,
+                                             rocblas_gemm_algo_standard, 0, 0));
+                } else {
+                    MRS_BLAS(rocblas_gemm_ex(bb->blas, rocblas_operation_none, rocblas_operation_none, nb, (int)rows, dm, &one, lw.in_proj, t, ip,
+                                             bb->pf_normed, t, dm, &zero, bb->pf_bulk, t, nb, bb->pf_bulk, t, nb, rocblas_datatype_f32_r,
+                                             rocblas_gemm_algo_standard, 0, 0));
+                }
                 MRS_BLAS(rocblas_gemm_ex(bb->blas, rocblas_operation_none, rocblas_operation_none, ns, (int)rows, dm, &one,
                                          (const char *)lw.in_proj + (size_t)nb * es, t, ip, bb->pf_normed, t, dm, &zero, bb->pf_proj,
                                          rocblas_datatype_f32_r, ns, bb->pf_proj, rocblas_datatype_f32_r, ns, rocblas_datatype_f32_r,
