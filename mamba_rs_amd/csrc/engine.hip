@@ -215,7 +215,24 @@ struct LayerDev {
     int s4d;
 };
 
-constexpr int kFoldXprojFloats = 32768;   // largest [d_inner/16][rows][xdbl] block of shares the folded x_proj may use
+constexpr int64_t kFoldXprojFloats = 1 << 20;   // largest [d_inner/16][rows][xdbl] block of shares the folded x_proj may use
+// Rows up to which x_proj rides in the in_proj launch (MRS_DECODE_FOLD_ROWS overrides).  Every step workgroup of a batch
+// row re-reads that row's d_inner / 16 shares, so the sum grows with the batch while the launch it saves does not:
+// measured at the 130m shape, the step went 420 -> 369 us at 8 rows, 467 -> 414 us at 16, even at 32, 622 -> 658 us at 64
+// (1024-thread step workgroups, a quarter of the re-reads, were slower still: 701 us).
+static int fold_rows_max() {
+    static const int v = [] {
+        if (getenv("MRS_DECODE_NO_FOLDED_XPROJ")) return 0;
+        const char *e = getenv("MRS_DECODE_FOLD_ROWS");
+        return e ? atoi(e) : 16;
+    }();
+    return v;
+}
+// ... and only while a row's shares stay small (30 KB at d_inner 1536); wider models keep the four-row limit
+static int fold_rows_for(int di, int xd) {
+    const bool small = (int64_t)(di / 16) * xd * (int64_t)sizeof(float) <= 32768;
+    return small ? fold_rows_max() : std::min(4, fold_rows_max());
+}
 
 struct Scratch {  // activations for M rows
     int64_t rows = 0;
@@ -285,11 +302,9 @@ static int alloc_scratch(mrs_backbone *bb, Scratch *s, int64_t rows, int T) {
     MRS_TRY(dev_alloc(bb, &s->y, rows * di * es));
     MRS_TRY(dev_alloc(bb, &s->out, rows * dm * es));
     if (T == 1) MRS_TRY(dev_alloc(bb, (void **)&s->partials, rows * (size_t)((dm + 15) / 16) * sizeof(float)));
-    if (T == 1 && bb->skinny && rows <= 4) {
-        static const bool no_fold = getenv("MRS_DECODE_NO_FOLDED_XPROJ") != nullptr;
-        if (!no_fold) {
-            MRS_TRY(dev_alloc(bb, (void **)&s->xpart, (size_t)kFoldXprojFloats * sizeof(float)));
-        }
+    if (T == 1 && bb->skinny && rows <= fold_rows_for(di, xd)) {
+        const int64_t need = (int64_t)(di / 16) * rows * bb->xd;
+        if (need <= kFoldXprojFloats) MRS_TRY(dev_alloc(bb, (void **)&s->xpart, (size_t)need * sizeof(float)));
     }
     if (T > 1) {
         s->scan_ws_bytes = mrs_ssm_scan_workspace_bytes(bb->batch, T, di, bb->cfg.d_state);
@@ -373,8 +388,8 @@ static int run_layers(mrs_backbone *bb, Scratch *s, int T) {
             SkinnyEpi inp = {};
             inp.mode = 1; inp.conv_state = conv; inp.conv_w = lw.conv_w; inp.conv_b = lw.conv_b; inp.u = s->u; inp.di = di; inp.dc = dc;
             inp.row_scale = 1; inp.partials = s->partials; inp.n_partials = P; inp.eps = bb->cfg.rms_norm_eps;
-            // a few rows: x_proj rides in the same launch (its 16-column shares are summed by the last workgroup to finish)
-            const bool fold_x = s->xpart && B <= 4 && xd <= 256 && (int64_t)(di / 16) * B * xd <= kFoldXprojFloats && lw.dt_t_step &&
+            // up to 16 rows: x_proj rides in the same launch (its 16-column shares are summed by the step kernel)
+            const bool fold_x = s->xpart && B <= fold_rows_for(di, xd) && xd <= 256 && (int64_t)(di / 16) * B * xd <= kFoldXprojFloats && lw.dt_t_step &&
                                 di % (1024 / ds) == 0 && dr % 4 == 0 && (int64_t)B * dr <= kFuseDtProjLimit;
             if (fold_x) { inp.xw = lw.x_proj; inp.xd = xd; inp.xpart = s->xpart; }
             const StepFold fold = {s->xpart, di / 16, B, xd, dr, dr + ds};

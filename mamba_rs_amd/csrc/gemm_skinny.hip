@@ -315,17 +315,19 @@ __global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu
     }
     if constexpr (kConv) {
         if (ep.xw != nullptr && n0 < ep.di) {   // the same for the whole workgroup
-            __shared__ float ush[4][16];
-            if (tid < 64) ush[tid >> 4][tid & 15] = u_out;
+            // this tile's share of the x_proj rows: u[row, 16 columns] . W[16 columns, xd], f32, into [tile][row][xd]
+            __shared__ float ush[16][16];
+            if (tid < 256) ush[tid >> 4][tid & 15] = u_out;
             lds_barrier();
-            const int xd = ep.xd, P = M * xd;   // P <= 512 (checked by the launcher)
+            const int xd = ep.xd, rows_here = min(16, M - m0);
             const T *xw = reinterpret_cast<const T *>(ep.xw);
-            if (tid < P) {
-                const int m = tid / xd, j = tid - m * xd;
+            float *dst = ep.xpart + ((int64_t)blockIdx.x * M + m0) * xd;
+            for (int o = tid; o < rows_here * xd; o += kGemmWaves * 64) {
+                const int m = o / xd, j = o - m * xd;
                 float a = 0.0f;
 #pragma unroll
                 for (int c = 0; c < 16; c++) a = fmaf(ush[m][c], Store<T>::ld(xw + (int64_t)min(n0 + c, ep.di - 1) * xd + j), a);
-                ep.xpart[(int64_t)blockIdx.x * P + tid] = a;
+                dst[o] = a;
             }
         }
     }
@@ -484,7 +486,7 @@ int launch_skinny_gemm(hipStream_t st, int dtype, void *C, int out_f32, int64_t 
                                  "(got dtype=%d M=%d N=%d K=%d lda=%lld)", dtype, M, N, K, (long long)lda);
     if (ep.mode == 1 && (ep.dc < 1 || ep.dc > kMaxConvTaps || ep.di < 1 || ep.di > N || !ep.conv_state || !ep.conv_w || !ep.conv_b || !ep.u))
         return fail(MRS_E_SHAPE, "skinny gemm: bad in_proj epilogue (di=%d dc=%d)", ep.di, ep.dc);
-    if (ep.mode == 1 && ep.xw && (M > 4 || ep.xd < 1 || M * ep.xd > kGemmWaves * 64 || ep.di % 16 != 0 || !ep.xpart))
+    if (ep.mode == 1 && ep.xw && (ep.xd < 1 || ep.di % 16 != 0 || !ep.xpart))
         return fail(MRS_E_SHAPE, "skinny gemm: bad folded x_proj (M=%d xd=%d di=%d)", M, ep.xd, ep.di);
     if (ep.mode == 2 && (!ep.residual || !ep.partials || ep.n_partials != (N + 15) / 16 || (ep.next_norm_w && !ep.prenorm)))
         return fail(MRS_E_SHAPE, "skinny gemm: bad out_proj epilogue (n_partials=%d, column tiles=%d)", ep.n_partials, (N + 15) / 16);

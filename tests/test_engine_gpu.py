@@ -258,20 +258,20 @@ def test_wide_dt_rank_at_large_batch_runs_dt_proj_as_its_own_gemm():
         eng.close()
 
 
-@pytest.mark.parametrize("dm,batch", [(256, 1), (256, 3), (512, 4), (768, 2)])
+@pytest.mark.parametrize("dm,batch", [(256, 1), (256, 3), (512, 4), (768, 2), (768, 7), (256, 16), (512, 13)])
 def test_few_row_decode_chain_with_folded_x_proj_equals_the_many_row_chain(dm, batch):
-    """At one to four rows x_proj rides in the in_proj launch (per-tile shares summed by the last workgroup to finish) and
-    the projections take the lanes-along-the-row route; an engine of 8 rows runs x_proj as its own launch on the matrix
-    cores.  Same weights, same inputs: the rows must agree to 16-bit rounding, step after step, eager and replayed."""
+    """Up to 16 rows x_proj rides in the in_proj launch (per-tile shares, summed by the step kernel), and at one to four
+    rows the projections take the lanes-along-the-row route; an engine of 24 rows runs x_proj as its own launch on the
+    matrix cores.  Same weights, same inputs: the rows must agree to 16-bit rounding, step after step, eager and replayed."""
     cfg = MambaConfig(d_model=dm, d_state=16, d_conv=4, expand=2, n_layers=3)
     w = MambaWeights.random_lm(cfg, seed=dm + batch, std=0.05)
     few = GpuMambaBackbone.new_with_dtype(0, w, cfg, dm, batch, WeightDtype.BF16)
-    many = GpuMambaBackbone.new_with_dtype(0, w, cfg, dm, 8, WeightDtype.BF16)
+    many = GpuMambaBackbone.new_with_dtype(0, w, cfg, dm, 24, WeightDtype.BF16)
     rng = np.random.default_rng(dm)
     for t in range(24):
         if t == 8:
             few.capture_graph()
-        x = rng.standard_normal((8, dm)).astype(np.float32)
+        x = rng.standard_normal((24, dm)).astype(np.float32)
         a, b = few.step(x[:batch]), many.step(x)[:batch]
         assert np.isfinite(a).all()
         assert cosine(a, b) >= 0.9995 and scaled_err(a, b) < 3e-2, (t, cosine(a, b), scaled_err(a, b))
