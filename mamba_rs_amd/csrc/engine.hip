@@ -361,57 +361,77 @@ static int project_input(mrs_backbone *bb, float *residual, const float *input_d
 
 // The layer stack over `rows` = batch*T rows (T = 1: decode chain, T > 1: prefill chain), leaving the
 // final-norm output of every row (decode) or of the last step of each sequence (prefill) in temporal [batch, dm] f32.
+// Decode chain on the library's own GEMM for rows [r0, r0 + nr) of the batch, every layer, on stream st.  Three or
+// four kernels per layer:
+//   in_proj  on round(residual * norm_w) with the 1/rms row scale and the conv step + SiLU in its epilogue (only u and
+//            the gate half are written); up to 16 rows its x-half workgroups also leave their shares of the x_proj rows,
+//   x_proj   (above that row count),
+//   dt_proj + softplus + scan step + gate (summing the x_proj shares first where they were left),
+//   out_proj with the residual add as its epilogue, which also leaves each row's sum of squares (per 16-column tile)
+//            and round(residual * next norm_w) for the next layer's in_proj.
+// Rows are independent of each other from the first kernel to the last.  (Running the batch as two or four such chains
+// of 16-32 rows on forked streams inside the graph was measured: the branches did not overlap -- 631 us for one chain of 64
+// rows at the 130m shape, 722 us as two chains, 1112 us as four.)
+static int decode_chain(mrs_backbone *bb, Scratch *s, int r0, int nr, hipStream_t st) {
+    const int dm = bb->cfg.d_model, di = bb->di, ds = bb->cfg.d_state, dc = bb->cfg.d_conv, dr = bb->dr, xd = bb->xd;
+    const int B = bb->batch, dt = bb->dtype, L = bb->cfg.n_layers, P = dm / 16;
+    const size_t es = esize(dt);
+    float *residual = s->residual + (size_t)r0 * dm, *partials = s->partials + (size_t)r0 * P;
+    char *normed = (char *)s->normed + (size_t)r0 * dm * es, *proj = (char *)s->proj + (size_t)r0 * 2 * di * es;
+    char *u = (char *)s->u + (size_t)r0 * di * es, *xdbl = (char *)s->xdbl + (size_t)r0 * xd * es;
+    char *delta = (char *)s->delta + (size_t)r0 * di * es, *y = (char *)s->y + (size_t)r0 * di * es;
+    char *out = (char *)s->out + (size_t)r0 * dm * es;
+    float *xpart = s->xpart ? s->xpart + (size_t)r0 * (di / 16) * xd : nullptr;   // [tile][nr][xd] blocks, one per slice
+    const char *z = proj + (size_t)di * es;  // gate half of in_proj's output
+    for (int l = 0; l < L; l++) {
+        const LayerDev &lw = bb->layers[l];
+        float *conv = bb->conv_state + ((size_t)l * B + r0) * di * dc;
+        float *ssm = bb->ssm_state + ((size_t)l * B + r0) * di * ds;
+        if (l == 0) {
+            const float *src = bb->step_src ? bb->step_src + (size_t)r0 * dm : residual;
+            MRS_TRY(launch_prenorm_rows(st, dt, partials, P, normed, src, bb->step_src ? residual : nullptr, lw.norm_w, nr, dm));
+        }
+        SkinnyEpi inp = {};
+        inp.mode = 1; inp.conv_state = conv; inp.conv_w = lw.conv_w; inp.conv_b = lw.conv_b; inp.u = u; inp.di = di; inp.dc = dc;
+        inp.row_scale = 1; inp.partials = partials; inp.n_partials = P; inp.eps = bb->cfg.rms_norm_eps;
+        const bool fold_x = xpart && nr <= fold_rows_for(di, xd) && xd <= 256 && (int64_t)(di / 16) * nr * xd <= kFoldXprojFloats && lw.dt_t_step &&
+                            di % (1024 / ds) == 0 && dr % 4 == 0 && (int64_t)nr * dr <= kFuseDtProjLimit;
+        if (fold_x) { inp.xw = lw.x_proj; inp.xd = xd; inp.xpart = xpart; }
+        const StepFold fold = {xpart, di / 16, nr, xd, dr, dr + ds};
+        MRS_TRY(launch_skinny_gemm(st, dt, proj, 0, 2 * di, normed, dm, lw.in_proj_t, nr, 2 * di, dm, inp));
+        const SkinnyEpi none = {};
+        if (!fold_x) MRS_TRY(launch_skinny_gemm(st, dt, xdbl, 0, xd, u, di, lw.x_proj_t, nr, xd, di, none));
+        if ((int64_t)nr * dr > kFuseDtProjLimit && lw.dt_w_t && skinny_gemm_ok(dt, nr, di, dr, xd, xdbl, lw.dt_w_t)) {
+            // wide dt_rank at a large batch: dt_proj as a GEMM of its own, bias + softplus in the step kernel
+            MRS_TRY(launch_skinny_gemm(st, dt, delta, 0, di, xdbl, xd, lw.dt_w_t, nr, di, dr, none));
+            MRS_TRY(launch_ssm_step_fused(st, dt, ssm, y, delta, lw.dt_b, nullptr, nullptr, 0, 0, u, xdbl + es * dr, xdbl + es * (dr + ds), xd, z,
+                                          2 * di, 2, lw.a_neg, lw.D, nr, di, ds));
+        } else {
+            MRS_TRY(launch_ssm_step_fused(st, dt, ssm, y, delta, lw.dt_b, xdbl, lw.dt_t_step ? lw.dt_w_t : lw.dt_w, dr, lw.dt_t_step, u,
+                                          xdbl + es * dr, xdbl + es * (dr + ds), xd, z, 2 * di, 2, lw.a_neg, lw.D, nr, di, ds,
+                                          fold_x ? &fold : nullptr));
+        }
+        SkinnyEpi outp = {};
+        outp.mode = 2; outp.residual = residual; outp.partials = partials; outp.n_partials = P;
+        outp.next_norm_w = l + 1 < L ? bb->layers[l + 1].norm_w : nullptr; outp.prenorm = normed;
+        MRS_TRY(launch_skinny_gemm(st, dt, out, 0, dm, y, di, lw.out_proj_t, nr, dm, di, outp));
+    }
+    return MRS_OK;
+}
+
 static int run_layers(mrs_backbone *bb, Scratch *s, int T) {
     const int dm = bb->cfg.d_model, di = bb->di, ds = bb->cfg.d_state, dc = bb->cfg.d_conv, dr = bb->dr, xd = bb->xd;
     const int B = bb->batch, dt = bb->dtype;
     const int64_t rows = (int64_t)B * T;
     const size_t es = esize(dt);
     const int L = bb->cfg.n_layers;
-    for (int l = 0; l < L; l++) {
+    if (T == 1 && bb->skinny) MRS_TRY(decode_chain(bb, s, 0, B, bb->stream));
+    for (int l = 0; l < L && !(T == 1 && bb->skinny); l++) {
         const LayerDev &lw = bb->layers[l];
         float *conv = bb->conv_state + (size_t)l * B * di * dc;
         float *ssm = bb->ssm_state + (size_t)l * B * di * ds;
         const char *z = (const char *)s->proj + (size_t)di * es;  // gate half of in_proj's output
         const char *xb = (const char *)s->xdbl;
-        if (T == 1 && bb->skinny) {
-            // Decode chain on the library's own GEMM, four kernels per layer:
-            //   in_proj  on round(residual * norm_w) with the 1/rms row scale and the conv step + SiLU in its
-            //            epilogue (only u and the gate half are written),
-            //   x_proj,
-            //   dt_proj + softplus + scan step + gate,
-            //   out_proj with the residual add as its epilogue, which also leaves each row's sum of squares
-            //            (per 16-column tile) and round(residual * next norm_w) for the next layer's in_proj.
-            const int P = dm / 16;
-            if (l == 0)
-                MRS_TRY(launch_prenorm_rows(bb->stream, dt, s->partials, P, s->normed, bb->step_src ? bb->step_src : s->residual,
-                                            bb->step_src ? s->residual : nullptr, lw.norm_w, B, dm));
-            SkinnyEpi inp = {};
-            inp.mode = 1; inp.conv_state = conv; inp.conv_w = lw.conv_w; inp.conv_b = lw.conv_b; inp.u = s->u; inp.di = di; inp.dc = dc;
-            inp.row_scale = 1; inp.partials = s->partials; inp.n_partials = P; inp.eps = bb->cfg.rms_norm_eps;
-            // up to 16 rows: x_proj rides in the same launch (its 16-column shares are summed by the step kernel)
-            const bool fold_x = s->xpart && B <= fold_rows_for(di, xd) && xd <= 256 && (int64_t)(di / 16) * B * xd <= kFoldXprojFloats && lw.dt_t_step &&
-                                di % (1024 / ds) == 0 && dr % 4 == 0 && (int64_t)B * dr <= kFuseDtProjLimit;
-            if (fold_x) { inp.xw = lw.x_proj; inp.xd = xd; inp.xpart = s->xpart; }
-            const StepFold fold = {s->xpart, di / 16, B, xd, dr, dr + ds};
-            MRS_TRY(launch_skinny_gemm(bb->stream, dt, s->proj, 0, 2 * di, s->normed, dm, lw.in_proj_t, B, 2 * di, dm, inp));
-            const SkinnyEpi none = {};
-            if (!fold_x) MRS_TRY(launch_skinny_gemm(bb->stream, dt, s->xdbl, 0, xd, s->u, di, lw.x_proj_t, B, xd, di, none));
-            if ((int64_t)B * dr > kFuseDtProjLimit && lw.dt_w_t && skinny_gemm_ok(dt, B, di, dr, xd, s->xdbl, lw.dt_w_t)) {
-                // wide dt_rank at a large batch: dt_proj as a GEMM of its own, bias + softplus in the step kernel
-                MRS_TRY(launch_skinny_gemm(bb->stream, dt, s->delta, 0, di, s->xdbl, xd, lw.dt_w_t, B, di, dr, none));
-                MRS_TRY(launch_ssm_step_fused(bb->stream, dt, ssm, s->y, s->delta, lw.dt_b, nullptr, nullptr, 0, 0, s->u, xb + es * dr,
-                                              xb + es * (dr + ds), xd, z, 2 * di, 2, lw.a_neg, lw.D, B, di, ds));
-            } else {
-                MRS_TRY(launch_ssm_step_fused(bb->stream, dt, ssm, s->y, s->delta, lw.dt_b, s->xdbl, lw.dt_t_step ? lw.dt_w_t : lw.dt_w, dr,
-                                              lw.dt_t_step, s->u, xb + es * dr,
-                                              xb + es * (dr + ds), xd, z, 2 * di, 2, lw.a_neg, lw.D, B, di, ds, fold_x ? &fold : nullptr));
-            }
-            SkinnyEpi outp = {};
-            outp.mode = 2; outp.residual = s->residual; outp.partials = s->partials; outp.n_partials = P;
-            outp.next_norm_w = l + 1 < L ? bb->layers[l + 1].norm_w : nullptr; outp.prenorm = s->normed;
-            MRS_TRY(launch_skinny_gemm(bb->stream, dt, s->out, 0, dm, s->y, di, lw.out_proj_t, B, dm, di, outp));
-            continue;
-        }
         MRS_TRY(launch_add_rmsnorm(bb, s->residual, l == 0 ? nullptr : s->out, s->normed, false, lw.norm_w, rows, dm));
         if (T > 1 && lw.in_proj_t) MRS_TRY(gemm_rm_t(bb, dt, s->proj, 2 * di, s->normed, dm, lw.in_proj_t, (int)rows, 2 * di, dm));
         else MRS_TRY(gemm_rm(bb, dt, s->proj, 2 * di, s->normed, dm, lw.in_proj, (int)rows, 2 * di, dm));
