@@ -112,6 +112,11 @@ struct SkinnyEpi {
     const void *xw;      // [di][xd] activation type (row-major, not transposed), or null
     int xd;
     float *xpart;        // [di / 16][M][xd] f32
+    // mode 0, optional: K split over ksplit workgroups per tile (grid z), each leaving its f32 share in
+    // xpart[slice][M][N] -- the layout above, so the same reader sums them (a long K with few output tiles:
+    // x_proj of a wide model is 12 tiles over K = 5120)
+    int ksplit;
+    int kslice;          // set by the launcher: 32-wide k-steps per slice
 };
 bool skinny_gemm_ok(int dtype, int M, int N, int K, int64_t lda, const void *A, const void *Wt);
 int launch_skinny_gemm(hipStream_t st, int dtype, void *C, int out_f32, int64_t ldc, const void *A, int64_t lda, const void *Wt,

@@ -216,6 +216,18 @@ struct LayerDev {
 };
 
 constexpr int64_t kFoldXprojFloats = 1 << 20;   // largest [d_inner/16][rows][xdbl] block of shares the folded x_proj may use
+constexpr int kMaxXprojSlices = 16;
+// K slices of an x_proj launch of its own (0 = never split; MRS_DECODE_XPROJ_KSPLIT forces a count).  x_proj has few
+// output tiles and a long K -- 12 workgroups over K = 5120 at 16 rows of the 2.8b shape -- so its K is cut into slices
+// whose shares the step kernel sums, exactly as it sums the shares the in_proj launch leaves at few rows.
+static int xproj_slices(int rows, int xd, int di) {
+    static const int forced = getenv("MRS_DECODE_XPROJ_KSPLIT") ? atoi(getenv("MRS_DECODE_XPROJ_KSPLIT")) : -1;
+    const int tiles = ((xd + 15) / 16) * ((rows + 15) / 16), nk = di / 32;
+    int ks = forced >= 0 ? forced : 256 / tiles;
+    ks = std::min(std::min(ks, kMaxXprojSlices), nk / 8);   // at least one k-step per wave
+    return ks >= 2 ? ks : 1;
+}
+
 // Rows up to which x_proj rides in the in_proj launch (MRS_DECODE_FOLD_ROWS overrides).  Every step workgroup of a batch
 // row re-reads that row's d_inner / 16 shares, so the sum grows with the batch while the launch it saves does not:
 // measured at the 130m shape, the step went 420 -> 369 us at 8 rows, 467 -> 414 us at 16, even at 32, 622 -> 658 us at 64
@@ -239,7 +251,8 @@ struct Scratch {  // activations for M rows
     void *normed = nullptr, *proj = nullptr, *u = nullptr, *xdbl = nullptr, *delta = nullptr, *y = nullptr, *out = nullptr;
     float *residual = nullptr;
     float *partials = nullptr;  // [rows][d_model/16] row sums of squares, decode chain only
-    float *xpart = nullptr;     // decode chain, a few rows: per-tile shares of the folded x_proj
+    float *xpart = nullptr;     // decode chain: shares of the x_proj rows (per in_proj tile, or per K slice of x_proj)
+    int64_t xpart_floats = 0;
     void *scan_ws = nullptr;
     size_t scan_ws_bytes = 0;
     int T = 0;
@@ -302,9 +315,12 @@ static int alloc_scratch(mrs_backbone *bb, Scratch *s, int64_t rows, int T) {
     MRS_TRY(dev_alloc(bb, &s->y, rows * di * es));
     MRS_TRY(dev_alloc(bb, &s->out, rows * dm * es));
     if (T == 1) MRS_TRY(dev_alloc(bb, (void **)&s->partials, rows * (size_t)((dm + 15) / 16) * sizeof(float)));
-    if (T == 1 && bb->skinny && rows <= fold_rows_for(di, xd)) {
-        const int64_t need = (int64_t)(di / 16) * rows * bb->xd;
-        if (need <= kFoldXprojFloats) MRS_TRY(dev_alloc(bb, (void **)&s->xpart, (size_t)need * sizeof(float)));
+    if (T == 1 && bb->skinny) {
+        // shares of the x_proj rows: per 16-column tile of in_proj (few rows), else per K slice of a split x_proj
+        int64_t need = (int64_t)kMaxXprojSlices * rows * xd;
+        if (rows <= fold_rows_for(di, xd) && (int64_t)(di / 16) * rows * xd <= kFoldXprojFloats) need = std::max(need, (int64_t)(di / 16) * rows * xd);
+        s->xpart_floats = need;
+        MRS_TRY(dev_alloc(bb, (void **)&s->xpart, (size_t)need * sizeof(float)));
     }
     if (T > 1) {
         s->scan_ws_bytes = mrs_ssm_scan_workspace_bytes(bb->batch, T, di, bb->cfg.d_state);
@@ -394,13 +410,20 @@ static int decode_chain(mrs_backbone *bb, Scratch *s, int r0, int nr, hipStream_
         SkinnyEpi inp = {};
         inp.mode = 1; inp.conv_state = conv; inp.conv_w = lw.conv_w; inp.conv_b = lw.conv_b; inp.u = u; inp.di = di; inp.dc = dc;
         inp.row_scale = 1; inp.partials = partials; inp.n_partials = P; inp.eps = bb->cfg.rms_norm_eps;
-        const bool fold_x = xpart && nr <= fold_rows_for(di, xd) && xd <= 256 && (int64_t)(di / 16) * nr * xd <= kFoldXprojFloats && lw.dt_t_step &&
+        const bool fold_x = xpart && nr <= fold_rows_for(di, xd) && xd <= 256 && (int64_t)(di / 16) * nr * xd <= s->xpart_floats && lw.dt_t_step &&
                             di % (1024 / ds) == 0 && dr % 4 == 0 && (int64_t)nr * dr <= kFuseDtProjLimit;
         if (fold_x) { inp.xw = lw.x_proj; inp.xd = xd; inp.xpart = xpart; }
-        const StepFold fold = {xpart, di / 16, nr, xd, dr, dr + ds};
+        // x_proj as a launch of its own: K split into slices when the step kernel can sum the shares
+        const bool step_sums = xpart && xd <= 256 && lw.dt_t_step && di % (1024 / ds) == 0 && dr % 4 == 0 && (int64_t)nr * dr <= kFuseDtProjLimit;
+        const int ksplit = (!fold_x && step_sums) ? xproj_slices(nr, xd, di) : 1;
+        const StepFold fold = {xpart, fold_x ? di / 16 : ksplit, nr, xd, dr, dr + ds};
         MRS_TRY(launch_skinny_gemm(st, dt, proj, 0, 2 * di, normed, dm, lw.in_proj_t, nr, 2 * di, dm, inp));
         const SkinnyEpi none = {};
-        if (!fold_x) MRS_TRY(launch_skinny_gemm(st, dt, xdbl, 0, xd, u, di, lw.x_proj_t, nr, xd, di, none));
+        if (!fold_x) {
+            SkinnyEpi xp = {};
+            if (ksplit > 1) { xp.ksplit = ksplit; xp.xpart = xpart; }
+            MRS_TRY(launch_skinny_gemm(st, dt, xdbl, 0, xd, u, di, lw.x_proj_t, nr, xd, di, xp));
+        }
         if ((int64_t)nr * dr > kFuseDtProjLimit && lw.dt_w_t && skinny_gemm_ok(dt, nr, di, dr, xd, xdbl, lw.dt_w_t)) {
             // wide dt_rank at a large batch: dt_proj as a GEMM of its own, bias + softplus in the step kernel
             MRS_TRY(launch_skinny_gemm(st, dt, delta, 0, di, xdbl, xd, lw.dt_w_t, nr, di, dr, none));
@@ -409,7 +432,7 @@ static int decode_chain(mrs_backbone *bb, Scratch *s, int r0, int nr, hipStream_
         } else {
             MRS_TRY(launch_ssm_step_fused(st, dt, ssm, y, delta, lw.dt_b, xdbl, lw.dt_t_step ? lw.dt_w_t : lw.dt_w, dr, lw.dt_t_step, u,
                                           xdbl + es * dr, xdbl + es * (dr + ds), xd, z, 2 * di, 2, lw.a_neg, lw.D, nr, di, ds,
-                                          fold_x ? &fold : nullptr));
+                                          (fold_x || ksplit > 1) ? &fold : nullptr));
         }
         SkinnyEpi outp = {};
         outp.mode = 2; outp.residual = residual; outp.partials = partials; outp.n_partials = P;

@@ -92,7 +92,10 @@ __global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu
     __shared__ float gv[4][16];   // LPR != 0: the [row][column] sums of the workgroup
     const int n0 = blockIdx.x * 16, m0 = blockIdx.y * 16;
     const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, lr = l & 15, lg = l >> 4;
-    const int nk = K >> 5;
+    // k-steps of this workgroup: all of them, or slice blockIdx.z of gridDim.z (matrix-core route, plain store only)
+    const int nk_all = K >> 5;
+    const int k_lo = LPR == 0 ? (int)blockIdx.z * ep.kslice : 0;
+    const int nk = LPR == 0 ? min(nk_all, k_lo + ep.kslice) : nk_all;
     v4f acc = {0.f, 0.f, 0.f, 0.f};
     // Rows past M / columns past N are clamped to the last valid one: their products land in
     // accumulator elements that are never stored.
@@ -244,11 +247,11 @@ __global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu
             af[s] = ks < nk ? *reinterpret_cast<const uint4 *>(arow + 32 * ks) : make_uint4(0, 0, 0, 0);
         }
     };
-    request(w);
+    request(k_lo + w);
     row_scale();
     prefetch_epilogue();
-    for (int base = w; base < nk; base += kGemmWaves * kStepsPerBatch) {
-        if (base != w) request(base);
+    for (int base = k_lo + w; base < nk; base += kGemmWaves * kStepsPerBatch) {
+        if (base != k_lo + w) request(base);
 #pragma unroll
         for (int s = 0; s < kStepsPerBatch; s++) acc = Mma32<T>::mma(af[s], bf[s], acc);
     }
@@ -309,6 +312,8 @@ __global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu
             const T ur = (T)silu(o);
             reinterpret_cast<T *>(ep.u)[(int64_t)row * ep.di + col] = ur;
             u_out = Store<T>::ld(&ur);
+        } else if (EPI == 0 && LPR == 0 && gridDim.z > 1) {
+            ep.xpart[((int64_t)blockIdx.z * M + row) * N + col] = s;   // this slice's share, summed by the reader
         } else {
             store_out<TO>(C + (int64_t)row * ldc + col, s);
         }
@@ -447,11 +452,17 @@ __global__ __launch_bounds__(256) void transpose_kernel(T *__restrict__ Wt, cons
 
 template <typename T, typename TO>
 static int launch_skinny_t(hipStream_t st, TO *C, int64_t ldc, const T *A, int64_t lda, const T *Wt, int M, int N, int K,
-                           const SkinnyEpi &ep) {
-    const dim3 grid((unsigned)((N + 15) / 16), (unsigned)((M + 15) / 16)), block(kGemmWaves * 64);
+                           const SkinnyEpi &ep_in) {
+    SkinnyEpi ep = ep_in;
+    const dim3 block(kGemmWaves * 64);
     // one to four rows: the lanes-along-the-row route (64 lanes per weight row when a row is a multiple of 1 KB, else 32)
     static const bool no_rowwise = getenv("MRS_DECODE_NO_ROWWISE") != nullptr;
     const int lpr = (M > 4 || no_rowwise || (int64_t)K * 8 > 48 * 1024) ? 0 : (K % 512 == 0 ? 64 : (K % 256 == 0 ? 32 : 0));   // rows fit in LDS
+    const int ksplit = (ep.mode == 0 && ep.ksplit > 1) ? ep.ksplit : 1;
+    if (ksplit > 1 && (lpr != 0 || ep.row_scale || !ep.xpart || ksplit > (K >> 5)))
+        return fail(MRS_E_SHAPE, "skinny gemm: K split needs the matrix-core route, a plain product, a share buffer and ksplit <= K / 32 (ksplit=%d)", ksplit);
+    ep.kslice = ((K >> 5) + ksplit - 1) / ksplit;
+    const dim3 grid((unsigned)((N + 15) / 16), (unsigned)((M + 15) / 16), (unsigned)(((K >> 5) + ep.kslice - 1) / ep.kslice));
 #define MRS_SG(EPI_, PRO_)                                                                                                               \
     do {                                                                                                                                 \
         if (lpr == 64 && M == 1) hipLaunchKernelGGL((skinny_gemm_kernel<T, TO, EPI_, PRO_, 64, 1>), grid, block, 0, st, C, ldc, A, lda, Wt, M, N, K, ep); \
