@@ -237,23 +237,31 @@ __global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu
             }
         lds_barrier();
     } else {
-    uint4 bf[kStepsPerBatch], af[kStepsPerBatch];
-    auto request = [&](int base) {
+    // Two half-batches of fragments: the next one is requested as soon as the current one has been multiplied, so a
+    // long K (wide models: 20 k-steps per wave at K = 5120) streams instead of draining after every round of loads.
+    constexpr int kHalf = kStepsPerBatch / 2;
+    uint4 bf[2][kHalf], af[2][kHalf];
+    auto request = [&](int h, int base) {
 #pragma unroll
-        for (int s = 0; s < kStepsPerBatch; s++) {
+        for (int s = 0; s < kHalf; s++) {
             const int ks = base + s * kGemmWaves;
             // steps past K multiply zeros (every fragment is defined on every path)
-            bf[s] = ks < nk ? *reinterpret_cast<const uint4 *>(wrow + 32 * ks) : make_uint4(0, 0, 0, 0);
-            af[s] = ks < nk ? *reinterpret_cast<const uint4 *>(arow + 32 * ks) : make_uint4(0, 0, 0, 0);
+            bf[h][s] = ks < nk ? *reinterpret_cast<const uint4 *>(wrow + 32 * ks) : make_uint4(0, 0, 0, 0);
+            af[h][s] = ks < nk ? *reinterpret_cast<const uint4 *>(arow + 32 * ks) : make_uint4(0, 0, 0, 0);
         }
     };
-    request(k_lo + w);
+    constexpr int kStride = kGemmWaves * kHalf;   // k-steps one half-batch covers across the workgroup's waves
+    request(0, k_lo + w);
+    request(1, k_lo + w + kStride);
     row_scale();
     prefetch_epilogue();
-    for (int base = k_lo + w; base < nk; base += kGemmWaves * kStepsPerBatch) {
-        if (base != k_lo + w) request(base);
+    for (int base = k_lo + w; base < nk; base += 2 * kStride) {
 #pragma unroll
-        for (int s = 0; s < kStepsPerBatch; s++) acc = Mma32<T>::mma(af[s], bf[s], acc);
+        for (int s = 0; s < kHalf; s++) acc = Mma32<T>::mma(af[0][s], bf[0][s], acc);
+        request(0, base + 2 * kStride);   // past K: zeros, so a half-batch is never multiplied twice
+#pragma unroll
+        for (int s = 0; s < kHalf; s++) acc = Mma32<T>::mma(af[1][s], bf[1][s], acc);
+        request(1, base + 3 * kStride);
     }
     // K-split reduction: upper half of the waves parks its tile in LDS, lower half adds and parks the sums
     if (w >= kGemmWaves / 2) red[w - kGemmWaves / 2][l] = acc;
