@@ -329,6 +329,14 @@ typedef struct {
 MRS_API int mrs_lm_generate_batch(mrs_lm *lm, const int *prompts, const int *prompt_lens, const mrs_sample_params *params,
                                   int seen_includes_prompt, int *out_tokens, int out_stride, int *out_lens);
 
+/* GpuMambaLM::generate_streaming (src/module/gpu_lm.rs:334-377), batch-1 engines: the loop of mrs_lm_generate_batch with
+ * the penalty history over prompt + generated tokens and the prompt through the prefill path from 256 tokens on; every
+ * new token is handed to `cb` as soon as it exists (one host round trip per step).  A nonzero return from `cb` ends the
+ * generation early (the reference's callback cannot; returning 0 always reproduces it). */
+typedef int (*mrs_token_callback)(int token, void *user);
+MRS_API int mrs_lm_generate_streaming(mrs_lm *lm, const int *prompt, int prompt_len, const mrs_sample_params *params,
+                                      mrs_token_callback cb, void *user);
+
 /* ---- Mamba-3 SISO backbone engine (decode step) -------------------------------------------------
  * GpuMamba3Backbone (src/mamba3_siso/gpu/inference.rs:1487-1671): weights, per-layer state
  * (ssm [batch,nh,hd,ds], k [batch,nh,ds], v [batch,nh,hd], angle [batch,nh,n_rope], all f32) and scratch owned by

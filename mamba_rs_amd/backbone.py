@@ -16,6 +16,7 @@ from .config import MambaConfig, WeightDtype
 from .weights import MambaWeights
 
 _FP = POINTER(c_float)
+_TOKEN_CB = ctypes.CFUNCTYPE(c_int, c_int, c_void_p)
 
 
 class _CConfig(Structure):
@@ -70,6 +71,7 @@ def _bind():
         "mrs_lm_prefill": (c_int, [P, P, POINTER(c_int), c_int]),
         "mrs_lm_generate_batch": (c_int, [P, POINTER(c_int), POINTER(c_int), POINTER(_CSampleParams), c_int, POINTER(c_int), c_int,
                                           POINTER(c_int)]),
+        "mrs_lm_generate_streaming": (c_int, [P, POINTER(c_int), c_int, POINTER(_CSampleParams), _TOKEN_CB, c_void_p]),
     }
     for name, (res, args) in sigs.items():
         fn = getattr(lib, name)
@@ -306,6 +308,31 @@ class GpuMambaLM:
         _call("mrs_lm_generate_batch", self._h, flat.ctypes.data_as(POINTER(c_int)), lens.ctypes.data_as(POINTER(c_int)), cp,
               1 if seen_includes_prompt else 0, out.ctypes.data_as(POINTER(c_int)), stride, out_lens.ctypes.data_as(POINTER(c_int)))
         return [[int(t) for t in out[i, :out_lens[i]]] for i in range(B)]
+
+    def generate_streaming(self, prompt, params: SampleParams, callback):
+        """GpuMambaLM::generate_streaming (gpu_lm.rs:334-377), batch-1 engines: `callback(token)` runs for every new
+        token as soon as it exists; a true return value ends the generation early.  Returns nothing."""
+        if self.backbone.batch != 1:
+            raise ValueError("generate_streaming requires batch=1; use generate_batch for batch>1")
+        p = np.ascontiguousarray(list(prompt), dtype=np.int32)
+        eos = np.ascontiguousarray(params.eos_token_ids, dtype=np.int32)
+        cp = _CSampleParams()
+        cp.sampler = _CSampler(params.temperature, params.top_k, params.top_p, params.min_p, params.repetition_penalty)
+        cp.max_tokens, cp.n_eos, cp.seed = params.max_tokens, eos.size, params.seed & 0xFFFFFFFFFFFFFFFF
+        cp.eos_token_ids = eos.ctypes.data_as(POINTER(c_int)) if eos.size else None
+        raised = []
+
+        def trampoline(token, _user):
+            try:
+                return 1 if callback(int(token)) else 0
+            except BaseException as e:   # an exception must not unwind through the C frames: stop, re-raise after the call
+                raised.append(e)
+                return 1
+
+        _call("mrs_lm_generate_streaming", self._h, p.ctypes.data_as(POINTER(c_int)) if p.size else None, int(p.size), byref(cp),
+              _TOKEN_CB(trampoline), None)
+        if raised:
+            raise raised[0]
 
     def generate(self, prompt, max_tokens: int | None = None, params: SampleParams | None = None):
         """GpuMambaLM::generate for a batch-1 engine (gpu_lm.rs:323-377).  With `params` the reference's sampled loop

@@ -1087,8 +1087,10 @@ static int gen_forward(mrs_lm *lm) {
     return lm_logits(lm);
 }
 
-extern "C" int mrs_lm_generate_batch(mrs_lm *lm, const int *prompts, const int *prompt_lens, const mrs_sample_params *params,
-                                     int seen_includes_prompt, int *out_tokens, int out_stride, int *out_lens) {
+// The generation loop behind mrs_lm_generate_batch and mrs_lm_generate_streaming.  With a callback (batch 1) the host
+// looks at the slot after every step instead of every 16th and hands each new token over as it appears.
+static int gen_run(mrs_lm *lm, const int *prompts, const int *prompt_lens, const mrs_sample_params *params, int seen_includes_prompt,
+                   int *out_tokens, int out_stride, int *out_lens, mrs_token_callback cb, void *user) {
     if (!lm || !prompt_lens || !params || !out_tokens || !out_lens) return fail(MRS_E_NULL, "mrs_lm_generate_batch: null pointer");
     const LmHooks *bb = &lm->eng;
     hipStream_t st = bb->stream;
@@ -1166,7 +1168,8 @@ extern "C" int mrs_lm_generate_batch(mrs_lm *lm, const int *prompts, const int *
         MRS_TRY(gen_pick(lm));
         steps = max_tokens;
     }
-    int done = 0;
+    int done = 0, emitted = 0;
+    bool stopped = false;
     for (int s = 0; s < steps && running > 0; s++) {
         if (lm->gen_graph_ready) {
             MRS_HIP(hipGraphLaunch(lm->gen_graph_exec, st));
@@ -1187,7 +1190,20 @@ extern "C" int mrs_lm_generate_batch(mrs_lm *lm, const int *prompts, const int *
             MRS_TRY(gen_forward(lm));
             MRS_TRY(gen_pick(lm));
         }
-        if (++done % 16 == 0 || s + 1 == steps) {   // the only host round trip of the loop: is anyone still running?
+        if (cb) {
+            // streaming (one slot): the slot's output length and the token at the next unread position, every step
+            int olen_now = 0, tok = 0;
+            MRS_HIP(hipMemcpyAsync(&running, lm->gen.n_running, sizeof(int), hipMemcpyDeviceToHost, st));
+            MRS_HIP(hipMemcpyAsync(&olen_now, lm->gen.out_len, sizeof(int), hipMemcpyDeviceToHost, st));
+            if (emitted < lm->gen_dyn_host.out_stride)
+                MRS_HIP(hipMemcpyAsync(&tok, lm->gen_dyn_host.out + emitted, sizeof(int), hipMemcpyDeviceToHost, st));
+            MRS_HIP(hipStreamSynchronize(st));
+            ++done;
+            if (olen_now > emitted) {
+                emitted++;
+                if (cb(tok, user) != 0) { stopped = true; break; }   // the caller has seen enough
+            }
+        } else if (++done % 16 == 0 || s + 1 == steps) {   // the only host round trip of the loop: is anyone still running?
             MRS_HIP(hipMemcpyAsync(&running, lm->gen.n_running, sizeof(int), hipMemcpyDeviceToHost, st));
             MRS_HIP(hipStreamSynchronize(st));
         }
@@ -1196,5 +1212,27 @@ extern "C" int mrs_lm_generate_batch(mrs_lm *lm, const int *prompts, const int *
     MRS_HIP(hipMemcpy2DAsync(out_tokens, (size_t)out_stride * sizeof(int), lm->gen_dyn_host.out, (size_t)lm->gen_dyn_host.out_stride * sizeof(int),
                              (size_t)std::min(out_stride, lm->gen_dyn_host.out_stride) * sizeof(int), B, hipMemcpyDeviceToHost, st));
     MRS_HIP(hipStreamSynchronize(st));
+    if (cb) {
+        // stopped by the callback: what was handed over; else whatever the loop has not handed over yet (after a
+        // prefilled prompt the first token exists before the first step, so the hand-over runs one step behind)
+        if (stopped) out_lens[0] = emitted;
+        for (; !stopped && emitted < out_lens[0]; emitted++)
+            if (cb(out_tokens[emitted], user) != 0) { out_lens[0] = emitted + 1; break; }
+    }
     return MRS_OK;
+}
+
+extern "C" int mrs_lm_generate_batch(mrs_lm *lm, const int *prompts, const int *prompt_lens, const mrs_sample_params *params,
+                                     int seen_includes_prompt, int *out_tokens, int out_stride, int *out_lens) {
+    return gen_run(lm, prompts, prompt_lens, params, seen_includes_prompt, out_tokens, out_stride, out_lens, nullptr, nullptr);
+}
+
+extern "C" int mrs_lm_generate_streaming(mrs_lm *lm, const int *prompt, int prompt_len, const mrs_sample_params *params,
+                                         mrs_token_callback cb, void *user) {
+    if (!lm || !params || !cb) return fail(MRS_E_NULL, "mrs_lm_generate_streaming: null pointer");
+    if (lm->batch != 1) return fail(MRS_E_SHAPE, "mrs_lm_generate_streaming: batch=%d (a batch-1 engine; mrs_lm_generate_batch for more)", lm->batch);
+    if (params->max_tokens < 0) return fail(MRS_E_SHAPE, "mrs_lm_generate_streaming: max_tokens=%d", params->max_tokens);
+    std::vector<int> out((size_t)std::max(params->max_tokens, 1));
+    int n = 0;
+    return gen_run(lm, prompt, &prompt_len, params, 1, out.data(), (int)out.size(), &n, cb, user);
 }

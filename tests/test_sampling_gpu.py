@@ -258,6 +258,36 @@ def test_generate_long_prompt_takes_the_prefill_route():
     lm.close(); lm.backbone.close()
 
 
+@pytest.mark.parametrize("plen", [5, 300])
+def test_generate_streaming_hands_over_the_tokens_of_generate_one_by_one(plen):
+    """generate == collecting generate_streaming's callback (gpu_lm.rs:323-331), for a stepped prompt and for one that
+    takes the prefill route (where the first token exists before the first step); a callback may end the run early."""
+    lm, P, embed, table = small_lm(1)
+    rng = np.random.default_rng(plen)
+    prompt = [int(t) for t in rng.integers(0, 300, plen)]
+    sp = SampleParams(temperature=5.0, top_k=40, top_p=0.95, repetition_penalty=1.3, max_tokens=12, seed=21)
+    want = lm.generate(prompt, params=sp)
+    assert len(want) == 12
+    got = []
+    assert lm.generate_streaming(prompt, sp, got.append) is None
+    assert got == want
+    first = []
+    lm.generate_streaming(prompt, sp, lambda t: first.append(t) or len(first) == 4)
+    assert first == want[:4]
+    # EOS ends the stream without being handed over (the reference breaks before the callback)
+    eos = SampleParams(temperature=5.0, top_k=40, top_p=0.95, repetition_penalty=1.3, max_tokens=12, seed=21, eos_token_ids=[want[6]])
+    cut = []
+    lm.generate_streaming(prompt, eos, cut.append)
+    assert cut == want[:want.index(want[6])]
+    # an exception in the callback surfaces after the call, and the engine stays usable
+    def boom(t):
+        raise RuntimeError("stop")
+    with pytest.raises(RuntimeError, match="stop"):
+        lm.generate_streaming(prompt, sp, boom)
+    assert lm.generate(prompt, params=sp) == want
+    lm.close(); lm.backbone.close()
+
+
 def test_generate_batch_rejects_bad_arguments():
     from mamba_rs_amd import MambaHipError
     lm, *_ = small_lm(2)
