@@ -21,6 +21,17 @@
 
 namespace mrs {
 
+// a mod 2 pi in [0, 2 pi) (src/mamba3_siso/cpu/inference.rs:179-180 divides; an f64 division is a ~30-instruction
+// dependent sequence and this sits in a serial chain over time, so the quotient comes from the reciprocal and the
+// rare off-by-one of its floor is folded back).
+__device__ __forceinline__ double wrap_2pi(double a) {
+    const double two_pi = 6.283185307179586, inv_two_pi = 0.15915494309189535;
+    double r = fma(-two_pi, floor(a * inv_two_pi), a);
+    r = r < 0.0 ? r + two_pi : r;
+    return r >= two_pi ? r - two_pi : r;
+}
+
+
 constexpr float kPi = 3.14159265358979323846f;
 
 __device__ __forceinline__ float heavy_tail(float x) { return x >= 0.0f ? 1.0f + x : 1.0f / (1.0f - x); }
@@ -88,10 +99,7 @@ __global__ __launch_bounds__(1024) void m3_layer_step_kernel(
     if (own_a) {
         const int a = tid;
         const float delta = tanhf(ang_in) * kPi * dtv;
-        const double two_pi = 6.283185307179586;
-        double acc = (double)ang_old + (double)delta;
-        acc -= two_pi * floor(acc / two_pi);
-        const float an = (float)acc;
+        const float an = (float)wrap_2pi((double)ang_old + (double)delta);
         angle[bh * nr + a] = an;
         float sn, cs;
         sincosf(an, &sn, &cs);
@@ -143,20 +151,19 @@ __global__ __launch_bounds__(1024) void m3_layer_step_kernel(
 }
 
 // ---- prefill glue ---------------------------------------------------------------------------------
-// Three kernels in front of the chunked scan (the reference's m3_split, bcnorm_fwd x2, bc_bias_add x2, angle_dt_fwd,
+// Four kernels in front of the chunked scan (the reference's m3_split, bcnorm_fwd x2, bc_bias_add x2, angle_dt_fwd,
 // rope_fwd, kernels/mamba3_ops.cu:72-650):
 //   m3_scalars_kernel     row-parallel: dt = softplus(dd_dt + bias), a = min(-heavy_tail(dd_A), -a_floor),
 //                         trap = sigmoid(raw), and tanh(angle_raw) * pi per rope pair;
-//   m3_angle_scan_kernel  the rotation angle of (head, pair) at step t is the initial angle plus the running sum over
-//                         time of (tanh * pi) * dt_h (angle_dt_fwd is sequential over T per thread): here a workgroup
-//                         per (batch row, head) splits T into segments -- per-segment sums, an exclusive prefix over
-//                         the segments, then the running sums inside each segment -- in f64, wrapped to [0, 2 pi);
+//   m3_angle_sums/apply   the rotation angle of (head, pair) at step t is the initial angle plus the running sum over
+//                         time of (tanh * pi) * dt_h (angle_dt_fwd is sequential over T per thread): here T is cut into
+//                         segments -- per-segment sums, the segments before folded in, then the running sums inside
+//                         each segment -- in f64, wrapped to [0, 2 pi);
 //   m3_kq_kernel          row-parallel: B/C RMSNorm + per-head bias + rotation -> K, Q; x -> activation type.
-__device__ __forceinline__ double wrap_2pi(double a) {
-    const double two_pi = 6.283185307179586;
-    return a - two_pi * floor(a / two_pi);
-}
-
+// Time segments of the prefill's angle scan (workgroups per batch row).  Every workgroup reads the sums of the segments
+// before its own, so more segments mean more reads: at batch 4 x 4096 the two launches took 35 us with 32 segments,
+// 25 us with 64, 30 us with 128.
+constexpr int kAngleSegs = 64;
 // one thread per (row, j): j < nh -> the head scalars, j >= nh -> rope pair j - nh
 __global__ __launch_bounds__(256) void m3_scalars_kernel(float *__restrict__ dt_out, float *__restrict__ a_out, float *__restrict__ trap_out,
                                                          float *__restrict__ tanhpi_out, const float *__restrict__ proj, int64_t ip,
@@ -177,65 +184,99 @@ __global__ __launch_bounds__(256) void m3_scalars_kernel(float *__restrict__ dt_
     }
 }
 
-// grid = batch * nh, 1024 threads = nr_pad rope pairs (fast) x nsegs segments; angle_out [rows][nh][nr] f32
-__global__ __launch_bounds__(1024) void m3_angle_scan_kernel(float *__restrict__ angle_out, float *__restrict__ angle_state,
-                                                             const float *__restrict__ dt, const float *__restrict__ tanhpi, int Tlen,
-                                                             int nh, int nr, int nr_pad) {
-    __shared__ double part[1024];
-    const int b = blockIdx.x / nh, h = blockIdx.x - b * nh;
-    const int a = threadIdx.x % nr_pad, seg = threadIdx.x / nr_pad;
-    const int nsegs = 1024 / nr_pad;
+// Two launches over a grid of (batch row, time segment) workgroups; thread j of a workgroup owns entry j = h * nr + a of
+// the [nh][nr] angle row, so every load and store of a wave is one contiguous piece of a row (a thread per (pair,
+// segment) with the pairs of one head per workgroup read and wrote 64-byte pieces a row apart: 33 us for 25 MB).
+//   sums:  seg_sum[b][seg][j] = sum over the segment of (tanh * pi)[t][a] * dt[t][h] (f64); segment 0 also snapshots
+//          the entering angles, which the last segment of the second launch overwrites;
+//   apply: start = entering angle advanced over the segments before (wrapped after every segment), then the running
+//          sums inside the segment, wrapped after every step; angle_out [rows][nh][nr] f32.
+__global__ __launch_bounds__(1024) void m3_angle_sums_kernel(double *__restrict__ seg_sum, float *__restrict__ snap,
+                                                             const float *__restrict__ angle_state, const float *__restrict__ dt,
+                                                             const float *__restrict__ tanhpi, int Tlen, int nh, int nr, int nsegs) {
+    const int b = blockIdx.x / nsegs, seg = blockIdx.x - b * nsegs, per = nh * nr;
     const int seglen = (Tlen + nsegs - 1) / nsegs;
     const int t0 = min(Tlen, seg * seglen), t1 = min(Tlen, t0 + seglen);
-    const bool live = a < nr;
-    const float *dp = dt + (int64_t)b * Tlen * nh + h;
-    const float *tp = tanhpi + (int64_t)b * Tlen * nr + a;
-    // the per-step increments of this thread's segment, staged in registers in groups of 8 so that the loads of a
-    // group are in flight together (the running sum itself is a dependent chain)
-    double sum = 0.0;
-    if (live) {
+    for (int j = threadIdx.x; j < per; j += blockDim.x) {
+        const int h = j / nr, a = j - h * nr;
+        const float *dp = dt + (int64_t)b * Tlen * nh + h;
+        const float *tp = tanhpi + (int64_t)b * Tlen * nr + a;
+        double sum = 0.0;
+        // the operands of the next group of 8 steps are requested before the current group is added up
+        float xa[8], xb[8], na[8], nb[8];
+        auto request = [&](float (&a8)[8], float (&b8)[8], int tg) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const int t = max(t0, min(tg + i, t1 - 1));
+                a8[i] = tp[(int64_t)t * nr];
+                b8[i] = dp[(int64_t)t * nh];
+            }
+        };
+        if (t0 < t1) request(xa, xb, t0);
         for (int tg = t0; tg < t1; tg += 8) {
-            float d[8];
+            request(na, nb, tg + 8);
 #pragma unroll
-            for (int j = 0; j < 8; j++) {
-                const int t = min(tg + j, t1 - 1);
-                d[j] = tp[(int64_t)t * nr] * dp[(int64_t)t * nh];
+            for (int i = 0; i < 8; i++)
+                if (tg + i < t1) sum += (double)(xa[i] * xb[i]);
+#pragma unroll
+            for (int i = 0; i < 8; i++) { xa[i] = na[i]; xb[i] = nb[i]; }
+        }
+        seg_sum[((int64_t)b * nsegs + seg) * per + j] = sum;
+        if (seg == 0) snap[(int64_t)b * per + j] = angle_state[(int64_t)b * per + j];
+    }
+}
+
+__global__ __launch_bounds__(1024) void m3_angle_apply_kernel(float *__restrict__ angle_out, float *__restrict__ angle_state,
+                                                              const double *__restrict__ seg_sum, const float *__restrict__ snap,
+                                                              const float *__restrict__ dt, const float *__restrict__ tanhpi, int Tlen,
+                                                              int nh, int nr, int nsegs) {
+    const int b = blockIdx.x / nsegs, seg = blockIdx.x - b * nsegs, per = nh * nr;
+    const int seglen = (Tlen + nsegs - 1) / nsegs;
+    const int t0 = min(Tlen, seg * seglen), t1 = min(Tlen, t0 + seglen);
+    for (int j = threadIdx.x; j < per; j += blockDim.x) {
+        const int h = j / nr, a = j - h * nr;
+        const float *dp = dt + (int64_t)b * Tlen * nh + h;
+        const float *tp = tanhpi + (int64_t)b * Tlen * nr + a;
+        // A dependent f64 operation costs tens of cycles and a wrap is half a dozen of them, so wraps stay out of the
+        // serial chains: the segments before this one are summed unwrapped on four independent accumulators and wrapped
+        // once, and inside the segment the chain is the running sum alone, every output wrapped on its own (equal to
+        // wrapping after every step up to f64 rounding: the angles are only defined modulo 2 pi).
+        double p4[4] = {0.0, 0.0, 0.0, 0.0};
+        for (int s0 = 0; s0 < seg; s0 += 32) {
+            double v[32];
+#pragma unroll
+            for (int i = 0; i < 32; i++) v[i] = s0 + i < seg ? seg_sum[((int64_t)b * nsegs + s0 + i) * per + j] : 0.0;
+#pragma unroll
+            for (int i = 0; i < 32; i++) p4[i & 3] += v[i];
+        }
+        double acc = wrap_2pi((double)snap[(int64_t)b * per + j] + ((p4[0] + p4[1]) + (p4[2] + p4[3])));
+        float *out = angle_out + (int64_t)b * Tlen * per + j;
+        float xa[8], xb[8], na[8], nb[8];
+        auto request = [&](float (&a8)[8], float (&b8)[8], int tg) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const int t = max(t0, min(tg + i, t1 - 1));
+                a8[i] = tp[(int64_t)t * nr];
+                b8[i] = dp[(int64_t)t * nh];
             }
-#pragma unroll
-            for (int j = 0; j < 8; j++)
-                if (tg + j < t1) sum += (double)d[j];
-        }
-    }
-    part[seg * nr_pad + a] = sum;
-    __syncthreads();
-    if (seg == 0 && live) {
-        float *stp = angle_state + ((int64_t)b * nh + h) * nr + a;
-        double acc = (double)*stp;
-        for (int s2 = 0; s2 < nsegs; s2++) {
-            const double add = part[s2 * nr_pad + a];
-            part[s2 * nr_pad + a] = acc;
-            acc = wrap_2pi(acc + add);
-        }
-        *stp = (float)acc;
-    }
-    __syncthreads();
-    if (live) {
-        double acc = part[seg * nr_pad + a];
+        };
+        if (t0 < t1) request(xa, xb, t0);
         for (int tg = t0; tg < t1; tg += 8) {
-            float d[8];
+            request(na, nb, tg + 8);   // the next group's operands, before this group's chain
+            double run[8];
 #pragma unroll
-            for (int j = 0; j < 8; j++) {
-                const int t = min(tg + j, t1 - 1);
-                d[j] = tp[(int64_t)t * nr] * dp[(int64_t)t * nh];
+            for (int i = 0; i < 8; i++) {
+                acc += tg + i < t1 ? (double)(xa[i] * xb[i]) : 0.0;
+                run[i] = acc;
             }
 #pragma unroll
-            for (int j = 0; j < 8; j++) {
-                if (tg + j < t1) {
-                    acc = wrap_2pi(acc + (double)d[j]);
-                    angle_out[(((int64_t)b * Tlen + tg + j) * nh + h) * nr + a] = (float)acc;
-                }
-            }
+            for (int i = 0; i < 8; i++) { xa[i] = na[i]; xb[i] = nb[i]; }
+#pragma unroll
+            for (int i = 0; i < 8; i++)
+                if (tg + i < t1) out[(int64_t)(tg + i) * per] = (float)wrap_2pi(run[i]);
+            acc = wrap_2pi(acc);   // once per group: keeps the running sum small
         }
+        if (seg == nsegs - 1) angle_state[(int64_t)b * per + j] = (float)acc;
     }
 }
 
@@ -378,7 +419,8 @@ struct mrs_m3_backbone {
     int graph_ready;
     // prefill scratch for sequences of pf_T steps (0: not allocated)
     int pf_T;
-    float *pf_in, *pf_residual, *pf_proj, *pf_dt, *pf_a, *pf_trap, *pf_tanhpi, *pf_angle;
+    float *pf_in, *pf_residual, *pf_proj, *pf_dt, *pf_a, *pf_trap, *pf_tanhpi, *pf_angle, *pf_angle_snap;
+    double *pf_angle_sums;   // [batch][kAngleSegs][nh * n_rope] per-segment angle increments of the prefill
     void *pf_normed, *pf_bulk, *pf_x, *pf_K, *pf_Q, *pf_y, *pf_gated, *pf_out, *pf_ws;
     size_t pf_ws_bytes;
 };
@@ -680,6 +722,8 @@ extern "C" int mrs_m3_backbone_alloc_prefill_scratch(mrs_m3_backbone *bb, int T)
     MRS_TRY(dev_alloc3(bb, (void **)&bb->pf_trap, rows * nh * 4));
     MRS_TRY(dev_alloc3(bb, (void **)&bb->pf_tanhpi, rows * nrz * 4));
     MRS_TRY(dev_alloc3(bb, (void **)&bb->pf_angle, rows * nh * nrz * 4));
+    MRS_TRY(dev_alloc3(bb, (void **)&bb->pf_angle_sums, (size_t)bb->batch * kAngleSegs * nh * nrz * sizeof(double)));
+    MRS_TRY(dev_alloc3(bb, (void **)&bb->pf_angle_snap, (size_t)bb->batch * nh * nrz * 4));
     MRS_TRY(dev_alloc3(bb, &bb->pf_normed, rows * dm * es));
     MRS_TRY(dev_alloc3(bb, &bb->pf_x, rows * di * es));
     MRS_TRY(dev_alloc3(bb, &bb->pf_K, rows * nh * ds * es));
@@ -783,11 +827,14 @@ int prefill_body3(mrs_m3_backbone *bb, int T) {
             MRS_TRY(check_launch("m3_scalars_kernel"));
         }
         if (nr > 0) {
-            int nr_pad = 1;
-            while (nr_pad < nr) nr_pad <<= 1;
-            hipLaunchKernelGGL(m3_angle_scan_kernel, dim3((unsigned)(B * nh)), dim3(1024), 0, bb->stream, bb->pf_angle, ang, bb->pf_dt,
-                               bb->pf_tanhpi, T, nh, nr, nr_pad);
-            MRS_TRY(check_launch("m3_angle_scan_kernel"));
+            const int per = nh * nr, threads = std::min(1024, (per + 63) / 64 * 64);
+            const int nsegs = std::max(1, std::min(kAngleSegs, T / 8));
+            hipLaunchKernelGGL(m3_angle_sums_kernel, dim3((unsigned)(B * nsegs)), dim3((unsigned)threads), 0, bb->stream, bb->pf_angle_sums,
+                               bb->pf_angle_snap, ang, bb->pf_dt, bb->pf_tanhpi, T, nh, nr, nsegs);
+            MRS_TRY(check_launch("m3_angle_sums_kernel"));
+            hipLaunchKernelGGL(m3_angle_apply_kernel, dim3((unsigned)(B * nsegs)), dim3((unsigned)threads), 0, bb->stream, bb->pf_angle, ang,
+                               bb->pf_angle_sums, bb->pf_angle_snap, bb->pf_dt, bb->pf_tanhpi, T, nh, nr, nsegs);
+            MRS_TRY(check_launch("m3_angle_apply_kernel"));
         }
         // the chunked kernel reads x in place out of the bulk rows.  (Folding the SiLU gate into its y store was
         // measured and dropped: the scattered z reads cost the latency-bound kernel 54 us against 28 us for the
