@@ -341,6 +341,81 @@ __global__ __launch_bounds__(256) void m3_kq_kernel(
         for (int i = tid; i < di; i += 256) xout[r * di + i] = row[di + i];
 }
 
+// The same for one group (ngroups == 1), a wave per row and no LDS: every lane forms the row's two RMS values itself
+// (strided sums + a butterfly, the same order of additions as above), so nothing waits at a barrier and the operands
+// of several items are in flight together.  Four rows per workgroup.
+template <typename T>
+__global__ __launch_bounds__(256) void m3_kq_rows_kernel(
+    T *__restrict__ Kout, T *__restrict__ Qout, T *__restrict__ xout, const T *__restrict__ bulk, int64_t ldb,
+    const float *__restrict__ angle, const float *__restrict__ bnw, const float *__restrict__ cnw,
+    const float *__restrict__ b_bias, const float *__restrict__ c_bias, int64_t rows, int nh, int hd, int ds, int nr, float eps) {
+    const int w = threadIdx.x >> 6, l = threadIdx.x & 63;
+    const int64_t r = (int64_t)blockIdx.x * 4 + w;
+    if (r >= rows) return;   // whole waves leave; the kernel has no barrier
+    const int di = nh * hd;
+    const T *row = bulk + r * ldb, *Bp = row + 2 * di, *Cp = Bp + ds;
+    float ssb = 0.0f, ssc = 0.0f;
+    for (int n = l; n < ds; n += 64) {
+        const float b = Store<T>::ld(Bp + n), c = Store<T>::ld(Cp + n);
+        ssb = fmaf(b, b, ssb); ssc = fmaf(c, c, ssc);
+    }
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) { ssb += __shfl_xor(ssb, m, kWave); ssc += __shfl_xor(ssc, m, kWave); }
+    const float ib = 1.0f / sqrtf(ssb / (float)ds + eps), ic = 1.0f / sqrtf(ssc / (float)ds + eps);
+    const int quarter = ds / 4, items = nh * quarter;
+    struct alignas(4 * sizeof(T)) V4 { T v[4]; };
+    constexpr int kTrips = 3;   // items of a lane whose operands are requested together
+    for (int i0 = l; i0 < items; i0 += 64 * kTrips) {
+        V4 bv[kTrips], cv[kTrips];
+        float4 bw[kTrips], cw[kTrips], bb4[kTrips], cb4[kTrips];
+        float ang[kTrips][2];
+#pragma unroll
+        for (int t = 0; t < kTrips; t++) {
+            const int i = min(i0 + 64 * t, items - 1);   // past the end: an in-range item, computed and dropped
+            const int h = i / quarter, j4 = i - h * quarter, n = 4 * j4;
+            bv[t] = *reinterpret_cast<const V4 *>(Bp + n); cv[t] = *reinterpret_cast<const V4 *>(Cp + n);
+            bw[t] = *reinterpret_cast<const float4 *>(bnw + n); cw[t] = *reinterpret_cast<const float4 *>(cnw + n);
+            bb4[t] = *reinterpret_cast<const float4 *>(b_bias + h * ds + n); cb4[t] = *reinterpret_cast<const float4 *>(c_bias + h * ds + n);
+#pragma unroll
+            for (int pr = 0; pr < 2; pr++) ang[t][pr] = 2 * j4 + pr < nr ? angle[(r * nh + h) * nr + 2 * j4 + pr] : 0.0f;
+        }
+#pragma unroll
+        for (int t = 0; t < kTrips; t++) {
+            const int i = i0 + 64 * t;
+            if (i < items) {
+                const int h = i / quarter, j4 = i - h * quarter, n = 4 * j4;
+                float k[4] = {Store<T>::ld(&bv[t].v[0]) * ib * bw[t].x + bb4[t].x, Store<T>::ld(&bv[t].v[1]) * ib * bw[t].y + bb4[t].y,
+                              Store<T>::ld(&bv[t].v[2]) * ib * bw[t].z + bb4[t].z, Store<T>::ld(&bv[t].v[3]) * ib * bw[t].w + bb4[t].w};
+                float q[4] = {Store<T>::ld(&cv[t].v[0]) * ic * cw[t].x + cb4[t].x, Store<T>::ld(&cv[t].v[1]) * ic * cw[t].y + cb4[t].y,
+                              Store<T>::ld(&cv[t].v[2]) * ic * cw[t].z + cb4[t].z, Store<T>::ld(&cv[t].v[3]) * ic * cw[t].w + cb4[t].w};
+#pragma unroll
+                for (int pr = 0; pr < 2; pr++) {
+                    if (2 * j4 + pr < nr) {
+                        float s_, c_;
+                        if constexpr (sizeof(T) == 2) {
+                            // angles lie in [0, 2 pi): the hardware sine / cosine (absolute error of the order of 1e-6) is
+                            // far inside what a 16-bit K or Q can hold
+                            s_ = __sinf(ang[t][pr]); c_ = __cosf(ang[t][pr]);
+                        } else {
+                            sincosf(ang[t][pr], &s_, &c_);
+                        }
+                        const float k0 = k[2 * pr], k1 = k[2 * pr + 1], q0 = q[2 * pr], q1 = q[2 * pr + 1];
+                        k[2 * pr] = c_ * k0 - s_ * k1; k[2 * pr + 1] = s_ * k0 + c_ * k1;
+                        q[2 * pr] = c_ * q0 - s_ * q1; q[2 * pr + 1] = s_ * q0 + c_ * q1;
+                    }
+                }
+                V4 kv, qv;
+#pragma unroll
+                for (int e = 0; e < 4; e++) { Store<T>::st(&kv.v[e], k[e]); Store<T>::st(&qv.v[e], q[e]); }
+                *reinterpret_cast<V4 *>(Kout + (r * nh + h) * ds + n) = kv;
+                *reinterpret_cast<V4 *>(Qout + (r * nh + h) * ds + n) = qv;
+            }
+        }
+    }
+    if (xout)
+        for (int i = l; i < di; i += 64) xout[r * di + i] = row[di + i];
+}
+
 // gated[row, i] = y * silu(z), or RMSNormGated over each head first; z = the first d_inner elements of the bulk row.
 // One workgroup (256 threads) per row, a wave per head at a time for the normalised form.
 template <typename T>
@@ -748,6 +823,12 @@ int launch_kq_t(mrs_m3_backbone *bb, const Layer3 &lw, int64_t rows, const void 
     const int ng = c.ngroups, ds = c.d_state;
     const size_t lds = (size_t)(2 * ng * ds + 2 * ng) * sizeof(float);
     if (lds > 60000) return fail(MRS_E_SHAPE, "m3 K/Q kernel: ngroups * d_state too large for LDS (%zu bytes)", lds);
+    if (ng == 1 && ds % 4 == 0 && ldb % 4 == 0 && (2 * bb->nh * c.headdim) % 4 == 0) {
+        hipLaunchKernelGGL((m3_kq_rows_kernel<T>), dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, bb->stream, (T *)bb->pf_K, (T *)bb->pf_Q,
+                           copy_x ? (T *)bb->pf_x : nullptr, (const T *)bulk, ldb, bb->pf_angle, lw.bnw, lw.cnw, lw.b_bias, lw.c_bias, rows,
+                           bb->nh, c.headdim, ds, bb->nr, c.rms_norm_eps);
+        return check_launch("m3_kq_rows_kernel");
+    }
     hipLaunchKernelGGL((m3_kq_kernel<T>), dim3((unsigned)rows), dim3(256), lds, bb->stream, (T *)bb->pf_K, (T *)bb->pf_Q,
                        copy_x ? (T *)bb->pf_x : nullptr, (const T *)bulk, ldb, bb->pf_angle, lw.bnw, lw.cnw, lw.b_bias, lw.c_bias, bb->nh,
                        c.headdim, ng, ds, bb->nr, c.rms_norm_eps);
