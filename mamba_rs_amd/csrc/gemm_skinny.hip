@@ -465,9 +465,10 @@ static int launch_skinny_t(hipStream_t st, TO *C, int64_t ldc, const T *A, int64
     const dim3 block(kGemmWaves * 64);
     // one to four rows: the lanes-along-the-row route (64 lanes per weight row when a row is a multiple of 1 KB, else 32)
     static const bool no_rowwise = getenv("MRS_DECODE_NO_ROWWISE") != nullptr;
-    const int lpr = (M > 4 || no_rowwise || (int64_t)K * 8 > 48 * 1024) ? 0 : (K % 512 == 0 ? 64 : (K % 256 == 0 ? 32 : 0));   // rows fit in LDS
+    int lpr = (M > 4 || no_rowwise || (int64_t)K * 8 > 48 * 1024) ? 0 : (K % 512 == 0 ? 64 : (K % 256 == 0 ? 32 : 0));   // rows fit in LDS
     const int ksplit = (ep.mode == 0 && ep.ksplit > 1) ? ep.ksplit : 1;
-    if (ksplit > 1 && (lpr != 0 || ep.row_scale || !ep.xpart || ksplit > (K >> 5)))
+    if (ksplit > 1) lpr = 0;   // a split K runs on the matrix-core route at any row count
+    if (ksplit > 1 && (ep.row_scale || !ep.xpart || ksplit > (K >> 5)))
         return fail(MRS_E_SHAPE, "skinny gemm: K split needs the matrix-core route, a plain product, a share buffer and ksplit <= K / 32 (ksplit=%d)", ksplit);
     ep.kslice = ((K >> 5) + ksplit - 1) / ksplit;
     const dim3 grid((unsigned)((N + 15) / 16), (unsigned)((M + 15) / 16), (unsigned)(((K >> 5) + ep.kslice - 1) / ep.kslice));

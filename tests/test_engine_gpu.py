@@ -258,6 +258,31 @@ def test_wide_dt_rank_at_large_batch_runs_dt_proj_as_its_own_gemm():
         eng.close()
 
 
+@pytest.mark.parametrize("B", [1, 3, 20])
+def test_wide_model_runs_x_proj_as_a_split_k_launch(B):
+    """d_inner 2048 x xdbl 96: a row's per-tile shares would be 48 KB, so x_proj does not ride in the in_proj launch; it
+    runs as its own launch with K cut into slices whose shares the step kernel sums -- on the matrix cores also at one to
+    four rows.  Checked against the CPU route on storage-rounded weights, step after step."""
+    cfg = MambaConfig(d_model=1024, d_state=16, d_conv=4, expand=2, n_layers=2)
+    w = MambaWeights.init(cfg, 1024, 45)
+    w.input_proj_w = np.zeros(0, np.float32); w.input_proj_b = np.zeros(0, np.float32)
+    P = oracle_params(w, cfg, 1024, round_to=orc.BF16)
+    P.input_proj_w[:] = np.eye(1024, dtype=np.float32); P.input_proj_b[:] = 0
+    rng = np.random.default_rng(B)
+    eng = GpuMambaBackbone.new_with_dtype(0, w, cfg, 1024, B, WeightDtype.BF16)
+    x = rng.standard_normal((5, B, 1024)).astype(np.float32)
+    rows = sorted({0, B - 1})
+    st = {b: orc.m1_zero_state(P) for b in rows}
+    for t in range(5):
+        if t == 2:
+            eng.capture_graph()
+        got = eng.step(x[t])
+        for b in rows:
+            want = orc.m1_backbone_step(P, x[t, b], *st[b])
+            assert cosine(got[b], want) >= 0.999, (B, t, b)
+    eng.close()
+
+
 @pytest.mark.parametrize("dm,batch", [(256, 1), (256, 3), (512, 4), (768, 2), (768, 7), (256, 16), (512, 13)])
 def test_few_row_decode_chain_with_folded_x_proj_equals_the_many_row_chain(dm, batch):
     """Up to 16 rows x_proj rides in the in_proj launch (per-tile shares, summed by the step kernel), and at one to four
