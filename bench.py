@@ -340,7 +340,14 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch one 256 MiB device copy (a known-size kernel to scale rocprof FETCH_SIZE/WRITE_SIZE by)")
     ap.add_argument("--big", action="store_true", help="also run the 2.8b-shape LM leg (several minutes of host-side init)")
+    ap.add_argument("--legs", default="lm,m1_kernels,m3,m3_engine",
+                    help="comma list of the extras to run: lm, m1_kernels, m3, m3_engine (for profiling one leg at a time)")
     args = ap.parse_args()
+    legs = {x.strip() for x in args.legs.split(",") if x.strip()}
+    unknown = legs - {"lm", "m1_kernels", "m3", "m3_engine"}
+    if unknown:
+        print(f"bench.py: unknown --legs entries {sorted(unknown)}", file=sys.stderr)
+        sys.exit(2)
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus must be 1 (no multi-GPU path exists)", file=sys.stderr)
         sys.exit(2)
@@ -376,11 +383,15 @@ def main():
         out["cpu_baseline"] = cpu_leg(inp, shape, nbytes)
     if not args.no_extras:
         extras = {}
-        extras["lm_130m_shape_bf16"] = lm_leg("130m-shape", dict(d_model=768, d_state=16, d_conv=4, expand=2, n_layers=24), 50280,
-                                              (8, 2048), [64, 1], 256)
-        extras["m1_kernels_130m_shape_bf16"] = m1_kernels_leg()
-        extras["mamba3_768_bf16"] = m3_leg()
-        extras["mamba3_768_bf16"]["backbone"] = m3_engine_leg()
+        if "lm" in legs:
+            extras["lm_130m_shape_bf16"] = lm_leg("130m-shape", dict(d_model=768, d_state=16, d_conv=4, expand=2, n_layers=24), 50280,
+                                                  (8, 2048), [64, 1], 256)
+        if "m1_kernels" in legs:
+            extras["m1_kernels_130m_shape_bf16"] = m1_kernels_leg()
+        if "m3" in legs or "m3_engine" in legs:
+            extras["mamba3_768_bf16"] = m3_leg() if "m3" in legs else {}
+        if "m3_engine" in legs:
+            extras["mamba3_768_bf16"]["backbone"] = m3_engine_leg()
         if args.big:
             extras["lm_2.8b_shape_bf16"] = lm_leg("2.8b-shape", dict(d_model=2560, d_state=16, d_conv=4, expand=2, n_layers=64), 50280,
                                                   (4, 4096), [1, 16, 128], 128)
