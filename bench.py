@@ -170,6 +170,53 @@ def lm_leg(name, cfg_kw, vocab, prefill_bt, decode_b, decode_steps, seed=42):
     return out
 
 
+def c1_leg():
+    """The tiny CPU-runnable configuration (d_model 128, 2 layers, d_state 16, f32, batch 1, T 256; weights
+    MambaWeights::init seed 42, input N(0,1)): the f32 engine's prefill and graph decode on the GPU, the oracle's
+    restatement of the reference CPU prefill / step beside them, and the largest relative difference between the two."""
+    import numpy as np
+    import orc
+    from mamba_rs_amd import GpuMambaBackbone, MambaConfig, MambaWeights
+    cfg = MambaConfig(d_model=128, d_state=16, d_conv=4, expand=2, n_layers=2)
+    T = 256
+    w = MambaWeights.init(cfg, 128, 42)
+    P = orc.M1Params(128, 16, 4, 2, 2, 128, seed=42)
+    x = np.random.default_rng(42).standard_normal((1, T, 128)).astype(np.float32)
+    eng = GpuMambaBackbone.new(0, w, cfg, 128, 1)
+    got = eng.prefill_sequence(x)                     # warm-up; leaves the input on the device
+    times = []
+    for _ in range(5):
+        eng.reset(); eng.sync()
+        t0 = time.perf_counter(); eng.prefill_device(eng.prefill_input_ptr(), T); eng.sync(); times.append(time.perf_counter() - t0)
+    tp = sorted(times)[2]
+    cs, ss = orc.m1_zero_state(P)
+    want = orc.m1_backbone_prefill(P, x[0], cs, ss)[-1]
+    err = float(np.abs(got.reshape(-1) - want).max() / max(np.abs(want).max(), 1e-30))
+    ctimes = []
+    for _ in range(5):
+        cs, ss = orc.m1_zero_state(P)
+        t0 = time.perf_counter(); orc.m1_backbone_prefill(P, x[0], cs, ss); ctimes.append(time.perf_counter() - t0)
+    tc = sorted(ctimes)[2]
+    eng.reset(); eng.step(x[0, 0:1]); eng.capture_graph()
+    for _ in range(8):
+        eng.step_gpu_only()
+    eng.sync()
+    t0 = time.perf_counter()
+    for _ in range(256):
+        eng.step_gpu_only()
+    eng.sync()
+    td = (time.perf_counter() - t0) / 256
+    t0 = time.perf_counter()
+    for t in range(64):
+        orc.m1_backbone_step(P, x[0, t], cs, ss)
+    tcs = (time.perf_counter() - t0) / 64
+    eng.close()
+    return {"config": "d_model 128, 2 layers, d_state 16, f32, batch 1, T 256",
+            "gpu_prefill": {"ms": tp * 1e3, "tok_per_s": T / tp}, "gpu_decode_us_per_step": td * 1e6,
+            "cpu_port_prefill": {"ms": tc * 1e3, "tok_per_s": T / tc, "cores": orc.num_threads()},
+            "cpu_port_decode_us_per_step": tcs * 1e6, "prefill_last_step_max_rel_diff_gpu_vs_cpu_port": err}
+
+
 def m1_kernels_leg():
     """The other Mamba-1 kernels of the path at the 130m shape (bf16 storage), each against its HBM roofline:
     causal conv1d + SiLU over batch 8 x T 2048 reading the x half of in_proj's rows in place, and the decode
@@ -340,11 +387,11 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch one 256 MiB device copy (a known-size kernel to scale rocprof FETCH_SIZE/WRITE_SIZE by)")
     ap.add_argument("--big", action="store_true", help="also run the 2.8b-shape LM leg (several minutes of host-side init)")
-    ap.add_argument("--legs", default="lm,m1_kernels,m3,m3_engine",
-                    help="comma list of the extras to run: lm, m1_kernels, m3, m3_engine (for profiling one leg at a time)")
+    ap.add_argument("--legs", default="c1,lm,m1_kernels,m3,m3_engine",
+                    help="comma list of the extras to run: c1, lm, m1_kernels, m3, m3_engine (for profiling one leg at a time)")
     args = ap.parse_args()
     legs = {x.strip() for x in args.legs.split(",") if x.strip()}
-    unknown = legs - {"lm", "m1_kernels", "m3", "m3_engine"}
+    unknown = legs - {"c1", "lm", "m1_kernels", "m3", "m3_engine"}
     if unknown:
         print(f"bench.py: unknown --legs entries {sorted(unknown)}", file=sys.stderr)
         sys.exit(2)
@@ -383,6 +430,8 @@ def main():
         out["cpu_baseline"] = cpu_leg(inp, shape, nbytes)
     if not args.no_extras:
         extras = {}
+        if "c1" in legs:
+            extras["tiny_f32_cpu_config"] = c1_leg()
         if "lm" in legs:
             extras["lm_130m_shape_bf16"] = lm_leg("130m-shape", dict(d_model=768, d_state=16, d_conv=4, expand=2, n_layers=24), 50280,
                                                   (8, 2048), [64, 1], 256)

@@ -263,7 +263,7 @@ struct mrs_backbone {
     mrs_m1_config cfg;
     int input_dim, batch, dtype, di, dr, xd, identity_proj, device;
     const float *step_src;  // decode step: where layer 0 reads its input rows (null: the residual buffer itself)
-    int skinny;  // decode projections on the library's own matrix-core GEMM (16-bit storage, batch <= 64, K % 32 == 0)
+    int skinny;  // decode projections on the library's own GEMM (16-bit storage: batch <= 64, K % 32 == 0; f32: batch <= 4, K % 128 == 0)
     hipStream_t stream;
     rocblas_handle blas;
     std::vector<LayerDev> layers;
@@ -416,7 +416,7 @@ static int decode_chain(mrs_backbone *bb, Scratch *s, int r0, int nr, hipStream_
         if (fold_x) { inp.xw = lw.x_proj; inp.xd = xd; inp.xpart = xpart; }
         // x_proj as a launch of its own: K split into slices when the step kernel can sum the shares
         const bool step_sums = xpart && xd <= 256 && lw.dt_t_step && di % (1024 / ds) == 0 && dr % 4 == 0 && (int64_t)nr * dr <= kFuseDtProjLimit;
-        const int ksplit = (!fold_x && step_sums) ? xproj_slices(nr, xd, di) : 1;
+        const int ksplit = (!fold_x && step_sums && dt != MRS_F32) ? xproj_slices(nr, xd, di) : 1;
         const StepFold fold = {xpart, fold_x ? di / 16 : ksplit, nr, xd, dr, dr + ds};
         MRS_TRY(launch_skinny_gemm(st, dt, proj, 0, 2 * di, normed, dm, lw.in_proj_t, nr, 2 * di, dm, inp));
         const SkinnyEpi none = {};
@@ -563,6 +563,10 @@ extern "C" int mrs_backbone_create(mrs_backbone **out, int gpu_ordinal, const mr
     {
         static const bool off = [] { const char *e = getenv("MRS_DECODE_LIBRARY_GEMM"); return e && atoi(e) != 0; }();
         bb->skinny = !off && (dtype == MRS_BF16 || dtype == MRS_F16) && batch <= 64 && dm % 32 == 0 && di % 32 == 0;
+        // f32 storage: the same chain on the row-wise route of the GEMM (one to four rows, rows of the operand in LDS)
+        if (!off && dtype == MRS_F32 && batch <= 4 && dm % 128 == 0 && di % 128 == 0 && (int64_t)di * 16 <= 48 * 1024 &&
+            getenv("MRS_DECODE_NO_ROWWISE") == nullptr)
+            bb->skinny = 1;
     }
     int *flag = nullptr;
     MRS_CREATE_TRY(dev_alloc(bb, (void **)&flag, sizeof(int)));

@@ -53,9 +53,16 @@ template <> struct Dot2<f16_t> {
         return __builtin_amdgcn_fdot2(__builtin_bit_cast(v2h, a), __builtin_bit_cast(v2h, b), c, false);
     }
 };
+// the products of one 16-byte piece of each operand: 8 elements of a 16-bit type (four v_dot2), 4 of f32
 template <typename T> __device__ __forceinline__ float dot8(uint4 a, uint4 b, float c) {
-    c = Dot2<T>::f(a.x, b.x, c); c = Dot2<T>::f(a.y, b.y, c); c = Dot2<T>::f(a.z, b.z, c);
-    return Dot2<T>::f(a.w, b.w, c);
+    if constexpr (sizeof(T) == 4) {
+        c = fmaf(__uint_as_float(a.x), __uint_as_float(b.x), c); c = fmaf(__uint_as_float(a.y), __uint_as_float(b.y), c);
+        c = fmaf(__uint_as_float(a.z), __uint_as_float(b.z), c);
+        return fmaf(__uint_as_float(a.w), __uint_as_float(b.w), c);
+    } else {
+        c = Dot2<T>::f(a.x, b.x, c); c = Dot2<T>::f(a.y, b.y, c); c = Dot2<T>::f(a.z, b.z, c);
+        return Dot2<T>::f(a.w, b.w, c);
+    }
 }
 
 template <typename TO> __device__ __forceinline__ void store_out(TO *p, float v) { Store<TO>::st(p, v); }
@@ -99,6 +106,7 @@ __global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu
     v4f acc = {0.f, 0.f, 0.f, 0.f};
     // Rows past M / columns past N are clamped to the last valid one: their products land in
     // accumulator elements that are never stored.
+    constexpr int EPV = 16 / (int)sizeof(T);   // elements per 16-byte piece
     const T *wrow = Wt + (int64_t)min(n0 + lr, N - 1) * K + 8 * lg;
     const T *arow = A + (int64_t)min(m0 + lr, M - 1) * lda + 8 * lg;
     float inv = 1.0f;
@@ -152,10 +160,10 @@ __global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu
         constexpr int NC = LPR == 64 ? 2 : 1;           // columns a lane works on (with 32 lanes per row each half-wave has its own)
         constexpr int JB = LPR == 64 ? 2 : 4;             // pieces per column requested together
         const int ll = l & (LPR - 1), half = LPR == 64 ? 0 : (l >> 5);
-        const int per = (K >> 3) / LPR;                 // 16-byte pieces of a row per lane
+        const int per = (K / EPV) / LPR;                 // 16-byte pieces of a row per lane
         const T *wp[NC];
 #pragma unroll
-        for (int t = 0; t < NC; t++) wp[t] = Wt + (int64_t)min(n0 + 2 * w + (LPR == 64 ? t : half), N - 1) * K + 8 * ll;
+        for (int t = 0; t < NC; t++) wp[t] = Wt + (int64_t)min(n0 + 2 * w + (LPR == 64 ? t : half), N - 1) * K + EPV * ll;
         float sum[NC][MR];
 #pragma unroll
         for (int t = 0; t < NC; t++)
@@ -169,10 +177,10 @@ __global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu
 #pragma unroll
                 for (int j = 0; j < J1; j++) {
                     if (jb + j < per) {
-                        const int off = 8 * LPR * (jb + j);
+                        const int off = EPV * LPR * (jb + j);
 #pragma unroll
                         for (int t = 0; t < NC; t++) wv[t][j] = *reinterpret_cast<const uint4 *>(wp[t] + off);
-                        av[j] = *reinterpret_cast<const uint4 *>(A + 8 * ll + off);
+                        av[j] = *reinterpret_cast<const uint4 *>(A + EPV * ll + off);
                     }
                 }
 #pragma unroll
@@ -186,11 +194,11 @@ __global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu
         } else {
         // two to four rows go through LDS once per workgroup: read per wave from memory they would add M/2 times the
         // weight bytes to what the workgroup pulls through its L1, which is what bounds this kernel
-        extern __shared__ uint4 a_lds[];                // [MR][K / 8]
-        const int kq = K >> 3;
+        extern __shared__ uint4 a_lds[];                // [MR][K / EPV]
+        const int kq = K / EPV;
         for (int i = tid; i < MR * kq; i += kGemmWaves * 64) {
             const int m = i / kq, q = i - m * kq;
-            a_lds[i] = *reinterpret_cast<const uint4 *>(A + (int64_t)min(m, M - 1) * lda + 8 * q);
+            a_lds[i] = *reinterpret_cast<const uint4 *>(A + (int64_t)min(m, M - 1) * lda + EPV * q);
         }
         // the first round of weight loads is issued before the barrier that publishes the rows
         uint4 wv[NC][JB];
@@ -198,7 +206,7 @@ __global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu
         for (int j = 0; j < JB; j++)
             if (j < per) {
 #pragma unroll
-                for (int t = 0; t < NC; t++) wv[t][j] = *reinterpret_cast<const uint4 *>(wp[t] + 8 * LPR * j);
+                for (int t = 0; t < NC; t++) wv[t][j] = *reinterpret_cast<const uint4 *>(wp[t] + EPV * LPR * j);
             }
         lds_barrier();   // the rows are in LDS; the weight loads above stay in flight
         for (int jb = 0; jb < per; jb += JB) {
@@ -207,7 +215,7 @@ __global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu
             for (int j = 0; j < JB; j++)
                 if (jb + JB + j < per) {
 #pragma unroll
-                    for (int t = 0; t < NC; t++) nx[t][j] = *reinterpret_cast<const uint4 *>(wp[t] + 8 * LPR * (jb + JB + j));
+                    for (int t = 0; t < NC; t++) nx[t][j] = *reinterpret_cast<const uint4 *>(wp[t] + EPV * LPR * (jb + JB + j));
                 }
 #pragma unroll
             for (int j = 0; j < JB; j++) {
@@ -236,7 +244,7 @@ __global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu
                 if (ll == 0) gv[m][2 * w + (LPR == 64 ? t : half)] = v;
             }
         lds_barrier();
-    } else {
+    } else if constexpr (sizeof(T) == 2) {
     // Two half-batches of fragments: the next one is requested as soon as the current one has been multiplied, so a
     // long K (wide models: 20 k-steps per wave at K = 5120) streams instead of draining after every round of loads.
     constexpr int kHalf = kStepsPerBatch / 2;
@@ -464,10 +472,13 @@ static int launch_skinny_t(hipStream_t st, TO *C, int64_t ldc, const T *A, int64
     SkinnyEpi ep = ep_in;
     const dim3 block(kGemmWaves * 64);
     // one to four rows: the lanes-along-the-row route (64 lanes per weight row when a row is a multiple of 1 KB, else 32)
+    constexpr int EPV = 16 / (int)sizeof(T);   // elements per 16-byte piece
     static const bool no_rowwise = getenv("MRS_DECODE_NO_ROWWISE") != nullptr;
-    int lpr = (M > 4 || no_rowwise || (int64_t)K * 8 > 48 * 1024) ? 0 : (K % 512 == 0 ? 64 : (K % 256 == 0 ? 32 : 0));   // rows fit in LDS
+    int lpr = (M > 4 || no_rowwise || (int64_t)K * 4 * sizeof(T) > 48 * 1024) ? 0   // four rows must fit in LDS
+                                                                               : (K % (64 * EPV) == 0 ? 64 : (K % (32 * EPV) == 0 ? 32 : 0));
     const int ksplit = (ep.mode == 0 && ep.ksplit > 1) ? ep.ksplit : 1;
     if (ksplit > 1) lpr = 0;   // a split K runs on the matrix-core route at any row count
+    if (sizeof(T) == 4 && lpr == 0) return fail(MRS_E_SHAPE, "skinny gemm: f32 storage runs on the row-wise route only (M <= 4, K %% 128 == 0, no K split)");
     if (ksplit > 1 && (ep.row_scale || !ep.xpart || ksplit > (K >> 5)))
         return fail(MRS_E_SHAPE, "skinny gemm: K split needs the matrix-core route, a plain product, a share buffer and ksplit <= K / 32 (ksplit=%d)", ksplit);
     ep.kslice = ((K >> 5) + ksplit - 1) / ksplit;
@@ -475,11 +486,11 @@ static int launch_skinny_t(hipStream_t st, TO *C, int64_t ldc, const T *A, int64
 #define MRS_SG(EPI_, PRO_)                                                                                                               \
     do {                                                                                                                                 \
         if (lpr == 64 && M == 1) hipLaunchKernelGGL((skinny_gemm_kernel<T, TO, EPI_, PRO_, 64, 1>), grid, block, 0, st, C, ldc, A, lda, Wt, M, N, K, ep); \
-        else if (lpr == 64 && M == 2) hipLaunchKernelGGL((skinny_gemm_kernel<T, TO, EPI_, PRO_, 64, 2>), grid, block, (size_t)K * 4, st, C, ldc, A, lda, Wt, M, N, K, ep); \
-        else if (lpr == 32 && M == 2) hipLaunchKernelGGL((skinny_gemm_kernel<T, TO, EPI_, PRO_, 32, 2>), grid, block, (size_t)K * 4, st, C, ldc, A, lda, Wt, M, N, K, ep); \
-        else if (lpr == 64) hipLaunchKernelGGL((skinny_gemm_kernel<T, TO, EPI_, PRO_, 64, 4>), grid, block, (size_t)K * 8, st, C, ldc, A, lda, Wt, M, N, K, ep);     \
+        else if (lpr == 64 && M == 2) hipLaunchKernelGGL((skinny_gemm_kernel<T, TO, EPI_, PRO_, 64, 2>), grid, block, (size_t)K * 2 * sizeof(T), st, C, ldc, A, lda, Wt, M, N, K, ep); \
+        else if (lpr == 32 && M == 2) hipLaunchKernelGGL((skinny_gemm_kernel<T, TO, EPI_, PRO_, 32, 2>), grid, block, (size_t)K * 2 * sizeof(T), st, C, ldc, A, lda, Wt, M, N, K, ep); \
+        else if (lpr == 64) hipLaunchKernelGGL((skinny_gemm_kernel<T, TO, EPI_, PRO_, 64, 4>), grid, block, (size_t)K * 4 * sizeof(T), st, C, ldc, A, lda, Wt, M, N, K, ep);     \
         else if (lpr == 32 && M == 1) hipLaunchKernelGGL((skinny_gemm_kernel<T, TO, EPI_, PRO_, 32, 1>), grid, block, 0, st, C, ldc, A, lda, Wt, M, N, K, ep); \
-        else if (lpr == 32) hipLaunchKernelGGL((skinny_gemm_kernel<T, TO, EPI_, PRO_, 32, 4>), grid, block, (size_t)K * 8, st, C, ldc, A, lda, Wt, M, N, K, ep);     \
+        else if (lpr == 32) hipLaunchKernelGGL((skinny_gemm_kernel<T, TO, EPI_, PRO_, 32, 4>), grid, block, (size_t)K * 4 * sizeof(T), st, C, ldc, A, lda, Wt, M, N, K, ep);     \
         else hipLaunchKernelGGL((skinny_gemm_kernel<T, TO, EPI_, PRO_>), grid, block, 0, st, C, ldc, A, lda, Wt, M, N, K, ep);           \
     } while (0)
     const bool pro = ep.row_scale != 0;
@@ -495,6 +506,9 @@ static int launch_skinny_t(hipStream_t st, TO *C, int64_t ldc, const T *A, int64
 }
 
 bool skinny_gemm_ok(int dtype, int M, int N, int K, int64_t lda, const void *A, const void *Wt) {
+    if (dtype == MRS_F32)   // row-wise route only: one to four rows, K a multiple of 32 lanes x 4 elements, rows that fit in LDS
+        return M >= 1 && M <= 4 && N >= 1 && K >= 128 && K % 128 == 0 && (int64_t)K * 16 <= 48 * 1024 && lda % 4 == 0 && aligned(A, 16) &&
+               aligned(Wt, 16) && getenv("MRS_DECODE_NO_ROWWISE") == nullptr;
     return (dtype == MRS_BF16 || dtype == MRS_F16) && M >= 1 && M <= 64 && N >= 1 && K >= 32 && K % 32 == 0 && lda % 8 == 0 &&
            aligned(A, 16) && aligned(Wt, 16);
 }
@@ -502,8 +516,9 @@ bool skinny_gemm_ok(int dtype, int M, int N, int K, int64_t lda, const void *A, 
 int launch_skinny_gemm(hipStream_t st, int dtype, void *C, int out_f32, int64_t ldc, const void *A, int64_t lda, const void *Wt,
                        int M, int N, int K, const SkinnyEpi &ep) {
     if (!skinny_gemm_ok(dtype, M, N, K, lda, A, Wt))
-        return fail(MRS_E_SHAPE, "skinny gemm: needs 16-bit storage, 1 <= M <= 64, K %% 32 == 0, lda %% 8 == 0, 16-byte aligned A and Wt "
-                                 "(got dtype=%d M=%d N=%d K=%d lda=%lld)", dtype, M, N, K, (long long)lda);
+        return fail(MRS_E_SHAPE, "skinny gemm: needs 16-bit storage with 1 <= M <= 64, K %% 32 == 0, lda %% 8 == 0, or f32 storage with M <= 4, "
+                                 "K %% 128 == 0, lda %% 4 == 0; 16-byte aligned A and Wt (got dtype=%d M=%d N=%d K=%d lda=%lld)", dtype, M, N, K,
+                    (long long)lda);
     if (ep.mode == 1 && (ep.dc < 1 || ep.dc > kMaxConvTaps || ep.di < 1 || ep.di > N || !ep.conv_state || !ep.conv_w || !ep.conv_b || !ep.u))
         return fail(MRS_E_SHAPE, "skinny gemm: bad in_proj epilogue (di=%d dc=%d)", ep.di, ep.dc);
     if (ep.mode == 1 && ep.xw && (ep.xd < 1 || ep.di % 16 != 0 || !ep.xpart))
@@ -512,6 +527,7 @@ int launch_skinny_gemm(hipStream_t st, int dtype, void *C, int out_f32, int64_t 
         return fail(MRS_E_SHAPE, "skinny gemm: bad out_proj epilogue (n_partials=%d, column tiles=%d)", ep.n_partials, (N + 15) / 16);
     if (ep.row_scale && (!ep.partials || ep.n_partials < 1))
         return fail(MRS_E_SHAPE, "skinny gemm: row scale without partial sums");
+    if (dtype == MRS_F32) return launch_skinny_t<float, float>(st, (float *)C, ldc, (const float *)A, lda, (const float *)Wt, M, N, K, ep);
     if (dtype == MRS_BF16) {
         if (out_f32) return launch_skinny_t<bf16_t, float>(st, (float *)C, ldc, (const bf16_t *)A, lda, (const bf16_t *)Wt, M, N, K, ep);
         return launch_skinny_t<bf16_t, bf16_t>(st, (bf16_t *)C, ldc, (const bf16_t *)A, lda, (const bf16_t *)Wt, M, N, K, ep);
@@ -524,7 +540,7 @@ int launch_prenorm_rows(hipStream_t st, int dtype, float *partials, int n_partia
                         const float *w, int M, int K) {
     if (dtype == MRS_BF16) hipLaunchKernelGGL((prenorm_rows_kernel<bf16_t>), dim3((unsigned)M), dim3(256), 0, st, partials, n_partials, (bf16_t *)prenorm, x, copy_to, w, K);
     else if (dtype == MRS_F16) hipLaunchKernelGGL((prenorm_rows_kernel<f16_t>), dim3((unsigned)M), dim3(256), 0, st, partials, n_partials, (f16_t *)prenorm, x, copy_to, w, K);
-    else return fail(MRS_E_DTYPE, "prenorm rows: 16-bit storage only");
+    else hipLaunchKernelGGL((prenorm_rows_kernel<float>), dim3((unsigned)M), dim3(256), 0, st, partials, n_partials, (float *)prenorm, x, copy_to, w, K);
     return check_launch("prenorm_rows_kernel");
 }
 

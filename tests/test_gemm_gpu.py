@@ -35,6 +35,22 @@ def test_gemm_skinny_matches_f64_matmul(shape, dtype, out_f32):
     assert_close(host(c), ref, orc.F32 if out_f32 else dtype, "C")
 
 
+@pytest.mark.parametrize("shape", [(1, 300, 256), (1, 3072, 768), (2, 40, 512), (3, 33, 128), (4, 1536, 1536), (4, 7, 384)])
+def test_gemm_skinny_f32_storage_on_the_row_wise_route(shape):
+    """f32 operands: one to four rows, lanes along the weight row, plain multiply-adds (K a multiple of 128)."""
+    M, N, K = shape
+    rng = np.random.default_rng(M * 1000 + N)
+    a = rng.standard_normal((M, K)).astype(np.float32)
+    w = (rng.standard_normal((K, N)) / np.sqrt(K)).astype(np.float32)
+    print(f"case gemm_skinny f32 shape={shape}", flush=True)
+    wt = ops.transpose(dev(w))
+    c = ops.gemm_skinny(dev(a), wt)
+    assert_close(host(c), a.astype(np.float64) @ w.astype(np.float64), orc.F32, "C")
+    from mamba_rs_amd import MambaHipError
+    with pytest.raises(MambaHipError):   # five rows: f32 has no matrix-core route
+        ops.gemm_skinny(dev(rng.standard_normal((5, K)).astype(np.float32)), wt)
+
+
 def test_gemm_skinny_strided_rows_and_f32_transpose():
     """A may be a view into wider rows (e.g. a slice of a projection); transpose also serves f32 tables."""
     rng = np.random.default_rng(3)
