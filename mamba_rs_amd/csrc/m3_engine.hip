@@ -12,8 +12,9 @@
 //      registers, y = H q + D x, and the SiLU gate (optionally RMSNormGated over the head) -- the formulas of
 //      mamba3_layer_step (src/mamba3_siso/cpu/inference.rs:68-258) and kernels/mamba3_ops.cu;
 //   3. out_proj with the residual add, the next layer's pre-scaled operand and row sums of squares as epilogue.
-// f32 storage (or shapes the skinny GEMM does not take) runs RMSNorm + rocBLAS GEMMs around the same step kernel.
+// Shapes the skinny GEMM does not take (f32 storage above four rows among them) run RMSNorm + rocBLAS GEMMs around the same step kernel.
 #include "common.hpp"
+#include <stdlib.h>
 #include "glue.hpp"
 #include <rocblas/rocblas.h>
 #include <new>
@@ -664,6 +665,9 @@ extern "C" int mrs_m3_backbone_create(mrs_m3_backbone **out, int gpu_ordinal, co
     }
     const int dm = cfg->d_model, di = bb->di, ip = bb->ip, L = cfg->n_layers;
     bb->skinny = (dtype == MRS_BF16 || dtype == MRS_F16) && batch <= 64 && dm % 32 == 0 && di % 32 == 0;
+    // f32 storage: the row-wise route of the same GEMM, one to four rows
+    if (dtype == MRS_F32 && batch <= 4 && dm % 128 == 0 && di % 128 == 0 && (int64_t)di * 16 <= 48 * 1024 && getenv("MRS_DECODE_NO_ROWWISE") == nullptr)
+        bb->skinny = 1;
     float *stage = nullptr;
     {
         size_t big = (size_t)dm * ip;

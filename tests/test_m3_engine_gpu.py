@@ -75,6 +75,28 @@ def test_f32_engine_steps_match_cpu_reference_path(ci):
     eng.close()
 
 
+@pytest.mark.parametrize("B", [1, 3])
+def test_f32_engine_on_the_own_gemm_chain_matches_cpu_reference_path(B):
+    """d_model and d_inner multiples of 128, one to four rows: the f32 engine takes the three-kernel layer (row-wise
+    GEMM route on 4-byte operands) instead of the library chain; same bar as the library chain, eager and replayed."""
+    cfg = Mamba3Config(d_model=128, d_state=32, expand=2, headdim=32, ngroups=1, n_layers=2, rope_fraction=0.5)
+    w = perturbed(cfg, 40, 77)
+    P = oracle_params(w, cfg, 40)
+    eng = GpuMamba3Backbone.new(0, w, cfg, 40, B)
+    st = [P.zero_state() for _ in range(B)]
+    rng = np.random.default_rng(B)
+    x = rng.standard_normal((48, B, 40)).astype(np.float32)
+    worst = 0.0
+    for t in range(48):
+        if t == 16:
+            eng.capture_graph()
+        got = eng.step(x[t])
+        for b in range(B):
+            worst = max(worst, scaled_err(got[b], orc.m3_backbone_step(P, x[t, b], st[b])))
+    assert worst < 2e-4, worst
+    eng.close()
+
+
 def test_batch_rows_are_independent_and_graph_equals_eager():
     cfg = CONFIGS[0]
     w = perturbed(cfg, 64, 5)
