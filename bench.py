@@ -217,6 +217,36 @@ def c1_leg():
             "cpu_port_decode_us_per_step": tcs * 1e6, "prefill_last_step_max_rel_diff_gpu_vs_cpu_port": err}
 
 
+def default_configs_leg():
+    """The reference's two default configurations (MambaConfig::default: d_model 128, 3 layers, src/config.rs:174-186;
+    Mamba3Config::default: d_model 128, 4 layers, headdim 16, src/mamba3_siso/config.rs:132-150), f32, one step in a
+    hipGraph: the quantity behind the reference's published "GPU step" figures (docs/mamba1-benchmarks.md:111-115,
+    docs/mamba3-benchmarks.md:16; other hardware, quoted beside ours, never a ratio)."""
+    import numpy as np
+    from mamba_rs_amd import GpuMambaBackbone, GpuMamba3Backbone, MambaConfig, MambaWeights, Mamba3Config, Mamba3Weights
+
+    def run(eng, x, n=400):
+        eng.step(x); eng.capture_graph()
+        for _ in range(10):
+            eng.step_gpu_only()
+        eng.sync()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            eng.step_gpu_only()
+        eng.sync()
+        eng.close()
+        return (time.perf_counter() - t0) / n * 1e6
+
+    out = {"published_rtx6000ada_us": {"m1_b1_graph": 79, "m1_b128_graph": 139, "m3_b1_graph": 87}}
+    c1 = MambaConfig(d_model=128, d_state=16, d_conv=4, expand=2, n_layers=3)
+    c3 = Mamba3Config(d_model=128, d_state=16, expand=2, headdim=16, ngroups=1, n_layers=4, rope_fraction=0.5, a_floor=1e-4)
+    for B in (1, 128):
+        x = np.random.default_rng(B).standard_normal((B, 128)).astype(np.float32)
+        out[f"m1_step_us_b{B}"] = run(GpuMambaBackbone.new(0, MambaWeights.init(c1, 128, 42), c1, 128, B), x)
+        out[f"m3_step_us_b{B}"] = run(GpuMamba3Backbone.new(0, Mamba3Weights.init(c3, 128, 42), c3, 128, B), x)
+    return out
+
+
 def m1_kernels_leg():
     """The other Mamba-1 kernels of the path at the 130m shape (bf16 storage), each against its HBM roofline:
     causal conv1d + SiLU over batch 8 x T 2048 reading the x half of in_proj's rows in place, and the decode
@@ -432,6 +462,7 @@ def main():
         extras = {}
         if "c1" in legs:
             extras["tiny_f32_cpu_config"] = c1_leg()
+            extras["reference_default_configs_f32"] = default_configs_leg()
         if "lm" in legs:
             extras["lm_130m_shape_bf16"] = lm_leg("130m-shape", dict(d_model=768, d_state=16, d_conv=4, expand=2, n_layers=24), 50280,
                                                   (8, 2048), [64, 1], 256)
