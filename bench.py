@@ -237,13 +237,31 @@ def default_configs_leg():
         eng.close()
         return (time.perf_counter() - t0) / n * 1e6
 
-    out = {"published_rtx6000ada_us": {"m1_b1_graph": 79, "m1_b128_graph": 139, "m3_b1_graph": 87}}
+    out = {"published_rtx6000ada": {"m1_step_us_b1_graph": 79, "m1_step_us_b128_graph": 139, "m3_step_us_b1_graph": 87,
+                                    "m3_synthetic_lm_tok_per_s_graph": {"f32": 5778, "bf16": 5824}}}
     c1 = MambaConfig(d_model=128, d_state=16, d_conv=4, expand=2, n_layers=3)
     c3 = Mamba3Config(d_model=128, d_state=16, expand=2, headdim=16, ngroups=1, n_layers=4, rope_fraction=0.5, a_floor=1e-4)
     for B in (1, 128):
         x = np.random.default_rng(B).standard_normal((B, 128)).astype(np.float32)
         out[f"m1_step_us_b{B}"] = run(GpuMambaBackbone.new(0, MambaWeights.init(c1, 128, 42), c1, 128, B), x)
         out[f"m3_step_us_b{B}"] = run(GpuMamba3Backbone.new(0, Mamba3Weights.init(c3, 128, 42), c3, 128, B), x)
+    # the reference's synthetic Mamba-3 LM (tests/bench_bf16_vs_f32.rs:148-215: d_model 256, 8 layers, headdim 16, vocab 256,
+    # a_floor 0.0625; prompt [1..5], 100 greedy tokens, second run timed)
+    from mamba_rs_amd import GpuMamba3LM, SampleParams, WeightDtype
+    cl = Mamba3Config(d_model=256, d_state=16, expand=2, headdim=16, ngroups=1, n_layers=8, rope_fraction=0.5, a_floor=0.0625)
+    wl = Mamba3Weights.init(cl, 256, 0xB00B)
+    wl.input_proj_w = np.zeros(0, np.float32); wl.input_proj_b = np.zeros(0, np.float32)   # the LM feeds embeddings straight in
+    embed = ((np.random.default_rng(0xBEEF).random((256, 256), dtype=np.float32) - np.float32(0.5)) * np.float32(0.1))
+    sp = SampleParams(temperature=0.0, max_tokens=100)
+    lm_out = {}
+    for name, dt in (("f32", WeightDtype.F32), ("bf16", WeightDtype.BF16)):
+        bb = GpuMamba3Backbone.new_with_dtype(0, wl, cl, 256, 1, dt)
+        lm = GpuMamba3LM(bb, embed)
+        lm.generate([1, 2, 3, 4, 5], params=sp)
+        t0 = time.perf_counter(); toks = lm.generate([1, 2, 3, 4, 5], params=sp); dt_s = time.perf_counter() - t0
+        lm_out[name] = len(toks) / dt_s
+        lm.close(); bb.close()
+    out["m3_synthetic_lm_tok_per_s"] = lm_out
     return out
 
 
