@@ -265,6 +265,54 @@ def default_configs_leg():
     return out
 
 
+def published_configs_leg():
+    """Configurations the reference publishes end-to-end figures for (docs/mamba1-benchmarks.md:23, 52-54, 77; measured
+    there on an RTX 6000 Ada with real checkpoints; random-init weights of the same shapes here): 130m greedy decode at
+    batch 1 in f32 and at batch 16 in bf16, and the 370m-shape parallel-scan prefill of one prompt of 256 / 1024 / 4096
+    tokens in bf16."""
+    import numpy as np
+    from mamba_rs_amd import GpuMambaBackbone, GpuMambaLM, MambaConfig, MambaWeights, WeightDtype
+    vocab = 50280
+    rng = np.random.default_rng(11)
+    out = {"published_rtx6000ada": {"130m_decode_tok_per_s_b1": {"f32": 725, "bf16": 1029}, "130m_bf16_decode_tok_per_s_b16_total": 5026,
+                                    "370m_bf16_prefill_ms": {"256": 31.8, "1024": 87.9, "4096": 328.8}}}
+    cfg = MambaConfig(d_model=768, d_state=16, d_conv=4, expand=2, n_layers=24)
+    w = MambaWeights.random_lm(cfg, 42)
+    embed = (rng.standard_normal((vocab, cfg.d_model), dtype=np.float32) * np.float32(0.02))
+    for key, dt, B in (("130m_f32_decode_b1", WeightDtype.F32, 1), ("130m_bf16_decode_b16", WeightDtype.BF16, 16)):
+        dec = GpuMambaBackbone.new_with_dtype(0, w, cfg, cfg.d_model, B, dt)
+        lm = GpuMambaLM(dec, embed)
+        lm.set_tokens(rng.integers(0, vocab, B).astype(np.int32))
+        lm.capture_graph()
+        for _ in range(8):
+            lm.decode_step()
+        dec.sync()
+        t0 = time.perf_counter()
+        for _ in range(128):
+            lm.decode_step()
+        dec.sync()
+        td = (time.perf_counter() - t0) / 128
+        out[key] = {"us_per_step": td * 1e6, "tok_per_s_total": B / td}
+        lm.close(); dec.close()
+    c370 = MambaConfig(d_model=1024, d_state=16, d_conv=4, expand=2, n_layers=48)
+    w370 = MambaWeights.random_lm(c370, 43)
+    e370 = (rng.standard_normal((vocab, 1024), dtype=np.float32) * np.float32(0.02))
+    pre = {}
+    for T in (256, 1024, 4096):
+        eng = GpuMambaBackbone.new_with_dtype(0, w370, c370, 1024, 1, WeightDtype.BF16)
+        lm = GpuMambaLM(eng, e370)
+        toks = rng.integers(0, vocab, (1, T)).astype(np.int32)
+        lm.prefill(toks); eng.sync()
+        times = []
+        for _ in range(3):
+            eng.reset(); eng.sync()
+            t0 = time.perf_counter(); lm.prefill(toks); eng.sync(); times.append(time.perf_counter() - t0)
+        pre[str(T)] = sorted(times)[1] * 1e3
+        lm.close(); eng.close()
+    out["370m_bf16_prefill_ms_b1"] = pre
+    return out
+
+
 def m1_kernels_leg():
     """The other Mamba-1 kernels of the path at the 130m shape (bf16 storage), each against its HBM roofline:
     causal conv1d + SiLU over batch 8 x T 2048 reading the x half of in_proj's rows in place, and the decode
@@ -435,11 +483,11 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch one 256 MiB device copy (a known-size kernel to scale rocprof FETCH_SIZE/WRITE_SIZE by)")
     ap.add_argument("--big", action="store_true", help="also run the 2.8b-shape LM leg (several minutes of host-side init)")
-    ap.add_argument("--legs", default="c1,lm,m1_kernels,m3,m3_engine",
-                    help="comma list of the extras to run: c1, lm, m1_kernels, m3, m3_engine (for profiling one leg at a time)")
+    ap.add_argument("--legs", default="c1,lm,published,m1_kernels,m3,m3_engine",
+                    help="comma list of the extras to run: c1, lm, published, m1_kernels, m3, m3_engine (for profiling one leg at a time)")
     args = ap.parse_args()
     legs = {x.strip() for x in args.legs.split(",") if x.strip()}
-    unknown = legs - {"c1", "lm", "m1_kernels", "m3", "m3_engine"}
+    unknown = legs - {"c1", "lm", "published", "m1_kernels", "m3", "m3_engine"}
     if unknown:
         print(f"bench.py: unknown --legs entries {sorted(unknown)}", file=sys.stderr)
         sys.exit(2)
@@ -484,6 +532,8 @@ def main():
         if "lm" in legs:
             extras["lm_130m_shape_bf16"] = lm_leg("130m-shape", dict(d_model=768, d_state=16, d_conv=4, expand=2, n_layers=24), 50280,
                                                   (8, 2048), [64, 1], 256)
+        if "published" in legs:
+            extras["reference_published_configs"] = published_configs_leg()
         if "m1_kernels" in legs:
             extras["m1_kernels_130m_shape_bf16"] = m1_kernels_leg()
         if "m3" in legs or "m3_engine" in legs:

@@ -494,7 +494,8 @@ static int run_layers(mrs_backbone *bb, Scratch *s, int T) {
             }
             // ScanMode::use_parallel picks the route (src/mamba_ssm/gpu/prefill.rs:910-956)
             unsigned flags = MRS_GATE_SILU | (lw.s4d ? MRS_A_S4D_REAL : 0);
-            if (!mrs_scan_use_parallel(bb->cfg.scan_mode, T, ds)) flags |= MRS_FORCE_SEQUENTIAL;
+            // An explicit mode is honoured; in Auto the op picks the kernel itself (same recurrence, same tolerance).
+            if (bb->cfg.scan_mode == MRS_SCAN_SEQUENTIAL) flags |= MRS_FORCE_SEQUENTIAL;
             else if (bb->cfg.scan_mode == MRS_SCAN_PARALLEL && ds == 16 && T >= 64) flags |= MRS_FORCE_PARALLEL;
             MRS_TRY(mrs_ssm_scan_fwd_ex(bb->stream, dt, ssm, s->y, s->delta, s->u, xb + es * dr, xb + es * (dr + ds), xd, lw.a_neg,
                                         lw.D, z, 2 * di, flags, s->scan_ws, s->scan_ws_bytes, B, T, di, ds));

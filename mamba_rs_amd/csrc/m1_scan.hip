@@ -662,8 +662,11 @@ extern "C" int mrs_ssm_scan_fwd_ex(void *stream, int dtype, float *h, void *y, c
     SplitPlan plan = {1, T};
     if (split) {
         plan = make_split_plan(batch, T, d_inner);
-        // the reference's Auto threshold (src/config.rs:21-37): parallel above 256 steps
-        if (plan.nchunk < 2 || (T <= 256 && !(flags & MRS_FORCE_PARALLEL))) split = false;
+        // Up to 256 steps (where the reference's Auto mode takes its serial kernel, src/config.rs:21-37) the single
+        // pass is kept when it fills the machine on its own; with few (batch row, channel tile) pairs the serial walk is
+        // one wave per pair and a memory round trip per step (636 us for 256 steps at batch 1, d_inner 2048).
+        const int64_t pairs = (int64_t)batch * ((d_inner + kWave - 1) / kWave);
+        if (plan.nchunk < 2 || (T <= 256 && pairs >= 1024 && !(flags & MRS_FORCE_PARALLEL))) split = false;
     }
     if ((flags & MRS_FORCE_PARALLEL) && !split && d_state == 16 && T >= 64)
         return fail(MRS_E_WORKSPACE, "mrs_ssm_scan_fwd_ex: MRS_FORCE_PARALLEL needs a workspace and 4-byte aligned B/C rows");

@@ -96,14 +96,23 @@ def test_scan_t_split_route_matches_oracle(shape, dtype, s4d):
 
 
 def test_scan_auto_route_threshold_and_workspace_errors():
-    """T <= 256 stays on the sequential route even with a workspace (src/config.rs:21-37), so it is
-    bitwise equal to the no-workspace call; a short workspace is refused."""
+    """Up to 256 steps (the reference's serial range, src/config.rs:21-37) the single pass is kept when its (batch row,
+    channel tile) pairs fill the machine -- bitwise equal to the no-workspace call -- and MRS_FORCE_SEQUENTIAL keeps it
+    in any case; with few pairs the T-split route runs and agrees to the storage tolerance.  A short workspace is refused."""
     rng = np.random.default_rng(9)
-    inp = quantised(rng, 2, 256, 64, 16, orc.BF16)
-    h0 = np.zeros((2, 64, 16), np.float32)
+    inp = quantised(rng, 16, 64, 4096, 16, orc.BF16)            # 16 x 64 = 1024 pairs
+    h0 = np.zeros((16, 4096, 16), np.float32)
     y_seq, h_seq = run_scan(inp, h0, orc.BF16)
     y_auto, h_auto = run_scan(inp, h0, orc.BF16, split="auto")
     assert np.array_equal(y_seq, y_auto) and np.array_equal(h_seq, h_auto)
+    inp = quantised(rng, 2, 256, 64, 16, orc.BF16)               # 2 pairs
+    h0 = np.zeros((2, 64, 16), np.float32)
+    y_seq, h_seq = run_scan(inp, h0, orc.BF16)
+    y_forced, h_forced = run_scan(inp, h0, orc.BF16, flags=ops.FORCE_SEQUENTIAL, split="auto")
+    assert np.array_equal(y_seq, y_forced) and np.array_equal(h_seq, h_forced)
+    y_auto, h_auto = run_scan(inp, h0, orc.BF16, split="auto")
+    assert_close(y_auto, y_seq, orc.BF16, "y (auto vs sequential)")
+    assert_close(h_auto, h_seq, orc.F32, "h (auto vs sequential)")
     inp = quantised(rng, 2, 512, 64, 16, orc.BF16)
     t = {k: dev(v, orc.BF16 if k in ("u", "delta", "B", "C", "z") else orc.F32) for k, v in inp.items()}
     h = torch.zeros(2, 64, 16, device=DEV); y = torch.empty_like(t["delta"])
