@@ -17,18 +17,38 @@ namespace mrs {
 
 constexpr int kNPL = 16;  // state entries held per lane
 
+// Raw (unconverted) element types, so loads can be issued well ahead of the arithmetic that widens and uses them.
+template <typename T> struct RawElem { using type = uint16_t; };
+template <> struct RawElem<float> { using type = float; };
+__device__ __forceinline__ float widen(float v, const float *) { return v; }
+__device__ __forceinline__ float widen(uint16_t v, const bf16_t *) { return __uint_as_float((uint32_t)v << 16); }
+__device__ __forceinline__ float widen(uint16_t v, const f16_t *) { return (float)__builtin_bit_cast(_Float16, v); }
+template <typename T> __device__ __forceinline__ typename RawElem<T>::type raw_ld(const T *p) {
+    return *reinterpret_cast<const typename RawElem<T>::type *>(p);
+}
+
 // ---------------------------------------------------------------------------
 // Generic sequential kernel.  LPC lanes share one channel, lane g of the group
 // owning states n in [16g, 16g+16); any d_state <= 16*LPC, any d_inner.
 // One wave per (batch row, tile of 64/LPC channels); time runs serially.
+// A wave alone on its SIMD has nothing to hide a memory round trip behind, so
+// time is walked in blocks of 16 steps: the operands of the next block are
+// requested (raw, into registers) before the current block is computed --
+// delta / u / gate per lane, the block's B and C rows spread over the lanes and
+// handed round through LDS.  (One request per step was 2.5 us per step.)
 // ---------------------------------------------------------------------------
+constexpr int kSeqBlock = 16;
 template <typename T, int LPC, bool S4D, int GATE>
 __global__ __launch_bounds__(kWave) void ssm_scan_seq_kernel(
     float *__restrict__ h, T *__restrict__ y, const T *__restrict__ delta, const T *__restrict__ u,
     const T *__restrict__ Bm, const T *__restrict__ Cm, int64_t bc_stride,
     const float *__restrict__ a_neg, const float *__restrict__ Dp, const T *__restrict__ gate,
     int64_t gate_stride, int Tlen, int di, int ds, int tiles) {
+    using raw_t = typename RawElem<T>::type;
     constexpr int CPW = kWave / LPC;
+    constexpr int W = kNPL * LPC;                      // padded row width in LDS
+    constexpr int NBC = kSeqBlock * W / kWave;         // B (and C) elements of a block per lane
+    __shared__ alignas(16) raw_t bc[2][2][kSeqBlock * W];   // [buffer][B | C][step][n]
     const int b = blockIdx.x / tiles;
     const int tile = blockIdx.x - b * tiles;
     const int lane = threadIdx.x;
@@ -48,38 +68,81 @@ __global__ __launch_bounds__(kWave) void ssm_scan_seq_kernel(
     }
     const float a20 = a_neg[(int64_t)dd * ds] * kLog2e;  // S4D: a2[n] = (n+1)*a20
     const float Dd = Dp[dd];
-
     const int64_t row0 = (int64_t)b * Tlen;
-    for (int t = 0; t < Tlen; t++) {
-        const int64_t row = row0 + t;
-        const int64_t i = row * di + dd;
-        const float dl = Store<T>::ld(delta + i);
-        const float uu = Store<T>::ld(u + i);
-        const float du = dl * uu;
-        float acc = (g == 0) ? Dd * uu : 0.0f;
-        const T *Br = Bm + row * bc_stride + n0;
-        const T *Cr = Cm + row * bc_stride + n0;
-        float pw = 0.0f, p1 = 0.0f;
-        if (S4D) {
-            p1 = fast_exp2(dl * a20);
-            pw = (LPC == 1) ? p1 : fast_exp2(dl * a20 * (float)(n0 + 1));
+
+    raw_t rd[kSeqBlock], ru[kSeqBlock], rg[kSeqBlock], nd[kSeqBlock], nu[kSeqBlock], ng[kSeqBlock];
+    raw_t nB[NBC], nC[NBC];
+    auto request = [&](raw_t (&xd)[kSeqBlock], raw_t (&xu)[kSeqBlock], raw_t (&xg)[kSeqBlock], int tb) {
+#pragma unroll
+        for (int s = 0; s < kSeqBlock; s++) {
+            const int64_t row = row0 + min(tb + s, Tlen - 1);   // past the end: the last row again, computed and dropped
+            xd[s] = raw_ld(delta + row * di + dd);
+            xu[s] = raw_ld(u + row * di + dd);
+            if (GATE) xg[s] = raw_ld(gate + row * gate_stride + dd);
         }
 #pragma unroll
-        for (int j = 0; j < kNPL; j++) {
-            const bool nv = (n0 + j) < ds;
-            const float Bn = nv ? Store<T>::ld(Br + j) : 0.0f;
-            const float Cn = nv ? Store<T>::ld(Cr + j) : 0.0f;
-            float da;
-            if (S4D) { da = pw; pw *= p1; }
-            else da = fast_exp2(dl * a2[j]);
-            hs[j] = fmaf(da, hs[j], du * Bn);
-            acc = fmaf(hs[j], Cn, acc);
+        for (int i = 0; i < NBC; i++) {
+            const int e = lane + kWave * i, s = e / W, n = e - s * W;
+            const int64_t row = row0 + min(tb + s, Tlen - 1);
+            const int nn = min(n, ds - 1);                      // padding columns: an in-range element, never used
+            nB[i] = raw_ld(Bm + row * bc_stride + nn);
+            nC[i] = raw_ld(Cm + row * bc_stride + nn);
         }
+    };
+    auto publish = [&](int buf) {
 #pragma unroll
-        for (int m = 1; m < LPC; m <<= 1) acc += __shfl_xor(acc, m, kWave);
-        if (GATE == 1) acc *= Store<T>::ld(gate + row * gate_stride + dd);
-        if (GATE == 2) acc *= silu(Store<T>::ld(gate + row * gate_stride + dd));
-        if (live && g == 0) Store<T>::st(y + i, acc);
+        for (int i = 0; i < NBC; i++) {
+            bc[buf][0][lane + kWave * i] = nB[i];
+            bc[buf][1][lane + kWave * i] = nC[i];
+        }
+    };
+    request(rd, ru, rg, 0);
+    publish(0);
+    int buf = 0;
+    for (int tb = 0; tb < Tlen; tb += kSeqBlock, buf ^= 1) {
+        lds_barrier();   // the block's rows are in LDS (one wave: orders its own LDS traffic, global loads stay in flight)
+        if (tb + kSeqBlock < Tlen) request(nd, nu, ng, tb + kSeqBlock);
+#pragma unroll
+        for (int s = 0; s < kSeqBlock; s++) {
+            const int t = tb + s;
+            if (t < Tlen) {
+                const float dl = widen(rd[s], (const T *)nullptr);
+                const float uu = widen(ru[s], (const T *)nullptr);
+                const float du = dl * uu;
+                float acc = (g == 0) ? Dd * uu : 0.0f;
+                // the lane's 16 B and 16 C values of this step as whole 16-byte LDS reads (read unconditionally, masked
+                // below: a conditional read per element became a branch and a wait per element)
+                struct alignas(16) RawRow { raw_t v[kNPL]; };
+                const RawRow Br = *reinterpret_cast<const RawRow *>(&bc[buf][0][s * W + n0]);
+                const RawRow Cr = *reinterpret_cast<const RawRow *>(&bc[buf][1][s * W + n0]);
+                float pw = 0.0f, p1 = 0.0f;
+                if (S4D) {
+                    p1 = fast_exp2(dl * a20);
+                    pw = (LPC == 1) ? p1 : fast_exp2(dl * a20 * (float)(n0 + 1));
+                }
+#pragma unroll
+                for (int j = 0; j < kNPL; j++) {
+                    const bool nv = (n0 + j) < ds;
+                    const float Bn = nv ? widen(Br.v[j], (const T *)nullptr) : 0.0f;
+                    const float Cn = nv ? widen(Cr.v[j], (const T *)nullptr) : 0.0f;
+                    float da;
+                    if (S4D) { da = pw; pw *= p1; }
+                    else da = fast_exp2(dl * a2[j]);
+                    hs[j] = fmaf(da, hs[j], du * Bn);
+                    acc = fmaf(hs[j], Cn, acc);
+                }
+#pragma unroll
+                for (int m = 1; m < LPC; m <<= 1) acc += __shfl_xor(acc, m, kWave);
+                if (GATE == 1) acc *= widen(rg[s], (const T *)nullptr);
+                if (GATE == 2) acc *= silu(widen(rg[s], (const T *)nullptr));
+                if (live && g == 0) Store<T>::st(y + (row0 + t) * di + dd, acc);
+            }
+        }
+        if (tb + kSeqBlock < Tlen) {
+            publish(buf ^ 1);
+#pragma unroll
+            for (int s = 0; s < kSeqBlock; s++) { rd[s] = nd[s]; ru[s] = nu[s]; rg[s] = ng[s]; }
+        }
     }
     if (live) {
 #pragma unroll
@@ -181,10 +244,6 @@ static SplitWs carve_workspace(float *base, int batch, int Tlen, int di, int nch
     return w;
 }
 
-// Raw (unconverted) element types, so loads can be issued a group of steps ahead
-// of the arithmetic that widens and uses them.
-template <typename T> struct RawElem { using type = uint16_t; };
-template <> struct RawElem<float> { using type = float; };
 // Per-lane activation access through a buffer resource: address = base (scalar
 // registers) + per-step scalar offset + per-lane 32-bit offset, so the row walk costs
 // no vector ALU work.  num_records bounds the slab; offsets here stay below 2^31.
@@ -206,9 +265,6 @@ template <typename T> struct LaneBuf {
         }
     }
 };
-__device__ __forceinline__ float widen(float v, const float *) { return v; }
-__device__ __forceinline__ float widen(uint16_t v, const bf16_t *) { return __uint_as_float((uint32_t)v << 16); }
-__device__ __forceinline__ float widen(uint16_t v, const f16_t *) { return (float)__builtin_bit_cast(_Float16, v); }
 
 // One row of B or C (16 values).  The address is wave-uniform, so these are scalar
 // loads; 16-bit rows come as 8 packed dwords and are unpacked on the scalar ALU.
