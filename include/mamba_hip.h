@@ -226,10 +226,11 @@ typedef struct {            /* MambaWeights, src/weights.rs:51-64 */
 
 /* ---- decode projections --------------------------------------------------------------------
  * The reference sends the decode chain's projections to cuBLAS (gemm_ex call sites
- * src/mamba_ssm/gpu/blas.rs:78-96, 721-737; tied head :709-740).  At batch <= 64 this library runs them
+ * src/mamba_ssm/gpu/blas.rs:78-96, 721-737; tied head :709-740).  At batch <= 128 this library runs them
  * on its own matrix-core kernel over a TRANSPOSED weight.
  *   mrs_gemm_skinny: C[M,N] (row stride ldc; dtype, or f32 when out_f32) = A[M,K] (row stride lda) . Wt[N,K]^T
- *     dtype f16/bf16 only, 1 <= M <= 64, K % 32 == 0, lda % 8 == 0, A and Wt 16-byte aligned; f32 accumulate.
+ *     dtype f16/bf16: 1 <= M <= 128, K % 32 == 0, lda % 8 == 0; f32: 1 <= M <= 4, K % 128 == 0, lda % 4 == 0; A and Wt
+ *     16-byte aligned; f32 accumulate.
  *   mrs_transpose:   Wt[N,K] = W[K,N]^T (any dtype; builds the operand above from the reference's [K,N] layout). */
 MRS_API int mrs_gemm_skinny(void *stream, int dtype, void *C, int out_f32, int64_t ldc, const void *A, int64_t lda,
                             const void *Wt, int M, int N, int K);

@@ -88,7 +88,7 @@ int launch_ssm_step_fused(hipStream_t st, int dtype, float *h, void *y, const vo
 int launch_conv1d_step(hipStream_t st, int dtype, void *out, float *state, const void *new_x, int64_t x_stride,
                        const float *weight, const float *bias, int batch, int d_inner, int d_conv, int apply_silu);
 
-// Skinny (M <= 64) 16-bit GEMM on a transposed weight, with the decode chain's fused prologue / epilogues.
+// Skinny (M <= 128) 16-bit GEMM on a transposed weight, with the decode chain's fused prologue / epilogues.
 struct SkinnyEpi {
     int mode;            // 0: store C
                          // 1: in_proj  -- conv step + SiLU on columns < di, gate columns stored
@@ -118,6 +118,7 @@ struct SkinnyEpi {
     int ksplit;
     int kslice;          // set by the launcher: 32-wide k-steps per slice
 };
+int skinny_max_rows();   // rows the 16-bit matrix-core route takes (128; MRS_SKINNY_MAX_ROWS overrides)
 bool skinny_gemm_ok(int dtype, int M, int N, int K, int64_t lda, const void *A, const void *Wt);
 int launch_skinny_gemm(hipStream_t st, int dtype, void *C, int out_f32, int64_t ldc, const void *A, int64_t lda, const void *Wt,
                        int M, int N, int K, const SkinnyEpi &ep);

@@ -242,10 +242,8 @@ static int fold_rows_max() {
 }
 // ... and only while a row's shares stay small (30 KB at d_inner 1536): at d_inner 5120 they are 245 KB per row, re-read by
 // each of the row's 80 step workgroups (2.8b-shape step at batch 1: 2.13 ms without the fold, 2.68 ms with it)
-static int fold_rows_for(int di, int xd) {
-    const bool small = (int64_t)(di / 16) * xd * (int64_t)sizeof(float) <= 32768;
-    return small ? fold_rows_max() : 0;
-}
+static bool narrow_model(int di, int xd) { return (int64_t)(di / 16) * xd * (int64_t)sizeof(float) <= 32768; }
+static int fold_rows_for(int di, int xd) { return narrow_model(di, xd) ? fold_rows_max() : 0; }
 
 struct Scratch {  // activations for M rows
     int64_t rows = 0;
@@ -263,7 +261,7 @@ struct mrs_backbone {
     mrs_m1_config cfg;
     int input_dim, batch, dtype, di, dr, xd, identity_proj, device;
     const float *step_src;  // decode step: where layer 0 reads its input rows (null: the residual buffer itself)
-    int skinny;  // decode projections on the library's own GEMM (16-bit storage: batch <= 64, K % 32 == 0; f32: batch <= 4, K % 128 == 0)
+    int skinny;  // decode projections on the library's own GEMM (16-bit storage: batch <= 128 or 64, K % 32 == 0; f32: batch <= 4, K % 128 == 0)
     hipStream_t stream;
     rocblas_handle blas;
     std::vector<LayerDev> layers;
@@ -563,7 +561,10 @@ extern "C" int mrs_backbone_create(mrs_backbone **out, int gpu_ordinal, const mr
     bb->layers.resize(L);
     {
         static const bool off = [] { const char *e = getenv("MRS_DECODE_LIBRARY_GEMM"); return e && atoi(e) != 0; }();
-        bb->skinny = !off && (dtype == MRS_BF16 || dtype == MRS_F16) && batch <= 64 && dm % 32 == 0 && di % 32 == 0;
+        // Rows up to which the own chain beats the library chain, measured: 128 at the 130m shape (989 vs 1179 us per step;
+        // at 256 rows 1490 vs 1392), 64 at the 2.8b shape (a tie there).  "Narrow" as for the x_proj shares.
+        const int max_rows = std::min(skinny_max_rows(), narrow_model(di, xd) ? 128 : 64);
+        bb->skinny = !off && (dtype == MRS_BF16 || dtype == MRS_F16) && batch <= max_rows && dm % 32 == 0 && di % 32 == 0;
         // f32 storage: the same chain on the row-wise route of the GEMM (one to four rows, rows of the operand in LDS)
         if (!off && dtype == MRS_F32 && batch <= 4 && dm % 128 == 0 && di % 128 == 0 && (int64_t)di * 16 <= 48 * 1024 &&
             getenv("MRS_DECODE_NO_ROWWISE") == nullptr)

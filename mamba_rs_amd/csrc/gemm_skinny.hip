@@ -1,4 +1,4 @@
-// Skinny GEMM for the decode chain: C[M,N] = A[M,K] . Wt[N,K]^T with M <= 64 rows (the batch),
+// Skinny GEMM for the decode chain: C[M,N] = A[M,K] . Wt[N,K]^T with M <= 128 rows (the batch),
 // 16-bit operands, f32 accumulate on the matrix cores.
 //
 // The reference sends every decode projection to the vendor GEMM (cuBLAS call sites
@@ -505,18 +505,23 @@ static int launch_skinny_t(hipStream_t st, TO *C, int64_t ldc, const T *A, int64
     return check_launch("skinny_gemm_kernel");
 }
 
+int skinny_max_rows() {
+    static const int v = [] { const char *e = getenv("MRS_SKINNY_MAX_ROWS"); const int n = e ? atoi(e) : 128; return n < 1 ? 1 : (n > 1024 ? 1024 : n); }();
+    return v;
+}
+
 bool skinny_gemm_ok(int dtype, int M, int N, int K, int64_t lda, const void *A, const void *Wt) {
     if (dtype == MRS_F32)   // row-wise route only: one to four rows, K a multiple of 32 lanes x 4 elements, rows that fit in LDS
         return M >= 1 && M <= 4 && N >= 1 && K >= 128 && K % 128 == 0 && (int64_t)K * 16 <= 48 * 1024 && lda % 4 == 0 && aligned(A, 16) &&
                aligned(Wt, 16) && getenv("MRS_DECODE_NO_ROWWISE") == nullptr;
-    return (dtype == MRS_BF16 || dtype == MRS_F16) && M >= 1 && M <= 64 && N >= 1 && K >= 32 && K % 32 == 0 && lda % 8 == 0 &&
+    return (dtype == MRS_BF16 || dtype == MRS_F16) && M >= 1 && M <= skinny_max_rows() && N >= 1 && K >= 32 && K % 32 == 0 && lda % 8 == 0 &&
            aligned(A, 16) && aligned(Wt, 16);
 }
 
 int launch_skinny_gemm(hipStream_t st, int dtype, void *C, int out_f32, int64_t ldc, const void *A, int64_t lda, const void *Wt,
                        int M, int N, int K, const SkinnyEpi &ep) {
     if (!skinny_gemm_ok(dtype, M, N, K, lda, A, Wt))
-        return fail(MRS_E_SHAPE, "skinny gemm: needs 16-bit storage with 1 <= M <= 64, K %% 32 == 0, lda %% 8 == 0, or f32 storage with M <= 4, "
+        return fail(MRS_E_SHAPE, "skinny gemm: needs 16-bit storage with 1 <= M <= 128, K %% 32 == 0, lda %% 8 == 0, or f32 storage with M <= 4, "
                                  "K %% 128 == 0, lda %% 4 == 0; 16-byte aligned A and Wt (got dtype=%d M=%d N=%d K=%d lda=%lld)", dtype, M, N, K,
                     (long long)lda);
     if (ep.mode == 1 && (ep.dc < 1 || ep.dc > kMaxConvTaps || ep.di < 1 || ep.di > N || !ep.conv_state || !ep.conv_w || !ep.conv_b || !ep.u))

@@ -154,7 +154,7 @@ def transpose(w):
 
 
 def gemm_skinny(a, wt, *, out_f32: bool = False):
-    """C[M,N] = A[M,K] . Wt[N,K]^T for the decode chain (M <= 64, 16-bit operands, f32 accumulate): the
+    """C[M,N] = A[M,K] . Wt[N,K]^T for the decode chain (M <= 128 with 16-bit operands, M <= 4 with f32; f32 accumulate): the
     projections the reference sends to cuBLAS (src/mamba_ssm/gpu/blas.rs:78-96)."""
     _dev(wt)
     if not a.is_cuda:

@@ -258,6 +258,29 @@ def test_wide_dt_rank_at_large_batch_runs_dt_proj_as_its_own_gemm():
         eng.close()
 
 
+@pytest.mark.parametrize("B", [100, 128])
+def test_narrow_model_keeps_the_own_chain_up_to_128_rows(B):
+    """Above 64 rows (up to 128 for narrow models) the decode chain still runs on the library's own GEMM, with dt_proj as
+    a launch of its own (batch x dt_rank above the fusion limit).  First, middle and last row against the CPU route."""
+    cfg = MambaConfig(d_model=768, d_state=16, d_conv=4, expand=2, n_layers=2)
+    w = MambaWeights.random_lm(cfg, seed=B, std=0.05)
+    P = oracle_params(w, cfg, 768, round_to=orc.BF16)
+    P.input_proj_w[:] = np.eye(768, dtype=np.float32); P.input_proj_b[:] = 0
+    rng = np.random.default_rng(B)
+    eng = GpuMambaBackbone.new_with_dtype(0, w, cfg, 768, B, WeightDtype.BF16)
+    x = rng.standard_normal((4, B, 768)).astype(np.float32)
+    rows = (0, B // 2, B - 1)
+    st = {b: orc.m1_zero_state(P) for b in rows}
+    for t in range(4):
+        if t == 2:
+            eng.capture_graph()
+        got = eng.step(x[t])
+        for b in rows:
+            want = orc.m1_backbone_step(P, x[t, b], *st[b])
+            assert cosine(got[b], want) >= 0.999, (B, t, b)
+    eng.close()
+
+
 @pytest.mark.parametrize("B", [1, 3, 20])
 def test_wide_model_runs_x_proj_as_a_split_k_launch(B):
     """d_inner 2048 x xdbl 96: a row's per-tile shares would be 48 KB, so x_proj does not ride in the in_proj launch; it

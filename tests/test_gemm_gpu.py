@@ -13,7 +13,7 @@ ops = pytest.importorskip("mamba_rs_amd.ops")
 
 # (M, N, K): the 130m decode projections at batch 64 and 1, ragged M / N, the smallest K
 SHAPES = [(64, 3072, 768), (64, 80, 1536), (64, 768, 1536), (1, 3072, 768), (1, 80, 1536), (5, 33, 32), (17, 100, 96),
-          (48, 16, 2560), (33, 1000, 64), (64, 50, 1024),
+          (48, 16, 2560), (33, 1000, 64), (64, 50, 1024), (128, 768, 1536), (97, 80, 1536), (100, 3072, 768),
           # one to four rows: lanes-along-the-row route (64 lanes per weight row at K % 512 == 0, 32 at K % 256 == 0)
           (1, 10240, 2560), (1, 192, 5120), (2, 2560, 5120), (3, 100, 512), (4, 33, 768), (1, 7, 256), (4, 3072, 768), (2, 50, 1280)]
 
@@ -66,9 +66,9 @@ def test_gemm_skinny_strided_rows_and_f32_transpose():
 
 def test_gemm_skinny_rejects_bad_arguments():
     from mamba_rs_amd import MambaHipError
-    a = torch.zeros(65, 64, device=DEV, dtype=torch.bfloat16)
+    a = torch.zeros(129, 64, device=DEV, dtype=torch.bfloat16)
     wt = torch.zeros(16, 64, device=DEV, dtype=torch.bfloat16)
-    with pytest.raises(MambaHipError) as e:   # M > 64
+    with pytest.raises(MambaHipError) as e:   # M > 128
         ops.gemm_skinny(a, wt)
     assert e.value.code == -2
     with pytest.raises(MambaHipError) as e:   # K not a multiple of 32
