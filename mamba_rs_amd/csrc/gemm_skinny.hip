@@ -466,6 +466,11 @@ __global__ __launch_bounds__(256) void transpose_kernel(T *__restrict__ Wt, cons
         if (n0 + r < N && k0 + tx < K) Wt[(int64_t)(n0 + r) * K + k0 + tx] = tile[tx][r];
 }
 
+static bool no_rowwise_route() {
+    static const bool v = getenv("MRS_DECODE_NO_ROWWISE") != nullptr;
+    return v;
+}
+
 template <typename T, typename TO>
 static int launch_skinny_t(hipStream_t st, TO *C, int64_t ldc, const T *A, int64_t lda, const T *Wt, int M, int N, int K,
                            const SkinnyEpi &ep_in) {
@@ -473,7 +478,7 @@ static int launch_skinny_t(hipStream_t st, TO *C, int64_t ldc, const T *A, int64
     const dim3 block(kGemmWaves * 64);
     // one to four rows: the lanes-along-the-row route (64 lanes per weight row when a row is a multiple of 1 KB, else 32)
     constexpr int EPV = 16 / (int)sizeof(T);   // elements per 16-byte piece
-    static const bool no_rowwise = getenv("MRS_DECODE_NO_ROWWISE") != nullptr;
+    const bool no_rowwise = no_rowwise_route();
     int lpr = (M > 4 || no_rowwise || (int64_t)K * 4 * sizeof(T) > 48 * 1024) ? 0   // four rows must fit in LDS
                                                                                : (K % (64 * EPV) == 0 ? 64 : (K % (32 * EPV) == 0 ? 32 : 0));
     const int ksplit = (ep.mode == 0 && ep.ksplit > 1) ? ep.ksplit : 1;
@@ -513,7 +518,7 @@ int skinny_max_rows() {
 bool skinny_gemm_ok(int dtype, int M, int N, int K, int64_t lda, const void *A, const void *Wt) {
     if (dtype == MRS_F32)   // row-wise route only: one to four rows, K a multiple of 32 lanes x 4 elements, rows that fit in LDS
         return M >= 1 && M <= 4 && N >= 1 && K >= 128 && K % 128 == 0 && (int64_t)K * 16 <= 48 * 1024 && lda % 4 == 0 && aligned(A, 16) &&
-               aligned(Wt, 16) && getenv("MRS_DECODE_NO_ROWWISE") == nullptr;
+               aligned(Wt, 16) && !no_rowwise_route();
     return (dtype == MRS_BF16 || dtype == MRS_F16) && M >= 1 && M <= skinny_max_rows() && N >= 1 && K >= 32 && K % 32 == 0 && lda % 8 == 0 &&
            aligned(A, 16) && aligned(Wt, 16);
 }
