@@ -281,20 +281,22 @@ __global__ __launch_bounds__(1024) void m3_angle_apply_kernel(float *__restrict_
     }
 }
 
-// one workgroup (256 threads) per row.  bulk: rows of ldb elements [z:di | x:di | B:ng*ds | C:ng*ds | ...] in the
-// activation type; xout may be null (x is then read in place by the scan).
+// one workgroup (256 threads) per row.  bulk: rows of ldb elements [z:di | x:di | ...] in the activation type; bc: rows
+// of ldbc f32 [B:ng*ds | C:ng*ds | ...] (the projection keeps them in f32, as the decode step sees them); xout may be
+// null (x is then read in place by the scan).
 template <typename T>
 __global__ __launch_bounds__(256) void m3_kq_kernel(
     T *__restrict__ Kout, T *__restrict__ Qout, T *__restrict__ xout, const T *__restrict__ bulk, int64_t ldb,
-    const float *__restrict__ angle, const float *__restrict__ bnw, const float *__restrict__ cnw,
+    const float *__restrict__ bc, int64_t ldbc, const float *__restrict__ angle, const float *__restrict__ bnw, const float *__restrict__ cnw,
     const float *__restrict__ b_bias, const float *__restrict__ c_bias, int nh, int hd, int ng, int ds, int nr, float eps) {
     extern __shared__ float smem[];
     const int di = nh * hd, ngds = ng * ds;
     float *bn = smem, *cn = bn + ngds, *inv = cn + ngds;
     const int64_t r = blockIdx.x;
     const T *row = bulk + r * ldb;
+    const float *bcr = bc + r * ldbc;
     const int tid = threadIdx.x;
-    for (int i = tid; i < ngds; i += 256) { bn[i] = Store<T>::ld(row + 2 * di + i); cn[i] = Store<T>::ld(row + 2 * di + ngds + i); }
+    for (int i = tid; i < ngds; i += 256) { bn[i] = bcr[i]; cn[i] = bcr[ngds + i]; }
     __syncthreads();
     // one wave-sized slice per (B or C, group): 2*ng reductions of ds values
     {
@@ -348,16 +350,17 @@ __global__ __launch_bounds__(256) void m3_kq_kernel(
 template <typename T>
 __global__ __launch_bounds__(256) void m3_kq_rows_kernel(
     T *__restrict__ Kout, T *__restrict__ Qout, T *__restrict__ xout, const T *__restrict__ bulk, int64_t ldb,
-    const float *__restrict__ angle, const float *__restrict__ bnw, const float *__restrict__ cnw,
+    const float *__restrict__ bc, int64_t ldbc, const float *__restrict__ angle, const float *__restrict__ bnw, const float *__restrict__ cnw,
     const float *__restrict__ b_bias, const float *__restrict__ c_bias, int64_t rows, int nh, int hd, int ds, int nr, float eps) {
     const int w = threadIdx.x >> 6, l = threadIdx.x & 63;
     const int64_t r = (int64_t)blockIdx.x * 4 + w;
     if (r >= rows) return;   // whole waves leave; the kernel has no barrier
     const int di = nh * hd;
-    const T *row = bulk + r * ldb, *Bp = row + 2 * di, *Cp = Bp + ds;
+    const T *row = bulk + r * ldb;
+    const float *Bp = bc + r * ldbc, *Cp = Bp + ds;
     float ssb = 0.0f, ssc = 0.0f;
     for (int n = l; n < ds; n += 64) {
-        const float b = Store<T>::ld(Bp + n), c = Store<T>::ld(Cp + n);
+        const float b = Bp[n], c = Cp[n];
         ssb = fmaf(b, b, ssb); ssc = fmaf(c, c, ssc);
     }
 #pragma unroll
@@ -367,14 +370,14 @@ __global__ __launch_bounds__(256) void m3_kq_rows_kernel(
     struct alignas(4 * sizeof(T)) V4 { T v[4]; };
     constexpr int kTrips = 3;   // items of a lane whose operands are requested together
     for (int i0 = l; i0 < items; i0 += 64 * kTrips) {
-        V4 bv[kTrips], cv[kTrips];
+        float4 bv[kTrips], cv[kTrips];
         float4 bw[kTrips], cw[kTrips], bb4[kTrips], cb4[kTrips];
         float ang[kTrips][2];
 #pragma unroll
         for (int t = 0; t < kTrips; t++) {
             const int i = min(i0 + 64 * t, items - 1);   // past the end: an in-range item, computed and dropped
             const int h = i / quarter, j4 = i - h * quarter, n = 4 * j4;
-            bv[t] = *reinterpret_cast<const V4 *>(Bp + n); cv[t] = *reinterpret_cast<const V4 *>(Cp + n);
+            bv[t] = *reinterpret_cast<const float4 *>(Bp + n); cv[t] = *reinterpret_cast<const float4 *>(Cp + n);
             bw[t] = *reinterpret_cast<const float4 *>(bnw + n); cw[t] = *reinterpret_cast<const float4 *>(cnw + n);
             bb4[t] = *reinterpret_cast<const float4 *>(b_bias + h * ds + n); cb4[t] = *reinterpret_cast<const float4 *>(c_bias + h * ds + n);
 #pragma unroll
@@ -385,10 +388,10 @@ __global__ __launch_bounds__(256) void m3_kq_rows_kernel(
             const int i = i0 + 64 * t;
             if (i < items) {
                 const int h = i / quarter, j4 = i - h * quarter, n = 4 * j4;
-                float k[4] = {Store<T>::ld(&bv[t].v[0]) * ib * bw[t].x + bb4[t].x, Store<T>::ld(&bv[t].v[1]) * ib * bw[t].y + bb4[t].y,
-                              Store<T>::ld(&bv[t].v[2]) * ib * bw[t].z + bb4[t].z, Store<T>::ld(&bv[t].v[3]) * ib * bw[t].w + bb4[t].w};
-                float q[4] = {Store<T>::ld(&cv[t].v[0]) * ic * cw[t].x + cb4[t].x, Store<T>::ld(&cv[t].v[1]) * ic * cw[t].y + cb4[t].y,
-                              Store<T>::ld(&cv[t].v[2]) * ic * cw[t].z + cb4[t].z, Store<T>::ld(&cv[t].v[3]) * ic * cw[t].w + cb4[t].w};
+                float k[4] = {bv[t].x * ib * bw[t].x + bb4[t].x, bv[t].y * ib * bw[t].y + bb4[t].y,
+                              bv[t].z * ib * bw[t].z + bb4[t].z, bv[t].w * ib * bw[t].w + bb4[t].w};
+                float q[4] = {cv[t].x * ic * cw[t].x + cb4[t].x, cv[t].y * ic * cw[t].y + cb4[t].y,
+                              cv[t].z * ic * cw[t].z + cb4[t].z, cv[t].w * ic * cw[t].w + cb4[t].w};
 #pragma unroll
                 for (int pr = 0; pr < 2; pr++) {
                     if (2 * j4 + pr < nr) {
@@ -793,8 +796,9 @@ extern "C" int mrs_m3_backbone_alloc_prefill_scratch(mrs_m3_backbone *bb, int T)
     const size_t nrz = bb->nr > 0 ? bb->nr : 1;
     MRS_TRY(dev_alloc3(bb, (void **)&bb->pf_in, rows * bb->input_dim * 4));
     MRS_TRY(dev_alloc3(bb, (void **)&bb->pf_residual, rows * dm * 4));
-    // f32 storage: the whole in_proj result; 16-bit: its f32 scalar columns only, the bulk columns live in pf_bulk
-    const size_t nbulk = 2 * di + 2 * (size_t)c.ngroups * ds;
+    // f32 storage: the whole in_proj result; 16-bit: its f32 columns only (B, C, head scalars, angle inputs), the bulk
+    // columns (z, x) live in pf_bulk
+    const size_t nbulk = 2 * di;
     MRS_TRY(dev_alloc3(bb, (void **)&bb->pf_proj, rows * (bb->dtype == MRS_F32 ? ip : ip - nbulk) * 4));
     MRS_TRY(dev_alloc3(bb, &bb->pf_bulk, bb->dtype == MRS_F32 ? 16 : rows * nbulk * es));
     MRS_TRY(dev_alloc3(bb, (void **)&bb->pf_dt, rows * nh * 4));
@@ -823,19 +827,19 @@ extern "C" int mrs_m3_backbone_alloc_prefill_scratch(mrs_m3_backbone *bb, int T)
 namespace {
 
 template <typename T>
-int launch_kq_t(mrs_m3_backbone *bb, const Layer3 &lw, int64_t rows, const void *bulk, int64_t ldb, bool copy_x) {
+int launch_kq_t(mrs_m3_backbone *bb, const Layer3 &lw, int64_t rows, const void *bulk, int64_t ldb, const float *bc, int64_t ldbc, bool copy_x) {
     const mrs_m3_config &c = bb->cfg;
     const int ng = c.ngroups, ds = c.d_state;
     const size_t lds = (size_t)(2 * ng * ds + 2 * ng) * sizeof(float);
     if (lds > 60000) return fail(MRS_E_SHAPE, "m3 K/Q kernel: ngroups * d_state too large for LDS (%zu bytes)", lds);
-    if (ng == 1 && ds % 4 == 0 && ldb % 4 == 0 && (2 * bb->nh * c.headdim) % 4 == 0) {
+    if (ng == 1 && ds % 4 == 0 && ldbc % 4 == 0 && aligned(bc, 16)) {
         hipLaunchKernelGGL((m3_kq_rows_kernel<T>), dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, bb->stream, (T *)bb->pf_K, (T *)bb->pf_Q,
-                           copy_x ? (T *)bb->pf_x : nullptr, (const T *)bulk, ldb, bb->pf_angle, lw.bnw, lw.cnw, lw.b_bias, lw.c_bias, rows,
+                           copy_x ? (T *)bb->pf_x : nullptr, (const T *)bulk, ldb, bc, ldbc, bb->pf_angle, lw.bnw, lw.cnw, lw.b_bias, lw.c_bias, rows,
                            bb->nh, c.headdim, ds, bb->nr, c.rms_norm_eps);
         return check_launch("m3_kq_rows_kernel");
     }
     hipLaunchKernelGGL((m3_kq_kernel<T>), dim3((unsigned)rows), dim3(256), lds, bb->stream, (T *)bb->pf_K, (T *)bb->pf_Q,
-                       copy_x ? (T *)bb->pf_x : nullptr, (const T *)bulk, ldb, bb->pf_angle, lw.bnw, lw.cnw, lw.b_bias, lw.c_bias, bb->nh,
+                       copy_x ? (T *)bb->pf_x : nullptr, (const T *)bulk, ldb, bc, ldbc, bb->pf_angle, lw.bnw, lw.cnw, lw.b_bias, lw.c_bias, bb->nh,
                        c.headdim, ng, ds, bb->nr, c.rms_norm_eps);
     return check_launch("m3_kq_kernel");
 }
@@ -876,11 +880,13 @@ int prefill_body3(mrs_m3_backbone *bb, int T) {
         float *ssm = bb->ssm + (size_t)l * B * nh * hd * ds, *kst = bb->kst + (size_t)l * B * nh * ds;
         float *vst = bb->vst + (size_t)l * B * nh * hd, *ang = bb->angle + (size_t)l * B * nh * (nr > 0 ? nr : 1);
         MRS_TRY(launch_add_rmsnorm3(bb, bb->pf_residual, l == 0 ? nullptr : bb->pf_out, bb->pf_normed, false, lw.norm_w, rows));
-        // in_proj.  The bulk columns (z, x, B, C) come out in the storage type; the head scalars and angle inputs
-        // (dd_dt, dd_A, trap, angles: the last 3 nh + nr columns) in f32 whatever the storage type -- two GEMMs over
-        // column slices of the same weight for 16-bit storage, one for f32.
-        const int nb = 2 * di + 2 * c.ngroups * ds, ns = ip - nb;
-        const void *bulk; int64_t ldb; const float *scp; int64_t lds_;
+        // in_proj.  The bulk columns (z, x) come out in the storage type; B, C, the head scalars and the angle inputs
+        // (the last 2 ng ds + 3 nh + nr columns) in f32 whatever the storage type, as the decode step sees them -- two
+        // GEMMs over column slices of the same weight for 16-bit storage, one for f32.  (The bulk slice is 2 d_inner wide
+        // on purpose: with B and C in it the 768-wide shape's 3200 columns cost the vendor kernel a third more time
+        // than 3072 do.)
+        const int nb = 2 * di, ns = ip - nb, nbc = 2 * c.ngroups * ds;
+        const void *bulk; int64_t ldb; const float *scp, *bcp; int64_t lds_;
         {
             const float one = 1.0f, zero = 0.0f;
             const rocblas_datatype t = blas_type3(dt);
@@ -888,7 +894,7 @@ int prefill_body3(mrs_m3_backbone *bb, int T) {
                 MRS_BLAS(rocblas_gemm_ex(bb->blas, rocblas_operation_none, rocblas_operation_none, ip, (int)rows, dm, &one, lw.in_proj, t, ip,
                                          bb->pf_normed, t, dm, &zero, bb->pf_proj, t, ip, bb->pf_proj, t, ip, rocblas_datatype_f32_r,
                                          rocblas_gemm_algo_standard, 0, 0));
-                bulk = bb->pf_proj; ldb = ip; scp = bb->pf_proj + nb; lds_ = ip;
+                bulk = bb->pf_proj; ldb = ip; bcp = bb->pf_proj + nb; scp = bcp + nbc; lds_ = ip;
             } else {
                 if (lw.in_proj_t) {   // the vendor kernels for the transposed operand are faster at these shapes (its first nb rows)
                     MRS_BLAS(rocblas_gemm_ex(bb->blas, rocblas_operation_transpose, rocblas_operation_none, nb, (int)rows, dm, &one, lw.in_proj_t,
@@ -899,11 +905,18 @@ int prefill_body3(mrs_m3_backbone *bb, int T) {
                                              bb->pf_normed, t, dm, &zero, bb->pf_bulk, t, nb, bb->pf_bulk, t, nb, rocblas_datatype_f32_r,
                                              rocblas_gemm_algo_standard, 0, 0));
                 }
-                MRS_BLAS(rocblas_gemm_ex(bb->blas, rocblas_operation_none, rocblas_operation_none, ns, (int)rows, dm, &one,
-                                         (const char *)lw.in_proj + (size_t)nb * es, t, ip, bb->pf_normed, t, dm, &zero, bb->pf_proj,
-                                         rocblas_datatype_f32_r, ns, bb->pf_proj, rocblas_datatype_f32_r, ns, rocblas_datatype_f32_r,
-                                         rocblas_gemm_algo_standard, 0, 0));
-                bulk = bb->pf_bulk; ldb = nb; scp = bb->pf_proj; lds_ = ns;
+                if (lw.in_proj_t) {
+                    MRS_BLAS(rocblas_gemm_ex(bb->blas, rocblas_operation_transpose, rocblas_operation_none, ns, (int)rows, dm, &one,
+                                             (const char *)lw.in_proj_t + (size_t)nb * dm * es, t, dm, bb->pf_normed, t, dm, &zero, bb->pf_proj,
+                                             rocblas_datatype_f32_r, ns, bb->pf_proj, rocblas_datatype_f32_r, ns, rocblas_datatype_f32_r,
+                                             rocblas_gemm_algo_standard, 0, 0));
+                } else {
+                    MRS_BLAS(rocblas_gemm_ex(bb->blas, rocblas_operation_none, rocblas_operation_none, ns, (int)rows, dm, &one,
+                                             (const char *)lw.in_proj + (size_t)nb * es, t, ip, bb->pf_normed, t, dm, &zero, bb->pf_proj,
+                                             rocblas_datatype_f32_r, ns, bb->pf_proj, rocblas_datatype_f32_r, ns, rocblas_datatype_f32_r,
+                                             rocblas_gemm_algo_standard, 0, 0));
+                }
+                bulk = bb->pf_bulk; ldb = nb; bcp = bb->pf_proj; scp = bcp + nbc; lds_ = ns;
             }
         }
         {
@@ -926,7 +939,7 @@ int prefill_body3(mrs_m3_backbone *bb, int T) {
         // measured and dropped: the scattered z reads cost the latency-bound kernel 54 us against 28 us for the
         // separate gate pass.)
         const bool in_place = chunked_ok && dt != MRS_F32 && ldb % 8 == 0 && di % 8 == 0;
-        MRS_DISPATCH_DTYPE(dt, T_, MRS_TRY(launch_kq_t<T_>(bb, lw, rows, bulk, ldb, !in_place)));
+        MRS_DISPATCH_DTYPE(dt, T_, MRS_TRY(launch_kq_t<T_>(bb, lw, rows, bulk, ldb, bcp, lds_, !in_place)));
         if (in_place) {
             const char *xb = (const char *)bulk + (size_t)di * es;
             MRS_TRY(m3_ssd_fwd_ex(bb->stream, dt, ssm, kst, vst, bb->pf_y, xb, ldb, bb->pf_K, bb->pf_Q, bb->pf_dt, bb->pf_trap, bb->pf_a, lw.D,
