@@ -30,6 +30,7 @@
 // B[k=4(l/16)..+3][n=l%16], and C/D[m=4(l/16)+i][n=l%16], i = 0..3.
 #include "common.hpp"
 #include <stdlib.h>
+#include <algorithm>
 
 namespace mrs {
 
@@ -38,8 +39,6 @@ typedef short v4s __attribute__((ext_vector_type(4)));
 typedef _Float16 v4h __attribute__((ext_vector_type(4)));
 
 constexpr int kCS = 64;  // chunk size (the reference's CHUNK_SIZE, src/mamba3_siso/gpu/state.rs:97)
-constexpr int kPad = 8;  // halfword padding of LDS rows (keeps rows 16-byte aligned, staggers banks)
-
 template <typename T> struct Mma;
 template <> struct Mma<bf16_t> {
     __device__ static __forceinline__ v4f mma(uint2 a, uint2 b, v4f c) {
@@ -69,19 +68,28 @@ template <> struct Mma<f16_t> {
     }
 };
 
+constexpr int kPad = 8;  // halfword padding of LDS rows: 64-wide rows are 36 dwords, which spreads the 16 rows x 4 dwords that
+                         // half a wave reads as operand fragments over all banks (measured: with 40-dword rows half of
+                         // the LDS cycles of the pass were bank conflicts; an XOR swizzle of unpadded rows gave the same
+                         // conflict count as this padding and cost address arithmetic)
+
 template <int HD, int DS> struct alignas(16) SsdSmem {
-    static constexpr int NW = HD / 16;
     alignas(16) uint16_t Qs[kCS][DS + kPad];       // Q rows
     alignas(16) uint16_t Ks[kCS][DS + kPad];       // K rows
-    alignas(16) uint16_t Kt[DS][kCS + kPad];       // K transposed: Kt[n][t]
-    alignas(16) uint16_t Xt[NW][16][kCS + kPad];   // per wave: x slice transposed, Xt[p][t]
-    alignas(16) float sc[NW][5][kCS];              // per wave: dA, scale, gamma, exp(dA), w
+    alignas(16) uint16_t Xs[kCS][HD + kPad];       // x rows of this head
+    alignas(16) float sc[5][kCS];                  // dA, scale, gamma, exp(dA), w
     alignas(16) uint2 Ps[10][kWave];               // the 10 causal 16x16 tiles of P as A-operand fragments, by lane
 };
 
-// Kt rows are XOR-swizzled in units of four steps so that the 16-bit transposing stores of a wave
-// (8 rows x 8 column groups) land in 32 distinct banks; fragment reads take 4 consecutive steps and are unaffected.
-__device__ __forceinline__ int kt_swz(int n) { return ((n >> 3) & 7) << 2; }
+// A 16x16x16 operand fragment whose contraction index runs along the ROWS of a row-major LDS tile (K^T and x as the
+// state update and P x need them): ds_read_b64_tr_b16 hands lane (lr, lg) the four values tile[k0 + 4 lg + e][m0 + lr],
+// e = 0..3, when the lanes of each 16-lane group point at the 4-row x 16-column block that holds them -- lane lr at
+// row lr / 4, columns 4 (lr % 4)...  No transposed copy of the tile is kept.
+__device__ __forceinline__ uint2 lds_frag_tr(const uint16_t *tile, int ld, int k0, int m0, int lr, int lg) {
+    const uint16_t *p = tile + (k0 + 4 * lg + (lr >> 2)) * ld + m0 + 4 * (lr & 3);
+    const v4s v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((v4s __attribute__((address_space(3))) *)p);
+    return __builtin_bit_cast(uint2, v);
+}
 
 // Super-chunk split of one launch: nsc super-chunks of cps chunks each; the three buffers live in
 // the caller's workspace (null when nsc == 1).
@@ -94,8 +102,42 @@ struct SsdSplit {
     int64_t x_stride;     // elements between consecutive rows of x (d_inner for a dense x)
 };
 
+// Cross-lane moves on the data-parallel-primitive path of the vector ALU (no LDS round trip, unlike the shuffle
+// builtins): the value of the lane above (lane 63 keeps its own), and an inclusive sum over the 64 lanes -- shifts of
+// 1, 2, 4, 8 inside each row of 16 lanes, then the last lane of rows 0 and 2 added to rows 1 and 3, then lane 31 to the
+// upper half.  Lanes without a source add zero.
+__device__ __forceinline__ float lane_above(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, v), __builtin_bit_cast(int, v), 0x130, 0xf, 0xf, false));   // wave_shl:1
+}
+template <int CTRL, int ROWS> __device__ __forceinline__ float dpp_add(float v) {
+    return v + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROWS, 0xf, false));
+}
+__device__ __forceinline__ float wave_inclusive_sum(float v) {
+    v = dpp_add<0x111, 0xf>(v);   // row_shr:1
+    v = dpp_add<0x112, 0xf>(v);   // row_shr:2
+    v = dpp_add<0x114, 0xf>(v);   // row_shr:4
+    v = dpp_add<0x118, 0xf>(v);   // row_shr:8
+    v = dpp_add<0x142, 0xa>(v);   // row_bcast:15 into rows 1 and 3
+    v = dpp_add<0x143, 0xc>(v);   // row_bcast:31 into rows 2 and 3
+    return v;
+}
+
+// Buffer resources for the per-chunk traffic of a workgroup: the address of an access is a scalar base, a scalar offset
+// that moves with the chunk and a 32-bit lane offset fixed for the whole walk, so the walk costs no vector integer
+// work (64-bit multiplies and adds per access otherwise).  A slab (one batch row of a tensor) stays below 2^31 bytes;
+// the launcher checks that.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t slab_rsrc(const void *base, int64_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)bytes, 0x00020000);
+}
+__device__ __forceinline__ uint4 slab_ld128(__amdgpu_buffer_rsrc_t r, unsigned voff, unsigned soff) {
+    return __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0));
+}
+__device__ __forceinline__ float slab_ldf(__amdgpu_buffer_rsrc_t r, unsigned voff, unsigned soff) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0));
+}
+
 template <typename T, int HD, int DS, bool STATE_ONLY>
-__global__ __launch_bounds__(HD * 4) void m3_ssd_kernel(
+__global__ __launch_bounds__(HD * 4) __attribute__((amdgpu_waves_per_eu(HD == 64 ? 3 : 1))) void m3_ssd_kernel(
     float *__restrict__ ssm, float *__restrict__ kst, float *__restrict__ vst, T *__restrict__ y,
     const T *__restrict__ x, const T *__restrict__ K, const T *__restrict__ Q,
     const float *__restrict__ dt, const float *__restrict__ trap, const float *__restrict__ a_val,
@@ -109,7 +151,8 @@ __global__ __launch_bounds__(HD * 4) void m3_ssd_kernel(
     const int nscg = STATE_ONLY ? sp.nsc - 1 : sp.nsc;   // the state-only pass skips the last super-chunk
     const int bhi = blockIdx.x / nscg, sc = blockIdx.x - bhi * nscg;
     const int b = bhi / nh, h = bhi - b * nh;
-    const int tid = threadIdx.x, w = tid >> 6, l = tid & 63;
+    const int tid = threadIdx.x, l = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave index, in a scalar register: what depends on it alone branches without masks
     const int lr = l & 15, lg = l >> 4;            // fragment row/col index and k-group
     const int di = nh * HD;
     const int64_t bh = (int64_t)b * nh + h;
@@ -166,32 +209,40 @@ __global__ __launch_bounds__(HD * 4) void m3_ssd_kernel(
     // ---- global -> register prefetch of one chunk ----
     uint4 rq[NV], rk[NV], rx[2];
     float rdt, rtr, ra, ndt0, ntr0;
+    const unsigned es = (unsigned)sizeof(T);
+    const int64_t kq_row = (int64_t)nh * DS;   // elements between consecutive steps of Q / K
+    const __amdgpu_buffer_rsrc_t qbuf = slab_rsrc(Q + ((int64_t)b * Tlen * nh + h) * DS, ((int64_t)Tlen * kq_row - h * DS) * es);
+    const __amdgpu_buffer_rsrc_t kbuf = slab_rsrc(K + ((int64_t)b * Tlen * nh + h) * DS, ((int64_t)Tlen * kq_row - h * DS) * es);
+    const __amdgpu_buffer_rsrc_t xbuf =
+        slab_rsrc(x + (int64_t)b * Tlen * sp.x_stride + h * HD + 16 * w, ((int64_t)Tlen * sp.x_stride - h * HD - 16 * w) * es);
+    const int64_t sc_bytes = ((int64_t)Tlen * nh - h) * 4;
+    const __amdgpu_buffer_rsrc_t dtbuf = slab_rsrc(dt + (int64_t)b * Tlen * nh + h, sc_bytes);
+    const __amdgpu_buffer_rsrc_t trbuf = slab_rsrc(trap + (int64_t)b * Tlen * nh + h, sc_bytes);
+    const __amdgpu_buffer_rsrc_t abuf = slab_rsrc(a_val + (int64_t)b * Tlen * nh + h, sc_bytes);
+    const __amdgpu_buffer_rsrc_t ybuf = slab_rsrc(y + (int64_t)b * Tlen * di + h * HD + 16 * w, ((int64_t)Tlen * di - h * HD - 16 * w) * es);
+    unsigned kq_voff[NV];
+#pragma unroll
+    for (int v = 0; v < NV; v++) {
+        const int vi = tid + v * NTHR, row = vi / VPR, col = (vi % VPR) * 8;
+        kq_voff[v] = vi < NVEC ? (unsigned)(row * (int)kq_row + col) * es : 0u;   // lanes past the tile read a valid element and drop it
+    }
+    const unsigned x_voff = (unsigned)l * (unsigned)sp.x_stride * es, sc_voff = (unsigned)l * (unsigned)nh * 4u;
+    const unsigned y_voff = (unsigned)(4 * lg * di + lr) * es;
+    // Accesses past the end of the batch row (the tail of a last, partial chunk) fall outside the resources: loads give
+    // zero and stores are dropped by the bounds check, which covers the vector offset -- so the chunk's offset goes there.
     auto prefetch = [&](int c) {
         const int t0 = c * kCS;
+        const unsigned kq_c = (unsigned)t0 * (unsigned)kq_row * es, x_c = (unsigned)t0 * (unsigned)sp.x_stride * es, sc_c = (unsigned)t0 * (unsigned)nh * 4u;
 #pragma unroll
         for (int v = 0; v < NV; v++) {
-            const int vi = tid + v * NTHR, row = vi / VPR, col = (vi % VPR) * 8;
-            const int t = t0 + row;
-            if (vi < NVEC && t < Tlen) {
-                const int64_t off = (((int64_t)b * Tlen + t) * nh + h) * DS + col;
-                if (!STATE_ONLY) rq[v] = *reinterpret_cast<const uint4 *>(Q + off);
-                rk[v] = *reinterpret_cast<const uint4 *>(K + off);
-            } else {
-                rq[v] = make_uint4(0, 0, 0, 0);
-                rk[v] = make_uint4(0, 0, 0, 0);
-            }
+            if (!STATE_ONLY) rq[v] = slab_ld128(qbuf, kq_voff[v] + kq_c, 0);
+            rk[v] = slab_ld128(kbuf, kq_voff[v] + kq_c, 0);
         }
-        const int t = t0 + l;  // lane = step
-        if (t < Tlen) {
-            const int64_t xo = ((int64_t)b * Tlen + t) * sp.x_stride + h * HD + 16 * w;
-            rx[0] = *reinterpret_cast<const uint4 *>(x + xo);
-            rx[1] = *reinterpret_cast<const uint4 *>(x + xo + 8);
-            const int64_t so = ((int64_t)b * Tlen + t) * nh + h;
-            rdt = dt[so]; rtr = trap[so]; ra = a_val[so];
-        } else {
-            rx[0] = make_uint4(0, 0, 0, 0); rx[1] = make_uint4(0, 0, 0, 0);
-            rdt = 0.f; rtr = 0.f; ra = 0.f;
-        }
+        rx[0] = slab_ld128(xbuf, x_voff + x_c, 0);
+        rx[1] = slab_ld128(xbuf, x_voff + x_c + 16u, 0);
+        rdt = slab_ldf(dtbuf, sc_voff + sc_c, 0);
+        rtr = slab_ldf(trbuf, sc_voff + sc_c, 0);
+        ra = slab_ldf(abuf, sc_voff + sc_c, 0);
         const int tn = t0 + kCS;  // first step of the next chunk, for the shifted gamma of step 63
         if (tn < Tlen) {
             const int64_t so = ((int64_t)b * Tlen + tn) * nh + h;
@@ -208,45 +259,28 @@ __global__ __launch_bounds__(HD * 4) void m3_ssd_kernel(
         for (int v = 0; v < NV; v++) {
             const int vi = tid + v * NTHR, row = vi / VPR, col = (vi % VPR) * 8;
             if (vi >= NVEC) continue;
-            if (!STATE_ONLY) {
-                *reinterpret_cast<uint4 *>(&sm.Qs[row][col]) = rq[v];
-                *reinterpret_cast<uint4 *>(&sm.Ks[row][col]) = rk[v];
-            }
-            const unsigned kw[4] = {rk[v].x, rk[v].y, rk[v].z, rk[v].w};
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                sm.Kt[col + 2 * j][row ^ kt_swz(col)] = (uint16_t)(kw[j] & 0xffffu);
-                sm.Kt[col + 2 * j + 1][row ^ kt_swz(col)] = (uint16_t)(kw[j] >> 16);
-            }
+            if (!STATE_ONLY) *reinterpret_cast<uint4 *>(&sm.Qs[row][col]) = rq[v];
+            *reinterpret_cast<uint4 *>(&sm.Ks[row][col]) = rk[v];
         }
-        {
-            const unsigned xw[8] = {rx[0].x, rx[0].y, rx[0].z, rx[0].w, rx[1].x, rx[1].y, rx[1].z, rx[1].w};
-#pragma unroll
-            for (int j = 0; j < 8; j++) {
-                sm.Xt[w][2 * j][l] = (uint16_t)(xw[j] & 0xffffu);
-                sm.Xt[w][2 * j + 1][l] = (uint16_t)(xw[j] >> 16);
-            }
-        }
+        *reinterpret_cast<uint4 *>(&sm.Xs[l][16 * w]) = rx[0];       // lane = step: its 16 values of this wave's columns
+        *reinterpret_cast<uint4 *>(&sm.Xs[l][16 * w + 8]) = rx[1];
         // ---- per-step scalars, lane = step ----
         float dAend;
         {
-            float dtn = __shfl_down(rdt, 1, kWave), trn = __shfl_down(rtr, 1, kWave);
+            float dtn = lane_above(rdt), trn = lane_above(rtr);
             if (l == 63) { dtn = ndt0; trn = ntr0; }
             if (t0 + l + 1 >= Tlen) { dtn = 0.f; trn = 1.f; }       // no step after the last one
             const float gam = rdt * rtr;
             const float scl = fmaf(dtn, 1.0f - trn, gam);
-            float dA = ra * rdt;
-#pragma unroll
-            for (int m = 1; m < kWave; m <<= 1) {                    // inclusive scan over the 64 steps
-                const float o = __shfl_up(dA, m, kWave);
-                if (l >= m) dA += o;
+            const float dA = wave_inclusive_sum(ra * rdt);   // cumulative log-decay over the 64 steps
+            dAend = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, dA), 63));
+            if (w == 0) {   // every wave forms the same values (each needs dAend in its registers); one copy is kept
+                sm.sc[0][l] = dA;
+                sm.sc[1][l] = scl;
+                sm.sc[2][l] = gam;
+                sm.sc[3][l] = fast_exp2(dA * kLog2e);
+                sm.sc[4][l] = fast_exp2((dAend - dA) * kLog2e) * scl;
             }
-            dAend = __shfl(dA, 63, kWave);
-            sm.sc[w][0][l] = dA;
-            sm.sc[w][1][l] = scl;
-            sm.sc[w][2][l] = gam;
-            sm.sc[w][3][l] = fast_exp2(dA * kLog2e);
-            sm.sc[w][4][l] = fast_exp2((dAend - dA) * kLog2e) * scl;
         }
         lds_barrier();  // tiles visible to every wave
         if (c + 1 < c_end) prefetch(c + 1);
@@ -256,8 +290,8 @@ __global__ __launch_bounds__(HD * 4) void m3_ssd_kernel(
         uint2 xf[4], xwf[4];
 #pragma unroll
         for (int kt = 0; kt < 4; kt++) {
-            xf[kt] = *reinterpret_cast<const uint2 *>(&sm.Xt[w][lr][16 * kt + 4 * lg]);
-            const float4 wv = *reinterpret_cast<const float4 *>(&sm.sc[w][4][16 * kt + 4 * lg]);
+            xf[kt] = lds_frag_tr(&sm.Xs[0][0], HD + kPad, 16 * kt, 16 * w, lr, lg);
+            const float4 wv = *reinterpret_cast<const float4 *>(&sm.sc[4][16 * kt + 4 * lg]);
             float xv[4];
             Mma<T>::unpack(xf[kt], xv);
             xwf[kt] = Mma<T>::pack(xv[0] * wv.x, xv[1] * wv.y, xv[2] * wv.z, xv[3] * wv.w);
@@ -283,19 +317,20 @@ __global__ __launch_bounds__(HD * 4) void m3_ssd_kernel(
                         const uint2 qf = *reinterpret_cast<const uint2 *>(&sm.Qs[16 * it + lr][16 * kk + 4 * lg]);
                         g = Mma<T>::mma(kf, qf, g);
                     }
-                    const float dAt = sm.sc[w][0][16 * it + lr];
-                    const float4 dAs = *reinterpret_cast<const float4 *>(&sm.sc[w][0][16 * js + 4 * lg]);
-                    const float4 scs = *reinterpret_cast<const float4 *>(&sm.sc[w][1][16 * js + 4 * lg]);
+                    const float dAt = sm.sc[0][16 * it + lr];
+                    const float4 dAs = *reinterpret_cast<const float4 *>(&sm.sc[0][16 * js + 4 * lg]);
+                    const float4 scs = *reinterpret_cast<const float4 *>(&sm.sc[1][16 * js + 4 * lg]);
                     const float das[4] = {dAs.x, dAs.y, dAs.z, dAs.w}, sc4[4] = {scs.x, scs.y, scs.z, scs.w};
+                    const float gam_t = (js == it) ? sm.sc[2][16 * it + lr] : 0.f;
                     float pv[4];
 #pragma unroll
                     for (int i = 0; i < 4; i++) {
-                        const float dec = fast_exp2((dAt - das[i]) * kLog2e);
+                        const float dec = fast_exp2((dAt - das[i]) * kLog2e);   // above the diagonal: dropped below, whatever it is
                         pv[i] = g[i] * sc4[i] * dec;
-                        if (js == it) {  // diagonal tile: strict causality, skip term on the diagonal
+                        if (js == it) {  // diagonal tile: strict causality, skip term on the diagonal (selects, no branches)
                             const int s = 4 * lg + i;
-                            if (s > lr) pv[i] = 0.f;
-                            else if (s == lr) pv[i] = fmaf(sm.sc[w][2][16 * it + lr], g[i], Dh);
+                            const float dg = fmaf(gam_t, g[i], Dh);
+                            pv[i] = s > lr ? 0.f : (s == lr ? dg : pv[i]);
                         }
                     }
                     sm.Ps[tix][l] = Mma<T>::pack(pv[0], pv[1], pv[2], pv[3]);  // A operand: P[t=lr][s=4lg+i]
@@ -309,7 +344,7 @@ __global__ __launch_bounds__(HD * 4) void m3_ssd_kernel(
             v4f s = St[jn] * decay;
 #pragma unroll
             for (int kt = 0; kt < 4; kt++) {
-                const uint2 ktf = *reinterpret_cast<const uint2 *>(&sm.Kt[16 * jn + lr][(16 * kt + 4 * lg) ^ kt_swz(16 * jn + lr)]);
+                const uint2 ktf = lds_frag_tr(&sm.Ks[0][0], DS + kPad, 16 * kt, 16 * jn, lr, lg);   // K^T[n = 16 jn + lr][t = 16 kt + 4 lg + e]
                 s = Mma<T>::mma(ktf, xwf[kt], s);
             }
             St[jn] = s;
@@ -326,16 +361,16 @@ __global__ __launch_bounds__(HD * 4) void m3_ssd_kernel(
                     acc = Mma<T>::mma(qf, Sf[kk], acc);
                 }
                 {
-                    const float4 e = *reinterpret_cast<const float4 *>(&sm.sc[w][3][16 * it + 4 * lg]);
+                    const float4 e = *reinterpret_cast<const float4 *>(&sm.sc[3][16 * it + 4 * lg]);
                     acc[0] *= e.x; acc[1] *= e.y; acc[2] *= e.z; acc[3] *= e.w;
                 }
 #pragma unroll
                 for (int js = 0; js <= it; js++) acc = Mma<T>::mma(sm.Ps[it * (it + 1) / 2 + js][l], xf[js], acc);
                 // store y rows t = t0+16it+4lg+i, column p = 16w+lr
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const int t = t0 + 16 * it + 4 * lg + i;
-                    if (t < Tlen) Store<T>::st(y + ((int64_t)b * Tlen + t) * di + h * HD + 16 * w + lr, acc[i]);
+                for (int i = 0; i < 4; i++) {   // rows past the sequence are dropped by the bounds check
+                    const T yv = (T)acc[i];
+                    __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(uint16_t, yv), ybuf, y_voff + (unsigned)(t0 + 16 * it + i) * (unsigned)di * es, 0, 0);
                 }
             }
         }
@@ -474,6 +509,10 @@ int mrs::m3_ssd_fwd_ex(void *stream, int dtype, float *ssm_state, float *k_state
     if (x_stride < di_) return fail(MRS_E_SHAPE, "%s: row stride below d_inner", fn);
     if (dtype == MRS_F32 && x_stride != di_) return fail(MRS_E_SHAPE, "%s: strided x needs 16-bit storage", fn);
     if (x_stride % 8 != 0) return fail(MRS_E_ALIGN, "%s: x row stride must be a multiple of 8 elements", fn);
+    {   // the kernel addresses one batch row of a tensor with 32-bit byte offsets
+        const int64_t widest = std::max<int64_t>(x_stride, std::max<int64_t>(di_, (int64_t)nheads * d_state));
+        if ((int64_t)T * widest * 4 >= 0x7fffffffLL) return fail(MRS_E_SHAPE, "%s: one batch row of x, y, K or Q exceeds 2^31 bytes", fn);
+    }
     if (dtype != MRS_F32 && dtype != MRS_F16 && dtype != MRS_BF16) return fail(MRS_E_DTYPE, "%s: dtype %d is not f32/f16/bf16", fn, dtype);
     if (!ssm_state || !k_state || !v_state || !y || !x || !K || !Q || !dt || !trap || !a_val || !D)
         return fail(MRS_E_NULL, "%s: null pointer", fn);
