@@ -103,12 +103,8 @@ struct SsdSplit {
 };
 
 // Cross-lane moves on the data-parallel-primitive path of the vector ALU (no LDS round trip, unlike the shuffle
-// builtins): the value of the lane above (lane 63 keeps its own), and an inclusive sum over the 64 lanes -- shifts of
-// 1, 2, 4, 8 inside each row of 16 lanes, then the last lane of rows 0 and 2 added to rows 1 and 3, then lane 31 to the
+// builtins): an inclusive sum over the 64 lanes -- shifts of 1, 2, 4, 8 inside each row of 16 lanes, then the last lane of rows 0 and 2 added to rows 1 and 3, then lane 31 to the
 // upper half.  Lanes without a source add zero.
-__device__ __forceinline__ float lane_above(float v) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, v), __builtin_bit_cast(int, v), 0x130, 0xf, 0xf, false));   // wave_shl:1
-}
 template <int CTRL, int ROWS> __device__ __forceinline__ float dpp_add(float v) {
     return v + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROWS, 0xf, false));
 }
@@ -207,14 +203,16 @@ __global__ __launch_bounds__(HD * 4) __attribute__((amdgpu_waves_per_eu(HD == 64
     float dAsum = 0.0f;
 
     // ---- global -> register prefetch of one chunk ----
-    uint4 rq[NV], rk[NV], rx[2];
-    float rdt, rtr, ra, ndt0, ntr0;
+    struct Pre {
+        uint4 rq[NV], rk[NV], rx[2];
+        float rdt, rtr, ra, rdtn, rtrn;   // lane = step: dt, trap, a of the step and dt, trap of the step after it
+    };
     const unsigned es = (unsigned)sizeof(T);
     const int64_t kq_row = (int64_t)nh * DS;   // elements between consecutive steps of Q / K
     const __amdgpu_buffer_rsrc_t qbuf = slab_rsrc(Q + ((int64_t)b * Tlen * nh + h) * DS, ((int64_t)Tlen * kq_row - h * DS) * es);
     const __amdgpu_buffer_rsrc_t kbuf = slab_rsrc(K + ((int64_t)b * Tlen * nh + h) * DS, ((int64_t)Tlen * kq_row - h * DS) * es);
     const __amdgpu_buffer_rsrc_t xbuf =
-        slab_rsrc(x + (int64_t)b * Tlen * sp.x_stride + h * HD + 16 * w, ((int64_t)Tlen * sp.x_stride - h * HD - 16 * w) * es);
+        slab_rsrc(x + (int64_t)b * Tlen * sp.x_stride + h * HD, ((int64_t)Tlen * sp.x_stride - h * HD) * es);
     const int64_t sc_bytes = ((int64_t)Tlen * nh - h) * 4;
     const __amdgpu_buffer_rsrc_t dtbuf = slab_rsrc(dt + (int64_t)b * Tlen * nh + h, sc_bytes);
     const __amdgpu_buffer_rsrc_t trbuf = slab_rsrc(trap + (int64_t)b * Tlen * nh + h, sc_bytes);
@@ -226,32 +224,40 @@ __global__ __launch_bounds__(HD * 4) __attribute__((amdgpu_waves_per_eu(HD == 64
         const int vi = tid + v * NTHR, row = vi / VPR, col = (vi % VPR) * 8;
         kq_voff[v] = vi < NVEC ? (unsigned)(row * (int)kq_row + col) * es : 0u;   // lanes past the tile read a valid element and drop it
     }
-    const unsigned x_voff = (unsigned)l * (unsigned)sp.x_stride * es, sc_voff = (unsigned)l * (unsigned)nh * 4u;
+    // the x tile (64 steps x HD) is fetched like the Q / K tiles, whole rows by neighbouring lanes: HD / 8 vectors a row,
+    // two vectors a thread for any HD (a lane fetching its own step's row piece touched 64 cache lines per instruction)
+    constexpr int VPRX = HD / 8;
+    unsigned x_voff[2];
+    int x_row[2], x_col[2];
+#pragma unroll
+    for (int v = 0; v < 2; v++) {
+        const int vi = tid + v * NTHR;
+        x_row[v] = vi / VPRX; x_col[v] = (vi % VPRX) * 8;
+        x_voff[v] = (unsigned)(x_row[v] * (int)sp.x_stride + x_col[v]) * es;
+    }
+    const unsigned sc_voff = (unsigned)l * (unsigned)nh * 4u;
     const unsigned y_voff = (unsigned)(4 * lg * di + lr) * es;
     // Accesses past the end of the batch row (the tail of a last, partial chunk) fall outside the resources: loads give
     // zero and stores are dropped by the bounds check, which covers the vector offset -- so the chunk's offset goes there.
-    auto prefetch = [&](int c) {
+    auto prefetch = [&](Pre &r, int c) {
         const int t0 = c * kCS;
         const unsigned kq_c = (unsigned)t0 * (unsigned)kq_row * es, x_c = (unsigned)t0 * (unsigned)sp.x_stride * es, sc_c = (unsigned)t0 * (unsigned)nh * 4u;
 #pragma unroll
         for (int v = 0; v < NV; v++) {
-            if (!STATE_ONLY) rq[v] = slab_ld128(qbuf, kq_voff[v] + kq_c, 0);
-            rk[v] = slab_ld128(kbuf, kq_voff[v] + kq_c, 0);
+            if (!STATE_ONLY) r.rq[v] = slab_ld128(qbuf, kq_voff[v] + kq_c, 0);
+            r.rk[v] = slab_ld128(kbuf, kq_voff[v] + kq_c, 0);
         }
-        rx[0] = slab_ld128(xbuf, x_voff + x_c, 0);
-        rx[1] = slab_ld128(xbuf, x_voff + x_c + 16u, 0);
-        rdt = slab_ldf(dtbuf, sc_voff + sc_c, 0);
-        rtr = slab_ldf(trbuf, sc_voff + sc_c, 0);
-        ra = slab_ldf(abuf, sc_voff + sc_c, 0);
-        const int tn = t0 + kCS;  // first step of the next chunk, for the shifted gamma of step 63
-        if (tn < Tlen) {
-            const int64_t so = ((int64_t)b * Tlen + tn) * nh + h;
-            ndt0 = dt[so]; ntr0 = trap[so];
-        } else { ndt0 = 0.f; ntr0 = 1.f; }
+        r.rx[0] = slab_ld128(xbuf, x_voff[0] + x_c, 0);
+        r.rx[1] = slab_ld128(xbuf, x_voff[1] + x_c, 0);
+        r.rdt = slab_ldf(dtbuf, sc_voff + sc_c, 0);
+        r.rtr = slab_ldf(trbuf, sc_voff + sc_c, 0);
+        r.ra = slab_ldf(abuf, sc_voff + sc_c, 0);
+        r.rdtn = slab_ldf(dtbuf, sc_voff + sc_c + (unsigned)nh * 4u, 0);   // the shifted gamma needs the step after (zero past the row)
+        r.rtrn = slab_ldf(trbuf, sc_voff + sc_c + (unsigned)nh * 4u, 0);
     };
 
-    prefetch(c_begin);
-    for (int c = c_begin; c < c_end; c++) {
+    // One chunk from the registers of `r`; once they are in LDS the chunk c_next is requested into them.
+    auto chunk = [&](Pre &r, int c, int c_next) {
         const int t0 = c * kCS;
         lds_barrier();  // every wave is done reading the previous chunk's tiles (LDS only: y stores and the prefetch stay in flight)
         // ---- registers -> LDS ----
@@ -259,20 +265,19 @@ __global__ __launch_bounds__(HD * 4) __attribute__((amdgpu_waves_per_eu(HD == 64
         for (int v = 0; v < NV; v++) {
             const int vi = tid + v * NTHR, row = vi / VPR, col = (vi % VPR) * 8;
             if (vi >= NVEC) continue;
-            if (!STATE_ONLY) *reinterpret_cast<uint4 *>(&sm.Qs[row][col]) = rq[v];
-            *reinterpret_cast<uint4 *>(&sm.Ks[row][col]) = rk[v];
+            if (!STATE_ONLY) *reinterpret_cast<uint4 *>(&sm.Qs[row][col]) = r.rq[v];
+            *reinterpret_cast<uint4 *>(&sm.Ks[row][col]) = r.rk[v];
         }
-        *reinterpret_cast<uint4 *>(&sm.Xs[l][16 * w]) = rx[0];       // lane = step: its 16 values of this wave's columns
-        *reinterpret_cast<uint4 *>(&sm.Xs[l][16 * w + 8]) = rx[1];
+        *reinterpret_cast<uint4 *>(&sm.Xs[x_row[0]][x_col[0]]) = r.rx[0];
+        *reinterpret_cast<uint4 *>(&sm.Xs[x_row[1]][x_col[1]]) = r.rx[1];
         // ---- per-step scalars, lane = step ----
         float dAend;
         {
-            float dtn = lane_above(rdt), trn = lane_above(rtr);
-            if (l == 63) { dtn = ndt0; trn = ntr0; }
+            float dtn = r.rdtn, trn = r.rtrn;
             if (t0 + l + 1 >= Tlen) { dtn = 0.f; trn = 1.f; }       // no step after the last one
-            const float gam = rdt * rtr;
+            const float gam = r.rdt * r.rtr;
             const float scl = fmaf(dtn, 1.0f - trn, gam);
-            const float dA = wave_inclusive_sum(ra * rdt);   // cumulative log-decay over the 64 steps
+            const float dA = wave_inclusive_sum(r.ra * r.rdt);   // cumulative log-decay over the 64 steps
             dAend = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, dA), 63));
             if (w == 0) {   // every wave forms the same values (each needs dAend in its registers); one copy is kept
                 sm.sc[0][l] = dA;
@@ -283,7 +288,7 @@ __global__ __launch_bounds__(HD * 4) __attribute__((amdgpu_waves_per_eu(HD == 64
             }
         }
         lds_barrier();  // tiles visible to every wave
-        if (c + 1 < c_end) prefetch(c + 1);
+        if (c_next < c_end) prefetch(r, c_next);
         dAsum += dAend;
 
         // ---- x fragments: lane holds x[t=16kt+4lg+i][p=16w+lr]; also scaled by w[t] for the state update ----
@@ -374,6 +379,21 @@ __global__ __launch_bounds__(HD * 4) __attribute__((amdgpu_waves_per_eu(HD == 64
                 }
             }
         }
+    };
+    if (STATE_ONLY) {
+        // The state-only pass does little arithmetic per chunk, so its walk is as long as a memory round trip per chunk
+        // allows: two chunks are kept in flight (registers are not scarce here).
+        Pre ra_, rb_;
+        prefetch(ra_, c_begin);
+        if (c_begin + 1 < c_end) prefetch(rb_, c_begin + 1);
+        for (int c = c_begin; c < c_end; c += 2) {
+            chunk(ra_, c, c + 2);
+            if (c + 1 < c_end) chunk(rb_, c + 1, c + 3);
+        }
+    } else {
+        Pre r_;
+        prefetch(r_, c_begin);
+        for (int c = c_begin; c < c_end; c++) chunk(r_, c, c + 1);
     }
     if (STATE_ONLY) {
         const int64_t slot = bh * (sp.nsc - 1) + sc;
