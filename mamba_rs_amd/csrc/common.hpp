@@ -132,10 +132,14 @@ int launch_prenorm_rows(hipStream_t st, int dtype, float *partials, int n_partia
                         const float *w, int M, int K);
 
 // mrs_m3_ssd_fwd with x read in place out of wider rows (x_stride elements apart, 0 = dense; 16-bit storage only).
+// With `gen` the kernel forms K and Q itself (K and Q are not read and may be null): K = rot(angle, bn + b_bias[head]),
+// Q = rot(angle, cn + c_bias[head]) with bn / cn the normalised and weighted B / C rows (f32, bc_stride floats apart),
+// angle [batch, T, nheads, n_rope] and the first n_rope pairs of a row turned.  headdim = d_state = 64, 16-bit storage.
+struct SsdGenArgs { const float *bn, *cn; int64_t bc_stride; const float *angle, *b_bias, *c_bias; int n_rope; };
 int m3_ssd_fwd_ex(void *stream, int dtype, float *ssm_state, float *k_state, float *v_state, void *y, const void *x,
                   int64_t x_stride, const void *K, const void *Q, const float *dt, const float *trap, const float *a_val,
                   const float *D, void *workspace, size_t workspace_bytes, unsigned flags, int batch, int T, int nheads,
-                  int headdim, int d_state, int chunk_size);
+                  int headdim, int d_state, int chunk_size, const SsdGenArgs *gen = nullptr);
 
 // What the LM loop (embedding gather, head, argmax / sampling, generation bookkeeping) needs from a backbone engine;
 // the Mamba-1 and the Mamba-3 engine each fill one in.  All functions are stream-ordered on `stream`.

@@ -420,6 +420,24 @@ __global__ __launch_bounds__(256) void m3_kq_rows_kernel(
         for (int i = l; i < di; i += 64) xout[r * di + i] = row[di + i];
 }
 
+// The part of K and Q that all heads share, for the scan kernel that forms K and Q itself (one group, d_state 64):
+// out[row] = [B * rsqrt(mean(B^2) + eps) * bnw | C * rsqrt(mean(C^2) + eps) * cnw] in f32 (bcnorm_fwd, ops/norms.rs:50-80);
+// the per-head bias and the rotation happen where the tiles are built.  A wave per row, a lane per coordinate.
+__global__ __launch_bounds__(256) void m3_bcn_rows_kernel(float *__restrict__ out, const float *__restrict__ bc, int64_t ldbc,
+                                                          const float *__restrict__ bnw, const float *__restrict__ cnw, int64_t rows, float eps) {
+    constexpr int ds = 64;
+    const int w = threadIdx.x >> 6, l = threadIdx.x & 63;
+    const int64_t r = (int64_t)blockIdx.x * 4 + w;
+    if (r >= rows) return;   // whole waves leave; the kernel has no barrier
+    const float b = bc[r * ldbc + l], c = bc[r * ldbc + ds + l];
+    float ssb = b * b, ssc = c * c;
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) { ssb += __shfl_xor(ssb, m, kWave); ssc += __shfl_xor(ssc, m, kWave); }
+    const float ib = 1.0f / sqrtf(ssb / (float)ds + eps), ic = 1.0f / sqrtf(ssc / (float)ds + eps);
+    out[r * (2 * ds) + l] = b * ib * bnw[l];
+    out[r * (2 * ds) + ds + l] = c * ic * cnw[l];
+}
+
 // gated[row, i] = y * silu(z), or RMSNormGated over each head first; z = the first d_inner elements of the bulk row.
 // One workgroup (256 threads) per row, a wave per head at a time for the normalised form.
 template <typename T>
@@ -500,6 +518,7 @@ struct mrs_m3_backbone {
     int pf_T;
     float *pf_in, *pf_residual, *pf_proj, *pf_dt, *pf_a, *pf_trap, *pf_tanhpi, *pf_angle, *pf_angle_snap;
     double *pf_angle_sums;   // [batch][kAngleSegs][nh * n_rope] per-segment angle increments of the prefill
+    float *pf_bcn;           // [rows][2 * d_state] normalised and weighted B | C rows for the scan that forms K and Q itself
     void *pf_normed, *pf_bulk, *pf_x, *pf_K, *pf_Q, *pf_y, *pf_gated, *pf_out, *pf_ws;
     size_t pf_ws_bytes;
 };
@@ -808,6 +827,7 @@ extern "C" int mrs_m3_backbone_alloc_prefill_scratch(mrs_m3_backbone *bb, int T)
     MRS_TRY(dev_alloc3(bb, (void **)&bb->pf_angle, rows * nh * nrz * 4));
     MRS_TRY(dev_alloc3(bb, (void **)&bb->pf_angle_sums, (size_t)bb->batch * kAngleSegs * nh * nrz * sizeof(double)));
     MRS_TRY(dev_alloc3(bb, (void **)&bb->pf_angle_snap, (size_t)bb->batch * nh * nrz * 4));
+    MRS_TRY(dev_alloc3(bb, (void **)&bb->pf_bcn, rows * 2 * ds * 4));
     MRS_TRY(dev_alloc3(bb, &bb->pf_normed, rows * dm * es));
     MRS_TRY(dev_alloc3(bb, &bb->pf_x, rows * di * es));
     MRS_TRY(dev_alloc3(bb, &bb->pf_K, rows * nh * ds * es));
@@ -875,6 +895,7 @@ int prefill_body3(mrs_m3_backbone *bb, int T) {
                                  rocblas_gemm_algo_standard, 0, 0));
     }
     const bool chunked_ok = (hd == 16 || hd == 32 || hd == 64) && (ds == 16 || ds == 32 || ds == 64);
+    const bool no_fused_kq = getenv("MRS_M3_NO_FUSED_KQ") != nullptr;   // keeps the separate K / Q pass (measurement, tests)
     for (int l = 0; l < L; l++) {
         const Layer3 &lw = bb->layers[l];
         float *ssm = bb->ssm + (size_t)l * B * nh * hd * ds, *kst = bb->kst + (size_t)l * B * nh * ds;
@@ -939,15 +960,28 @@ int prefill_body3(mrs_m3_backbone *bb, int T) {
         // measured and dropped: the scattered z reads cost the latency-bound kernel 54 us against 28 us for the
         // separate gate pass.)
         const bool in_place = chunked_ok && dt != MRS_F32 && ldb % 8 == 0 && di % 8 == 0;
-        MRS_DISPATCH_DTYPE(dt, T_, MRS_TRY(launch_kq_t<T_>(bb, lw, rows, bulk, ldb, bcp, lds_, !in_place)));
-        if (in_place) {
+        // one group at headdim = d_state = 64 with the rope pairs in fours: the scan builds its K and Q tiles from the
+        // normalised B / C rows and the angles, so the [rows, nheads, d_state] K and Q never exist in memory
+        const bool fused_kq = in_place && hd == 64 && ds == 64 && c.ngroups == 1 && nr > 0 && nr % 4 == 0 && !no_fused_kq;
+        if (fused_kq) {
+            hipLaunchKernelGGL(m3_bcn_rows_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, bb->stream, bb->pf_bcn, bcp, lds_, lw.bnw, lw.cnw,
+                               rows, c.rms_norm_eps);
+            MRS_TRY(check_launch("m3_bcn_rows_kernel"));
+            const SsdGenArgs gen = {bb->pf_bcn, bb->pf_bcn + ds, 2 * (int64_t)ds, bb->pf_angle, lw.b_bias, lw.c_bias, nr};
+            const char *xb = (const char *)bulk + (size_t)di * es;
+            MRS_TRY(m3_ssd_fwd_ex(bb->stream, dt, ssm, kst, vst, bb->pf_y, xb, ldb, nullptr, nullptr, bb->pf_dt, bb->pf_trap, bb->pf_a, lw.D,
+                                  bb->pf_ws, bb->pf_ws_bytes, MRS_M3_CARRY_STATE, B, T, nh, hd, ds, 64, &gen));
+        } else if (in_place) {
+            MRS_DISPATCH_DTYPE(dt, T_, MRS_TRY(launch_kq_t<T_>(bb, lw, rows, bulk, ldb, bcp, lds_, false)));
             const char *xb = (const char *)bulk + (size_t)di * es;
             MRS_TRY(m3_ssd_fwd_ex(bb->stream, dt, ssm, kst, vst, bb->pf_y, xb, ldb, bb->pf_K, bb->pf_Q, bb->pf_dt, bb->pf_trap, bb->pf_a, lw.D,
                                   bb->pf_ws, bb->pf_ws_bytes, MRS_M3_CARRY_STATE, B, T, nh, hd, ds, 64));
         } else if (chunked_ok) {
+            MRS_DISPATCH_DTYPE(dt, T_, MRS_TRY(launch_kq_t<T_>(bb, lw, rows, bulk, ldb, bcp, lds_, true)));
             MRS_TRY(mrs_m3_ssd_fwd(bb->stream, dt, ssm, kst, vst, bb->pf_y, bb->pf_x, bb->pf_K, bb->pf_Q, bb->pf_dt, bb->pf_trap, bb->pf_a, lw.D,
                                    bb->pf_ws, bb->pf_ws_bytes, MRS_M3_CARRY_STATE, B, T, nh, hd, ds, 64));
         } else {
+            MRS_DISPATCH_DTYPE(dt, T_, MRS_TRY(launch_kq_t<T_>(bb, lw, rows, bulk, ldb, bcp, lds_, true)));
             float *al = (float *)bb->pf_ws, *be = al + rows * nh, *ga = be + rows * nh;
             MRS_TRY(mrs_m3_compute_abg(bb->stream, al, be, ga, bb->pf_dt, bb->pf_a, bb->pf_trap, rows * nh));
             MRS_TRY(mrs_m3_seq_fwd(bb->stream, dt, ssm, kst, vst, bb->pf_y, bb->pf_x, bb->pf_K, bb->pf_Q, al, be, ga, lw.D, B, T, nh, hd, ds));

@@ -79,6 +79,7 @@ template <int HD, int DS> struct alignas(16) SsdSmem {
     alignas(16) uint16_t Xs[kCS][HD + kPad];       // x rows of this head
     alignas(16) float sc[5][kCS];                  // dA, scale, gamma, exp(dA), w
     alignas(16) uint2 Ps[10][kWave];               // the 10 causal 16x16 tiles of P as A-operand fragments, by lane
+    alignas(16) float gb[2][DS];                   // GEN: the head's B and C biases
 };
 
 // A 16x16x16 operand fragment whose contraction index runs along the ROWS of a row-major LDS tile (K^T and x as the
@@ -100,6 +101,12 @@ struct SsdSplit {
     int nsc, cps;
     // engine-only extra: x rows may sit inside wider rows (read in place from a projection)
     int64_t x_stride;     // elements between consecutive rows of x (d_inner for a dense x)
+    // engine-only extra: K and Q formed inside the kernel (GEN), K = rot(angle, bn + b_bias[h]), Q = rot(angle, cn + c_bias[h]);
+    // bn / cn: the normalised and weighted B / C rows, f32, g_bcs floats apart; angle [batch, T, nh, g_nr]; the first g_nr
+    // pairs of a row are rotated (g_nr a multiple of 4)
+    const float *g_bn, *g_cn, *g_ang, *g_bb, *g_cb;
+    int64_t g_bcs;
+    int g_nr;
 };
 
 // Cross-lane moves on the data-parallel-primitive path of the vector ALU (no LDS round trip, unlike the shuffle
@@ -132,7 +139,7 @@ __device__ __forceinline__ float slab_ldf(__amdgpu_buffer_rsrc_t r, unsigned vof
     return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0));
 }
 
-template <typename T, int HD, int DS, bool STATE_ONLY>
+template <typename T, int HD, int DS, bool STATE_ONLY, bool GEN>
 __global__ __launch_bounds__(HD * 4) __attribute__((amdgpu_waves_per_eu(HD == 64 ? 3 : 1))) void m3_ssd_kernel(
     float *__restrict__ ssm, float *__restrict__ kst, float *__restrict__ vst, T *__restrict__ y,
     const T *__restrict__ x, const T *__restrict__ K, const T *__restrict__ Q,
@@ -204,7 +211,8 @@ __global__ __launch_bounds__(HD * 4) __attribute__((amdgpu_waves_per_eu(HD == 64
 
     // ---- global -> register prefetch of one chunk ----
     struct Pre {
-        uint4 rq[NV], rk[NV], rx[2];
+        // plain: the Q / K vectors of the thread; GEN: two f32 vectors of cn / bn for each of them, and the 4 angles
+        uint4 rq[NV * (GEN ? 2 : 1)], rk[NV * (GEN ? 2 : 1)], rang[GEN ? NV : 1], rx[2];
         float rdt, rtr, ra, rdtn, rtrn;   // lane = step: dt, trap, a of the step and dt, trap of the step after it
     };
     const unsigned es = (unsigned)sizeof(T);
@@ -224,6 +232,23 @@ __global__ __launch_bounds__(HD * 4) __attribute__((amdgpu_waves_per_eu(HD == 64
         const int vi = tid + v * NTHR, row = vi / VPR, col = (vi % VPR) * 8;
         kq_voff[v] = vi < NVEC ? (unsigned)(row * (int)kq_row + col) * es : 0u;   // lanes past the tile read a valid element and drop it
     }
+    // GEN: the same (row, 8 columns) items read bn / cn (f32) and the 4 angles of their pairs instead of K / Q
+    const int g_col = (tid % VPR) * 8;             // the thread's columns, the same for each of its vectors
+    const bool g_rot = g_col < 2 * sp.g_nr;        // its pairs are rotated (all four or none: g_nr is a multiple of 4)
+    const __amdgpu_buffer_rsrc_t bnbuf = slab_rsrc(GEN ? sp.g_bn + (int64_t)b * Tlen * sp.g_bcs : nullptr, GEN ? (int64_t)Tlen * sp.g_bcs * 4 : 0);
+    const __amdgpu_buffer_rsrc_t cnbuf = slab_rsrc(GEN ? sp.g_cn + (int64_t)b * Tlen * sp.g_bcs : nullptr, GEN ? (int64_t)Tlen * sp.g_bcs * 4 : 0);
+    const __amdgpu_buffer_rsrc_t angbuf =
+        slab_rsrc(GEN ? sp.g_ang + ((int64_t)b * Tlen * nh + h) * sp.g_nr : nullptr, GEN ? ((int64_t)Tlen * nh - h) * sp.g_nr * 4 : 0);
+    unsigned bc_voff[NV], ang_voff[NV];
+#pragma unroll
+    for (int v = 0; v < NV; v++) {
+        const int vi = tid + v * NTHR, row = vi / VPR;
+        bc_voff[v] = GEN && vi < NVEC ? (unsigned)(row * (int)sp.g_bcs + g_col) * 4u : 0u;
+        ang_voff[v] = GEN && vi < NVEC && g_rot ? (unsigned)(row * nh * sp.g_nr + g_col / 2) * 4u : 0u;
+    }
+    if (GEN) {   // visible to every wave after the barrier at the top of the first chunk
+        for (int n = tid; n < DS; n += NTHR) { sm.gb[0][n] = sp.g_bb[h * DS + n]; sm.gb[1][n] = sp.g_cb[h * DS + n]; }
+    }
     // the x tile (64 steps x HD) is fetched like the Q / K tiles, whole rows by neighbouring lanes: HD / 8 vectors a row,
     // two vectors a thread for any HD (a lane fetching its own step's row piece touched 64 cache lines per instruction)
     constexpr int VPRX = HD / 8;
@@ -242,10 +267,24 @@ __global__ __launch_bounds__(HD * 4) __attribute__((amdgpu_waves_per_eu(HD == 64
     auto prefetch = [&](Pre &r, int c) {
         const int t0 = c * kCS;
         const unsigned kq_c = (unsigned)t0 * (unsigned)kq_row * es, x_c = (unsigned)t0 * (unsigned)sp.x_stride * es, sc_c = (unsigned)t0 * (unsigned)nh * 4u;
+        if constexpr (GEN) {
+            const unsigned bc_c = (unsigned)t0 * (unsigned)sp.g_bcs * 4u, ang_c = (unsigned)t0 * (unsigned)(nh * sp.g_nr) * 4u;
 #pragma unroll
-        for (int v = 0; v < NV; v++) {
-            if (!STATE_ONLY) r.rq[v] = slab_ld128(qbuf, kq_voff[v] + kq_c, 0);
-            r.rk[v] = slab_ld128(kbuf, kq_voff[v] + kq_c, 0);
+            for (int v = 0; v < NV; v++) {
+                if (!STATE_ONLY) {
+                    r.rq[2 * v] = slab_ld128(cnbuf, bc_voff[v] + bc_c, 0);
+                    r.rq[2 * v + 1] = slab_ld128(cnbuf, bc_voff[v] + bc_c + 16u, 0);
+                }
+                r.rk[2 * v] = slab_ld128(bnbuf, bc_voff[v] + bc_c, 0);
+                r.rk[2 * v + 1] = slab_ld128(bnbuf, bc_voff[v] + bc_c + 16u, 0);
+                r.rang[v] = slab_ld128(angbuf, ang_voff[v] + ang_c, 0);   // lanes without rotated pairs: some angle, not used
+            }
+        } else {
+#pragma unroll
+            for (int v = 0; v < NV; v++) {
+                if (!STATE_ONLY) r.rq[v] = slab_ld128(qbuf, kq_voff[v] + kq_c, 0);
+                r.rk[v] = slab_ld128(kbuf, kq_voff[v] + kq_c, 0);
+            }
         }
         r.rx[0] = slab_ld128(xbuf, x_voff[0] + x_c, 0);
         r.rx[1] = slab_ld128(xbuf, x_voff[1] + x_c, 0);
@@ -265,8 +304,34 @@ __global__ __launch_bounds__(HD * 4) __attribute__((amdgpu_waves_per_eu(HD == 64
         for (int v = 0; v < NV; v++) {
             const int vi = tid + v * NTHR, row = vi / VPR, col = (vi % VPR) * 8;
             if (vi >= NVEC) continue;
-            if (!STATE_ONLY) *reinterpret_cast<uint4 *>(&sm.Qs[row][col]) = r.rq[v];
-            *reinterpret_cast<uint4 *>(&sm.Ks[row][col]) = r.rk[v];
+            if constexpr (GEN) {
+                // K = rot(bn + b_bias), Q = rot(cn + c_bias): pairs (2j, 2j+1), j < g_nr, turned by the step's angle
+                // (hardware sine / cosine: angles lie in [0, 2 pi), the results are stored in 16 bits); lanes whose
+                // pairs are not rotated turn by zero
+                const float4 an = __builtin_bit_cast(float4, r.rang[v]);
+                const float ang[4] = {g_rot ? an.x : 0.f, g_rot ? an.y : 0.f, g_rot ? an.z : 0.f, g_rot ? an.w : 0.f};
+                float sn[4], cs[4];
+#pragma unroll
+                for (int pr = 0; pr < 4; pr++) { sn[pr] = __sinf(ang[pr]); cs[pr] = __cosf(ang[pr]); }
+                auto form = [&](const uint4 &lo, const uint4 &hi, const float *bias) {
+                    const float4 b0 = *reinterpret_cast<const float4 *>(bias + col), b1 = *reinterpret_cast<const float4 *>(bias + col + 4);
+                    const float4 v0 = __builtin_bit_cast(float4, lo), v1 = __builtin_bit_cast(float4, hi);
+                    const float k[8] = {v0.x + b0.x, v0.y + b0.y, v0.z + b0.z, v0.w + b0.w, v1.x + b1.x, v1.y + b1.y, v1.z + b1.z, v1.w + b1.w};
+                    float o[8];
+#pragma unroll
+                    for (int pr = 0; pr < 4; pr++) {
+                        o[2 * pr] = cs[pr] * k[2 * pr] - sn[pr] * k[2 * pr + 1];
+                        o[2 * pr + 1] = sn[pr] * k[2 * pr] + cs[pr] * k[2 * pr + 1];
+                    }
+                    const uint2 p0 = Mma<T>::pack(o[0], o[1], o[2], o[3]), p1 = Mma<T>::pack(o[4], o[5], o[6], o[7]);
+                    return make_uint4(p0.x, p0.y, p1.x, p1.y);
+                };
+                if (!STATE_ONLY) *reinterpret_cast<uint4 *>(&sm.Qs[row][col]) = form(r.rq[2 * v], r.rq[2 * v + 1], sm.gb[1]);
+                *reinterpret_cast<uint4 *>(&sm.Ks[row][col]) = form(r.rk[2 * v], r.rk[2 * v + 1], sm.gb[0]);
+            } else {
+                if (!STATE_ONLY) *reinterpret_cast<uint4 *>(&sm.Qs[row][col]) = r.rq[v];
+                *reinterpret_cast<uint4 *>(&sm.Ks[row][col]) = r.rk[v];
+            }
         }
         *reinterpret_cast<uint4 *>(&sm.Xs[x_row[0]][x_col[0]]) = r.rx[0];
         *reinterpret_cast<uint4 *>(&sm.Xs[x_row[1]][x_col[1]]) = r.rx[1];
@@ -410,7 +475,18 @@ __global__ __launch_bounds__(HD * 4) __attribute__((amdgpu_waves_per_eu(HD == 64
     for (int jn = 0; jn < KN; jn++)
         *reinterpret_cast<float4 *>(ssm + srow + 16 * jn) = make_float4(St[jn][0], St[jn][1], St[jn][2], St[jn][3]);
     const int64_t last = (int64_t)b * Tlen + (Tlen - 1);
-    for (int n = tid; n < DS; n += NTHR) kst[bh * DS + n] = Store<T>::ld(K + (last * nh + h) * DS + n);
+    if constexpr (GEN) {   // K of the last step, as the tiles above form it (rounded to the storage type like a K read from memory)
+        for (int n = tid; n < DS; n += NTHR) {
+            const int j = n >> 1;
+            const float k0 = sp.g_bn[last * sp.g_bcs + 2 * j] + sp.g_bb[h * DS + 2 * j], k1 = sp.g_bn[last * sp.g_bcs + 2 * j + 1] + sp.g_bb[h * DS + 2 * j + 1];
+            const float a = j < sp.g_nr ? sp.g_ang[(last * nh + h) * sp.g_nr + j] : 0.f;
+            const float sn = __sinf(a), cs = __cosf(a);
+            const T kv = (T)((n & 1) ? sn * k0 + cs * k1 : cs * k0 - sn * k1);
+            kst[bh * DS + n] = (float)kv;
+        }
+    } else {
+        for (int n = tid; n < DS; n += NTHR) kst[bh * DS + n] = Store<T>::ld(K + (last * nh + h) * DS + n);
+    }
     for (int p = tid; p < HD; p += NTHR) vst[bh * HD + p] = Store<T>::ld(x + last * sp.x_stride + h * HD + p);
 }
 
@@ -460,10 +536,20 @@ template <typename T, int HD, int DS>
 static void launch_ssd_shape(hipStream_t st, float *ssm, float *kst, float *vst, void *y, const void *x,
                              const void *K, const void *Q, const float *dt, const float *trap,
                              const float *a_val, const float *D, SsdSplit sp, int batch, int Tlen, int nh, int carry) {
+    if constexpr (HD == 64 && DS == 64) {   // the one shape the in-kernel K / Q route is built for
+        if (sp.g_bn) {
+            if (sp.nsc > 1)
+                hipLaunchKernelGGL((m3_ssd_kernel<T, HD, DS, true, true>), dim3((unsigned)(batch * nh * (sp.nsc - 1))), dim3(HD * 4), 0, st,
+                                   ssm, kst, vst, (T *)y, (const T *)x, (const T *)K, (const T *)Q, dt, trap, a_val, D, sp, Tlen, nh, carry);
+            hipLaunchKernelGGL((m3_ssd_kernel<T, HD, DS, false, true>), dim3((unsigned)(batch * nh * sp.nsc)), dim3(HD * 4), 0, st, ssm, kst, vst,
+                               (T *)y, (const T *)x, (const T *)K, (const T *)Q, dt, trap, a_val, D, sp, Tlen, nh, carry);
+            return;
+        }
+    }
     if (sp.nsc > 1)
-        hipLaunchKernelGGL((m3_ssd_kernel<T, HD, DS, true>), dim3((unsigned)(batch * nh * (sp.nsc - 1))), dim3(HD * 4), 0, st,
+        hipLaunchKernelGGL((m3_ssd_kernel<T, HD, DS, true, false>), dim3((unsigned)(batch * nh * (sp.nsc - 1))), dim3(HD * 4), 0, st,
                            ssm, kst, vst, (T *)y, (const T *)x, (const T *)K, (const T *)Q, dt, trap, a_val, D, sp, Tlen, nh, carry);
-    hipLaunchKernelGGL((m3_ssd_kernel<T, HD, DS, false>), dim3((unsigned)(batch * nh * sp.nsc)), dim3(HD * 4), 0, st, ssm, kst, vst,
+    hipLaunchKernelGGL((m3_ssd_kernel<T, HD, DS, false, false>), dim3((unsigned)(batch * nh * sp.nsc)), dim3(HD * 4), 0, st, ssm, kst, vst,
                        (T *)y, (const T *)x, (const T *)K, (const T *)Q, dt, trap, a_val, D, sp, Tlen, nh, carry);
 }
 
@@ -515,15 +601,23 @@ extern "C" int mrs_m3_ssd_fwd(void *stream, int dtype, float *ssm_state, float *
                               unsigned flags, int batch, int T, int nheads, int headdim, int d_state,
                               int chunk_size) {
     return mrs::m3_ssd_fwd_ex(stream, dtype, ssm_state, k_state, v_state, y, x, 0, K, Q, dt, trap, a_val, D, workspace,
-                              workspace_bytes, flags, batch, T, nheads, headdim, d_state, chunk_size);
+                              workspace_bytes, flags, batch, T, nheads, headdim, d_state, chunk_size, nullptr);
 }
 
 // x_stride = 0 means dense rows (d_inner); a wider stride needs 16-bit storage (the f32 route runs the recurrence kernel).
 int mrs::m3_ssd_fwd_ex(void *stream, int dtype, float *ssm_state, float *k_state, float *v_state, void *y, const void *x,
                        int64_t x_stride, const void *K, const void *Q, const float *dt,
                        const float *trap, const float *a_val, const float *D, void *workspace, size_t workspace_bytes,
-                       unsigned flags, int batch, int T, int nheads, int headdim, int d_state, int chunk_size) {
+                       unsigned flags, int batch, int T, int nheads, int headdim, int d_state, int chunk_size, const SsdGenArgs *gen) {
     const char *fn = "mrs_m3_ssd_fwd";
+    if (gen) {   // K and Q formed inside the kernel: K and Q themselves are not read
+        if (dtype == MRS_F32 || headdim != 64 || d_state != 64 || gen->n_rope % 4 != 0 || 2 * gen->n_rope > d_state || gen->bc_stride % 4 != 0 ||
+            !gen->bn || !gen->cn || !gen->angle || !gen->b_bias || !gen->c_bias || !aligned(gen->bn, 16) || !aligned(gen->cn, 16) || !aligned(gen->angle, 16))
+            return fail(MRS_E_SHAPE, "%s: in-kernel K / Q needs 16-bit storage, headdim = d_state = 64, rope pairs in fours, aligned rows", fn);
+        if ((int64_t)T * std::max<int64_t>(gen->bc_stride, (int64_t)nheads * gen->n_rope) * 4 >= 0x7fffffffLL)
+            return fail(MRS_E_SHAPE, "%s: one batch row of the B / C rows or the angles exceeds 2^31 bytes", fn);
+        K = Q = x;   // placeholders for the checks below
+    }
     const int64_t di_ = (int64_t)nheads * headdim;
     if (x_stride == 0) x_stride = di_;
     if (x_stride < di_) return fail(MRS_E_SHAPE, "%s: row stride below d_inner", fn);
@@ -564,7 +658,11 @@ int mrs::m3_ssd_fwd_ex(void *stream, int dtype, float *ssm_state, float *k_state
     if (!aligned(x, 16) || !aligned(K, 16) || !aligned(Q, 16) || !aligned(ssm_state, 16) || !aligned(k_state, 16))
         return fail(MRS_E_ALIGN, "%s: x, K, Q, ssm_state, k_state must be 16-byte aligned", fn);
     // Super-chunk split when the caller's workspace holds it; otherwise one workgroup walks the whole sequence.
-    SsdSplit sp = {nullptr, nullptr, nullptr, 1, (T + kCS - 1) / kCS, x_stride};
+    SsdSplit sp = {nullptr, nullptr, nullptr, 1, (T + kCS - 1) / kCS, x_stride, nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0};
+    auto with_gen = [&](SsdSplit &o) {
+        if (gen) { o.g_bn = gen->bn; o.g_cn = gen->cn; o.g_ang = gen->angle; o.g_bb = gen->b_bias; o.g_cb = gen->c_bias; o.g_bcs = gen->bc_stride; o.g_nr = gen->n_rope; }
+    };
+    with_gen(sp);
     {
         int nsc, cps;
         ssd_plan(batch, T, nheads, nsc, cps);
@@ -572,7 +670,8 @@ int mrs::m3_ssd_fwd_ex(void *stream, int dtype, float *ssm_state, float *k_state
         const size_t need = ssd_split_bytes(batch, nheads, headdim, d_state, nsc, &o_dA, &o_init);
         if (nsc > 1 && workspace && workspace_bytes >= need && aligned(workspace, 16)) {
             char *ws = (char *)workspace;
-            sp = SsdSplit{(float *)ws, (float *)(ws + o_dA), (float *)(ws + o_init), nsc, cps, x_stride};
+            sp = SsdSplit{(float *)ws, (float *)(ws + o_dA), (float *)(ws + o_init), nsc, cps, x_stride, nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0};
+            with_gen(sp);
         }
     }
     if (dtype == MRS_BF16) return launch_ssd<bf16_t>(st, ssm_state, k_state, v_state, y, x, K, Q, dt, trap, a_val, D, sp, batch, T, nheads, headdim, d_state, carry);

@@ -158,7 +158,7 @@ def test_create_rejects_bad_configs():
 # ---- prefill ------------------------------------------------------------------------------------------
 
 PREFILL_CASES = [(0, 150, WeightDtype.F32), (1, 97, WeightDtype.F32), (2, 130, WeightDtype.F32),
-                 (0, 200, WeightDtype.BF16), (2, 200, WeightDtype.BF16), (1, 70, WeightDtype.F16)]
+                 (0, 200, WeightDtype.BF16), (2, 200, WeightDtype.BF16), (1, 70, WeightDtype.F16), (2, 333, WeightDtype.F16)]
 
 
 @pytest.mark.parametrize("ci,T,dtype", PREFILL_CASES)
@@ -228,3 +228,42 @@ def test_prefill_twice_continues_the_state_and_unsupported_chunk_shape_takes_the
         want = orc.m3_backbone_step(P, xs[0, t], st)
     assert scaled_err(last[0], want) < 5e-4
     eng.close()
+
+
+@pytest.mark.parametrize("dtype,T", [(WeightDtype.BF16, 1100), (WeightDtype.F16, 257)])
+def test_scan_that_forms_K_and_Q_itself_equals_the_separate_K_Q_pass(dtype, T, monkeypatch):
+    """headdim = d_state = 64, one group, 16-bit storage: the prefill's scan builds its K / Q tiles from the normalised
+    B / C rows and the angles.  With MRS_M3_NO_FUSED_KQ set the engine writes K and Q with the separate kernel instead;
+    both routes round the same K and Q to 16 bits (they differ by one fused multiply-add rounding in f32 before that), so
+    the two prefills agree far inside the 16-bit bar: last output, every state, and the steps after the handoff.
+    T covers the split into super-chunks (state-only pass) and a ragged last chunk."""
+    cfg = CONFIGS[2]
+    w = perturbed(cfg, 64, 91)
+    w.input_proj_w = np.zeros(0, np.float32)
+    B = 2
+    rng = np.random.default_rng(17)
+    xs = rng.standard_normal((B, T + 3, 64)).astype(np.float32)
+    res = {}
+    for route in ("fused", "separate"):
+        if route == "separate":
+            monkeypatch.setenv("MRS_M3_NO_FUSED_KQ", "1")
+        else:
+            monkeypatch.delenv("MRS_M3_NO_FUSED_KQ", raising=False)
+        print(f"case m3 prefill K/Q route={route} T={T} dtype={dtype}", flush=True)
+        eng = GpuMamba3Backbone.new_with_dtype(0, w, cfg, 64, B, dtype)
+        last = eng.prefill_sequence(xs[:, :T]).copy()
+        states = [eng.download_state(l) for l in range(cfg.n_layers)]
+        after = np.stack([eng.step(xs[:, T + i]).copy() for i in range(3)])
+        res[route] = (last, states, after)
+        eng.close()
+    fa, se = res["fused"], res["separate"]
+    assert np.isfinite(fa[0]).all()
+    assert scaled_err(fa[0], se[0]) < 1e-2 and cosine(fa[0].ravel(), se[0].ravel()) >= 0.9999
+    assert scaled_err(fa[2], se[2]) < 1e-2
+    for l in range(cfg.n_layers):
+        for a, b in zip(fa[1][l][:3], se[1][l][:3]):      # ssm, k, v
+            assert scaled_err(a, b) < 1e-2, l
+        if l == 0:   # the first layer's angles see the same input on both routes
+            assert np.array_equal(fa[1][l][3], se[1][l][3])
+        else:        # later layers accumulate the 16-bit differences of the layers below over T steps
+            assert np.max(np.abs(np.sin(fa[1][l][3]) - np.sin(se[1][l][3]))) < 0.05
