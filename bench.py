@@ -487,7 +487,7 @@ def main():
                     help="comma list of the extras to run: c1, lm, published, m1_kernels, m3, m3_engine (for profiling one leg at a time)")
     args = ap.parse_args()
     legs = {x.strip() for x in args.legs.split(",") if x.strip()}
-    unknown = legs - {"c1", "lm", "published", "m1_kernels", "m3", "m3_engine"}
+    unknown = legs - {"c1", "lm", "published", "m1_kernels", "m3", "m3_engine", "m3_prefill"}
     if unknown:
         print(f"bench.py: unknown --legs entries {sorted(unknown)}", file=sys.stderr)
         sys.exit(2)
@@ -536,10 +536,12 @@ def main():
             extras["reference_published_configs"] = published_configs_leg()
         if "m1_kernels" in legs:
             extras["m1_kernels_130m_shape_bf16"] = m1_kernels_leg()
-        if "m3" in legs or "m3_engine" in legs:
+        if "m3" in legs or "m3_engine" in legs or "m3_prefill" in legs:
             extras["mamba3_768_bf16"] = m3_leg() if "m3" in legs else {}
         if "m3_engine" in legs:
             extras["mamba3_768_bf16"]["backbone"] = m3_engine_leg()
+        elif "m3_prefill" in legs:   # the backbone's prefill alone (not a default leg: the command behind its profile)
+            extras["mamba3_768_bf16"]["backbone"] = m3_engine_leg(batches=())
         if args.big:
             extras["lm_2.8b_shape_bf16"] = lm_leg("2.8b-shape", dict(d_model=2560, d_state=16, d_conv=4, expand=2, n_layers=64), 50280,
                                                   (4, 4096), [1, 16, 128], 128)

@@ -107,6 +107,7 @@ struct SsdSplit {
     const float *g_bn, *g_cn, *g_ang, *g_bb, *g_cb;
     int64_t g_bcs;
     int g_nr;
+    int g_groups;         // batch rows x super-chunks of the launch (set per launch)
 };
 
 // Cross-lane moves on the data-parallel-primitive path of the vector ALU (no LDS round trip, unlike the shuffle
@@ -152,8 +153,18 @@ __global__ __launch_bounds__(HD * 4) __attribute__((amdgpu_waves_per_eu(HD == 64
     __shared__ SsdSmem<HD, DS> sm;
 
     const int nscg = STATE_ONLY ? sp.nsc - 1 : sp.nsc;   // the state-only pass skips the last super-chunk
-    const int bhi = blockIdx.x / nscg, sc = blockIdx.x - bhi * nscg;
-    const int b = bhi / nh, h = bhi - b * nh;
+    int b, h, sc;
+    if constexpr (GEN) {
+        // Workgroups go to the 8 L2 domains of the chip round-robin by index.  The heads of one (batch row, super-chunk)
+        // read the same B / C rows, and neighbouring heads share the cache lines of the angle rows: all of them take
+        // indices of one residue mod 8, so they meet in one L2.  The grid is padded to whole rounds of 8 groups.
+        const int slot = blockIdx.x >> 3, g = (slot / nh) * 8 + (blockIdx.x & 7);
+        if (g >= sp.g_groups) return;   // padding: the whole workgroup leaves before any barrier
+        h = slot % nh; b = g / nscg; sc = g - b * nscg;
+    } else {
+        const int bhi = blockIdx.x / nscg;
+        sc = blockIdx.x - bhi * nscg; b = bhi / nh; h = bhi - b * nh;
+    }
     const int tid = threadIdx.x, l = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave index, in a scalar register: what depends on it alone branches without masks
     const int lr = l & 15, lg = l >> 4;            // fragment row/col index and k-group
@@ -538,10 +549,14 @@ static void launch_ssd_shape(hipStream_t st, float *ssm, float *kst, float *vst,
                              const float *a_val, const float *D, SsdSplit sp, int batch, int Tlen, int nh, int carry) {
     if constexpr (HD == 64 && DS == 64) {   // the one shape the in-kernel K / Q route is built for
         if (sp.g_bn) {
-            if (sp.nsc > 1)
-                hipLaunchKernelGGL((m3_ssd_kernel<T, HD, DS, true, true>), dim3((unsigned)(batch * nh * (sp.nsc - 1))), dim3(HD * 4), 0, st,
+            auto padded = [&](int groups) { return dim3((unsigned)((groups + 7) / 8 * 8 * nh)); };
+            if (sp.nsc > 1) {
+                sp.g_groups = batch * (sp.nsc - 1);
+                hipLaunchKernelGGL((m3_ssd_kernel<T, HD, DS, true, true>), padded(sp.g_groups), dim3(HD * 4), 0, st,
                                    ssm, kst, vst, (T *)y, (const T *)x, (const T *)K, (const T *)Q, dt, trap, a_val, D, sp, Tlen, nh, carry);
-            hipLaunchKernelGGL((m3_ssd_kernel<T, HD, DS, false, true>), dim3((unsigned)(batch * nh * sp.nsc)), dim3(HD * 4), 0, st, ssm, kst, vst,
+            }
+            sp.g_groups = batch * sp.nsc;
+            hipLaunchKernelGGL((m3_ssd_kernel<T, HD, DS, false, true>), padded(sp.g_groups), dim3(HD * 4), 0, st, ssm, kst, vst,
                                (T *)y, (const T *)x, (const T *)K, (const T *)Q, dt, trap, a_val, D, sp, Tlen, nh, carry);
             return;
         }
@@ -658,7 +673,7 @@ int mrs::m3_ssd_fwd_ex(void *stream, int dtype, float *ssm_state, float *k_state
     if (!aligned(x, 16) || !aligned(K, 16) || !aligned(Q, 16) || !aligned(ssm_state, 16) || !aligned(k_state, 16))
         return fail(MRS_E_ALIGN, "%s: x, K, Q, ssm_state, k_state must be 16-byte aligned", fn);
     // Super-chunk split when the caller's workspace holds it; otherwise one workgroup walks the whole sequence.
-    SsdSplit sp = {nullptr, nullptr, nullptr, 1, (T + kCS - 1) / kCS, x_stride, nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0};
+    SsdSplit sp = {nullptr, nullptr, nullptr, 1, (T + kCS - 1) / kCS, x_stride, nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0, 0};
     auto with_gen = [&](SsdSplit &o) {
         if (gen) { o.g_bn = gen->bn; o.g_cn = gen->cn; o.g_ang = gen->angle; o.g_bb = gen->b_bias; o.g_cb = gen->c_bias; o.g_bcs = gen->bc_stride; o.g_nr = gen->n_rope; }
     };
@@ -670,7 +685,7 @@ int mrs::m3_ssd_fwd_ex(void *stream, int dtype, float *ssm_state, float *k_state
         const size_t need = ssd_split_bytes(batch, nheads, headdim, d_state, nsc, &o_dA, &o_init);
         if (nsc > 1 && workspace && workspace_bytes >= need && aligned(workspace, 16)) {
             char *ws = (char *)workspace;
-            sp = SsdSplit{(float *)ws, (float *)(ws + o_dA), (float *)(ws + o_init), nsc, cps, x_stride, nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0};
+            sp = SsdSplit{(float *)ws, (float *)(ws + o_dA), (float *)(ws + o_init), nsc, cps, x_stride, nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0, 0};
             with_gen(sp);
         }
     }
