@@ -278,6 +278,13 @@ __global__ __launch_bounds__(HD * 4) __attribute__((amdgpu_waves_per_eu(HD == 64
     auto prefetch = [&](Pre &r, int c) {
         const int t0 = c * kCS;
         const unsigned kq_c = (unsigned)t0 * (unsigned)kq_row * es, x_c = (unsigned)t0 * (unsigned)sp.x_stride * es, sc_c = (unsigned)t0 * (unsigned)nh * 4u;
+        // The step scalars go first: loads return in order, and the compiler moves the first uses of these small values
+        // ahead of the next request, so whoever waits for them must not wait for the tiles requested after them as well.
+        r.rdt = slab_ldf(dtbuf, sc_voff + sc_c, 0);
+        r.rtr = slab_ldf(trbuf, sc_voff + sc_c, 0);
+        r.ra = slab_ldf(abuf, sc_voff + sc_c, 0);
+        r.rdtn = slab_ldf(dtbuf, sc_voff + sc_c + (unsigned)nh * 4u, 0);   // the shifted gamma needs the step after (zero past the row)
+        r.rtrn = slab_ldf(trbuf, sc_voff + sc_c + (unsigned)nh * 4u, 0);
         if constexpr (GEN) {
             const unsigned bc_c = (unsigned)t0 * (unsigned)sp.g_bcs * 4u, ang_c = (unsigned)t0 * (unsigned)(nh * sp.g_nr) * 4u;
 #pragma unroll
@@ -299,11 +306,6 @@ __global__ __launch_bounds__(HD * 4) __attribute__((amdgpu_waves_per_eu(HD == 64
         }
         r.rx[0] = slab_ld128(xbuf, x_voff[0] + x_c, 0);
         r.rx[1] = slab_ld128(xbuf, x_voff[1] + x_c, 0);
-        r.rdt = slab_ldf(dtbuf, sc_voff + sc_c, 0);
-        r.rtr = slab_ldf(trbuf, sc_voff + sc_c, 0);
-        r.ra = slab_ldf(abuf, sc_voff + sc_c, 0);
-        r.rdtn = slab_ldf(dtbuf, sc_voff + sc_c + (unsigned)nh * 4u, 0);   // the shifted gamma needs the step after (zero past the row)
-        r.rtrn = slab_ldf(trbuf, sc_voff + sc_c + (unsigned)nh * 4u, 0);
     };
 
     // One chunk from the registers of `r`; once they are in LDS the chunk c_next is requested into them.
