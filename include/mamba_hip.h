@@ -254,13 +254,16 @@ MRS_API int mrs_backbone_capture_graph(mrs_backbone *bb);
 /* alloc_prefill_scratch / prefill_sequence[_mixed] (inference.rs:1752-1831; src/mamba_ssm/gpu/prefill.rs:676-1049):
  * input [batch, T, input_dim] f32 on the host; the whole sequence runs through the layers, the state ends
  * positioned after token T (so step continues), output_last (may be NULL) receives norm_f of the last position
- * [batch, d_model].  One sequence length per engine (scratch is sized once). T >= 2. */
+ * [batch, d_model].  T >= 2.  The scratch follows T: kept while T repeats, released and re-made (device synchronise +
+ * hipFree/hipMalloc) when a call brings another T -- the reference allocates it per call (src/module/gpu_lm.rs:543-551). */
 MRS_API int mrs_backbone_alloc_prefill_scratch(mrs_backbone *bb, int T);
 MRS_API int mrs_backbone_prefill_sequence(mrs_backbone *bb, const float *input, int T, float *output_last);
 /* Same, input already on the device ([batch,T,input_dim] f32); does not synchronise. */
 MRS_API int mrs_backbone_prefill_device(mrs_backbone *bb, const float *input_dev, int T);
 /* temporal_ptr / input buffer / stream accessors (inference.rs:1717-1737) and state access for tests. */
 MRS_API float *mrs_backbone_temporal_ptr(mrs_backbone *bb);
+/* download_temporal (inference.rs:1727-1737): the last step's / prefill's final-norm rows [batch, d_model] to the host; synchronises. */
+MRS_API int mrs_backbone_download_temporal(mrs_backbone *bb, float *out);
 MRS_API float *mrs_backbone_input_ptr(mrs_backbone *bb);
 MRS_API float *mrs_backbone_prefill_input_ptr(mrs_backbone *bb);
 MRS_API void *mrs_backbone_stream(mrs_backbone *bb);
@@ -391,7 +394,7 @@ MRS_API int mrs_m3_backbone_download_state(mrs_m3_backbone *bb, int layer, float
  * split/bcnorm/bias/rope glue of kernels/mamba3_ops.cu in one kernel, mrs_m3_ssd_fwd with carried state, gate, out_proj),
  * continuing from the engine's state and leaving it positioned for step().  The reference's GPU forward of a layer over T
  * is gpu_forward_mamba3_layer (src/mamba3_siso/gpu/forward.rs:27); its CPU prefill mamba3_siso/cpu/prefill.rs:151-572.
- * One sequence length per engine (scratch is allocated on first use or by alloc_prefill_scratch). */
+ * The scratch follows T: allocated on first use or by alloc_prefill_scratch, re-made when a call brings another T. */
 MRS_API int mrs_m3_backbone_alloc_prefill_scratch(mrs_m3_backbone *bb, int T);
 MRS_API int mrs_m3_backbone_prefill_sequence(mrs_m3_backbone *bb, const float *input, int T, float *out_last);
 MRS_API int mrs_m3_backbone_prefill_device(mrs_m3_backbone *bb, int T);

@@ -53,6 +53,7 @@ def _bind():
         "mrs_backbone_prefill_sequence": (c_int, [P, _FP, c_int, _FP]),
         "mrs_backbone_prefill_device": (c_int, [P, P, c_int]),
         "mrs_backbone_temporal_ptr": (P, [P]),
+        "mrs_backbone_download_temporal": (c_int, [P, _FP]),
         "mrs_backbone_input_ptr": (P, [P]),
         "mrs_backbone_prefill_input_ptr": (P, [P]),
         "mrs_backbone_stream": (P, [P]),
@@ -198,6 +199,12 @@ class GpuMambaBackbone:
 
     def temporal_ptr(self) -> int:
         return _bind().mrs_backbone_temporal_ptr(self._h)
+
+    def download_temporal(self) -> np.ndarray:
+        """download_temporal (inference.rs:1727-1737): final-norm rows of the last step / prefill, [batch, d_model]."""
+        out = np.empty((self.batch, self.cfg.d_model), np.float32)
+        _call("mrs_backbone_download_temporal", self._h, _fp(out))
+        return out
 
     def temporal_dtype(self) -> WeightDtype:
         return WeightDtype.F32

@@ -267,6 +267,7 @@ struct mrs_backbone {
     std::vector<LayerDev> layers;
     float *input_proj_w, *input_proj_b, *norm_f;
     std::vector<void *> allocs;
+    std::vector<void *> prefill_allocs;  // the prefill scratch alone: released and re-made when the sequence length changes
     float *conv_state, *ssm_state;
     float *d_input, *temporal;
     void *temporal_t;  // decode: temporal once more in the storage type (16-bit engines), the LM head's operand
@@ -639,6 +640,7 @@ extern "C" void mrs_backbone_destroy(mrs_backbone *bb) {
     if (bb->graph_exec) hipGraphExecDestroy(bb->graph_exec);
     if (bb->graph) hipGraphDestroy(bb->graph);
     for (void *p : bb->allocs) hipFree(p);
+    for (void *p : bb->prefill_allocs) hipFree(p);
     if (bb->blas) rocblas_destroy_handle(bb->blas);
     if (bb->stream) hipStreamDestroy(bb->stream);
     delete bb;
@@ -706,21 +708,35 @@ extern "C" int mrs_backbone_capture_graph(mrs_backbone *bb) {
     return MRS_OK;
 }
 
+// Prefill scratch follows the sequence length of the call, as the reference allocates it per call
+// (src/module/gpu_lm.rs:543-551): the buffers are kept while T stays the same and re-made when it changes.
+// Not for use while a capture is open on the engine's stream (it allocates and frees).
+static void release_prefill_scratch(mrs_backbone *bb) {
+    if (bb->stream) hipStreamSynchronize(bb->stream);   // no kernel may still be reading the old buffers
+    for (void *p : bb->prefill_allocs) hipFree(p);
+    bb->prefill_allocs.clear();
+    bb->prefill_s = Scratch();
+    bb->prefill_in = nullptr;
+}
+
 extern "C" int mrs_backbone_alloc_prefill_scratch(mrs_backbone *bb, int T) {
     if (!bb) return fail(MRS_E_NULL, "mrs_backbone_alloc_prefill_scratch: null engine");
-    if (T < 1) return fail(MRS_E_SHAPE, "mrs_backbone_alloc_prefill_scratch: T=%d", T);
+    if (T < 2) return fail(MRS_E_SHAPE, "mrs_backbone_alloc_prefill_scratch: T=%d (prefill needs T >= 2; use step for one token)", T);
+    if ((int64_t)bb->batch * T * bb->di > 0x7fffffffLL) return fail(MRS_E_SHAPE, "prefill: batch*T*d_inner exceeds i32");
     if (bb->prefill_s.rows && bb->prefill_s.T == T) return MRS_OK;
-    if (bb->prefill_s.rows) return fail(MRS_E_SHAPE, "prefill scratch already sized for T=%d (one sequence length per engine)", bb->prefill_s.T);
-    MRS_TRY(alloc_scratch(bb, &bb->prefill_s, (int64_t)bb->batch * T, T));
-    MRS_TRY(dev_alloc(bb, (void **)&bb->prefill_in, (size_t)bb->batch * T * bb->input_dim * 4));
-    return MRS_OK;
+    if (bb->prefill_s.rows) release_prefill_scratch(bb);
+    const size_t mark = bb->allocs.size();
+    int rc = alloc_scratch(bb, &bb->prefill_s, (int64_t)bb->batch * T, T);
+    if (!rc) rc = dev_alloc(bb, (void **)&bb->prefill_in, (size_t)bb->batch * T * bb->input_dim * 4);
+    bb->prefill_allocs.assign(bb->allocs.begin() + mark, bb->allocs.end());
+    bb->allocs.resize(mark);
+    if (rc) release_prefill_scratch(bb);
+    return rc;
 }
 
 extern "C" int mrs_backbone_prefill_device(mrs_backbone *bb, const float *input_dev, int T) {
     if (!bb || !input_dev) return fail(MRS_E_NULL, "mrs_backbone_prefill_device: null pointer");
     MRS_TRY(mrs_backbone_alloc_prefill_scratch(bb, T));
-    if ((int64_t)bb->batch * T * bb->di > 0x7fffffffLL) return fail(MRS_E_SHAPE, "prefill: batch*T*d_inner exceeds i32");
-    if (T == 1) return fail(MRS_E_SHAPE, "prefill needs T >= 2; use step for one token");
     MRS_TRY(project_input(bb, bb->prefill_s.residual, input_dev, (int64_t)bb->batch * T));
     return run_layers(bb, &bb->prefill_s, T);
 }
@@ -737,6 +753,12 @@ extern "C" int mrs_backbone_prefill_sequence(mrs_backbone *bb, const float *inpu
 
 extern "C" void *mrs_backbone_stream(mrs_backbone *bb) { return bb ? (void *)bb->stream : nullptr; }
 extern "C" float *mrs_backbone_temporal_ptr(mrs_backbone *bb) { return bb ? bb->temporal : nullptr; }
+extern "C" int mrs_backbone_download_temporal(mrs_backbone *bb, float *out) {
+    if (!bb || !out) return fail(MRS_E_NULL, "mrs_backbone_download_temporal: null pointer");
+    MRS_HIP(hipMemcpyAsync(out, bb->temporal, (size_t)bb->batch * bb->cfg.d_model * 4, hipMemcpyDeviceToHost, bb->stream));
+    MRS_HIP(hipStreamSynchronize(bb->stream));
+    return MRS_OK;
+}
 extern "C" float *mrs_backbone_input_ptr(mrs_backbone *bb) { return bb ? bb->d_input : nullptr; }
 extern "C" float *mrs_backbone_prefill_input_ptr(mrs_backbone *bb) { return bb ? bb->prefill_in : nullptr; }
 extern "C" int mrs_backbone_sync(mrs_backbone *bb) {
@@ -885,7 +907,9 @@ extern "C" int mrs_lm_create(mrs_lm **out, mrs_backbone *bb, const float *embed,
 // as [vocab_padded, d_model] like the embedding table, so the logits GEMM is the same call on another pointer.
 extern "C" int mrs_lm_set_untied_head(mrs_lm *lm, const float *lm_head) {
     if (!lm || !lm_head) return fail(MRS_E_NULL, "mrs_lm_set_untied_head: null pointer");
-    if (lm->graph_ready) return fail(MRS_E_SHAPE, "mrs_lm_set_untied_head: set the head before capturing the graph");
+    // both graphs bake the head's table pointer in at capture time
+    if (lm->graph_ready || lm->gen_graph_ready)
+        return fail(MRS_E_SHAPE, "mrs_lm_set_untied_head: set the head before capturing a graph (decode_step capture or a first generate call)");
     const LmHooks *bb = &lm->eng;
     const size_t es = esize(lm->dtype), ne = (size_t)lm->vocab_padded * lm->dm;
     std::vector<float> host;

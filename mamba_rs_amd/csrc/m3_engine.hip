@@ -507,6 +507,7 @@ struct mrs_m3_backbone {
     rocblas_handle blas;
     std::vector<Layer3> layers;
     std::vector<void *> allocs;
+    std::vector<void *> pf_allocs;   // the prefill scratch alone: released and re-made when the sequence length changes
     float *input_proj_w, *input_proj_b, *norm_f;
     float *ssm, *kst, *vst, *angle;          // [L][batch]...
     float *d_input, *temporal, *residual, *proj, *partials;
@@ -641,6 +642,7 @@ extern "C" void mrs_m3_backbone_destroy(mrs_m3_backbone *bb) {
     if (bb->graph_exec) hipGraphExecDestroy(bb->graph_exec);
     if (bb->graph) hipGraphDestroy(bb->graph);
     for (void *p : bb->allocs) hipFree(p);
+    for (void *p : bb->pf_allocs) hipFree(p);
     if (bb->blas) rocblas_destroy_handle(bb->blas);
     if (bb->stream) hipStreamDestroy(bb->stream);
     delete bb;
@@ -802,12 +804,32 @@ extern "C" int mrs_m3_backbone_capture_graph(mrs_m3_backbone *bb) {
 }
 
 // ---- prefill -----------------------------------------------------------------------------------------
+// Prefill scratch follows the sequence length of the call (the reference allocates it per call,
+// src/module/gpu_lm3.rs): kept while T stays the same, released and re-made when it changes.  Not for use while a
+// capture is open on the engine's stream.
+static int alloc_prefill_scratch3(mrs_m3_backbone *bb, int T);
 extern "C" int mrs_m3_backbone_alloc_prefill_scratch(mrs_m3_backbone *bb, int T) {
     const char *fn = "mrs_m3_backbone_alloc_prefill_scratch";
     if (!bb) return fail(MRS_E_NULL, "%s: null engine", fn);
     if (T < 1) return fail(MRS_E_SHAPE, "%s: T=%d", fn, T);
     if (bb->pf_T == T) return MRS_OK;
-    if (bb->pf_T) return fail(MRS_E_SHAPE, "%s: scratch already allocated for T=%d (one sequence length per engine)", fn, bb->pf_T);
+    auto release = [&]() {
+        hipStreamSynchronize(bb->stream);   // no kernel may still be reading the old buffers
+        for (void *p : bb->pf_allocs) hipFree(p);
+        bb->pf_allocs.clear();
+        bb->pf_T = 0; bb->pf_in = nullptr;
+    };
+    if (bb->pf_T) release();
+    const size_t mark = bb->allocs.size();
+    const int rc = alloc_prefill_scratch3(bb, T);
+    bb->pf_allocs.assign(bb->allocs.begin() + mark, bb->allocs.end());
+    bb->allocs.resize(mark);
+    if (rc) release();
+    return rc;
+}
+
+static int alloc_prefill_scratch3(mrs_m3_backbone *bb, int T) {
+    const char *fn = "mrs_m3_backbone_alloc_prefill_scratch";
     const mrs_m3_config &c = bb->cfg;
     const size_t rows = (size_t)bb->batch * T, es = esize3(bb->dtype), dm = c.d_model, di = bb->di, nh = bb->nh, ds = c.d_state, ip = bb->ip;
     if ((int64_t)rows * ip > 0x7fffffffLL) return fail(MRS_E_SHAPE, "%s: batch*T*in_proj_dim exceeds i32", fn);

@@ -209,9 +209,10 @@ def test_engine_rejects_bad_config():
     eng = GpuMambaBackbone.new(0, w, cfg, 10, 1)
     with pytest.raises(ValueError):
         eng.step(np.zeros(3, np.float32))
-    eng.alloc_prefill_scratch(16)
     with pytest.raises(MambaHipError):
-        eng.alloc_prefill_scratch(32)                     # one sequence length per engine
+        eng.alloc_prefill_scratch(1)                      # one token is a step, not a prefill
+    eng.alloc_prefill_scratch(16)
+    eng.alloc_prefill_scratch(32)                         # the scratch follows the sequence length
     eng.close()
 
 
