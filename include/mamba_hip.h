@@ -107,6 +107,24 @@ MRS_API int mrs_ssm_scan_fwd_ex(void *stream, int dtype, float *h, void *y, cons
                         void *workspace, size_t workspace_bytes,
                         int batch, int T, int d_inner, int d_state);
 
+/* mrs_ssm_scan_fwd_ex without the workspace argument, for callers that cannot allocate device memory: code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
+ * reference (whose launch site allocates nothing either, because its kernel keeps no chunk summaries in memory).
+ * The chunk summaries of the T-split route go to a device buffer the library holds itself -- one
+ * MRS_SCAN_STATIC_SCRATCH_BYTES block per GPU, resident until the process ends -- so the call allocates nothing
+ * and frees nothing.  Same arguments, routes and results as mrs_ssm_scan_fwd_ex given a workspace of that size.
+ *   - A shape with mrs_ssm_scan_workspace_bytes() > MRS_SCAN_STATIC_SCRATCH_BYTES is refused (MRS_E_WORKSPACE);
+ *     the benchmark shapes (8 x 2048 x 1536 and 4 x 4096 x 5120, d_state 16) need 15.4 MB and 15.6 MB.
+ *   - The first call on a GPU looks the buffer's address up (hipGetSymbolAddress, no allocation); make that call
+ *     outside a graph capture.
+ *   - All calls on one GPU share the one buffer: two calls that overlap in time on the same GPU (different
+ *     streams, or graphs replayed side by side) race.  Serialise them or use mrs_ssm_scan_fwd_ex. */
+#define MRS_SCAN_STATIC_SCRATCH_BYTES (32u << 20)
+MRS_API int mrs_ssm_scan_fwd_static(void *stream, int dtype, float *h, void *y, const void *delta, const void *u,
+                        const void *B, const void *C, int64_t bc_stride, const float *a_neg,
+                        const float *D, const void *gate, int64_t gate_stride, unsigned flags,
+                        int batch, int T, int d_inner, int d_state);
+
 /* ---- Mamba-1 selective scan, one step (decode) ------------------------------
  * ssm_step_forward_{..} (kernels/mamba_ssm.cu:26-116; src/mamba_ssm/gpu/inference.rs:669-698):
  * delta,u,y [batch,d_inner]; B,C [batch,d_state]. */

@@ -12,6 +12,7 @@
 // whole sequence and is written back once.
 #include "common.hpp"
 #include <stdlib.h>
+#include <mutex>
 
 namespace mrs {
 
@@ -692,25 +693,25 @@ extern "C" size_t mrs_ssm_scan_workspace_bytes(int batch, int T, int d_inner, in
     return (bytes + 255) & ~(size_t)255;
 }
 
-extern "C" int mrs_ssm_scan_fwd_ex(void *stream, int dtype, float *h, void *y, const void *delta,
-                                   const void *u, const void *B, const void *C, int64_t bc_stride,
-                                   const float *a_neg, const float *D, const void *gate, int64_t gate_stride,
-                                   unsigned flags, void *workspace, size_t workspace_bytes, int batch, int T,
-                                   int d_inner, int d_state) {
-    int rc = scan_check("mrs_ssm_scan_fwd_ex", dtype, h, y, delta, u, B, C, a_neg, D, bc_stride, batch, T, d_inner, d_state);
+// Shared body of the scan entry points: argument checks, route choice, launches.  `fn` names the caller in messages.
+static int scan_dispatch(const char *fn, void *stream, int dtype, float *h, void *y, const void *delta, const void *u,
+                         const void *B, const void *C, int64_t bc_stride, const float *a_neg, const float *D,
+                         const void *gate, int64_t gate_stride, unsigned flags, void *workspace, size_t workspace_bytes,
+                         int batch, int T, int d_inner, int d_state) {
+    int rc = scan_check(fn, dtype, h, y, delta, u, B, C, a_neg, D, bc_stride, batch, T, d_inner, d_state);
     if (rc) return rc;
     int gate_mode = 0;
     if ((flags & MRS_GATE_PREACT) && (flags & MRS_GATE_SILU))
-        return fail(MRS_E_SHAPE, "mrs_ssm_scan_fwd_ex: MRS_GATE_PREACT and MRS_GATE_SILU are exclusive");
+        return fail(MRS_E_SHAPE, "%s: MRS_GATE_PREACT and MRS_GATE_SILU are exclusive", fn);
     if (flags & MRS_GATE_PREACT) gate_mode = 1;
     if (flags & MRS_GATE_SILU) gate_mode = 2;
-    if (gate_mode && !gate) return fail(MRS_E_NULL, "mrs_ssm_scan_fwd_ex: gate flag set but gate is NULL");
+    if (gate_mode && !gate) return fail(MRS_E_NULL, "%s: gate flag set but gate is NULL", fn);
     if (gate_stride == 0) gate_stride = d_inner;
-    if (gate_mode && gate_stride < d_inner) return fail(MRS_E_SHAPE, "mrs_ssm_scan_fwd_ex: gate_stride=%lld < d_inner=%d", (long long)gate_stride, d_inner);
+    if (gate_mode && gate_stride < d_inner) return fail(MRS_E_SHAPE, "%s: gate_stride=%lld < d_inner=%d", fn, (long long)gate_stride, d_inner);
     const bool s4d = (flags & MRS_A_S4D_REAL) != 0;
     hipStream_t st = as_stream(stream);
     if ((flags & MRS_FORCE_SEQUENTIAL) && (flags & MRS_FORCE_PARALLEL))
-        return fail(MRS_E_SHAPE, "mrs_ssm_scan_fwd_ex: MRS_FORCE_SEQUENTIAL and MRS_FORCE_PARALLEL are exclusive");
+        return fail(MRS_E_SHAPE, "%s: MRS_FORCE_SEQUENTIAL and MRS_FORCE_PARALLEL are exclusive", fn);
     // T-split route: d_state 16, rows of B/C readable as packed dwords, a workspace to put the chunk summaries in.
     const size_t es = (dtype == MRS_F32) ? 4 : 2;
     const bool rows_ok = aligned(B, 4) && aligned(C, 4) && (bc_stride * es) % 4 == 0;
@@ -725,17 +726,71 @@ extern "C" int mrs_ssm_scan_fwd_ex(void *stream, int dtype, float *h, void *y, c
         if (plan.nchunk < 2 || (T <= 256 && pairs >= 1024 && !(flags & MRS_FORCE_PARALLEL))) split = false;
     }
     if ((flags & MRS_FORCE_PARALLEL) && !split && d_state == 16 && T >= 64)
-        return fail(MRS_E_WORKSPACE, "mrs_ssm_scan_fwd_ex: MRS_FORCE_PARALLEL needs a workspace and 4-byte aligned B/C rows");
+        return fail(MRS_E_WORKSPACE, "%s: MRS_FORCE_PARALLEL needs a workspace and 4-byte aligned B/C rows", fn);
     if (split) {
         const size_t need = split_workspace_bytes(batch, T, d_inner, plan.nchunk);
         if (workspace_bytes < need)
-            return fail(MRS_E_WORKSPACE, "mrs_ssm_scan_fwd_ex: workspace %zu bytes < %zu needed", workspace_bytes, need);
-        if (!aligned(workspace, 256)) return fail(MRS_E_ALIGN, "mrs_ssm_scan_fwd_ex: workspace must be 256-byte aligned");
+            return fail(MRS_E_WORKSPACE, "%s: workspace %zu bytes < %zu needed", fn, workspace_bytes, need);
+        if (!aligned(workspace, 256)) return fail(MRS_E_ALIGN, "%s: workspace must be 256-byte aligned", fn);
         MRS_DISPATCH_DTYPE(dtype, T_, return launch_split<T_>(st, s4d, gate_mode, h, y, delta, u, B, C, bc_stride, a_neg, D, gate, gate_stride,
                                                              (float *)workspace, plan, batch, T, d_inner));
     }
     MRS_DISPATCH_DTYPE(dtype, T_, return launch_seq<T_>(st, s4d, gate_mode, h, y, delta, u, B, C, bc_stride, a_neg, D, gate, gate_stride, batch, T, d_inner, d_state));
     return MRS_OK;
+}
+
+extern "C" int mrs_ssm_scan_fwd_ex(void *stream, int dtype, float *h, void *y, const void *delta,
+                                   const void *u, const void *B, const void *C, int64_t bc_stride,
+                                   const float *a_neg, const float *D, const void *gate, int64_t gate_stride,
+                                   unsigned flags, void *workspace, size_t workspace_bytes, int batch, int T,
+                                   int d_inner, int d_state) {
+    return scan_dispatch("mrs_ssm_scan_fwd_ex", stream, dtype, h, y, delta, u, B, C, bc_stride, a_neg, D, gate, gate_stride, flags,
+                         workspace, workspace_bytes, batch, T, d_inner, d_state);
+}
+
+// ---- the scan without any allocation: chunk summaries in a buffer the library itself holds ---------------------------
+// File-scope device array, one copy per GPU the library runs on, held until the process ends.  In host code the name is
+// only a handle for hipGetSymbolAddress; kernels and every other use get the per-device address looked up below.
+constexpr size_t kStaticScanScratchBytes = MRS_SCAN_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScanScratchBytes];
+
+constexpr int kMaxDevices = 64;
+static void *g_scratch_ptr[kMaxDevices];   // device address of `scratch` on each GPU, looked up once with that GPU current
+static std::mutex g_scratch_mu;
+
+static int static_scratch_for_current_device(const char *fn, void **out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail(MRS_E_HIP, "%s: hipGetDevice: %s", fn, hipGetErrorString(e));
+    if (dev < 0 || dev >= kMaxDevices) return fail(MRS_E_HIP, "%s: device ordinal %d outside 0..%d", fn, dev, kMaxDevices - 1);
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) return fail(MRS_E_HIP, "%s: hipGetSymbolAddress(scratch) on device %d: %s", fn, dev, hipGetErrorString(e));
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return MRS_OK;
+}
+
+extern "C" int mrs_ssm_scan_fwd_static(void *stream, int dtype, float *h, void *y, const void *delta,
+                                       const void *u, const void *B, const void *C, int64_t bc_stride,
+                                       const float *a_neg, const float *D, const void *gate, int64_t gate_stride,
+                                       unsigned flags, int batch, int T, int d_inner, int d_state) {
+    const char *fn = "mrs_ssm_scan_fwd_static";
+    // the size test comes first and touches no GPU: a shape whose chunk summaries do not fit is refused, never shrunk
+    const size_t need = mrs_ssm_scan_workspace_bytes(batch, T, d_inner, d_state);
+    if (need > kStaticScanScratchBytes)
+        return fail(MRS_E_WORKSPACE, "%s: this shape needs %zu bytes of chunk summaries, the built-in buffer holds %zu; use mrs_ssm_scan_fwd_ex with a workspace",
+                    fn, need, kStaticScanScratchBytes);
+    void *ws = nullptr;
+    int rc = static_scratch_for_current_device(fn, &ws);
+    if (rc) return rc;
+    // Every float the second pass reads from the buffer is written by the first pass of the same call (chunk states,
+    // step sums, the copy of h, the regrouped B and widened C rows), so nothing has to start at zero.
+    return scan_dispatch(fn, stream, dtype, h, y, delta, u, B, C, bc_stride, a_neg, D, gate, gate_stride, flags, ws,
+                         kStaticScanScratchBytes, batch, T, d_inner, d_state);
 }
 
 extern "C" int mrs_ssm_scan_fwd(void *stream, int dtype, float *h, void *y, const void *delta,

@@ -74,11 +74,15 @@ def ssm_scan_workspace_bytes(batch: int, T: int, d_inner: int, d_state: int) -> 
     return int(_lib.load().mrs_ssm_scan_workspace_bytes(batch, T, d_inner, d_state))
 
 
-def ssm_scan_fwd(h, y, delta, u, B, C, a_neg, D, *, gate=None, flags: int = 0, workspace=None):
+SCAN_STATIC_SCRATCH_BYTES = 32 << 20
+
+
+def ssm_scan_fwd(h, y, delta, u, B, C, a_neg, D, *, gate=None, flags: int = 0, workspace=None, static_scratch: bool = False):
     """Selective scan over a whole sequence; h [B,di,ds] is updated in place, y is written.
 
     delta,u,y (and gate) are [batch,T,d_inner]; B and C are [batch,T,d_state] or
-    strided views into xdbl [batch,T,xd] (same row stride for both)."""
+    strided views into xdbl [batch,T,xd] (same row stride for both).  With static_scratch the call goes to
+    mrs_ssm_scan_fwd_static: no workspace argument, the chunk summaries live in the library's own per-GPU buffer."""
     batch, T, di = delta.shape
     ds = a_neg.shape[1]
     _dev(h, y, delta, u, a_neg, D, workspace); _f32(h, a_neg, D)
@@ -96,6 +100,12 @@ def ssm_scan_fwd(h, y, delta, u, B, C, a_neg, D, *, gate=None, flags: int = 0, w
         if gate.shape != delta.shape or gate.stride(2) != 1 or gate.stride(0) != T * gate.stride(1):
             raise ValueError("gate must be [batch,T,d_inner], row-dense over [batch*T], unit inner stride")
         gate_stride = gate.stride(1)
+    if static_scratch:
+        if workspace is not None:
+            raise ValueError("static_scratch takes no workspace")
+        _lib.call("mrs_ssm_scan_fwd_static", _stream(), int(dt), _p(h), _p(y), _p(delta), _p(u), _p(B), _p(C), bc_stride,
+                  _p(a_neg), _p(D), _p(gate), gate_stride, flags, batch, T, di, ds)
+        return y
     ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
     _lib.call("mrs_ssm_scan_fwd_ex", _stream(), int(dt), _p(h), _p(y), _p(delta), _p(u), _p(B), _p(C), bc_stride,
               _p(a_neg), _p(D), _p(gate), gate_stride, flags, _p(workspace), ws_bytes, batch, T, di, ds)

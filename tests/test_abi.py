@@ -58,6 +58,16 @@ def test_argument_errors_need_no_gpu():
     assert e.value.code == -1 and "null" in e.value.message
 
 
+def test_static_scratch_scan_refuses_oversized_shapes_before_touching_a_gpu():
+    """mrs_ssm_scan_fwd_static: a shape whose chunk summaries exceed the built-in buffer is refused by size alone."""
+    from mamba_rs_amd import MambaHipError, _lib, ops
+    assert _lib.load().mrs_ssm_scan_workspace_bytes(8, 2048, 1536, 16) <= ops.SCAN_STATIC_SCRATCH_BYTES
+    assert _lib.load().mrs_ssm_scan_workspace_bytes(4, 4096, 5120, 16) <= ops.SCAN_STATIC_SCRATCH_BYTES
+    with pytest.raises(MambaHipError) as e:
+        _lib.call("mrs_ssm_scan_fwd_static", None, 2, 1, 1, 1, 1, 1, 1, 16, 1, 1, None, 0, 0, 128, 4000, 256, 16)
+    assert e.value.code == -4 and "built-in buffer" in e.value.message
+
+
 def test_config_validate_bounds():
     # src/config.rs:108-170
     from mamba_rs_amd import MambaConfig
