@@ -114,12 +114,13 @@ MRS_API int mrs_ssm_scan_fwd_ex(void *stream, int dtype, float *h, void *y, cons
  * MRS_SCAN_STATIC_SCRATCH_BYTES block per GPU, resident until the process ends -- so the call allocates nothing
  * and frees nothing.  Same arguments, routes and results as mrs_ssm_scan_fwd_ex given a workspace of that size.
  *   - A shape with mrs_ssm_scan_workspace_bytes() > MRS_SCAN_STATIC_SCRATCH_BYTES is refused (MRS_E_WORKSPACE);
- *     the benchmark shapes (8 x 2048 x 1536 and 4 x 4096 x 5120, d_state 16) need 15.4 MB and 15.6 MB.
+ *     the benchmark shapes (8 x 2048 x 1536 and 4 x 4096 x 5120, d_state 16) need 13.3 MB and 13.8 MB; only very wide
+ *     batches (batch x d_inner above about 120 000 channels) need more.
  *   - The first call on a GPU looks the buffer's address up (hipGetSymbolAddress, no allocation); make that call
  *     outside a graph capture.
  *   - All calls on one GPU share the one buffer: two calls that overlap in time on the same GPU (different
  *     streams, or graphs replayed side by side) race.  Serialise them or use mrs_ssm_scan_fwd_ex. */
-#define MRS_SCAN_STATIC_SCRATCH_BYTES (32u << 20)
+#define MRS_SCAN_STATIC_SCRATCH_BYTES (16u << 20)
 MRS_API int mrs_ssm_scan_fwd_static(void *stream, int dtype, float *h, void *y, const void *delta, const void *u,
                         const void *B, const void *C, int64_t bc_stride, const float *a_neg,
                         const float *D, const void *gate, int64_t gate_stride, unsigned flags,

@@ -190,24 +190,33 @@ static int launch_seq(hipStream_t st, bool s4d, int gate_mode, float *h, void *y
 // ---------------------------------------------------------------------------
 // T-split route (d_state == 16).  The sequence is cut into C chunks of L steps;
 // one wave owns (batch row, 64-channel tile, chunk), lane = channel, the 16
-// states of a channel in that lane's registers, B_t/C_t rows in scalar registers.
+// states of a channel in that lane's registers.
 //   pass A  chunk_state_kernel: chunk-end state S_c reached from a zero entering
 //           state (chunk 0: from the caller's h) and sum_t delta over the chunk,
-//           for chunks 0..C-2; saves a copy of the caller's h; extra blocks widen
-//           16-bit B/C rows to f32 once so pass B reads them with plain scalar loads.
+//           for chunks 0..C-2; saves a copy of the caller's h.
 //   pass B  chunk_out_kernel: folds the summaries of the chunks before it into its
 //           entering state  h_in(c) = exp(a * sum delta_{c-1}) h_in(c-1) + S_{c-1},
 //           then runs the recurrence over its chunk writing y; the last chunk
 //           writes the final state back to h.
 // The composition law (a,b)o(a',b') = (aa', a'b + b') makes this equal to the
 // serial scan up to rounding.
+//
+// How the B_t / C_t rows (wave-uniform, 16 values each) reach the arithmetic: a wave copies the rows of 16 steps at a
+// time into its own 4 KB of LDS as f32 (lane l brings elements 4(l%4)..+3 of row l/4), two such spans ahead of their
+// use, and every step reads back 16 bytes per lane: lane l gets X[4(l%4) + k] in register k.  Within each group of four
+// lanes the whole row is then present, and the two consumers take it from there at no cost in instructions:
+//   * the matrix core: v_mfma_f32_4x4x1 number k with register k as its A operand gives result register a of lane l
+//     A(lane 4(l/4)+a) * B(lane l) = X[4a+k] * (delta u)[l]  --  the rank-1 state update for state 4a+k;
+//   * the vector ALU through the DPP quad broadcast: an operand "register k of quad lane a" is X[4a+k] on every lane.
+// So state n = 4a+k lives in state register 4k+a (a 4x4 transpose of the natural order, kStateOfReg below).
 // ---------------------------------------------------------------------------
 struct SplitPlan {
     int nchunk;  // C
     int len;     // L
 };
 
-constexpr int kGroup = 4;  // steps per prefetch group; chunk lengths are multiples of 2*kGroup
+constexpr int kGroup = 8;            // steps per activation prefetch group
+constexpr int kSpan = 2 * kGroup;    // steps per loop iteration and per staged block of B / C rows; chunk lengths are multiples
 
 static SplitPlan make_split_plan(int batch, int Tlen, int di) {
     const int tiles = (di + kWave - 1) / kWave;
@@ -218,7 +227,7 @@ static SplitPlan make_split_plan(int batch, int Tlen, int di) {
     if (c > Tlen / 32) c = Tlen / 32;            // chunks of at least 32 steps
     if (c < 1) c = 1;
     int len = (Tlen + c - 1) / c;
-    len = (len + 2 * kGroup - 1) / (2 * kGroup) * (2 * kGroup);
+    len = (len + kSpan - 1) / kSpan * kSpan;
     c = (Tlen + len - 1) / len;
     return {c, len};
 }
@@ -227,20 +236,16 @@ struct SplitWs {
     float *h0copy;  // [B][16][di]
     float *S;       // [B][C-1][16][di]
     float *sumd;    // [B][C-1][di]
-    float *Bt;      // [B*T][4][4] B rows as f32, regrouped: Bt[r][i][q] = B[r][4q+i]
-    float *Cf;      // [B*T][16] widened C rows (16-bit storage only)
     size_t floats;
 };
 
 static SplitWs carve_workspace(float *base, int batch, int Tlen, int di, int nchunk) {
+    (void)Tlen;
     SplitWs w;
     size_t o = 0;
     w.h0copy = base + o; o += (size_t)batch * 16 * di;
     w.S = base + o; o += (size_t)batch * (nchunk - 1) * 16 * di;
     w.sumd = base + o; o += (size_t)batch * (nchunk - 1) * di;
-    o = (o + 63) & ~(size_t)63;  // 256-byte aligned rows for the scalar loads
-    w.Bt = base + o; o += (size_t)batch * Tlen * 16;
-    w.Cf = base + o; o += (size_t)batch * Tlen * 16;
     w.floats = o;
     return w;
 }
@@ -267,38 +272,41 @@ template <typename T> struct LaneBuf {
     }
 };
 
-// One row of B or C (16 values).  The address is wave-uniform, so these are scalar
-// loads; 16-bit rows come as 8 packed dwords and are unpacked on the scalar ALU.
-template <typename T> struct RowRaw { uint32_t w[8]; };
-template <> struct RowRaw<float> { float w[16]; };
+typedef float v4f __attribute__((ext_vector_type(4)));
 
-template <typename T> __device__ __forceinline__ void row_ld(const T *r, RowRaw<T> &o) {
-    const uint32_t *w = reinterpret_cast<const uint32_t *>(r);
+// state held in state register r (see the header comment): a 4x4 transpose, its own inverse
+__host__ __device__ constexpr int kStateOfReg(int r) { return 4 * (r % 4) + r / 4; }
+
+// A lane's piece of a span of rows: elements 4(l%4)..+3 of row l/4, raw (two dwords of 16-bit values or four floats).
+template <typename T> struct RowPiece { uint32_t w[sizeof(T) == 4 ? 4 : 2]; };
+template <typename T>
+__device__ __forceinline__ void piece_ld(RowPiece<T> &o, const T *rows, int64_t stride, int row) {
+    const uint32_t *p = reinterpret_cast<const uint32_t *>(rows + (int64_t)row * stride + 4 * (threadIdx.x & 3));
 #pragma unroll
-    for (int j = 0; j < 8; j++) o.w[j] = w[j];
+    for (int j = 0; j < (int)(sizeof(T) == 4 ? 4 : 2); j++) o.w[j] = p[j];
 }
-template <> __device__ __forceinline__ void row_ld<float>(const float *r, RowRaw<float> &o) {
-#pragma unroll
-    for (int j = 0; j < 16; j++) o.w[j] = r[j];
+__device__ __forceinline__ v4f piece_widen(const RowPiece<float> &r, const float *) {
+    return v4f{__uint_as_float(r.w[0]), __uint_as_float(r.w[1]), __uint_as_float(r.w[2]), __uint_as_float(r.w[3])};
 }
-__device__ __forceinline__ void row_unpack(const RowRaw<float> &r, float (&o)[16], const float *) {
-#pragma unroll
-    for (int j = 0; j < 16; j++) o[j] = r.w[j];
+__device__ __forceinline__ v4f piece_widen(const RowPiece<bf16_t> &r, const bf16_t *) {
+    return v4f{__uint_as_float(r.w[0] << 16), __uint_as_float(r.w[0] & 0xffff0000u), __uint_as_float(r.w[1] << 16),
+               __uint_as_float(r.w[1] & 0xffff0000u)};
 }
-__device__ __forceinline__ void row_unpack(const RowRaw<bf16_t> &r, float (&o)[16], const bf16_t *) {
-#pragma unroll
-    for (int j = 0; j < 8; j++) {
-        o[2 * j] = __uint_as_float(r.w[j] << 16);
-        o[2 * j + 1] = __uint_as_float(r.w[j] & 0xffff0000u);
+__device__ __forceinline__ v4f piece_widen(const RowPiece<f16_t> &r, const f16_t *) {
+    return v4f{(float)__builtin_bit_cast(_Float16, (uint16_t)(r.w[0] & 0xffffu)), (float)__builtin_bit_cast(_Float16, (uint16_t)(r.w[0] >> 16)),
+               (float)__builtin_bit_cast(_Float16, (uint16_t)(r.w[1] & 0xffffu)), (float)__builtin_bit_cast(_Float16, (uint16_t)(r.w[1] >> 16))};
+}
+
+// The wave's staged rows: [slot = span parity][row][16] f32, one such array per tensor.
+struct StagedRows {
+    float v[2][kSpan][16];
+    __device__ __forceinline__ void publish(int slot, const v4f &x) {
+        *reinterpret_cast<v4f *>(&v[slot][threadIdx.x >> 2][4 * (threadIdx.x & 3)]) = x;
     }
-}
-__device__ __forceinline__ void row_unpack(const RowRaw<f16_t> &r, float (&o)[16], const f16_t *) {
-#pragma unroll
-    for (int j = 0; j < 8; j++) {
-        o[2 * j] = (float)__builtin_bit_cast(_Float16, (uint16_t)(r.w[j] & 0xffffu));
-        o[2 * j + 1] = (float)__builtin_bit_cast(_Float16, (uint16_t)(r.w[j] >> 16));
+    __device__ __forceinline__ v4f read(int slot, int row) const {
+        return *reinterpret_cast<const v4f *>(&v[slot][row][4 * (threadIdx.x & 3)]);
     }
-}
+};
 
 // Decay factors of one step: da[n] = 2^(dl * a2[n]); S4D: a2[n] = (n+1) a2[0] -> powers of one exp.
 template <bool S4D>
@@ -308,6 +316,22 @@ __device__ __forceinline__ void decay16(float dl, const float (&a2)[16], float (
         da[0] = p1;
 #pragma unroll
         for (int j = 1; j < 16; j++) da[j] = da[j - 1] * p1;
+    } else {
+#pragma unroll
+        for (int j = 0; j < 16; j++) da[j] = fast_exp2(dl * a2[j]);
+    }
+}
+
+// The same with the power chain as a tree (depth 4 instead of 15), 15 multiplies all the same.
+template <bool S4D>
+__device__ __forceinline__ void decay16_tree(float dl, const float (&a2)[16], float (&da)[16]) {
+    if (S4D) {
+        const float p = fast_exp2(dl * a2[0]);
+        da[0] = p; da[1] = p * p; da[2] = da[1] * p; da[3] = da[1] * da[1];
+#pragma unroll
+        for (int j = 4; j < 8; j++) da[j] = da[3] * da[j - 4];
+#pragma unroll
+        for (int j = 8; j < 16; j++) da[j] = da[7] * da[j - 8];
     } else {
 #pragma unroll
         for (int j = 0; j < 16; j++) da[j] = fast_exp2(dl * a2[j]);
@@ -326,7 +350,7 @@ __device__ __forceinline__ void load_a2(float (&a2)[16], const float *__restrict
 
 // Entering state of chunk c (c >= 1) from the summaries of chunks 0..c-1, in direct form:
 //   h_in(c) = sum_{k<c} exp(a * sum_{k<m<c} sumdelta_m) (.) S_k        (S_0 already holds h0's share)
-// The terms are independent, so the loads of S_k stream instead of forming a load->fma chain.
+// The terms are independent, so the loads of S_k stream instead of forming a load->fma chain.  hs[n] is state n.
 constexpr int kMaxChunks = 32;
 template <bool S4D>
 __device__ __forceinline__ void fold_entering_state(float (&hs)[16], const float (&a2)[16],
@@ -346,30 +370,89 @@ __device__ __forceinline__ void fold_entering_state(float (&hs)[16], const float
     }
 }
 
+// Issue priority by progress.  The instruction arbiter of a SIMD serves its oldest ready wave first, so waves that start
+// together finish one after the other and the last one ends up alone on the SIMD, where it cannot fill the vector ALU
+// (measured: three waves per SIMD finished at 73, 103 and 132 thousand ticks).  A wave therefore lowers its own priority
+// as it gets through its chunk -- after 1/2, 3/4 and 7/8 of its spans -- so whoever is behind is served first and the
+// waves of a SIMD stay together until the last eighth.
+__device__ __forceinline__ void set_progress_priority(int done, int total) {
+    if (done * 8 >= total * 7) __builtin_amdgcn_s_setprio(0);
+    else if (done * 4 >= total * 3) __builtin_amdgcn_s_setprio(1);
+    else if (done * 2 >= total) __builtin_amdgcn_s_setprio(2);
+    else __builtin_amdgcn_s_setprio(3);
+}
+
+// Lanes of a partial channel tile beyond d_inner address their activations at an offset outside every buffer
+// resource: their loads return zero and their stores are dropped, so the time loops carry no lane predicate.
+constexpr unsigned kDeadLaneOffset = 0x7f000000u;
+
+// Sixteen multiply-adds whose first operand is read through the DPP quad broadcast (all four lanes of a group read
+// lane a's register).  The compiler does not fold a DPP move into v_fmac, hence the assembly; it also does not count
+// these as vector instructions when it places the wait states that a matrix-core result or a freshly written DPP
+// source needs before a vector instruction may read it (4-5 and 2), so each block opens with instructions of its own
+// that read none of those registers.
+//
+// Pass B:  acc = D*u + sum_{k,a} c[k](quad lane a) * h[4k+a], and the first half of the SiLU gate rides in front:
+// e = 2^(z * -log2 e).  Three leading instructions (one of them double length) plus the s_nop cover a matrix result
+// written by the instruction just before the block.
+__device__ __forceinline__ void dot16_quad(float &acc, float &e, float Dd, float uu, float z, const v4f &c, const float (&h)[16]) {
+    asm("v_mul_f32 %0, %2, %3\n\t"
+        "v_mul_f32 %1, 0xbfb8aa3b, %4\n\t"
+        "v_exp_f32 %1, %1\n\t"
+        "s_nop 1\n\t"
+        "v_fmac_f32_dpp %0, %5, %9 quad_perm:[0,0,0,0] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+        "v_fmac_f32_dpp %0, %5, %10 quad_perm:[1,1,1,1] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+        "v_fmac_f32_dpp %0, %5, %11 quad_perm:[2,2,2,2] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+        "v_fmac_f32_dpp %0, %5, %12 quad_perm:[3,3,3,3] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+        "v_fmac_f32_dpp %0, %6, %13 quad_perm:[0,0,0,0] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+        "v_fmac_f32_dpp %0, %6, %14 quad_perm:[1,1,1,1] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+        "v_fmac_f32_dpp %0, %6, %15 quad_perm:[2,2,2,2] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+        "v_fmac_f32_dpp %0, %6, %16 quad_perm:[3,3,3,3] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+        "v_fmac_f32_dpp %0, %7, %17 quad_perm:[0,0,0,0] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+        "v_fmac_f32_dpp %0, %7, %18 quad_perm:[1,1,1,1] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+        "v_fmac_f32_dpp %0, %7, %19 quad_perm:[2,2,2,2] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+        "v_fmac_f32_dpp %0, %7, %20 quad_perm:[3,3,3,3] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+        "v_fmac_f32_dpp %0, %8, %21 quad_perm:[0,0,0,0] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+        "v_fmac_f32_dpp %0, %8, %22 quad_perm:[1,1,1,1] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+        "v_fmac_f32_dpp %0, %8, %23 quad_perm:[2,2,2,2] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+        "v_fmac_f32_dpp %0, %8, %24 quad_perm:[3,3,3,3] row_mask:0xf bank_mask:0xf bound_ctrl:1"
+        : "=&v"(acc), "=&v"(e)
+        : "v"(Dd), "v"(uu), "v"(z), "v"(c[0]), "v"(c[1]), "v"(c[2]), "v"(c[3]), "v"(h[0]), "v"(h[1]), "v"(h[2]), "v"(h[3]), "v"(h[4]),
+          "v"(h[5]), "v"(h[6]), "v"(h[7]), "v"(h[8]), "v"(h[9]), "v"(h[10]), "v"(h[11]), "v"(h[12]), "v"(h[13]), "v"(h[14]), "v"(h[15]));
+}
+
+// Pass A (direct form, S4D):  s[4k+a] += v^(n+1-ish) * b[k](quad lane a) for the states n = 4a+k in the order n = 0..15,
+// with the power chain v <- v * x between them (a dependent chain costs no issue slot here) and the step's running sum
+// of delta: v enters as x * (delta u), leaves as x^16 * (delta u).  Two plain instructions lead, so a freshly written b
+// register is two instructions old before the first DPP read.
+__device__ __forceinline__ void chain16_quad(float (&s)[16], float &sd, float x, float du, float dl, const v4f &b) {
+    float v;
+#define MRS_QF(R, K, A) "v_fmac_f32_dpp %" #R ", %" #K ", %16 quad_perm:[" #A "," #A "," #A "," #A "] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+#define MRS_MX "v_mul_f32 %16, %16, %18\n\t"
+    asm("v_mul_f32 %16, %18, %19\n\t"
+        "v_add_f32 %17, %17, %20\n\t"
+        // n = 0..15: state register 4k+a with k = n % 4, a = n / 4; b[k] are operands 21..24
+        MRS_QF(0, 21, 0) MRS_MX MRS_QF(4, 22, 0) MRS_MX MRS_QF(8, 23, 0) MRS_MX MRS_QF(12, 24, 0) MRS_MX
+        MRS_QF(1, 21, 1) MRS_MX MRS_QF(5, 22, 1) MRS_MX MRS_QF(9, 23, 1) MRS_MX MRS_QF(13, 24, 1) MRS_MX
+        MRS_QF(2, 21, 2) MRS_MX MRS_QF(6, 22, 2) MRS_MX MRS_QF(10, 23, 2) MRS_MX MRS_QF(14, 24, 2) MRS_MX
+        MRS_QF(3, 21, 3) MRS_MX MRS_QF(7, 22, 3) MRS_MX MRS_QF(11, 23, 3) MRS_MX MRS_QF(15, 24, 3)
+        : "+v"(s[0]), "+v"(s[1]), "+v"(s[2]), "+v"(s[3]), "+v"(s[4]), "+v"(s[5]), "+v"(s[6]), "+v"(s[7]), "+v"(s[8]), "+v"(s[9]),
+          "+v"(s[10]), "+v"(s[11]), "+v"(s[12]), "+v"(s[13]), "+v"(s[14]), "+v"(s[15]), "=&v"(v), "+v"(sd)
+        : "v"(x), "v"(du), "v"(dl), "v"(b[0]), "v"(b[1]), "v"(b[2]), "v"(b[3]));
+#undef MRS_QF
+#undef MRS_MX
+}
+
 template <typename T, bool S4D>
 __global__ __launch_bounds__(kWave) void chunk_state_kernel(
     const float *__restrict__ h, const T *__restrict__ delta, const T *__restrict__ u,
-    const T *__restrict__ Bm, const T *__restrict__ Cm, int64_t bc_stride,
+    const T *__restrict__ Bm, int64_t bc_stride,
     const float *__restrict__ a_neg, float *__restrict__ h0copy, float *__restrict__ S,
-    float *__restrict__ sumd, float *__restrict__ Bt, float *__restrict__ Cf, int batch, int Tlen,
-    int di, int tiles, int nchunk, int len, int n_state_blocks) {
+    float *__restrict__ sumd, int Tlen, int di, int tiles, int nchunk, int len) {
     using raw_t = typename RawElem<T>::type;
-    if ((int)blockIdx.x >= n_state_blocks) {
-        // 64 rows of B and C as f32: lane = (row % 4, column).  B is regrouped so that the four
-        // values a lane feeds to the outer-product MFMAs of pass B are one 16-byte load.
-        const int64_t rows = (int64_t)batch * Tlen;
-        const int64_t r0 = (int64_t)(blockIdx.x - n_state_blocks) * 64;
-        const int col = threadIdx.x & 15, sub = threadIdx.x >> 4;
-#pragma unroll 4
-        for (int k = 0; k < 16; k++) {
-            const int64_t r = r0 + 4 * k + sub;
-            if (r < rows) {
-                Bt[r * 16 + (col & 3) * 4 + (col >> 2)] = Store<T>::ld(Bm + r * bc_stride + col);
-                if (sizeof(T) != 4) Cf[r * 16 + col] = Store<T>::ld(Cm + r * bc_stride + col);
-            }
-        }
-        return;
-    }
+    __shared__ alignas(16) StagedRows Bs;
+    // Chunks 0 .. nchunk-2 only, and chunk lengths are multiples of kSpan: every step of this wave's chunk
+    // exists, so the walk has no tail.
     const int nc1 = nchunk - 1;
     const int tile = blockIdx.x % tiles;
     const int rest = blockIdx.x / tiles;
@@ -377,11 +460,10 @@ __global__ __launch_bounds__(kWave) void chunk_state_kernel(
     const int b = rest / nc1;
     const int d0 = tile * kWave;
     const bool live = d0 + (int)threadIdx.x < di;
-    const unsigned lx = live ? threadIdx.x : (unsigned)(di - 1 - d0);  // dead lanes shadow the last live channel
-    const int dd = d0 + (int)lx;
-    const unsigned lxb = lx * (unsigned)sizeof(T);
+    const int dd = live ? d0 + (int)threadIdx.x : di - 1;   // plain loads of dead lanes shadow the last live channel
+    const unsigned lxb = live ? threadIdx.x * (unsigned)sizeof(T) : kDeadLaneOffset;
 
-    float hs[16], a2[16];
+    float hs[16], a2[16];   // hs[n]: state n
     load_a2<S4D>(a2, a_neg, dd);
 #pragma unroll
     for (int j = 0; j < 16; j++) hs[j] = 0.0f;
@@ -392,116 +474,117 @@ __global__ __launch_bounds__(kWave) void chunk_state_kernel(
             if (live) h0copy[((int64_t)b * 16 + j) * di + dd] = hs[j];
         }
     }
-    const int t0 = c * len, t1 = min(Tlen, t0 + len);
+    const int t0 = c * len;
     const int64_t row0 = (int64_t)b * Tlen;
     const int64_t slab = (int64_t)Tlen * di - d0;  // elements from this wave's base to the end of batch row b
     const LaneBuf<T> dbuf(delta + row0 * di + d0, slab), ubuf(u + row0 * di + d0, slab);
     const unsigned row_bytes = (unsigned)di * (unsigned)sizeof(T);
     const T *Bp = Bm + row0 * bc_stride;
     float sd = 0.0f;
+    const int nspans = len / kSpan;
+    const int prow = threadIdx.x >> 2;   // the row of a span this lane stages
 
     raw_t rdA[kGroup], ruA[kGroup], rdB[kGroup], ruB[kGroup];
-    auto load_group = [&](raw_t (&rd)[kGroup], raw_t (&ru)[kGroup], int tg) {
+    auto load_group = [&](raw_t (&rd)[kGroup], raw_t (&ru)[kGroup], int tg) {   // steps tg .. tg+7 (tg clamped into the chunk)
+        unsigned o = (unsigned)max(tg, t0) * row_bytes;
 #pragma unroll
-        for (int k = 0; k < kGroup; k++) {
-            const unsigned off = (unsigned)min(tg + k, t1 - 1) * row_bytes;
-            rd[k] = dbuf.ld(lxb, off);
-            ru[k] = ubuf.ld(lxb, off);
+        for (int k = 0; k < kGroup; k++, o += row_bytes) {
+            rd[k] = dbuf.ld(lxb, o);
+            ru[k] = ubuf.ld(lxb, o);
         }
     };
-    RowRaw<T> curB;
-    row_ld(Bp + (int64_t)t0 * bc_stride, curB);
-    auto compute_group = [&](const raw_t (&rd)[kGroup], const raw_t (&ru)[kGroup], int tg) {
-#pragma unroll
-        for (int k = 0; k < kGroup; k++) {
-            const int t = tg + k;
-            if (t < t1) {
-                RowRaw<T> nxtB;
-                row_ld(Bp + (int64_t)min(t + 1, t1 - 1) * bc_stride, nxtB);
-                const float dl = widen(rd[k], (const T *)nullptr);
-                const float uu = widen(ru[k], (const T *)nullptr);
-                const float du = dl * uu;
-                float Bv[16], da[16];
-                row_unpack(curB, Bv, (const T *)nullptr);
-                decay16<S4D>(dl, a2, da);
-                sd += dl;
-#pragma unroll
-                for (int j = 0; j < 16; j++) {
-                    hs[j] *= da[j];
-                    hs[j] = fmaf(du, Bv[j], hs[j]);
-                }
-                curB = nxtB;
-            }
-        }
-    };
+    RowPiece<T> nb;
     if (S4D) {
         // Direct form, walking the chunk backwards: the weight of step s in the chunk-end
         // state is prod_{r>s} exp(delta_r a_n) = x_s^(n+1) with x_s = 2^(a2[0] * sum_{r>s} delta_r),
         // so one exp, a power chain and one multiply-add per state -- no decay of a running state.
-        float S16[16];
+        float S16[16];   // S16[r]: state kStateOfReg(r)
 #pragma unroll
         for (int j = 0; j < 16; j++) S16[j] = 0.0f;
-        const int nsteps = t1 - t0;
-        const int ngroups = (nsteps + kGroup - 1) / kGroup;  // chunk lengths are multiples of 2*kGroup except the tail
-        // The B rows of a group are fetched (scalar loads) together with its activations, a whole
-        // group ahead of their use: one-step lookahead does not cover a scalar-cache miss.
-        constexpr int kRows = (sizeof(T) == 2) ? kGroup : 1;  // f32 rows are too wide to hold 2x4 of them in SGPRs
-        RowRaw<T> rowsA[kRows], rowsB[kRows];
-        auto load_group_at = [&](raw_t (&rd)[kGroup], raw_t (&ru)[kGroup], RowRaw<T> (&rows)[kRows], int g) {
+        // spans are walked last to first; span s sits in slot s & 1, span s-1 is published while s is computed and
+        // the rows of span s-2 requested
+        {
+            RowPiece<T> first;
+            piece_ld(first, Bp, bc_stride, t0 + (nspans - 1) * kSpan + prow);
+            Bs.publish((nspans - 1) & 1, piece_widen(first, (const T *)nullptr));
+        }
+        piece_ld(nb, Bp, bc_stride, t0 + max(nspans - 2, 0) * kSpan + prow);
+        load_group(rdB, ruB, t0 + (nspans - 1) * kSpan + kGroup);
+        v4f bv = Bs.read((nspans - 1) & 1, kSpan - 1);
+        for (int sp = nspans - 1; sp >= 0; sp--) {
+            const int ts = t0 + sp * kSpan, slot = sp & 1;
+            set_progress_priority(nspans - 1 - sp, nspans);
+            Bs.publish(slot ^ 1, piece_widen(nb, (const T *)nullptr));
+            piece_ld(nb, Bp, bc_stride, t0 + max(sp - 2, 0) * kSpan + prow);
+            load_group(rdA, ruA, ts);
+            auto back = [&](const raw_t (&rd)[kGroup], const raw_t (&ru)[kGroup], int base) {
 #pragma unroll
-            for (int k = 0; k < kGroup; k++) {
-                const int tt = max(t0, min(t0 + g * kGroup + k, t1 - 1));
-                rd[k] = dbuf.ld(lxb, (unsigned)tt * row_bytes);
-                ru[k] = ubuf.ld(lxb, (unsigned)tt * row_bytes);
-                if (kRows == kGroup) row_ld(Bp + (int64_t)tt * bc_stride, rows[k]);
-            }
-        };
-        row_ld(Bp + (int64_t)(t1 - 1) * bc_stride, curB);
-        auto back_group = [&](const raw_t (&rd)[kGroup], const raw_t (&ru)[kGroup], const RowRaw<T> (&rows)[kRows], int g) {
-#pragma unroll
-            for (int k = kGroup - 1; k >= 0; k--) {
-                const int t = t0 + g * kGroup + k;
-                if (g >= 0 && t < t1) {
-                    RowRaw<T> nxtB;
-                    if (kRows == 1) row_ld(Bp + (int64_t)max(t - 1, t0) * bc_stride, nxtB);
+                for (int k = kGroup - 1; k >= 0; k--) {
+                    const int j = base + k;                               // row of the span
+                    const v4f bcur = bv;
+                    bv = j > 0 ? Bs.read(slot, j - 1) : Bs.read(slot ^ 1, kSpan - 1);   // the step after this one
                     const float dl = widen(rd[k], (const T *)nullptr);
                     const float uu = widen(ru[k], (const T *)nullptr);
-                    float Bv[16];
-                    if (kRows == kGroup) row_unpack(rows[k], Bv, (const T *)nullptr);
-                    else row_unpack(curB, Bv, (const T *)nullptr);
                     const float x = fast_exp2(a2[0] * sd);
-                    float v = x * (dl * uu);
-                    S16[0] = fmaf(v, Bv[0], S16[0]);
-#pragma unroll
-                    for (int j = 1; j < 16; j++) {
-                        v *= x;
-                        S16[j] = fmaf(v, Bv[j], S16[j]);
-                    }
-                    sd += dl;
-                    if (kRows == 1) curB = nxtB;
+                    chain16_quad(S16, sd, x, dl * uu, dl, bcur);
                 }
-            }
-        };
-        load_group_at(rdA, ruA, rowsA, ngroups - 1);
-        for (int g = ngroups - 1; g >= 0; g -= 2) {
-            load_group_at(rdB, ruB, rowsB, g - 1);
-            back_group(rdA, ruA, rowsA, g);
-            load_group_at(rdA, ruA, rowsA, g - 2);
-            back_group(rdB, ruB, rowsB, g - 1);
+            };
+            back(rdB, ruB, kGroup);
+            load_group(rdB, ruB, ts - kGroup);
+            back(rdA, ruA, 0);
         }
         // entering state (chunk 0 only; zero otherwise) decayed over the whole chunk
         float da[16];
         decay16<true>(sd, a2, da);
 #pragma unroll
-        for (int j = 0; j < 16; j++) hs[j] = fmaf(da[j], hs[j], S16[j]);
+        for (int j = 0; j < 16; j++) hs[j] = fmaf(da[j], hs[j], S16[4 * (j % 4) + j / 4]);
     } else {
-        load_group(rdA, ruA, t0);
-        for (int tg = t0; tg < t1; tg += 2 * kGroup) {
-            load_group(rdB, ruB, tg + kGroup);
-            compute_group(rdA, ruA, tg);
-            load_group(rdA, ruA, tg + 2 * kGroup);
-            compute_group(rdB, ruB, tg + kGroup);
+        // General A: the recurrence itself, forwards, with the rank-1 update on the matrix core as in pass B.
+        float hr[16];   // hr[r]: state kStateOfReg(r)
+#pragma unroll
+        for (int r = 0; r < 16; r++) hr[r] = hs[kStateOfReg(r)];
+        {
+            RowPiece<T> first;
+            piece_ld(first, Bp, bc_stride, t0 + prow);
+            Bs.publish(0, piece_widen(first, (const T *)nullptr));
         }
+        piece_ld(nb, Bp, bc_stride, t0 + min(1, nspans - 1) * kSpan + prow);
+        load_group(rdA, ruA, t0);
+        v4f bv = Bs.read(0, 0);
+        for (int sp = 0; sp < nspans; sp++) {
+            const int ts = t0 + sp * kSpan, slot = sp & 1;
+            set_progress_priority(sp, nspans);
+            Bs.publish(slot ^ 1, piece_widen(nb, (const T *)nullptr));
+            piece_ld(nb, Bp, bc_stride, t0 + min(sp + 2, nspans - 1) * kSpan + prow);
+            load_group(rdB, ruB, ts + kGroup);
+            auto fwd = [&](const raw_t (&rd)[kGroup], const raw_t (&ru)[kGroup], int base) {
+#pragma unroll
+                for (int k = 0; k < kGroup; k++) {
+                    const int j = base + k;
+                    const v4f bcur = bv;
+                    bv = j < kSpan - 1 ? Bs.read(slot, j + 1) : Bs.read(slot ^ 1, 0);
+                    const float dl = widen(rd[k], (const T *)nullptr);
+                    const float uu = widen(ru[k], (const T *)nullptr);
+                    const float du = dl * uu;
+                    float da[16];
+                    decay16_tree<false>(dl, a2, da);
+                    sd += dl;
+#pragma unroll
+                    for (int q = 0; q < 4; q++) {
+                        v4f hq = {hr[4 * q] * da[kStateOfReg(4 * q)], hr[4 * q + 1] * da[kStateOfReg(4 * q + 1)],
+                                  hr[4 * q + 2] * da[kStateOfReg(4 * q + 2)], hr[4 * q + 3] * da[kStateOfReg(4 * q + 3)]};
+                        hq = __builtin_amdgcn_mfma_f32_4x4x1f32(bcur[q], du, hq, 0, 0, 0);
+#pragma unroll
+                        for (int i = 0; i < 4; i++) hr[4 * q + i] = hq[i];
+                    }
+                }
+            };
+            fwd(rdA, ruA, 0);
+            load_group(rdA, ruA, min(ts + kSpan, t0 + len - kGroup));
+            fwd(rdB, ruB, kGroup);
+        }
+#pragma unroll
+        for (int r = 0; r < 16; r++) hs[kStateOfReg(r)] = hr[r];
     }
     if (live) {
         const int64_t sbase = (int64_t)b * nc1 + c;
@@ -511,110 +594,129 @@ __global__ __launch_bounds__(kWave) void chunk_state_kernel(
     }
 }
 
-typedef float v4f __attribute__((ext_vector_type(4)));
-
-// Bt: regrouped f32 B rows from pass A; Cf: f32 C rows of stride cf_stride (the widened
-// copy, or the caller's rows at f32 storage).
-//
-// The rank-1 update h[n] += (delta*u)[channel] * B[n] of a wave is an outer product
-// (64 channels) x (16 states): four v_mfma_f32_4x4x1 (16 blocks of 4x4, K = 1) do it on
-// the matrix core with the decayed state as the accumulator -- lane l receives, in
-// result register i, A(lane 4*(l/4)+i) * B(lane l) + C: A carries B[4q+i], B carries the
-// lane's own delta*u -- which takes 16 multiply-adds per step off the vector ALU.
+// Pass B.  The time loop has no tail and no lane predicate: rows at and beyond T lie outside the buffer resources
+// (loads return zero: delta = 0 leaves the state as it is, stores are dropped), and so do the lanes of a partial tile.
 template <typename T, bool S4D, int GATE>
 __global__ __launch_bounds__(kWave) void chunk_out_kernel(
     float *__restrict__ h, T *__restrict__ y, const T *__restrict__ delta, const T *__restrict__ u,
-    const float *__restrict__ Bt, const float *__restrict__ Cf, int64_t cf_stride,
+    const T *__restrict__ Bm, const T *__restrict__ Cm, int64_t bc_stride,
     const float *__restrict__ a_neg, const float *__restrict__ Dp, const T *__restrict__ gate, int64_t gate_stride,
     const float *__restrict__ h0copy, const float *__restrict__ S, const float *__restrict__ sumd,
     int Tlen, int di, int tiles, int nchunk, int len) {
     using raw_t = typename RawElem<T>::type;
+    __shared__ alignas(16) StagedRows Bs, Cs;
     const int tile = blockIdx.x % tiles;
     const int rest = blockIdx.x / tiles;
     const int c = rest % nchunk;
     const int b = rest / nchunk;
     const int d0 = tile * kWave;
     const bool live = d0 + (int)threadIdx.x < di;
-    const unsigned lx = live ? threadIdx.x : (unsigned)(di - 1 - d0);
-    const int dd = d0 + (int)lx;
-    const unsigned lxb = lx * (unsigned)sizeof(T);
+    const int dd = live ? d0 + (int)threadIdx.x : di - 1;
+    const unsigned lxb = live ? threadIdx.x * (unsigned)sizeof(T) : kDeadLaneOffset;
 
-    float hs[16], a2[16];
+    float hn[16], a2[16], hs[16], ar[16];   // hn[n]: state n; hs[r], ar[r]: state kStateOfReg(r)
     load_a2<S4D>(a2, a_neg, dd);
     if (c == 0) {
 #pragma unroll
-        for (int j = 0; j < 16; j++) hs[j] = h0copy[((int64_t)b * 16 + j) * di + dd];
+        for (int j = 0; j < 16; j++) hn[j] = h0copy[((int64_t)b * 16 + j) * di + dd];
     } else {
-        fold_entering_state<S4D>(hs, a2, S, sumd, b, c, nchunk, di, dd);
+        fold_entering_state<S4D>(hn, a2, S, sumd, b, c, nchunk, di, dd);
     }
+#pragma unroll
+    for (int r = 0; r < 16; r++) { hs[r] = hn[kStateOfReg(r)]; ar[r] = a2[kStateOfReg(r)]; }
     const float Dd = Dp[dd];
     const int t0 = c * len, t1 = min(Tlen, t0 + len);
+    const int tl = Tlen - 1;
     const int64_t row0 = (int64_t)b * Tlen;
     const int64_t slab = (int64_t)Tlen * di - d0;
     const LaneBuf<T> dbuf(delta + row0 * di + d0, slab), ubuf(u + row0 * di + d0, slab);
     const LaneBuf<T> gbuf(GATE ? gate + row0 * gate_stride + d0 : delta, GATE ? (int64_t)Tlen * gate_stride - d0 : 0), ybuf(y + row0 * di + d0, slab);
     const unsigned row_bytes = (unsigned)di * (unsigned)sizeof(T);
     const unsigned gate_row_bytes = (unsigned)gate_stride * (unsigned)sizeof(T);
-    const __amdgpu_buffer_rsrc_t btbuf =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(Bt + row0 * 16), 0, (int)((int64_t)Tlen * 64), 0x00020000);
-    const unsigned bt_lane = (threadIdx.x & 3) * 16;  // this lane's 4 floats inside a regrouped row
-    const float *Cp = Cf + row0 * cf_stride;
+    const T *Bp = Bm + row0 * bc_stride, *Cp = Cm + row0 * bc_stride;
+    const int prow = threadIdx.x >> 2;
 
     raw_t rdA[kGroup], ruA[kGroup], rgA[kGroup], rdB[kGroup], ruB[kGroup], rgB[kGroup];
-    v4f bvA[kGroup], bvB[kGroup];
-    auto load_group = [&](raw_t (&rd)[kGroup], raw_t (&ru)[kGroup], raw_t (&rg)[kGroup], v4f (&bv)[kGroup], int tg) {
+    auto load_group = [&](raw_t (&rd)[kGroup], raw_t (&ru)[kGroup], raw_t (&rg)[kGroup], int tg) {
+        unsigned o = (unsigned)tg * row_bytes, og = (unsigned)tg * gate_row_bytes;
 #pragma unroll
-        for (int k = 0; k < kGroup; k++) {
-            const unsigned tt = (unsigned)min(tg + k, t1 - 1);
-            rd[k] = dbuf.ld(lxb, tt * row_bytes);
-            ru[k] = ubuf.ld(lxb, tt * row_bytes);
-            if (GATE) rg[k] = gbuf.ld(lxb, tt * gate_row_bytes);
-            bv[k] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(btbuf, bt_lane, tt * 64u, 0));
+        for (int k = 0; k < kGroup; k++, o += row_bytes, og += gate_row_bytes) {
+            rd[k] = dbuf.ld(lxb, o);
+            ru[k] = ubuf.ld(lxb, o);
+            if (GATE) rg[k] = gbuf.ld(lxb, og);
         }
     };
-    RowRaw<float> curC;
-    row_ld(Cp + (int64_t)t0 * cf_stride, curC);
-    auto compute_group = [&](const raw_t (&rd)[kGroup], const raw_t (&ru)[kGroup], const raw_t (&rg)[kGroup],
-                             const v4f (&bv)[kGroup], int tg) {
+    const int nspans = (t1 - t0 + kSpan - 1) / kSpan;
+    RowPiece<T> nb, nc;
+    {
+        RowPiece<T> fb, fc;
+        piece_ld(fb, Bp, bc_stride, min(t0 + prow, tl));
+        piece_ld(fc, Cp, bc_stride, min(t0 + prow, tl));
+        Bs.publish(0, piece_widen(fb, (const T *)nullptr));
+        Cs.publish(0, piece_widen(fc, (const T *)nullptr));
+    }
+    piece_ld(nb, Bp, bc_stride, min(t0 + kSpan + prow, tl));
+    piece_ld(nc, Cp, bc_stride, min(t0 + kSpan + prow, tl));
+    load_group(rdA, ruA, rgA, t0);
+    v4f bv = Bs.read(0, 0), cv = Cs.read(0, 0);
+    for (int sp = 0; sp < nspans; sp++) {
+        const int ts = t0 + sp * kSpan, slot = sp & 1;
+        set_progress_priority(sp, nspans);
+        // span sp+1 into the other slot (its rows were requested a span ago), then the request for span sp+2
+        Bs.publish(slot ^ 1, piece_widen(nb, (const T *)nullptr));
+        Cs.publish(slot ^ 1, piece_widen(nc, (const T *)nullptr));
+        piece_ld(nb, Bp, bc_stride, min(ts + 2 * kSpan + prow, tl));
+        piece_ld(nc, Cp, bc_stride, min(ts + 2 * kSpan + prow, tl));
+        load_group(rdB, ruB, rgB, ts + kGroup);
+        auto steps = [&](const raw_t (&rd)[kGroup], const raw_t (&ru)[kGroup], const raw_t (&rg)[kGroup], int base) {
+            unsigned yo = (unsigned)(ts + base) * row_bytes;
 #pragma unroll
-        for (int k = 0; k < kGroup; k++) {
-            const int t = tg + k;
-            if (t < t1) {
-                RowRaw<float> nxtC;
-                row_ld(Cp + (int64_t)min(t + 1, t1 - 1) * cf_stride, nxtC);
+            for (int k = 0; k < kGroup; k++, yo += row_bytes) {
+                const int j = base + k;
+                const v4f bcur = bv, ccur = cv;
+                bv = j < kSpan - 1 ? Bs.read(slot, j + 1) : Bs.read(slot ^ 1, 0);   // the rows of the next step
+                cv = j < kSpan - 1 ? Cs.read(slot, j + 1) : Cs.read(slot ^ 1, 0);
                 const float dl = widen(rd[k], (const T *)nullptr);
                 const float uu = widen(ru[k], (const T *)nullptr);
                 const float du = dl * uu;
                 float da[16];
-                decay16<S4D>(dl, a2, da);
-                float acc = Dd * uu;
+                if (S4D) {
+                    float dn[16];
+                    decay16_tree<true>(dl, a2, dn);
 #pragma unroll
-                for (int q = 0; q < 4; q++) {
-                    v4f hq = {hs[4 * q] * da[4 * q], hs[4 * q + 1] * da[4 * q + 1], hs[4 * q + 2] * da[4 * q + 2],
-                              hs[4 * q + 3] * da[4 * q + 3]};
-                    hq = __builtin_amdgcn_mfma_f32_4x4x1f32(bv[k][q], du, hq, 0, 0, 0);
+                    for (int r = 0; r < 16; r++) da[r] = dn[kStateOfReg(r)];
+                } else {
 #pragma unroll
-                    for (int i = 0; i < 4; i++) hs[4 * q + i] = hq[i];
+                    for (int r = 0; r < 16; r++) da[r] = fast_exp2(dl * ar[r]);
                 }
+                v4f hq[4];
 #pragma unroll
-                for (int j = 0; j < 16; j++) acc = fmaf(hs[j], curC.w[j], acc);
-                if (GATE == 1) acc *= widen(rg[k], (const T *)nullptr);
-                if (GATE == 2) acc *= silu(widen(rg[k], (const T *)nullptr));
-                if (live) ybuf.st(acc, lxb, (unsigned)t * row_bytes);
-                curC = nxtC;
+                for (int q = 0; q < 4; q++)
+                    hq[q] = v4f{hs[4 * q] * da[4 * q], hs[4 * q + 1] * da[4 * q + 1], hs[4 * q + 2] * da[4 * q + 2], hs[4 * q + 3] * da[4 * q + 3]};
+                // the four matrix instructions back to back: one between vector instructions costs a pipeline switch each way
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int q = 0; q < 4; q++) hq[q] = __builtin_amdgcn_mfma_f32_4x4x1f32(bcur[q], du, hq[q], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int q = 0; q < 4; q++)
+#pragma unroll
+                    for (int i = 0; i < 4; i++) hs[4 * q + i] = hq[q][i];
+                float acc, e;
+                const float z = GATE ? widen(rg[k], (const T *)nullptr) : 0.0f;
+                dot16_quad(acc, e, Dd, uu, z, ccur, hs);
+                if (GATE == 1) acc *= z;
+                if (GATE == 2) acc *= z * fast_rcp(1.0f + e);
+                ybuf.st(acc, lxb, yo);
             }
-        }
-    };
-    load_group(rdA, ruA, rgA, bvA, t0);
-    for (int tg = t0; tg < t1; tg += 2 * kGroup) {
-        load_group(rdB, ruB, rgB, bvB, tg + kGroup);
-        compute_group(rdA, ruA, rgA, bvA, tg);
-        load_group(rdA, ruA, rgA, bvA, tg + 2 * kGroup);
-        compute_group(rdB, ruB, rgB, bvB, tg + kGroup);
+        };
+        steps(rdA, ruA, rgA, 0);
+        load_group(rdA, ruA, rgA, ts + kSpan);
+        steps(rdB, ruB, rgB, kGroup);
     }
     if (c == nchunk - 1 && live) {
 #pragma unroll
-        for (int j = 0; j < 16; j++) h[((int64_t)b * di + dd) * 16 + j] = hs[j];
+        for (int r = 0; r < 16; r++) h[((int64_t)b * di + dd) * 16 + kStateOfReg(r)] = hs[r];
     }
 }
 
@@ -629,18 +731,14 @@ static int launch_split_s4d(hipStream_t st, int gate_mode, float *h, T *y, const
     const int tiles = (di + kWave - 1) / kWave;
     const int C = plan.nchunk, L = plan.len;
     const SplitWs w = carve_workspace(ws, batch, Tlen, di, C);
-    const int n_state = batch * (C - 1) * tiles;
-    const int n_widen = (int)(((int64_t)batch * Tlen + 63) / 64);
     const dim3 block(kWave);
-    const dim3 gridA((unsigned)(n_state + n_widen)), gridB((unsigned)(batch * C * tiles));
-    hipLaunchKernelGGL((chunk_state_kernel<T, S4D>), gridA, block, 0, st, h, delta, u, Bm, Cm, bc_stride, a_neg,
-                       w.h0copy, w.S, w.sumd, w.Bt, w.Cf, batch, Tlen, di, tiles, C, L, n_state);
+    const dim3 gridA((unsigned)(batch * (C - 1) * tiles)), gridB((unsigned)(batch * C * tiles));
+    hipLaunchKernelGGL((chunk_state_kernel<T, S4D>), gridA, block, 0, st, h, delta, u, Bm, bc_stride, a_neg,
+                       w.h0copy, w.S, w.sumd, Tlen, di, tiles, C, L);
     int rc = check_launch("chunk_state_kernel");
     if (rc) return rc;
-    const float *Cf = IsF32<T>::value ? reinterpret_cast<const float *>(Cm) : w.Cf;
-    const int64_t bcf = IsF32<T>::value ? bc_stride : 16;
-#define MRS_LAUNCH(G)                                                                                   \
-    hipLaunchKernelGGL((chunk_out_kernel<T, S4D, G>), gridB, block, 0, st, h, y, delta, u, w.Bt, Cf, bcf, \
+#define MRS_LAUNCH(G)                                                                                      \
+    hipLaunchKernelGGL((chunk_out_kernel<T, S4D, G>), gridB, block, 0, st, h, y, delta, u, Bm, Cm, bc_stride, \
                        a_neg, D, gate, gate_stride, w.h0copy, w.S, w.sumd, Tlen, di, tiles, C, L)
     if (gate_mode == 0) MRS_LAUNCH(0);
     else if (gate_mode == 1) MRS_LAUNCH(1);

@@ -74,7 +74,7 @@ def ssm_scan_workspace_bytes(batch: int, T: int, d_inner: int, d_state: int) -> 
     return int(_lib.load().mrs_ssm_scan_workspace_bytes(batch, T, d_inner, d_state))
 
 
-SCAN_STATIC_SCRATCH_BYTES = 32 << 20
+SCAN_STATIC_SCRATCH_BYTES = 16 << 20
 
 
 def ssm_scan_fwd(h, y, delta, u, B, C, a_neg, D, *, gate=None, flags: int = 0, workspace=None, static_scratch: bool = False):

@@ -64,7 +64,7 @@ def test_static_scratch_scan_refuses_oversized_shapes_before_touching_a_gpu():
     assert _lib.load().mrs_ssm_scan_workspace_bytes(8, 2048, 1536, 16) <= ops.SCAN_STATIC_SCRATCH_BYTES
     assert _lib.load().mrs_ssm_scan_workspace_bytes(4, 4096, 5120, 16) <= ops.SCAN_STATIC_SCRATCH_BYTES
     with pytest.raises(MambaHipError) as e:
-        _lib.call("mrs_ssm_scan_fwd_static", None, 2, 1, 1, 1, 1, 1, 1, 16, 1, 1, None, 0, 0, 128, 4000, 256, 16)
+        _lib.call("mrs_ssm_scan_fwd_static", None, 2, 1, 1, 1, 1, 1, 1, 16, 1, 1, None, 0, 0, 40, 512, 4096, 16)
     assert e.value.code == -4 and "built-in buffer" in e.value.message
 
 
