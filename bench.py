@@ -19,9 +19,27 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBPS = 8000.0
-# HBM bytes per scan call (both kernels) from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script, each counter
-# scaled by what it reads for a 256 MiB device copy (--copy-calibration): 282.4 MiB read + 63.5 MiB written.
-MEASURED_SCAN_TRAFFIC_BYTES = int((2.0 * (50767 + 92635) + 1.0 * (15056 + 49920)) * 1024)
+SCAN_PROFILE = os.path.join(ROOT, "profiles", "m1_scan_c2_bf16.md")
+
+
+def profiled_scan_traffic():
+    """HBM bytes per scan call (both kernels) as the committed rocprofv3 FETCH_SIZE / WRITE_SIZE summary states them
+    (a line `traffic_bytes_per_call: N` and one `kernels_sha16: X` naming the kernel source it was taken from).  A counter
+    run cannot share a process with the timed run, so the figure is read, not measured here; it is reported as null when
+    the kernel source has changed since the profile was taken."""
+    import hashlib
+    import re
+    try:
+        text = open(SCAN_PROFILE).read()
+        n = int(re.search(r"^traffic_bytes_per_call:\s*(\d+)", text, re.M).group(1))
+        sha = re.search(r"^kernels_sha16:\s*([0-9a-f]{16})", text, re.M).group(1)
+    except (OSError, AttributeError, ValueError):
+        return None, "no profile"
+    src = os.path.join(ROOT, "mamba_rs_amd", "csrc", "m1_scan.hip")
+    now = hashlib.sha256(open(src, "rb").read()).hexdigest()[:16]
+    if now != sha:
+        return None, f"stale: profile taken from m1_scan.hip {sha}, source is {now}"
+    return n, "profiles/m1_scan_c2_bf16.md"
 
 
 def scan_algorithmic_bytes(batch, T, di, ds, s, gated=True):
@@ -84,7 +102,18 @@ def gpu_leg(args, inp, shape):
     torch.cuda.synchronize()
     med_ms = sorted(x.elapsed_time(y_) for x, y_ in per)[len(per) // 2]
     assert torch.isfinite(y.float()).all().item()
-    return dict(ms_per_step=ev_ms / args.steps, wall_ms_per_step=wall_ms / args.steps, median_launch_ms=med_ms)
+    # the same launch without the S4D-real shortcut: what a trained checkpoint (a general A) gets
+    gen_flags = ops.GATE_SILU
+    for _ in range(3):
+        ops.ssm_scan_fwd(h, y, delta, u, Bm, Cm, a_neg, D, gate=z, flags=gen_flags, workspace=ws)
+    ga, gb = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    ga.record()
+    for _ in range(20):
+        ops.ssm_scan_fwd(h, y, delta, u, Bm, Cm, a_neg, D, gate=z, flags=gen_flags, workspace=ws)
+    gb.record()
+    torch.cuda.synchronize()
+    return dict(ms_per_step=ev_ms / args.steps, wall_ms_per_step=wall_ms / args.steps, median_launch_ms=med_ms,
+                general_a_ms_per_step=ga.elapsed_time(gb) / 20)
 
 
 def cpu_leg(inp, shape, nbytes, budget_s=12.0):
@@ -111,16 +140,50 @@ def cpu_leg(inp, shape, nbytes, budget_s=12.0):
                 ms_per_step=best * 1e3)
 
 
-def lm_leg(name, cfg_kw, vocab, prefill_bt, decode_b, decode_steps, seed=42):
+def cpu_prefill_sample(cfg_kw, sample_layers, sample_tokens, full_tokens, seed=42):
+    """The oracle's restatement of the reference's CPU forward_prefill (PrefillMode::Parallel,
+    src/mamba_ssm/cpu/prefill.rs:420-696) on a bounded sample: `sample_layers` of the model's layers over one sequence of
+    `sample_tokens` tokens, all host cores; scaled linearly in layers and tokens (the pipeline is O(layers x T)) to the
+    full workload.  A port (the Rust binary needs cargo, probed below), a baseline only."""
+    import shutil
+    import numpy as np
+    import orc
+    from mamba_rs_amd import MambaConfig
+    cfg = MambaConfig(**{**cfg_kw, "n_layers": sample_layers})
+    P = orc.M1Params(cfg.d_model, cfg.d_state, cfg.d_conv, cfg.expand, sample_layers, cfg.d_model, seed=seed)
+    x = (np.random.default_rng(seed).standard_normal((sample_tokens, cfg.d_model)) * 0.02).astype(np.float32)
+    cs, ss = orc.m1_zero_state(P)
+    orc.m1_backbone_prefill(P, x[:8], cs, ss, identity_proj=True)          # warm-up
+    times = []
+    for _ in range(3):
+        cs, ss = orc.m1_zero_state(P)
+        t0 = time.perf_counter(); orc.m1_backbone_prefill(P, x, cs, ss, identity_proj=True); times.append(time.perf_counter() - t0)
+    ts = sorted(times)[1]
+    scale = (cfg_kw["n_layers"] / sample_layers) * (full_tokens / sample_tokens)
+    return {"kind": "port", "cargo_on_box": shutil.which("cargo") is not None, "cores": orc.num_threads(),
+            "sample": f"{sample_layers} of {cfg_kw['n_layers']} layers x {sample_tokens} tokens of one sequence, f32, median of 3",
+            "sample_ms": ts * 1e3, "scaled_to_full_ms": ts * scale * 1e3, "tok_per_s": full_tokens / (ts * scale)}
+
+
+def lm_leg(name, cfg_kw, vocab, prefill_bt, decode_b, decode_steps, seed=42, shared_layer=False, cpu_sample=None,
+           with_generate=True):
     """Prefill tok/s and greedy-decode us/step of a random-init LM-shaped backbone (bf16 storage):
-    token ids -> device embedding gather -> backbone (-> tied head -> argmax for decode)."""
+    token ids -> device embedding gather -> backbone (-> tied head -> argmax for decode).  With shared_layer the model's
+    layers all hold one layer's random weights (timing only: the kernels and their operand sizes are those of the full
+    model, the host-side initialisation is one layer's)."""
     import numpy as np
     from mamba_rs_amd import GpuMambaBackbone, GpuMambaLM, MambaConfig, MambaWeights, WeightDtype
     cfg = MambaConfig(**cfg_kw)
-    w = MambaWeights.random_lm(cfg, seed)
+    if shared_layer:
+        w = MambaWeights.random_lm(MambaConfig(**{**cfg_kw, "n_layers": 1}), seed)
+        w.layers = w.layers * cfg.n_layers
+    else:
+        w = MambaWeights.random_lm(cfg, seed)
     rng = np.random.default_rng(seed + 1)
     embed = (rng.standard_normal((vocab, cfg.d_model), dtype=np.float32) * np.float32(0.02))
     out = {"model": name}
+    if shared_layer:
+        out["weights"] = "one layer's random weights in every layer (timing only)"
     pb, pt = prefill_bt
     pre = GpuMambaBackbone.new_with_dtype(0, w, cfg, cfg.d_model, pb, WeightDtype.BF16)
     lm_p = GpuMambaLM(pre, embed)
@@ -133,6 +196,8 @@ def lm_leg(name, cfg_kw, vocab, prefill_bt, decode_b, decode_steps, seed=42):
     tp = sorted(times)[1]
     out["prefill"] = {"batch": pb, "seq_len": pt, "ms": tp * 1e3, "tok_per_s": pb * pt / tp}
     lm_p.close(); pre.close()
+    if cpu_sample:
+        out["cpu_port_prefill"] = cpu_prefill_sample(cfg_kw, cpu_sample[0], cpu_sample[1], pb * pt, seed)
     dec_out = []
     for db in (decode_b if isinstance(decode_b, (list, tuple)) else [decode_b]):
         dec = GpuMambaBackbone.new_with_dtype(0, w, cfg, cfg.d_model, db, WeightDtype.BF16)
@@ -155,15 +220,16 @@ def lm_leg(name, cfg_kw, vocab, prefill_bt, decode_b, decode_steps, seed=42):
         step_bytes = cfg.n_layers * layer_bytes + ((vocab + 63) // 64 * 64) * dm * es
         entry = {"batch": db, "steps": decode_steps, "us_per_step": td * 1e6, "tok_per_s": db / td,
                  "algorithmic_bytes_per_step": step_bytes, "hbm_frac": step_bytes / td / 1e9 / HBM_PEAK_GBPS}
-        # batched generation with the sampler in the loop: ragged prompts of 8..12 tokens, 128 new tokens per slot
-        from mamba_rs_amd import SampleParams
-        prompts = [[int(t) for t in rng.integers(0, vocab, 8 + (i % 5))] for i in range(db)]
-        params = [SampleParams(temperature=0.8, top_k=50, top_p=0.9, max_tokens=128, seed=i) for i in range(db)]
-        lm_d.generate_batch(prompts, params)                       # warm-up (captures the step)
-        t0 = time.perf_counter(); gen = lm_d.generate_batch(prompts, params); tg = time.perf_counter() - t0
-        n_gen = sum(len(g) for g in gen)
-        entry["generate_batch"] = {"sampler": "temperature 0.8, top_k 50, top_p 0.9", "new_tokens": n_gen, "ms": tg * 1e3,
-                                   "us_per_step": tg / (12 + 128) * 1e6, "gen_tok_per_s": n_gen / tg}
+        if with_generate:
+            # batched generation with the sampler in the loop: ragged prompts of 8..12 tokens, 128 new tokens per slot
+            from mamba_rs_amd import SampleParams
+            prompts = [[int(t) for t in rng.integers(0, vocab, 8 + (i % 5))] for i in range(db)]
+            params = [SampleParams(temperature=0.8, top_k=50, top_p=0.9, max_tokens=128, seed=i) for i in range(db)]
+            lm_d.generate_batch(prompts, params)                       # warm-up (captures the step)
+            t0 = time.perf_counter(); gen = lm_d.generate_batch(prompts, params); tg = time.perf_counter() - t0
+            n_gen = sum(len(g) for g in gen)
+            entry["generate_batch"] = {"sampler": "temperature 0.8, top_k 50, top_p 0.9", "new_tokens": n_gen, "ms": tg * 1e3,
+                                       "us_per_step": tg / (12 + 128) * 1e6, "gen_tok_per_s": n_gen / tg}
         dec_out.append(entry)
         lm_d.close(); dec.close()
     out["decode"] = dec_out
@@ -482,12 +548,12 @@ def main():
     ap.add_argument("--no-extras", action="store_true", help="only the headline scan line (no LM / Mamba-3 legs)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch one 256 MiB device copy (a known-size kernel to scale rocprof FETCH_SIZE/WRITE_SIZE by)")
-    ap.add_argument("--big", action="store_true", help="also run the 2.8b-shape LM leg (several minutes of host-side init)")
-    ap.add_argument("--legs", default="c1,lm,published,m1_kernels,m3,m3_engine",
-                    help="comma list of the extras to run: c1, lm, published, m1_kernels, m3, m3_engine (for profiling one leg at a time)")
+    ap.add_argument("--big", action="store_true", help="the 2.8b-shape LM leg with 64 independently initialised layers (minutes of host-side init) instead of one shared layer")
+    ap.add_argument("--legs", default="c1,lm,lm28,published,m1_kernels,m3,m3_engine",
+                    help="comma list of the extras to run: c1, lm, lm28, published, m1_kernels, m3, m3_engine (for profiling one leg at a time)")
     args = ap.parse_args()
     legs = {x.strip() for x in args.legs.split(",") if x.strip()}
-    unknown = legs - {"c1", "lm", "published", "m1_kernels", "m3", "m3_engine", "m3_prefill"}
+    unknown = legs - {"c1", "lm", "lm28", "published", "m1_kernels", "m3", "m3_engine", "m3_prefill"}
     if unknown:
         print(f"bench.py: unknown --legs entries {sorted(unknown)}", file=sys.stderr)
         sys.exit(2)
@@ -500,6 +566,7 @@ def main():
     inp = make_inputs(*shape)
     g = gpu_leg(args, inp, shape)
     gbps = nbytes / (g["ms_per_step"] * 1e-3) / 1e9
+    traffic, traffic_source = profiled_scan_traffic()
     out = {
         "metric": "m1_selective_scan_hbm_GBps",
         "value": gbps,
@@ -511,14 +578,16 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32",
+        "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": "isolated Mamba-1 selective scan forward, batch 8 x T 2048 x d_inner 1536 x d_state 16, "
                                "bf16 storage, f32 compute, SiLU gate fused, S4D-real A",
-                   "tokens_per_step": batch * T, "storage": "bf16"},
+                   "tokens_per_step": batch * T, "storage": "bf16", "compute": "f32",
+                   "general_A_ms_per_step": g["general_a_ms_per_step"],
+                   "general_A_note": "the same launch without the S4D-real flag (a trained checkpoint's A): 16 exponentials per step instead of one"},
         "tokens_per_s": batch * T / (g["ms_per_step"] * 1e-3),
         "roofline": {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": gbps / HBM_PEAK_GBPS, "traffic": MEASURED_SCAN_TRAFFIC_BYTES,
+                     "frac": gbps / HBM_PEAK_GBPS, "traffic": traffic, "traffic_source": traffic_source,
                      "kernels": ["chunk_state_kernel", "chunk_out_kernel"],
                      "algorithmic_bytes_per_launch": nbytes, "median_launch_ms": g["median_launch_ms"]},
     }
@@ -531,7 +600,7 @@ def main():
             extras["reference_default_configs_f32"] = default_configs_leg()
         if "lm" in legs:
             extras["lm_130m_shape_bf16"] = lm_leg("130m-shape", dict(d_model=768, d_state=16, d_conv=4, expand=2, n_layers=24), 50280,
-                                                  (8, 2048), [64, 1], 256)
+                                                  (8, 2048), [64, 1], 256, cpu_sample=(24, 256))
         if "published" in legs:
             extras["reference_published_configs"] = published_configs_leg()
         if "m1_kernels" in legs:
@@ -542,9 +611,10 @@ def main():
             extras["mamba3_768_bf16"]["backbone"] = m3_engine_leg()
         elif "m3_prefill" in legs:   # the backbone's prefill alone (not a default leg: the command behind its profile)
             extras["mamba3_768_bf16"]["backbone"] = m3_engine_leg(batches=())
-        if args.big:
+        if "lm28" in legs or args.big:
             extras["lm_2.8b_shape_bf16"] = lm_leg("2.8b-shape", dict(d_model=2560, d_state=16, d_conv=4, expand=2, n_layers=64), 50280,
-                                                  (4, 4096), [1, 16, 128], 128)
+                                                  (4, 4096), [1, 16, 128], 128, shared_layer=not args.big, cpu_sample=(2, 64),
+                                                  with_generate=False)
         out["extras"] = extras
     print(json.dumps(out))
 

@@ -350,8 +350,11 @@ __device__ __forceinline__ void load_a2(float (&a2)[16], const float *__restrict
 
 // Entering state of chunk c (c >= 1) from the summaries of chunks 0..c-1, in direct form:
 //   h_in(c) = sum_{k<c} exp(a * sum_{k<m<c} sumdelta_m) (.) S_k        (S_0 already holds h0's share)
-// The terms are independent, so the loads of S_k stream instead of forming a load->fma chain.  hs[n] is state n.
+// The terms are independent; the summaries are fetched four chunks at a time (68 loads in flight), so the fold costs
+// a few memory round trips instead of one per chunk -- every wave of pass B sits through it before its first step.
+// hs[n] is state n.
 constexpr int kMaxChunks = 32;
+constexpr int kFoldBatch = 4;
 template <bool S4D>
 __device__ __forceinline__ void fold_entering_state(float (&hs)[16], const float (&a2)[16],
                                                     const float *__restrict__ S, const float *__restrict__ sumd,
@@ -360,13 +363,25 @@ __device__ __forceinline__ void fold_entering_state(float (&hs)[16], const float
 #pragma unroll
     for (int j = 0; j < 16; j++) hs[j] = S[((sbase + c - 1) * 16 + j) * di + dd];  // k = c-1: weight 1
     float suffix = 0.0f;  // sum of sumdelta_m over k < m < c
-#pragma unroll 2
-    for (int k = c - 2; k >= 0; k--) {
-        suffix += sumd[(sbase + k + 1) * di + dd];
-        float da[16];
-        decay16<S4D>(suffix, a2, da);
+    for (int k0 = c - 2; k0 >= 0; k0 -= kFoldBatch) {
+        float Sv[kFoldBatch][16], sm[kFoldBatch];
 #pragma unroll
-        for (int j = 0; j < 16; j++) hs[j] = fmaf(da[j], S[((sbase + k) * 16 + j) * di + dd], hs[j]);
+        for (int i = 0; i < kFoldBatch; i++) {
+            const int k = max(k0 - i, 0);     // past the front: chunk 0 again, loaded and not used
+            sm[i] = sumd[(sbase + k + 1) * di + dd];
+#pragma unroll
+            for (int j = 0; j < 16; j++) Sv[i][j] = S[((sbase + k) * 16 + j) * di + dd];
+        }
+#pragma unroll
+        for (int i = 0; i < kFoldBatch; i++) {
+            if (k0 - i >= 0) {                // wave-uniform
+                suffix += sm[i];
+                float da[16];
+                decay16_tree<S4D>(suffix, a2, da);
+#pragma unroll
+                for (int j = 0; j < 16; j++) hs[j] = fmaf(da[j], Sv[i][j], hs[j]);
+            }
+        }
     }
 }
 
@@ -614,17 +629,6 @@ __global__ __launch_bounds__(kWave) void chunk_out_kernel(
     const int dd = live ? d0 + (int)threadIdx.x : di - 1;
     const unsigned lxb = live ? threadIdx.x * (unsigned)sizeof(T) : kDeadLaneOffset;
 
-    float hn[16], a2[16], hs[16], ar[16];   // hn[n]: state n; hs[r], ar[r]: state kStateOfReg(r)
-    load_a2<S4D>(a2, a_neg, dd);
-    if (c == 0) {
-#pragma unroll
-        for (int j = 0; j < 16; j++) hn[j] = h0copy[((int64_t)b * 16 + j) * di + dd];
-    } else {
-        fold_entering_state<S4D>(hn, a2, S, sumd, b, c, nchunk, di, dd);
-    }
-#pragma unroll
-    for (int r = 0; r < 16; r++) { hs[r] = hn[kStateOfReg(r)]; ar[r] = a2[kStateOfReg(r)]; }
-    const float Dd = Dp[dd];
     const int t0 = c * len, t1 = min(Tlen, t0 + len);
     const int tl = Tlen - 1;
     const int64_t row0 = (int64_t)b * Tlen;
@@ -647,17 +651,29 @@ __global__ __launch_bounds__(kWave) void chunk_out_kernel(
         }
     };
     const int nspans = (t1 - t0 + kSpan - 1) / kSpan;
-    RowPiece<T> nb, nc;
-    {
-        RowPiece<T> fb, fc;
-        piece_ld(fb, Bp, bc_stride, min(t0 + prow, tl));
-        piece_ld(fc, Cp, bc_stride, min(t0 + prow, tl));
-        Bs.publish(0, piece_widen(fb, (const T *)nullptr));
-        Cs.publish(0, piece_widen(fc, (const T *)nullptr));
-    }
+    // Everything the first steps need is requested before the entering state is folded, so the memory round trips of
+    // the prologue overlap instead of following one another (it is a startup bubble for the whole chip: all waves of a
+    // launch are in it at the same time).
+    RowPiece<T> nb, nc, fb, fc;
+    piece_ld(fb, Bp, bc_stride, min(t0 + prow, tl));
+    piece_ld(fc, Cp, bc_stride, min(t0 + prow, tl));
     piece_ld(nb, Bp, bc_stride, min(t0 + kSpan + prow, tl));
     piece_ld(nc, Cp, bc_stride, min(t0 + kSpan + prow, tl));
     load_group(rdA, ruA, rgA, t0);
+    const float Dd = Dp[dd];
+
+    float hn[16], a2[16], hs[16], ar[16];   // hn[n]: state n; hs[r], ar[r]: state kStateOfReg(r)
+    load_a2<S4D>(a2, a_neg, dd);
+    if (c == 0) {
+#pragma unroll
+        for (int j = 0; j < 16; j++) hn[j] = h0copy[((int64_t)b * 16 + j) * di + dd];
+    } else {
+        fold_entering_state<S4D>(hn, a2, S, sumd, b, c, nchunk, di, dd);
+    }
+#pragma unroll
+    for (int r = 0; r < 16; r++) { hs[r] = hn[kStateOfReg(r)]; ar[r] = a2[kStateOfReg(r)]; }
+    Bs.publish(0, piece_widen(fb, (const T *)nullptr));
+    Cs.publish(0, piece_widen(fc, (const T *)nullptr));
     v4f bv = Bs.read(0, 0), cv = Cs.read(0, 0);
     for (int sp = 0; sp < nspans; sp++) {
         const int ts = t0 + sp * kSpan, slot = sp & 1;
