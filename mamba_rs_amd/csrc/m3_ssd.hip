@@ -311,6 +311,16 @@ __global__ __launch_bounds__(HD * 4) __attribute__((amdgpu_waves_per_eu(HD == 64
     // One chunk from the registers of `r`; once they are in LDS the chunk c_next is requested into them.
     auto chunk = [&](Pre &r, int c, int c_next) {
         const int t0 = c * kCS;
+        // Issue priority falls with progress (after 1/2, 3/4, 7/8 of the walk): the arbiter of a SIMD serves its oldest wave
+        // first, so the workgroups sharing a compute unit would otherwise finish one after the other and the last one run
+        // alone; with the one that is behind served first they finish together.
+        {
+            const int done = c - c_begin, total = c_end - c_begin;
+            if (done * 8 >= total * 7) __builtin_amdgcn_s_setprio(0);
+            else if (done * 4 >= total * 3) __builtin_amdgcn_s_setprio(1);
+            else if (done * 2 >= total) __builtin_amdgcn_s_setprio(2);
+            else __builtin_amdgcn_s_setprio(3);
+        }
         lds_barrier();  // every wave is done reading the previous chunk's tiles (LDS only: y stores and the prefetch stay in flight)
         // ---- registers -> LDS ----
 #pragma unroll
