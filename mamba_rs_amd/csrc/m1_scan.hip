@@ -218,13 +218,34 @@ struct SplitPlan {
 constexpr int kGroup = 8;            // steps per activation prefetch group
 constexpr int kSpan = 2 * kGroup;    // steps per loop iteration and per staged block of B / C rows; chunk lengths are multiples
 
+// Chunk count: the waves of a launch (chunks x batch rows x channel tiles) should come to about three per SIMD -- what
+// keeps the vector ALU issuing -- and fill the 1024 SIMDs of the chip evenly: a SIMD with one wave more than the others
+// sets the time of the launch (4 x 4096 x 5120: 9 chunks = 2880 waves 375 us, 10 chunks = 3200 waves 404 us).
+constexpr int kSimds = 1024;   // 256 compute units x 4
 static SplitPlan make_split_plan(int batch, int Tlen, int di) {
     const int tiles = (di + kWave - 1) / kWave;
     const int64_t base = (int64_t)batch * tiles;
-    static const int target = [] { const char *e = getenv("MRS_SCAN_TARGET_WAVES"); return e ? atoi(e) : 3072; }();
-    int c = (int)((target + base - 1) / base);  // ~3 waves per SIMD on 1024 SIMDs
-    if (c > 32) c = 32;                          // the entering-state fold is O(C) per wave
-    if (c > Tlen / 32) c = Tlen / 32;            // chunks of at least 32 steps
+    static const int target = [] { const char *e = getenv("MRS_SCAN_TARGET_WAVES"); return e ? atoi(e) : 0; }();
+    int cmax = 32;                               // the entering-state fold is O(C) per wave
+    if (cmax > Tlen / 32) cmax = Tlen / 32;      // chunks of at least 32 steps
+    int c;
+    if (target > 0) {
+        c = (int)((target + base - 1) / base);
+    } else {
+        // between two and three and a half waves per SIMD, the fullest last round wins, fewer waves on a tie
+        // (3840 waves at that shape: 421 us)
+        int lo = (int)(2 * kSimds / base), hi = (int)((7 * kSimds / 2 + base - 1) / base);
+        if (lo < 2) lo = 2;
+        if (hi < lo) hi = lo;
+        c = hi;
+        double best = -1.0;
+        for (int k = lo; k <= hi; k++) {
+            const int64_t waves = k * base, rounds = (waves + kSimds - 1) / kSimds;
+            const double fill = (double)waves / (double)(rounds * kSimds);
+            if (fill > best + 1e-9) { best = fill; c = k; }
+        }
+    }
+    if (c > cmax) c = cmax;
     if (c < 1) c = 1;
     int len = (Tlen + c - 1) / c;
     len = (len + kSpan - 1) / kSpan * kSpan;
