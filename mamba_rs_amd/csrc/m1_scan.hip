@@ -295,6 +295,14 @@ template <typename T> struct LaneBuf {
 
 typedef float v4f __attribute__((ext_vector_type(4)));
 
+// Raw activation values of the T-split kernels sit zero-extended in a register of their own: as 16-bit values the
+// compiler packs them in pairs and spends vector instructions on packing and unpacking.
+template <typename T> struct Raw32 { using type = uint32_t; };
+template <> struct Raw32<float> { using type = float; };
+__device__ __forceinline__ float widen32(float v, const float *) { return v; }
+__device__ __forceinline__ float widen32(uint32_t v, const bf16_t *) { return __uint_as_float(v << 16); }
+__device__ __forceinline__ float widen32(uint32_t v, const f16_t *) { return (float)__builtin_bit_cast(_Float16, (uint16_t)v); }
+
 // state held in state register r (see the header comment): a 4x4 transpose, its own inverse
 __host__ __device__ constexpr int kStateOfReg(int r) { return 4 * (r % 4) + r / 4; }
 
@@ -485,7 +493,7 @@ __global__ __launch_bounds__(kWave) void chunk_state_kernel(
     const T *__restrict__ Bm, int64_t bc_stride,
     const float *__restrict__ a_neg, float *__restrict__ h0copy, float *__restrict__ S,
     float *__restrict__ sumd, int Tlen, int di, int tiles, int nchunk, int len) {
-    using raw_t = typename RawElem<T>::type;
+    using raw_t = typename Raw32<T>::type;
     __shared__ alignas(16) StagedRows Bs;
     // Chunks 0 .. nchunk-2 only, and chunk lengths are multiples of kSpan: every step of this wave's chunk
     // exists, so the walk has no tail.
@@ -559,8 +567,8 @@ __global__ __launch_bounds__(kWave) void chunk_state_kernel(
                     const int j = base + k;                               // row of the span
                     const v4f bcur = bv;
                     bv = j > 0 ? Bs.read(slot, j - 1) : Bs.read(slot ^ 1, kSpan - 1);   // the step after this one
-                    const float dl = widen(rd[k], (const T *)nullptr);
-                    const float uu = widen(ru[k], (const T *)nullptr);
+                    const float dl = widen32(rd[k], (const T *)nullptr);
+                    const float uu = widen32(ru[k], (const T *)nullptr);
                     const float x = fast_exp2(a2[0] * sd);
                     chain16_quad(S16, sd, x, dl * uu, dl, bcur);
                 }
@@ -599,8 +607,8 @@ __global__ __launch_bounds__(kWave) void chunk_state_kernel(
                     const int j = base + k;
                     const v4f bcur = bv;
                     bv = j < kSpan - 1 ? Bs.read(slot, j + 1) : Bs.read(slot ^ 1, 0);
-                    const float dl = widen(rd[k], (const T *)nullptr);
-                    const float uu = widen(ru[k], (const T *)nullptr);
+                    const float dl = widen32(rd[k], (const T *)nullptr);
+                    const float uu = widen32(ru[k], (const T *)nullptr);
                     const float du = dl * uu;
                     float da[16];
                     decay16_tree<false>(dl, a2, da);
@@ -639,7 +647,7 @@ __global__ __launch_bounds__(kWave) void chunk_out_kernel(
     const float *__restrict__ a_neg, const float *__restrict__ Dp, const T *__restrict__ gate, int64_t gate_stride,
     const float *__restrict__ h0copy, const float *__restrict__ S, const float *__restrict__ sumd,
     int Tlen, int di, int tiles, int nchunk, int len) {
-    using raw_t = typename RawElem<T>::type;
+    using raw_t = typename Raw32<T>::type;
     __shared__ alignas(16) StagedRows Bs, Cs;
     const int tile = blockIdx.x % tiles;
     const int rest = blockIdx.x / tiles;
@@ -713,8 +721,8 @@ __global__ __launch_bounds__(kWave) void chunk_out_kernel(
                 const v4f bcur = bv, ccur = cv;
                 bv = j < kSpan - 1 ? Bs.read(slot, j + 1) : Bs.read(slot ^ 1, 0);   // the rows of the next step
                 cv = j < kSpan - 1 ? Cs.read(slot, j + 1) : Cs.read(slot ^ 1, 0);
-                const float dl = widen(rd[k], (const T *)nullptr);
-                const float uu = widen(ru[k], (const T *)nullptr);
+                const float dl = widen32(rd[k], (const T *)nullptr);
+                const float uu = widen32(ru[k], (const T *)nullptr);
                 const float du = dl * uu;
                 float da[16];
                 if (S4D) {
@@ -740,7 +748,7 @@ __global__ __launch_bounds__(kWave) void chunk_out_kernel(
 #pragma unroll
                     for (int i = 0; i < 4; i++) hs[4 * q + i] = hq[q][i];
                 float acc, e;
-                const float z = GATE ? widen(rg[k], (const T *)nullptr) : 0.0f;
+                const float z = GATE ? widen32(rg[k], (const T *)nullptr) : 0.0f;
                 dot16_quad(acc, e, Dd, uu, z, ccur, hs);
                 if (GATE == 1) acc *= z;
                 if (GATE == 2) acc *= z * fast_rcp(1.0f + e);

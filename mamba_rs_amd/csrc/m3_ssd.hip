@@ -470,7 +470,8 @@ __global__ __launch_bounds__(HD * 4) __attribute__((amdgpu_waves_per_eu(HD == 64
     };
     if (STATE_ONLY) {
         // The state-only pass does little arithmetic per chunk, so its walk is as long as a memory round trip per chunk
-        // allows: two chunks are kept in flight (registers are not scarce here).
+        // allows: two chunks are kept in flight (registers are not scarce here).  The full pass does not have the registers
+        // for that: with a second set it spills at the 168 registers that three waves per SIMD allow (measured: 55 -> 93 us).
         Pre ra_, rb_;
         prefetch(ra_, c_begin);
         if (c_begin + 1 < c_end) prefetch(rb_, c_begin + 1);
