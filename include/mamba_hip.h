@@ -114,7 +114,7 @@ MRS_API int mrs_ssm_scan_fwd_ex(void *stream, int dtype, float *h, void *y, cons
  * MRS_SCAN_STATIC_SCRATCH_BYTES block per GPU, resident until the process ends -- so the call allocates nothing
  * and frees nothing.  Same arguments, routes and results as mrs_ssm_scan_fwd_ex given a workspace of that size.
  *   - A shape with mrs_ssm_scan_workspace_bytes() > MRS_SCAN_STATIC_SCRATCH_BYTES is refused (MRS_E_WORKSPACE);
- *     the benchmark shapes (8 x 2048 x 1536 and 4 x 4096 x 5120, d_state 16) need 13.3 MB and 13.8 MB; only very wide
+ *     the benchmark shapes (8 x 2048 x 1536 and 4 x 4096 x 5120, d_state 16) need 13.3 MB and 12.5 MB; only very wide
  *     batches (batch x d_inner above about 120 000 channels) need more.
  *   - The first call on a GPU looks the buffer's address up (hipGetSymbolAddress, no allocation); make that call
  *     outside a graph capture.

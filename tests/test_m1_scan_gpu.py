@@ -166,19 +166,20 @@ def test_scan_reads_b_c_in_place_from_xdbl(dtype):
 def test_scan_full_size_channel_subset_and_linearity():
     """The isolated-scan workload (B=8, T=2048, d_inner=1536, d_state=16, bf16, gated):
     channels are independent, so the oracle is run on a subset of channels of the
-    full-size launch; plus linearity in u (h0 = 0, f32 state): scan(2u) = 2 scan(u) exactly."""
+    full-size launch, once per A route; plus linearity in u (h0 = 0, f32 state): scan(2u) = 2 scan(u) exactly."""
     rng = np.random.default_rng(4)
     batch, T, di, ds = 8, 2048, 1536, 16
     inp = quantised(rng, batch, T, di, ds, orc.BF16)
     h0 = np.zeros((batch, di, ds), np.float32)
-    y, h = run_scan(inp, h0, orc.BF16, 2, flags=ops.A_S4D_REAL, split="auto")
     sel = np.sort(rng.choice(di, 48, replace=False))
     sub = dict(delta=inp["delta"][:, :, sel], u=inp["u"][:, :, sel], z=inp["z"][:, :, sel], B=inp["B"], C=inp["C"],
                a_neg=inp["a_neg"][sel], D=inp["D"][sel])
     y_ref, h_ref = orc.m1_scan_f64(h0[:, sel], sub["delta"], sub["u"], sub["B"], sub["C"], sub["a_neg"], sub["D"],
                                    gate=sub["z"], gate_mode=2)
-    assert_close(y[:, :, sel], y_ref, orc.BF16, "y[subset]")
-    assert_close(h[:, sel], h_ref, orc.F32, "h[subset]")
+    for flags in (ops.A_S4D_REAL, 0):     # the power-chain kernels and the general-A kernels (a trained checkpoint's)
+        y, h = run_scan(inp, h0, orc.BF16, 2, flags=flags, split="auto")
+        assert_close(y[:, :, sel], y_ref, orc.BF16, f"y[subset] flags={flags}")
+        assert_close(h[:, sel], h_ref, orc.F32, f"h[subset] flags={flags}")
     inp2 = dict(inp); inp2["u"] = inp["u"] * 2.0          # exact in bf16
     y2, h2 = run_scan(inp2, h0, orc.BF16, 0, flags=ops.A_S4D_REAL, split="auto")
     y1, h1 = run_scan(inp, h0, orc.BF16, 0, flags=ops.A_S4D_REAL, split="auto")
