@@ -201,22 +201,6 @@ __global__ __launch_bounds__(HD * 4) __attribute__((amdgpu_waves_per_eu(HD == 64
                     *reinterpret_cast<float4 *>(sp.Sinit + srow + 16 * jn) = make_float4(St[jn][0], St[jn][1], St[jn][2], St[jn][3]);
             }
         }
-    } else if (!STATE_ONLY) {
-        // entering state of super-chunk sc from the local states of the earlier ones (the state-only
-        // pass accumulates every later super-chunk from zero)
-        float run = 0.0f;
-        for (int k = sc - 1; k >= 0; k--) {
-            const int64_t slot = bh * (sp.nsc - 1) + k;
-            const float dec = fast_exp2(run * kLog2e);
-            const float *src = sp.Sloc + slot * (HD * DS) + (16 * w + lr) * DS + 4 * lg;
-#pragma unroll
-            for (int jn = 0; jn < KN; jn++) {
-                const float4 s = *reinterpret_cast<const float4 *>(src + 16 * jn);
-                St[jn] = (v4f){fmaf(dec, s.x, St[jn][0]), fmaf(dec, s.y, St[jn][1]), fmaf(dec, s.z, St[jn][2]),
-                               fmaf(dec, s.w, St[jn][3])};
-            }
-            run += sp.dAtot[slot];
-        }
     }
     float dAsum = 0.0f;
 
@@ -468,6 +452,38 @@ __global__ __launch_bounds__(HD * 4) __attribute__((amdgpu_waves_per_eu(HD == 64
             }
         }
     };
+    // Entering state of super-chunk sc from the local states of the earlier ones (the state-only pass accumulates every
+    // later super-chunk from zero):  sum_k exp(sum_{k<m<sc} dA_m) S_k.  The super-chunk's first chunk is requested before
+    // this, the local states are fetched four at a time and the decays come from one lane-parallel suffix sum; one state
+    // per memory round trip, each behind a dependent scalar load, kept the last super-chunk's workgroup in its prologue
+    // for 22 thousand cycles of a walk of 100 thousand.
+    auto fold_entering_state = [&]() {
+        const int64_t slot0 = bh * (sp.nsc - 1);
+        const float mine = l < sc ? sp.dAtot[slot0 + l] : 0.0f;               // nsc <= 32: a wave holds them all
+        const float upto = wave_inclusive_sum(mine);
+        const float total = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, upto), 63));
+        const float dec_l = fast_exp2((total - upto) * kLog2e);               // lane k: exp(sum_{k<m<sc} dA_m)
+        constexpr int kFB = 4;
+        for (int k0 = sc - 1; k0 >= 0; k0 -= kFB) {
+            float4 sv[kFB][KN];
+#pragma unroll
+            for (int i = 0; i < kFB; i++) {
+                const int k = max(k0 - i, 0);                                  // past the front: state 0 again, fetched and not used
+                const float *src = sp.Sloc + (slot0 + k) * (HD * DS) + (16 * w + lr) * DS + 4 * lg;
+#pragma unroll
+                for (int jn = 0; jn < KN; jn++) sv[i][jn] = *reinterpret_cast<const float4 *>(src + 16 * jn);
+            }
+#pragma unroll
+            for (int i = 0; i < kFB; i++) {
+                if (k0 - i < 0) continue;                                      // uniform over the workgroup
+                const float dec = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, dec_l), k0 - i));
+#pragma unroll
+                for (int jn = 0; jn < KN; jn++)
+                    St[jn] = (v4f){fmaf(dec, sv[i][jn].x, St[jn][0]), fmaf(dec, sv[i][jn].y, St[jn][1]), fmaf(dec, sv[i][jn].z, St[jn][2]),
+                                   fmaf(dec, sv[i][jn].w, St[jn][3])};
+            }
+        }
+    };
     if (STATE_ONLY) {
         // The state-only pass does little arithmetic per chunk, so its walk is as long as a memory round trip per chunk
         // allows: two chunks are kept in flight (registers are not scarce here).  The full pass does not have the registers
@@ -482,6 +498,7 @@ __global__ __launch_bounds__(HD * 4) __attribute__((amdgpu_waves_per_eu(HD == 64
     } else {
         Pre r_;
         prefetch(r_, c_begin);
+        if (sc > 0) fold_entering_state();
         for (int c = c_begin; c < c_end; c++) chunk(r_, c, c + 1);
     }
     if (STATE_ONLY) {
