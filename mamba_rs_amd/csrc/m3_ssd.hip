@@ -78,6 +78,7 @@ template <int HD, int DS> struct alignas(16) SsdSmem {
     alignas(16) uint16_t Ks[kCS][DS + kPad];       // K rows
     alignas(16) uint16_t Xs[kCS][HD + kPad];       // x rows of this head
     alignas(16) float sc[5][kCS];                  // dA, scale, gamma, exp(dA), w
+    float dAend;                                   // the chunk's total log-decay
     alignas(16) uint2 Ps[10][kWave];               // the 10 causal 16x16 tiles of P as A-operand fragments, by lane
     alignas(16) float gb[2][DS];                   // GEN: the head's B and C biases
 };
@@ -208,7 +209,7 @@ __global__ __launch_bounds__(HD * 4) __attribute__((amdgpu_waves_per_eu(HD == 64
     struct Pre {
         // plain: the Q / K vectors of the thread; GEN: two f32 vectors of cn / bn for each of them, and the 4 angles
         uint4 rq[NV * (GEN ? 2 : 1)], rk[NV * (GEN ? 2 : 1)], rang[GEN ? NV : 1], rx[2];
-        float rdt, rtr, ra, rdtn, rtrn;   // lane = step: dt, trap, a of the step and dt, trap of the step after it
+        float rdt, rtr, ra, rdtn, rtrn;   // wave 0 only.  lane = step: dt, trap, a of the step; dt, trap of the step after the chunk (every lane the same)
     };
     const unsigned es = (unsigned)sizeof(T);
     const int64_t kq_row = (int64_t)nh * DS;   // elements between consecutive steps of Q / K
@@ -264,11 +265,17 @@ __global__ __launch_bounds__(HD * 4) __attribute__((amdgpu_waves_per_eu(HD == 64
         const unsigned kq_c = (unsigned)t0 * (unsigned)kq_row * es, x_c = (unsigned)t0 * (unsigned)sp.x_stride * es, sc_c = (unsigned)t0 * (unsigned)nh * 4u;
         // The step scalars go first: loads return in order, and the compiler moves the first uses of these small values
         // ahead of the next request, so whoever waits for them must not wait for the tiles requested after them as well.
-        r.rdt = slab_ldf(dtbuf, sc_voff + sc_c, 0);
-        r.rtr = slab_ldf(trbuf, sc_voff + sc_c, 0);
-        r.ra = slab_ldf(abuf, sc_voff + sc_c, 0);
-        r.rdtn = slab_ldf(dtbuf, sc_voff + sc_c + (unsigned)nh * 4u, 0);   // the shifted gamma needs the step after (zero past the row)
-        r.rtrn = slab_ldf(trbuf, sc_voff + sc_c + (unsigned)nh * 4u, 0);
+        // Wave 0 alone fetches them: a step's scalars of one head are 4 bytes in a row of nh, so each of these loads
+        // touches as many cache lines as it has lanes -- with every wave fetching all five arrays the scalars were most of
+        // the workgroup's memory requests (measured with the loads taken out: state-only pass 39 -> 25 us, full pass
+        // 70 -> 59 us on the route that forms K and Q).  The step after the chunk is one address for all lanes.
+        if (w == 0) {
+            r.rdt = slab_ldf(dtbuf, sc_voff + sc_c, 0);
+            r.rtr = slab_ldf(trbuf, sc_voff + sc_c, 0);
+            r.ra = slab_ldf(abuf, sc_voff + sc_c, 0);
+            r.rdtn = slab_ldf(dtbuf, sc_c + (unsigned)(kCS * nh) * 4u, 0);   // zero past the row
+            r.rtrn = slab_ldf(trbuf, sc_c + (unsigned)(kCS * nh) * 4u, 0);
+        }
         if constexpr (GEN) {
             const unsigned bc_c = (unsigned)t0 * (unsigned)sp.g_bcs * 4u, ang_c = (unsigned)t0 * (unsigned)(nh * sp.g_nr) * 4u;
 #pragma unroll
@@ -342,24 +349,25 @@ __global__ __launch_bounds__(HD * 4) __attribute__((amdgpu_waves_per_eu(HD == 64
         }
         *reinterpret_cast<uint4 *>(&sm.Xs[x_row[0]][x_col[0]]) = r.rx[0];
         *reinterpret_cast<uint4 *>(&sm.Xs[x_row[1]][x_col[1]]) = r.rx[1];
-        // ---- per-step scalars, lane = step ----
-        float dAend;
-        {
-            float dtn = r.rdtn, trn = r.rtrn;
+        // ---- per-step scalars, lane = step (wave 0) ----
+        if (w == 0) {
+            // dt, trap of the step after this one: the next lane's, and for the last lane the step after the chunk
+            float dtn = __shfl_down(r.rdt, 1), trn = __shfl_down(r.rtr, 1);
+            if (l == kCS - 1) { dtn = r.rdtn; trn = r.rtrn; }
             if (t0 + l + 1 >= Tlen) { dtn = 0.f; trn = 1.f; }       // no step after the last one
             const float gam = r.rdt * r.rtr;
             const float scl = fmaf(dtn, 1.0f - trn, gam);
             const float dA = wave_inclusive_sum(r.ra * r.rdt);   // cumulative log-decay over the 64 steps
-            dAend = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, dA), 63));
-            if (w == 0) {   // every wave forms the same values (each needs dAend in its registers); one copy is kept
-                sm.sc[0][l] = dA;
-                sm.sc[1][l] = scl;
-                sm.sc[2][l] = gam;
-                sm.sc[3][l] = fast_exp2(dA * kLog2e);
-                sm.sc[4][l] = fast_exp2((dAend - dA) * kLog2e) * scl;
-            }
+            const float tot = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, dA), 63));
+            sm.sc[0][l] = dA;
+            sm.sc[1][l] = scl;
+            sm.sc[2][l] = gam;
+            sm.sc[3][l] = fast_exp2(dA * kLog2e);
+            sm.sc[4][l] = fast_exp2((tot - dA) * kLog2e) * scl;
+            if (l == 0) sm.dAend = tot;
         }
-        lds_barrier();  // tiles visible to every wave
+        lds_barrier();  // tiles and scalars visible to every wave
+        const float dAend = sm.dAend;
         if (c_next < c_end) prefetch(r, c_next);
         dAsum += dAend;
 
