@@ -165,23 +165,47 @@ __global__ __launch_bounds__(1024) void m3_layer_step_kernel(
 // before its own, so more segments mean more reads: at batch 4 x 4096 the two launches took 35 us with 32 segments,
 // 25 us with 64, 30 us with 128.
 constexpr int kAngleSegs = 64;
-// one thread per (row, j): j < nh -> the head scalars, j >= nh -> rope pair j - nh
-__global__ __launch_bounds__(256) void m3_scalars_kernel(float *__restrict__ dt_out, float *__restrict__ a_out, float *__restrict__ trap_out,
-                                                         float *__restrict__ tanhpi_out, const float *__restrict__ proj, int64_t ip,
-                                                         const float *__restrict__ dt_bias, int64_t rows, int nh, int nr, int sc_off,
+// One workgroup per 64 consecutive rows, a thread per (row, j) with j fastest: j < nh -> the head scalars, j >= nh -> rope
+// pair j - nh.  When the scan wants its per-head inputs with the steps of a head next to each other (dtT, aT, trapT:
+// [batch, nh, T]) the tile is turned in LDS, so those stores are 256-byte runs as well.
+__global__ __launch_bounds__(1024) void m3_scalars_kernel(float *__restrict__ dt_out, float *__restrict__ a_out, float *__restrict__ trap_out,
+                                                         float *__restrict__ tanhpi_out, float *__restrict__ dtT, float *__restrict__ aT,
+                                                         float *__restrict__ trapT, const float *__restrict__ proj, int64_t ip,
+                                                         const float *__restrict__ dt_bias, int64_t rows, int Tlen, int nh, int nr, int sc_off,
                                                          float a_floor) {
-    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    extern __shared__ float turned[];   // [3][nh][65]
+    const int64_t r0 = (int64_t)blockIdx.x * 64;
     const int per = nh + nr;
-    if (idx >= rows * per) return;
-    const int64_t r = idx / per;
-    const int j = (int)(idx - r * per);
-    const float *sc = proj + r * ip + sc_off;
-    if (j < nh) {
-        dt_out[r * nh + j] = softplus20(sc[j] + dt_bias[j]);
-        a_out[r * nh + j] = fminf(-heavy_tail(sc[nh + j]), -a_floor);
-        trap_out[r * nh + j] = sigmoidf_fast(sc[2 * nh + j]);
-    } else {
-        tanhpi_out[r * nr + (j - nh)] = tanhf(sc[3 * nh + (j - nh)]) * kPi;
+    for (int i = threadIdx.x; i < 64 * per; i += (int)blockDim.x) {
+        const int rl = i / per, j = i - rl * per;
+        const int64_t r = r0 + rl;
+        if (r >= rows) continue;
+        const float *sc = proj + r * ip + sc_off;
+        if (j < nh) {
+            const float d = softplus20(sc[j] + dt_bias[j]);
+            const float a = fminf(-heavy_tail(sc[nh + j]), -a_floor);
+            const float tr = sigmoidf_fast(sc[2 * nh + j]);
+            dt_out[r * nh + j] = d;
+            a_out[r * nh + j] = a;
+            trap_out[r * nh + j] = tr;
+            if (dtT) {
+                turned[(0 * nh + j) * 65 + rl] = d;
+                turned[(1 * nh + j) * 65 + rl] = a;
+                turned[(2 * nh + j) * 65 + rl] = tr;
+            }
+        } else {
+            tanhpi_out[r * nr + (j - nh)] = tanhf(sc[3 * nh + (j - nh)]) * kPi;
+        }
+    }
+    if (!dtT) return;
+    __syncthreads();
+    for (int i = threadIdx.x; i < 3 * nh * 64; i += (int)blockDim.x) {
+        const int rl = i & 63, hj = i >> 6, arr = hj / nh, h = hj - arr * nh;
+        const int64_t r = r0 + rl;
+        if (r >= rows) continue;
+        const int64_t b = r / Tlen, t = r - b * Tlen;
+        float *dst = arr == 0 ? dtT : (arr == 1 ? aT : trapT);
+        dst[(b * nh + h) * Tlen + t] = turned[hj * 65 + rl];
     }
 }
 
@@ -191,7 +215,7 @@ __global__ __launch_bounds__(256) void m3_scalars_kernel(float *__restrict__ dt_
 //   sums:  seg_sum[b][seg][j] = sum over the segment of (tanh * pi)[t][a] * dt[t][h] (f64); segment 0 also snapshots
 //          the entering angles, which the last segment of the second launch overwrites;
 //   apply: start = entering angle advanced over the segments before (wrapped after every segment), then the running
-//          sums inside the segment, wrapped after every step; angle_out [rows][nh][nr] f32.
+//          sums inside the segment, wrapped after every step; angle_out [rows][nh][nr] f32 (or head-major, see below).
 __global__ __launch_bounds__(1024) void m3_angle_sums_kernel(double *__restrict__ seg_sum, float *__restrict__ snap,
                                                              const float *__restrict__ angle_state, const float *__restrict__ dt,
                                                              const float *__restrict__ tanhpi, int Tlen, int nh, int nr, int nsegs) {
@@ -230,7 +254,7 @@ __global__ __launch_bounds__(1024) void m3_angle_sums_kernel(double *__restrict_
 __global__ __launch_bounds__(1024) void m3_angle_apply_kernel(float *__restrict__ angle_out, float *__restrict__ angle_state,
                                                               const double *__restrict__ seg_sum, const float *__restrict__ snap,
                                                               const float *__restrict__ dt, const float *__restrict__ tanhpi, int Tlen,
-                                                              int nh, int nr, int nsegs) {
+                                                              int nh, int nr, int nsegs, int head_major) {
     const int b = blockIdx.x / nsegs, seg = blockIdx.x - b * nsegs, per = nh * nr;
     const int seglen = (Tlen + nsegs - 1) / nsegs;
     const int t0 = min(Tlen, seg * seglen), t1 = min(Tlen, t0 + seglen);
@@ -251,7 +275,9 @@ __global__ __launch_bounds__(1024) void m3_angle_apply_kernel(float *__restrict_
             for (int i = 0; i < 32; i++) p4[i & 3] += v[i];
         }
         double acc = wrap_2pi((double)snap[(int64_t)b * per + j] + ((p4[0] + p4[1]) + (p4[2] + p4[3])));
-        float *out = angle_out + (int64_t)b * Tlen * per + j;
+        // angle_out [rows][nh][nr], or with the steps of a head next to each other: [batch][nh][T][nr]
+        float *out = angle_out + (head_major ? ((int64_t)b * nh + h) * Tlen * nr + a : (int64_t)b * Tlen * per + j);
+        const int out_step = head_major ? nr : per;
         float xa[8], xb[8], na[8], nb[8];
         auto request = [&](float (&a8)[8], float (&b8)[8], int tg) {
 #pragma unroll
@@ -274,7 +300,7 @@ __global__ __launch_bounds__(1024) void m3_angle_apply_kernel(float *__restrict_
             for (int i = 0; i < 8; i++) { xa[i] = na[i]; xb[i] = nb[i]; }
 #pragma unroll
             for (int i = 0; i < 8; i++)
-                if (tg + i < t1) out[(int64_t)(tg + i) * per] = (float)wrap_2pi(run[i]);
+                if (tg + i < t1) out[(int64_t)(tg + i) * out_step] = (float)wrap_2pi(run[i]);
             acc = wrap_2pi(acc);   // once per group: keeps the running sum small
         }
         if (seg == nsegs - 1) angle_state[(int64_t)b * per + j] = (float)acc;
@@ -518,6 +544,7 @@ struct mrs_m3_backbone {
     // prefill scratch for sequences of pf_T steps (0: not allocated)
     int pf_T;
     float *pf_in, *pf_residual, *pf_proj, *pf_dt, *pf_a, *pf_trap, *pf_tanhpi, *pf_angle, *pf_angle_snap;
+    float *pf_dtT, *pf_aT, *pf_trapT;   // [batch, nh, T] copies of dt, a, trap for the scan that forms K and Q itself
     double *pf_angle_sums;   // [batch][kAngleSegs][nh * n_rope] per-segment angle increments of the prefill
     float *pf_bcn;           // [rows][2 * d_state] normalised and weighted B | C rows for the scan that forms K and Q itself
     void *pf_normed, *pf_bulk, *pf_x, *pf_K, *pf_Q, *pf_y, *pf_gated, *pf_out, *pf_ws;
@@ -845,6 +872,9 @@ static int alloc_prefill_scratch3(mrs_m3_backbone *bb, int T) {
     MRS_TRY(dev_alloc3(bb, (void **)&bb->pf_dt, rows * nh * 4));
     MRS_TRY(dev_alloc3(bb, (void **)&bb->pf_a, rows * nh * 4));
     MRS_TRY(dev_alloc3(bb, (void **)&bb->pf_trap, rows * nh * 4));
+    MRS_TRY(dev_alloc3(bb, (void **)&bb->pf_dtT, rows * nh * 4));
+    MRS_TRY(dev_alloc3(bb, (void **)&bb->pf_aT, rows * nh * 4));
+    MRS_TRY(dev_alloc3(bb, (void **)&bb->pf_trapT, rows * nh * 4));
     MRS_TRY(dev_alloc3(bb, (void **)&bb->pf_tanhpi, rows * nrz * 4));
     MRS_TRY(dev_alloc3(bb, (void **)&bb->pf_angle, rows * nh * nrz * 4));
     MRS_TRY(dev_alloc3(bb, (void **)&bb->pf_angle_sums, (size_t)bb->batch * kAngleSegs * nh * nrz * sizeof(double)));
@@ -962,10 +992,21 @@ int prefill_body3(mrs_m3_backbone *bb, int T) {
                 bulk = bb->pf_bulk; ldb = nb; bcp = bb->pf_proj; scp = bcp + nbc; lds_ = ns;
             }
         }
+        // the chunked kernel reads x in place out of the bulk rows.  (Folding the SiLU gate into its y store was
+        // measured and dropped: the scattered z reads cost the latency-bound kernel 54 us against 28 us for the
+        // separate gate pass.)
+        const bool in_place = chunked_ok && dt != MRS_F32 && ldb % 8 == 0 && di % 8 == 0;
+        // one group at headdim = d_state = 64 with the rope pairs in fours: the scan builds its K and Q tiles from the
+        // normalised B / C rows and the angles, so the [rows, nheads, d_state] K and Q never exist in memory
+        const bool fused_kq = in_place && hd == 64 && ds == 64 && c.ngroups == 1 && nr > 0 && nr % 4 == 0 && !no_fused_kq;
+        // that scan reads a head's step scalars and angles as runs of steps (a chunk's 64 steps of one head are 256
+        // bytes instead of 4 bytes in each of 64 rows): the kernels in front of it write them that way
+        const size_t turned_bytes = (size_t)3 * nh * 65 * sizeof(float);
+        const bool head_major = fused_kq && turned_bytes <= 48 * 1024;
         {
-            const int64_t n = rows * (nh + nr);
-            hipLaunchKernelGGL(m3_scalars_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, bb->stream, bb->pf_dt, bb->pf_a, bb->pf_trap,
-                               bb->pf_tanhpi, scp, lds_, lw.dt_bias, rows, nh, nr, 0, c.a_floor);
+            hipLaunchKernelGGL(m3_scalars_kernel, dim3((unsigned)((rows + 63) / 64)), dim3(1024), head_major ? turned_bytes : 0, bb->stream,
+                               bb->pf_dt, bb->pf_a, bb->pf_trap, bb->pf_tanhpi, head_major ? bb->pf_dtT : nullptr, bb->pf_aT, bb->pf_trapT, scp,
+                               lds_, lw.dt_bias, rows, T, nh, nr, 0, c.a_floor);
             MRS_TRY(check_launch("m3_scalars_kernel"));
         }
         if (nr > 0) {
@@ -975,23 +1016,17 @@ int prefill_body3(mrs_m3_backbone *bb, int T) {
                                bb->pf_angle_snap, ang, bb->pf_dt, bb->pf_tanhpi, T, nh, nr, nsegs);
             MRS_TRY(check_launch("m3_angle_sums_kernel"));
             hipLaunchKernelGGL(m3_angle_apply_kernel, dim3((unsigned)(B * nsegs)), dim3((unsigned)threads), 0, bb->stream, bb->pf_angle, ang,
-                               bb->pf_angle_sums, bb->pf_angle_snap, bb->pf_dt, bb->pf_tanhpi, T, nh, nr, nsegs);
+                               bb->pf_angle_sums, bb->pf_angle_snap, bb->pf_dt, bb->pf_tanhpi, T, nh, nr, nsegs, head_major ? 1 : 0);
             MRS_TRY(check_launch("m3_angle_apply_kernel"));
         }
-        // the chunked kernel reads x in place out of the bulk rows.  (Folding the SiLU gate into its y store was
-        // measured and dropped: the scattered z reads cost the latency-bound kernel 54 us against 28 us for the
-        // separate gate pass.)
-        const bool in_place = chunked_ok && dt != MRS_F32 && ldb % 8 == 0 && di % 8 == 0;
-        // one group at headdim = d_state = 64 with the rope pairs in fours: the scan builds its K and Q tiles from the
-        // normalised B / C rows and the angles, so the [rows, nheads, d_state] K and Q never exist in memory
-        const bool fused_kq = in_place && hd == 64 && ds == 64 && c.ngroups == 1 && nr > 0 && nr % 4 == 0 && !no_fused_kq;
         if (fused_kq) {
             hipLaunchKernelGGL(m3_bcn_rows_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, bb->stream, bb->pf_bcn, bcp, lds_, lw.bnw, lw.cnw,
                                rows, c.rms_norm_eps);
             MRS_TRY(check_launch("m3_bcn_rows_kernel"));
-            const SsdGenArgs gen = {bb->pf_bcn, bb->pf_bcn + ds, 2 * (int64_t)ds, bb->pf_angle, lw.b_bias, lw.c_bias, nr};
+            const SsdGenArgs gen = {bb->pf_bcn, bb->pf_bcn + ds, 2 * (int64_t)ds, bb->pf_angle, lw.b_bias, lw.c_bias, nr, head_major ? 1 : 0};
             const char *xb = (const char *)bulk + (size_t)di * es;
-            MRS_TRY(m3_ssd_fwd_ex(bb->stream, dt, ssm, kst, vst, bb->pf_y, xb, ldb, nullptr, nullptr, bb->pf_dt, bb->pf_trap, bb->pf_a, lw.D,
+            MRS_TRY(m3_ssd_fwd_ex(bb->stream, dt, ssm, kst, vst, bb->pf_y, xb, ldb, nullptr, nullptr, head_major ? bb->pf_dtT : bb->pf_dt,
+                                  head_major ? bb->pf_trapT : bb->pf_trap, head_major ? bb->pf_aT : bb->pf_a, lw.D,
                                   bb->pf_ws, bb->pf_ws_bytes, MRS_M3_CARRY_STATE, B, T, nh, hd, ds, 64, &gen));
         } else if (in_place) {
             MRS_DISPATCH_DTYPE(dt, T_, MRS_TRY(launch_kq_t<T_>(bb, lw, rows, bulk, ldb, bcp, lds_, false)));

@@ -109,6 +109,7 @@ struct SsdSplit {
     int64_t g_bcs;
     int g_nr;
     int g_groups;         // batch rows x super-chunks of the launch (set per launch)
+    int g_head_major;     // dt, trap, a_val are [batch, nh, T] and the angles [batch, nh, T, g_nr]
 };
 
 // Cross-lane moves on the data-parallel-primitive path of the vector ALU (no LDS round trip, unlike the shuffle
@@ -189,7 +190,7 @@ __global__ __launch_bounds__(HD * 4) __attribute__((amdgpu_waves_per_eu(HD == 64
             }
         } else if (carry) {
             // S_in = ssm + dt_0 (1 - trap_0) v_in (x) k_in : the beta term of step 0, which belongs to the carried state
-            const int64_t t0row = (int64_t)b * Tlen * nh + h;
+            const int64_t t0row = (GEN && sp.g_head_major) ? ((int64_t)b * nh + h) * Tlen : (int64_t)b * Tlen * nh + h;
             const float sgm1 = dt[t0row] * (1.0f - trap[t0row]);
             const float vin = vst[bh * HD + 16 * w + lr];
 #pragma unroll
@@ -217,10 +218,14 @@ __global__ __launch_bounds__(HD * 4) __attribute__((amdgpu_waves_per_eu(HD == 64
     const __amdgpu_buffer_rsrc_t kbuf = slab_rsrc(K + ((int64_t)b * Tlen * nh + h) * DS, ((int64_t)Tlen * kq_row - h * DS) * es);
     const __amdgpu_buffer_rsrc_t xbuf =
         slab_rsrc(x + (int64_t)b * Tlen * sp.x_stride + h * HD, ((int64_t)Tlen * sp.x_stride - h * HD) * es);
-    const int64_t sc_bytes = ((int64_t)Tlen * nh - h) * 4;
-    const __amdgpu_buffer_rsrc_t dtbuf = slab_rsrc(dt + (int64_t)b * Tlen * nh + h, sc_bytes);
-    const __amdgpu_buffer_rsrc_t trbuf = slab_rsrc(trap + (int64_t)b * Tlen * nh + h, sc_bytes);
-    const __amdgpu_buffer_rsrc_t abuf = slab_rsrc(a_val + (int64_t)b * Tlen * nh + h, sc_bytes);
+    // step scalars of this head: a row of nh apart ([batch, T, nh], the reference's layout) or next to each other
+    const bool hm = GEN && sp.g_head_major;
+    const int sc_step = hm ? 1 : nh;               // floats between consecutive steps
+    const int64_t sc_base = hm ? ((int64_t)b * nh + h) * Tlen : (int64_t)b * Tlen * nh + h;
+    const int64_t sc_bytes = hm ? (int64_t)Tlen * 4 : ((int64_t)Tlen * nh - h) * 4;
+    const __amdgpu_buffer_rsrc_t dtbuf = slab_rsrc(dt + sc_base, sc_bytes);
+    const __amdgpu_buffer_rsrc_t trbuf = slab_rsrc(trap + sc_base, sc_bytes);
+    const __amdgpu_buffer_rsrc_t abuf = slab_rsrc(a_val + sc_base, sc_bytes);
     const __amdgpu_buffer_rsrc_t ybuf = slab_rsrc(y + (int64_t)b * Tlen * di + h * HD + 16 * w, ((int64_t)Tlen * di - h * HD - 16 * w) * es);
     unsigned kq_voff[NV];
 #pragma unroll
@@ -233,14 +238,16 @@ __global__ __launch_bounds__(HD * 4) __attribute__((amdgpu_waves_per_eu(HD == 64
     const bool g_rot = g_col < 2 * sp.g_nr;        // its pairs are rotated (all four or none: g_nr is a multiple of 4)
     const __amdgpu_buffer_rsrc_t bnbuf = slab_rsrc(GEN ? sp.g_bn + (int64_t)b * Tlen * sp.g_bcs : nullptr, GEN ? (int64_t)Tlen * sp.g_bcs * 4 : 0);
     const __amdgpu_buffer_rsrc_t cnbuf = slab_rsrc(GEN ? sp.g_cn + (int64_t)b * Tlen * sp.g_bcs : nullptr, GEN ? (int64_t)Tlen * sp.g_bcs * 4 : 0);
+    const int ang_step = hm ? sp.g_nr : nh * sp.g_nr;   // floats between the angle rows of consecutive steps
     const __amdgpu_buffer_rsrc_t angbuf =
-        slab_rsrc(GEN ? sp.g_ang + ((int64_t)b * Tlen * nh + h) * sp.g_nr : nullptr, GEN ? ((int64_t)Tlen * nh - h) * sp.g_nr * 4 : 0);
+        slab_rsrc(GEN ? sp.g_ang + (hm ? ((int64_t)b * nh + h) * Tlen : (int64_t)b * Tlen * nh + h) * sp.g_nr : nullptr,
+                  GEN ? (hm ? (int64_t)Tlen : (int64_t)Tlen * nh - h) * sp.g_nr * 4 : 0);
     unsigned bc_voff[NV], ang_voff[NV];
 #pragma unroll
     for (int v = 0; v < NV; v++) {
         const int vi = tid + v * NTHR, row = vi / VPR;
         bc_voff[v] = GEN && vi < NVEC ? (unsigned)(row * (int)sp.g_bcs + g_col) * 4u : 0u;
-        ang_voff[v] = GEN && vi < NVEC && g_rot ? (unsigned)(row * nh * sp.g_nr + g_col / 2) * 4u : 0u;
+        ang_voff[v] = GEN && vi < NVEC && g_rot ? (unsigned)(row * ang_step + g_col / 2) * 4u : 0u;
     }
     if (GEN) {   // visible to every wave after the barrier at the top of the first chunk
         for (int n = tid; n < DS; n += NTHR) { sm.gb[0][n] = sp.g_bb[h * DS + n]; sm.gb[1][n] = sp.g_cb[h * DS + n]; }
@@ -256,13 +263,13 @@ __global__ __launch_bounds__(HD * 4) __attribute__((amdgpu_waves_per_eu(HD == 64
         x_row[v] = vi / VPRX; x_col[v] = (vi % VPRX) * 8;
         x_voff[v] = (unsigned)(x_row[v] * (int)sp.x_stride + x_col[v]) * es;
     }
-    const unsigned sc_voff = (unsigned)l * (unsigned)nh * 4u;
+    const unsigned sc_voff = (unsigned)l * (unsigned)sc_step * 4u;
     const unsigned y_voff = (unsigned)(4 * lg * di + lr) * es;
     // Accesses past the end of the batch row (the tail of a last, partial chunk) fall outside the resources: loads give
     // zero and stores are dropped by the bounds check, which covers the vector offset -- so the chunk's offset goes there.
     auto prefetch = [&](Pre &r, int c) {
         const int t0 = c * kCS;
-        const unsigned kq_c = (unsigned)t0 * (unsigned)kq_row * es, x_c = (unsigned)t0 * (unsigned)sp.x_stride * es, sc_c = (unsigned)t0 * (unsigned)nh * 4u;
+        const unsigned kq_c = (unsigned)t0 * (unsigned)kq_row * es, x_c = (unsigned)t0 * (unsigned)sp.x_stride * es, sc_c = (unsigned)t0 * (unsigned)sc_step * 4u;
         // The step scalars go first: loads return in order, and the compiler moves the first uses of these small values
         // ahead of the next request, so whoever waits for them must not wait for the tiles requested after them as well.
         // Wave 0 alone fetches them: a step's scalars of one head are 4 bytes in a row of nh, so each of these loads
@@ -273,11 +280,11 @@ __global__ __launch_bounds__(HD * 4) __attribute__((amdgpu_waves_per_eu(HD == 64
             r.rdt = slab_ldf(dtbuf, sc_voff + sc_c, 0);
             r.rtr = slab_ldf(trbuf, sc_voff + sc_c, 0);
             r.ra = slab_ldf(abuf, sc_voff + sc_c, 0);
-            r.rdtn = slab_ldf(dtbuf, sc_c + (unsigned)(kCS * nh) * 4u, 0);   // zero past the row
-            r.rtrn = slab_ldf(trbuf, sc_c + (unsigned)(kCS * nh) * 4u, 0);
+            r.rdtn = slab_ldf(dtbuf, sc_c + (unsigned)(kCS * sc_step) * 4u, 0);   // zero past the row
+            r.rtrn = slab_ldf(trbuf, sc_c + (unsigned)(kCS * sc_step) * 4u, 0);
         }
         if constexpr (GEN) {
-            const unsigned bc_c = (unsigned)t0 * (unsigned)sp.g_bcs * 4u, ang_c = (unsigned)t0 * (unsigned)(nh * sp.g_nr) * 4u;
+            const unsigned bc_c = (unsigned)t0 * (unsigned)sp.g_bcs * 4u, ang_c = (unsigned)t0 * (unsigned)ang_step * 4u;
 #pragma unroll
             for (int v = 0; v < NV; v++) {
                 if (!STATE_ONLY) {
@@ -528,7 +535,7 @@ __global__ __launch_bounds__(HD * 4) __attribute__((amdgpu_waves_per_eu(HD == 64
         for (int n = tid; n < DS; n += NTHR) {
             const int j = n >> 1;
             const float k0 = sp.g_bn[last * sp.g_bcs + 2 * j] + sp.g_bb[h * DS + 2 * j], k1 = sp.g_bn[last * sp.g_bcs + 2 * j + 1] + sp.g_bb[h * DS + 2 * j + 1];
-            const float a = j < sp.g_nr ? sp.g_ang[(last * nh + h) * sp.g_nr + j] : 0.f;
+            const float a = j < sp.g_nr ? sp.g_ang[(hm ? ((int64_t)b * nh + h) * Tlen + (Tlen - 1) : last * nh + h) * sp.g_nr + j] : 0.f;
             const float sn = __sinf(a), cs = __cosf(a);
             const T kv = (T)((n & 1) ? sn * k0 + cs * k1 : cs * k0 - sn * k1);
             kst[bh * DS + n] = (float)kv;
@@ -711,9 +718,9 @@ int mrs::m3_ssd_fwd_ex(void *stream, int dtype, float *ssm_state, float *k_state
     if (!aligned(x, 16) || !aligned(K, 16) || !aligned(Q, 16) || !aligned(ssm_state, 16) || !aligned(k_state, 16))
         return fail(MRS_E_ALIGN, "%s: x, K, Q, ssm_state, k_state must be 16-byte aligned", fn);
     // Super-chunk split when the caller's workspace holds it; otherwise one workgroup walks the whole sequence.
-    SsdSplit sp = {nullptr, nullptr, nullptr, 1, (T + kCS - 1) / kCS, x_stride, nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0, 0};
+    SsdSplit sp = {nullptr, nullptr, nullptr, 1, (T + kCS - 1) / kCS, x_stride, nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0, 0, 0};
     auto with_gen = [&](SsdSplit &o) {
-        if (gen) { o.g_bn = gen->bn; o.g_cn = gen->cn; o.g_ang = gen->angle; o.g_bb = gen->b_bias; o.g_cb = gen->c_bias; o.g_bcs = gen->bc_stride; o.g_nr = gen->n_rope; }
+        if (gen) { o.g_bn = gen->bn; o.g_cn = gen->cn; o.g_ang = gen->angle; o.g_bb = gen->b_bias; o.g_cb = gen->c_bias; o.g_bcs = gen->bc_stride; o.g_nr = gen->n_rope; o.g_head_major = gen->head_major; }
     };
     with_gen(sp);
     {
@@ -723,7 +730,7 @@ int mrs::m3_ssd_fwd_ex(void *stream, int dtype, float *ssm_state, float *k_state
         const size_t need = ssd_split_bytes(batch, nheads, headdim, d_state, nsc, &o_dA, &o_init);
         if (nsc > 1 && workspace && workspace_bytes >= need && aligned(workspace, 16)) {
             char *ws = (char *)workspace;
-            sp = SsdSplit{(float *)ws, (float *)(ws + o_dA), (float *)(ws + o_init), nsc, cps, x_stride, nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0, 0};
+            sp = SsdSplit{(float *)ws, (float *)(ws + o_dA), (float *)(ws + o_init), nsc, cps, x_stride, nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0, 0, 0};
             with_gen(sp);
         }
     }
