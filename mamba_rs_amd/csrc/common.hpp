@@ -133,12 +133,13 @@ int launch_prenorm_rows(hipStream_t st, int dtype, float *partials, int n_partia
 
 // mrs_m3_ssd_fwd with x read in place out of wider rows (x_stride elements apart, 0 = dense; 16-bit storage only).
 // With `gen` the kernel forms K and Q itself (K and Q are not read and may be null): K = rot(angle, bn + b_bias[head]),
-// Q = rot(angle, cn + c_bias[head]) with bn / cn the normalised and weighted B / C rows (f32, bc_stride floats apart),
+// Q = rot(angle, cn + c_bias[head]) with bn / cn the normalised and weighted B / C rows (storage type, bc_stride elements
+// apart -- the reference's bcnorm_fwd_* stores them in the activation type as well, kernels/mamba3_ops.cu:1193-1230),
 // angle [batch, T, nheads, n_rope] and the first n_rope pairs of a row turned.  headdim = d_state = 64, 16-bit storage.
 // head_major: the caller keeps what the kernel reads per (head, step) with the steps of a head next to each other --
 // dt, trap, a_val as [batch, nheads, T] and angle as [batch, nheads, T, n_rope] -- so a chunk's 64 steps are a few whole
 // cache lines instead of a piece of 64 different ones.
-struct SsdGenArgs { const float *bn, *cn; int64_t bc_stride; const float *angle, *b_bias, *c_bias; int n_rope; int head_major; };
+struct SsdGenArgs { const void *bn, *cn; int64_t bc_stride; const float *angle, *b_bias, *c_bias; int n_rope; int head_major; };
 int m3_ssd_fwd_ex(void *stream, int dtype, float *ssm_state, float *k_state, float *v_state, void *y, const void *x,
                   int64_t x_stride, const void *K, const void *Q, const float *dt, const float *trap, const float *a_val,
                   const float *D, void *workspace, size_t workspace_bytes, unsigned flags, int batch, int T, int nheads,

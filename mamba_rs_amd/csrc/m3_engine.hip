@@ -447,9 +447,13 @@ __global__ __launch_bounds__(256) void m3_kq_rows_kernel(
 }
 
 // The part of K and Q that all heads share, for the scan kernel that forms K and Q itself (one group, d_state 64):
-// out[row] = [B * rsqrt(mean(B^2) + eps) * bnw | C * rsqrt(mean(C^2) + eps) * cnw] in f32 (bcnorm_fwd, ops/norms.rs:50-80);
-// the per-head bias and the rotation happen where the tiles are built.  A wave per row, a lane per coordinate.
-__global__ __launch_bounds__(256) void m3_bcn_rows_kernel(float *__restrict__ out, const float *__restrict__ bc, int64_t ldbc,
+// out[row] = [B * rsqrt(mean(B^2) + eps) * bnw | C * rsqrt(mean(C^2) + eps) * cnw] (bcnorm_fwd, ops/norms.rs:50-80), formed in
+// f32 from the f32 projection and stored in the activation type, as the reference's bcnorm_fwd_{bf16,f16} stores it
+// (kernels/mamba3_ops.cu:1193-1230): the rows are read by every head's workgroup for every chunk, and at 16 bits they are
+// half the cache lines.  The per-head bias and the rotation happen where the tiles are built.  A wave per row, a lane per
+// coordinate.
+template <typename T>
+__global__ __launch_bounds__(256) void m3_bcn_rows_kernel(T *__restrict__ out, const float *__restrict__ bc, int64_t ldbc,
                                                           const float *__restrict__ bnw, const float *__restrict__ cnw, int64_t rows, float eps) {
     constexpr int ds = 64;
     const int w = threadIdx.x >> 6, l = threadIdx.x & 63;
@@ -460,8 +464,8 @@ __global__ __launch_bounds__(256) void m3_bcn_rows_kernel(float *__restrict__ ou
 #pragma unroll
     for (int m = 32; m >= 1; m >>= 1) { ssb += __shfl_xor(ssb, m, kWave); ssc += __shfl_xor(ssc, m, kWave); }
     const float ib = 1.0f / sqrtf(ssb / (float)ds + eps), ic = 1.0f / sqrtf(ssc / (float)ds + eps);
-    out[r * (2 * ds) + l] = b * ib * bnw[l];
-    out[r * (2 * ds) + ds + l] = c * ic * cnw[l];
+    Store<T>::st(out + r * (2 * ds) + l, b * ib * bnw[l]);
+    Store<T>::st(out + r * (2 * ds) + ds + l, c * ic * cnw[l]);
 }
 
 // gated[row, i] = y * silu(z), or RMSNormGated over each head first; z = the first d_inner elements of the bulk row.
@@ -546,7 +550,7 @@ struct mrs_m3_backbone {
     float *pf_in, *pf_residual, *pf_proj, *pf_dt, *pf_a, *pf_trap, *pf_tanhpi, *pf_angle, *pf_angle_snap;
     float *pf_dtT, *pf_aT, *pf_trapT;   // [batch, nh, T] copies of dt, a, trap for the scan that forms K and Q itself
     double *pf_angle_sums;   // [batch][kAngleSegs][nh * n_rope] per-segment angle increments of the prefill
-    float *pf_bcn;           // [rows][2 * d_state] normalised and weighted B | C rows for the scan that forms K and Q itself
+    void *pf_bcn;            // [rows][2 * d_state] normalised and weighted B | C rows (activation type) for the scan that forms K and Q itself
     void *pf_normed, *pf_bulk, *pf_x, *pf_K, *pf_Q, *pf_y, *pf_gated, *pf_out, *pf_ws;
     size_t pf_ws_bytes;
 };
@@ -879,7 +883,7 @@ static int alloc_prefill_scratch3(mrs_m3_backbone *bb, int T) {
     MRS_TRY(dev_alloc3(bb, (void **)&bb->pf_angle, rows * nh * nrz * 4));
     MRS_TRY(dev_alloc3(bb, (void **)&bb->pf_angle_sums, (size_t)bb->batch * kAngleSegs * nh * nrz * sizeof(double)));
     MRS_TRY(dev_alloc3(bb, (void **)&bb->pf_angle_snap, (size_t)bb->batch * nh * nrz * 4));
-    MRS_TRY(dev_alloc3(bb, (void **)&bb->pf_bcn, rows * 2 * ds * 4));
+    MRS_TRY(dev_alloc3(bb, &bb->pf_bcn, rows * 2 * ds * es));
     MRS_TRY(dev_alloc3(bb, &bb->pf_normed, rows * dm * es));
     MRS_TRY(dev_alloc3(bb, &bb->pf_x, rows * di * es));
     MRS_TRY(dev_alloc3(bb, &bb->pf_K, rows * nh * ds * es));
@@ -1020,10 +1024,10 @@ int prefill_body3(mrs_m3_backbone *bb, int T) {
             MRS_TRY(check_launch("m3_angle_apply_kernel"));
         }
         if (fused_kq) {
-            hipLaunchKernelGGL(m3_bcn_rows_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, bb->stream, bb->pf_bcn, bcp, lds_, lw.bnw, lw.cnw,
-                               rows, c.rms_norm_eps);
+            MRS_DISPATCH_DTYPE(dt, T_, hipLaunchKernelGGL(m3_bcn_rows_kernel<T_>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, bb->stream,
+                                                          (T_ *)bb->pf_bcn, bcp, lds_, lw.bnw, lw.cnw, rows, c.rms_norm_eps));
             MRS_TRY(check_launch("m3_bcn_rows_kernel"));
-            const SsdGenArgs gen = {bb->pf_bcn, bb->pf_bcn + ds, 2 * (int64_t)ds, bb->pf_angle, lw.b_bias, lw.c_bias, nr, head_major ? 1 : 0};
+            const SsdGenArgs gen = {bb->pf_bcn, (const char *)bb->pf_bcn + (size_t)ds * es, 2 * (int64_t)ds, bb->pf_angle, lw.b_bias, lw.c_bias, nr, head_major ? 1 : 0};
             const char *xb = (const char *)bulk + (size_t)di * es;
             MRS_TRY(m3_ssd_fwd_ex(bb->stream, dt, ssm, kst, vst, bb->pf_y, xb, ldb, nullptr, nullptr, head_major ? bb->pf_dtT : bb->pf_dt,
                                   head_major ? bb->pf_trapT : bb->pf_trap, head_major ? bb->pf_aT : bb->pf_a, lw.D,

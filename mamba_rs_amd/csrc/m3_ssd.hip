@@ -103,9 +103,10 @@ struct SsdSplit {
     // engine-only extra: x rows may sit inside wider rows (read in place from a projection)
     int64_t x_stride;     // elements between consecutive rows of x (d_inner for a dense x)
     // engine-only extra: K and Q formed inside the kernel (GEN), K = rot(angle, bn + b_bias[h]), Q = rot(angle, cn + c_bias[h]);
-    // bn / cn: the normalised and weighted B / C rows, f32, g_bcs floats apart; angle [batch, T, nh, g_nr]; the first g_nr
-    // pairs of a row are rotated (g_nr a multiple of 4)
-    const float *g_bn, *g_cn, *g_ang, *g_bb, *g_cb;
+    // bn / cn: the normalised and weighted B / C rows in the storage type, g_bcs elements apart; angle [batch, T, nh, g_nr];
+    // the first g_nr pairs of a row are rotated (g_nr a multiple of 4)
+    const void *g_bn, *g_cn;
+    const float *g_ang, *g_bb, *g_cb;
     int64_t g_bcs;
     int g_nr;
     int g_groups;         // batch rows x super-chunks of the launch (set per launch)
@@ -208,8 +209,8 @@ __global__ __launch_bounds__(HD * 4) __attribute__((amdgpu_waves_per_eu(HD == 64
 
     // ---- global -> register prefetch of one chunk ----
     struct Pre {
-        // plain: the Q / K vectors of the thread; GEN: two f32 vectors of cn / bn for each of them, and the 4 angles
-        uint4 rq[NV * (GEN ? 2 : 1)], rk[NV * (GEN ? 2 : 1)], rang[GEN ? NV : 1], rx[2];
+        // the Q / K vectors of the thread (GEN: of the rows they are formed from, and the 4 angles of their pairs)
+        uint4 rq[NV], rk[NV], rang[GEN ? NV : 1], rx[2];
         float rdt, rtr, ra, rdtn, rtrn;   // wave 0 only.  lane = step: dt, trap, a of the step; dt, trap of the step after the chunk (every lane the same)
     };
     const unsigned es = (unsigned)sizeof(T);
@@ -236,8 +237,8 @@ __global__ __launch_bounds__(HD * 4) __attribute__((amdgpu_waves_per_eu(HD == 64
     // GEN: the same (row, 8 columns) items read bn / cn (f32) and the 4 angles of their pairs instead of K / Q
     const int g_col = (tid % VPR) * 8;             // the thread's columns, the same for each of its vectors
     const bool g_rot = g_col < 2 * sp.g_nr;        // its pairs are rotated (all four or none: g_nr is a multiple of 4)
-    const __amdgpu_buffer_rsrc_t bnbuf = slab_rsrc(GEN ? sp.g_bn + (int64_t)b * Tlen * sp.g_bcs : nullptr, GEN ? (int64_t)Tlen * sp.g_bcs * 4 : 0);
-    const __amdgpu_buffer_rsrc_t cnbuf = slab_rsrc(GEN ? sp.g_cn + (int64_t)b * Tlen * sp.g_bcs : nullptr, GEN ? (int64_t)Tlen * sp.g_bcs * 4 : 0);
+    const __amdgpu_buffer_rsrc_t bnbuf = slab_rsrc(GEN ? (const T *)sp.g_bn + (int64_t)b * Tlen * sp.g_bcs : nullptr, GEN ? (int64_t)Tlen * sp.g_bcs * es : 0);
+    const __amdgpu_buffer_rsrc_t cnbuf = slab_rsrc(GEN ? (const T *)sp.g_cn + (int64_t)b * Tlen * sp.g_bcs : nullptr, GEN ? (int64_t)Tlen * sp.g_bcs * es : 0);
     const int ang_step = hm ? sp.g_nr : nh * sp.g_nr;   // floats between the angle rows of consecutive steps
     const __amdgpu_buffer_rsrc_t angbuf =
         slab_rsrc(GEN ? sp.g_ang + (hm ? ((int64_t)b * nh + h) * Tlen : (int64_t)b * Tlen * nh + h) * sp.g_nr : nullptr,
@@ -246,7 +247,7 @@ __global__ __launch_bounds__(HD * 4) __attribute__((amdgpu_waves_per_eu(HD == 64
 #pragma unroll
     for (int v = 0; v < NV; v++) {
         const int vi = tid + v * NTHR, row = vi / VPR;
-        bc_voff[v] = GEN && vi < NVEC ? (unsigned)(row * (int)sp.g_bcs + g_col) * 4u : 0u;
+        bc_voff[v] = GEN && vi < NVEC ? (unsigned)(row * (int)sp.g_bcs + g_col) * es : 0u;
         ang_voff[v] = GEN && vi < NVEC && g_rot ? (unsigned)(row * ang_step + g_col / 2) * 4u : 0u;
     }
     if (GEN) {   // visible to every wave after the barrier at the top of the first chunk
@@ -284,15 +285,11 @@ __global__ __launch_bounds__(HD * 4) __attribute__((amdgpu_waves_per_eu(HD == 64
             r.rtrn = slab_ldf(trbuf, sc_c + (unsigned)(kCS * sc_step) * 4u, 0);
         }
         if constexpr (GEN) {
-            const unsigned bc_c = (unsigned)t0 * (unsigned)sp.g_bcs * 4u, ang_c = (unsigned)t0 * (unsigned)ang_step * 4u;
+            const unsigned bc_c = (unsigned)t0 * (unsigned)sp.g_bcs * es, ang_c = (unsigned)t0 * (unsigned)ang_step * 4u;
 #pragma unroll
             for (int v = 0; v < NV; v++) {
-                if (!STATE_ONLY) {
-                    r.rq[2 * v] = slab_ld128(cnbuf, bc_voff[v] + bc_c, 0);
-                    r.rq[2 * v + 1] = slab_ld128(cnbuf, bc_voff[v] + bc_c + 16u, 0);
-                }
-                r.rk[2 * v] = slab_ld128(bnbuf, bc_voff[v] + bc_c, 0);
-                r.rk[2 * v + 1] = slab_ld128(bnbuf, bc_voff[v] + bc_c + 16u, 0);
+                if (!STATE_ONLY) r.rq[v] = slab_ld128(cnbuf, bc_voff[v] + bc_c, 0);
+                r.rk[v] = slab_ld128(bnbuf, bc_voff[v] + bc_c, 0);
                 r.rang[v] = slab_ld128(angbuf, ang_voff[v] + ang_c, 0);   // lanes without rotated pairs: some angle, not used
             }
         } else {
@@ -334,10 +331,12 @@ __global__ __launch_bounds__(HD * 4) __attribute__((amdgpu_waves_per_eu(HD == 64
                 float sn[4], cs[4];
 #pragma unroll
                 for (int pr = 0; pr < 4; pr++) { sn[pr] = __sinf(ang[pr]); cs[pr] = __cosf(ang[pr]); }
-                auto form = [&](const uint4 &lo, const uint4 &hi, const float *bias) {
+                auto form = [&](const uint4 &raw, const float *bias) {
                     const float4 b0 = *reinterpret_cast<const float4 *>(bias + col), b1 = *reinterpret_cast<const float4 *>(bias + col + 4);
-                    const float4 v0 = __builtin_bit_cast(float4, lo), v1 = __builtin_bit_cast(float4, hi);
-                    const float k[8] = {v0.x + b0.x, v0.y + b0.y, v0.z + b0.z, v0.w + b0.w, v1.x + b1.x, v1.y + b1.y, v1.z + b1.z, v1.w + b1.w};
+                    float v0[4], v1[4];
+                    Mma<T>::unpack(make_uint2(raw.x, raw.y), v0);
+                    Mma<T>::unpack(make_uint2(raw.z, raw.w), v1);
+                    const float k[8] = {v0[0] + b0.x, v0[1] + b0.y, v0[2] + b0.z, v0[3] + b0.w, v1[0] + b1.x, v1[1] + b1.y, v1[2] + b1.z, v1[3] + b1.w};
                     float o[8];
 #pragma unroll
                     for (int pr = 0; pr < 4; pr++) {
@@ -347,8 +346,8 @@ __global__ __launch_bounds__(HD * 4) __attribute__((amdgpu_waves_per_eu(HD == 64
                     const uint2 p0 = Mma<T>::pack(o[0], o[1], o[2], o[3]), p1 = Mma<T>::pack(o[4], o[5], o[6], o[7]);
                     return make_uint4(p0.x, p0.y, p1.x, p1.y);
                 };
-                if (!STATE_ONLY) *reinterpret_cast<uint4 *>(&sm.Qs[row][col]) = form(r.rq[2 * v], r.rq[2 * v + 1], sm.gb[1]);
-                *reinterpret_cast<uint4 *>(&sm.Ks[row][col]) = form(r.rk[2 * v], r.rk[2 * v + 1], sm.gb[0]);
+                if (!STATE_ONLY) *reinterpret_cast<uint4 *>(&sm.Qs[row][col]) = form(r.rq[v], sm.gb[1]);
+                *reinterpret_cast<uint4 *>(&sm.Ks[row][col]) = form(r.rk[v], sm.gb[0]);
             } else {
                 if (!STATE_ONLY) *reinterpret_cast<uint4 *>(&sm.Qs[row][col]) = r.rq[v];
                 *reinterpret_cast<uint4 *>(&sm.Ks[row][col]) = r.rk[v];
@@ -534,7 +533,8 @@ __global__ __launch_bounds__(HD * 4) __attribute__((amdgpu_waves_per_eu(HD == 64
     if constexpr (GEN) {   // K of the last step, as the tiles above form it (rounded to the storage type like a K read from memory)
         for (int n = tid; n < DS; n += NTHR) {
             const int j = n >> 1;
-            const float k0 = sp.g_bn[last * sp.g_bcs + 2 * j] + sp.g_bb[h * DS + 2 * j], k1 = sp.g_bn[last * sp.g_bcs + 2 * j + 1] + sp.g_bb[h * DS + 2 * j + 1];
+            const T *bnl = (const T *)sp.g_bn + last * sp.g_bcs;
+            const float k0 = Store<T>::ld(bnl + 2 * j) + sp.g_bb[h * DS + 2 * j], k1 = Store<T>::ld(bnl + 2 * j + 1) + sp.g_bb[h * DS + 2 * j + 1];
             const float a = j < sp.g_nr ? sp.g_ang[(hm ? ((int64_t)b * nh + h) * Tlen + (Tlen - 1) : last * nh + h) * sp.g_nr + j] : 0.f;
             const float sn = __sinf(a), cs = __cosf(a);
             const T kv = (T)((n & 1) ? sn * k0 + cs * k1 : cs * k0 - sn * k1);
@@ -671,7 +671,7 @@ int mrs::m3_ssd_fwd_ex(void *stream, int dtype, float *ssm_state, float *k_state
                        unsigned flags, int batch, int T, int nheads, int headdim, int d_state, int chunk_size, const SsdGenArgs *gen) {
     const char *fn = "mrs_m3_ssd_fwd";
     if (gen) {   // K and Q formed inside the kernel: K and Q themselves are not read
-        if (dtype == MRS_F32 || headdim != 64 || d_state != 64 || gen->n_rope % 4 != 0 || 2 * gen->n_rope > d_state || gen->bc_stride % 4 != 0 ||
+        if (dtype == MRS_F32 || headdim != 64 || d_state != 64 || gen->n_rope % 4 != 0 || 2 * gen->n_rope > d_state || gen->bc_stride % 8 != 0 ||
             !gen->bn || !gen->cn || !gen->angle || !gen->b_bias || !gen->c_bias || !aligned(gen->bn, 16) || !aligned(gen->cn, 16) || !aligned(gen->angle, 16))
             return fail(MRS_E_SHAPE, "%s: in-kernel K / Q needs 16-bit storage, headdim = d_state = 64, rope pairs in fours, aligned rows", fn);
         if ((int64_t)T * std::max<int64_t>(gen->bc_stride, (int64_t)nheads * gen->n_rope) * 4 >= 0x7fffffffLL)
