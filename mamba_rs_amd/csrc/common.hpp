@@ -139,7 +139,10 @@ int launch_prenorm_rows(hipStream_t st, int dtype, float *partials, int n_partia
 // head_major: the caller keeps what the kernel reads per (head, step) with the steps of a head next to each other --
 // dt, trap, a_val as [batch, nheads, T] and angle as [batch, nheads, T, n_rope] -- so a chunk's 64 steps are a few whole
 // cache lines instead of a piece of 64 different ones.
-struct SsdGenArgs { const void *bn, *cn; int64_t bc_stride; const float *angle, *b_bias, *c_bias; int n_rope; int head_major; };
+// gate: when not null, y leaves as y * silu(gate) (rows of gate_stride elements in the storage type, the first nheads *
+// headdim of each used) -- the plain SiLU gate of the layer, folded into the store of the output tile.
+struct SsdGenArgs { const void *bn, *cn; int64_t bc_stride; const float *angle, *b_bias, *c_bias; int n_rope; int head_major;
+                    const void *gate; int64_t gate_stride; };
 int m3_ssd_fwd_ex(void *stream, int dtype, float *ssm_state, float *k_state, float *v_state, void *y, const void *x,
                   int64_t x_stride, const void *K, const void *Q, const float *dt, const float *trap, const float *a_val,
                   const float *D, void *workspace, size_t workspace_bytes, unsigned flags, int batch, int T, int nheads,

@@ -111,6 +111,9 @@ struct SsdSplit {
     int g_nr;
     int g_groups;         // batch rows x super-chunks of the launch (set per launch)
     int g_head_major;     // dt, trap, a_val are [batch, nh, T] and the angles [batch, nh, T, g_nr]
+    // engine-only extra: y leaves multiplied by silu(z), z rows g_zs elements apart in the storage type (GATE)
+    const void *g_z;
+    int64_t g_zs;
 };
 
 // Cross-lane moves on the data-parallel-primitive path of the vector ALU (no LDS round trip, unlike the shuffle
@@ -143,7 +146,7 @@ __device__ __forceinline__ float slab_ldf(__amdgpu_buffer_rsrc_t r, unsigned vof
     return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0));
 }
 
-template <typename T, int HD, int DS, bool STATE_ONLY, bool GEN>
+template <typename T, int HD, int DS, bool STATE_ONLY, bool GEN, bool GATE = false>
 __global__ __launch_bounds__(HD * 4) __attribute__((amdgpu_waves_per_eu(HD == 64 ? 3 : 1))) void m3_ssd_kernel(
     float *__restrict__ ssm, float *__restrict__ kst, float *__restrict__ vst, T *__restrict__ y,
     const T *__restrict__ x, const T *__restrict__ K, const T *__restrict__ Q,
@@ -210,7 +213,7 @@ __global__ __launch_bounds__(HD * 4) __attribute__((amdgpu_waves_per_eu(HD == 64
     // ---- global -> register prefetch of one chunk ----
     struct Pre {
         // the Q / K vectors of the thread (GEN: of the rows they are formed from, and the 4 angles of their pairs)
-        uint4 rq[NV], rk[NV], rang[GEN ? NV : 1], rx[2];
+        uint4 rq[NV], rk[NV], rang[GEN ? NV : 1], rx[2], rz[GATE ? 2 : 1];   // rz: the gate rows of the chunk, laid out like x
         float rdt, rtr, ra, rdtn, rtrn;   // wave 0 only.  lane = step: dt, trap, a of the step; dt, trap of the step after the chunk (every lane the same)
     };
     const unsigned es = (unsigned)sizeof(T);
@@ -227,7 +230,7 @@ __global__ __launch_bounds__(HD * 4) __attribute__((amdgpu_waves_per_eu(HD == 64
     const __amdgpu_buffer_rsrc_t dtbuf = slab_rsrc(dt + sc_base, sc_bytes);
     const __amdgpu_buffer_rsrc_t trbuf = slab_rsrc(trap + sc_base, sc_bytes);
     const __amdgpu_buffer_rsrc_t abuf = slab_rsrc(a_val + sc_base, sc_bytes);
-    const __amdgpu_buffer_rsrc_t ybuf = slab_rsrc(y + (int64_t)b * Tlen * di + h * HD + 16 * w, ((int64_t)Tlen * di - h * HD - 16 * w) * es);
+    const __amdgpu_buffer_rsrc_t ybuf = slab_rsrc(y + (int64_t)b * Tlen * di + h * HD, ((int64_t)Tlen * di - h * HD) * es);
     unsigned kq_voff[NV];
 #pragma unroll
     for (int v = 0; v < NV; v++) {
@@ -265,7 +268,14 @@ __global__ __launch_bounds__(HD * 4) __attribute__((amdgpu_waves_per_eu(HD == 64
         x_voff[v] = (unsigned)(x_row[v] * (int)sp.x_stride + x_col[v]) * es;
     }
     const unsigned sc_voff = (unsigned)l * (unsigned)sc_step * 4u;
-    const unsigned y_voff = (unsigned)(4 * lg * di + lr) * es;
+    const __amdgpu_buffer_rsrc_t zbuf = slab_rsrc(GATE ? (const T *)sp.g_z + (int64_t)b * Tlen * sp.g_zs + h * HD : nullptr,
+                                                  GATE ? ((int64_t)Tlen * sp.g_zs - h * HD) * es : 0);
+    unsigned z_voff[2];
+#pragma unroll
+    for (int v = 0; v < 2; v++) z_voff[v] = GATE ? (unsigned)(x_row[v] * (int)sp.g_zs + x_col[v]) * es : 0u;
+    unsigned y_voff[2];   // the y tile leaves like the x tile comes in: whole rows by neighbouring lanes, 16 bytes a lane
+#pragma unroll
+    for (int v = 0; v < 2; v++) y_voff[v] = (unsigned)(x_row[v] * di + x_col[v]) * es;
     // Accesses past the end of the batch row (the tail of a last, partial chunk) fall outside the resources: loads give
     // zero and stores are dropped by the bounds check, which covers the vector offset -- so the chunk's offset goes there.
     auto prefetch = [&](Pre &r, int c) {
@@ -301,6 +311,11 @@ __global__ __launch_bounds__(HD * 4) __attribute__((amdgpu_waves_per_eu(HD == 64
         }
         r.rx[0] = slab_ld128(xbuf, x_voff[0] + x_c, 0);
         r.rx[1] = slab_ld128(xbuf, x_voff[1] + x_c, 0);
+        if constexpr (GATE) {
+            const unsigned z_c = (unsigned)t0 * (unsigned)sp.g_zs * es;
+            r.rz[0] = slab_ld128(zbuf, z_voff[0] + z_c, 0);
+            r.rz[1] = slab_ld128(zbuf, z_voff[1] + z_c, 0);
+        }
     };
 
     // One chunk from the registers of `r`; once they are in LDS the chunk c_next is requested into them.
@@ -355,6 +370,8 @@ __global__ __launch_bounds__(HD * 4) __attribute__((amdgpu_waves_per_eu(HD == 64
         }
         *reinterpret_cast<uint4 *>(&sm.Xs[x_row[0]][x_col[0]]) = r.rx[0];
         *reinterpret_cast<uint4 *>(&sm.Xs[x_row[1]][x_col[1]]) = r.rx[1];
+        uint4 zc[GATE ? 2 : 1];   // this chunk's gate rows: the registers of `r` take the next chunk's below
+        if constexpr (GATE) { zc[0] = r.rz[0]; zc[1] = r.rz[1]; }
         // ---- per-step scalars, lane = step (wave 0) ----
         if (w == 0) {
             // dt, trap of the step after this one: the next lane's, and for the last lane the step after the chunk
@@ -457,12 +474,32 @@ __global__ __launch_bounds__(HD * 4) __attribute__((amdgpu_waves_per_eu(HD == 64
                 }
 #pragma unroll
                 for (int js = 0; js <= it; js++) acc = Mma<T>::mma(sm.Ps[it * (it + 1) / 2 + js][l], xf[js], acc);
-                // store y rows t = t0+16it+4lg+i, column p = 16w+lr
+                // y rows t = 16it+4lg+i, column p = 16w+lr into the tile that held x (its fragments are in registers since
+                // the second barrier): a lane's four values are 2 bytes each in four different rows, and stored to memory
+                // like that they were 32-byte pieces, sixteen instructions a wave
 #pragma unroll
-                for (int i = 0; i < 4; i++) {   // rows past the sequence are dropped by the bounds check
+                for (int i = 0; i < 4; i++) {
                     const T yv = (T)acc[i];
-                    __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(uint16_t, yv), ybuf, y_voff + (unsigned)(t0 + 16 * it + i) * (unsigned)di * es, 0, 0);
+                    sm.Xs[16 * it + 4 * lg + i][16 * w + lr] = __builtin_bit_cast(uint16_t, yv);
                 }
+            }
+            lds_barrier();  // the y tile is complete
+#pragma unroll
+            for (int v = 0; v < 2; v++) {   // rows past the sequence are dropped by the bounds check
+                uint4 yv = *reinterpret_cast<const uint4 *>(&sm.Xs[x_row[v]][x_col[v]]);
+                if constexpr (GATE) {   // y * silu(z), rounded like the separate gate pass rounds it (y to the storage type first)
+                    float yf[8], zf[8];
+                    Mma<T>::unpack(make_uint2(yv.x, yv.y), *reinterpret_cast<float(*)[4]>(yf));
+                    Mma<T>::unpack(make_uint2(yv.z, yv.w), *reinterpret_cast<float(*)[4]>(yf + 4));
+                    Mma<T>::unpack(make_uint2(zc[v].x, zc[v].y), *reinterpret_cast<float(*)[4]>(zf));
+                    Mma<T>::unpack(make_uint2(zc[v].z, zc[v].w), *reinterpret_cast<float(*)[4]>(zf + 4));
+#pragma unroll
+                    for (int e = 0; e < 8; e++) yf[e] *= silu(zf[e]);
+                    const uint2 lo = Mma<T>::pack(yf[0], yf[1], yf[2], yf[3]), hi = Mma<T>::pack(yf[4], yf[5], yf[6], yf[7]);
+                    yv = make_uint4(lo.x, lo.y, hi.x, hi.y);
+                }
+                typedef unsigned v4u __attribute__((ext_vector_type(4)));
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, yv), ybuf, y_voff[v] + (unsigned)t0 * (unsigned)di * es, 0, 0);
             }
         }
     };
@@ -601,8 +638,12 @@ static void launch_ssd_shape(hipStream_t st, float *ssm, float *kst, float *vst,
                                    ssm, kst, vst, (T *)y, (const T *)x, (const T *)K, (const T *)Q, dt, trap, a_val, D, sp, Tlen, nh, carry);
             }
             sp.g_groups = batch * sp.nsc;
-            hipLaunchKernelGGL((m3_ssd_kernel<T, HD, DS, false, true>), padded(sp.g_groups), dim3(HD * 4), 0, st, ssm, kst, vst,
-                               (T *)y, (const T *)x, (const T *)K, (const T *)Q, dt, trap, a_val, D, sp, Tlen, nh, carry);
+            if (sp.g_z)
+                hipLaunchKernelGGL((m3_ssd_kernel<T, HD, DS, false, true, true>), padded(sp.g_groups), dim3(HD * 4), 0, st, ssm, kst, vst,
+                                   (T *)y, (const T *)x, (const T *)K, (const T *)Q, dt, trap, a_val, D, sp, Tlen, nh, carry);
+            else
+                hipLaunchKernelGGL((m3_ssd_kernel<T, HD, DS, false, true>), padded(sp.g_groups), dim3(HD * 4), 0, st, ssm, kst, vst,
+                                   (T *)y, (const T *)x, (const T *)K, (const T *)Q, dt, trap, a_val, D, sp, Tlen, nh, carry);
             return;
         }
     }
@@ -672,7 +713,8 @@ int mrs::m3_ssd_fwd_ex(void *stream, int dtype, float *ssm_state, float *k_state
     const char *fn = "mrs_m3_ssd_fwd";
     if (gen) {   // K and Q formed inside the kernel: K and Q themselves are not read
         if (dtype == MRS_F32 || headdim != 64 || d_state != 64 || gen->n_rope % 4 != 0 || 2 * gen->n_rope > d_state || gen->bc_stride % 8 != 0 ||
-            !gen->bn || !gen->cn || !gen->angle || !gen->b_bias || !gen->c_bias || !aligned(gen->bn, 16) || !aligned(gen->cn, 16) || !aligned(gen->angle, 16))
+            !gen->bn || !gen->cn || !gen->angle || !gen->b_bias || !gen->c_bias || !aligned(gen->bn, 16) || !aligned(gen->cn, 16) || !aligned(gen->angle, 16) ||
+            (gen->gate && (!aligned(gen->gate, 16) || gen->gate_stride % 8 != 0 || (int64_t)T * gen->gate_stride * 2 >= 0x7fffffffLL)))
             return fail(MRS_E_SHAPE, "%s: in-kernel K / Q needs 16-bit storage, headdim = d_state = 64, rope pairs in fours, aligned rows", fn);
         if ((int64_t)T * std::max<int64_t>(gen->bc_stride, (int64_t)nheads * gen->n_rope) * 4 >= 0x7fffffffLL)
             return fail(MRS_E_SHAPE, "%s: one batch row of the B / C rows or the angles exceeds 2^31 bytes", fn);
@@ -715,12 +757,12 @@ int mrs::m3_ssd_fwd_ex(void *stream, int dtype, float *ssm_state, float *k_state
         }
         return mrs_m3_seq_fwd(stream, dtype, ssm_state, k_state, v_state, y, x, K, Q, al, be, ga, D, batch, T, nheads, headdim, d_state);
     }
-    if (!aligned(x, 16) || !aligned(K, 16) || !aligned(Q, 16) || !aligned(ssm_state, 16) || !aligned(k_state, 16))
-        return fail(MRS_E_ALIGN, "%s: x, K, Q, ssm_state, k_state must be 16-byte aligned", fn);
+    if (!aligned(x, 16) || !aligned(y, 16) || !aligned(K, 16) || !aligned(Q, 16) || !aligned(ssm_state, 16) || !aligned(k_state, 16))
+        return fail(MRS_E_ALIGN, "%s: x, y, K, Q, ssm_state, k_state must be 16-byte aligned", fn);
     // Super-chunk split when the caller's workspace holds it; otherwise one workgroup walks the whole sequence.
-    SsdSplit sp = {nullptr, nullptr, nullptr, 1, (T + kCS - 1) / kCS, x_stride, nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0, 0, 0};
+    SsdSplit sp = {nullptr, nullptr, nullptr, 1, (T + kCS - 1) / kCS, x_stride, nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0, 0, 0, nullptr, 0};
     auto with_gen = [&](SsdSplit &o) {
-        if (gen) { o.g_bn = gen->bn; o.g_cn = gen->cn; o.g_ang = gen->angle; o.g_bb = gen->b_bias; o.g_cb = gen->c_bias; o.g_bcs = gen->bc_stride; o.g_nr = gen->n_rope; o.g_head_major = gen->head_major; }
+        if (gen) { o.g_bn = gen->bn; o.g_cn = gen->cn; o.g_ang = gen->angle; o.g_bb = gen->b_bias; o.g_cb = gen->c_bias; o.g_bcs = gen->bc_stride; o.g_nr = gen->n_rope; o.g_head_major = gen->head_major; o.g_z = gen->gate; o.g_zs = gen->gate_stride; }
     };
     with_gen(sp);
     {
@@ -730,7 +772,7 @@ int mrs::m3_ssd_fwd_ex(void *stream, int dtype, float *ssm_state, float *k_state
         const size_t need = ssd_split_bytes(batch, nheads, headdim, d_state, nsc, &o_dA, &o_init);
         if (nsc > 1 && workspace && workspace_bytes >= need && aligned(workspace, 16)) {
             char *ws = (char *)workspace;
-            sp = SsdSplit{(float *)ws, (float *)(ws + o_dA), (float *)(ws + o_init), nsc, cps, x_stride, nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0, 0, 0};
+            sp = SsdSplit{(float *)ws, (float *)(ws + o_dA), (float *)(ws + o_init), nsc, cps, x_stride, nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0, 0, 0, nullptr, 0};
             with_gen(sp);
         }
     }
