@@ -168,11 +168,19 @@ constexpr int kAngleSegs = 64;
 // One workgroup per 64 consecutive rows, a thread per (row, j) with j fastest: j < nh -> the head scalars, j >= nh -> rope
 // pair j - nh.  When the scan wants its per-head inputs with the steps of a head next to each other (dtT, aT, trapT:
 // [batch, nh, T]) the tile is turned in LDS, so those stores are 256-byte runs as well.
+// bcn_out (optional, one group at d_state 64): the normalised and weighted B | C rows for the scan that forms K and Q
+// itself -- out[row] = [B * rsqrt(mean(B^2) + eps) * bnw | C * rsqrt(mean(C^2) + eps) * cnw] (bcnorm_fwd, ops/norms.rs:50-80),
+// formed in f32 from the f32 projection and stored in the activation type, as the reference's bcnorm_fwd_{bf16,f16} stores
+// them (kernels/mamba3_ops.cu:1193-1230): every head's workgroup reads these rows for every chunk, and at 16 bits they are
+// half the cache lines.  A wave per row, a lane per coordinate; the per-head bias and the rotation happen where the tiles
+// are built.  (As a launch of its own this took 5.4 us, nearly all of it the fixed cost of a launch.)
+template <typename T>
 __global__ __launch_bounds__(1024) void m3_scalars_kernel(float *__restrict__ dt_out, float *__restrict__ a_out, float *__restrict__ trap_out,
                                                          float *__restrict__ tanhpi_out, float *__restrict__ dtT, float *__restrict__ aT,
                                                          float *__restrict__ trapT, const float *__restrict__ proj, int64_t ip,
                                                          const float *__restrict__ dt_bias, int64_t rows, int Tlen, int nh, int nr, int sc_off,
-                                                         float a_floor) {
+                                                         float a_floor, T *__restrict__ bcn_out, const float *__restrict__ bc, int64_t ldbc,
+                                                         const float *__restrict__ bnw, const float *__restrict__ cnw, float eps) {
     extern __shared__ float turned[];   // [3][nh][65]
     const int64_t r0 = (int64_t)blockIdx.x * 64;
     const int per = nh + nr;
@@ -195,6 +203,21 @@ __global__ __launch_bounds__(1024) void m3_scalars_kernel(float *__restrict__ dt
             }
         } else {
             tanhpi_out[r * nr + (j - nh)] = tanhf(sc[3 * nh + (j - nh)]) * kPi;
+        }
+    }
+    if (bcn_out) {
+        constexpr int ds = 64;
+        const int w = threadIdx.x >> 6, l = threadIdx.x & 63, nw = (int)blockDim.x >> 6;
+        for (int rl = w; rl < 64; rl += nw) {
+            const int64_t r = r0 + rl;
+            if (r >= rows) break;   // whole waves
+            const float b = bc[r * ldbc + l], c = bc[r * ldbc + ds + l];
+            float ssb = b * b, ssc = c * c;
+#pragma unroll
+            for (int m = 32; m >= 1; m >>= 1) { ssb += __shfl_xor(ssb, m, kWave); ssc += __shfl_xor(ssc, m, kWave); }
+            const float ib = 1.0f / sqrtf(ssb / (float)ds + eps), ic = 1.0f / sqrtf(ssc / (float)ds + eps);
+            Store<T>::st(bcn_out + r * (2 * ds) + l, b * ib * bnw[l]);
+            Store<T>::st(bcn_out + r * (2 * ds) + ds + l, c * ic * cnw[l]);
         }
     }
     if (!dtT) return;
@@ -444,28 +467,6 @@ __global__ __launch_bounds__(256) void m3_kq_rows_kernel(
     }
     if (xout)
         for (int i = l; i < di; i += 64) xout[r * di + i] = row[di + i];
-}
-
-// The part of K and Q that all heads share, for the scan kernel that forms K and Q itself (one group, d_state 64):
-// out[row] = [B * rsqrt(mean(B^2) + eps) * bnw | C * rsqrt(mean(C^2) + eps) * cnw] (bcnorm_fwd, ops/norms.rs:50-80), formed in
-// f32 from the f32 projection and stored in the activation type, as the reference's bcnorm_fwd_{bf16,f16} stores it
-// (kernels/mamba3_ops.cu:1193-1230): the rows are read by every head's workgroup for every chunk, and at 16 bits they are
-// half the cache lines.  The per-head bias and the rotation happen where the tiles are built.  A wave per row, a lane per
-// coordinate.
-template <typename T>
-__global__ __launch_bounds__(256) void m3_bcn_rows_kernel(T *__restrict__ out, const float *__restrict__ bc, int64_t ldbc,
-                                                          const float *__restrict__ bnw, const float *__restrict__ cnw, int64_t rows, float eps) {
-    constexpr int ds = 64;
-    const int w = threadIdx.x >> 6, l = threadIdx.x & 63;
-    const int64_t r = (int64_t)blockIdx.x * 4 + w;
-    if (r >= rows) return;   // whole waves leave; the kernel has no barrier
-    const float b = bc[r * ldbc + l], c = bc[r * ldbc + ds + l];
-    float ssb = b * b, ssc = c * c;
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) { ssb += __shfl_xor(ssb, m, kWave); ssc += __shfl_xor(ssc, m, kWave); }
-    const float ib = 1.0f / sqrtf(ssb / (float)ds + eps), ic = 1.0f / sqrtf(ssc / (float)ds + eps);
-    Store<T>::st(out + r * (2 * ds) + l, b * ib * bnw[l]);
-    Store<T>::st(out + r * (2 * ds) + ds + l, c * ic * cnw[l]);
 }
 
 // gated = y * silu(z) as a plain stream: a thread owns 16 bytes (8 values of 16-bit storage) of four consecutive rows and
@@ -1047,9 +1048,11 @@ int prefill_body3(mrs_m3_backbone *bb, int T) {
         const size_t turned_bytes = (size_t)3 * nh * 65 * sizeof(float);
         const bool head_major = fused_kq && turned_bytes <= 48 * 1024;
         {
-            hipLaunchKernelGGL(m3_scalars_kernel, dim3((unsigned)((rows + 63) / 64)), dim3(1024), head_major ? turned_bytes : 0, bb->stream,
-                               bb->pf_dt, bb->pf_a, bb->pf_trap, bb->pf_tanhpi, head_major ? bb->pf_dtT : nullptr, bb->pf_aT, bb->pf_trapT, scp,
-                               lds_, lw.dt_bias, rows, T, nh, nr, 0, c.a_floor);
+            MRS_DISPATCH_DTYPE(dt, T_, hipLaunchKernelGGL(m3_scalars_kernel<T_>, dim3((unsigned)((rows + 63) / 64)), dim3(1024),
+                                                          head_major ? turned_bytes : 0, bb->stream, bb->pf_dt, bb->pf_a, bb->pf_trap, bb->pf_tanhpi,
+                                                          head_major ? bb->pf_dtT : nullptr, bb->pf_aT, bb->pf_trapT, scp, lds_, lw.dt_bias, rows, T, nh,
+                                                          nr, 0, c.a_floor, fused_kq ? (T_ *)bb->pf_bcn : nullptr, bcp, lds_, lw.bnw, lw.cnw,
+                                                          c.rms_norm_eps));
             MRS_TRY(check_launch("m3_scalars_kernel"));
         }
         if (nr > 0) {
@@ -1064,9 +1067,6 @@ int prefill_body3(mrs_m3_backbone *bb, int T) {
         }
         bool gate_in_scan = false;
         if (fused_kq) {
-            MRS_DISPATCH_DTYPE(dt, T_, hipLaunchKernelGGL(m3_bcn_rows_kernel<T_>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, bb->stream,
-                                                          (T_ *)bb->pf_bcn, bcp, lds_, lw.bnw, lw.cnw, rows, c.rms_norm_eps));
-            MRS_TRY(check_launch("m3_bcn_rows_kernel"));
             // the plain SiLU gate rides on the scan's output store (z = the first d_inner elements of the bulk rows): no gate
             // pass, and y itself is never written
             gate_in_scan = !c.is_outproj_norm && ldb % 8 == 0;
