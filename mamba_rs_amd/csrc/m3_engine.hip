@@ -165,15 +165,18 @@ __global__ __launch_bounds__(1024) void m3_layer_step_kernel(
 // before its own, so more segments mean more reads: at batch 4 x 4096 the two launches took 35 us with 32 segments,
 // 25 us with 64, 30 us with 128.
 constexpr int kAngleSegs = 64;
-// One workgroup per 64 consecutive rows, a thread per (row, j) with j fastest: j < nh -> the head scalars, j >= nh -> rope
+// One workgroup per kScalarRows consecutive rows, a thread per (row, j) with j fastest: j < nh -> the head scalars, j >= nh -> rope
 // pair j - nh.  When the scan wants its per-head inputs with the steps of a head next to each other (dtT, aT, trapT:
-// [batch, nh, T]) the tile is turned in LDS, so those stores are 256-byte runs as well.
+// [batch, nh, T]) the tile is turned in LDS, so those stores are runs of kScalarRows floats.  Few rows per workgroup: every
+// phase is then a single trip with all of its loads in flight at once (64 rows per workgroup, two to five dependent trips
+// per phase: 13.9 us; the work itself is a few microseconds).
 // bcn_out (optional, one group at d_state 64): the normalised and weighted B | C rows for the scan that forms K and Q
 // itself -- out[row] = [B * rsqrt(mean(B^2) + eps) * bnw | C * rsqrt(mean(C^2) + eps) * cnw] (bcnorm_fwd, ops/norms.rs:50-80),
 // formed in f32 from the f32 projection and stored in the activation type, as the reference's bcnorm_fwd_{bf16,f16} stores
 // them (kernels/mamba3_ops.cu:1193-1230): every head's workgroup reads these rows for every chunk, and at 16 bits they are
 // half the cache lines.  A wave per row, a lane per coordinate; the per-head bias and the rotation happen where the tiles
 // are built.  (As a launch of its own this took 5.4 us, nearly all of it the fixed cost of a launch.)
+constexpr int kScalarRows = 16;
 template <typename T>
 __global__ __launch_bounds__(1024) void m3_scalars_kernel(float *__restrict__ dt_out, float *__restrict__ a_out, float *__restrict__ trap_out,
                                                          float *__restrict__ tanhpi_out, float *__restrict__ dtT, float *__restrict__ aT,
@@ -181,10 +184,11 @@ __global__ __launch_bounds__(1024) void m3_scalars_kernel(float *__restrict__ dt
                                                          const float *__restrict__ dt_bias, int64_t rows, int Tlen, int nh, int nr, int sc_off,
                                                          float a_floor, T *__restrict__ bcn_out, const float *__restrict__ bc, int64_t ldbc,
                                                          const float *__restrict__ bnw, const float *__restrict__ cnw, float eps) {
-    extern __shared__ float turned[];   // [3][nh][65]
-    const int64_t r0 = (int64_t)blockIdx.x * 64;
+    extern __shared__ float turned[];   // [3][nh][kScalarRows + 1]
+    constexpr int R = kScalarRows;
+    const int64_t r0 = (int64_t)blockIdx.x * R;
     const int per = nh + nr;
-    for (int i = threadIdx.x; i < 64 * per; i += (int)blockDim.x) {
+    for (int i = threadIdx.x; i < R * per; i += (int)blockDim.x) {
         const int rl = i / per, j = i - rl * per;
         const int64_t r = r0 + rl;
         if (r >= rows) continue;
@@ -197,9 +201,9 @@ __global__ __launch_bounds__(1024) void m3_scalars_kernel(float *__restrict__ dt
             a_out[r * nh + j] = a;
             trap_out[r * nh + j] = tr;
             if (dtT) {
-                turned[(0 * nh + j) * 65 + rl] = d;
-                turned[(1 * nh + j) * 65 + rl] = a;
-                turned[(2 * nh + j) * 65 + rl] = tr;
+                turned[(0 * nh + j) * (R + 1) + rl] = d;
+                turned[(1 * nh + j) * (R + 1) + rl] = a;
+                turned[(2 * nh + j) * (R + 1) + rl] = tr;
             }
         } else {
             tanhpi_out[r * nr + (j - nh)] = tanhf(sc[3 * nh + (j - nh)]) * kPi;
@@ -208,7 +212,7 @@ __global__ __launch_bounds__(1024) void m3_scalars_kernel(float *__restrict__ dt
     if (bcn_out) {
         constexpr int ds = 64;
         const int w = threadIdx.x >> 6, l = threadIdx.x & 63, nw = (int)blockDim.x >> 6;
-        for (int rl = w; rl < 64; rl += nw) {
+        for (int rl = w; rl < R; rl += nw) {
             const int64_t r = r0 + rl;
             if (r >= rows) break;   // whole waves
             const float b = bc[r * ldbc + l], c = bc[r * ldbc + ds + l];
@@ -222,13 +226,13 @@ __global__ __launch_bounds__(1024) void m3_scalars_kernel(float *__restrict__ dt
     }
     if (!dtT) return;
     __syncthreads();
-    for (int i = threadIdx.x; i < 3 * nh * 64; i += (int)blockDim.x) {
-        const int rl = i & 63, hj = i >> 6, arr = hj / nh, h = hj - arr * nh;
+    for (int i = threadIdx.x; i < 3 * nh * R; i += (int)blockDim.x) {
+        const int rl = i % R, hj = i / R, arr = hj / nh, h = hj - arr * nh;
         const int64_t r = r0 + rl;
         if (r >= rows) continue;
         const int64_t b = r / Tlen, t = r - b * Tlen;
         float *dst = arr == 0 ? dtT : (arr == 1 ? aT : trapT);
-        dst[(b * nh + h) * Tlen + t] = turned[hj * 65 + rl];
+        dst[(b * nh + h) * Tlen + t] = turned[hj * (R + 1) + rl];
     }
 }
 
@@ -1045,10 +1049,10 @@ int prefill_body3(mrs_m3_backbone *bb, int T) {
         const bool fused_kq = in_place && hd == 64 && ds == 64 && c.ngroups == 1 && nr > 0 && nr % 4 == 0 && !no_fused_kq;
         // that scan reads a head's step scalars and angles as runs of steps (a chunk's 64 steps of one head are 256
         // bytes instead of 4 bytes in each of 64 rows): the kernels in front of it write them that way
-        const size_t turned_bytes = (size_t)3 * nh * 65 * sizeof(float);
+        const size_t turned_bytes = (size_t)3 * nh * (kScalarRows + 1) * sizeof(float);
         const bool head_major = fused_kq && turned_bytes <= 48 * 1024;
         {
-            MRS_DISPATCH_DTYPE(dt, T_, hipLaunchKernelGGL(m3_scalars_kernel<T_>, dim3((unsigned)((rows + 63) / 64)), dim3(1024),
+            MRS_DISPATCH_DTYPE(dt, T_, hipLaunchKernelGGL(m3_scalars_kernel<T_>, dim3((unsigned)((rows + kScalarRows - 1) / kScalarRows)), dim3(1024),
                                                           head_major ? turned_bytes : 0, bb->stream, bb->pf_dt, bb->pf_a, bb->pf_trap, bb->pf_tanhpi,
                                                           head_major ? bb->pf_dtT : nullptr, bb->pf_aT, bb->pf_trapT, scp, lds_, lw.dt_bias, rows, T, nh,
                                                           nr, 0, c.a_floor, fused_kq ? (T_ *)bb->pf_bcn : nullptr, bcp, lds_, lw.bnw, lw.cnw,
