@@ -75,8 +75,14 @@ __global__ __launch_bounds__(64) void conv1d_seq_silu_stream_kernel(
     // below sit in scalar registers (a per-lane resource makes the compiler loop over its distinct values at every access)
     const int nvec = di / VEC;
     const int nblk = (nvec + (int)blockDim.x - 1) / (int)blockDim.x;
-    const int cvb = blockIdx.x % nblk;
-    const int rest = blockIdx.x / nblk;
+    // Workgroups go to the chip's 8 L2 domains round-robin by index; each domain is given a contiguous eighth of the work
+    // instead, so the chunk that re-reads the d_conv-1 rows before its first step finds them in the L2 that the chunk
+    // before it filled (with neighbouring chunks in different domains those rows came from memory twice: 69.6 MB
+    // fetched for 50.3 MB of x).
+    const unsigned n8 = gridDim.x / 8;
+    const unsigned bid = blockIdx.x < 8 * n8 ? (blockIdx.x & 7) * n8 + (blockIdx.x >> 3) : blockIdx.x;
+    const int cvb = (int)(bid % (unsigned)nblk);
+    const int rest = (int)(bid / (unsigned)nblk);
     const int chunk = rest % nchunk;
     const int b = rest / nchunk;
     const int cv = cvb * (int)blockDim.x + (int)threadIdx.x;
