@@ -86,7 +86,11 @@ MRS_API int mrs_a_neg_is_s4d_real(void *stream, int *flag_out, const float *a_ne
  *   delta,u[batch, T, d_inner]       dtype (delta after softplus)
  *   B, C   [batch, T, d_state]       dtype
  *   a_neg  [d_inner, d_state] f32,  D [d_inner] f32
- * d_state in 1..=256, T >= 1.  Uses no workspace: always the sequential route. */
+ * d_state in 1..=256, T >= 1.  This symbol keeps the reference's argument list, which has no room for a workspace, and
+ * therefore always takes the sequential kernel (one wave per 64 channels of a batch row: about 0.9 ms at
+ * 8 x 2048 x 1536 where the T-split route takes 0.1 ms).  A caller replacing the *parallel* launch site
+ * (src/mamba_ssm/gpu/prefill.rs:910-933) should bind mrs_ssm_scan_fwd_ex (workspace) or mrs_ssm_scan_fwd_static
+ * (none) instead. */
 MRS_API int mrs_ssm_scan_fwd(void *stream, int dtype, float *h, void *y, const void *delta, const void *u,
                      const void *B, const void *C, const float *a_neg, const float *D,
                      int batch, int T, int d_inner, int d_state);
