@@ -204,7 +204,8 @@ MRS_API int mrs_m3_compute_abg(void *stream, float *alpha, float *beta, float *g
  * written back.  MRS_M3_CARRY_STATE continues from the entering state instead (prefill
  * after an earlier window, handing over to mrs_m3_step); the reference has no such mode.
  * chunk_size must be 64; headdim and d_state multiples of 16 with headdim <= 64, d_state <= 64
- * for the matrix-core path -- other shapes are refused (use mrs_m3_seq_fwd). */
+ * for the matrix-core path -- other shapes are refused (use mrs_m3_seq_fwd).  x, y, K, Q, ssm_state and k_state
+ * 16-byte aligned (MRS_E_ALIGN otherwise): tiles are moved as 16-byte row pieces. */
 enum { MRS_M3_CARRY_STATE = 1u << 0 };
 MRS_API size_t mrs_m3_ssd_workspace_bytes(int batch, int T, int nheads, int headdim, int d_state, int chunk_size);
 MRS_API int mrs_m3_ssd_fwd(void *stream, int dtype, float *ssm_state, float *k_state, float *v_state, void *y,

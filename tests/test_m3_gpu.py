@@ -167,3 +167,8 @@ def test_m3_rejects_bad_arguments():
         ops.m3_ssd_fwd(torch.zeros(1, 2, 48, 16, device=DEV), kst, torch.zeros(1, 2, 48, device=DEV), torch.empty_like(x48), x48, K, Q,
                        dev(inp["dt"]), dev(inp["trap"]), dev(inp["a_val"]), dev(inp["D"]))
     assert e.value.code == -2
+    # tiles move as 16-byte row pieces: an output that starts 2 bytes off a 16-byte boundary is refused, not written
+    y_off = torch.empty(x.numel() + 8, device=DEV, dtype=torch.bfloat16)[1:1 + x.numel()].view(x.shape)
+    with pytest.raises(MambaHipError) as e:
+        ops.m3_ssd_fwd(ssm, kst, vst, y_off, x, K, Q, dev(inp["dt"]), dev(inp["trap"]), dev(inp["a_val"]), dev(inp["D"]))
+    assert e.value.code == -5
