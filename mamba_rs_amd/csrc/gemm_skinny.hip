@@ -389,26 +389,41 @@ __global__ __launch_bounds__(256) void prenorm_rows_kernel(float *__restrict__ p
 // while the current tile is in its epilogue, and the transpose through LDS is private to each wave (no workgroup
 // barrier).  Measured at the 130m prefill shape (50 MB of delta per layer): 25.7 us with one tile per workgroup, 22.4 us
 // walking row tiles, 26.5 us walking along the rows instead, 21.2 us with the one-branch softplus20_16.
-template <typename T, int KS>
+// WLDS: the weight fragments live in LDS instead of registers.  From dt_rank 97 up (KS >= 4: the 2.8b shape has dt_rank
+// 160) 16 registers per k-step for them left two waves per SIMD (178 registers at KS = 6) and the op ran at a third of
+// its write rate (102 us for 168 MB); read back from LDS as they are used they cost a 16-byte LDS read per matrix
+// instruction and the kernel keeps four to five waves per SIMD.
+template <typename T, int KS, bool WLDS = (KS >= 4)>
 __global__ __launch_bounds__(256) void dt_proj_softplus_kernel(T *__restrict__ delta, const T *__restrict__ dt_in, int64_t xs,
                                                                const T *__restrict__ wt, const float *__restrict__ bias, int64_t rows,
                                                                int di, int dr) {
     __shared__ alignas(16) T tile[4][16][64 + 8];
+    __shared__ alignas(16) T wlds[WLDS ? 64 : 1][WLDS ? KS * 32 + 8 : 8];   // [column][k], k zero-padded to 32 KS
     const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, lr = l & 15, lg = l >> 4;
     const int n0 = blockIdx.x * 64;
     const int64_t n_tiles = (rows + 63) / 64;
     // weight fragments and bias of this workgroup's 64 columns
-    uint4 bf[KS][4];
+    uint4 bf[WLDS ? 1 : KS][4];
     float bv[4];
 #pragma unroll
     for (int nt = 0; nt < 4; nt++) {
         const int col = min(n0 + 16 * nt + lr, di - 1);
         bv[nt] = bias[col];
+        if constexpr (!WLDS) {
 #pragma unroll
-        for (int ks = 0; ks < KS; ks++) {
-            const int k = 32 * ks + 8 * lg;   // dt_rank % 8 == 0: a lane's 8 values are all inside or all outside
-            bf[ks][nt] = k < dr ? *reinterpret_cast<const uint4 *>(wt + (int64_t)col * dr + k) : make_uint4(0, 0, 0, 0);
+            for (int ks = 0; ks < KS; ks++) {
+                const int k = 32 * ks + 8 * lg;   // dt_rank % 8 == 0: a lane's 8 values are all inside or all outside
+                bf[ks][nt] = k < dr ? *reinterpret_cast<const uint4 *>(wt + (int64_t)col * dr + k) : make_uint4(0, 0, 0, 0);
+            }
         }
+    }
+    if constexpr (WLDS) {
+        for (int i = tid; i < 64 * KS * 4; i += 256) {   // 16-byte pieces: column i / (4 KS), k = 8 (i % (4 KS))
+            const int c = i / (KS * 4), k = 8 * (i - c * (KS * 4));
+            const int col = min(n0 + c, di - 1);
+            *reinterpret_cast<uint4 *>(&wlds[c][k]) = k < dr ? *reinterpret_cast<const uint4 *>(wt + (int64_t)col * dr + k) : make_uint4(0, 0, 0, 0);
+        }
+        __syncthreads();
     }
     auto load_a = [&](int64_t rt, uint4 (&af)[KS]) {
         const int64_t arow = min(rt * 64 + 16 * w + lr, rows - 1);
@@ -429,7 +444,12 @@ __global__ __launch_bounds__(256) void dt_proj_softplus_kernel(T *__restrict__ d
         for (int nt = 0; nt < 4; nt++) {
             acc[nt] = (v4f){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int ks = 0; ks < KS; ks++) acc[nt] = Mma32<T>::mma(af[ks], bf[ks][nt], acc[nt]);
+            for (int ks = 0; ks < KS; ks++) {
+                uint4 b;
+                if constexpr (WLDS) b = *reinterpret_cast<const uint4 *>(&wlds[16 * nt + lr][32 * ks + 8 * lg]);
+                else b = bf[ks][nt];
+                acc[nt] = Mma32<T>::mma(af[ks], b, acc[nt]);
+            }
         }
 #pragma unroll
         for (int nt = 0; nt < 4; nt++) {
