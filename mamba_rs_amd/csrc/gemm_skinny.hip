@@ -390,9 +390,10 @@ __global__ __launch_bounds__(256) void prenorm_rows_kernel(float *__restrict__ p
 // barrier).  Measured at the 130m prefill shape (50 MB of delta per layer): 25.7 us with one tile per workgroup, 22.4 us
 // walking row tiles, 26.5 us walking along the rows instead, 21.2 us with the one-branch softplus20_16.
 // WLDS: the weight fragments live in LDS instead of registers.  From dt_rank 97 up (KS >= 4: the 2.8b shape has dt_rank
-// 160) 16 registers per k-step for them left two waves per SIMD (178 registers at KS = 6) and the op ran at a third of
-// its write rate (102 us for 168 MB); read back from LDS as they are used they cost a 16-byte LDS read per matrix
-// instruction and the kernel keeps four to five waves per SIMD.
+// 160) 16 registers per k-step for them left two waves per SIMD (178 registers at KS = 6); read back from LDS as they are
+// used they cost a 16-byte LDS read per matrix instruction and the kernel keeps four waves per SIMD (2.8b shape, 168 MB of
+// delta: 102 -> 91 us).  What bounds it there is no longer this kernel's shape but its blocking: each of the 80 column
+// blocks re-reads the 6.3 MB of dt_in rows (0.5 GB through L2), which only square tiles of a real GEMM would cut.
 template <typename T, int KS, bool WLDS = (KS >= 4)>
 __global__ __launch_bounds__(256) void dt_proj_softplus_kernel(T *__restrict__ delta, const T *__restrict__ dt_in, int64_t xs,
                                                                const T *__restrict__ wt, const float *__restrict__ bias, int64_t rows,
