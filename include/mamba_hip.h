@@ -284,6 +284,12 @@ MRS_API int mrs_backbone_alloc_prefill_scratch(mrs_backbone *bb, int T);
 MRS_API int mrs_backbone_prefill_sequence(mrs_backbone *bb, const float *input, int T, float *output_last);
 /* Same, input already on the device ([batch,T,input_dim] f32); does not synchronise. */
 MRS_API int mrs_backbone_prefill_device(mrs_backbone *bb, const float *input_dev, int T);
+/* Vendor-GEMM selection for the prefill projections (no counterpart in the reference, which takes cuBLAS's default
+ * choice, src/mamba_ssm/gpu/blas.rs:771-811).  With it on, the first prefill that brings a projection shape of 1024 rows
+ * or more times every kernel the GEMM library offers for it (a few seconds per shape, once per engine) and later
+ * prefills use the fastest; results stay within the storage tolerance (another kernel sums in another order).  Off by
+ * default; MRS_GEMM_TUNE=1 in the environment turns it on for every engine at creation. */
+MRS_API int mrs_backbone_set_gemm_tuning(mrs_backbone *bb, int on);
 /* temporal_ptr / input buffer / stream accessors (inference.rs:1717-1737) and state access for tests. */
 MRS_API float *mrs_backbone_temporal_ptr(mrs_backbone *bb);
 /* download_temporal (inference.rs:1727-1737): the last step's / prefill's final-norm rows [batch, d_model] to the host; synchronises. */
@@ -422,6 +428,8 @@ MRS_API int mrs_m3_backbone_download_state(mrs_m3_backbone *bb, int layer, float
 MRS_API int mrs_m3_backbone_alloc_prefill_scratch(mrs_m3_backbone *bb, int T);
 MRS_API int mrs_m3_backbone_prefill_sequence(mrs_m3_backbone *bb, const float *input, int T, float *out_last);
 MRS_API int mrs_m3_backbone_prefill_device(mrs_m3_backbone *bb, int T);
+/* As mrs_backbone_set_gemm_tuning, for the Mamba-3 engine's in_proj / out_proj. */
+MRS_API int mrs_m3_backbone_set_gemm_tuning(mrs_m3_backbone *bb, int on);
 MRS_API float *mrs_m3_backbone_prefill_input_ptr(mrs_m3_backbone *bb);
 
 /* GpuMamba3LM (src/module/gpu_lm3.rs:54-400): the LM loop over a Mamba-3 backbone (identity input_proj).  The handle is

@@ -54,6 +54,7 @@ def _bind():
         "mrs_backbone_prefill_device": (c_int, [P, P, c_int]),
         "mrs_backbone_temporal_ptr": (P, [P]),
         "mrs_backbone_download_temporal": (c_int, [P, _FP]),
+        "mrs_backbone_set_gemm_tuning": (c_int, [P, c_int]),
         "mrs_backbone_input_ptr": (P, [P]),
         "mrs_backbone_prefill_input_ptr": (P, [P]),
         "mrs_backbone_stream": (P, [P]),
@@ -196,6 +197,11 @@ class GpuMambaBackbone:
 
     def sync(self):
         _call("mrs_backbone_sync", self._h)
+
+    def set_gemm_tuning(self, on: bool = True):
+        """Time the GEMM library's kernels for each prefill projection shape once and keep the fastest (a few seconds
+        per shape at the first prefill of that length)."""
+        _call("mrs_backbone_set_gemm_tuning", self._h, 1 if on else 0)
 
     def temporal_ptr(self) -> int:
         return _bind().mrs_backbone_temporal_ptr(self._h)

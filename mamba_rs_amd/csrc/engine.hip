@@ -17,6 +17,7 @@
 // storage), the selective scan reading B/C and the raw gate in place, out_proj.
 #include "common.hpp"
 #include "glue.hpp"
+#include "gemm_tune.hpp"
 #include <rocblas/rocblas.h>
 #include <stdlib.h>
 #include <new>
@@ -264,6 +265,7 @@ struct mrs_backbone {
     int skinny;  // decode projections on the library's own GEMM (16-bit storage: batch <= 128 or 64, K % 32 == 0; f32: batch <= 4, K % 128 == 0)
     hipStream_t stream;
     rocblas_handle blas;
+    GemmTuner *tuner;       // vendor-kernel choice for the prefill projections (off unless asked for)
     std::vector<LayerDev> layers;
     float *input_proj_w, *input_proj_b, *norm_f;
     std::vector<void *> allocs;
@@ -331,21 +333,15 @@ static int alloc_scratch(mrs_backbone *bb, Scratch *s, int64_t rows, int T) {
 
 // C[M,N] = A[M,K] (row stride lda) . W[K,N], all row-major; f32 accumulate.
 static int gemm_rm(mrs_backbone *bb, int dtype, void *C, int ldc, const void *A, int lda, const void *W, int M, int N, int K) {
-    const float one = 1.0f, zero = 0.0f;
     const rocblas_datatype t = blas_type(dtype);
-    MRS_BLAS(rocblas_gemm_ex(bb->blas, rocblas_operation_none, rocblas_operation_none, N, M, K, &one, W, t, N, A, t, lda,
-                             &zero, C, t, ldc, C, t, ldc, rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0));
-    return MRS_OK;
+    return gemm_ex_tuned(bb->tuner, bb->blas, bb->stream, 0, N, M, K, W, t, N, A, t, lda, C, t, ldc);
 }
 
 // The same product from the transposed copy Wt[N,K] (kept for the decode chain): the vendor kernels for this operand
 // order are faster at the prefill shapes (76 vs 84-92 us for in_proj at 16384 x 3072 x 768).
 static int gemm_rm_t(mrs_backbone *bb, int dtype, void *C, int ldc, const void *A, int lda, const void *Wt, int M, int N, int K) {
-    const float one = 1.0f, zero = 0.0f;
     const rocblas_datatype t = blas_type(dtype);
-    MRS_BLAS(rocblas_gemm_ex(bb->blas, rocblas_operation_transpose, rocblas_operation_none, N, M, K, &one, Wt, t, K, A, t, lda,
-                             &zero, C, t, ldc, C, t, ldc, rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0));
-    return MRS_OK;
+    return gemm_ex_tuned(bb->tuner, bb->blas, bb->stream, 1, N, M, K, Wt, t, K, A, t, lda, C, t, ldc);
 }
 
 static int launch_add_rmsnorm(mrs_backbone *bb, float *residual, const void *add, void *out, bool out_f32, const float *w,
@@ -546,6 +542,8 @@ extern "C" int mrs_backbone_create(mrs_backbone **out, int gpu_ordinal, const mr
         if (e != hipSuccess) { delete bb; return fail(MRS_E_HIP, "hipStreamCreate: %s", hipGetErrorString(e)); }
         if (rocblas_create_handle(&bb->blas) != rocblas_status_success) { hipStreamDestroy(bb->stream); delete bb; return fail(MRS_E_HIP, "rocblas_create_handle failed"); }
         rocblas_set_stream(bb->blas, bb->stream);
+        bb->tuner = gemm_tuner_create();
+        { const char *e = getenv("MRS_GEMM_TUNE"); gemm_tuner_enable(bb->tuner, e && atoi(e) != 0); }
         rocblas_set_pointer_mode(bb->blas, rocblas_pointer_mode_host);
     }
     const int dm = cfg->d_model, di = bb->di, ds = cfg->d_state, dc = cfg->d_conv, dr = bb->dr, xd = bb->xd, L = cfg->n_layers;
@@ -641,6 +639,7 @@ extern "C" void mrs_backbone_destroy(mrs_backbone *bb) {
     if (bb->graph) hipGraphDestroy(bb->graph);
     for (void *p : bb->allocs) hipFree(p);
     for (void *p : bb->prefill_allocs) hipFree(p);
+    gemm_tuner_destroy(bb->tuner);
     if (bb->blas) rocblas_destroy_handle(bb->blas);
     if (bb->stream) hipStreamDestroy(bb->stream);
     delete bb;
@@ -757,6 +756,11 @@ extern "C" int mrs_backbone_download_temporal(mrs_backbone *bb, float *out) {
     if (!bb || !out) return fail(MRS_E_NULL, "mrs_backbone_download_temporal: null pointer");
     MRS_HIP(hipMemcpyAsync(out, bb->temporal, (size_t)bb->batch * bb->cfg.d_model * 4, hipMemcpyDeviceToHost, bb->stream));
     MRS_HIP(hipStreamSynchronize(bb->stream));
+    return MRS_OK;
+}
+extern "C" int mrs_backbone_set_gemm_tuning(mrs_backbone *bb, int on) {
+    if (!bb) return fail(MRS_E_NULL, "mrs_backbone_set_gemm_tuning: null engine");
+    gemm_tuner_enable(bb->tuner, on);
     return MRS_OK;
 }
 extern "C" float *mrs_backbone_input_ptr(mrs_backbone *bb) { return bb ? bb->d_input : nullptr; }

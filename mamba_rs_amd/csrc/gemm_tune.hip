@@ -1,0 +1,116 @@
+// Vendor-GEMM solution selection for the prefill projections: see gemm_tune.hpp.
+#define ROCBLAS_BETA_FEATURES_API 1
+#include "common.hpp"
+#include "gemm_tune.hpp"
+#include <rocblas/rocblas.h>
+#include <algorithm>
+#include <map>
+#include <new>
+#include <tuple>
+#include <utility>
+#include <vector>
+
+namespace mrs {
+
+struct GemmTuner {
+    int enabled = 0;
+    // (trans_a, m, n, k, lda, ldb, ldc, a_type, b_type, c_type) -> solution index (0: the library's default)
+    std::map<std::tuple<int, int, int, int, int, int, int, int, int, int>, int> best;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+};
+
+GemmTuner *gemm_tuner_create() { return new (std::nothrow) GemmTuner(); }
+void gemm_tuner_destroy(GemmTuner *t) {
+    if (!t) return;
+    if (t->e0) hipEventDestroy(t->e0);
+    if (t->e1) hipEventDestroy(t->e1);
+    delete t;
+}
+void gemm_tuner_enable(GemmTuner *t, int on) { if (t) t->enabled = on ? 1 : 0; }
+int gemm_tuner_enabled(const GemmTuner *t) { return t ? t->enabled : 0; }
+
+namespace {
+
+struct Problem {
+    rocblas_handle h;
+    rocblas_operation ta;
+    int m, n, k, lda, ldb, ldc;
+    const void *A, *B;
+    void *C;
+    rocblas_datatype at, bt, ct;
+};
+
+rocblas_status run(const Problem &p, rocblas_gemm_algo algo, int solution) {
+    const float one = 1.0f, zero = 0.0f;
+    return rocblas_gemm_ex(p.h, p.ta, rocblas_operation_none, p.m, p.n, p.k, &one, p.A, p.at, p.lda, p.B, p.bt, p.ldb, &zero, p.C, p.ct,
+                           p.ldc, p.C, p.ct, p.ldc, rocblas_datatype_f32_r, algo, solution, 0);
+}
+
+// microseconds per call over `reps` back-to-back calls after one untimed call; negative if the solution refuses the problem
+float time_solution(GemmTuner *t, hipStream_t st, const Problem &p, rocblas_gemm_algo algo, int solution, int reps) {
+    if (run(p, algo, solution) != rocblas_status_success) return -1.0f;
+    if (hipEventRecord(t->e0, st) != hipSuccess) return -1.0f;
+    for (int i = 0; i < reps; i++)
+        if (run(p, algo, solution) != rocblas_status_success) return -1.0f;
+    if (hipEventRecord(t->e1, st) != hipSuccess || hipEventSynchronize(t->e1) != hipSuccess) return -1.0f;
+    float ms = 0.0f;
+    if (hipEventElapsedTime(&ms, t->e0, t->e1) != hipSuccess) return -1.0f;
+    return ms * 1000.0f / (float)reps;
+}
+
+int pick_solution(GemmTuner *t, hipStream_t st, const Problem &p) {
+    if (!t->e0 && (hipEventCreate(&t->e0) != hipSuccess || hipEventCreate(&t->e1) != hipSuccess)) return 0;
+    const float one = 1.0f, zero = 0.0f;
+    int n = 0;
+    if (rocblas_gemm_ex_get_solutions(p.h, p.ta, rocblas_operation_none, p.m, p.n, p.k, &one, p.A, p.at, p.lda, p.B, p.bt, p.ldb, &zero, p.C,
+                                      p.ct, p.ldc, p.C, p.ct, p.ldc, rocblas_datatype_f32_r, rocblas_gemm_algo_solution_index, 0, nullptr,
+                                      &n) != rocblas_status_success || n <= 0)
+        return 0;
+    std::vector<int> sols((size_t)n);
+    if (rocblas_gemm_ex_get_solutions(p.h, p.ta, rocblas_operation_none, p.m, p.n, p.k, &one, p.A, p.at, p.lda, p.B, p.bt, p.ldb, &zero, p.C,
+                                      p.ct, p.ldc, p.C, p.ct, p.ldc, rocblas_datatype_f32_r, rocblas_gemm_algo_solution_index, 0,
+                                      sols.data(), &n) != rocblas_status_success)
+        return 0;
+    // one timed call each, then the eight fastest again over five calls, against the default choice measured the same way
+    std::vector<std::pair<float, int>> first;
+    for (int i = 0; i < n; i++) {
+        const float us = time_solution(t, st, p, rocblas_gemm_algo_solution_index, sols[(size_t)i], 1);
+        if (us > 0.0f) first.push_back({us, sols[(size_t)i]});
+    }
+    std::sort(first.begin(), first.end());
+    float best_us = time_solution(t, st, p, rocblas_gemm_algo_standard, 0, 5);
+    int best = 0;
+    if (best_us <= 0.0f) best_us = 3.0e38f;
+    for (size_t i = 0; i < std::min<size_t>(8, first.size()); i++) {
+        const float us = time_solution(t, st, p, rocblas_gemm_algo_solution_index, first[i].second, 5);
+        if (us > 0.0f && us < best_us * 0.97f) { best_us = us; best = first[i].second; }   // 3 %: below that the default stays
+    }
+    return best;
+}
+
+}  // namespace
+
+int gemm_ex_tuned(GemmTuner *t, void *blas_handle, hipStream_t st, int trans_a, int m, int n, int k, const void *A, int a_type,
+                  int lda, const void *B, int b_type, int ldb, void *C, int c_type, int ldc) {
+    Problem p = {(rocblas_handle)blas_handle, trans_a ? rocblas_operation_transpose : rocblas_operation_none, m, n, k, lda, ldb, ldc, A, B, C,
+                 (rocblas_datatype)a_type, (rocblas_datatype)b_type, (rocblas_datatype)c_type};
+    int solution = 0;
+    if (t && t->enabled && n >= kTuneMinCols) {
+        const auto key = std::make_tuple(trans_a ? 1 : 0, m, n, k, lda, ldb, ldc, a_type, b_type, c_type);
+        const auto it = t->best.find(key);
+        if (it != t->best.end()) {
+            solution = it->second;
+        } else {
+            hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+            if (hipStreamIsCapturing(st, &cap) == hipSuccess && cap == hipStreamCaptureStatusNone) {
+                solution = pick_solution(t, st, p);
+                t->best[key] = solution;
+            }
+        }
+    }
+    const rocblas_status s = run(p, solution ? rocblas_gemm_algo_solution_index : rocblas_gemm_algo_standard, solution);
+    if (s != rocblas_status_success) return fail(MRS_E_HIP, "rocblas_gemm_ex (m=%d n=%d k=%d, solution %d): status %d", m, n, k, solution, (int)s);
+    return MRS_OK;
+}
+
+}  // namespace mrs

@@ -14,6 +14,7 @@
 //   3. out_proj with the residual add, the next layer's pre-scaled operand and row sums of squares as epilogue.
 // Shapes the skinny GEMM does not take (f32 storage above four rows among them) run RMSNorm + rocBLAS GEMMs around the same step kernel.
 #include "common.hpp"
+#include "gemm_tune.hpp"
 #include <stdlib.h>
 #include "glue.hpp"
 #include <rocblas/rocblas.h>
@@ -572,6 +573,7 @@ struct mrs_m3_backbone {
     int input_dim, batch, dtype, di, nh, ip, nr, identity_proj, device, skinny;
     hipStream_t stream;
     rocblas_handle blas;
+    GemmTuner *tuner;       // vendor-kernel choice for the prefill projections (off unless asked for)
     std::vector<Layer3> layers;
     std::vector<void *> allocs;
     std::vector<void *> pf_allocs;   // the prefill scratch alone: released and re-made when the sequence length changes
@@ -618,11 +620,8 @@ int upload_bulk3(mrs_m3_backbone *bb, void **dst, const float *src, size_t n, fl
 
 // C[M,N] (f32 or storage type) = A[M,K] . W[K,N], row-major, f32 accumulate (library GEMM)
 int gemm3(mrs_m3_backbone *bb, void *C, bool c_f32, const void *A, const void *W, int M, int N, int K) {
-    const float one = 1.0f, zero = 0.0f;
     const rocblas_datatype t = blas_type3(bb->dtype), ct = c_f32 ? rocblas_datatype_f32_r : t;
-    MRS_BLAS(rocblas_gemm_ex(bb->blas, rocblas_operation_none, rocblas_operation_none, N, M, K, &one, W, t, N, A, t, K, &zero, C, ct, N, C,
-                             ct, N, rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0));
-    return MRS_OK;
+    return gemm_ex_tuned(bb->tuner, bb->blas, bb->stream, 0, N, M, K, W, t, N, A, t, K, C, ct, N);
 }
 
 template <typename T>
@@ -711,6 +710,7 @@ extern "C" void mrs_m3_backbone_destroy(mrs_m3_backbone *bb) {
     if (bb->graph) hipGraphDestroy(bb->graph);
     for (void *p : bb->allocs) hipFree(p);
     for (void *p : bb->pf_allocs) hipFree(p);
+    gemm_tuner_destroy(bb->tuner);
     if (bb->blas) rocblas_destroy_handle(bb->blas);
     if (bb->stream) hipStreamDestroy(bb->stream);
     delete bb;
@@ -753,6 +753,8 @@ extern "C" int mrs_m3_backbone_create(mrs_m3_backbone **out, int gpu_ordinal, co
         if (e != hipSuccess) { delete bb; return fail(MRS_E_HIP, "hipStreamCreate: %s", hipGetErrorString(e)); }
         if (rocblas_create_handle(&bb->blas) != rocblas_status_success) { hipStreamDestroy(bb->stream); delete bb; return fail(MRS_E_HIP, "rocblas_create_handle failed"); }
         rocblas_set_stream(bb->blas, bb->stream);
+        bb->tuner = gemm_tuner_create();
+        { const char *e = getenv("MRS_GEMM_TUNE"); gemm_tuner_enable(bb->tuner, e && atoi(e) != 0); }
         rocblas_set_pointer_mode(bb->blas, rocblas_pointer_mode_host);
     }
     const int dm = cfg->d_model, di = bb->di, ip = bb->ip, L = cfg->n_layers;
@@ -1009,40 +1011,26 @@ int prefill_body3(mrs_m3_backbone *bb, int T) {
         const int nb = 2 * di, ns = ip - nb, nbc = 2 * c.ngroups * ds;
         const void *bulk; int64_t ldb; const float *scp, *bcp; int64_t lds_;
         {
-            const float one = 1.0f, zero = 0.0f;
-            const rocblas_datatype t = blas_type3(dt);
+            const rocblas_datatype t = blas_type3(dt), f32t = rocblas_datatype_f32_r;
+            auto gemm = [&](int ta, int m, const void *W, int ldw, void *C, rocblas_datatype ct, int ldc) {
+                return gemm_ex_tuned(bb->tuner, bb->blas, bb->stream, ta, m, (int)rows, dm, W, t, ldw, bb->pf_normed, t, dm, C, ct, ldc);
+            };
             if (dt == MRS_F32) {
-                MRS_BLAS(rocblas_gemm_ex(bb->blas, rocblas_operation_none, rocblas_operation_none, ip, (int)rows, dm, &one, lw.in_proj, t, ip,
-                                         bb->pf_normed, t, dm, &zero, bb->pf_proj, t, ip, bb->pf_proj, t, ip, rocblas_datatype_f32_r,
-                                         rocblas_gemm_algo_standard, 0, 0));
+                MRS_TRY(gemm(0, ip, lw.in_proj, ip, bb->pf_proj, t, ip));
                 bulk = bb->pf_proj; ldb = ip; bcp = bb->pf_proj + nb; scp = bcp + nbc; lds_ = ip;
             } else {
-                if (lw.in_proj_t) {   // the vendor kernels for the transposed operand are faster at these shapes (its first nb rows)
-                    MRS_BLAS(rocblas_gemm_ex(bb->blas, rocblas_operation_transpose, rocblas_operation_none, nb, (int)rows, dm, &one, lw.in_proj_t,
-                                             t, dm, bb->pf_normed, t, dm, &zero, bb->pf_bulk, t, nb, bb->pf_bulk, t, nb, rocblas_datatype_f32_r,
-                                             rocblas_gemm_algo_standard, 0, 0));
-                } else {
-                    MRS_BLAS(rocblas_gemm_ex(bb->blas, rocblas_operation_none, rocblas_operation_none, nb, (int)rows, dm, &one, lw.in_proj, t, ip,
-                                             bb->pf_normed, t, dm, &zero, bb->pf_bulk, t, nb, bb->pf_bulk, t, nb, rocblas_datatype_f32_r,
-                                             rocblas_gemm_algo_standard, 0, 0));
-                }
+                // the vendor kernels for the transposed operand are faster at these shapes (the copy's first nb rows, then the rest)
                 if (lw.in_proj_t) {
-                    MRS_BLAS(rocblas_gemm_ex(bb->blas, rocblas_operation_transpose, rocblas_operation_none, ns, (int)rows, dm, &one,
-                                             (const char *)lw.in_proj_t + (size_t)nb * dm * es, t, dm, bb->pf_normed, t, dm, &zero, bb->pf_proj,
-                                             rocblas_datatype_f32_r, ns, bb->pf_proj, rocblas_datatype_f32_r, ns, rocblas_datatype_f32_r,
-                                             rocblas_gemm_algo_standard, 0, 0));
+                    MRS_TRY(gemm(1, nb, lw.in_proj_t, dm, bb->pf_bulk, t, nb));
+                    MRS_TRY(gemm(1, ns, (const char *)lw.in_proj_t + (size_t)nb * dm * es, dm, bb->pf_proj, f32t, ns));
                 } else {
-                    MRS_BLAS(rocblas_gemm_ex(bb->blas, rocblas_operation_none, rocblas_operation_none, ns, (int)rows, dm, &one,
-                                             (const char *)lw.in_proj + (size_t)nb * es, t, ip, bb->pf_normed, t, dm, &zero, bb->pf_proj,
-                                             rocblas_datatype_f32_r, ns, bb->pf_proj, rocblas_datatype_f32_r, ns, rocblas_datatype_f32_r,
-                                             rocblas_gemm_algo_standard, 0, 0));
+                    MRS_TRY(gemm(0, nb, lw.in_proj, ip, bb->pf_bulk, t, nb));
+                    MRS_TRY(gemm(0, ns, (const char *)lw.in_proj + (size_t)nb * es, ip, bb->pf_proj, f32t, ns));
                 }
                 bulk = bb->pf_bulk; ldb = nb; bcp = bb->pf_proj; scp = bcp + nbc; lds_ = ns;
             }
         }
-        // the chunked kernel reads x in place out of the bulk rows.  (Folding the SiLU gate into its y store was
-        // measured and dropped: the scattered z reads cost the latency-bound kernel 54 us against 28 us for the
-        // separate gate pass.)
+        // the chunked kernel reads x (and the gate z) in place out of the bulk rows
         const bool in_place = chunked_ok && dt != MRS_F32 && ldb % 8 == 0 && di % 8 == 0;
         // one group at headdim = d_state = 64 with the rope pairs in fours: the scan builds its K and Q tiles from the
         // normalised B / C rows and the angles, so the [rows, nheads, d_state] K and Q never exist in memory
@@ -1108,6 +1096,12 @@ int prefill_body3(mrs_m3_backbone *bb, int T) {
 }
 
 }  // namespace
+
+extern "C" int mrs_m3_backbone_set_gemm_tuning(mrs_m3_backbone *bb, int on) {
+    if (!bb) return fail(MRS_E_NULL, "mrs_m3_backbone_set_gemm_tuning: null engine");
+    gemm_tuner_enable(bb->tuner, on);
+    return MRS_OK;
+}
 
 // Runs the sequences already in prefill_input_ptr() ([batch, T, input_dim] f32), continuing from the engine's state and
 // leaving it positioned for step(); norm_f output of the last position in temporal_ptr().

@@ -203,6 +203,7 @@ def _bind():
         "mrs_m3_backbone_alloc_prefill_scratch": (c_int, [P, c_int]),
         "mrs_m3_backbone_prefill_sequence": (c_int, [P, _FP, c_int, _FP]),
         "mrs_m3_backbone_prefill_device": (c_int, [P, c_int]),
+        "mrs_m3_backbone_set_gemm_tuning": (c_int, [P, c_int]),
         "mrs_m3_backbone_prefill_input_ptr": (P, [P]),
     }
     for name, (res, args) in sigs.items():
@@ -308,6 +309,10 @@ class GpuMamba3Backbone:
 
     def sync(self):
         _call("mrs_m3_backbone_sync", self._h)
+
+    def set_gemm_tuning(self, on: bool = True):
+        """Time the GEMM library's kernels for each prefill projection shape once and keep the fastest."""
+        _call("mrs_m3_backbone_set_gemm_tuning", self._h, 1 if on else 0)
 
     def temporal_ptr(self) -> int:
         return _bind().mrs_m3_backbone_temporal_ptr(self._h)

@@ -328,3 +328,33 @@ def test_few_row_decode_chain_with_folded_x_proj_equals_the_many_row_chain(dm, b
         (ca, sa), (cb, sb) = few.download_state(layer), many.download_state(layer)
         assert cosine(sa, sb[:batch]) >= 0.9995 and cosine(ca, cb[:batch]) >= 0.9995
     few.close(); many.close()
+
+
+def test_prefill_with_tuned_vendor_gemms_matches_the_default_choice_and_the_cpu_route():
+    """set_gemm_tuning: the first prefill of 1024 rows or more times the GEMM library's kernels for each projection
+    shape and later prefills run the fastest.  Another kernel sums in another order, so the tuned prefill is held to
+    the untuned one by cosine and, like it, to the CPU route; tuned runs repeat bit for bit."""
+    cfg = MambaConfig(d_model=256, d_state=16, d_conv=4, expand=2, n_layers=2)
+    w = MambaWeights.init(cfg, 256, 77)
+    P = oracle_params(w, cfg, 256, round_to=orc.BF16)
+    B, T = 2, 512
+    xs = (np.random.default_rng(5).standard_normal((B, T, 256)) * 0.5).astype(np.float32)
+    eng = GpuMambaBackbone.new_with_dtype(0, w, cfg, 256, B, WeightDtype.BF16)
+    print("case prefill, default vendor kernels", flush=True)
+    base = eng.prefill_sequence(xs).copy()
+    base_ssm = [eng.download_state(l)[1].copy() for l in range(2)]
+    eng.set_gemm_tuning(True)
+    runs = []
+    for i in range(3):
+        print(f"case prefill, tuned vendor kernels, run {i}", flush=True)
+        eng.reset()
+        runs.append((eng.prefill_sequence(xs).copy(), [eng.download_state(l)[1].copy() for l in range(2)]))
+    for last, ssm in runs[1:]:
+        assert np.array_equal(last, runs[0][0]) and all(np.array_equal(a, b) for a, b in zip(ssm, runs[0][1]))
+    assert cosine(runs[0][0], base) >= 0.9999
+    for l in range(2):
+        assert cosine(runs[0][1][l], base_ssm[l]) >= 0.9999
+    conv, ssm = orc.m1_zero_state(P)
+    want = orc.m1_backbone_prefill(P, xs[1], conv, ssm)
+    assert cosine(runs[0][0][1], want[-1]) >= 0.999
+    eng.close()
