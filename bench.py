@@ -169,7 +169,7 @@ DEFAULT_LEGS = "c1,lm,lm28,published,m1_kernels,m3,m3_engine"
 
 
 def lm_leg(name, cfg_kw, vocab, prefill_bt, decode_b, decode_steps, seed=42, shared_layer=False, cpu_sample=None,
-           with_generate=True, gemm_tuning=False):
+           with_generate=True, gemm_tuning=False, decode_graph=True):
     """Prefill tok/s and greedy-decode us/step of a random-init LM-shaped backbone (bf16 storage):
     token ids -> device embedding gather -> backbone (-> tied head -> argmax for decode).  With shared_layer the model's
     layers all hold one layer's random weights (timing only: the kernels and their operand sizes are those of the full
@@ -217,18 +217,29 @@ def lm_leg(name, cfg_kw, vocab, prefill_bt, decode_b, decode_steps, seed=42, sha
         out["cpu_port_prefill"] = cpu_prefill_sample(cfg_kw, cpu_sample[0], cpu_sample[1], pb * pt, seed)
     dec_out = []
     for db in (decode_b if isinstance(decode_b, (list, tuple)) else [decode_b]):
-        dec = GpuMambaBackbone.new_with_dtype(0, w, cfg, cfg.d_model, db, WeightDtype.BF16)
-        lm_d = GpuMambaLM(dec, embed)
-        lm_d.set_tokens(rng.integers(0, vocab, db).astype(np.int32))
-        lm_d.capture_graph()
-        for _ in range(8):
-            lm_d.decode_step()
-        dec.sync()
-        t0 = time.perf_counter()
-        for _ in range(decode_steps):
-            lm_d.decode_step()
-        dec.sync()
-        td = (time.perf_counter() - t0) / decode_steps
+        def timed_decode(tuned):
+            dec = GpuMambaBackbone.new_with_dtype(0, w, cfg, cfg.d_model, db, WeightDtype.BF16)
+            if tuned:
+                dec.set_gemm_tuning(True)                  # takes effect in the eager step that precedes the capture
+            lm_d = GpuMambaLM(dec, embed)
+            lm_d.set_tokens(rng.integers(0, vocab, db).astype(np.int32))
+            if decode_graph:
+                lm_d.capture_graph()
+            for _ in range(8):
+                lm_d.decode_step()
+            dec.sync()
+            t0 = time.perf_counter()
+            for _ in range(decode_steps):
+                lm_d.decode_step()
+            dec.sync()
+            return dec, lm_d, (time.perf_counter() - t0) / decode_steps
+        # from 65 rows (wide models) or 129 rows up the projections of a decode step go to the GEMM library as well
+        tune_decode = gemm_tuning and db > 64
+        td_default = None
+        if tune_decode:
+            dec, lm_d, td_default = timed_decode(False)
+            lm_d.close(); dec.close()
+        dec, lm_d, td = timed_decode(tune_decode)
         tk = lm_d.get_tokens()
         assert ((tk >= 0) & (tk < vocab)).all()
         es = 2
@@ -237,7 +248,12 @@ def lm_leg(name, cfg_kw, vocab, prefill_bt, decode_b, decode_steps, seed=42, sha
         step_bytes = cfg.n_layers * layer_bytes + ((vocab + 63) // 64 * 64) * dm * es
         entry = {"batch": db, "steps": decode_steps, "us_per_step": td * 1e6, "tok_per_s": db / td,
                  "algorithmic_bytes_per_step": step_bytes, "hbm_frac": step_bytes / td / 1e9 / HBM_PEAK_GBPS}
-        if with_generate:
+        if td_default is not None:
+            entry["vendor_gemm_kernels"] = "timed once, fastest kept"
+            entry["us_per_step_with_default_vendor_kernels"] = td_default * 1e6
+        if not decode_graph:
+            entry["launch"] = "kernel by kernel (no hipGraph)"
+        if with_generate and decode_graph:
             # batched generation with the sampler in the loop: ragged prompts of 8..12 tokens, 128 new tokens per slot
             from mamba_rs_amd import SampleParams
             prompts = [[int(t) for t in rng.integers(0, vocab, 8 + (i % 5))] for i in range(db)]
@@ -568,6 +584,9 @@ def main():
     ap.add_argument("--big", action="store_true", help="the 2.8b-shape LM leg with 64 independently initialised layers (minutes of host-side init) instead of one shared layer")
     ap.add_argument("--gemm-tune", choices=["auto", "on", "off"], default="auto",
                     help="prefill legs of the LM engines pick their vendor GEMM kernels by timing them (auto: in the full default run only)")
+    ap.add_argument("--lm-no-graph", action="store_true",
+                    help="the decode steps of the lm / lm28 legs launch kernel by kernel instead of replaying a hipGraph, and the "
+                         "generation runs are skipped (for kernel traces of those steps)")
     ap.add_argument("--legs", default=DEFAULT_LEGS,
                     help="comma list of the extras to run: c1, lm, lm28, published, m1_kernels, m3, m3_engine (for profiling one leg at a time)")
     args = ap.parse_args()
@@ -620,7 +639,8 @@ def main():
             extras["reference_default_configs_f32"] = default_configs_leg()
         if "lm" in legs:
             extras["lm_130m_shape_bf16"] = lm_leg("130m-shape", dict(d_model=768, d_state=16, d_conv=4, expand=2, n_layers=24), 50280,
-                                                  (8, 2048), [64, 1], 256, cpu_sample=(24, 256), gemm_tuning=tune)
+                                                  (8, 2048), [64, 1], 256, cpu_sample=(24, 256), gemm_tuning=tune,
+                                                  decode_graph=not args.lm_no_graph)
         if "published" in legs:
             extras["reference_published_configs"] = published_configs_leg()
         if "m1_kernels" in legs:
@@ -634,7 +654,7 @@ def main():
         if "lm28" in legs or args.big:
             extras["lm_2.8b_shape_bf16"] = lm_leg("2.8b-shape", dict(d_model=2560, d_state=16, d_conv=4, expand=2, n_layers=64), 50280,
                                                   (4, 4096), [1, 16, 128], 128, shared_layer=not args.big, cpu_sample=(2, 64),
-                                                  with_generate=False, gemm_tuning=tune)
+                                                  with_generate=False, gemm_tuning=tune, decode_graph=not args.lm_no_graph)
         out["extras"] = extras
     print(json.dumps(out))
 

@@ -284,11 +284,13 @@ MRS_API int mrs_backbone_alloc_prefill_scratch(mrs_backbone *bb, int T);
 MRS_API int mrs_backbone_prefill_sequence(mrs_backbone *bb, const float *input, int T, float *output_last);
 /* Same, input already on the device ([batch,T,input_dim] f32); does not synchronise. */
 MRS_API int mrs_backbone_prefill_device(mrs_backbone *bb, const float *input_dev, int T);
-/* Vendor-GEMM selection for the prefill projections (no counterpart in the reference, which takes cuBLAS's default
- * choice, src/mamba_ssm/gpu/blas.rs:771-811).  With it on, the first prefill that brings a projection shape of 1024 rows
- * or more times every kernel the GEMM library offers for it (a few seconds per shape, once per engine) and later
- * prefills use the fastest; results stay within the storage tolerance (another kernel sums in another order).  Off by
- * default; MRS_GEMM_TUNE=1 in the environment turns it on for every engine at creation. */
+/* Vendor-GEMM selection for the projections that go to the GEMM library: prefill, and decode steps of engines past the
+ * own chain's row limit (no counterpart in the reference, which takes cuBLAS's default choice,
+ * src/mamba_ssm/gpu/blas.rs:771-811).  With it on, the first call outside a stream capture that brings a projection
+ * shape of 32 rows or more times every kernel the library offers for it (a few seconds per shape, once per engine) and
+ * later calls use the fastest -- for decode that call is the eager step before mrs_backbone_capture_graph /
+ * mrs_lm_capture_graph, so turn it on before capturing.  Results stay within the storage tolerance (another kernel sums
+ * in another order).  Off by default; MRS_GEMM_TUNE=1 in the environment turns it on for every engine at creation. */
 MRS_API int mrs_backbone_set_gemm_tuning(mrs_backbone *bb, int on);
 /* temporal_ptr / input buffer / stream accessors (inference.rs:1717-1737) and state access for tests. */
 MRS_API float *mrs_backbone_temporal_ptr(mrs_backbone *bb);

@@ -199,8 +199,9 @@ class GpuMambaBackbone:
         _call("mrs_backbone_sync", self._h)
 
     def set_gemm_tuning(self, on: bool = True):
-        """Time the GEMM library's kernels for each prefill projection shape once and keep the fastest (a few seconds
-        per shape at the first prefill of that length)."""
+        """Time the GEMM library's kernels for each projection shape once and keep the fastest (a few seconds per shape
+        at the first prefill of a given length, or at the eager decode step that precedes capture_graph when the batch
+        is past the own chain's row limit: call it before capturing)."""
         _call("mrs_backbone_set_gemm_tuning", self._h, 1 if on else 0)
 
     def temporal_ptr(self) -> int:

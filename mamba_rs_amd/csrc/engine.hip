@@ -452,7 +452,7 @@ static int run_layers(mrs_backbone *bb, Scratch *s, int T) {
         const char *z = (const char *)s->proj + (size_t)di * es;  // gate half of in_proj's output
         const char *xb = (const char *)s->xdbl;
         MRS_TRY(launch_add_rmsnorm(bb, s->residual, l == 0 ? nullptr : s->out, s->normed, false, lw.norm_w, rows, dm));
-        if (T > 1 && lw.in_proj_t) MRS_TRY(gemm_rm_t(bb, dt, s->proj, 2 * di, s->normed, dm, lw.in_proj_t, (int)rows, 2 * di, dm));
+        if (lw.in_proj_t) MRS_TRY(gemm_rm_t(bb, dt, s->proj, 2 * di, s->normed, dm, lw.in_proj_t, (int)rows, 2 * di, dm));
         else MRS_TRY(gemm_rm(bb, dt, s->proj, 2 * di, s->normed, dm, lw.in_proj, (int)rows, 2 * di, dm));
         if (T == 1) {
             MRS_TRY(launch_conv1d_step(bb->stream, dt, s->u, conv, s->proj, 2 * di, lw.conv_w, lw.conv_b, B, di, dc, 1));
@@ -495,7 +495,7 @@ static int run_layers(mrs_backbone *bb, Scratch *s, int T) {
             MRS_TRY(mrs_ssm_scan_fwd_ex(bb->stream, dt, ssm, s->y, s->delta, s->u, xb + es * dr, xb + es * (dr + ds), xd, lw.a_neg,
                                         lw.D, z, 2 * di, flags, s->scan_ws, s->scan_ws_bytes, B, T, di, ds));
         }
-        if (T > 1 && lw.out_proj_t) MRS_TRY(gemm_rm_t(bb, dt, s->out, dm, s->y, di, lw.out_proj_t, (int)rows, dm, di));
+        if (lw.out_proj_t) MRS_TRY(gemm_rm_t(bb, dt, s->out, dm, s->y, di, lw.out_proj_t, (int)rows, dm, di));
         else MRS_TRY(gemm_rm(bb, dt, s->out, dm, s->y, di, lw.out_proj, (int)rows, dm, di));
     }
     if (T == 1) {
@@ -594,15 +594,18 @@ extern "C" int mrs_backbone_create(mrs_backbone **out, int gpu_ordinal, const mr
             MRS_CREATE_TRY(dev_alloc(bb, &d.dt_w_t, (size_t)dr * di * esize(bb->dtype)));
             MRS_CREATE_TRY(launch_transpose(bb->stream, bb->dtype, d.dt_w_t, d.dt_w, dr, di));
         }
-        if (bb->skinny) {
-            // transposed copies for the decode chain (one more copy of the bulk weights in HBM)
+        if (bb->skinny || bb->dtype != MRS_F32) {
+            // transposed copies (one more copy of the bulk weights in HBM): the decode chain's own GEMM reads them, and the
+            // vendor kernels for this operand order are the faster ones for in_proj and out_proj from 128 rows up
             const size_t es_ = esize(bb->dtype);
             MRS_CREATE_TRY(dev_alloc(bb, &d.in_proj_t, (size_t)dm * 2 * di * es_));
-            MRS_CREATE_TRY(dev_alloc(bb, &d.x_proj_t, (size_t)di * xd * es_));
             MRS_CREATE_TRY(dev_alloc(bb, &d.out_proj_t, (size_t)di * dm * es_));
             MRS_CREATE_TRY(launch_transpose(bb->stream, bb->dtype, d.in_proj_t, d.in_proj, dm, 2 * di));
-            MRS_CREATE_TRY(launch_transpose(bb->stream, bb->dtype, d.x_proj_t, d.x_proj, di, xd));
             MRS_CREATE_TRY(launch_transpose(bb->stream, bb->dtype, d.out_proj_t, d.out_proj, di, dm));
+        }
+        if (bb->skinny) {
+            MRS_CREATE_TRY(dev_alloc(bb, &d.x_proj_t, (size_t)di * xd * esize(bb->dtype)));
+            MRS_CREATE_TRY(launch_transpose(bb->stream, bb->dtype, d.x_proj_t, d.x_proj, di, xd));
         }
         // a_neg = -exp(a_log) once at load (exp_negate, src/mamba_ssm/gpu/inference.rs:266-282)
         MRS_CREATE_TRY(dev_alloc(bb, (void **)&d.a_neg, (size_t)di * ds * 4));

@@ -71,18 +71,20 @@ int pick_solution(GemmTuner *t, hipStream_t st, const Problem &p) {
                                       p.ct, p.ldc, p.C, p.ct, p.ldc, rocblas_datatype_f32_r, rocblas_gemm_algo_solution_index, 0,
                                       sols.data(), &n) != rocblas_status_success)
         return 0;
-    // one timed call each, then the eight fastest again over five calls, against the default choice measured the same way
+    // one timed call each, then the eight fastest again over five or more calls, against the default choice measured the same way
     std::vector<std::pair<float, int>> first;
     for (int i = 0; i < n; i++) {
         const float us = time_solution(t, st, p, rocblas_gemm_algo_solution_index, sols[(size_t)i], 1);
         if (us > 0.0f) first.push_back({us, sols[(size_t)i]});
     }
     std::sort(first.begin(), first.end());
-    float best_us = time_solution(t, st, p, rocblas_gemm_algo_standard, 0, 5);
+    // (a short problem is repeated until the timed stretch is some 300 us, so that the event pair's own cost does not decide)
+    const int reps = first.empty() ? 5 : std::max(5, std::min(40, (int)(300.0f / std::max(first[0].first, 1.0f))));
+    float best_us = time_solution(t, st, p, rocblas_gemm_algo_standard, 0, reps);
     int best = 0;
     if (best_us <= 0.0f) best_us = 3.0e38f;
     for (size_t i = 0; i < std::min<size_t>(8, first.size()); i++) {
-        const float us = time_solution(t, st, p, rocblas_gemm_algo_solution_index, first[i].second, 5);
+        const float us = time_solution(t, st, p, rocblas_gemm_algo_solution_index, first[i].second, reps);
         if (us > 0.0f && us < best_us * 0.97f) { best_us = us; best = first[i].second; }   // 3 %: below that the default stays
     }
     return best;

@@ -358,3 +358,32 @@ def test_prefill_with_tuned_vendor_gemms_matches_the_default_choice_and_the_cpu_
     want = orc.m1_backbone_prefill(P, xs[1], conv, ssm)
     assert cosine(runs[0][0][1], want[-1]) >= 0.999
     eng.close()
+
+
+@pytest.mark.parametrize("tuned", [False, True])
+def test_decode_above_the_own_chain_limit_runs_the_projections_from_the_transposed_copies(tuned):
+    """130 rows at d_model 768: past the own chain's limit, so in_proj and out_proj go to the GEMM library reading the
+    transposed weight copies, x_proj and dt_proj reading the originals.  Eager steps, then replays of the captured step;
+    with set_gemm_tuning the step that precedes the capture times the library's kernels for the four shapes and the
+    graph holds the chosen ones.  First, middle and last row against the CPU route on storage-rounded weights."""
+    B = 130
+    cfg = MambaConfig(d_model=768, d_state=16, d_conv=4, expand=2, n_layers=2)
+    w = MambaWeights.random_lm(cfg, seed=B, std=0.05)
+    P = oracle_params(w, cfg, 768, round_to=orc.BF16)
+    P.input_proj_w[:] = np.eye(768, dtype=np.float32); P.input_proj_b[:] = 0
+    rng = np.random.default_rng(B)
+    eng = GpuMambaBackbone.new_with_dtype(0, w, cfg, 768, B, WeightDtype.BF16)
+    if tuned:
+        eng.set_gemm_tuning(True)
+    x = rng.standard_normal((5, B, 768)).astype(np.float32)
+    rows = (0, B // 2, B - 1)
+    st = {b: orc.m1_zero_state(P) for b in rows}
+    for t in range(5):
+        print(f"case library-chain decode, tuned={tuned}, step {t}", flush=True)
+        if t == 2:
+            eng.capture_graph()
+        got = eng.step(x[t])
+        for b in rows:
+            want = orc.m1_backbone_step(P, x[t, b], *st[b])
+            assert cosine(got[b], want) >= 0.999, (t, b)
+    eng.close()
