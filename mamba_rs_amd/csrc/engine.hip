@@ -560,9 +560,11 @@ extern "C" int mrs_backbone_create(mrs_backbone **out, int gpu_ordinal, const mr
     bb->layers.resize(L);
     {
         static const bool off = [] { const char *e = getenv("MRS_DECODE_LIBRARY_GEMM"); return e && atoi(e) != 0; }();
-        // Rows up to which the own chain beats the library chain, measured: 128 at the 130m shape (989 vs 1179 us per step;
-        // at 256 rows 1490 vs 1392), 64 at the 2.8b shape (a tie there).  "Narrow" as for the x_proj shares.
-        const int max_rows = std::min(skinny_max_rows(), narrow_model(di, xd) ? 128 : 64);
+        // Rows up to which the own chain beats the library chain (in_proj / out_proj from the transposed copies, default
+        // vendor kernels), measured: 128 at the 130m shape (1032 vs 1091 us per step; at 256 rows 1490 vs 1392), 40 at the
+        // 2.8b shape (32 rows 5.13 vs 8.35 ms, 40 rows 5.74 vs 5.92, 48 rows 6.13 vs 5.98, 64 rows 7.58 vs 6.19).  "Narrow"
+        // as for the x_proj shares.
+        const int max_rows = std::min(skinny_max_rows(), narrow_model(di, xd) ? 128 : 40);
         bb->skinny = !off && (dtype == MRS_BF16 || dtype == MRS_F16) && batch <= max_rows && dm % 32 == 0 && di % 32 == 0;
         // f32 storage: the same chain on the row-wise route of the GEMM (one to four rows, rows of the operand in LDS)
         if (!off && dtype == MRS_F32 && batch <= 4 && dm % 128 == 0 && di % 128 == 0 && (int64_t)di * 16 <= 48 * 1024 &&

@@ -118,6 +118,65 @@ __global__ __launch_bounds__(256) void add_rmsnorm_rows_kernel(float *__restrict
     }
 }
 
+// Decode-sized row counts past the own chain's limit (64 to 255 rows): one workgroup per row with the same 16-byte
+// accesses, every load of the row issued before the first use (a row of 2560 is 2.5 pieces per lane: one round trip to
+// memory, a reduction through LDS, one store).  Same arithmetic as add_rmsnorm_kernel.
+template <typename T, typename TO, int TRIPS>
+__global__ __launch_bounds__(256) void add_rmsnorm_block_kernel(float *__restrict__ residual, const T *__restrict__ add,
+                                                                TO *__restrict__ out, const float *__restrict__ w, float eps, int dm) {
+    __shared__ float part[4];
+    const int64_t row = blockIdx.x;
+    const int nv = dm >> 2;
+    float4 *r4 = reinterpret_cast<float4 *>(residual + row * dm);
+    struct alignas(4 * sizeof(T)) V4 { T v[4]; };
+    struct alignas(4 * sizeof(TO)) O4 { TO v[4]; };
+    const V4 *a4 = reinterpret_cast<const V4 *>(add ? add + row * dm : nullptr);
+    const float4 *w4 = reinterpret_cast<const float4 *>(w);
+    float4 v[TRIPS], ww[TRIPS];
+    V4 a[TRIPS];
+#pragma unroll
+    for (int k = 0; k < TRIPS; k++) {
+        const int c = threadIdx.x + 256 * k;
+        if (c < nv) {
+            v[k] = r4[c];
+            if (add) a[k] = a4[c];
+            ww[k] = w4[c];
+        }
+    }
+    float ss = 0.0f;
+#pragma unroll
+    for (int k = 0; k < TRIPS; k++) {
+        const int c = threadIdx.x + 256 * k;
+        if (c < nv) {
+            if (add) {
+                v[k].x += Store<T>::ld(&a[k].v[0]); v[k].y += Store<T>::ld(&a[k].v[1]);
+                v[k].z += Store<T>::ld(&a[k].v[2]); v[k].w += Store<T>::ld(&a[k].v[3]);
+                r4[c] = v[k];
+            }
+            ss = fmaf(v[k].x, v[k].x, ss); ss = fmaf(v[k].y, v[k].y, ss); ss = fmaf(v[k].z, v[k].z, ss); ss = fmaf(v[k].w, v[k].w, ss);
+        }
+    }
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) ss += __shfl_xor(ss, m, kWave);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    ss = part[0] + part[1] + part[2] + part[3];
+    float rms = sqrtf(ss / (float)dm + eps);
+    if (!isfinite(rms) || rms < 1e-20f) rms = 1.0f;
+    const float inv = 1.0f / rms;
+    O4 *o4 = reinterpret_cast<O4 *>(out + row * dm);
+#pragma unroll
+    for (int k = 0; k < TRIPS; k++) {
+        const int c = threadIdx.x + 256 * k;
+        if (c < nv) {
+            O4 o;
+            Store<TO>::st(&o.v[0], v[k].x * inv * ww[k].x); Store<TO>::st(&o.v[1], v[k].y * inv * ww[k].y);
+            Store<TO>::st(&o.v[2], v[k].z * inv * ww[k].z); Store<TO>::st(&o.v[3], v[k].w * inv * ww[k].w);
+            o4[c] = o;
+        }
+    }
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void cast_from_f32_kernel(T *__restrict__ out, const float *__restrict__ in, int64_t n) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -136,6 +195,15 @@ template <typename T>
 inline void launch_add_rmsnorm_typed(hipStream_t st, float *residual, const void *add, void *out, bool out_f32, void *out2, const float *w,
                                      float eps, int64_t rows, int dm, int64_t out_stride) {
     const dim3 grid((unsigned)rows), block(256);
+    if (rows >= 64 && rows < 256 && dm % 4 == 0 && dm <= 4096 && out_stride == dm && !out2 && !out_f32) {
+#define MRS_BLK(TR) hipLaunchKernelGGL((add_rmsnorm_block_kernel<T, T, TR>), grid, block, 0, st, residual, (const T *)add, (T *)out, w, eps, dm)
+        const int trips = (dm / 4 + 255) / 256;
+        if (trips <= 1) MRS_BLK(1);
+        else if (trips <= 2) MRS_BLK(2);
+        else MRS_BLK(4);
+#undef MRS_BLK
+        return;
+    }
     if (rows >= 256 && dm % 4 == 0 && dm <= 4096 && out_stride == dm && !out2 && !out_f32) {
         const dim3 g4((unsigned)((rows + 3) / 4));
 #define MRS_ROWS(TR) hipLaunchKernelGGL((add_rmsnorm_rows_kernel<T, T, TR>), g4, block, 0, st, residual, (const T *)add, (T *)out, w, eps, rows, dm)

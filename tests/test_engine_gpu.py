@@ -238,15 +238,15 @@ def test_16bit_engine_batch_above_64_takes_the_library_gemm_chain():
 
 def test_wide_dt_rank_at_large_batch_runs_dt_proj_as_its_own_gemm():
     """batch x dt_rank above the fusion limit (4096): the decode step takes delta from a GEMM instead of forming it
-    inside the step kernel -- own-GEMM chain at batch 64 (d_model 1024 -> dt_rank 64... 64 x 64 = 4096 is still fused,
-    so d_model 1056 -> dt_rank 66 is not a multiple of 32; use d_model 2048 -> dt_rank 128) and library chain at batch 65."""
+    inside the step kernel -- own-GEMM chain at batch 40, the last row count it takes for a wide model (d_model 2048 ->
+    dt_rank 128, 40 x 128 = 5120), and library chain at batch 41 and 65."""
     cfg = MambaConfig(d_model=2048, d_state=16, d_conv=4, expand=1, n_layers=1)
     w = MambaWeights.init(cfg, 2048, 44)
     w.input_proj_w = np.zeros(0, np.float32); w.input_proj_b = np.zeros(0, np.float32)
     P = oracle_params(w, cfg, 2048, round_to=orc.BF16)
     P.input_proj_w[:] = np.eye(2048, dtype=np.float32); P.input_proj_b[:] = 0
     rng = np.random.default_rng(4)
-    for B in (64, 65):
+    for B in (40, 41, 65):
         eng = GpuMambaBackbone.new_with_dtype(0, w, cfg, 2048, B, WeightDtype.BF16)
         x = rng.standard_normal((4, B, 2048)).astype(np.float32)
         rows = (0, B - 1)
