@@ -17,7 +17,7 @@ namespace mrs {
 
 constexpr int kMaxConv = 8;  // reference limit, src/config.rs:154-159
 
-template <typename T, bool SILU>
+template <typename T, bool SILU, bool DC4 = false>
 __global__ __launch_bounds__(256) void conv1d_step_kernel(
     T *__restrict__ out, float *__restrict__ state, const T *__restrict__ new_x, int64_t x_stride,
     const float *__restrict__ weight, const float *__restrict__ bias, int64_t total, int di, int dc) {
@@ -28,6 +28,16 @@ __global__ __launch_bounds__(256) void conv1d_step_kernel(
     float *st = state + r * dc;
     const float *w = weight + (int64_t)d * dc;
     float s = bias[d];
+    if constexpr (DC4) {
+        // d_conv 4 with 16-byte aligned state and taps: the window and the taps as one 16-byte access each (three 4-byte loads at a 16-byte lane stride
+        // ask for every cache line of the wave's window three times)
+        const float4 sv = *reinterpret_cast<const float4 *>(st), wv = *reinterpret_cast<const float4 *>(w);
+        const float xn = Store<T>::ld(new_x + xi);
+        s = fmaf(sv.y, wv.x, s); s = fmaf(sv.z, wv.y, s); s = fmaf(sv.w, wv.z, s); s = fmaf(xn, wv.w, s);
+        *reinterpret_cast<float4 *>(st) = make_float4(sv.y, sv.z, sv.w, xn);
+        Store<T>::st(out + r, SILU ? silu(s) : s);
+        return;
+    }
     float win[kMaxConv];
 #pragma unroll
     for (int k = 0; k < kMaxConv; k++)
@@ -250,8 +260,10 @@ int launch_conv1d_step(hipStream_t st, int dtype, void *out, float *state, const
     const int64_t blocks = (total + 255) / 256;
     if (blocks > 0x7fffffffLL) return fail(MRS_E_SHAPE, "conv1d step: grid too large");
     const dim3 grid((unsigned)blocks), block(256);
+    const bool dc4 = d_conv == 4 && aligned(state, 16) && aligned(weight, 16);
     MRS_DISPATCH_DTYPE(dtype, T_, {
-        if (apply_silu) hipLaunchKernelGGL((conv1d_step_kernel<T_, true>), grid, block, 0, st, (T_ *)out, state, (const T_ *)new_x, x_stride, weight, bias, total, d_inner, d_conv);
+        if (apply_silu && dc4) hipLaunchKernelGGL((conv1d_step_kernel<T_, true, true>), grid, block, 0, st, (T_ *)out, state, (const T_ *)new_x, x_stride, weight, bias, total, d_inner, d_conv);
+        else if (apply_silu) hipLaunchKernelGGL((conv1d_step_kernel<T_, true>), grid, block, 0, st, (T_ *)out, state, (const T_ *)new_x, x_stride, weight, bias, total, d_inner, d_conv);
         else hipLaunchKernelGGL((conv1d_step_kernel<T_, false>), grid, block, 0, st, (T_ *)out, state, (const T_ *)new_x, x_stride, weight, bias, total, d_inner, d_conv);
     });
     return check_launch("conv1d_step_kernel");
