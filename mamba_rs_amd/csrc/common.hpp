@@ -124,6 +124,21 @@ int launch_skinny_gemm(hipStream_t st, int dtype, void *C, int out_f32, int64_t 
                        int M, int N, int K, const SkinnyEpi &ep);
 int launch_transpose(hipStream_t st, int dtype, void *Wt, const void *W, int K, int N);
 // delta[r, d] = softplus(round(dt_in[r, :] . wt[d, :]) + bias[d]) for 16-bit storage; wt is the transposed [d_inner][dt_rank] weight
+// A whole f32 backbone step in one launch for small models (one workgroup per batch row; csrc/tiny_step.hip).  All
+// pointers are device memory; weights row-major as the engine holds them (in_proj [dm][2 di], x_proj [di][xd],
+// dt_w [dt_rank][di], out_proj [di][dm], in_w [input_dim][dm] or null for the identity input projection).
+struct TinyStepLayer {
+    const float *norm_w, *in_proj, *conv_w, *conv_b, *x_proj, *dt_w, *dt_b, *a_neg, *D, *out_proj;
+};
+struct TinyStepArgs {
+    const TinyStepLayer *layers;
+    const float *input, *in_w, *in_b, *norm_f;
+    float *conv_state, *ssm_state, *temporal;
+    float eps;
+    int n_layers, batch, input_dim, dm, di, ds, dc, dr, xd;
+};
+bool tiny_step_ok(int dtype, int input_dim, int dm, int di, int ds, int dc, int dr, int xd);
+int launch_tiny_step(hipStream_t st, const TinyStepArgs &a);
 bool dt_proj_softplus_ok(int dtype, int di, int dr, int64_t xs, const void *delta, const void *dt_in, const void *wt);
 int launch_dt_proj_softplus(hipStream_t st, int dtype, void *delta, const void *dt_in, int64_t xs, const void *wt, const float *bias,
                             int64_t rows, int di, int dr);

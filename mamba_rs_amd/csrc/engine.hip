@@ -212,7 +212,7 @@ struct LayerDev {
     void *in_proj, *x_proj, *dt_w, *out_proj;
     void *dt_w_t;  // [d_inner][dt_rank] copy: the fused decode step (when dt_t_step) and the prefill dt_proj+softplus kernel read it
     int dt_t_step;
-    void *in_proj_t, *x_proj_t, *out_proj_t;  // [N][K] copies for the decode chain's own GEMM (null: library GEMM)
+    void *in_proj_t, *x_proj_t, *out_proj_t;  // [N][K] copies: in / out for every 16-bit engine (own GEMM and vendor GEMM read them), x for the own chain only
     int s4d;
 };
 
@@ -266,6 +266,7 @@ struct mrs_backbone {
     hipStream_t stream;
     rocblas_handle blas;
     GemmTuner *tuner;       // vendor-kernel choice for the prefill projections (off unless asked for)
+    TinyStepLayer *tiny_layers;   // small f32 models: the layer table of the single-launch step (null: kernel chains)
     std::vector<LayerDev> layers;
     float *input_proj_w, *input_proj_b, *norm_f;
     std::vector<void *> allocs;
@@ -337,8 +338,8 @@ static int gemm_rm(mrs_backbone *bb, int dtype, void *C, int ldc, const void *A,
     return gemm_ex_tuned(bb->tuner, bb->blas, bb->stream, 0, N, M, K, W, t, N, A, t, lda, C, t, ldc);
 }
 
-// The same product from the transposed copy Wt[N,K] (kept for the decode chain): the vendor kernels for this operand
-// order are faster at the prefill shapes (76 vs 84-92 us for in_proj at 16384 x 3072 x 768).
+// The same product from the transposed copy Wt[N,K]: the vendor kernels for this operand order are faster at the prefill
+// shapes (76 vs 84-92 us for in_proj at 16384 x 3072 x 768) and at decode row counts (128 x 2560 x 5120: 14.7 vs 46 us).
 static int gemm_rm_t(mrs_backbone *bb, int dtype, void *C, int ldc, const void *A, int lda, const void *Wt, int M, int N, int K) {
     const rocblas_datatype t = blas_type(dtype);
     return gemm_ex_tuned(bb->tuner, bb->blas, bb->stream, 1, N, M, K, Wt, t, K, A, t, lda, C, t, ldc);
@@ -622,6 +623,22 @@ extern "C" int mrs_backbone_create(mrs_backbone **out, int gpu_ordinal, const mr
         d.s4d = hflag;
     }
     MRS_CREATE_TRY(upload_f32(bb, &bb->norm_f, w->norm_f_weight, dm));
+    {
+        // small f32 models: a step is one launch (MRS_DECODE_NO_TINY=1 keeps the kernel chains)
+        const char *e = getenv("MRS_DECODE_NO_TINY");
+        if (!(e && atoi(e) != 0) && tiny_step_ok(dtype, input_dim, dm, di, ds, dc, dr, xd) && (!identity || input_dim == dm)) {
+            std::vector<TinyStepLayer> tl((size_t)L);
+            for (int l = 0; l < L; l++) {
+                const LayerDev &d = bb->layers[l];
+                tl[(size_t)l] = {d.norm_w, (const float *)d.in_proj, d.conv_w, d.conv_b, (const float *)d.x_proj, (const float *)d.dt_w, d.dt_b, d.a_neg,
+                                 d.D, (const float *)d.out_proj};
+            }
+            MRS_CREATE_TRY(dev_alloc(bb, (void **)&bb->tiny_layers, (size_t)L * sizeof(TinyStepLayer)));
+            hipError_t he = hipMemcpyAsync(bb->tiny_layers, tl.data(), (size_t)L * sizeof(TinyStepLayer), hipMemcpyHostToDevice, bb->stream);
+            if (he == hipSuccess) he = hipStreamSynchronize(bb->stream);   // tl leaves scope below
+            if (he != hipSuccess) { mrs_backbone_destroy(bb); return fail(MRS_E_HIP, "layer table upload: %s", hipGetErrorString(he)); }
+        }
+    }
     MRS_CREATE_TRY(dev_alloc(bb, (void **)&bb->conv_state, (size_t)L * batch * di * dc * 4));
     MRS_CREATE_TRY(dev_alloc(bb, (void **)&bb->ssm_state, (size_t)L * batch * di * ds * 4));
     MRS_CREATE_TRY(dev_alloc(bb, (void **)&bb->d_input, (size_t)batch * input_dim * 4));
@@ -659,6 +676,15 @@ extern "C" int mrs_backbone_reset(mrs_backbone *bb) {
 }
 
 static int step_body(mrs_backbone *bb) {
+    if (bb->tiny_layers) {
+        TinyStepArgs a = {};
+        a.layers = bb->tiny_layers; a.input = bb->d_input;
+        a.in_w = bb->identity_proj ? nullptr : bb->input_proj_w; a.in_b = bb->identity_proj ? nullptr : bb->input_proj_b;
+        a.norm_f = bb->norm_f; a.conv_state = bb->conv_state; a.ssm_state = bb->ssm_state; a.temporal = bb->temporal;
+        a.eps = bb->cfg.rms_norm_eps; a.n_layers = bb->cfg.n_layers; a.batch = bb->batch; a.input_dim = bb->input_dim;
+        a.dm = bb->cfg.d_model; a.di = bb->di; a.ds = bb->cfg.d_state; a.dc = bb->cfg.d_conv; a.dr = bb->dr; a.xd = bb->xd;
+        return launch_tiny_step(bb->stream, a);
+    }
     // identity projection on the own-GEMM chain: the first layer's prenorm kernel reads the input and writes the
     // residual stream itself, so no copy is needed
     bb->step_src = (bb->identity_proj && bb->skinny) ? bb->d_input : nullptr;

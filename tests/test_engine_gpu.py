@@ -387,3 +387,56 @@ def test_decode_above_the_own_chain_limit_runs_the_projections_from_the_transpos
             want = orc.m1_backbone_step(P, x[t, b], *st[b])
             assert cosine(got[b], want) >= 0.999, (t, b)
     eng.close()
+
+
+@pytest.mark.parametrize("shape", [
+    # d_model, d_state, d_conv, expand, layers, input_dim, batch
+    (128, 16, 4, 2, 3, 128, 1),      # the reference's default configuration
+    (128, 16, 4, 2, 2, 128, 128),    # ... at the published batch size
+    (64, 8, 2, 2, 2, 24, 5),         # input projection, short window, d_state 8
+    (256, 64, 4, 2, 2, 256, 3),      # dt_rank 16 (two rounds of dt weights), d_state 64: four passes of the scan step
+    (96, 4, 3, 1, 4, 40, 7),         # expand 1, d_state 4, odd sizes
+])
+def test_small_f32_models_step_in_one_launch(shape, monkeypatch):
+    """f32 engines with d_inner <= 512 run a backbone step as one kernel (one workgroup per batch row walks input
+    projection, every layer and the final norm).  Held to the CPU route step after step (outputs 1e-4 of their scale, conv window
+    and SSM state of every layer at the end), to the kernel chains it replaces (MRS_DECODE_NO_TINY=1 at creation), and
+    to itself: graph replays and a second engine give the same bits."""
+    dm, ds, dc, ex, L, idim, B = shape
+    cfg = MambaConfig(d_model=dm, d_state=ds, d_conv=dc, expand=ex, n_layers=L)
+    w = MambaWeights.init(cfg, idim, 7)
+    P = oracle_params(w, cfg, idim)
+    rng = np.random.default_rng(dm + B)
+    steps = 6
+    x = rng.standard_normal((steps, B, idim)).astype(np.float32)
+    rows = sorted({0, B // 2, B - 1})
+    st = {b: orc.m1_zero_state(P) for b in rows}
+    print(f"case one-launch step {shape}", flush=True)
+    eng = GpuMambaBackbone.new(0, w, cfg, idim, B)
+    outs = []
+    for t in range(steps):
+        if t == 3:
+            eng.capture_graph()
+        got = eng.step(x[t])
+        outs.append(got.copy())
+        for b in rows:
+            want = orc.m1_backbone_step(P, x[t, b], *st[b])
+            assert scaled_err(got[b], want) < 1e-4, (t, b)
+    for l in range(L):
+        conv, ssm = eng.download_state(l)
+        di = cfg.d_inner()
+        for b in rows:
+            # (the GPU keeps d_conv window slots, the CPU route d_conv - 1)
+            assert np.allclose(conv[b][:, 1:], st[b][0][l].reshape(di, dc - 1), atol=1e-5), (l, b)
+            assert scaled_err(ssm[b], st[b][1][l].reshape(di, ds)) < 1e-4, (l, b)
+    eng.close()
+    eng2 = GpuMambaBackbone.new(0, w, cfg, idim, B)
+    for t in range(steps):
+        assert np.array_equal(eng2.step(x[t]), outs[t]), t
+    eng2.close()
+    monkeypatch.setenv("MRS_DECODE_NO_TINY", "1")
+    print(f"case kernel chains {shape}", flush=True)
+    ref = GpuMambaBackbone.new(0, w, cfg, idim, B)
+    for t in range(steps):
+        assert scaled_err(ref.step(x[t]), outs[t]) < 1e-4, t
+    ref.close()
