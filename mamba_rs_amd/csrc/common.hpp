@@ -137,6 +137,20 @@ struct TinyStepArgs {
     float eps;
     int n_layers, batch, input_dim, dm, di, ds, dc, dr, xd;
 };
+// The same for the Mamba-3 SISO backbone (csrc/tiny_m3_step.hip): in_proj [dm][ip], out_proj [di][dm] row-major f32;
+// states as the engine holds them ([layer][batch]...).
+struct TinyM3StepLayer {
+    const float *norm_w, *in_proj, *dt_bias, *bnw, *cnw, *b_bias, *c_bias, *D, *ngw, *out_proj;
+};
+struct TinyM3StepArgs {
+    const TinyM3StepLayer *layers;
+    const float *input, *in_w, *in_b, *norm_f;
+    float *ssm, *kst, *vst, *angle, *temporal;
+    float eps, a_floor;
+    int n_layers, batch, input_dim, dm, di, nh, hd, ds, ng, nr, ip, outproj_norm;
+};
+bool tiny_m3_step_ok(int dtype, int input_dim, int dm, int di, int nh, int hd, int ds, int ng, int nr, int ip);
+int launch_tiny_m3_step(hipStream_t st, const TinyM3StepArgs &a);
 bool tiny_step_ok(int dtype, int input_dim, int dm, int di, int ds, int dc, int dr, int xd);
 int launch_tiny_step(hipStream_t st, const TinyStepArgs &a);
 bool dt_proj_softplus_ok(int dtype, int di, int dr, int64_t xs, const void *delta, const void *dt_in, const void *wt);

@@ -17,27 +17,12 @@
 #include "gemm_tune.hpp"
 #include <stdlib.h>
 #include "glue.hpp"
+#include "m3_math.hpp"
 #include <rocblas/rocblas.h>
 #include <new>
 #include <vector>
 
 namespace mrs {
-
-// a mod 2 pi in [0, 2 pi) (src/mamba3_siso/cpu/inference.rs:179-180 divides; an f64 division is a ~30-instruction
-// dependent sequence and this sits in a serial chain over time, so the quotient comes from the reciprocal and the
-// rare off-by-one of its floor is folded back).
-__device__ __forceinline__ double wrap_2pi(double a) {
-    const double two_pi = 6.283185307179586, inv_two_pi = 0.15915494309189535;
-    double r = fma(-two_pi, floor(a * inv_two_pi), a);
-    r = r < 0.0 ? r + two_pi : r;
-    return r >= two_pi ? r - two_pi : r;
-}
-
-
-constexpr float kPi = 3.14159265358979323846f;
-
-__device__ __forceinline__ float heavy_tail(float x) { return x >= 0.0f ? 1.0f + x : 1.0f / (1.0f - x); }
-__device__ __forceinline__ float sigmoidf_fast(float x) { return fast_rcp(1.0f + fast_exp2(-x * kLog2e)); }
 
 // One workgroup per (batch row, head); blockDim.x = hd * LG, LG = ds / 4 lanes per state row.
 // proj: [batch, ip] f32 = [z:di | x:di | B:ng*ds | C:ng*ds | dd_dt:nh | dd_A:nh | trap:nh | angles:nr]
@@ -574,6 +559,7 @@ struct mrs_m3_backbone {
     hipStream_t stream;
     rocblas_handle blas;
     GemmTuner *tuner;       // vendor-kernel choice for the prefill projections (off unless asked for)
+    TinyM3StepLayer *tiny_layers;   // small f32 models: the layer table of the single-launch step (null: kernel chains)
     std::vector<Layer3> layers;
     std::vector<void *> allocs;
     std::vector<void *> pf_allocs;   // the prefill scratch alone: released and re-made when the sequence length changes
@@ -645,6 +631,16 @@ int launch_layer_step_t(mrs_m3_backbone *bb, int l) {
 
 int step_body3(mrs_m3_backbone *bb) {
     const mrs_m3_config &c = bb->cfg;
+    if (bb->tiny_layers) {
+        TinyM3StepArgs a = {};
+        a.layers = bb->tiny_layers; a.input = bb->d_input;
+        a.in_w = bb->identity_proj ? nullptr : bb->input_proj_w; a.in_b = bb->identity_proj ? nullptr : bb->input_proj_b;
+        a.norm_f = bb->norm_f; a.ssm = bb->ssm; a.kst = bb->kst; a.vst = bb->vst; a.angle = bb->angle; a.temporal = bb->temporal;
+        a.eps = c.rms_norm_eps; a.a_floor = c.a_floor; a.n_layers = c.n_layers; a.batch = bb->batch; a.input_dim = bb->input_dim;
+        a.dm = c.d_model; a.di = bb->di; a.nh = bb->nh; a.hd = c.headdim; a.ds = c.d_state; a.ng = c.ngroups; a.nr = bb->nr; a.ip = bb->ip;
+        a.outproj_norm = c.is_outproj_norm;
+        return launch_tiny_m3_step(bb->stream, a);
+    }
     const int dm = c.d_model, di = bb->di, B = bb->batch, dt = bb->dtype, L = c.n_layers, ip = bb->ip;
     const int P = (dm + 15) / 16;
     // residual <- input (identity) or input . W + b
@@ -802,6 +798,21 @@ extern "C" int mrs_m3_backbone_create(mrs_m3_backbone **out, int gpu_ordinal, co
         }
     }
     MRS_CREATE_TRY(upload_f32_3(bb, &bb->norm_f, w->norm_f_weight, dm));
+    {
+        // small f32 models: a step is one launch (MRS_DECODE_NO_TINY=1 keeps the kernel chains)
+        const char *e = getenv("MRS_DECODE_NO_TINY");
+        if (!(e && atoi(e) != 0) && tiny_m3_step_ok(dtype, input_dim, dm, di, nh, cfg->headdim, ds, cfg->ngroups, bb->nr, ip)) {
+            std::vector<TinyM3StepLayer> tl((size_t)L);
+            for (int l = 0; l < L; l++) {
+                const Layer3 &d = bb->layers[l];
+                tl[(size_t)l] = {d.norm_w, (const float *)d.in_proj, d.dt_bias, d.bnw, d.cnw, d.b_bias, d.c_bias, d.D, d.ngw, (const float *)d.out_proj};
+            }
+            MRS_CREATE_TRY(dev_alloc3(bb, (void **)&bb->tiny_layers, (size_t)L * sizeof(TinyM3StepLayer)));
+            hipError_t he = hipMemcpyAsync(bb->tiny_layers, tl.data(), (size_t)L * sizeof(TinyM3StepLayer), hipMemcpyHostToDevice, bb->stream);
+            if (he == hipSuccess) he = hipStreamSynchronize(bb->stream);   // tl leaves scope below
+            if (he != hipSuccess) { mrs_m3_backbone_destroy(bb); return fail(MRS_E_HIP, "%s: layer table upload: %s", fn, hipGetErrorString(he)); }
+        }
+    }
     const size_t B = batch, hd = cfg->headdim, na = bb->nr > 0 ? bb->nr : 1, es = esize3(dtype);
     MRS_CREATE_TRY(dev_alloc3(bb, (void **)&bb->ssm, (size_t)L * B * nh * hd * ds * 4));
     MRS_CREATE_TRY(dev_alloc3(bb, (void **)&bb->kst, (size_t)L * B * nh * ds * 4));

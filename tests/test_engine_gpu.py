@@ -394,11 +394,12 @@ def test_decode_above_the_own_chain_limit_runs_the_projections_from_the_transpos
     (128, 16, 4, 2, 3, 128, 1),      # the reference's default configuration
     (128, 16, 4, 2, 2, 128, 128),    # ... at the published batch size
     (64, 8, 2, 2, 2, 24, 5),         # input projection, short window, d_state 8
-    (256, 64, 4, 2, 2, 256, 3),      # dt_rank 16 (two rounds of dt weights), d_state 64: four passes of the scan step
+    (128, 64, 4, 2, 2, 128, 3),      # d_state 64: eight passes of the scan step
+    (192, 16, 4, 1, 2, 192, 2),      # dt_rank 12: a second round of dt weights
     (96, 4, 3, 1, 4, 40, 7),         # expand 1, d_state 4, odd sizes
 ])
 def test_small_f32_models_step_in_one_launch(shape, monkeypatch):
-    """f32 engines with d_inner <= 512 run a backbone step as one kernel (one workgroup per batch row walks input
+    """Small f32 engines (every product at most three rounds of sixteen weight rows per lane) run a backbone step as one kernel (one workgroup per batch row walks input
     projection, every layer and the final norm).  Held to the CPU route step after step (outputs 1e-4 of their scale, conv window
     and SSM state of every layer at the end), to the kernel chains it replaces (MRS_DECODE_NO_TINY=1 at creation), and
     to itself: graph replays and a second engine give the same bits."""

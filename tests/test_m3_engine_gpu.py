@@ -272,3 +272,52 @@ def test_scan_that_forms_K_and_Q_itself_equals_the_separate_K_Q_pass(dtype, T, m
         assert np.max(np.abs(np.sin(fa[1][l][3]) - np.sin(se[1][l][3]))) < 0.2
     print("route difference: last", scaled_err(fa[0], se[0]), "layer-0 ssm", scaled_err(fa[1][0][0], se[1][0][0]),
           "top ssm", scaled_err(fa[1][-1][0], se[1][-1][0]), flush=True)
+
+
+@pytest.mark.parametrize("case", [
+    # config, input_dim, batch
+    (Mamba3Config(d_model=128, d_state=16, expand=2, headdim=16, ngroups=1, n_layers=4, rope_fraction=0.5, a_floor=1e-4), 128, 1),   # the reference's default
+    (Mamba3Config(d_model=128, d_state=16, expand=2, headdim=16, ngroups=1, n_layers=2, rope_fraction=0.5, a_floor=1e-4), 128, 128),
+    (Mamba3Config(d_model=64, d_state=32, expand=2, headdim=32, ngroups=2, n_layers=2, rope_fraction=1.0, is_outproj_norm=True), 24, 5),
+    (Mamba3Config(d_model=96, d_state=16, expand=2, headdim=16, ngroups=3, n_layers=3, rope_fraction=0.5), 40, 3),
+])
+def test_small_f32_models_step_in_one_launch(case, monkeypatch):
+    """f32 engines whose in_proj row is a multiple of four floats and fits in LDS run a backbone step as one kernel (one
+    workgroup per batch row).  Held to the CPU route step after step (outputs and every state of the last layer), to the
+    kernel chains it replaces (MRS_DECODE_NO_TINY=1 at creation), and to itself across graph replays and a second engine."""
+    cfg, idim, B = case
+    w = perturbed(cfg, idim, 11)
+    P = oracle_params(w, cfg, idim)
+    rng = np.random.default_rng(B + cfg.d_model)
+    steps = 24
+    x = rng.standard_normal((steps, B, idim)).astype(np.float32)
+    rows = sorted({0, B // 2, B - 1})
+    st = {b: P.zero_state() for b in rows}
+    print(f"case m3 one-launch step d_model={cfg.d_model} batch={B}", flush=True)
+    eng = GpuMamba3Backbone.new(0, w, cfg, idim, B)
+    outs = []
+    worst = 0.0
+    for t in range(steps):
+        if t == 8:
+            eng.capture_graph()
+        got = eng.step(x[t])
+        outs.append(got.copy())
+        for b in rows:
+            worst = max(worst, scaled_err(got[b], orc.m3_backbone_step(P, x[t, b], st[b])))
+    assert worst < 2e-4, worst
+    L = cfg.n_layers - 1
+    ssm, k, v, ang = eng.download_state(L)
+    for b in rows:
+        assert scaled_err(ssm[b], st[b][0][L]) < 2e-4 and scaled_err(k[b], st[b][1][L]) < 2e-4 and scaled_err(v[b], st[b][2][L]) < 2e-4, b
+        if cfg.num_rope_angles():
+            assert np.max(np.abs(np.sin(ang[b]) - np.sin(st[b][3][L]))) < 1e-3 and np.max(np.abs(np.cos(ang[b]) - np.cos(st[b][3][L]))) < 1e-3
+    eng.close()
+    eng2 = GpuMamba3Backbone.new(0, w, cfg, idim, B)
+    for t in range(steps):
+        assert np.array_equal(eng2.step(x[t]), outs[t]), t
+    eng2.close()
+    monkeypatch.setenv("MRS_DECODE_NO_TINY", "1")
+    ref = GpuMamba3Backbone.new(0, w, cfg, idim, B)
+    for t in range(steps):
+        assert scaled_err(ref.step(x[t]), outs[t]) < 2e-4, t
+    ref.close()
