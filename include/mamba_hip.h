@@ -294,6 +294,17 @@ MRS_API int mrs_backbone_prefill_device(mrs_backbone *bb, const float *input_dev
 MRS_API int mrs_backbone_set_gemm_tuning(mrs_backbone *bb, int on);
 /* temporal_ptr / input buffer / stream accessors (inference.rs:1717-1737) and state access for tests. */
 MRS_API float *mrs_backbone_temporal_ptr(mrs_backbone *bb);
+/* temporal_dtype (inference.rs:1720-1724): the dtype code of the buffer temporal_ptr returns.  This engine keeps that
+ * buffer in f32 for every storage type, so the answer is MRS_F32; a caller that binds temporal_ptr must ask, because
+ * the reference's mixed engine answers with its storage type. */
+MRS_API int mrs_backbone_temporal_dtype(mrs_backbone *bb);
+/* Which decode route the engine chose at creation (no counterpart in the reference; for tests and benchmarks that must
+ * know what they measured): a whole step in one launch (small f32 models), the library's own fused kernel chain, or
+ * the chain built on the vendor GEMM. */
+#define MRS_DECODE_LIBRARY_CHAIN 0
+#define MRS_DECODE_OWN_CHAIN 1
+#define MRS_DECODE_ONE_LAUNCH 2
+MRS_API int mrs_backbone_decode_route(mrs_backbone *bb);
 /* download_temporal (inference.rs:1727-1737): the last step's / prefill's final-norm rows [batch, d_model] to the host; synchronises. */
 MRS_API int mrs_backbone_download_temporal(mrs_backbone *bb, float *out);
 MRS_API float *mrs_backbone_input_ptr(mrs_backbone *bb);
@@ -418,6 +429,9 @@ MRS_API int mrs_m3_backbone_step_gpu_only(mrs_m3_backbone *bb);   /* input alrea
 MRS_API int mrs_m3_backbone_reset(mrs_m3_backbone *bb);
 MRS_API int mrs_m3_backbone_capture_graph(mrs_m3_backbone *bb);
 MRS_API float *mrs_m3_backbone_temporal_ptr(mrs_m3_backbone *bb);
+/* temporal_dtype (src/mamba3_siso/gpu/inference.rs:1561-1563) and the decode route, as for the Mamba-1 engine */
+MRS_API int mrs_m3_backbone_temporal_dtype(mrs_m3_backbone *bb);
+MRS_API int mrs_m3_backbone_decode_route(mrs_m3_backbone *bb);
 MRS_API float *mrs_m3_backbone_input_ptr(mrs_m3_backbone *bb);
 MRS_API void *mrs_m3_backbone_stream(mrs_m3_backbone *bb);
 MRS_API int mrs_m3_backbone_sync(mrs_m3_backbone *bb);

@@ -53,6 +53,8 @@ def _bind():
         "mrs_backbone_prefill_sequence": (c_int, [P, _FP, c_int, _FP]),
         "mrs_backbone_prefill_device": (c_int, [P, P, c_int]),
         "mrs_backbone_temporal_ptr": (P, [P]),
+        "mrs_backbone_temporal_dtype": (c_int, [P]),
+        "mrs_backbone_decode_route": (c_int, [P]),
         "mrs_backbone_download_temporal": (c_int, [P, _FP]),
         "mrs_backbone_set_gemm_tuning": (c_int, [P, c_int]),
         "mrs_backbone_input_ptr": (P, [P]),
@@ -214,7 +216,11 @@ class GpuMambaBackbone:
         return out
 
     def temporal_dtype(self) -> WeightDtype:
-        return WeightDtype.F32
+        return WeightDtype(_bind().mrs_backbone_temporal_dtype(self._h))
+
+    def decode_route(self) -> int:
+        """0: chain on the vendor GEMM, 1: the library's own fused chain, 2: a whole step in one launch."""
+        return _bind().mrs_backbone_decode_route(self._h)
 
     def input_ptr(self) -> int:
         return _bind().mrs_backbone_input_ptr(self._h)

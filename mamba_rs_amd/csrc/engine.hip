@@ -783,6 +783,12 @@ extern "C" int mrs_backbone_prefill_sequence(mrs_backbone *bb, const float *inpu
 
 extern "C" void *mrs_backbone_stream(mrs_backbone *bb) { return bb ? (void *)bb->stream : nullptr; }
 extern "C" float *mrs_backbone_temporal_ptr(mrs_backbone *bb) { return bb ? bb->temporal : nullptr; }
+// the buffer behind temporal_ptr is f32 whatever the storage type (the 16-bit copy the LM head reads is internal)
+extern "C" int mrs_backbone_temporal_dtype(mrs_backbone *bb) { return bb ? MRS_F32 : -1; }
+extern "C" int mrs_backbone_decode_route(mrs_backbone *bb) {
+    if (!bb) return -1;
+    return bb->tiny_layers ? MRS_DECODE_ONE_LAUNCH : bb->skinny ? MRS_DECODE_OWN_CHAIN : MRS_DECODE_LIBRARY_CHAIN;
+}
 extern "C" int mrs_backbone_download_temporal(mrs_backbone *bb, float *out) {
     if (!bb || !out) return fail(MRS_E_NULL, "mrs_backbone_download_temporal: null pointer");
     MRS_HIP(hipMemcpyAsync(out, bb->temporal, (size_t)bb->batch * bb->cfg.d_model * 4, hipMemcpyDeviceToHost, bb->stream));

@@ -924,16 +924,19 @@ extern "C" int mrs_ssm_scan_fwd_static(void *stream, int dtype, float *h, void *
                                        const float *a_neg, const float *D, const void *gate, int64_t gate_stride,
                                        unsigned flags, int batch, int T, int d_inner, int d_state) {
     const char *fn = "mrs_ssm_scan_fwd_static";
-    // the size test comes first and touches no GPU: a shape whose chunk summaries do not fit is refused, never shrunk
+    // argument checks and the size test come first and touch no GPU: a shape whose chunk summaries do not fit is refused,
+    // never shrunk
+    int rc = scan_check(fn, dtype, h, y, delta, u, B, C, a_neg, D, bc_stride, batch, T, d_inner, d_state);
+    if (rc) return rc;
     const size_t need = mrs_ssm_scan_workspace_bytes(batch, T, d_inner, d_state);
     if (need > kStaticScanScratchBytes)
         return fail(MRS_E_WORKSPACE, "%s: this shape needs %zu bytes of chunk summaries, the built-in buffer holds %zu; use mrs_ssm_scan_fwd_ex with a workspace",
                     fn, need, kStaticScanScratchBytes);
     void *ws = nullptr;
-    int rc = static_scratch_for_current_device(fn, &ws);
+    rc = static_scratch_for_current_device(fn, &ws);
     if (rc) return rc;
     // Every float the second pass reads from the buffer is written by the first pass of the same call (chunk states,
-    // step sums, the copy of h, the regrouped B and widened C rows), so nothing has to start at zero.
+    // step sums, the copy of h), so nothing has to start at zero.
     return scan_dispatch(fn, stream, dtype, h, y, delta, u, B, C, bc_stride, a_neg, D, gate, gate_stride, flags, ws,
                          kStaticScanScratchBytes, batch, T, d_inner, d_state);
 }

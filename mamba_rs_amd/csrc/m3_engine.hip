@@ -1137,6 +1137,11 @@ extern "C" int mrs_m3_backbone_prefill_sequence(mrs_m3_backbone *bb, const float
 extern "C" float *mrs_m3_backbone_prefill_input_ptr(mrs_m3_backbone *bb) { return bb ? bb->pf_in : nullptr; }
 
 extern "C" float *mrs_m3_backbone_temporal_ptr(mrs_m3_backbone *bb) { return bb ? bb->temporal : nullptr; }
+extern "C" int mrs_m3_backbone_temporal_dtype(mrs_m3_backbone *bb) { return bb ? MRS_F32 : -1; }
+extern "C" int mrs_m3_backbone_decode_route(mrs_m3_backbone *bb) {
+    if (!bb) return -1;
+    return bb->tiny_layers ? MRS_DECODE_ONE_LAUNCH : bb->skinny ? MRS_DECODE_OWN_CHAIN : MRS_DECODE_LIBRARY_CHAIN;
+}
 extern "C" float *mrs_m3_backbone_input_ptr(mrs_m3_backbone *bb) { return bb ? bb->d_input : nullptr; }
 extern "C" void *mrs_m3_backbone_stream(mrs_m3_backbone *bb) { return bb ? (void *)bb->stream : nullptr; }
 extern "C" int mrs_m3_backbone_sync(mrs_m3_backbone *bb) {

@@ -15,16 +15,16 @@ namespace {
 __global__ __launch_bounds__(kTinyThreads) void tiny_m3_backbone_step_kernel(TinyM3StepArgs a) {
     extern __shared__ float lds[];
     const int dm = a.dm, di = a.di, nh = a.nh, hd = a.hd, ds = a.ds, ng = a.ng, nr = a.nr, ip = a.ip;
-    const int xin_n = a.input_dim > dm ? a.input_dim : dm;
+    const int xin_n = rup4(a.input_dim > dm ? a.input_dim : dm), di4 = rup4(di);
     float *res = lds;                   // [dm]       residual stream of this row
-    float *xin = res + dm;              // [max(dm, input_dim)] operand of the product in flight
+    float *xin = res + rup4(dm);        // [max(dm, input_dim)] operand of the product in flight
     float *proj = xin + xin_n;          // [ip]       in_proj output: z | x | B | C | dd_dt | dd_A | trap | angles
-    float *kl = proj + ip;              // [nh ds]    K of every head (normalised, biased, rotated B)
-    float *ql = kl + nh * ds;           // [nh ds]    Q of every head
-    float *yr = ql + nh * ds;           // [di]       y before the gate
-    float *yg = yr + di;                // [di]       gated y: out_proj's operand
-    float *ginv = yg + di;              // [2 ng]     1 / rms of the raw B and C rows per group
-    float *part = ginv + ((2 * ng + 3) & ~3);   // [kTinyPart]
+    float *kl = proj + rup4(ip);        // [nh ds]    K of every head (normalised, biased, rotated B)
+    float *ql = kl + rup4(nh * ds);     // [nh ds]    Q of every head
+    float *yr = ql + rup4(nh * ds);     // [di]       y before the gate
+    float *yg = yr + di4;               // [di]       gated y: out_proj's operand
+    float *ginv = yg + di4;             // [2 ng]     1 / rms of the raw B and C rows per group
+    float *part = ginv + rup4(2 * ng);  // [kTinyPart]
     float *red = part + kTinyPart;      // [waves]
     const int tid = threadIdx.x, b = blockIdx.x;
     const int lg = ds >> 2, per_head = hd * lg, tasks = nh * per_head;   // one lane-task per float4 of SSM state
@@ -148,8 +148,8 @@ __global__ __launch_bounds__(kTinyThreads) void tiny_m3_backbone_step_kernel(Tin
 }
 
 size_t tiny_m3_lds_bytes(int input_dim, int dm, int di, int nh, int ds, int ng, int ip) {
-    const int xin_n = input_dim > dm ? input_dim : dm;
-    return sizeof(float) * ((size_t)dm + xin_n + ip + 2 * (size_t)nh * ds + 2 * (size_t)di + ((2 * ng + 3) & ~3) + kTinyPart + kTinyThreads / 64);
+    const int xin_n = rup4(input_dim > dm ? input_dim : dm);
+    return sizeof(float) * ((size_t)rup4(dm) + xin_n + rup4(ip) + 2 * (size_t)rup4(nh * ds) + 2 * (size_t)rup4(di) + rup4(2 * ng) + kTinyPart + kTinyThreads / 64);
 }
 
 }  // namespace

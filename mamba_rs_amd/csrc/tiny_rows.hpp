@@ -11,6 +11,11 @@ constexpr int kTinyPre = 2;          // passes of the scan step whose state is r
 constexpr int kTinySlices = 16;      // most k slices per product (their partial sums are added serially)
 constexpr int kTinyPart = 2048;      // floats of k-slice partial sums: (N / 4 column quads) x (k slices) <= 512 threads x 4
 
+// Every array carved out of the workgroup's LDS starts on a 16-byte boundary: some of them (the partial sums, K and Q of the
+// Mamba-3 step) are read and written as float4, and an array in front of them whose length is not a multiple of four
+// floats (an input row wider than d_model, an odd d_inner) would otherwise shift them off it.
+__host__ __device__ constexpr int rup4(int n) { return (n + 3) & ~3; }
+
 // out[n] = bias[n] + sum_k x[k] W[k][n] for n < N; W row-major [K][N] in global memory, x and out in LDS, N % 4 == 0 and
 // N <= 2048.  A thread owns four consecutive columns over one slice of K (16-byte weight loads, consecutive lanes on
 // consecutive quads, sixteen rows requested before the first multiply-add); the slices' partial sums meet in LDS and are

@@ -16,15 +16,15 @@ namespace {
 __global__ __launch_bounds__(kTinyThreads) void tiny_backbone_step_kernel(TinyStepArgs a) {
     extern __shared__ float lds[];
     const int dm = a.dm, di = a.di, ds = a.ds, dc = a.dc, dr = a.dr, xd = a.xd;
-    const int xin_n = a.input_dim > dm ? a.input_dim : dm;
+    const int xin_n = rup4(a.input_dim > dm ? a.input_dim : dm), di4 = rup4(di);
     float *res = lds;                   // [dm]      residual stream of this row
-    float *xin = res + dm;              // [max(dm, input_dim)] operand of the product in flight (input row, normed row)
+    float *xin = res + rup4(dm);        // [max(dm, input_dim)] operand of the product in flight (input row, normed row)
     float *proj = xin + xin_n;          // [2 di]    in_proj output: x half, gate half
-    float *u = proj + 2 * di;           // [di]      conv + SiLU output
-    float *dl = u + di;                 // [di]      delta
-    float *y = dl + di;                 // [di]      gated scan output
-    float *xdbl = y + di;               // [xd]      x_proj output: dt input, B, C
-    float *part = xdbl + ((xd + 3) & ~3);   // [kTinyPart]
+    float *u = proj + rup4(2 * di);     // [di]      conv + SiLU output
+    float *dl = u + di4;                // [di]      delta
+    float *y = dl + di4;                // [di]      gated scan output
+    float *xdbl = y + di4;              // [xd]      x_proj output: dt input, B, C
+    float *part = xdbl + rup4(xd);      // [kTinyPart]
     float *red = part + kTinyPart;      // [waves]
     const int tid = threadIdx.x, b = blockIdx.x;
     const int lg = ds >> 2, rows_pp = kTinyThreads / lg;   // scan step: ds / 4 lanes per channel, one float4 of state each
@@ -155,8 +155,8 @@ __global__ __launch_bounds__(kTinyThreads) void tiny_backbone_step_kernel(TinySt
 }
 
 size_t tiny_lds_bytes(const TinyStepArgs &a) {
-    const int xin_n = a.input_dim > a.dm ? a.input_dim : a.dm;
-    return sizeof(float) * ((size_t)a.dm + xin_n + 2 * (size_t)a.di + 3 * (size_t)a.di + ((a.xd + 3) & ~3) + kTinyPart + kTinyThreads / 64);
+    const int xin_n = rup4(a.input_dim > a.dm ? a.input_dim : a.dm);
+    return sizeof(float) * ((size_t)rup4(a.dm) + xin_n + rup4(2 * a.di) + 3 * (size_t)rup4(a.di) + rup4(a.xd) + kTinyPart + kTinyThreads / 64);
 }
 
 }  // namespace
@@ -166,7 +166,7 @@ bool tiny_step_ok(int dtype, int input_dim, int dm, int di, int ds, int dc, int 
     if (sweep_rounds(input_dim, dm) > kTinyMaxRounds || sweep_rounds(dm, 2 * di) > kTinyMaxRounds || sweep_rounds(di, xd) > kTinyMaxRounds ||
         sweep_rounds(di, dm) > kTinyMaxRounds)
         return false;
-    return dtype == MRS_F32 && dm >= 4 && dm % 4 == 0 && dm <= 1024 && di % 2 == 0 && di >= 2 && di <= 512 && xd % 4 == 0 && xd >= 4 &&
+    return dtype == MRS_F32 && dm >= 4 && dm % 4 == 0 && dm <= 1024 && di % 4 == 0 && di >= 4 && di <= 512 && xd % 4 == 0 && xd >= 4 &&
            xd <= 1024 && (ds == 4 || ds == 8 || ds == 16 || ds == 32 || ds == 64) && dc >= 1 && dc <= 8 && dr >= 1 && input_dim >= 1 &&
            input_dim <= 4096 && xd == dr + 2 * ds;
 }

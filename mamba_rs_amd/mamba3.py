@@ -196,6 +196,8 @@ def _bind():
         "mrs_m3_backbone_reset": (c_int, [P]),
         "mrs_m3_backbone_capture_graph": (c_int, [P]),
         "mrs_m3_backbone_temporal_ptr": (P, [P]),
+        "mrs_m3_backbone_temporal_dtype": (c_int, [P]),
+        "mrs_m3_backbone_decode_route": (c_int, [P]),
         "mrs_m3_backbone_input_ptr": (P, [P]),
         "mrs_m3_backbone_stream": (P, [P]),
         "mrs_m3_backbone_sync": (c_int, [P]),
@@ -316,6 +318,13 @@ class GpuMamba3Backbone:
 
     def temporal_ptr(self) -> int:
         return _bind().mrs_m3_backbone_temporal_ptr(self._h)
+
+    def temporal_dtype(self) -> WeightDtype:
+        return WeightDtype(_bind().mrs_m3_backbone_temporal_dtype(self._h))
+
+    def decode_route(self) -> int:
+        """0: chain on the vendor GEMM, 1: the library's own fused chain, 2: a whole step in one launch."""
+        return _bind().mrs_m3_backbone_decode_route(self._h)
 
     def input_ptr(self) -> int:
         return _bind().mrs_m3_backbone_input_ptr(self._h)

@@ -193,19 +193,22 @@ def test_28b_shape_decode_follows_the_cpu_route(w28, B):
     eng.close()
 
 
-def test_28b_shape_prefill_follows_the_cpu_route(w28):
-    """4 x 512 through the 2.8b-shape layers (T-split scan at d_inner 5120 = 80 channel tiles, dt_proj with K = 160):
-    rows 0 and 3 against the CPU prefill, then the hand-off step."""
+@pytest.mark.parametrize("T", [512, 4096])
+def test_28b_shape_prefill_follows_the_cpu_route(w28, T):
+    """4 x 512 and 4 x 4096 (the benchmarked prefill: a scan plan of nine chunks of 464 steps) through the 2.8b-shape
+    layers (T-split scan at d_inner 5120 = 80 channel tiles, dt_proj with K = 160): rows 0 and 3 against the CPU
+    prefill, then the hand-off step."""
     w, P = w28
-    B, T = 4, 512
-    print("case 2.8b-shape prefill 4 x 512", flush=True)
+    B = 4
+    print(f"case 2.8b-shape prefill 4 x {T}", flush=True)
     eng = GpuMambaBackbone.new_with_dtype(0, w, CFG_28B, 2560, B, WeightDtype.BF16)
-    rng = np.random.default_rng(29)
+    rng = np.random.default_rng(29 + T)
     x = orc.round_to(rng.standard_normal((B, T + 1, 2560)).astype(np.float32), orc.BF16)
     last = eng.prefill_sequence(x[:, :T])
     state = eng.download_state(1)[1]
     nxt = eng.step(x[:, T])
     for b in (0, 3):
+        print(f"  CPU route, row {b}", flush=True)
         conv, ssm = orc.m1_zero_state(P)
         ref = orc.m1_backbone_prefill(P, x[b, :T], conv, ssm, identity_proj=True)
         assert cosine(last[b], ref[-1]) >= COS, (b, cosine(last[b], ref[-1]))

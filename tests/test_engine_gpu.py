@@ -396,7 +396,10 @@ def test_decode_above_the_own_chain_limit_runs_the_projections_from_the_transpos
     (64, 8, 2, 2, 2, 24, 5),         # input projection, short window, d_state 8
     (128, 64, 4, 2, 2, 128, 3),      # d_state 64: eight passes of the scan step
     (192, 16, 4, 1, 2, 192, 2),      # dt_rank 12: a second round of dt weights
-    (96, 4, 3, 1, 4, 40, 7),         # expand 1, d_state 4, odd sizes
+    (128, 4, 3, 1, 4, 40, 7),        # expand 1, d_state 4 (one pass of 512 rows), dt_rank 8, x_proj row of 16
+    (128, 16, 4, 2, 2, 130, 3),      # input row wider than d_model and not a multiple of four floats
+    (64, 8, 4, 3, 2, 64, 2),         # expand 3
+    (36, 16, 2, 3, 2, 36, 2),        # dt_rank 3: an x_proj row of 35 floats is outside the route, kernel chains on both sides
 ])
 def test_small_f32_models_step_in_one_launch(shape, monkeypatch):
     """Small f32 engines (every product at most three rounds of sixteen weight rows per lane) run a backbone step as one kernel (one workgroup per batch row walks input
@@ -414,6 +417,9 @@ def test_small_f32_models_step_in_one_launch(shape, monkeypatch):
     st = {b: orc.m1_zero_state(P) for b in rows}
     print(f"case one-launch step {shape}", flush=True)
     eng = GpuMambaBackbone.new(0, w, cfg, idim, B)
+    xd = cfg.dt_rank() + 2 * ds
+    assert (eng.decode_route() == 2) == (xd % 4 == 0), (shape, eng.decode_route())   # 2 = the whole step in one launch
+    assert eng.temporal_dtype() == WeightDtype.F32
     outs = []
     for t in range(steps):
         if t == 3:
@@ -438,6 +444,7 @@ def test_small_f32_models_step_in_one_launch(shape, monkeypatch):
     monkeypatch.setenv("MRS_DECODE_NO_TINY", "1")
     print(f"case kernel chains {shape}", flush=True)
     ref = GpuMambaBackbone.new(0, w, cfg, idim, B)
+    assert ref.decode_route() != 2
     for t in range(steps):
         assert scaled_err(ref.step(x[t]), outs[t]) < 1e-4, t
     ref.close()

@@ -163,15 +163,19 @@ def test_scan_reads_b_c_in_place_from_xdbl(dtype):
     assert_close(h, h_ref, orc.F32, "h")
 
 
-def test_scan_full_size_channel_subset_and_linearity():
-    """The isolated-scan workload (B=8, T=2048, d_inner=1536, d_state=16, bf16, gated):
-    channels are independent, so the oracle is run on a subset of channels of the
-    full-size launch, once per A route; plus linearity in u (h0 = 0, f32 state): scan(2u) = 2 scan(u) exactly."""
-    rng = np.random.default_rng(4)
-    batch, T, di, ds = 8, 2048, 1536, 16
+@pytest.mark.parametrize("shape", [(8, 2048, 1536), (4, 4096, 5120)])
+def test_scan_full_size_channel_subset_and_linearity(shape):
+    """The isolated-scan workload (B=8, T=2048, d_inner=1536, d_state=16, bf16, gated) and the scan of a 2.8b-shape
+    prefill layer (4 x 4096 x 5120: nine chunks of 464 steps over 80 channel tiles): channels are independent, so the
+    oracle is run on a subset of channels of the full-size launch, once per A route; plus linearity in u (h0 = 0, f32
+    state): scan(2u) = 2 scan(u) exactly."""
+    batch, T, di = shape
+    ds = 16
+    rng = np.random.default_rng(4 + di)
+    print(f"case full-size scan {batch} x {T} x {di}", flush=True)
     inp = quantised(rng, batch, T, di, ds, orc.BF16)
     h0 = np.zeros((batch, di, ds), np.float32)
-    sel = np.sort(rng.choice(di, 48, replace=False))
+    sel = np.sort(rng.choice(di, 48 if di == 1536 else 24, replace=False))
     sub = dict(delta=inp["delta"][:, :, sel], u=inp["u"][:, :, sel], z=inp["z"][:, :, sel], B=inp["B"], C=inp["C"],
                a_neg=inp["a_neg"][sel], D=inp["D"][sel])
     y_ref, h_ref = orc.m1_scan_f64(h0[:, sel], sub["delta"], sub["u"], sub["B"], sub["C"], sub["a_neg"], sub["D"],

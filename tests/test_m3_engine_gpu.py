@@ -280,6 +280,7 @@ def test_scan_that_forms_K_and_Q_itself_equals_the_separate_K_Q_pass(dtype, T, m
     (Mamba3Config(d_model=128, d_state=16, expand=2, headdim=16, ngroups=1, n_layers=2, rope_fraction=0.5, a_floor=1e-4), 128, 128),
     (Mamba3Config(d_model=64, d_state=32, expand=2, headdim=32, ngroups=2, n_layers=2, rope_fraction=1.0, is_outproj_norm=True), 24, 5),
     (Mamba3Config(d_model=96, d_state=16, expand=2, headdim=16, ngroups=3, n_layers=3, rope_fraction=0.5), 40, 3),
+    (Mamba3Config(d_model=128, d_state=16, expand=2, headdim=16, ngroups=1, n_layers=2, rope_fraction=0.5, a_floor=1e-4), 130, 3),   # input row wider than d_model, 2 mod 4
 ])
 def test_small_f32_models_step_in_one_launch(case, monkeypatch):
     """f32 engines whose in_proj row is a multiple of four floats and fits in LDS run a backbone step as one kernel (one
@@ -295,6 +296,7 @@ def test_small_f32_models_step_in_one_launch(case, monkeypatch):
     st = {b: P.zero_state() for b in rows}
     print(f"case m3 one-launch step d_model={cfg.d_model} batch={B}", flush=True)
     eng = GpuMamba3Backbone.new(0, w, cfg, idim, B)
+    assert eng.decode_route() == 2, eng.decode_route()   # the whole step in one launch
     outs = []
     worst = 0.0
     for t in range(steps):
@@ -318,6 +320,7 @@ def test_small_f32_models_step_in_one_launch(case, monkeypatch):
     eng2.close()
     monkeypatch.setenv("MRS_DECODE_NO_TINY", "1")
     ref = GpuMamba3Backbone.new(0, w, cfg, idim, B)
+    assert ref.decode_route() != 2
     for t in range(steps):
         assert scaled_err(ref.step(x[t]), outs[t]) < 2e-4, t
     ref.close()

@@ -56,10 +56,11 @@ def test_static_scratch_scan_equals_the_workspace_scan_on_two_calls_in_a_row():
     assert abs(torch.cuda.mem_get_info()[0] - free0) < (12 << 20)
 
 
-def test_static_scratch_scan_at_the_benchmark_shape():
+@pytest.mark.parametrize("shape", [(8, 2048, 1536), (4, 4096, 5120)])
+def test_static_scratch_scan_at_the_benchmark_shapes(shape):
     rng = np.random.default_rng(71)
-    print("case static scan: 8 x 2048 x 1536 bf16 gated (bit-equality only)", flush=True)
-    run_both(rng, 8, 2048, 1536, orc.BF16, True, check_oracle=False)
+    print(f"case static scan: {shape} bf16 gated (bit-equality only)", flush=True)
+    run_both(rng, *shape, orc.BF16, True, check_oracle=False)
 
 
 def test_static_scratch_scan_refuses_shapes_beyond_its_buffer():
