@@ -22,24 +22,34 @@ HBM_PEAK_GBPS = 8000.0
 SCAN_PROFILE = os.path.join(ROOT, "profiles", "m1_scan_c2_bf16.md")
 
 
-def profiled_scan_traffic():
-    """HBM bytes per scan call (both kernels) as the committed rocprofv3 FETCH_SIZE / WRITE_SIZE summary states them
-    (a line `traffic_bytes_per_call: N` and one `kernels_sha16: X` naming the kernel source it was taken from).  A counter
-    run cannot share a process with the timed run, so the figure is read, not measured here; it is reported as null when
-    the kernel source has changed since the profile was taken."""
+def profile_figures(profile, source, keys):
+    """Figures a committed rocprofv3 summary states in machine-readable lines (`key: number`), together with the hash of
+    the kernel source they were taken from (`kernels_sha16: X`).  Counter runs cannot share a process with the timed
+    run, so these are read, not measured here; every figure is None when the kernel source has changed since."""
     import hashlib
     import re
+    path = os.path.join(ROOT, "profiles", profile)
     try:
-        text = open(SCAN_PROFILE).read()
-        n = int(re.search(r"^traffic_bytes_per_call:\s*(\d+)", text, re.M).group(1))
+        text = open(path).read()
         sha = re.search(r"^kernels_sha16:\s*([0-9a-f]{16})", text, re.M).group(1)
-    except (OSError, AttributeError, ValueError):
-        return None, "no profile"
-    src = os.path.join(ROOT, "mamba_rs_amd", "csrc", "m1_scan.hip")
-    now = hashlib.sha256(open(src, "rb").read()).hexdigest()[:16]
+    except (OSError, AttributeError):
+        return {k: None for k in keys}, "no profile"
+    now = hashlib.sha256(open(os.path.join(ROOT, "mamba_rs_amd", "csrc", source), "rb").read()).hexdigest()[:16]
     if now != sha:
-        return None, f"stale: profile taken from m1_scan.hip {sha}, source is {now}"
-    return n, "profiles/m1_scan_c2_bf16.md"
+        return {k: None for k in keys}, f"stale: profile taken from {source} {sha}, source is {now}"
+    out = {}
+    for k in keys:
+        m = re.search(r"^" + re.escape(k) + r":\s*([0-9.eE+-]+)", text, re.M)
+        out[k] = float(m.group(1)) if m else None
+    return out, "profiles/" + profile
+
+
+def profiled_scan_traffic():
+    """HBM bytes per scan call (both kernels) from the FETCH_SIZE / WRITE_SIZE summary, and the instruction-issue time
+    of the call from the instruction counters of the same file."""
+    f, src = profile_figures("m1_scan_c2_bf16.md", "m1_scan.hip", ["traffic_bytes_per_call", "issue_bound_us_per_call"])
+    n = f["traffic_bytes_per_call"]
+    return (int(n) if n is not None else None), f["issue_bound_us_per_call"], src
 
 
 def scan_algorithmic_bytes(batch, T, di, ds, s, gated=True):
@@ -166,6 +176,49 @@ def cpu_prefill_sample(cfg_kw, sample_layers, sample_tokens, full_tokens, seed=4
 
 
 DEFAULT_LEGS = "c1,lm,lm28,published,m1_kernels,m3,m3_engine"
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+
+
+def m1_step_bytes(cfg, B, es, vocab=0):
+    """Algorithmic bytes of one decode step of a Mamba-1 backbone: every layer's weights once, conv and SSM state read
+    and written, the residual row; plus the tied head's table when a vocabulary is given."""
+    dm, di, ds, dc, dr = cfg.d_model, cfg.d_inner(), cfg.d_state, cfg.d_conv, cfg.dt_rank()
+    layer = es * (dm * 2 * di + di * (dr + 2 * ds) + dr * di + di * dm) + 2 * 4 * B * di * (ds + dc) + 2 * 4 * B * dm
+    return cfg.n_layers * layer + ((vocab + 63) // 64 * 64) * dm * es
+
+
+def m3_step_bytes(cfg, B, es):
+    dm, di, nh, hd, ds, ip = cfg.d_model, cfg.d_inner(), cfg.nheads(), cfg.headdim, cfg.d_state, cfg.in_proj_out_dim()
+    return cfg.n_layers * (es * (dm * ip + di * dm) + 2 * 4 * B * nh * (hd * ds + ds + hd) + 2 * 4 * B * dm)
+
+
+def m3_prefill_roofline(cfg, batch, T, seconds, es=2):
+    """A Mamba-3 prefill against the two rooflines: the chunked scan's bytes per layer (x, Q, K read + y written + the
+    step scalars) and the matrix work (two projections + the scan's four contractions per chunk)."""
+    M = batch * T
+    dm, di, nh, hd, ds, ip = cfg.d_model, cfg.d_inner(), cfg.nheads(), cfg.headdim, cfg.d_state, cfg.in_proj_out_dim()
+    nbytes = (4 * M * di * es + 12 * M * nh) * cfg.n_layers
+    flops = (2.0 * M * (dm * ip + di * dm) + 4 * 2.0 * 64 * hd * ds * (M // 64) * nh) * cfg.n_layers
+    return {"scan_algorithmic_bytes": nbytes, "hbm_frac": nbytes / seconds / 1e9 / HBM_PEAK_GBPS,
+            "matrix_flop": flops, "mfma_frac": flops / seconds / 1e12 / MFMA_BF16_PEAK_TFLOPS}
+
+
+def m1_prefill_roofline(cfg, batch, T, seconds, es=2):
+    """A Mamba-1 prefill against the two rooflines: the bytes its own streaming kernels must move per layer (selective
+    scan with the gate read, conv1d + SiLU: delta,u,z read + y written + B,C + state; x read + u written + window) and
+    the matrix work of its four projections (2 M N K each, bf16 operands, f32 sums)."""
+    M = batch * T
+    dm, di, ds, dc, dr = cfg.d_model, cfg.d_inner(), cfg.d_state, cfg.d_conv, cfg.dt_rank()
+    xd = dr + 2 * ds
+    scan = scan_algorithmic_bytes(batch, T, di, ds, es, gated=True)
+    conv = 2 * M * di * es + 2 * 4 * batch * di * dc + 4 * di * (dc + 1)
+    flops = 2.0 * M * (dm * 2 * di + di * xd + dr * di + di * dm) * cfg.n_layers
+    nbytes = (scan + conv) * cfg.n_layers
+    return {"scan_conv_algorithmic_bytes": nbytes, "hbm_frac": nbytes / seconds / 1e9 / HBM_PEAK_GBPS,
+            "gemm_flop": flops, "mfma_frac": flops / seconds / 1e12 / MFMA_BF16_PEAK_TFLOPS,
+            "note": "hbm_frac: bytes of the scan and conv kernels of every layer / whole prefill time / 8 TB/s; mfma_frac: "
+                    "projection flops / whole prefill time / 2.5 PFLOP/s (dense bf16); each is a share of one prefill that "
+                    "does both kinds of work in sequence"}
 
 
 def lm_leg(name, cfg_kw, vocab, prefill_bt, decode_b, decode_steps, seed=42, shared_layer=False, cpu_sample=None,
@@ -212,6 +265,7 @@ def lm_leg(name, cfg_kw, vocab, prefill_bt, decode_b, decode_steps, seed=42, sha
         tt = sorted(times)[1]
         out["prefill"] = {"batch": pb, "seq_len": pt, "ms": tt * 1e3, "tok_per_s": pb * pt / tt, "vendor_gemm_kernels": "timed once, fastest kept",
                           "tuning_s": tune_s, "ms_with_default_vendor_kernels": tp * 1e3}
+    out["prefill"]["roofline"] = m1_prefill_roofline(cfg, pb, pt, out["prefill"]["ms"] * 1e-3)
     lm_p.close(); pre.close()
     if cpu_sample:
         out["cpu_port_prefill"] = cpu_prefill_sample(cfg_kw, cpu_sample[0], cpu_sample[1], pb * pt, seed)
@@ -242,10 +296,7 @@ def lm_leg(name, cfg_kw, vocab, prefill_bt, decode_b, decode_steps, seed=42, sha
         dec, lm_d, td = timed_decode(tune_decode)
         tk = lm_d.get_tokens()
         assert ((tk >= 0) & (tk < vocab)).all()
-        es = 2
-        di, dm, ds, dc, dr = cfg.d_inner(), cfg.d_model, cfg.d_state, cfg.d_conv, cfg.dt_rank()
-        layer_bytes = es * (dm * 2 * di + di * (dr + 2 * ds) + dr * di + di * dm) + 2 * 4 * db * di * (ds + dc) + 2 * 4 * db * dm
-        step_bytes = cfg.n_layers * layer_bytes + ((vocab + 63) // 64 * 64) * dm * es
+        step_bytes = m1_step_bytes(cfg, db, 2, vocab)
         entry = {"batch": db, "steps": decode_steps, "us_per_step": td * 1e6, "tok_per_s": db / td,
                  "algorithmic_bytes_per_step": step_bytes, "hbm_frac": step_bytes / td / 1e9 / HBM_PEAK_GBPS}
         if td_default is not None:
@@ -262,7 +313,8 @@ def lm_leg(name, cfg_kw, vocab, prefill_bt, decode_b, decode_steps, seed=42, sha
             t0 = time.perf_counter(); gen = lm_d.generate_batch(prompts, params); tg = time.perf_counter() - t0
             n_gen = sum(len(g) for g in gen)
             entry["generate_batch"] = {"sampler": "temperature 0.8, top_k 50, top_p 0.9", "new_tokens": n_gen, "ms": tg * 1e3,
-                                       "us_per_step": tg / (12 + 128) * 1e6, "gen_tok_per_s": n_gen / tg}
+                                       "us_per_step": tg / (12 + 128) * 1e6, "gen_tok_per_s": n_gen / tg,
+                                       "hbm_frac": step_bytes / (tg / (12 + 128)) / 1e9 / HBM_PEAK_GBPS}
         dec_out.append(entry)
         lm_d.close(); dec.close()
     out["decode"] = dec_out
@@ -310,8 +362,13 @@ def c1_leg():
         orc.m1_backbone_step(P, x[0, t], cs, ss)
     tcs = (time.perf_counter() - t0) / 64
     eng.close()
+    roof = m1_prefill_roofline(cfg, 1, T, tp, es=4)
+    roof["mfma_frac"] = None     # f32 projections do not run on the bf16 matrix path
+    dm, di, ds, dc, dr = 128, 256, 16, 4, 8
+    step_bytes = 2 * (4 * (dm * 2 * di + di * (dr + 2 * ds) + dr * di + di * dm) + 2 * 4 * di * (ds + dc) + 2 * 4 * dm)
     return {"config": "d_model 128, 2 layers, d_state 16, f32, batch 1, T 256",
-            "gpu_prefill": {"ms": tp * 1e3, "tok_per_s": T / tp}, "gpu_decode_us_per_step": td * 1e6,
+            "gpu_prefill": {"ms": tp * 1e3, "tok_per_s": T / tp, "roofline": roof}, "gpu_decode_us_per_step": td * 1e6,
+            "gpu_decode_hbm_frac": step_bytes / td / 1e9 / HBM_PEAK_GBPS,
             "cpu_port_prefill": {"ms": tc * 1e3, "tok_per_s": T / tc, "cores": orc.num_threads()},
             "cpu_port_decode_us_per_step": tcs * 1e6, "prefill_last_step_max_rel_diff_gpu_vs_cpu_port": err}
 
@@ -344,6 +401,8 @@ def default_configs_leg():
         x = np.random.default_rng(B).standard_normal((B, 128)).astype(np.float32)
         out[f"m1_step_us_b{B}"] = run(GpuMambaBackbone.new(0, MambaWeights.init(c1, 128, 42), c1, 128, B), x)
         out[f"m3_step_us_b{B}"] = run(GpuMamba3Backbone.new(0, Mamba3Weights.init(c3, 128, 42), c3, 128, B), x)
+        out[f"m1_step_hbm_frac_b{B}"] = m1_step_bytes(c1, B, 4) / out[f"m1_step_us_b{B}"] / 1e3 / HBM_PEAK_GBPS
+        out[f"m3_step_hbm_frac_b{B}"] = m3_step_bytes(c3, B, 4) / out[f"m3_step_us_b{B}"] / 1e3 / HBM_PEAK_GBPS
     # the reference's synthetic Mamba-3 LM (tests/bench_bf16_vs_f32.rs:148-215: d_model 256, 8 layers, headdim 16, vocab 256,
     # a_floor 0.0625; prompt [1..5], 100 greedy tokens, second run timed)
     from mamba_rs_amd import GpuMamba3LM, SampleParams, WeightDtype
@@ -359,6 +418,7 @@ def default_configs_leg():
         lm.generate([1, 2, 3, 4, 5], params=sp)
         t0 = time.perf_counter(); toks = lm.generate([1, 2, 3, 4, 5], params=sp); dt_s = time.perf_counter() - t0
         lm_out[name] = len(toks) / dt_s
+        lm_out[name + "_hbm_frac"] = (m3_step_bytes(cl, 1, 4 if name == "f32" else 2) + 256 * 256 * (4 if name == "f32" else 2)) * lm_out[name] / 1e9 / HBM_PEAK_GBPS
         lm.close(); bb.close()
     out["m3_synthetic_lm_tok_per_s"] = lm_out
     return out
@@ -391,7 +451,8 @@ def published_configs_leg():
             lm.decode_step()
         dec.sync()
         td = (time.perf_counter() - t0) / 128
-        out[key] = {"us_per_step": td * 1e6, "tok_per_s_total": B / td}
+        out[key] = {"us_per_step": td * 1e6, "tok_per_s_total": B / td,
+                    "hbm_frac": m1_step_bytes(cfg, B, dt.size_bytes(), vocab) / td / 1e9 / HBM_PEAK_GBPS}
         lm.close(); dec.close()
     c370 = MambaConfig(d_model=1024, d_state=16, d_conv=4, expand=2, n_layers=48)
     w370 = MambaWeights.random_lm(c370, 43)
@@ -407,6 +468,7 @@ def published_configs_leg():
             eng.reset(); eng.sync()
             t0 = time.perf_counter(); lm.prefill(toks); eng.sync(); times.append(time.perf_counter() - t0)
         pre[str(T)] = sorted(times)[1] * 1e3
+        pre[str(T) + "_roofline"] = m1_prefill_roofline(c370, 1, T, sorted(times)[1])
         lm.close(); eng.close()
     out["370m_bf16_prefill_ms_b1"] = pre
     return out
@@ -512,10 +574,18 @@ def m3_leg():
         for _ in range(24):
             ops.m3_step(s1, k1, v1, y1, x1, K1, Q1, a1, b1, g1, t["D"])
     us_step = timeit(g.replay, 50) / 24
+    prof, prof_src = profile_figures("m3_ssd_c4_bf16.md", "m3_ssd.hip", ["traffic_bytes_per_call", "mfma_busy_frac_full_pass", "mfma_busy_frac_state_pass"])
+    flop = 4 * 2 * 64 * 64 * 64 * B * (T // 64) * nh
+    step_state_bytes = 2 * 4 * nh * (hd * ds + ds + hd) + 4 * nh * hd * 2
     return {"ssd_prefill_layer": {"batch": B, "seq_len": T, "us": us, "algorithmic_bytes": nbytes, "GBps": nbytes / us / 1e3,
                                   "hbm_frac": nbytes / us / 1e3 / HBM_PEAK_GBPS, "tok_per_s_layer": B * T / us * 1e6,
-                                  "mfma_flop": 4 * 2 * 64 * 64 * 64 * B * (T // 64) * nh},
-            "decode_step_kernel_b1": {"us_per_layer_call_in_graph": us_step}}
+                                  "mfma_flop": flop, "mfma_frac": flop / us / 1e6 / MFMA_BF16_PEAK_TFLOPS,
+                                  "measured_traffic_bytes": prof["traffic_bytes_per_call"],
+                                  "traffic_over_algorithmic": (prof["traffic_bytes_per_call"] / nbytes) if prof["traffic_bytes_per_call"] else None,
+                                  "measured_mfma_busy_frac": {"full_pass": prof["mfma_busy_frac_full_pass"], "state_pass": prof["mfma_busy_frac_state_pass"]},
+                                  "counters_source": prof_src},
+            "decode_step_kernel_b1": {"us_per_layer_call_in_graph": us_step, "algorithmic_bytes": step_state_bytes,
+                                      "hbm_frac": step_state_bytes / us_step / 1e3 / HBM_PEAK_GBPS}}
 
 
 def m3_engine_leg(steps=512, batches=(1, 16), prefill_bt=(4, 4096)):
@@ -537,7 +607,7 @@ def m3_engine_leg(steps=512, batches=(1, 16), prefill_bt=(4, 4096)):
         pre.reset(); pre.sync()
         t0 = time.perf_counter(); pre.prefill_device(pt); pre.sync(); times.append(time.perf_counter() - t0)
     tp = sorted(times)[1]
-    prefill = {"batch": pb, "seq_len": pt, "ms": tp * 1e3, "tok_per_s": pb * pt / tp}
+    prefill = {"batch": pb, "seq_len": pt, "ms": tp * 1e3, "tok_per_s": pb * pt / tp, "roofline": m3_prefill_roofline(cfg, pb, pt, tp)}
     pre.close()
     for B in batches:
         eng = GpuMamba3Backbone.new_with_dtype(0, w, cfg, 768, B, WeightDtype.BF16)
@@ -551,8 +621,7 @@ def m3_engine_leg(steps=512, batches=(1, 16), prefill_bt=(4, 4096)):
             eng.step_gpu_only()
         eng.sync()
         td = (time.perf_counter() - t0) / steps
-        layer_bytes = 2 * (dm * ip + di * dm) + 2 * 4 * B * nh * (hd * ds + ds + hd) + 2 * 4 * B * dm
-        step_bytes = cfg.n_layers * layer_bytes
+        step_bytes = m3_step_bytes(cfg, B, 2)
         entry = {"batch": B, "steps": steps, "us_per_step": td * 1e6, "algorithmic_bytes_per_step": step_bytes,
                  "hbm_frac": step_bytes / td / 1e9 / HBM_PEAK_GBPS}
         if B == 1:
@@ -565,7 +634,8 @@ def m3_engine_leg(steps=512, batches=(1, 16), prefill_bt=(4, 4096)):
             sp = SampleParams(temperature=0.0, max_tokens=100)
             lm.generate(prompt, params=sp)
             t0 = time.perf_counter(); toks = lm.generate(prompt, params=sp); tg = time.perf_counter() - t0
-            entry["lm_greedy_100_tokens"] = {"ms": tg * 1e3, "tok_per_s": len(toks) / tg}
+            entry["lm_greedy_100_tokens"] = {"ms": tg * 1e3, "tok_per_s": len(toks) / tg,
+                                             "hbm_frac": (step_bytes + (vocab + 63) // 64 * 64 * dm * 2) * len(toks) / tg / 1e9 / HBM_PEAK_GBPS}
             lm.close()
         out.append(entry)
         eng.close()
@@ -604,7 +674,9 @@ def main():
     inp = make_inputs(*shape)
     g = gpu_leg(args, inp, shape)
     gbps = nbytes / (g["ms_per_step"] * 1e-3) / 1e9
-    traffic, traffic_source = profiled_scan_traffic()
+    traffic, issue_us, traffic_source = profiled_scan_traffic()
+    us = g["ms_per_step"] * 1e3
+    gen_us = g["general_a_ms_per_step"] * 1e3
     out = {
         "metric": "m1_selective_scan_hbm_GBps",
         "value": gbps,
@@ -627,7 +699,16 @@ def main():
         "roofline": {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": gbps / HBM_PEAK_GBPS, "traffic": traffic, "traffic_source": traffic_source,
                      "kernels": ["chunk_state_kernel", "chunk_out_kernel"],
-                     "algorithmic_bytes_per_launch": nbytes, "median_launch_ms": g["median_launch_ms"]},
+                     "algorithmic_bytes_per_launch": nbytes, "median_launch_ms": g["median_launch_ms"],
+                     # what the two kernels are bound by in fact: the instruction issue of the SIMDs (f32 without packed math)
+                     "issue": {"bound": "instruction issue (1024 SIMDs; two plain instructions per issue window of 2.02 ns from "
+                                        "two different waves, a DPP-operand instruction a whole window, v_exp / v_rcp / "
+                                        "v_mfma_f32_4x4x1 two windows)",
+                               "model_us_per_call": issue_us, "frac": (issue_us / us) if issue_us else None,
+                               "source": traffic_source},
+                     # the same launch on the kernels a trained checkpoint's A takes (no S4D-real shortcut)
+                     "general_A": {"bound": "hbm", "achieved": nbytes / gen_us / 1e3, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                                   "frac": nbytes / gen_us / 1e3 / HBM_PEAK_GBPS, "ms_per_step": g["general_a_ms_per_step"]}},
     }
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_leg(inp, shape, nbytes)

@@ -203,12 +203,16 @@ static int launch_seq(hipStream_t st, bool s4d, int gate_mode, float *h, void *y
 //
 // How the B_t / C_t rows (wave-uniform, 16 values each) reach the arithmetic: a wave copies the rows of 16 steps at a
 // time into its own 4 KB of LDS as f32 (lane l brings elements 4(l%4)..+3 of row l/4), two such spans ahead of their
-// use, and every step reads back 16 bytes per lane: lane l gets X[4(l%4) + k] in register k.  Within each group of four
-// lanes the whole row is then present, and the two consumers take it from there at no cost in instructions:
-//   * the matrix core: v_mfma_f32_4x4x1 number k with register k as its A operand gives result register a of lane l
-//     A(lane 4(l/4)+a) * B(lane l) = X[4a+k] * (delta u)[l]  --  the rank-1 state update for state 4a+k;
-//   * the vector ALU through the DPP quad broadcast: an operand "register k of quad lane a" is X[4a+k] on every lane.
-// So state n = 4a+k lives in state register 4k+a (a 4x4 transpose of the natural order, kStateOfReg below).
+// use.  The two consumers read them back in two ways:
+//   * the rank-1 state update of pass B runs on the matrix core: every lane reads 16 bytes, lane l gets X[4(l%4) + k] in
+//     register k, and v_mfma_f32_4x4x1 number k with register k as its A operand gives result register a of lane l
+//     A(lane 4(l/4)+a) * B(lane l) = X[4a+k] * (delta u)[l]  --  so state n = 4a+k lives in state register 4k+a (a 4x4
+//     transpose of the natural order, kStateOfReg below);
+//   * the multiply-adds with a row as the uniform factor (the output dot of pass B, the summary of pass A) take the
+//     row as ordinary registers: four 16-byte LDS reads with one address for all lanes put the whole row on every
+//     lane.  A SIMD issues two plain f32 instructions per issue slot when two of its waves have one ready, but an
+//     instruction with a DPP operand (the quad broadcast these kernels used before) takes the slot alone: sixteen of
+//     them per step cost sixteen slots, sixteen plain ones and the four reads cost ten.
 // ---------------------------------------------------------------------------
 struct SplitPlan {
     int nchunk;  // C
@@ -337,6 +341,10 @@ struct StagedRows {
     __device__ __forceinline__ v4f read(int slot, int row) const {
         return *reinterpret_cast<const v4f *>(&v[slot][row][4 * (threadIdx.x & 3)]);
     }
+    // elements 4q..4q+3 of a row, the same on every lane
+    __device__ __forceinline__ v4f read_all(int slot, int row, int q) const {
+        return *reinterpret_cast<const v4f *>(&v[slot][row][4 * q]);
+    }
 };
 
 // Decay factors of one step: da[n] = 2^(dl * a2[n]); S4D: a2[n] = (n+1) a2[0] -> powers of one exp.
@@ -432,63 +440,6 @@ __device__ __forceinline__ void set_progress_priority(int done, int total) {
 // resource: their loads return zero and their stores are dropped, so the time loops carry no lane predicate.
 constexpr unsigned kDeadLaneOffset = 0x7f000000u;
 
-// Sixteen multiply-adds whose first operand is read through the DPP quad broadcast (all four lanes of a group read
-// lane a's register).  The compiler does not fold a DPP move into v_fmac, hence the assembly; it also does not count
-// these as vector instructions when it places the wait states that a matrix-core result or a freshly written DPP
-// source needs before a vector instruction may read it (4-5 and 2), so each block opens with instructions of its own
-// that read none of those registers.
-//
-// Pass B:  acc = D*u + sum_{k,a} c[k](quad lane a) * h[4k+a], and the first half of the SiLU gate rides in front:
-// e = 2^(z * -log2 e).  Three leading instructions (one of them double length) plus the s_nop cover a matrix result
-// written by the instruction just before the block.
-__device__ __forceinline__ void dot16_quad(float &acc, float &e, float Dd, float uu, float z, const v4f &c, const float (&h)[16]) {
-    asm("v_mul_f32 %0, %2, %3\n\t"
-        "v_mul_f32 %1, 0xbfb8aa3b, %4\n\t"
-        "v_exp_f32 %1, %1\n\t"
-        "s_nop 1\n\t"
-        "v_fmac_f32_dpp %0, %5, %9 quad_perm:[0,0,0,0] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
-        "v_fmac_f32_dpp %0, %5, %10 quad_perm:[1,1,1,1] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
-        "v_fmac_f32_dpp %0, %5, %11 quad_perm:[2,2,2,2] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
-        "v_fmac_f32_dpp %0, %5, %12 quad_perm:[3,3,3,3] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
-        "v_fmac_f32_dpp %0, %6, %13 quad_perm:[0,0,0,0] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
-        "v_fmac_f32_dpp %0, %6, %14 quad_perm:[1,1,1,1] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
-        "v_fmac_f32_dpp %0, %6, %15 quad_perm:[2,2,2,2] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
-        "v_fmac_f32_dpp %0, %6, %16 quad_perm:[3,3,3,3] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
-        "v_fmac_f32_dpp %0, %7, %17 quad_perm:[0,0,0,0] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
-        "v_fmac_f32_dpp %0, %7, %18 quad_perm:[1,1,1,1] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
-        "v_fmac_f32_dpp %0, %7, %19 quad_perm:[2,2,2,2] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
-        "v_fmac_f32_dpp %0, %7, %20 quad_perm:[3,3,3,3] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
-        "v_fmac_f32_dpp %0, %8, %21 quad_perm:[0,0,0,0] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
-        "v_fmac_f32_dpp %0, %8, %22 quad_perm:[1,1,1,1] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
-        "v_fmac_f32_dpp %0, %8, %23 quad_perm:[2,2,2,2] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
-        "v_fmac_f32_dpp %0, %8, %24 quad_perm:[3,3,3,3] row_mask:0xf bank_mask:0xf bound_ctrl:1"
-        : "=&v"(acc), "=&v"(e)
-        : "v"(Dd), "v"(uu), "v"(z), "v"(c[0]), "v"(c[1]), "v"(c[2]), "v"(c[3]), "v"(h[0]), "v"(h[1]), "v"(h[2]), "v"(h[3]), "v"(h[4]),
-          "v"(h[5]), "v"(h[6]), "v"(h[7]), "v"(h[8]), "v"(h[9]), "v"(h[10]), "v"(h[11]), "v"(h[12]), "v"(h[13]), "v"(h[14]), "v"(h[15]));
-}
-
-// Pass A (direct form, S4D):  s[4k+a] += v^(n+1-ish) * b[k](quad lane a) for the states n = 4a+k in the order n = 0..15,
-// with the power chain v <- v * x between them (a dependent chain costs no issue slot here) and the step's running sum
-// of delta: v enters as x * (delta u), leaves as x^16 * (delta u).  Two plain instructions lead, so a freshly written b
-// register is two instructions old before the first DPP read.
-__device__ __forceinline__ void chain16_quad(float (&s)[16], float &sd, float x, float du, float dl, const v4f &b) {
-    float v;
-#define MRS_QF(R, K, A) "v_fmac_f32_dpp %" #R ", %" #K ", %16 quad_perm:[" #A "," #A "," #A "," #A "] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
-#define MRS_MX "v_mul_f32 %16, %16, %18\n\t"
-    asm("v_mul_f32 %16, %18, %19\n\t"
-        "v_add_f32 %17, %17, %20\n\t"
-        // n = 0..15: state register 4k+a with k = n % 4, a = n / 4; b[k] are operands 21..24
-        MRS_QF(0, 21, 0) MRS_MX MRS_QF(4, 22, 0) MRS_MX MRS_QF(8, 23, 0) MRS_MX MRS_QF(12, 24, 0) MRS_MX
-        MRS_QF(1, 21, 1) MRS_MX MRS_QF(5, 22, 1) MRS_MX MRS_QF(9, 23, 1) MRS_MX MRS_QF(13, 24, 1) MRS_MX
-        MRS_QF(2, 21, 2) MRS_MX MRS_QF(6, 22, 2) MRS_MX MRS_QF(10, 23, 2) MRS_MX MRS_QF(14, 24, 2) MRS_MX
-        MRS_QF(3, 21, 3) MRS_MX MRS_QF(7, 22, 3) MRS_MX MRS_QF(11, 23, 3) MRS_MX MRS_QF(15, 24, 3)
-        : "+v"(s[0]), "+v"(s[1]), "+v"(s[2]), "+v"(s[3]), "+v"(s[4]), "+v"(s[5]), "+v"(s[6]), "+v"(s[7]), "+v"(s[8]), "+v"(s[9]),
-          "+v"(s[10]), "+v"(s[11]), "+v"(s[12]), "+v"(s[13]), "+v"(s[14]), "+v"(s[15]), "=&v"(v), "+v"(sd)
-        : "v"(x), "v"(du), "v"(dl), "v"(b[0]), "v"(b[1]), "v"(b[2]), "v"(b[3]));
-#undef MRS_QF
-#undef MRS_MX
-}
-
 template <typename T, bool S4D>
 __global__ __launch_bounds__(kWave) void chunk_state_kernel(
     const float *__restrict__ h, const T *__restrict__ delta, const T *__restrict__ u,
@@ -544,7 +495,7 @@ __global__ __launch_bounds__(kWave) void chunk_state_kernel(
         // Direct form, walking the chunk backwards: the weight of step s in the chunk-end
         // state is prod_{r>s} exp(delta_r a_n) = x_s^(n+1) with x_s = 2^(a2[0] * sum_{r>s} delta_r),
         // so one exp, a power chain and one multiply-add per state -- no decay of a running state.
-        float S16[16];   // S16[r]: state kStateOfReg(r)
+        float S16[16];   // S16[n]: state n
 #pragma unroll
         for (int j = 0; j < 16; j++) S16[j] = 0.0f;
         // spans are walked last to first; span s sits in slot s & 1, span s-1 is published while s is computed and
@@ -556,7 +507,6 @@ __global__ __launch_bounds__(kWave) void chunk_state_kernel(
         }
         piece_ld(nb, Bp, bc_stride, t0 + max(nspans - 2, 0) * kSpan + prow);
         load_group(rdB, ruB, t0 + (nspans - 1) * kSpan + kGroup);
-        v4f bv = Bs.read((nspans - 1) & 1, kSpan - 1);
         for (int sp = nspans - 1; sp >= 0; sp--) {
             const int ts = t0 + sp * kSpan, slot = sp & 1;
             set_progress_priority(nspans - 1 - sp, nspans);
@@ -567,12 +517,19 @@ __global__ __launch_bounds__(kWave) void chunk_state_kernel(
 #pragma unroll
                 for (int k = kGroup - 1; k >= 0; k--) {
                     const int j = base + k;                               // row of the span
-                    const v4f bcur = bv;
-                    bv = j > 0 ? Bs.read(slot, j - 1) : Bs.read(slot ^ 1, kSpan - 1);   // the step after this one
+                    v4f ball[4];
+#pragma unroll
+                    for (int q = 0; q < 4; q++) ball[q] = Bs.read_all(slot, j, q);
                     const float dl = widen32(rd[k], (const T *)nullptr);
                     const float uu = widen32(ru[k], (const T *)nullptr);
                     const float x = fast_exp2(a2[0] * sd);
-                    chain16_quad(S16, sd, x, dl * uu, dl, bcur);
+                    float v = x * (dl * uu);
+                    sd += dl;
+#pragma unroll
+                    for (int n = 0; n < 16; n++) {
+                        S16[n] = fmaf(v, ball[n >> 2][n & 3], S16[n]);
+                        if (n < 15) v *= x;
+                    }
                 }
             };
             back(rdB, ruB, kGroup);
@@ -583,7 +540,7 @@ __global__ __launch_bounds__(kWave) void chunk_state_kernel(
         float da[16];
         decay16<true>(sd, a2, da);
 #pragma unroll
-        for (int j = 0; j < 16; j++) hs[j] = fmaf(da[j], hs[j], S16[4 * (j % 4) + j / 4]);
+        for (int j = 0; j < 16; j++) hs[j] = fmaf(da[j], hs[j], S16[j]);
     } else {
         // General A: the recurrence itself, forwards, with the rank-1 update on the matrix core as in pass B.
         float hr[16];   // hr[r]: state kStateOfReg(r)
@@ -705,7 +662,7 @@ __global__ __launch_bounds__(kWave) void chunk_out_kernel(
     for (int r = 0; r < 16; r++) { hs[r] = hn[kStateOfReg(r)]; ar[r] = a2[kStateOfReg(r)]; }
     Bs.publish(0, piece_widen(fb, (const T *)nullptr));
     Cs.publish(0, piece_widen(fc, (const T *)nullptr));
-    v4f bv = Bs.read(0, 0), cv = Cs.read(0, 0);
+    v4f bv = Bs.read(0, 0);
     for (int sp = 0; sp < nspans; sp++) {
         const int ts = t0 + sp * kSpan, slot = sp & 1;
         set_progress_priority(sp, nspans);
@@ -720,9 +677,11 @@ __global__ __launch_bounds__(kWave) void chunk_out_kernel(
 #pragma unroll
             for (int k = 0; k < kGroup; k++, yo += row_bytes) {
                 const int j = base + k;
-                const v4f bcur = bv, ccur = cv;
-                bv = j < kSpan - 1 ? Bs.read(slot, j + 1) : Bs.read(slot ^ 1, 0);   // the rows of the next step
-                cv = j < kSpan - 1 ? Cs.read(slot, j + 1) : Cs.read(slot ^ 1, 0);
+                const v4f bcur = bv;
+                bv = j < kSpan - 1 ? Bs.read(slot, j + 1) : Bs.read(slot ^ 1, 0);   // the B row of the next step, a quad piece per lane
+                v4f call[4];
+#pragma unroll
+                for (int q = 0; q < 4; q++) call[q] = Cs.read_all(slot, j, q);      // this step's C row, whole, on every lane
                 const float dl = widen32(rd[k], (const T *)nullptr);
                 const float uu = widen32(ru[k], (const T *)nullptr);
                 const float du = dl * uu;
@@ -751,7 +710,10 @@ __global__ __launch_bounds__(kWave) void chunk_out_kernel(
                     for (int i = 0; i < 4; i++) hs[4 * q + i] = hq[q][i];
                 float acc, e;
                 const float z = GATE ? widen32(rg[k], (const T *)nullptr) : 0.0f;
-                dot16_quad(acc, e, Dd, uu, z, ccur, hs);
+                acc = Dd * uu;
+                e = fast_exp2(z * -kLog2e);
+#pragma unroll
+                for (int r = 0; r < 16; r++) acc = fmaf(call[kStateOfReg(r) >> 2][kStateOfReg(r) & 3], hs[r], acc);
                 if (GATE == 1) acc *= z;
                 if (GATE == 2) acc *= z * fast_rcp(1.0f + e);
                 ybuf.st(acc, lxb, yo);
