@@ -51,7 +51,12 @@ enum {
     MRS_GATE_SILU = 1u << 1,   /* gate holds raw z: y *= z*sigmoid(z) (split_gate_silu + elementwise_mul fused) */
     MRS_A_S4D_REAL = 1u << 2,  /* caller asserts a_neg[d,n] = (n+1)*a_neg[d,0] to 4 ulp; see mrs_a_neg_is_s4d_real */
     MRS_FORCE_SEQUENTIAL = 1u << 3, /* ignore the T-split route */
-    MRS_FORCE_PARALLEL = 1u << 4    /* use the T-split route even for short T */
+    MRS_FORCE_PARALLEL = 1u << 4,   /* use the T-split route even for short T, and its one-launch form at any size */
+    MRS_SCAN_FLAGS_ZERO = 1u << 5,  /* T-split route: the caller vouches that the first mrs_ssm_scan_flag_bytes() bytes of
+                                       the workspace were zero before the first call and that nothing but this entry
+                                       point has written there since; saves the small kernel that clears them */
+    MRS_SCAN_TWO_LAUNCHES = 1u << 6 /* T-split route as two launches (no wave waits for another; also MRS_SCAN_TWO_LAUNCHES=1
+                                       in the environment) */
 };
 
 /* Library version (major*10000 + minor*100 + patch) and the last error text of
@@ -105,6 +110,17 @@ MRS_API int mrs_ssm_scan_fwd(void *stream, int dtype, float *h, void *y, const v
  *   workspace  mrs_ssm_scan_workspace_bytes() bytes of device memory, 256-byte
  *              aligned; NULL forces the sequential route. */
 MRS_API size_t mrs_ssm_scan_workspace_bytes(int batch, int T, int d_inner, int d_state);
+/* Where it is the faster form -- MRS_A_S4D_REAL and at least 2048 waves (batch x ceil(d_inner / 64) x chunks) -- the
+ * T-split route runs as ONE launch: every wave first summarises its chunk, publishes the summary and waits for the
+ * chunks before it (no counterpart in the reference, whose kernel keeps a block per (b, d) and needs no such hand-off).
+ * The flags the waves signal with are the first mrs_ssm_scan_flag_bytes(batch, d_inner) bytes of the workspace (256 KB
+ * whatever the shape, counted in mrs_ssm_scan_workspace_bytes); they must be zero when the launch starts and are zero
+ * again when it ends.  By default a small kernel clears them ahead of every call; a caller that zeroed them once (and
+ * lets nothing else write there) passes MRS_SCAN_FLAGS_ZERO and saves that kernel.  MRS_SCAN_TWO_LAUNCHES keeps the
+ * two-kernel form, MRS_FORCE_PARALLEL takes the one launch at any size and for any A.  A wave that waits some seconds
+ * for another (never seen; it would take a wave that does not get scheduled) writes NaN into its share
+ * of y and h rather than spin for ever. */
+MRS_API size_t mrs_ssm_scan_flag_bytes(int batch, int d_inner);
 MRS_API int mrs_ssm_scan_fwd_ex(void *stream, int dtype, float *h, void *y, const void *delta, const void *u,
                         const void *B, const void *C, int64_t bc_stride, const float *a_neg,
                         const float *D, const void *gate, int64_t gate_stride, unsigned flags,
@@ -118,7 +134,7 @@ MRS_API int mrs_ssm_scan_fwd_ex(void *stream, int dtype, float *h, void *y, cons
  * MRS_SCAN_STATIC_SCRATCH_BYTES block per GPU, resident until the process ends -- so the call allocates nothing
  * and frees nothing.  Same arguments, routes and results as mrs_ssm_scan_fwd_ex given a workspace of that size.
  *   - A shape with mrs_ssm_scan_workspace_bytes() > MRS_SCAN_STATIC_SCRATCH_BYTES is refused (MRS_E_WORKSPACE);
- *     the benchmark shapes (8 x 2048 x 1536 and 4 x 4096 x 5120, d_state 16) need 13.3 MB and 12.5 MB; only very wide
+ *     the benchmark shapes (8 x 2048 x 1536 and 4 x 4096 x 5120, d_state 16) need 13.6 MB and 12.8 MB; only very wide
  *     batches (batch x d_inner above about 120 000 channels) need more.
  *   - The first call on a GPU looks the buffer's address up (hipGetSymbolAddress, no allocation); make that call
  *     outside a graph capture.

@@ -29,6 +29,7 @@ _SIGNATURES = {
     "mrs_a_neg_is_s4d_real": (c_int, [_P, _P, _P, c_int, c_int]),
     "mrs_ssm_scan_fwd": (c_int, [_P, c_int, _P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int]),
     "mrs_ssm_scan_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
+    "mrs_ssm_scan_flag_bytes": (c_size_t, [c_int, c_int]),
     "mrs_ssm_scan_fwd_ex": (c_int, [_P, c_int, _P, _P, _P, _P, _P, _P, c_int64, _P, _P, _P, c_int64, c_uint, _P, c_size_t,
                                     c_int, c_int, c_int, c_int]),
     "mrs_ssm_scan_fwd_static": (c_int, [_P, c_int, _P, _P, _P, _P, _P, _P, c_int64, _P, _P, _P, c_int64, c_uint,

@@ -328,6 +328,8 @@ static int alloc_scratch(mrs_backbone *bb, Scratch *s, int64_t rows, int T) {
     if (T > 1) {
         s->scan_ws_bytes = mrs_ssm_scan_workspace_bytes(bb->batch, T, di, bb->cfg.d_state);
         MRS_TRY(dev_alloc(bb, &s->scan_ws, s->scan_ws_bytes));
+        // the flags of the one-launch scan start at zero here and every scan leaves them zero (MRS_SCAN_FLAGS_ZERO below)
+        MRS_HIP(hipMemsetAsync(s->scan_ws, 0, std::min(s->scan_ws_bytes, mrs_ssm_scan_flag_bytes(bb->batch, di)), bb->stream));
     }
     return MRS_OK;
 }
@@ -489,7 +491,7 @@ static int run_layers(mrs_backbone *bb, Scratch *s, int T) {
             MRS_TRY(check_launch("bias_softplus_kernel"));
             }
             // ScanMode::use_parallel picks the route (src/mamba_ssm/gpu/prefill.rs:910-956)
-            unsigned flags = MRS_GATE_SILU | (lw.s4d ? MRS_A_S4D_REAL : 0);
+            unsigned flags = MRS_GATE_SILU | MRS_SCAN_FLAGS_ZERO | (lw.s4d ? MRS_A_S4D_REAL : 0);
             // An explicit mode is honoured; in Auto the op picks the kernel itself (same recurrence, same tolerance).
             if (bb->cfg.scan_mode == MRS_SCAN_SEQUENTIAL) flags |= MRS_FORCE_SEQUENTIAL;
             else if (bb->cfg.scan_mode == MRS_SCAN_PARALLEL && ds == 16 && T >= 64) flags |= MRS_FORCE_PARALLEL;

@@ -260,16 +260,33 @@ static SplitPlan make_split_plan(int batch, int Tlen, int di) {
 }
 
 struct SplitWs {
+    unsigned *flags;  // [B][tiles][kMaxChunks]: chunk summary published (the one-launch route)
+    unsigned *done;   // [B][tiles]: waves that have folded their entering state
+    size_t flag_words;
     float *h0copy;  // [B][16][di]
     float *S;       // [B][C-1][16][di]
     float *sumd;    // [B][C-1][di]
-    size_t floats;
+    size_t floats;  // whole workspace, in 4-byte words
 };
 
+constexpr int kMaxChunks = 32;
+
+// The flag area comes first and has one size whatever the shape of the call, so that a buffer shared by calls of
+// different shapes (the library's static one, an engine's scratch) never has one call's summaries where another call's
+// flags are: it stays all zero between calls.  A call with more (batch row, channel tile) pairs than it holds takes the
+// two-launch form.
+constexpr size_t kFlagAreaWords = 65536;   // 256 KB: 1985 pairs of kMaxChunks flags + a counter
+static bool flags_fit(int batch, int di) {
+    return (size_t)batch * (size_t)((di + kWave - 1) / kWave) * (kMaxChunks + 1) <= kFlagAreaWords;
+}
 static SplitWs carve_workspace(float *base, int batch, int Tlen, int di, int nchunk) {
     (void)Tlen;
     SplitWs w;
-    size_t o = 0;
+    const size_t tiles = (size_t)((di + kWave - 1) / kWave);
+    w.flags = reinterpret_cast<unsigned *>(base);
+    w.done = w.flags + (size_t)batch * tiles * kMaxChunks;
+    w.flag_words = kFlagAreaWords;
+    size_t o = kFlagAreaWords;
     w.h0copy = base + o; o += (size_t)batch * 16 * di;
     w.S = base + o; o += (size_t)batch * (nchunk - 1) * 16 * di;
     w.sumd = base + o; o += (size_t)batch * (nchunk - 1) * di;
@@ -392,24 +409,35 @@ __device__ __forceinline__ void load_a2(float (&a2)[16], const float *__restrict
 // The terms are independent; the summaries are fetched four chunks at a time (68 loads in flight), so the fold costs
 // a few memory round trips instead of one per chunk -- every wave of pass B sits through it before its first step.
 // hs[n] is state n.
-constexpr int kMaxChunks = 32;
 constexpr int kFoldBatch = 4;
-template <bool S4D>
+// A float another wave of the same launch has published (the one-launch route): a relaxed load at agent scope, so that it
+// is served from where that wave's relaxed agent-scope store put it, whichever part of the chip either wave runs on.
+// Between launches the plain load does (the kernel boundary publishes).
+template <bool FUSED> __device__ __forceinline__ float pub_ld(const float *p) {
+    if constexpr (FUSED) return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    else return *p;
+}
+template <bool FUSED> __device__ __forceinline__ void pub_st(float *p, float v) {
+    if constexpr (FUSED) __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    else *p = v;
+}
+
+template <bool S4D, bool FUSED = false>
 __device__ __forceinline__ void fold_entering_state(float (&hs)[16], const float (&a2)[16],
                                                     const float *__restrict__ S, const float *__restrict__ sumd,
                                                     int b, int c, int nchunk, int di, int dd) {
     const int64_t sbase = (int64_t)b * (nchunk - 1);
 #pragma unroll
-    for (int j = 0; j < 16; j++) hs[j] = S[((sbase + c - 1) * 16 + j) * di + dd];  // k = c-1: weight 1
+    for (int j = 0; j < 16; j++) hs[j] = pub_ld<FUSED>(S + ((sbase + c - 1) * 16 + j) * di + dd);  // k = c-1: weight 1
     float suffix = 0.0f;  // sum of sumdelta_m over k < m < c
     for (int k0 = c - 2; k0 >= 0; k0 -= kFoldBatch) {
         float Sv[kFoldBatch][16], sm[kFoldBatch];
 #pragma unroll
         for (int i = 0; i < kFoldBatch; i++) {
             const int k = max(k0 - i, 0);     // past the front: chunk 0 again, loaded and not used
-            sm[i] = sumd[(sbase + k + 1) * di + dd];
+            sm[i] = pub_ld<FUSED>(sumd + (sbase + k + 1) * di + dd);
 #pragma unroll
-            for (int j = 0; j < 16; j++) Sv[i][j] = S[((sbase + k) * 16 + j) * di + dd];
+            for (int j = 0; j < 16; j++) Sv[i][j] = pub_ld<FUSED>(S + ((sbase + k) * 16 + j) * di + dd);
         }
 #pragma unroll
         for (int i = 0; i < kFoldBatch; i++) {
@@ -440,21 +468,19 @@ __device__ __forceinline__ void set_progress_priority(int done, int total) {
 // resource: their loads return zero and their stores are dropped, so the time loops carry no lane predicate.
 constexpr unsigned kDeadLaneOffset = 0x7f000000u;
 
-template <typename T, bool S4D>
-__global__ __launch_bounds__(kWave) void chunk_state_kernel(
-    const float *__restrict__ h, const T *__restrict__ delta, const T *__restrict__ u,
+// Pass A for the wave (batch row b, chunk c < nchunk - 1, channel tile).  Chunk lengths are multiples of kSpan: every
+// step of the chunk exists, so the walk has no tail.  FUSED: the wave is part of the one-launch route -- the summary is
+// published to the other waves of the launch (relaxed agent-scope stores, then the chunk's flag), and chunk 0 hands
+// the caller's state back in h_keep instead of through the h0copy buffer.
+template <typename T, bool S4D, bool FUSED>
+__device__ __forceinline__ void pass_a_body(
+    StagedRows &Bs, const float *__restrict__ h, const T *__restrict__ delta, const T *__restrict__ u,
     const T *__restrict__ Bm, int64_t bc_stride,
     const float *__restrict__ a_neg, float *__restrict__ h0copy, float *__restrict__ S,
-    float *__restrict__ sumd, int Tlen, int di, int tiles, int nchunk, int len) {
+    float *__restrict__ sumd, unsigned *__restrict__ flags, float (&h_keep)[16],
+    int Tlen, int di, int tiles, int nchunk, int len, int b, int c, int tile) {
     using raw_t = typename Raw32<T>::type;
-    __shared__ alignas(16) StagedRows Bs;
-    // Chunks 0 .. nchunk-2 only, and chunk lengths are multiples of kSpan: every step of this wave's chunk
-    // exists, so the walk has no tail.
     const int nc1 = nchunk - 1;
-    const int tile = blockIdx.x % tiles;
-    const int rest = blockIdx.x / tiles;
-    const int c = rest % nc1;
-    const int b = rest / nc1;
     const int d0 = tile * kWave;
     const bool live = d0 + (int)threadIdx.x < di;
     const int dd = live ? d0 + (int)threadIdx.x : di - 1;   // plain loads of dead lanes shadow the last live channel
@@ -468,7 +494,8 @@ __global__ __launch_bounds__(kWave) void chunk_state_kernel(
 #pragma unroll
         for (int j = 0; j < 16; j++) {
             hs[j] = h[((int64_t)b * di + dd) * 16 + j];
-            if (live) h0copy[((int64_t)b * 16 + j) * di + dd] = hs[j];
+            if constexpr (FUSED) h_keep[j] = hs[j];
+            else if (live) h0copy[((int64_t)b * 16 + j) * di + dd] = hs[j];
         }
     }
     const int t0 = c * len;
@@ -592,26 +619,48 @@ __global__ __launch_bounds__(kWave) void chunk_state_kernel(
     if (live) {
         const int64_t sbase = (int64_t)b * nc1 + c;
 #pragma unroll
-        for (int j = 0; j < 16; j++) S[(sbase * 16 + j) * di + dd] = hs[j];
-        sumd[sbase * di + dd] = sd;
+        for (int j = 0; j < 16; j++) pub_st<FUSED>(S + (sbase * 16 + j) * di + dd, hs[j]);
+        pub_st<FUSED>(sumd + sbase * di + dd, sd);
     }
+    if constexpr (FUSED) {
+        // the summary has arrived where the other waves will look for it before the flag says so
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        if (threadIdx.x == 0)
+            __hip_atomic_store(flags + ((int64_t)b * tiles + tile) * kMaxChunks + c, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
+template <typename T, bool S4D>
+__global__ __launch_bounds__(kWave) void chunk_state_kernel(
+    const float *__restrict__ h, const T *__restrict__ delta, const T *__restrict__ u,
+    const T *__restrict__ Bm, int64_t bc_stride,
+    const float *__restrict__ a_neg, float *__restrict__ h0copy, float *__restrict__ S,
+    float *__restrict__ sumd, int Tlen, int di, int tiles, int nchunk, int len) {
+    __shared__ alignas(16) StagedRows Bs;
+    const int nc1 = nchunk - 1;   // chunks 0 .. nchunk-2 only
+    const int tile = blockIdx.x % tiles;
+    const int rest = blockIdx.x / tiles;
+    float unused[16];
+    pass_a_body<T, S4D, false>(Bs, h, delta, u, Bm, bc_stride, a_neg, h0copy, S, sumd, nullptr, unused, Tlen, di, tiles, nchunk, len,
+                               rest / nc1, rest % nc1, tile);
 }
 
 // Pass B.  The time loop has no tail and no lane predicate: rows at and beyond T lie outside the buffer resources
 // (loads return zero: delta = 0 leaves the state as it is, stores are dropped), and so do the lanes of a partial tile.
-template <typename T, bool S4D, int GATE>
-__global__ __launch_bounds__(kWave) void chunk_out_kernel(
-    float *__restrict__ h, T *__restrict__ y, const T *__restrict__ delta, const T *__restrict__ u,
+// FUSED (the one-launch route): the summaries of the chunks before this one are other waves' work of the same launch --
+// the wave waits for their flags (a bounded wait: every wave reaches its end whatever happens), folds them through
+// agent-scope loads, and the last wave of a (batch row, channel tile) to have folded clears that pair's flags and
+// counter again, so that the flag area is all zero between launches.  Chunk 0 takes its entering state from h_keep.
+constexpr int kFlagSpinLimit = 1 << 22;
+template <typename T, bool S4D, int GATE, bool FUSED>
+__device__ __forceinline__ void pass_b_body(
+    StagedRows &Bs, StagedRows &Cs, float *__restrict__ h, T *__restrict__ y, const T *__restrict__ delta, const T *__restrict__ u,
     const T *__restrict__ Bm, const T *__restrict__ Cm, int64_t bc_stride,
     const float *__restrict__ a_neg, const float *__restrict__ Dp, const T *__restrict__ gate, int64_t gate_stride,
     const float *__restrict__ h0copy, const float *__restrict__ S, const float *__restrict__ sumd,
-    int Tlen, int di, int tiles, int nchunk, int len) {
+    unsigned *__restrict__ flags, unsigned *__restrict__ done, const float (&h_keep)[16],
+    int Tlen, int di, int tiles, int nchunk, int len, int b, int c, int tile) {
     using raw_t = typename Raw32<T>::type;
-    __shared__ alignas(16) StagedRows Bs, Cs;
-    const int tile = blockIdx.x % tiles;
-    const int rest = blockIdx.x / tiles;
-    const int c = rest % nchunk;
-    const int b = rest / nchunk;
     const int d0 = tile * kWave;
     const bool live = d0 + (int)threadIdx.x < di;
     const int dd = live ? d0 + (int)threadIdx.x : di - 1;
@@ -651,12 +700,44 @@ __global__ __launch_bounds__(kWave) void chunk_out_kernel(
     const float Dd = Dp[dd];
 
     float hn[16], a2[16], hs[16], ar[16];   // hn[n]: state n; hs[r], ar[r]: state kStateOfReg(r)
+    bool poison = false;
     load_a2<S4D>(a2, a_neg, dd);
     if (c == 0) {
 #pragma unroll
-        for (int j = 0; j < 16; j++) hn[j] = h0copy[((int64_t)b * 16 + j) * di + dd];
+        for (int j = 0; j < 16; j++) hn[j] = FUSED ? h_keep[j] : h0copy[((int64_t)b * 16 + j) * di + dd];
     } else {
-        fold_entering_state<S4D>(hn, a2, S, sumd, b, c, nchunk, di, dd);
+        if constexpr (FUSED) {
+            unsigned *fl = flags + ((int64_t)b * tiles + tile) * kMaxChunks;
+            bool arrived = false;
+            for (int spin = 0; spin < kFlagSpinLimit && !arrived; spin++) {
+                const unsigned f = (int)threadIdx.x < c ? __hip_atomic_load(fl + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 1u;
+                arrived = __builtin_amdgcn_ballot_w64(f == 0u) == 0;
+                if (!arrived) __builtin_amdgcn_s_sleep(8);
+            }
+            asm volatile("" ::: "memory");
+            // a summary that never came (seconds of waiting: the flag area was not zero, or two calls share the buffer):
+            // the wave goes on to its end, and its outputs say so -- NaN, not a plausible number
+            poison = !arrived;
+        }
+        fold_entering_state<S4D, FUSED>(hn, a2, S, sumd, b, c, nchunk, di, dd);
+        if constexpr (FUSED) {
+            if (poison) {
+#pragma unroll
+                for (int j = 0; j < 16; j++) hn[j] = __builtin_nanf("");
+            }
+            // every summary is in registers (the fold consumed them); the last of the nchunk - 1 folding waves of this
+            // (batch row, channel tile) leaves the pair's flags and counter zero for the next launch
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            unsigned *fl = flags + ((int64_t)b * tiles + tile) * kMaxChunks;
+            unsigned *dn = done + (int64_t)b * tiles + tile;
+            unsigned old = 0;
+            if (threadIdx.x == 0) old = __hip_atomic_fetch_add(dn, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            old = __builtin_amdgcn_readfirstlane(old);
+            if (old == (unsigned)(nchunk - 2)) {
+                if ((int)threadIdx.x < nchunk - 1) __hip_atomic_store(fl + threadIdx.x, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (threadIdx.x == 0) __hip_atomic_store(dn, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
     }
 #pragma unroll
     for (int r = 0; r < 16; r++) { hs[r] = hn[kStateOfReg(r)]; ar[r] = a2[kStateOfReg(r)]; }
@@ -729,19 +810,83 @@ __global__ __launch_bounds__(kWave) void chunk_out_kernel(
     }
 }
 
+template <typename T, bool S4D, int GATE>
+__global__ __launch_bounds__(kWave) void chunk_out_kernel(
+    float *__restrict__ h, T *__restrict__ y, const T *__restrict__ delta, const T *__restrict__ u,
+    const T *__restrict__ Bm, const T *__restrict__ Cm, int64_t bc_stride,
+    const float *__restrict__ a_neg, const float *__restrict__ Dp, const T *__restrict__ gate, int64_t gate_stride,
+    const float *__restrict__ h0copy, const float *__restrict__ S, const float *__restrict__ sumd,
+    int Tlen, int di, int tiles, int nchunk, int len) {
+    __shared__ alignas(16) StagedRows Bs, Cs;
+    const int tile = blockIdx.x % tiles;
+    const int rest = blockIdx.x / tiles;
+    const float unused[16] = {};
+    pass_b_body<T, S4D, GATE, false>(Bs, Cs, h, y, delta, u, Bm, Cm, bc_stride, a_neg, Dp, gate, gate_stride, h0copy, S, sumd, nullptr,
+                                     nullptr, unused, Tlen, di, tiles, nchunk, len, rest / nchunk, rest % nchunk, tile);
+}
+
+// Both passes in one launch: the wave (chunk c, batch row b, channel tile) summarises its chunk, publishes the summary,
+// waits for the chunks before it and walks its chunk again for the outputs.  Workgroups are numbered chunk-major, so a
+// wave only ever waits for waves with smaller indices (dispatched before it); the last chunk has nothing to summarise
+// and goes straight to waiting.  The flag area (kMaxChunks flags and a counter per (batch row, channel tile)) must be all
+// zero when the launch starts and is all zero again when it ends.
+template <typename T, bool S4D, int GATE>
+__global__ __launch_bounds__(kWave) void scan_fused_kernel(
+    float *__restrict__ h, T *__restrict__ y, const T *__restrict__ delta, const T *__restrict__ u,
+    const T *__restrict__ Bm, const T *__restrict__ Cm, int64_t bc_stride,
+    const float *__restrict__ a_neg, const float *__restrict__ Dp, const T *__restrict__ gate, int64_t gate_stride,
+    float *__restrict__ S, float *__restrict__ sumd, unsigned *__restrict__ flags, unsigned *__restrict__ done,
+    int batch, int Tlen, int di, int tiles, int nchunk, int len) {
+    __shared__ alignas(16) StagedRows Bs, Cs;
+    const int tile = blockIdx.x % tiles;
+    const int rest = blockIdx.x / tiles;
+    const int b = rest % batch, c = rest / batch;
+    float h_keep[16];
+#pragma unroll
+    for (int j = 0; j < 16; j++) h_keep[j] = 0.0f;
+    if (c < nchunk - 1)
+        pass_a_body<T, S4D, true>(Bs, h, delta, u, Bm, bc_stride, a_neg, nullptr, S, sumd, flags, h_keep, Tlen, di, tiles, nchunk, len, b, c, tile);
+    pass_b_body<T, S4D, GATE, true>(Bs, Cs, h, y, delta, u, Bm, Cm, bc_stride, a_neg, Dp, gate, gate_stride, nullptr, S, sumd, flags, done,
+                                    h_keep, Tlen, di, tiles, nchunk, len, b, c, tile);
+}
+
+// clears the flag area of the one-launch route (a kernel, not a memset: the call may be under stream capture)
+__global__ __launch_bounds__(256) void scan_flags_clear_kernel(unsigned *__restrict__ p, int n) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < n) p[i] = 0u;
+}
+
 template <typename T> struct IsF32 { static constexpr bool value = false; };
 template <> struct IsF32<float> { static constexpr bool value = true; };
 
+// one_launch: 0 = two launches (pass A, pass B); 1 = one launch behind a small kernel that clears the flag area;
+// 2 = one launch, the caller vouches that the flag area is all zero (MRS_SCAN_FLAGS_ZERO, or the library's own buffer)
 template <typename T, bool S4D>
 static int launch_split_s4d(hipStream_t st, int gate_mode, float *h, T *y, const T *delta, const T *u,
                             const T *Bm, const T *Cm, int64_t bc_stride, const float *a_neg,
                             const float *D, const T *gate, int64_t gate_stride, float *ws, SplitPlan plan, int batch,
-                            int Tlen, int di) {
+                            int Tlen, int di, int one_launch) {
     const int tiles = (di + kWave - 1) / kWave;
     const int C = plan.nchunk, L = plan.len;
     const SplitWs w = carve_workspace(ws, batch, Tlen, di, C);
     const dim3 block(kWave);
     const dim3 gridA((unsigned)(batch * (C - 1) * tiles)), gridB((unsigned)(batch * C * tiles));
+    if (one_launch) {
+        if (one_launch == 1) {
+            const int used = batch * tiles * (kMaxChunks + 1);   // the words this shape's waves touch
+            hipLaunchKernelGGL(scan_flags_clear_kernel, dim3((unsigned)((used + 255) / 256)), dim3(256), 0, st, w.flags, used);
+            int rc = check_launch("scan_flags_clear_kernel");
+            if (rc) return rc;
+        }
+#define MRS_LAUNCH(G)                                                                                        \
+    hipLaunchKernelGGL((scan_fused_kernel<T, S4D, G>), gridB, block, 0, st, h, y, delta, u, Bm, Cm, bc_stride, \
+                       a_neg, D, gate, gate_stride, w.S, w.sumd, w.flags, w.done, batch, Tlen, di, tiles, C, L)
+        if (gate_mode == 0) MRS_LAUNCH(0);
+        else if (gate_mode == 1) MRS_LAUNCH(1);
+        else MRS_LAUNCH(2);
+#undef MRS_LAUNCH
+        return check_launch("scan_fused_kernel");
+    }
     hipLaunchKernelGGL((chunk_state_kernel<T, S4D>), gridA, block, 0, st, h, delta, u, Bm, bc_stride, a_neg,
                        w.h0copy, w.S, w.sumd, Tlen, di, tiles, C, L);
     int rc = check_launch("chunk_state_kernel");
@@ -760,10 +905,10 @@ template <typename T>
 static int launch_split(hipStream_t st, bool s4d, int gate_mode, float *h, void *y, const void *delta,
                         const void *u, const void *Bm, const void *Cm, int64_t bc_stride,
                         const float *a_neg, const float *D, const void *gate, int64_t gate_stride, float *ws, SplitPlan plan,
-                        int batch, int Tlen, int di) {
+                        int batch, int Tlen, int di, int one_launch) {
 #define MRS_ARGS                                                                                       \
     st, gate_mode, h, (T *)y, (const T *)delta, (const T *)u, (const T *)Bm, (const T *)Cm, bc_stride, \
-        a_neg, D, (const T *)gate, gate_stride, ws, plan, batch, Tlen, di
+        a_neg, D, (const T *)gate, gate_stride, ws, plan, batch, Tlen, di, one_launch
     return s4d ? launch_split_s4d<T, true>(MRS_ARGS) : launch_split_s4d<T, false>(MRS_ARGS);
 #undef MRS_ARGS
 }
@@ -792,6 +937,11 @@ static int scan_check(const char *fn, int dtype, const void *h, const void *y, c
 
 using namespace mrs;
 
+extern "C" size_t mrs_ssm_scan_flag_bytes(int batch, int d_inner) {
+    (void)batch; (void)d_inner;   // one size for every shape
+    return kFlagAreaWords * sizeof(unsigned);
+}
+
 extern "C" size_t mrs_ssm_scan_workspace_bytes(int batch, int T, int d_inner, int d_state) {
     if (batch < 1 || T < 1 || d_inner < 1 || d_state != 16) return 256;
     const SplitPlan plan = make_split_plan(batch, T, d_inner);
@@ -804,7 +954,7 @@ extern "C" size_t mrs_ssm_scan_workspace_bytes(int batch, int T, int d_inner, in
 static int scan_dispatch(const char *fn, void *stream, int dtype, float *h, void *y, const void *delta, const void *u,
                          const void *B, const void *C, int64_t bc_stride, const float *a_neg, const float *D,
                          const void *gate, int64_t gate_stride, unsigned flags, void *workspace, size_t workspace_bytes,
-                         int batch, int T, int d_inner, int d_state) {
+                         int batch, int T, int d_inner, int d_state, bool own_buffer = false) {
     int rc = scan_check(fn, dtype, h, y, delta, u, B, C, a_neg, D, bc_stride, batch, T, d_inner, d_state);
     if (rc) return rc;
     int gate_mode = 0;
@@ -839,8 +989,19 @@ static int scan_dispatch(const char *fn, void *stream, int dtype, float *h, void
         if (workspace_bytes < need)
             return fail(MRS_E_WORKSPACE, "%s: workspace %zu bytes < %zu needed", fn, workspace_bytes, need);
         if (!aligned(workspace, 256)) return fail(MRS_E_ALIGN, "%s: workspace must be 256-byte aligned", fn);
+        // One launch for both passes where it wins: diagonal-real A (the per-step work of the general form hides the second
+        // launch already, and its longer waves wait longer on each other: 141 against 135 us at 8 x 2048 x 1536) and at
+        // least 2048 waves (a single 4096-step prompt at d_inner 2048 is 60 us in two launches, 63 in one).
+        // MRS_FORCE_PARALLEL takes the one launch at any size, MRS_SCAN_TWO_LAUNCHES (flag or environment) never does.
+        // The flag area is cleared by a small kernel first unless it is known to be zero (the caller's word, or the
+        // library's own buffer, which starts zeroed and is left zeroed by every launch).
+        static const bool env_two = [] { const char *e = getenv("MRS_SCAN_TWO_LAUNCHES"); return e && atoi(e) != 0; }();
+        const int64_t waves = (int64_t)batch * ((d_inner + kWave - 1) / kWave) * plan.nchunk;
+        const bool wins = (s4d && waves >= 2048) || (flags & MRS_FORCE_PARALLEL);
+        int one_launch = (env_two || (flags & MRS_SCAN_TWO_LAUNCHES) || !wins || !flags_fit(batch, d_inner)) ? 0
+                         : ((own_buffer || (flags & MRS_SCAN_FLAGS_ZERO)) ? 2 : 1);
         MRS_DISPATCH_DTYPE(dtype, T_, return launch_split<T_>(st, s4d, gate_mode, h, y, delta, u, B, C, bc_stride, a_neg, D, gate, gate_stride,
-                                                             (float *)workspace, plan, batch, T, d_inner));
+                                                             (float *)workspace, plan, batch, T, d_inner, one_launch));
     }
     MRS_DISPATCH_DTYPE(dtype, T_, return launch_seq<T_>(st, s4d, gate_mode, h, y, delta, u, B, C, bc_stride, a_neg, D, gate, gate_stride, batch, T, d_inner, d_state));
     return MRS_OK;
@@ -897,10 +1058,10 @@ extern "C" int mrs_ssm_scan_fwd_static(void *stream, int dtype, float *h, void *
     void *ws = nullptr;
     rc = static_scratch_for_current_device(fn, &ws);
     if (rc) return rc;
-    // Every float the second pass reads from the buffer is written by the first pass of the same call (chunk states,
-    // step sums, the copy of h), so nothing has to start at zero.
+    // Every float a wave reads from the buffer is written by another wave of the same call (chunk states, step sums);
+    // the flags those waves signal with start at zero (a file-scope device array does) and every launch leaves them zero.
     return scan_dispatch(fn, stream, dtype, h, y, delta, u, B, C, bc_stride, a_neg, D, gate, gate_stride, flags, ws,
-                         kStaticScanScratchBytes, batch, T, d_inner, d_state);
+                         kStaticScanScratchBytes, batch, T, d_inner, d_state, /*own_buffer=*/true);
 }
 
 extern "C" int mrs_ssm_scan_fwd(void *stream, int dtype, float *h, void *y, const void *delta,

@@ -19,6 +19,8 @@ GATE_SILU = 1 << 1
 A_S4D_REAL = 1 << 2
 FORCE_SEQUENTIAL = 1 << 3
 FORCE_PARALLEL = 1 << 4
+SCAN_FLAGS_ZERO = 1 << 5
+SCAN_TWO_LAUNCHES = 1 << 6
 
 
 def _stream() -> int:
@@ -72,6 +74,11 @@ def a_neg_is_s4d_real(a_neg: torch.Tensor) -> bool:
 
 def ssm_scan_workspace_bytes(batch: int, T: int, d_inner: int, d_state: int) -> int:
     return int(_lib.load().mrs_ssm_scan_workspace_bytes(batch, T, d_inner, d_state))
+
+
+def ssm_scan_flag_bytes(batch: int, d_inner: int) -> int:
+    """Leading bytes of a scan workspace that hold the one-launch route's flags (zero between calls)."""
+    return int(_lib.load().mrs_ssm_scan_flag_bytes(batch, d_inner))
 
 
 SCAN_STATIC_SCRATCH_BYTES = 16 << 20

@@ -190,6 +190,90 @@ def test_scan_full_size_channel_subset_and_linearity(shape):
     assert np.array_equal(h2, 2.0 * h1) and np.array_equal(y2, 2.0 * y1)
 
 
+@pytest.mark.parametrize("case", [
+    # batch, T, d_inner, dtype, S4D-real, gate mode
+    (3, 1000, 320, orc.BF16, True, 2),      # ragged last chunk, partial channel tile
+    (2, 300, 192, orc.F32, False, 0),
+    (1, 520, 128, orc.F16, True, 1),
+    (8, 2048, 1536, orc.BF16, True, 2),     # the benchmark shape
+    (4, 4096, 5120, orc.BF16, False, 2),    # the 2.8b-shape layer, general A
+])
+def test_scan_in_one_launch_equals_the_two_launch_route(case):
+    """The T-split route as one launch (every wave summarises its chunk, publishes the summary, waits for the chunks
+    before it) against the same two passes as two launches: the arithmetic is the same, so y and the final state must be
+    equal bit for bit -- with the flag area cleared by the op itself (the default), and vouched zero by the caller
+    (MRS_SCAN_FLAGS_ZERO) on three calls in a row over one workspace, which every call must leave all zero again.
+    MRS_FORCE_PARALLEL takes the one launch also where the library would not pick it (general A, few waves)."""
+    batch, T, di, dtype, s4d, gate_mode = case
+    ds = 16
+    rng = np.random.default_rng(T + di)
+    print(f"case one-launch scan {case}", flush=True)
+    inp = quantised(rng, batch, T, di, ds, dtype, s4d=s4d)
+    h0 = (rng.standard_normal((batch, di, ds)) * 0.1).astype(np.float32)
+    d = {k: dev(inp[k], dtype) for k in ("u", "delta", "B", "C", "z")}
+    a_neg, D = dev(inp["a_neg"]), dev(inp["D"])
+    base = GATE_FLAG[gate_mode] | (ops.A_S4D_REAL if s4d else 0)
+    gate = d["z"] if gate_mode else None
+    ws = torch.empty(ops.ssm_scan_workspace_bytes(batch, T, di, ds), dtype=torch.uint8, device=DEV).fill_(0xA5)
+    nflag = ops.ssm_scan_flag_bytes(batch, di)
+    assert 0 < nflag < ws.numel()
+
+    def run(extra):
+        h, y = dev(h0), torch.full_like(d["delta"], float("nan"))
+        ops.ssm_scan_fwd(h, y, d["delta"], d["u"], d["B"], d["C"], a_neg, D, gate=gate, flags=base | extra, workspace=ws)
+        torch.cuda.synchronize()
+        return y, h
+
+    y2, h2 = run(ops.SCAN_TWO_LAUNCHES)
+    assert torch.isfinite(y2.float()).all()
+    y1, h1 = run(ops.FORCE_PARALLEL)      # the flags this shape uses are cleared by the op (they held 0xA5 bytes)
+    assert torch.equal(y1, y2) and torch.equal(h1, h2)
+    ws[:nflag].zero_()                    # what a caller that passes MRS_SCAN_FLAGS_ZERO does once
+    for rep in range(3):
+        yz, hz = run(ops.SCAN_FLAGS_ZERO | ops.FORCE_PARALLEL)
+        assert torch.equal(yz, y2) and torch.equal(hz, h2), rep
+        assert int(ws[:nflag].max().item()) == 0, rep
+
+
+def test_scan_in_one_launch_replays_in_a_graph():
+    """The one-launch scan captured in a hipGraph (the static-scratch entry point: no workspace, nothing to clear) and
+    replayed with eager calls and synchronisations in between: every replay equals the eager result."""
+    rng = np.random.default_rng(77)
+    batch, T, di, ds = 2, 700, 256, 16
+    inp = quantised(rng, batch, T, di, ds, orc.BF16)
+    d = {k: dev(inp[k], orc.BF16) for k in ("u", "delta", "B", "C", "z")}
+    a_neg, D = dev(inp["a_neg"]), dev(inp["D"])
+    h0 = dev((rng.standard_normal((batch, di, ds)) * 0.1).astype(np.float32))
+    flags = ops.GATE_SILU | ops.A_S4D_REAL | ops.FORCE_PARALLEL     # the one launch although the shape is small
+
+    def call(h, y):
+        ops.ssm_scan_fwd(h, y, d["delta"], d["u"], d["B"], d["C"], a_neg, D, gate=d["z"], flags=flags, static_scratch=True)
+
+    h_e, y_e = h0.clone(), torch.empty_like(d["delta"])
+    call(h_e, y_e)
+    torch.cuda.synchronize()
+    h_g, y_g = h0.clone(), torch.empty_like(d["delta"])
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        call(h_g, y_g)                                  # warm-up on the capture stream
+        side.synchronize()
+        with torch.cuda.graph(g, stream=side):
+            call(h_g, y_g)
+    for rep in range(4):
+        print(f"case graph replay {rep}", flush=True)
+        h_g.copy_(h0); y_g.fill_(float("nan"))
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y_g, y_e) and torch.equal(h_g, h_e), rep
+        h_x, y_x = h0.clone(), torch.empty_like(d["delta"])
+        call(h_x, y_x)                                  # an eager call between replays shares the buffer, in stream order
+        torch.cuda.synchronize()
+        assert torch.equal(y_x, y_e)
+
+
 def test_scan_rejects_bad_arguments():
     rng = np.random.default_rng(5)
     inp = quantised(rng, 1, 4, 16, 16, orc.F32)
