@@ -40,6 +40,9 @@ _SIGNATURES = {
     "mrs_conv1d_step": (c_int, [_P, c_int, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int]),
     "mrs_conv1d_seq_silu": (c_int, [_P, c_int, _P, _P, _P, c_int64, _P, _P, c_int, c_int, c_int, c_int]),
     "mrs_gemm_skinny": (c_int, [_P, c_int, _P, c_int, c_int64, _P, c_int64, _P, c_int, c_int, c_int]),
+    "mrs_tiled_weight_bytes": (c_size_t, [c_int, c_int, c_int]),
+    "mrs_tile_weight": (c_int, [_P, c_int, _P, _P, c_int, c_int]),
+    "mrs_gemm_tiled": (c_int, [_P, c_int, _P, c_int, c_int64, _P, c_int64, _P, c_int, c_int, c_int]),
     "mrs_transpose": (c_int, [_P, c_int, _P, _P, c_int, c_int]),
     "mrs_xoshiro_seed": (None, [c_uint64, POINTER(c_uint64)]),
     "mrs_sample_tokens": (c_int, [_P, _P, _P, _P, c_int64, c_int, c_int, _P, _P, _P, _P]),

@@ -80,11 +80,18 @@ int check_launch(const char *what);
 // Internal launchers shared with the backbone engine (strides and fusions the public entry points do not expose).
 // StepFold: the step kernel forms the x_proj row itself from per-tile shares [n_tiles][rows][xd] f32 (summed in tile
 // order, rounded to the storage type); dt input at element 0, B at b_off, C at c_off of the row.
-struct StepFold { const float *xpart; int n_tiles, rows, xd, b_off, c_off; };
+// y_mt != 0: y is written in the tiled order of tiled_a_index (y_mt row tiles) instead of row-major.
+struct StepFold { const float *xpart; int n_tiles, rows, xd, b_off, c_off, y_mt; };
+// Element (row, k) of an activation matrix stored as the matrix-core A operand in lane order -- [k-step][row tile][lane][8],
+// lane = row % 16 + 16 * ((k % 32) / 8), mt row tiles of 16 rows -- so that a wave's load of one operand piece is one
+// contiguous kilobyte (gemm_wide.hip reads it; the kernels that produce such a matrix write it this way).
+__host__ __device__ inline int64_t tiled_a_index(int row, int k, int mt) {
+    return ((((int64_t)(k >> 5) * mt + (row >> 4)) * 64 + (row & 15) + 16 * ((k >> 3) & 3)) << 3) + (k & 7);
+}
 int launch_ssm_step_fused(hipStream_t st, int dtype, float *h, void *y, const void *delta, const float *dt_bias,
                           const void *dt_in, const void *dt_w, int dr, int dt_transposed, const void *u, const void *Bb, const void *Cb, int64_t bc_stride, const void *gate,
                           int64_t gate_stride, int gate_mode, const float *a_neg, const float *D, int batch,
-                          int di, int ds, const StepFold *fold = nullptr);
+                          int di, int ds, const StepFold *fold = nullptr, int y_mt = 0);
 int launch_conv1d_step(hipStream_t st, int dtype, void *out, float *state, const void *new_x, int64_t x_stride,
                        const float *weight, const float *bias, int batch, int d_inner, int d_conv, int apply_silu);
 
@@ -117,7 +124,20 @@ struct SkinnyEpi {
     // x_proj of a wide model is 12 tiles over K = 5120)
     int ksplit;
     int kslice;          // set by the launcher: 32-wide k-steps per slice
+    // tiled route (gemm_wide.hip) only: A is stored [k-step][row tile][lane][8] -- the matrix-core operand in lane order, 16-row
+    // tiles (tiled_a_index), rows past M present with any contents -- instead of row-major
+    int a_tiled;
+    int prenorm_mt;      // mode 2: != 0 writes prenorm in that tiled order (prenorm_mt row tiles) for the next tiled in_proj
 };
+// The same products from a TILED weight (gemm_wide.hip): 5..64 rows over a weight of megabytes.  Wp holds the 16 columns x 32 k
+// of each matrix-core operand as 1 KB in lane order, column tile by column tile (launch_tile_weight builds it from the
+// transposed weight Wt[N][K]; tiled_weight_elems() elements, columns padded to a multiple of 16).  Same epilogues, except
+// the x_proj shares (SkinnyEpi::xw, ksplit).
+bool tiled_gemm_ok(int dtype, int M, int N, int K, int64_t lda, const void *A, const void *Wp);
+size_t tiled_weight_elems(int N, int K);
+int launch_tile_weight(hipStream_t st, int dtype, void *Wp, const void *Wt, int N, int K);
+int launch_tiled_gemm(hipStream_t st, int dtype, void *C, int out_f32, int64_t ldc, const void *A, int64_t lda, const void *Wp, int M,
+                      int N, int K, const SkinnyEpi &ep);
 int skinny_max_rows();   // rows the 16-bit matrix-core route takes (128; MRS_SKINNY_MAX_ROWS overrides)
 bool skinny_gemm_ok(int dtype, int M, int N, int K, int64_t lda, const void *A, const void *Wt);
 int launch_skinny_gemm(hipStream_t st, int dtype, void *C, int out_f32, int64_t ldc, const void *A, int64_t lda, const void *Wt,
@@ -157,8 +177,9 @@ bool dt_proj_softplus_ok(int dtype, int di, int dr, int64_t xs, const void *delt
 int launch_dt_proj_softplus(hipStream_t st, int dtype, void *delta, const void *dt_in, int64_t xs, const void *wt, const float *bias,
                             int64_t rows, int di, int dr);
 // partials[row][0] = sum_k x[row][k]^2, partials[row][1..n_partials) = 0; prenorm[row][k] = round(x[row][k] * w[k])
+// a_mt != 0: prenorm is written in the tiled order of tiled_a_index with a_mt row tiles
 int launch_prenorm_rows(hipStream_t st, int dtype, float *partials, int n_partials, void *prenorm, const float *x, float *copy_to,
-                        const float *w, int M, int K);
+                        const float *w, int M, int K, int a_mt = 0);
 
 // mrs_m3_ssd_fwd with x read in place out of wider rows (x_stride elements apart, 0 = dense; 16-bit storage only).
 // With `gen` the kernel forms K and Q itself (K and Q are not read and may be null): K = rot(angle, bn + b_bias[head]),

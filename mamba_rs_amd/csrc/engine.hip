@@ -213,6 +213,7 @@ struct LayerDev {
     void *dt_w_t;  // [d_inner][dt_rank] copy: the fused decode step (when dt_t_step) and the prefill dt_proj+softplus kernel read it
     int dt_t_step;
     void *in_proj_t, *x_proj_t, *out_proj_t;  // [N][K] copies: in / out for every 16-bit engine (own GEMM and vendor GEMM read them), x for the own chain only
+    void *in_proj_p, *out_proj_p;  // tiled copies (gemm_wide.hip): wide models at 5..64 rows
     int s4d;
 };
 
@@ -262,6 +263,7 @@ struct mrs_backbone {
     mrs_m1_config cfg;
     int input_dim, batch, dtype, di, dr, xd, identity_proj, device;
     const float *step_src;  // decode step: where layer 0 reads its input rows (null: the residual buffer itself)
+    int tiled;   // own chain with in_proj / out_proj from tiled weights and tiled activation operands (wide models, 5..64 rows)
     int skinny;  // decode projections on the library's own GEMM (16-bit storage: batch <= 128 or 64, K % 32 == 0; f32: batch <= 4, K % 128 == 0)
     hipStream_t stream;
     rocblas_handle blas;
@@ -310,12 +312,14 @@ static int alloc_scratch(mrs_backbone *bb, Scratch *s, int64_t rows, int T) {
     const int dm = bb->cfg.d_model, di = bb->di, xd = bb->xd;
     s->rows = rows; s->T = T;
     MRS_TRY(dev_alloc(bb, (void **)&s->residual, rows * dm * sizeof(float)));
-    MRS_TRY(dev_alloc(bb, &s->normed, rows * dm * es));
+    // the tiled chain keeps the operands of in_proj and out_proj in 16-row tiles
+    const int64_t rows16 = (T == 1 && bb->tiled) ? (rows + 15) / 16 * 16 : rows;
+    MRS_TRY(dev_alloc(bb, &s->normed, rows16 * dm * es));
     MRS_TRY(dev_alloc(bb, &s->proj, rows * 2 * di * es));
     MRS_TRY(dev_alloc(bb, &s->u, rows * di * es));
     MRS_TRY(dev_alloc(bb, &s->xdbl, rows * xd * es));
     MRS_TRY(dev_alloc(bb, &s->delta, rows * di * es));
-    MRS_TRY(dev_alloc(bb, &s->y, rows * di * es));
+    MRS_TRY(dev_alloc(bb, &s->y, rows16 * di * es));
     MRS_TRY(dev_alloc(bb, &s->out, rows * dm * es));
     if (T == 1) MRS_TRY(dev_alloc(bb, (void **)&s->partials, rows * (size_t)((dm + 15) / 16) * sizeof(float)));
     if (T == 1 && bb->skinny) {
@@ -398,45 +402,62 @@ static int decode_chain(mrs_backbone *bb, Scratch *s, int r0, int nr, hipStream_
     char *out = (char *)s->out + (size_t)r0 * dm * es;
     float *xpart = s->xpart ? s->xpart + (size_t)r0 * (di / 16) * xd : nullptr;   // [tile][nr][xd] blocks, one per slice
     const char *z = proj + (size_t)di * es;  // gate half of in_proj's output
+    // tiled chain (the whole batch as one chain): normed and y are stored as matrix-core operands in 16-row tiles
+    const int a_mt = (bb->tiled && r0 == 0 && nr == B) ? (nr + 15) / 16 : 0;
+    // batch * dt_rank up to which dt_proj rides in the step kernel.  On the tiled chain the alternative is an x_proj launch
+    // that cannot split K (nobody would sum the shares): 12.5 us at 32 and 64 rows of the 2.8b shape, against 4.7 us split.
+    // Per step at that shape, dt_proj in the step kernel / on its own: 32 rows 3.57 / 3.84 ms, 48 rows 4.32 / 4.34, 64 rows 5.04 / 4.89.
+    static const int64_t wide_fuse = [] { const char *e = getenv("MRS_DECODE_FUSE_DT_LIMIT"); return e ? (int64_t)atoll(e) : (int64_t)6400; }();
+    const int64_t fuse_limit = a_mt ? wide_fuse : kFuseDtProjLimit;
     for (int l = 0; l < L; l++) {
         const LayerDev &lw = bb->layers[l];
         float *conv = bb->conv_state + ((size_t)l * B + r0) * di * dc;
         float *ssm = bb->ssm_state + ((size_t)l * B + r0) * di * ds;
         if (l == 0) {
             const float *src = bb->step_src ? bb->step_src + (size_t)r0 * dm : residual;
-            MRS_TRY(launch_prenorm_rows(st, dt, partials, P, normed, src, bb->step_src ? residual : nullptr, lw.norm_w, nr, dm));
+            MRS_TRY(launch_prenorm_rows(st, dt, partials, P, normed, src, bb->step_src ? residual : nullptr, lw.norm_w, nr, dm, a_mt));
         }
         SkinnyEpi inp = {};
         inp.mode = 1; inp.conv_state = conv; inp.conv_w = lw.conv_w; inp.conv_b = lw.conv_b; inp.u = u; inp.di = di; inp.dc = dc;
         inp.row_scale = 1; inp.partials = partials; inp.n_partials = P; inp.eps = bb->cfg.rms_norm_eps;
         const bool fold_x = xpart && nr <= fold_rows_for(di, xd) && xd <= 256 && (int64_t)(di / 16) * nr * xd <= s->xpart_floats && lw.dt_t_step &&
-                            di % (1024 / ds) == 0 && dr % 4 == 0 && (int64_t)nr * dr <= kFuseDtProjLimit;
+                            di % (1024 / ds) == 0 && dr % 4 == 0 && (int64_t)nr * dr <= fuse_limit;
         if (fold_x) { inp.xw = lw.x_proj; inp.xd = xd; inp.xpart = xpart; }
         // x_proj as a launch of its own: K split into slices when the step kernel can sum the shares
-        const bool step_sums = xpart && xd <= 256 && lw.dt_t_step && di % (1024 / ds) == 0 && dr % 4 == 0 && (int64_t)nr * dr <= kFuseDtProjLimit;
+        const bool step_sums = xpart && xd <= 256 && lw.dt_t_step && di % (1024 / ds) == 0 && dr % 4 == 0 && (int64_t)nr * dr <= fuse_limit;
         const int ksplit = (!fold_x && step_sums && dt != MRS_F32) ? xproj_slices(nr, xd, di) : 1;
         const StepFold fold = {xpart, fold_x ? di / 16 : ksplit, nr, xd, dr, dr + ds};
-        MRS_TRY(launch_skinny_gemm(st, dt, proj, 0, 2 * di, normed, dm, lw.in_proj_t, nr, 2 * di, dm, inp));
+        if (a_mt) {
+            inp.a_tiled = 1;
+            MRS_TRY(launch_tiled_gemm(st, dt, proj, 0, 2 * di, normed, dm, lw.in_proj_p, nr, 2 * di, dm, inp));
+        } else {
+            MRS_TRY(launch_skinny_gemm(st, dt, proj, 0, 2 * di, normed, dm, lw.in_proj_t, nr, 2 * di, dm, inp));
+        }
         const SkinnyEpi none = {};
         if (!fold_x) {
             SkinnyEpi xp = {};
             if (ksplit > 1) { xp.ksplit = ksplit; xp.xpart = xpart; }
             MRS_TRY(launch_skinny_gemm(st, dt, xdbl, 0, xd, u, di, lw.x_proj_t, nr, xd, di, xp));
         }
-        if ((int64_t)nr * dr > kFuseDtProjLimit && lw.dt_w_t && skinny_gemm_ok(dt, nr, di, dr, xd, xdbl, lw.dt_w_t)) {
+        if ((int64_t)nr * dr > fuse_limit && lw.dt_w_t && skinny_gemm_ok(dt, nr, di, dr, xd, xdbl, lw.dt_w_t)) {
             // wide dt_rank at a large batch: dt_proj as a GEMM of its own, bias + softplus in the step kernel
             MRS_TRY(launch_skinny_gemm(st, dt, delta, 0, di, xdbl, xd, lw.dt_w_t, nr, di, dr, none));
             MRS_TRY(launch_ssm_step_fused(st, dt, ssm, y, delta, lw.dt_b, nullptr, nullptr, 0, 0, u, xdbl + es * dr, xdbl + es * (dr + ds), xd, z,
-                                          2 * di, 2, lw.a_neg, lw.D, nr, di, ds));
+                                          2 * di, 2, lw.a_neg, lw.D, nr, di, ds, nullptr, a_mt));
         } else {
             MRS_TRY(launch_ssm_step_fused(st, dt, ssm, y, delta, lw.dt_b, xdbl, lw.dt_t_step ? lw.dt_w_t : lw.dt_w, dr, lw.dt_t_step, u,
                                           xdbl + es * dr, xdbl + es * (dr + ds), xd, z, 2 * di, 2, lw.a_neg, lw.D, nr, di, ds,
-                                          (fold_x || ksplit > 1) ? &fold : nullptr));
+                                          (fold_x || ksplit > 1) ? &fold : nullptr, a_mt));
         }
         SkinnyEpi outp = {};
         outp.mode = 2; outp.residual = residual; outp.partials = partials; outp.n_partials = P;
         outp.next_norm_w = l + 1 < L ? bb->layers[l + 1].norm_w : nullptr; outp.prenorm = normed;
-        MRS_TRY(launch_skinny_gemm(st, dt, out, 0, dm, y, di, lw.out_proj_t, nr, dm, di, outp));
+        if (a_mt) {
+            outp.a_tiled = 1; outp.prenorm_mt = a_mt;
+            MRS_TRY(launch_tiled_gemm(st, dt, out, 0, dm, y, di, lw.out_proj_p, nr, dm, di, outp));
+        } else {
+            MRS_TRY(launch_skinny_gemm(st, dt, out, 0, dm, y, di, lw.out_proj_t, nr, dm, di, outp));
+        }
     }
     return MRS_OK;
 }
@@ -567,8 +588,16 @@ extern "C" int mrs_backbone_create(mrs_backbone **out, int gpu_ordinal, const mr
         // vendor kernels), measured: 128 at the 130m shape (1032 vs 1091 us per step; at 256 rows 1490 vs 1392), 40 at the
         // 2.8b shape (32 rows 5.13 vs 8.35 ms, 40 rows 5.74 vs 5.92, 48 rows 6.13 vs 5.98, 64 rows 7.58 vs 6.19).  "Narrow"
         // as for the x_proj shares.
-        const int max_rows = std::min(skinny_max_rows(), narrow_model(di, xd) ? 128 : 40);
+        // Wide models from 5 rows up: in_proj / out_proj stream tiled weights (gemm_wide.hip), which carries the own chain
+        // up to 64 rows.
+        static const bool no_tiled = [] { const char *e = getenv("MRS_DECODE_NO_TILED"); return e && atoi(e) != 0; }();
+        static const int tiled_max_rows = [] { const char *e = getenv("MRS_DECODE_TILED_MAX_ROWS"); return e ? atoi(e) : 64; }();
+        const bool pow2_state = ds == 4 || ds == 8 || ds == 16 || ds == 32 || ds == 64 || ds == 128 || ds == 256;
+        bb->tiled = !off && !no_tiled && (dtype == MRS_BF16 || dtype == MRS_F16) && batch >= 5 && batch <= std::min(tiled_max_rows, 64) &&
+                    dm % 32 == 0 && di % 32 == 0 && (int64_t)dm * 2 * di >= (int64_t)8 << 20 && pow2_state && !narrow_model(di, xd);
+        const int max_rows = std::min(skinny_max_rows(), narrow_model(di, xd) ? 128 : (bb->tiled ? 64 : 40));
         bb->skinny = !off && (dtype == MRS_BF16 || dtype == MRS_F16) && batch <= max_rows && dm % 32 == 0 && di % 32 == 0;
+        if (!bb->skinny) bb->tiled = 0;
         // f32 storage: the same chain on the row-wise route of the GEMM (one to four rows, rows of the operand in LDS)
         if (!off && dtype == MRS_F32 && batch <= 4 && dm % 128 == 0 && di % 128 == 0 && (int64_t)di * 16 <= 48 * 1024 &&
             getenv("MRS_DECODE_NO_ROWWISE") == nullptr)
@@ -593,7 +622,7 @@ extern "C" int mrs_backbone_create(mrs_backbone **out, int gpu_ordinal, const mr
         MRS_CREATE_TRY(upload_f32(bb, &d.dt_b, src.dt_proj_b, di));
         MRS_CREATE_TRY(upload_f32(bb, &d.D, src.d_param, di));
         MRS_CREATE_TRY(upload_bulk(bb, &d.out_proj, src.out_proj_w, (size_t)di * dm, stage));
-        d.in_proj_t = d.x_proj_t = d.out_proj_t = d.dt_w_t = nullptr;
+        d.in_proj_t = d.x_proj_t = d.out_proj_t = d.dt_w_t = d.in_proj_p = d.out_proj_p = nullptr;
         d.dt_t_step = (ds == 4 || ds == 8 || ds == 16 || ds == 32 || ds == 64 || ds == 128 || ds == 256) && dr % ds == 0 && xd % 4 == 0;
         if (d.dt_t_step || (bb->dtype != MRS_F32 && dr % 8 == 0)) {
             MRS_CREATE_TRY(dev_alloc(bb, &d.dt_w_t, (size_t)dr * di * esize(bb->dtype)));
@@ -607,6 +636,13 @@ extern "C" int mrs_backbone_create(mrs_backbone **out, int gpu_ordinal, const mr
             MRS_CREATE_TRY(dev_alloc(bb, &d.out_proj_t, (size_t)di * dm * es_));
             MRS_CREATE_TRY(launch_transpose(bb->stream, bb->dtype, d.in_proj_t, d.in_proj, dm, 2 * di));
             MRS_CREATE_TRY(launch_transpose(bb->stream, bb->dtype, d.out_proj_t, d.out_proj, di, dm));
+        }
+        if (bb->tiled) {
+            const size_t es_ = esize(bb->dtype);
+            MRS_CREATE_TRY(dev_alloc(bb, &d.in_proj_p, tiled_weight_elems(2 * di, dm) * es_));
+            MRS_CREATE_TRY(dev_alloc(bb, &d.out_proj_p, tiled_weight_elems(dm, di) * es_));
+            MRS_CREATE_TRY(launch_tile_weight(bb->stream, bb->dtype, d.in_proj_p, d.in_proj_t, 2 * di, dm));
+            MRS_CREATE_TRY(launch_tile_weight(bb->stream, bb->dtype, d.out_proj_p, d.out_proj_t, dm, di));
         }
         if (bb->skinny) {
             MRS_CREATE_TRY(dev_alloc(bb, &d.x_proj_t, (size_t)di * xd * esize(bb->dtype)));

@@ -15,26 +15,11 @@
 //     straight through the depthwise conv step + SiLU (conv1d_step_forward_silu, kernels/conv1d.cu:85-115)
 //     and only u and the gate half are written.
 #include "common.hpp"
+#include "mfma_tiles.hpp"
 #include <stdlib.h>
 #include <algorithm>
 
 namespace mrs {
-
-typedef float v4f __attribute__((ext_vector_type(4)));
-typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
-typedef _Float16 v8h __attribute__((ext_vector_type(8)));
-
-template <typename T> struct Mma32;
-template <> struct Mma32<bf16_t> {
-    __device__ static __forceinline__ v4f mma(uint4 a, uint4 b, v4f c) {
-        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, b), c, 0, 0, 0);
-    }
-};
-template <> struct Mma32<f16_t> {
-    __device__ static __forceinline__ v4f mma(uint4 a, uint4 b, v4f c) {
-        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, b), c, 0, 0, 0);
-    }
-};
 
 constexpr int kGemmWaves = 8;
 constexpr int kMaxConvTaps = 8;
@@ -360,7 +345,7 @@ __global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu
 template <typename T>
 __global__ __launch_bounds__(256) void prenorm_rows_kernel(float *__restrict__ partials, int n_partials, T *__restrict__ prenorm,
                                                            const float *__restrict__ x, float *__restrict__ copy_to,
-                                                           const float *__restrict__ w, int K) {
+                                                           const float *__restrict__ w, int K, int a_mt) {
     __shared__ float part[4];
     const int64_t row = blockIdx.x;
     float ss = 0.0f;
@@ -368,7 +353,7 @@ __global__ __launch_bounds__(256) void prenorm_rows_kernel(float *__restrict__ p
         const float v = x[row * K + i];
         ss = fmaf(v, v, ss);
         if (copy_to) copy_to[row * K + i] = v;   // the residual stream, when x is the step's input buffer
-        Store<T>::st(prenorm + row * K + i, v * w[i]);
+        Store<T>::st(prenorm + (a_mt ? tiled_a_index((int)row, i, a_mt) : row * K + i), v * w[i]);
     }
 #pragma unroll
     for (int m = 32; m >= 1; m >>= 1) ss += __shfl_xor(ss, m, kWave);
@@ -568,10 +553,10 @@ int launch_skinny_gemm(hipStream_t st, int dtype, void *C, int out_f32, int64_t 
 }
 
 int launch_prenorm_rows(hipStream_t st, int dtype, float *partials, int n_partials, void *prenorm, const float *x, float *copy_to,
-                        const float *w, int M, int K) {
-    if (dtype == MRS_BF16) hipLaunchKernelGGL((prenorm_rows_kernel<bf16_t>), dim3((unsigned)M), dim3(256), 0, st, partials, n_partials, (bf16_t *)prenorm, x, copy_to, w, K);
-    else if (dtype == MRS_F16) hipLaunchKernelGGL((prenorm_rows_kernel<f16_t>), dim3((unsigned)M), dim3(256), 0, st, partials, n_partials, (f16_t *)prenorm, x, copy_to, w, K);
-    else hipLaunchKernelGGL((prenorm_rows_kernel<float>), dim3((unsigned)M), dim3(256), 0, st, partials, n_partials, (float *)prenorm, x, copy_to, w, K);
+                        const float *w, int M, int K, int a_mt) {
+    if (dtype == MRS_BF16) hipLaunchKernelGGL((prenorm_rows_kernel<bf16_t>), dim3((unsigned)M), dim3(256), 0, st, partials, n_partials, (bf16_t *)prenorm, x, copy_to, w, K, a_mt);
+    else if (dtype == MRS_F16) hipLaunchKernelGGL((prenorm_rows_kernel<f16_t>), dim3((unsigned)M), dim3(256), 0, st, partials, n_partials, (f16_t *)prenorm, x, copy_to, w, K, a_mt);
+    else hipLaunchKernelGGL((prenorm_rows_kernel<float>), dim3((unsigned)M), dim3(256), 0, st, partials, n_partials, (float *)prenorm, x, copy_to, w, K, a_mt);
     return check_launch("prenorm_rows_kernel");
 }
 

@@ -1,0 +1,340 @@
+// Decode GEMM for wide models: C[M,N] = A[M,K] . W[K,N] with 5 <= M <= 64 rows (the batch) and a weight of megabytes
+// (in_proj of the 2.8b shape: 2560 x 10240, 52 MB), 16-bit operands, f32 accumulate on the matrix cores.
+//
+// The reference sends these products to the vendor GEMM (cuBLAS call sites src/mamba_ssm/gpu/blas.rs:1138-1163).  At
+// this size the product is one pass over the weight and nothing else, so the kernel is built around that stream:
+//   * the weight is kept TILED: the 16 columns x 32 k of one v_mfma_f32_16x16x32 B operand are 1 KB of consecutive
+//     memory in lane order (lane l: column l % 16, k = 8 (l / 16) .. +7), the k-steps of a column tile follow each other.
+//     A wave's load instruction then fetches one whole kilobyte and a wave streams a contiguous region -- with the
+//     row-major transposed copy the same instruction touches sixteen 64-byte pieces 2 K bytes apart (measured on the
+//     2.8b in_proj at 16 rows: 18.5 us tiled, 21.8 us row-major, the rest of the kernel being equal);
+//   * a workgroup of 8 waves owns 16 NT output columns (NT column tiles) over ALL of K and all rows; its waves split K
+//     into eight contiguous ranges, so every weight byte is requested once, by one wave, and no sum leaves the
+//     workgroup: the eight partial tiles meet in LDS (splitting K over workgroups instead, with the slices meeting in
+//     memory behind an arrival counter, cost 4-6 us of store / count / reload round trips at the end of a 12 us stream);
+//   * a wave keeps R k-steps of operand pieces requested ahead in registers, weight tiles and activation rows of the
+//     same k-step side by side in the order they are used (the activation rows come from L2: 16 rows x 64 bytes per
+//     piece); the loop is one software pipeline without barriers;
+//   * the epilogues are those of gemm_skinny.hip (plain store, in_proj's conv step + SiLU, out_proj's residual add with
+//     the row's sums of squares), applied to the accumulators where they are: lane l holds rows 4 (l / 16) .. +3 of
+//     column l % 16 of a 16 x 16 tile, one tile per wave.
+#include "common.hpp"
+#include "mfma_tiles.hpp"
+#include <stdlib.h>
+#include <algorithm>
+
+namespace mrs {
+namespace {
+
+constexpr int kTiledWaves = 8;
+constexpr int kTiledThreads = kTiledWaves * 64;
+
+template <typename T, int MT, int NT, int R>
+__global__ __launch_bounds__(kTiledThreads) void tiled_gemm_kernel(void *__restrict__ Cv, int out_f32, int64_t ldc, const T *__restrict__ A,
+                                                                   int64_t lda, const T *__restrict__ Wp, int M, int N, int K, SkinnyEpi ep) {
+    __shared__ v4f red[kTiledWaves / 2][MT * NT][kWave];
+    __shared__ float inv_s[16 * MT];
+    const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), l = tid & 63, lr = l & 15, lg = l >> 4;
+    const int nks = K >> 5, per = (nks + kTiledWaves - 1) / kTiledWaves;
+    // wave w takes k-steps w, w + 8, w + 16, ...: at any moment the eight waves of the workgroup are reading eight
+    // consecutive kilobytes of each column tile
+    const int ntiles = (N + 15) >> 4;
+    // Operands through buffer resources that end where K ends: a piece past the end arrives as zeros and costs no memory
+    // traffic, so the loop below has no tail and no branch -- every wave runs the same ceil(per / R) rounds and the
+    // compiler can count the loads in flight exactly.
+    __amdgpu_buffer_rsrc_t wres[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; nt++) {
+        const T *base = Wp + (int64_t)min((int)blockIdx.x * NT + nt, ntiles - 1) * nks * 512;
+        wres[nt] = __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(base), 0, nks * 1024, 0x00020000);
+    }
+    // activation rows, row-major: the whole matrix is the range (a k-step past K meets zero weights; past the last row's
+    // end it is zero itself), rows past M repeat the last one.  Tiled (ep.a_tiled): [k-step][row tile][lane][8], the A
+    // operand in lane order like the weight, 16 MT rows.
+    const bool a_tiled = ep.a_tiled != 0;
+    const int a_records = a_tiled ? nks * MT * 1024 : (int)((((int64_t)(M - 1) * lda + K) * (int64_t)sizeof(T)));
+    const __amdgpu_buffer_rsrc_t ares = __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(A), 0, a_records, 0x00020000);
+    unsigned aoff[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; mt++)
+        aoff[mt] = a_tiled ? (unsigned)(mt * 1024 + 16 * l) : (unsigned)(((int64_t)min(16 * mt + lr, M - 1) * lda + 8 * lg) * (int64_t)sizeof(T));
+    const unsigned astep = a_tiled ? (unsigned)MT * 1024u : 64u;
+    const unsigned woff = 16u * (unsigned)l;
+    auto ldw = [&](int nt, int s_) {
+        return __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(wres[nt], woff, 1024u * (unsigned)(w + kTiledWaves * s_), 0));
+    };
+    auto lda_ = [&](int mt, int s_) {
+        const int ks = w + kTiledWaves * s_;
+        const unsigned so = ks < nks ? astep * (unsigned)ks : (unsigned)a_records;
+        return __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(ares, aoff[mt], so, 0));
+    };
+    // Epilogue work is spread over all threads: element e = tid + 512 j of the workgroup's MT NT tiles of 256 -- tile
+    // e / 256, row (e % 256) / 16 and column e % 16 of it -- so sixteen consecutive lanes share a row.  With one element
+    // per thread its epilogue operands (conv window, taps and bias; or residual and next norm weight) are requested
+    // here, ahead of the operand stream, and wait in registers.
+    constexpr int kTiles = MT * NT;
+    constexpr int EP = (kTiles + 1) / 2;
+    constexpr bool kPrefetch = EP == 1;
+    const int e_row0 = (tid >> 4) & 15, e_nl = tid & 15;
+    float4 pf_win = make_float4(0.f, 0.f, 0.f, 0.f), pf_tap = pf_win;
+    float pf_x = 0.0f, pf_y = 0.0f;
+    if constexpr (kPrefetch) {
+        const int tile = tid >> 8;
+        const int row = 16 * (tile / NT) + e_row0, col = 16 * ((int)blockIdx.x * NT + tile % NT) + e_nl;
+        if (tile < kTiles && row < M && col < N) {
+            if (ep.mode == 1 && col < ep.di && ep.dc == 4) {
+                pf_win = *reinterpret_cast<const float4 *>(ep.conv_state + ((int64_t)row * ep.di + col) * 4);
+                pf_tap = *reinterpret_cast<const float4 *>(ep.conv_w + (int64_t)col * 4);
+                pf_x = ep.conv_b[col];
+            } else if (ep.mode == 2) {
+                pf_x = ep.residual[(int64_t)row * N + col];
+                if (ep.next_norm_w) pf_y = ep.next_norm_w[col];
+            }
+        }
+    }
+    // RMSNorm folded around the product (gemm_skinny.hip): 1/rms of each row from its partial sums of squares.  Sixteen
+    // lanes share a row; its partial sums (up to 256 of them, a multiple of four) are requested here as 16-byte pieces,
+    // all at once and ahead of the operand stream -- summed one load at a time in a loop they were ten L2 round trips in
+    // a row before the first matrix instruction (5.5 us of a 21 us in_proj at d_model 2560).
+    constexpr int kScalePasses = MT > 2 ? 2 : 1;       // 32 rows per pass
+    const bool ps_fast = ep.row_scale && ep.n_partials % 4 == 0 && ep.n_partials <= 256;
+    float4 ps[kScalePasses][4];
+    if (ps_fast) {
+#pragma unroll
+        for (int h = 0; h < kScalePasses; h++) {
+            const float *pp = ep.partials + (int64_t)min((tid >> 4) + 32 * h, M - 1) * ep.n_partials;
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const int p4 = 4 * ((tid & 15) + 16 * q);
+                ps[h][q] = p4 < ep.n_partials ? *reinterpret_cast<const float4 *>(pp + p4) : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+        }
+    }
+    uint4 wr[R][NT], ar[R][MT];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+#pragma unroll
+        for (int nt = 0; nt < NT; nt++) wr[r][nt] = ldw(nt, r);
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) ar[r][mt] = lda_(mt, r);
+        __builtin_amdgcn_sched_barrier(0);   // requested in the order of use, as in the loop (the wait counts of its first round follow this order)
+    }
+    // RMSNorm folded around the product (gemm_skinny.hip), second half: the partial sums requested above are in
+    if (ep.row_scale) {
+        if (ps_fast) {
+#pragma unroll
+            for (int h = 0; h < kScalePasses; h++) {
+                float ss = 0.0f;
+#pragma unroll
+                for (int q = 0; q < 4; q++) ss += (ps[h][q].x + ps[h][q].y) + (ps[h][q].z + ps[h][q].w);
+#pragma unroll
+                for (int m = 8; m >= 1; m >>= 1) ss += __shfl_xor(ss, m, kWave);
+                float rms = sqrtf(ss / (float)K + ep.eps);
+                if (!isfinite(rms) || rms < 1e-20f) rms = 1.0f;
+                const int r = (tid >> 4) + 32 * h;
+                if ((tid & 15) == 0 && r < 16 * MT) inv_s[r] = 1.0f / rms;
+            }
+        } else {
+            for (int r = tid >> 4; r < 16 * MT; r += kTiledThreads / 16) {
+                const float *pp = ep.partials + (int64_t)min(r, M - 1) * ep.n_partials;
+                float ss = 0.0f;
+                for (int p = tid & 15; p < ep.n_partials; p += 16) ss += pp[p];
+#pragma unroll
+                for (int m = 8; m >= 1; m >>= 1) ss += __shfl_xor(ss, m, kWave);
+                float rms = sqrtf(ss / (float)K + ep.eps);
+                if (!isfinite(rms) || rms < 1e-20f) rms = 1.0f;
+                if ((tid & 15) == 0) inv_s[r] = 1.0f / rms;
+            }
+        }
+    }
+    v4f acc[MT][NT];
+#pragma unroll
+    for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+        for (int nt = 0; nt < NT; nt++) acc[mt][nt] = (v4f){0.f, 0.f, 0.f, 0.f};
+    for (int kb = 0; kb < per; kb += R) {
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+#pragma unroll
+            for (int nt = 0; nt < NT; nt++)
+#pragma unroll
+                for (int mt = 0; mt < MT; mt++) acc[mt][nt] = Mma32<T>::mma(ar[r][mt], wr[r][nt], acc[mt][nt]);
+#pragma unroll
+            for (int nt = 0; nt < NT; nt++) wr[r][nt] = ldw(nt, kb + r + R);
+#pragma unroll
+            for (int mt = 0; mt < MT; mt++) ar[r][mt] = lda_(mt, kb + r + R);
+            __builtin_amdgcn_sched_barrier(0);   // keep each refill right behind its use: the scheduler would gather the loads at the end of the round
+        }
+    }
+    // the eight K ranges meet in LDS: the upper four waves park their tiles, the lower four add them and park the sums;
+    // the thread that owns an element then adds its four sums in wave order (one fixed order of additions)
+    if (w >= kTiledWaves / 2) {
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+            for (int nt = 0; nt < NT; nt++) red[w - kTiledWaves / 2][mt * NT + nt][l] = acc[mt][nt];
+    }
+    lds_barrier();
+    if (w < kTiledWaves / 2) {
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+            for (int nt = 0; nt < NT; nt++) red[w][mt * NT + nt][l] += acc[mt][nt];
+    }
+    lds_barrier();
+    T *C = reinterpret_cast<T *>(Cv);
+    float *Cf = reinterpret_cast<float *>(Cv);
+#pragma unroll
+    for (int j = 0; j < EP; j++) {
+        const int tile = (tid >> 8) + 2 * j;            // the same for a whole wave
+        if (tile >= kTiles) break;
+        // element (ml, nl) of a 16 x 16 tile sits in lane 16 (ml / 4) + nl, register ml % 4 of the accumulator
+        const int ml = e_row0, nl = e_nl, lane = (ml >> 2) * 16 + nl, i = ml & 3;
+        float s = red[0][tile][lane][i];
+#pragma unroll
+        for (int q = 1; q < kTiledWaves / 2; q++) s += red[q][tile][lane][i];
+        const int ctile = (int)blockIdx.x * NT + tile % NT;
+        const int row = 16 * (tile / NT) + ml, col = 16 * ctile + nl;
+        const bool valid = row < M && col < N;
+        if (ep.row_scale) s *= inv_s[row];
+        if (ep.mode == 2) {
+            // out_proj: residual += out (rounded to the storage type as the stored projection would be); the row's sum of
+            // squares over these 16 columns and the pre-scaled operand of the next layer's in_proj
+            float sq = 0.0f;
+            if (valid) {
+                const T orr = (T)s;
+                const float res_old = kPrefetch ? pf_x : ep.residual[(int64_t)row * N + col];
+                const float nw = kPrefetch ? pf_y : (ep.next_norm_w ? ep.next_norm_w[col] : 0.0f);
+                const float rn = res_old + Store<T>::ld(&orr);
+                ep.residual[(int64_t)row * N + col] = rn;
+                sq = rn * rn;
+                if (ep.next_norm_w)
+                    Store<T>::st(reinterpret_cast<T *>(ep.prenorm) + (ep.prenorm_mt ? tiled_a_index(row, col, ep.prenorm_mt) : (int64_t)row * N + col), rn * nw);
+            }
+#pragma unroll
+            for (int m = 8; m >= 1; m >>= 1) sq += __shfl_xor(sq, m, kWave);
+            if (nl == 0 && row < M && 16 * ctile < N) ep.partials[(int64_t)row * ep.n_partials + ctile] = sq;
+        } else if (!valid) {
+        } else if (ep.mode == 1 && col < ep.di) {
+            // conv step on the value as in_proj would have stored it (conv1d_step_forward_silu, kernels/conv1d.cu:85-115)
+            const T xr = (T)s;
+            const float xnew = Store<T>::ld(&xr);
+            float *st = ep.conv_state + ((int64_t)row * ep.di + col) * ep.dc;
+            const float *cw = ep.conv_w + (int64_t)col * ep.dc;
+            float o;
+            if (ep.dc == 4) {   // window and taps are one aligned 16-byte vector each
+                const float4 win = kPrefetch ? pf_win : *reinterpret_cast<const float4 *>(st);
+                const float4 tap = kPrefetch ? pf_tap : *reinterpret_cast<const float4 *>(cw);
+                o = kPrefetch ? pf_x : ep.conv_b[col];
+                o = fmaf(win.y, tap.x, o); o = fmaf(win.z, tap.y, o); o = fmaf(win.w, tap.z, o); o = fmaf(xnew, tap.w, o);
+                *reinterpret_cast<float4 *>(st) = make_float4(win.y, win.z, win.w, xnew);
+            } else {
+                o = ep.conv_b[col];
+                for (int k = 0; k < ep.dc; k++) {
+                    const float wk = (k + 1 < ep.dc) ? st[k + 1] : xnew;
+                    o = fmaf(wk, cw[k], o);
+                    st[k] = wk;
+                }
+            }
+            Store<T>::st(reinterpret_cast<T *>(ep.u) + (int64_t)row * ep.di + col, silu(o));
+        } else if (out_f32) {
+            Cf[(int64_t)row * ldc + col] = s;
+        } else {
+            Store<T>::st(C + (int64_t)row * ldc + col, s);
+        }
+    }
+}
+
+// Wp[column tile][k-step][lane][8] from the transposed weight Wt[N][K]; columns past N are zero
+template <typename T>
+__global__ __launch_bounds__(256) void tile_weight_kernel(uint4 *__restrict__ Wp, const T *__restrict__ Wt, int N, int K, int64_t pieces) {
+    const int64_t p = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (p >= pieces) return;
+    const int lane = (int)(p & 63), nks = K >> 5;
+    const int64_t t = p >> 6;
+    const int ks = (int)(t % nks);
+    const int col = (int)(t / nks) * 16 + (lane & 15);
+    Wp[p] = col < N ? *reinterpret_cast<const uint4 *>(Wt + (int64_t)col * K + 32 * ks + 8 * (lane >> 4)) : make_uint4(0, 0, 0, 0);
+}
+
+int env_int(const char *name, int dflt) {
+    const char *e = getenv(name);
+    return e ? atoi(e) : dflt;
+}
+
+template <typename T>
+int launch_tiled_t(hipStream_t st, void *C, int out_f32, int64_t ldc, const T *A, int64_t lda, const T *Wp, int M, int N, int K,
+                   const SkinnyEpi &ep) {
+    const int mt = (M + 15) / 16;
+    // two column tiles per workgroup where the rows are many (a k-step's activation pieces serve both) and the chip stays
+    // full of workgroups (2.8b in_proj at 16 rows: 15.1 us with one tile per workgroup, 17.5 us with two; at 64 rows the same)
+    static const int force_nt = env_int("MRS_TILED_NT", 0);
+    const int ntiles = (N + 15) / 16;
+    const int nt = force_nt ? force_nt : ((ntiles >= 512 && mt >= 2) ? 2 : 1);
+    const dim3 grid((unsigned)((ntiles + nt - 1) / nt)), block(kTiledThreads);
+#define MRS_TG(MT_, NT_, R_) \
+    hipLaunchKernelGGL((tiled_gemm_kernel<T, MT_, NT_, R_>), grid, block, 0, st, C, out_f32, ldc, A, lda, Wp, M, N, K, ep)
+    switch (mt * 10 + nt) {
+        case 11: MRS_TG(1, 1, 10); break;
+        case 12: MRS_TG(1, 2, 8); break;
+        case 21: MRS_TG(2, 1, 8); break;
+        case 22: MRS_TG(2, 2, 6); break;
+        case 31: MRS_TG(3, 1, 6); break;
+        case 32: MRS_TG(3, 2, 5); break;
+        case 41: MRS_TG(4, 1, 5); break;
+        default: MRS_TG(4, 2, 4); break;
+    }
+#undef MRS_TG
+    return check_launch("tiled_gemm_kernel");
+}
+
+}  // namespace
+
+bool tiled_gemm_ok(int dtype, int M, int N, int K, int64_t lda, const void *A, const void *Wp) {
+    return (dtype == MRS_BF16 || dtype == MRS_F16) && M >= 1 && M <= 64 && N >= 1 && K >= 32 && K % 32 == 0 && lda % 8 == 0 && aligned(A, 16) &&
+           aligned(Wp, 16);
+}
+
+size_t tiled_weight_elems(int N, int K) { return (size_t)((N + 15) / 16) * 16 * (size_t)K; }
+
+int launch_tile_weight(hipStream_t st, int dtype, void *Wp, const void *Wt, int N, int K) {
+    if ((dtype != MRS_BF16 && dtype != MRS_F16) || K < 32 || K % 32 != 0 || N < 1 || !aligned(Wp, 16) || !aligned(Wt, 16))
+        return fail(MRS_E_SHAPE, "tile weight: 16-bit storage, K %% 32 == 0, 16-byte aligned operands (dtype=%d N=%d K=%d)", dtype, N, K);
+    const int64_t pieces = (int64_t)((N + 15) / 16) * (K >> 5) * 64;
+    hipLaunchKernelGGL((tile_weight_kernel<uint16_t>), dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0, st, (uint4 *)Wp, (const uint16_t *)Wt, N, K, pieces);
+    return check_launch("tile_weight_kernel");
+}
+
+int launch_tiled_gemm(hipStream_t st, int dtype, void *C, int out_f32, int64_t ldc, const void *A, int64_t lda, const void *Wp, int M,
+                      int N, int K, const SkinnyEpi &ep) {
+    if (!tiled_gemm_ok(dtype, M, N, K, lda, A, Wp))
+        return fail(MRS_E_SHAPE, "tiled gemm: needs 16-bit storage, 1 <= M <= 64, K %% 32 == 0, lda %% 8 == 0, 16-byte aligned A and weight "
+                                 "(got dtype=%d M=%d N=%d K=%d lda=%lld)", dtype, M, N, K, (long long)lda);
+    if (ep.xw || (ep.mode == 0 && ep.ksplit > 1) || ep.mode < 0 || ep.mode > 2)
+        return fail(MRS_E_SHAPE, "tiled gemm: the x_proj shares ride on the 16-row tiles of the row-major route only");
+    if (dtype == MRS_BF16) return launch_tiled_t<bf16_t>(st, C, out_f32, ldc, (const bf16_t *)A, lda, (const bf16_t *)Wp, M, N, K, ep);
+    return launch_tiled_t<f16_t>(st, C, out_f32, ldc, (const f16_t *)A, lda, (const f16_t *)Wp, M, N, K, ep);
+}
+
+}  // namespace mrs
+
+using namespace mrs;
+
+extern "C" size_t mrs_tiled_weight_bytes(int dtype, int N, int K) {
+    if ((dtype != MRS_BF16 && dtype != MRS_F16) || N < 1 || K < 32 || K % 32 != 0) return 0;
+    return tiled_weight_elems(N, K) * 2;
+}
+
+extern "C" int mrs_tile_weight(void *stream, int dtype, void *Wp, const void *Wt, int N, int K) {
+    if (!Wp || !Wt) return fail(MRS_E_NULL, "mrs_tile_weight: null pointer");
+    return launch_tile_weight(as_stream(stream), dtype, Wp, Wt, N, K);
+}
+
+extern "C" int mrs_gemm_tiled(void *stream, int dtype, void *C, int out_f32, int64_t ldc, const void *A, int64_t lda, const void *Wp,
+                              int M, int N, int K) {
+    if (!C || !A || !Wp) return fail(MRS_E_NULL, "mrs_gemm_tiled: null pointer");
+    if (ldc < N) return fail(MRS_E_SHAPE, "mrs_gemm_tiled: ldc=%lld < N=%d", (long long)ldc, N);
+    if (lda < K) return fail(MRS_E_SHAPE, "mrs_gemm_tiled: lda=%lld < K=%d", (long long)lda, K);
+    SkinnyEpi ep = {};
+    return launch_tiled_gemm(as_stream(stream), dtype, C, out_f32, ldc, A, lda, Wp, M, N, K, ep);
+}

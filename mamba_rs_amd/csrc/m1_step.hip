@@ -192,7 +192,7 @@ __global__ __launch_bounds__(256) void ssm_step_kernel(
             acc = fmaf(Dd, uu, acc);
             if (gate_mode == 1) acc *= gz;
             if (gate_mode == 2) acc *= silu(gz);
-            Store<T>::st(y + r, acc);
+            Store<T>::st(y + (fold.y_mt ? tiled_a_index(b, d, fold.y_mt) : r), acc);
         }
     }
 }
@@ -240,7 +240,7 @@ static int launch_step(hipStream_t st, float *h, void *y, const void *delta, con
                        const void *Bb, const void *Cb, int64_t bc_stride, const void *gate,
                        int64_t gate_stride, int gate_mode, const float *dt_bias, const void *dt_in,
                        const void *dt_w, int dr, int dt_transposed, const float *a_neg, const float *D, int batch, int di, int ds,
-                       const StepFold *fold = nullptr) {
+                       const StepFold *fold = nullptr, int y_mt = 0) {
     const int64_t total = (int64_t)batch * di;
     if (!gate) gate_mode = 0;
 #define MRS_ARGS h, (T *)y, (const T *)delta, (const T *)u, (const T *)Bb, (const T *)Cb, bc_stride, \
@@ -268,12 +268,15 @@ static int launch_step(hipStream_t st, float *h, void *y, const void *delta, con
                   dr <= fold->xd))
                 return fail(MRS_E_SHAPE, "ssm step: folded x_proj needs xd <= %d, d_inner %% %d == 0, 4-aligned B/C offsets, transposed dt_w",
                             kFoldMaxXd, 256 / lg);
-#define MRS_LGF(L) case L: hipLaunchKernelGGL((ssm_step_kernel<T, L, 2, true, true>), grid, block, 0, st, MRS_ARGS, *fold); break
+            StepFold folded = *fold;
+            folded.y_mt = y_mt;
+#define MRS_LGF(L) case L: hipLaunchKernelGGL((ssm_step_kernel<T, L, 2, true, true>), grid, block, 0, st, MRS_ARGS, folded); break
             switch (lg) { MRS_LGF(1); MRS_LGF(2); MRS_LGF(4); MRS_LGF(8); MRS_LGF(16); MRS_LGF(32); MRS_LGF(64); }
 #undef MRS_LGF
             return check_launch("ssm_step_kernel");
         }
-        const StepFold nofold = {};
+        StepFold nofold = {};
+        nofold.y_mt = y_mt;
         // (delta source, vector B/C): the transposed dt_w route implies vector rows (checked above)
         const int variant = dt_mode == 2 ? 4 : dt_mode * 2 + (vec_bc ? 1 : 0);
 #define MRS_LGV(L, DT_, V_) hipLaunchKernelGGL((ssm_step_kernel<T, L, DT_, V_>), grid, block, 0, st, MRS_ARGS, nofold)
@@ -291,7 +294,7 @@ static int launch_step(hipStream_t st, float *h, void *y, const void *delta, con
 #undef MRS_LG
 #undef MRS_LGV
     } else {
-        if (fold) return fail(MRS_E_SHAPE, "ssm step: folded x_proj needs d_state a power of two in 4..256");
+        if (fold || y_mt) return fail(MRS_E_SHAPE, "ssm step: folded x_proj and tiled y need d_state a power of two in 4..256");
         const int64_t blocks = (total + 255) / 256;
         if (blocks > 0x7fffffffLL) return fail(MRS_E_SHAPE, "ssm step: grid too large");
         hipLaunchKernelGGL((ssm_step_generic_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, st, MRS_ARGS);
@@ -304,9 +307,9 @@ int launch_ssm_step_fused(hipStream_t st, int dtype, float *h, void *y, const vo
                           const void *dt_in, const void *dt_w, int dr, int dt_transposed,
                           const void *u, const void *Bb, const void *Cb, int64_t bc_stride, const void *gate,
                           int64_t gate_stride, int gate_mode, const float *a_neg, const float *D, int batch,
-                          int di, int ds, const StepFold *fold) {
+                          int di, int ds, const StepFold *fold, int y_mt) {
     MRS_DISPATCH_DTYPE(dtype, T_, return launch_step<T_>(st, h, y, delta, u, Bb, Cb, bc_stride, gate, gate_stride, gate_mode,
-                                                         dt_bias, dt_in, dt_w, dr, dt_transposed, a_neg, D, batch, di, ds, fold));
+                                                         dt_bias, dt_in, dt_w, dr, dt_transposed, a_neg, D, batch, di, ds, fold, y_mt));
     return MRS_OK;
 }
 

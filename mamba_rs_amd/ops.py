@@ -186,6 +186,34 @@ def gemm_skinny(a, wt, *, out_f32: bool = False):
     return c
 
 
+def tile_weight(wt):
+    """The tiled copy of a transposed weight Wt[N,K] (f16/bf16): the operand of gemm_tiled; returns (tiled uint8 tensor, N)."""
+    if wt.dim() != 2 or not wt.is_contiguous():
+        raise ValueError("wt must be a contiguous [N,K] matrix")
+    _dev(wt)
+    N, K = wt.shape
+    dt = _act_dtype(wt)
+    nbytes = int(_lib.load().mrs_tiled_weight_bytes(int(dt), N, K))
+    if nbytes == 0:
+        raise ValueError("tile_weight: f16/bf16 storage and K % 32 == 0")
+    wp = torch.empty(nbytes, device=wt.device, dtype=torch.uint8)
+    _lib.call("mrs_tile_weight", _stream(), int(dt), _p(wp), _p(wt), N, K)
+    return wp, N
+
+
+def gemm_tiled(a, wp, N: int, *, out_f32: bool = False):
+    """C[M,N] = A[M,K] . W from the tiled weight of tile_weight (1 <= M <= 64 rows, 16-bit operands, f32 accumulate): the decode
+    projections of wide models, which the reference sends to cuBLAS (src/mamba_ssm/gpu/blas.rs:1138-1163)."""
+    _dev(wp)
+    if not a.is_cuda or a.dim() != 2 or a.stride(1) != 1:
+        raise ValueError("a must be a device matrix [M,K] with unit inner stride")
+    M, K = a.shape
+    dt = _act_dtype(a)
+    c = torch.empty(M, N, device=a.device, dtype=torch.float32 if out_f32 else a.dtype)
+    _lib.call("mrs_gemm_tiled", _stream(), int(dt), _p(c), 1 if out_f32 else 0, N, _p(a), a.stride(0), _p(wp), M, N, K)
+    return c
+
+
 def conv1d_seq_silu(u_out, state, x_branch, weight, bias):
     """Full-sequence causal conv + SiLU with state carry
     (conv1d_burnin_forward_nosave, kernels/conv1d.cu:209-315).

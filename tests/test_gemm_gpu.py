@@ -35,6 +35,51 @@ def test_gemm_skinny_matches_f64_matmul(shape, dtype, out_f32):
     assert_close(host(c), ref, orc.F32 if out_f32 else dtype, "C")
 
 
+# (M, N, K): the 2.8b decode projections at one to four 16-row tiles (whole and partly filled), N not a multiple of 16, a K
+# shorter than the eight waves' ranges, a K that does not divide by them
+TILED_SHAPES = [(16, 10240, 2560), (64, 10240, 2560), (5, 2560, 5120), (23, 2560, 5120), (40, 2560, 5120), (64, 2560, 5120),
+                (16, 200, 96), (33, 16, 32), (48, 1000, 1056), (1, 50, 256), (64, 8200, 64)]
+
+
+@pytest.mark.parametrize("dtype", [orc.BF16, orc.F16])
+@pytest.mark.parametrize("shape", TILED_SHAPES)
+def test_gemm_tiled_matches_f64_matmul(shape, dtype):
+    """The wide-model decode GEMM on a tiled weight (16 columns x 32 k of a matrix-core operand stored as one kilobyte):
+    the tiling of the transposed weight, then the product against a float64 matmul, storage-type and f32 results."""
+    M, N, K = shape
+    rng = np.random.default_rng(hash((shape, dtype)) & 0xFFFF)
+    a = quant(rng.standard_normal((M, K)).astype(np.float32), dtype)
+    w = quant((rng.standard_normal((K, N)) / np.sqrt(K)).astype(np.float32), dtype)
+    print(f"case gemm_tiled shape={shape} dtype={dtype}", flush=True)
+    wt = ops.transpose(dev(w, dtype))
+    wp, n = ops.tile_weight(wt)
+    assert n == N
+    # tile (column tile t, k-step s) holds, for lane l, the 8 elements Wt[16 t + l % 16][32 s + 8 (l / 16) .. +7]
+    tiles = host(wp.view(torch.int16)).reshape((N + 15) // 16, K // 32, 64, 8)
+    wt_bits = host(wt.view(torch.int16))
+    for t, s_, l in ((0, 0, 0), ((N - 1) // 16, K // 32 - 1, 37), ((N + 15) // 32, (K // 32) // 2, 63)):
+        col = 16 * t + l % 16
+        want = wt_bits[col, 32 * s_ + 8 * (l // 16): 32 * s_ + 8 * (l // 16) + 8] if col < N else np.zeros(8, np.int16)
+        assert np.array_equal(tiles[t, s_, l], want), (t, s_, l)
+    ref = a.astype(np.float64) @ w.astype(np.float64)
+    for out_f32 in (False, True):
+        c = ops.gemm_tiled(dev(a, dtype), wp, N, out_f32=out_f32)
+        assert_close(host(c), ref, orc.F32 if out_f32 else dtype, "C")
+    # strided rows of A
+    big = dev(np.concatenate([a, a], axis=1), dtype)
+    c = ops.gemm_tiled(big[:, K:], wp, N, out_f32=True)
+    assert_close(host(c), ref, orc.F32, "C from strided rows")
+
+
+def test_gemm_tiled_rejects_bad_arguments():
+    wt = torch.zeros(32, 64, device=DEV, dtype=torch.bfloat16)
+    wp, n = ops.tile_weight(wt)
+    with pytest.raises(RuntimeError, match="tiled gemm"):
+        ops.gemm_tiled(torch.zeros(65, 64, device=DEV, dtype=torch.bfloat16), wp, n)      # more than 64 rows
+    with pytest.raises(ValueError):
+        ops.tile_weight(torch.zeros(32, 48, device=DEV, dtype=torch.bfloat16))              # K % 32 != 0
+
+
 @pytest.mark.parametrize("shape", [(1, 300, 256), (1, 3072, 768), (2, 40, 512), (3, 33, 128), (4, 1536, 1536), (4, 7, 384)])
 def test_gemm_skinny_f32_storage_on_the_row_wise_route(shape):
     """f32 operands: one to four rows, lanes along the weight row, plain multiply-adds (K a multiple of 128)."""
