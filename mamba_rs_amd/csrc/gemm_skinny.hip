@@ -95,12 +95,39 @@ __global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu
     const T *wrow = Wt + (int64_t)min(n0 + lr, N - 1) * K + 8 * lg;
     const T *arow = A + (int64_t)min(m0 + lr, M - 1) * lda + 8 * lg;
     float inv = 1.0f;
+    // The partial sums of a row are requested together, before the operands stream, and added up after the product
+    // (in the order a loop over them would add them): loaded one at a time inside such a loop they were a chain of
+    // n_partials / 16 round trips to L2 ahead of the first operand request (ten at d_model 2560).
+    constexpr int kScaleAhead = 8;   // partial sums per lane requested ahead (d_model up to 2048; more would spill in_proj's variants); any beyond are loaded late
+    float psum[PRO == 1 ? kScaleAhead : 1];
+    auto row_scale_request = [&]() {
+        if (PRO == 1 && tid < 256) {
+            const float *pp = ep.partials + (int64_t)min(m0 + (tid >> 4), M - 1) * ep.n_partials;
+#pragma unroll
+            for (int j = 0; j < kScaleAhead; j++) {
+                const int p = (tid & 15) + 16 * j;
+                psum[j] = p < ep.n_partials ? pp[p] : 0.0f;
+            }
+        }
+    };
     auto row_scale = [&]() {
         if (PRO == 1 && tid < 256) {
             // epilogue thread (row tid/16, column tid%16): the 16 lanes of a row share the sum over the partials
             const float *pp = ep.partials + (int64_t)min(m0 + (tid >> 4), M - 1) * ep.n_partials;
             float ss = 0.0f;
-            for (int p = tid & 15; p < ep.n_partials; p += 16) ss += pp[p];
+#pragma unroll
+            for (int j = 0; j < kScaleAhead; j++) ss += psum[j];
+            if (ep.n_partials > 16 * kScaleAhead) {   // a wider row: the next eight per lane as one more round trip, then one at a time
+                float late[8];
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    const int p = (tid & 15) + 16 * (kScaleAhead + j);
+                    late[j] = p < ep.n_partials ? pp[p] : 0.0f;
+                }
+#pragma unroll
+                for (int j = 0; j < 8; j++) ss += late[j];
+                for (int p = (tid & 15) + 16 * (kScaleAhead + 8); p < ep.n_partials; p += 16) ss += pp[p];
+            }
 #pragma unroll
             for (int m = 8; m >= 1; m >>= 1) ss += __shfl_xor(ss, m, kWave);
             float rms = sqrtf(ss / (float)K + ep.eps);
@@ -140,7 +167,7 @@ __global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu
     // Requested up front, but on the matrix-core route behind the first round of operand loads: with several row
     // tiles the conv windows are a megabyte-scale read that would otherwise queue ahead of the operands.
     if constexpr (LPR != 0) {
-        row_scale();
+        row_scale_request();
         prefetch_epilogue();
         constexpr int NC = LPR == 64 ? 2 : 1;           // columns a lane works on (with 32 lanes per row each half-wave has its own)
         constexpr int JB = LPR == 64 ? 2 : 4;             // pieces per column requested together
@@ -219,6 +246,7 @@ __global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu
                 for (int t = 0; t < NC; t++) wv[t][j] = nx[t][j];
         }
         }
+        row_scale();
 #pragma unroll
         for (int t = 0; t < NC; t++)
 #pragma unroll
@@ -244,9 +272,9 @@ __global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu
         }
     };
     constexpr int kStride = kGemmWaves * kHalf;   // k-steps one half-batch covers across the workgroup's waves
+    row_scale_request();
     request(0, k_lo + w);
     request(1, k_lo + w + kStride);
-    row_scale();
     prefetch_epilogue();
     for (int base = k_lo + w; base < nk; base += 2 * kStride) {
 #pragma unroll
@@ -256,6 +284,7 @@ __global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu
         for (int s = 0; s < kHalf; s++) acc = Mma32<T>::mma(af[1][s], bf[1][s], acc);
         request(1, base + 3 * kStride);
     }
+    row_scale();
     // K-split reduction: upper half of the waves parks its tile in LDS, lower half adds and parks the sums
     if (w >= kGemmWaves / 2) red[w - kGemmWaves / 2][l] = acc;
     lds_barrier();   // LDS exchanges only: the epilogue's prefetched operands stay in flight
