@@ -778,7 +778,7 @@ def main():
             extras["mamba3_768_bf16"]["backbone"] = m3_engine_leg(batches=())
         if "lm28" in legs or args.big:
             extras["lm_2.8b_shape_bf16"] = lm_leg("2.8b-shape", dict(d_model=2560, d_state=16, d_conv=4, expand=2, n_layers=64), 50280,
-                                                  (4, 4096), [1, 16, 128], 128, shared_layer=not args.big, cpu_sample=(2, 64),
+                                                  (4, 4096), [1, 16, 64, 128], 128, shared_layer=not args.big, cpu_sample=(2, 64),
                                                   with_generate=False, gemm_tuning=tune, decode_graph=not args.lm_no_graph)
         out["extras"] = extras
     print(json.dumps(out))
