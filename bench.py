@@ -745,11 +745,11 @@ def main():
                      "kernels": ["scan_fused_kernel"],
                      "algorithmic_bytes_per_launch": nbytes, "median_launch_ms": g["median_launch_ms"],
                      # what the two kernels are bound by in fact: the instruction issue of the SIMDs (f32 without packed math)
-                     "issue": {"bound": "instruction issue (1024 SIMDs; two plain instructions per issue window of 2.02 ns from "
-                                        "two different waves, a DPP-operand instruction a whole window, v_exp / v_rcp / "
-                                        "v_mfma_f32_4x4x1 two windows)",
-                               "model_us_per_call": issue_us, "frac": (issue_us / us) if issue_us else None,
-                               "source": traffic_source},
+                     "valu": {"bound": "valu-issue",
+                              "model": "1024 SIMDs; two plain instructions per issue window of 2.02 ns from two different waves, a "
+                                       "DPP-operand instruction a whole window, v_exp / v_rcp / v_mfma_f32_4x4x1 two windows",
+                              "bound_us_per_call": issue_us, "achieved_us_per_call": us,
+                              "frac": (issue_us / us) if issue_us else None, "source": traffic_source},
                      # the same launch on the kernels a trained checkpoint's A takes (no S4D-real shortcut)
                      "general_A": {"bound": "hbm", "achieved": nbytes / gen_us / 1e3, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                                    "frac": nbytes / gen_us / 1e3 / HBM_PEAK_GBPS, "ms_per_step": g["general_a_ms_per_step"]}},

@@ -8,16 +8,26 @@
 //     A wave's load instruction then fetches one whole kilobyte and a wave streams a contiguous region -- with the
 //     row-major transposed copy the same instruction touches sixteen 64-byte pieces 2 K bytes apart (measured on the
 //     2.8b in_proj at 16 rows: 18.5 us tiled, 21.8 us row-major, the rest of the kernel being equal);
-//   * a workgroup of 8 waves owns 16 NT output columns (NT column tiles) over ALL of K and all rows; its waves split K
-//     into eight contiguous ranges, so every weight byte is requested once, by one wave, and no sum leaves the
-//     workgroup: the eight partial tiles meet in LDS (splitting K over workgroups instead, with the slices meeting in
-//     memory behind an arrival counter, cost 4-6 us of store / count / reload round trips at the end of a 12 us stream);
-//   * a wave keeps R k-steps of operand pieces requested ahead in registers, weight tiles and activation rows of the
-//     same k-step side by side in the order they are used (the activation rows come from L2: 16 rows x 64 bytes per
-//     piece); the loop is one software pipeline without barriers;
+//   * a workgroup owns 16 NT output columns (NT column tiles) over ALL of K and all rows.  Two or four of its eight
+//     waves stream the operands, wave w taking k-steps w, w + WS, ..., so every weight byte is requested once, by one
+//     wave, and no sum leaves the workgroup: the partial tiles meet in LDS (splitting K over workgroups instead, with
+//     the slices meeting in memory behind an arrival counter, cost 4-6 us of store / count / reload round trips at the
+//     end of a 12 us stream).  The other waves only share the epilogue: more streaming waves put more requests in
+//     front of the memory system at once and the stream gets slower, fewer epilogue threads make the end of the kernel
+//     a serial walk over the tile;
+//   * a streaming wave keeps R k-steps of operand pieces requested ahead in registers, weight tiles and activation
+//     pieces of the same k-step side by side in the order they are used.  The operands come through buffer resources
+//     that end where K ends (a piece past the end is zeros and no traffic), so the loop has no tail and no branch, and
+//     scheduling barriers keep every refill right behind its use: the compiler then waits for exactly the oldest
+//     k-step (vmcnt = everything younger) -- with conditional loads it waited for all of them every round;
+//   * the activation operand is read in the same tiled order (16 rows x 32 k = 1 KB in lane order, tiled_a_index) when
+//     its producer wrote it so (the decode chain does: prenorm, the out_proj epilogue and the step kernel write
+//     in_proj's and out_proj's operands tiled).  Row-major rows work too, but a load of sixteen 64-byte row pieces
+//     costs the L1 sixty-four tag look-ups where a tile costs eight (in_proj at 64 rows: 24 us tiled, 38 us row-major);
 //   * the epilogues are those of gemm_skinny.hip (plain store, in_proj's conv step + SiLU, out_proj's residual add with
-//     the row's sums of squares), applied to the accumulators where they are: lane l holds rows 4 (l / 16) .. +3 of
-//     column l % 16 of a 16 x 16 tile, one tile per wave.
+//     the row's sums of squares), one result element per thread and pass: element (row ml, column nl) of a 16 x 16 tile
+//     sits in lane 16 (ml / 4) + nl, register ml % 4 of the accumulator.  With one element per thread its epilogue
+//     operands and the row's partial sums of squares are requested before the operand stream and wait in registers.
 #include "common.hpp"
 #include "mfma_tiles.hpp"
 #include <stdlib.h>
@@ -26,18 +36,16 @@
 namespace mrs {
 namespace {
 
-constexpr int kTiledWaves = 8;
-constexpr int kTiledThreads = kTiledWaves * 64;
+constexpr int kTiledThreads = 512;   // eight waves per workgroup: WS of them stream the operands, all of them run the epilogue
 
-template <typename T, int MT, int NT, int R>
+template <typename T, int MT, int NT, int R, int WS = 8>
 __global__ __launch_bounds__(kTiledThreads) void tiled_gemm_kernel(void *__restrict__ Cv, int out_f32, int64_t ldc, const T *__restrict__ A,
                                                                    int64_t lda, const T *__restrict__ Wp, int M, int N, int K, SkinnyEpi ep) {
-    __shared__ v4f red[kTiledWaves / 2][MT * NT][kWave];
+    constexpr int kPark = WS >= 4 ? WS / 2 : WS;   // partial tiles that meet in LDS
+    __shared__ v4f red[kPark][MT * NT][kWave];
     __shared__ float inv_s[16 * MT];
     const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), l = tid & 63, lr = l & 15, lg = l >> 4;
-    const int nks = K >> 5, per = (nks + kTiledWaves - 1) / kTiledWaves;
-    // wave w takes k-steps w, w + 8, w + 16, ...: at any moment the eight waves of the workgroup are reading eight
-    // consecutive kilobytes of each column tile
+    const int nks = K >> 5, per = (nks + WS - 1) / WS;
     const int ntiles = (N + 15) >> 4;
     // Operands through buffer resources that end where K ends: a piece past the end arrives as zeros and costs no memory
     // traffic, so the loop below has no tail and no branch -- every wave runs the same ceil(per / R) rounds and the
@@ -61,19 +69,19 @@ __global__ __launch_bounds__(kTiledThreads) void tiled_gemm_kernel(void *__restr
     const unsigned astep = a_tiled ? (unsigned)MT * 1024u : 64u;
     const unsigned woff = 16u * (unsigned)l;
     auto ldw = [&](int nt, int s_) {
-        return __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(wres[nt], woff, 1024u * (unsigned)(w + kTiledWaves * s_), 0));
+        return __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(wres[nt], woff, 1024u * (unsigned)(w + WS * s_), 0));
     };
     auto lda_ = [&](int mt, int s_) {
-        const int ks = w + kTiledWaves * s_;
+        const int ks = w + WS * s_;
         const unsigned so = ks < nks ? astep * (unsigned)ks : (unsigned)a_records;
         return __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(ares, aoff[mt], so, 0));
     };
-    // Epilogue work is spread over all threads: element e = tid + 512 j of the workgroup's MT NT tiles of 256 -- tile
+    // Epilogue work is spread over all threads: element e = tid + (threads) j of the workgroup's MT NT tiles of 256 -- tile
     // e / 256, row (e % 256) / 16 and column e % 16 of it -- so sixteen consecutive lanes share a row.  With one element
     // per thread its epilogue operands (conv window, taps and bias; or residual and next norm weight) are requested
     // here, ahead of the operand stream, and wait in registers.
     constexpr int kTiles = MT * NT;
-    constexpr int EP = (kTiles + 1) / 2;
+    constexpr int EP = (kTiles * 256 + kTiledThreads - 1) / kTiledThreads;
     constexpr bool kPrefetch = EP == 1;
     const int e_row0 = (tid >> 4) & 15, e_nl = tid & 15;
     float4 pf_win = make_float4(0.f, 0.f, 0.f, 0.f), pf_tap = pf_win;
@@ -96,13 +104,14 @@ __global__ __launch_bounds__(kTiledThreads) void tiled_gemm_kernel(void *__restr
     // lanes share a row; its partial sums (up to 256 of them, a multiple of four) are requested here as 16-byte pieces,
     // all at once and ahead of the operand stream -- summed one load at a time in a loop they were ten L2 round trips in
     // a row before the first matrix instruction (5.5 us of a 21 us in_proj at d_model 2560).
-    constexpr int kScalePasses = MT > 2 ? 2 : 1;       // 32 rows per pass
+    constexpr int kRowsPerPass = kTiledThreads / 16;
+    constexpr int kScalePasses = (16 * MT + kRowsPerPass - 1) / kRowsPerPass;
     const bool ps_fast = ep.row_scale && ep.n_partials % 4 == 0 && ep.n_partials <= 256;
     float4 ps[kScalePasses][4];
     if (ps_fast) {
 #pragma unroll
         for (int h = 0; h < kScalePasses; h++) {
-            const float *pp = ep.partials + (int64_t)min((tid >> 4) + 32 * h, M - 1) * ep.n_partials;
+            const float *pp = ep.partials + (int64_t)min((tid >> 4) + kRowsPerPass * h, M - 1) * ep.n_partials;
 #pragma unroll
             for (int q = 0; q < 4; q++) {
                 const int p4 = 4 * ((tid & 15) + 16 * q);
@@ -110,14 +119,18 @@ __global__ __launch_bounds__(kTiledThreads) void tiled_gemm_kernel(void *__restr
             }
         }
     }
+    // waves 0 .. WS-1 stream the operands (wave w takes k-steps w, w + WS, ...); the others only share the epilogue
+    const bool streams = w < WS;
     uint4 wr[R][NT], ar[R][MT];
+    if (streams) {
 #pragma unroll
-    for (int r = 0; r < R; r++) {
+        for (int r = 0; r < R; r++) {
 #pragma unroll
-        for (int nt = 0; nt < NT; nt++) wr[r][nt] = ldw(nt, r);
+            for (int nt = 0; nt < NT; nt++) wr[r][nt] = ldw(nt, r);
 #pragma unroll
-        for (int mt = 0; mt < MT; mt++) ar[r][mt] = lda_(mt, r);
-        __builtin_amdgcn_sched_barrier(0);   // requested in the order of use, as in the loop (the wait counts of its first round follow this order)
+            for (int mt = 0; mt < MT; mt++) ar[r][mt] = lda_(mt, r);
+            __builtin_amdgcn_sched_barrier(0);   // requested in the order of use, as in the loop (the wait counts of its first round follow this order)
+        }
     }
     // RMSNorm folded around the product (gemm_skinny.hip), second half: the partial sums requested above are in
     if (ep.row_scale) {
@@ -131,7 +144,7 @@ __global__ __launch_bounds__(kTiledThreads) void tiled_gemm_kernel(void *__restr
                 for (int m = 8; m >= 1; m >>= 1) ss += __shfl_xor(ss, m, kWave);
                 float rms = sqrtf(ss / (float)K + ep.eps);
                 if (!isfinite(rms) || rms < 1e-20f) rms = 1.0f;
-                const int r = (tid >> 4) + 32 * h;
+                const int r = (tid >> 4) + kRowsPerPass * h;
                 if ((tid & 15) == 0 && r < 16 * MT) inv_s[r] = 1.0f / rms;
             }
         } else {
@@ -152,7 +165,7 @@ __global__ __launch_bounds__(kTiledThreads) void tiled_gemm_kernel(void *__restr
     for (int mt = 0; mt < MT; mt++)
 #pragma unroll
         for (int nt = 0; nt < NT; nt++) acc[mt][nt] = (v4f){0.f, 0.f, 0.f, 0.f};
-    for (int kb = 0; kb < per; kb += R) {
+    for (int kb = 0; streams && kb < per; kb += R) {
 #pragma unroll
         for (int r = 0; r < R; r++) {
 #pragma unroll
@@ -166,33 +179,42 @@ __global__ __launch_bounds__(kTiledThreads) void tiled_gemm_kernel(void *__restr
             __builtin_amdgcn_sched_barrier(0);   // keep each refill right behind its use: the scheduler would gather the loads at the end of the round
         }
     }
-    // the eight K ranges meet in LDS: the upper four waves park their tiles, the lower four add them and park the sums;
-    // the thread that owns an element then adds its four sums in wave order (one fixed order of additions)
-    if (w >= kTiledWaves / 2) {
+    // the K ranges meet in LDS: of four or eight streaming waves the upper half parks its tiles, the lower half adds them
+    // and parks the sums (one or two streaming waves just park); the thread that owns an element then adds the parked
+    // sums in wave order (one fixed order of additions)
+    if constexpr (WS >= 4) {
+        if (w >= WS / 2 && w < WS) {
+#pragma unroll
+            for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+                for (int nt = 0; nt < NT; nt++) red[w - WS / 2][mt * NT + nt][l] = acc[mt][nt];
+        }
+        lds_barrier();
+        if (w < WS / 2) {
+#pragma unroll
+            for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+                for (int nt = 0; nt < NT; nt++) red[w][mt * NT + nt][l] += acc[mt][nt];
+        }
+    } else if (streams) {
 #pragma unroll
         for (int mt = 0; mt < MT; mt++)
 #pragma unroll
-            for (int nt = 0; nt < NT; nt++) red[w - kTiledWaves / 2][mt * NT + nt][l] = acc[mt][nt];
-    }
-    lds_barrier();
-    if (w < kTiledWaves / 2) {
-#pragma unroll
-        for (int mt = 0; mt < MT; mt++)
-#pragma unroll
-            for (int nt = 0; nt < NT; nt++) red[w][mt * NT + nt][l] += acc[mt][nt];
+            for (int nt = 0; nt < NT; nt++) red[w][mt * NT + nt][l] = acc[mt][nt];
     }
     lds_barrier();
     T *C = reinterpret_cast<T *>(Cv);
     float *Cf = reinterpret_cast<float *>(Cv);
 #pragma unroll
     for (int j = 0; j < EP; j++) {
-        const int tile = (tid >> 8) + 2 * j;            // the same for a whole wave
+        const int e = tid + kTiledThreads * j;
+        const int tile = e >> 8;                        // the same for a whole wave
         if (tile >= kTiles) break;
         // element (ml, nl) of a 16 x 16 tile sits in lane 16 (ml / 4) + nl, register ml % 4 of the accumulator
-        const int ml = e_row0, nl = e_nl, lane = (ml >> 2) * 16 + nl, i = ml & 3;
+        const int ml = (e >> 4) & 15, nl = e & 15, lane = (ml >> 2) * 16 + nl, i = ml & 3;
         float s = red[0][tile][lane][i];
 #pragma unroll
-        for (int q = 1; q < kTiledWaves / 2; q++) s += red[q][tile][lane][i];
+        for (int q = 1; q < kPark; q++) s += red[q][tile][lane][i];
         const int ctile = (int)blockIdx.x * NT + tile % NT;
         const int row = 16 * (tile / NT) + ml, col = 16 * ctile + nl;
         const bool valid = row < M && col < N;
@@ -257,32 +279,29 @@ __global__ __launch_bounds__(256) void tile_weight_kernel(uint4 *__restrict__ Wp
     Wp[p] = col < N ? *reinterpret_cast<const uint4 *>(Wt + (int64_t)col * K + 32 * ks + 8 * (lane >> 4)) : make_uint4(0, 0, 0, 0);
 }
 
-int env_int(const char *name, int dflt) {
-    const char *e = getenv(name);
-    return e ? atoi(e) : dflt;
-}
-
 template <typename T>
 int launch_tiled_t(hipStream_t st, void *C, int out_f32, int64_t ldc, const T *A, int64_t lda, const T *Wp, int M, int N, int K,
                    const SkinnyEpi &ep) {
     const int mt = (M + 15) / 16;
-    // two column tiles per workgroup where the rows are many (a k-step's activation pieces serve both) and the chip stays
-    // full of workgroups (2.8b in_proj at 16 rows: 15.1 us with one tile per workgroup, 17.5 us with two; at 64 rows the same)
-    static const int force_nt = env_int("MRS_TILED_NT", 0);
     const int ntiles = (N + 15) / 16;
-    const int nt = force_nt ? force_nt : ((ntiles >= 512 && mt >= 2) ? 2 : 1);
+    // two column tiles per workgroup where the rows are many (a k-step's activation pieces serve both) and the chip stays
+    // full of workgroups
+    const int nt = (ntiles >= 512 && mt >= 2) ? 2 : 1;
+    // Streaming waves per workgroup (they split K): four at up to 16 rows, two above.  In the 2.8b-shape decode chain, per
+    // step with 1 / 2 / 4 / 8 of them: 16 rows 2.85 / 2.75 / 2.65 / 2.72 ms, 32 rows 3.48 / 3.35 / 3.44 / 3.62, 64 rows
+    // 5.29 / 4.77 / 4.81 / 4.92 -- more waves only put more requests in front of the memory system at once (alone, with
+    // a plain store, in_proj at 16 rows takes 13.7 us with one streaming wave and 18.3 us with eight).
     const dim3 grid((unsigned)((ntiles + nt - 1) / nt)), block(kTiledThreads);
-#define MRS_TG(MT_, NT_, R_) \
-    hipLaunchKernelGGL((tiled_gemm_kernel<T, MT_, NT_, R_>), grid, block, 0, st, C, out_f32, ldc, A, lda, Wp, M, N, K, ep)
+#define MRS_TG(MT_, NT_, R_, W_) \
+    hipLaunchKernelGGL((tiled_gemm_kernel<T, MT_, NT_, R_, W_>), grid, block, 0, st, C, out_f32, ldc, A, lda, Wp, M, N, K, ep)
     switch (mt * 10 + nt) {
-        case 11: MRS_TG(1, 1, 10); break;
-        case 12: MRS_TG(1, 2, 8); break;
-        case 21: MRS_TG(2, 1, 8); break;
-        case 22: MRS_TG(2, 2, 6); break;
-        case 31: MRS_TG(3, 1, 6); break;
-        case 32: MRS_TG(3, 2, 5); break;
-        case 41: MRS_TG(4, 1, 5); break;
-        default: MRS_TG(4, 2, 4); break;
+        case 11: MRS_TG(1, 1, 10, 4); break;
+        case 21: MRS_TG(2, 1, 8, 2); break;
+        case 22: MRS_TG(2, 2, 6, 2); break;
+        case 31: MRS_TG(3, 1, 6, 2); break;
+        case 32: MRS_TG(3, 2, 5, 2); break;
+        case 41: MRS_TG(4, 1, 5, 2); break;
+        default: MRS_TG(4, 2, 4, 2); break;
     }
 #undef MRS_TG
     return check_launch("tiled_gemm_kernel");
