@@ -275,12 +275,13 @@ typedef struct {            /* MambaWeights, src/weights.rs:51-64 */
 MRS_API int mrs_gemm_skinny(void *stream, int dtype, void *C, int out_f32, int64_t ldc, const void *A, int64_t lda,
                             const void *Wt, int M, int N, int K);
 MRS_API int mrs_transpose(void *stream, int dtype, void *Wt, const void *W, int K, int N);
-/* The same product for 5 <= M <= 64 rows over a weight of megabytes (wide models: in_proj of the 2.8b shape is 52 MB), from
- * a TILED weight: the 16 columns x 32 k of one matrix-core operand are 1 KB of consecutive memory, so the product is one
+/* The same product from a TILED weight (what the decode chain reads from 5 rows up; wide models: in_proj of the 2.8b shape
+ * is 52 MB): the 16 columns x 32 k of one matrix-core operand are 1 KB of consecutive memory, so the product is one
  * contiguous stream per wave (call sites src/mamba_ssm/gpu/blas.rs:1138-1163).
  *   mrs_tiled_weight_bytes: bytes of the tiled copy (columns padded to a multiple of 16); 0 for an unsupported dtype / K
  *   mrs_tile_weight:        Wp = tiled copy of the transposed weight Wt[N,K] (f16/bf16, K % 32 == 0, 16-byte aligned)
- *   mrs_gemm_tiled:         C[M,N] = A[M,K] . W; 1 <= M <= 64, K % 32 == 0, lda % 8 == 0, A and Wp 16-byte aligned */
+ *   mrs_gemm_tiled:         C[M,N] = A[M,K] . W; K % 32 == 0, lda % 8 == 0, A and Wp 16-byte aligned; 1 <= M <= 64 for a
+ *                           weight of 16 MB or more (column-tile kernel), 1 <= M <= 128 below that (16 x 16 tiles) */
 MRS_API size_t mrs_tiled_weight_bytes(int dtype, int N, int K);
 MRS_API int mrs_tile_weight(void *stream, int dtype, void *Wp, const void *Wt, int N, int K);
 MRS_API int mrs_gemm_tiled(void *stream, int dtype, void *C, int out_f32, int64_t ldc, const void *A, int64_t lda,

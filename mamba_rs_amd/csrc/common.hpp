@@ -124,10 +124,15 @@ struct SkinnyEpi {
     // x_proj of a wide model is 12 tiles over K = 5120)
     int ksplit;
     int kslice;          // set by the launcher: 32-wide k-steps per slice
-    // tiled route (gemm_wide.hip) only: A is stored [k-step][row tile][lane][8] -- the matrix-core operand in lane order, 16-row
+    // tiled route (gemm_wide.hip) and matrix-core route of gemm_skinny.hip: A is stored [k-step][row tile][lane][8] -- the matrix-core operand in lane order, 16-row
     // tiles (tiled_a_index), rows past M present with any contents -- instead of row-major
     int a_tiled;
     int prenorm_mt;      // mode 2: != 0 writes prenorm in that tiled order (prenorm_mt row tiles) for the next tiled in_proj
+    // matrix-core route of gemm_skinny.hip: the weight is the tiled copy (launch_tile_weight) instead of Wt[N][K]
+    int w_tiled;
+    // mode 1, optional: a second copy of u in tiled order (u_tiled_mt row tiles), the operand of a tiled x_proj
+    void *u_tiled;
+    int u_tiled_mt;
 };
 // The same products from a TILED weight (gemm_wide.hip): 5..64 rows over a weight of megabytes.  Wp holds the 16 columns x 32 k
 // of each matrix-core operand as 1 KB in lane order, column tile by column tile (launch_tile_weight builds it from the

@@ -213,7 +213,7 @@ struct LayerDev {
     void *dt_w_t;  // [d_inner][dt_rank] copy: the fused decode step (when dt_t_step) and the prefill dt_proj+softplus kernel read it
     int dt_t_step;
     void *in_proj_t, *x_proj_t, *out_proj_t;  // [N][K] copies: in / out for every 16-bit engine (own GEMM and vendor GEMM read them), x for the own chain only
-    void *in_proj_p, *out_proj_p;  // tiled copies (gemm_wide.hip): wide models at 5..64 rows
+    void *in_proj_p, *out_proj_p, *x_proj_p;  // tiled copies (launch_tile_weight): the own chain from 5 rows up
     int s4d;
 };
 
@@ -252,6 +252,7 @@ struct Scratch {  // activations for M rows
     void *normed = nullptr, *proj = nullptr, *u = nullptr, *xdbl = nullptr, *delta = nullptr, *y = nullptr, *out = nullptr;
     float *residual = nullptr;
     float *partials = nullptr;  // [rows][d_model/16] row sums of squares, decode chain only
+    void *u_tiled = nullptr;    // decode chain on tiled operands: u once more, in tile order (x_proj's operand)
     float *xpart = nullptr;     // decode chain: shares of the x_proj rows (per in_proj tile, or per K slice of x_proj)
     int64_t xpart_floats = 0;
     void *scan_ws = nullptr;
@@ -263,7 +264,8 @@ struct mrs_backbone {
     mrs_m1_config cfg;
     int input_dim, batch, dtype, di, dr, xd, identity_proj, device;
     const float *step_src;  // decode step: where layer 0 reads its input rows (null: the residual buffer itself)
-    int tiled;   // own chain with in_proj / out_proj from tiled weights and tiled activation operands (wide models, 5..64 rows)
+    int tiled;   // own chain from 5 rows up: the projections read tiled weights and tiled activation operands
+    int wide;    // ... and in_proj / out_proj run on the column-tile kernel of gemm_wide.hip (wide models, up to 64 rows)
     int skinny;  // decode projections on the library's own GEMM (16-bit storage: batch <= 128 or 64, K % 32 == 0; f32: batch <= 4, K % 128 == 0)
     hipStream_t stream;
     rocblas_handle blas;
@@ -317,6 +319,7 @@ static int alloc_scratch(mrs_backbone *bb, Scratch *s, int64_t rows, int T) {
     MRS_TRY(dev_alloc(bb, &s->normed, rows16 * dm * es));
     MRS_TRY(dev_alloc(bb, &s->proj, rows * 2 * di * es));
     MRS_TRY(dev_alloc(bb, &s->u, rows * di * es));
+    if (T == 1 && bb->tiled) MRS_TRY(dev_alloc(bb, &s->u_tiled, rows16 * di * es));
     MRS_TRY(dev_alloc(bb, &s->xdbl, rows * xd * es));
     MRS_TRY(dev_alloc(bb, &s->delta, rows * di * es));
     MRS_TRY(dev_alloc(bb, &s->y, rows16 * di * es));
@@ -408,7 +411,7 @@ static int decode_chain(mrs_backbone *bb, Scratch *s, int r0, int nr, hipStream_
     // that cannot split K (nobody would sum the shares): 12.5 us at 32 and 64 rows of the 2.8b shape, against 4.7 us split.
     // Per step at that shape, dt_proj in the step kernel / on its own: 32 rows 3.57 / 3.84 ms, 48 rows 4.32 / 4.34, 64 rows 5.04 / 4.89.
     static const int64_t wide_fuse = [] { const char *e = getenv("MRS_DECODE_FUSE_DT_LIMIT"); return e ? (int64_t)atoll(e) : (int64_t)6400; }();
-    const int64_t fuse_limit = a_mt ? wide_fuse : kFuseDtProjLimit;
+    const int64_t fuse_limit = (a_mt && bb->wide) ? wide_fuse : kFuseDtProjLimit;
     for (int l = 0; l < L; l++) {
         const LayerDev &lw = bb->layers[l];
         float *conv = bb->conv_state + ((size_t)l * B + r0) * di * dc;
@@ -428,8 +431,10 @@ static int decode_chain(mrs_backbone *bb, Scratch *s, int r0, int nr, hipStream_
         const int ksplit = (!fold_x && step_sums && dt != MRS_F32) ? xproj_slices(nr, xd, di) : 1;
         const StepFold fold = {xpart, fold_x ? di / 16 : ksplit, nr, xd, dr, dr + ds};
         if (a_mt) {
-            inp.a_tiled = 1;
-            MRS_TRY(launch_tiled_gemm(st, dt, proj, 0, 2 * di, normed, dm, lw.in_proj_p, nr, 2 * di, dm, inp));
+            inp.a_tiled = 1; inp.w_tiled = 1;
+            if (!fold_x) { inp.u_tiled = s->u_tiled; inp.u_tiled_mt = a_mt; }
+            if (bb->wide) MRS_TRY(launch_tiled_gemm(st, dt, proj, 0, 2 * di, normed, dm, lw.in_proj_p, nr, 2 * di, dm, inp));
+            else MRS_TRY(launch_skinny_gemm(st, dt, proj, 0, 2 * di, normed, dm, lw.in_proj_p, nr, 2 * di, dm, inp));
         } else {
             MRS_TRY(launch_skinny_gemm(st, dt, proj, 0, 2 * di, normed, dm, lw.in_proj_t, nr, 2 * di, dm, inp));
         }
@@ -437,7 +442,12 @@ static int decode_chain(mrs_backbone *bb, Scratch *s, int r0, int nr, hipStream_
         if (!fold_x) {
             SkinnyEpi xp = {};
             if (ksplit > 1) { xp.ksplit = ksplit; xp.xpart = xpart; }
-            MRS_TRY(launch_skinny_gemm(st, dt, xdbl, 0, xd, u, di, lw.x_proj_t, nr, xd, di, xp));
+            if (a_mt) {
+                xp.a_tiled = 1; xp.w_tiled = 1;
+                MRS_TRY(launch_skinny_gemm(st, dt, xdbl, 0, xd, s->u_tiled, di, lw.x_proj_p, nr, xd, di, xp));
+            } else {
+                MRS_TRY(launch_skinny_gemm(st, dt, xdbl, 0, xd, u, di, lw.x_proj_t, nr, xd, di, xp));
+            }
         }
         if ((int64_t)nr * dr > fuse_limit && lw.dt_w_t && skinny_gemm_ok(dt, nr, di, dr, xd, xdbl, lw.dt_w_t)) {
             // wide dt_rank at a large batch: dt_proj as a GEMM of its own, bias + softplus in the step kernel
@@ -453,8 +463,9 @@ static int decode_chain(mrs_backbone *bb, Scratch *s, int r0, int nr, hipStream_
         outp.mode = 2; outp.residual = residual; outp.partials = partials; outp.n_partials = P;
         outp.next_norm_w = l + 1 < L ? bb->layers[l + 1].norm_w : nullptr; outp.prenorm = normed;
         if (a_mt) {
-            outp.a_tiled = 1; outp.prenorm_mt = a_mt;
-            MRS_TRY(launch_tiled_gemm(st, dt, out, 0, dm, y, di, lw.out_proj_p, nr, dm, di, outp));
+            outp.a_tiled = 1; outp.w_tiled = 1; outp.prenorm_mt = a_mt;
+            if (bb->wide) MRS_TRY(launch_tiled_gemm(st, dt, out, 0, dm, y, di, lw.out_proj_p, nr, dm, di, outp));
+            else MRS_TRY(launch_skinny_gemm(st, dt, out, 0, dm, y, di, lw.out_proj_p, nr, dm, di, outp));
         } else {
             MRS_TRY(launch_skinny_gemm(st, dt, out, 0, dm, y, di, lw.out_proj_t, nr, dm, di, outp));
         }
@@ -588,16 +599,18 @@ extern "C" int mrs_backbone_create(mrs_backbone **out, int gpu_ordinal, const mr
         // vendor kernels), measured: 128 at the 130m shape (1032 vs 1091 us per step; at 256 rows 1490 vs 1392), 40 at the
         // 2.8b shape (32 rows 5.13 vs 8.35 ms, 40 rows 5.74 vs 5.92, 48 rows 6.13 vs 5.98, 64 rows 7.58 vs 6.19).  "Narrow"
         // as for the x_proj shares.
-        // Wide models from 5 rows up: in_proj / out_proj stream tiled weights (gemm_wide.hip), which carries the own chain
-        // up to 64 rows.
+        // From 5 rows up (the matrix-core route) the projections of the own chain read TILED operands -- weights tiled at load,
+        // activation operands written tiled by their producers.  On wide models in_proj / out_proj also run on the
+        // column-tile kernel of gemm_wide.hip, which carries the own chain up to 64 rows there.
         static const bool no_tiled = [] { const char *e = getenv("MRS_DECODE_NO_TILED"); return e && atoi(e) != 0; }();
         static const int tiled_max_rows = [] { const char *e = getenv("MRS_DECODE_TILED_MAX_ROWS"); return e ? atoi(e) : 64; }();
         const bool pow2_state = ds == 4 || ds == 8 || ds == 16 || ds == 32 || ds == 64 || ds == 128 || ds == 256;
-        bb->tiled = !off && !no_tiled && (dtype == MRS_BF16 || dtype == MRS_F16) && batch >= 5 && batch <= std::min(tiled_max_rows, 64) &&
-                    dm % 32 == 0 && di % 32 == 0 && (int64_t)dm * 2 * di >= (int64_t)8 << 20 && pow2_state && !narrow_model(di, xd);
-        const int max_rows = std::min(skinny_max_rows(), narrow_model(di, xd) ? 128 : (bb->tiled ? 64 : 40));
+        const bool can_tile = !off && !no_tiled && (dtype == MRS_BF16 || dtype == MRS_F16) && batch >= 5 && dm % 32 == 0 && di % 32 == 0 && pow2_state;
+        bb->wide = can_tile && batch <= std::min(tiled_max_rows, 64) && (int64_t)dm * 2 * di >= (int64_t)8 << 20 && !narrow_model(di, xd);
+        const int max_rows = std::min(skinny_max_rows(), narrow_model(di, xd) ? 128 : (bb->wide ? 64 : 40));
         bb->skinny = !off && (dtype == MRS_BF16 || dtype == MRS_F16) && batch <= max_rows && dm % 32 == 0 && di % 32 == 0;
-        if (!bb->skinny) bb->tiled = 0;
+        bb->tiled = can_tile && bb->skinny;
+        if (!bb->skinny) bb->wide = 0;
         // f32 storage: the same chain on the row-wise route of the GEMM (one to four rows, rows of the operand in LDS)
         if (!off && dtype == MRS_F32 && batch <= 4 && dm % 128 == 0 && di % 128 == 0 && (int64_t)di * 16 <= 48 * 1024 &&
             getenv("MRS_DECODE_NO_ROWWISE") == nullptr)
@@ -622,7 +635,7 @@ extern "C" int mrs_backbone_create(mrs_backbone **out, int gpu_ordinal, const mr
         MRS_CREATE_TRY(upload_f32(bb, &d.dt_b, src.dt_proj_b, di));
         MRS_CREATE_TRY(upload_f32(bb, &d.D, src.d_param, di));
         MRS_CREATE_TRY(upload_bulk(bb, &d.out_proj, src.out_proj_w, (size_t)di * dm, stage));
-        d.in_proj_t = d.x_proj_t = d.out_proj_t = d.dt_w_t = d.in_proj_p = d.out_proj_p = nullptr;
+        d.in_proj_t = d.x_proj_t = d.out_proj_t = d.dt_w_t = d.in_proj_p = d.out_proj_p = d.x_proj_p = nullptr;
         d.dt_t_step = (ds == 4 || ds == 8 || ds == 16 || ds == 32 || ds == 64 || ds == 128 || ds == 256) && dr % ds == 0 && xd % 4 == 0;
         if (d.dt_t_step || (bb->dtype != MRS_F32 && dr % 8 == 0)) {
             MRS_CREATE_TRY(dev_alloc(bb, &d.dt_w_t, (size_t)dr * di * esize(bb->dtype)));
@@ -647,6 +660,10 @@ extern "C" int mrs_backbone_create(mrs_backbone **out, int gpu_ordinal, const mr
         if (bb->skinny) {
             MRS_CREATE_TRY(dev_alloc(bb, &d.x_proj_t, (size_t)di * xd * esize(bb->dtype)));
             MRS_CREATE_TRY(launch_transpose(bb->stream, bb->dtype, d.x_proj_t, d.x_proj, di, xd));
+            if (bb->tiled) {
+                MRS_CREATE_TRY(dev_alloc(bb, &d.x_proj_p, tiled_weight_elems(xd, di) * esize(bb->dtype)));
+                MRS_CREATE_TRY(launch_tile_weight(bb->stream, bb->dtype, d.x_proj_p, d.x_proj_t, xd, di));
+            }
         }
         // a_neg = -exp(a_log) once at load (exp_negate, src/mamba_ssm/gpu/inference.rs:266-282)
         MRS_CREATE_TRY(dev_alloc(bb, (void **)&d.a_neg, (size_t)di * ds * 4));

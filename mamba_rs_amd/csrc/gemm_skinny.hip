@@ -92,8 +92,14 @@ __global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu
     // Rows past M / columns past N are clamped to the last valid one: their products land in
     // accumulator elements that are never stored.
     constexpr int EPV = 16 / (int)sizeof(T);   // elements per 16-byte piece
-    const T *wrow = Wt + (int64_t)min(n0 + lr, N - 1) * K + 8 * lg;
-    const T *arow = A + (int64_t)min(m0 + lr, M - 1) * lda + 8 * lg;
+    // Matrix-core route: either operand may be stored tiled -- the 16 x 32 piece of one matrix instruction as 1 KB in lane
+    // order (gemm_wide.hip: launch_tile_weight, tiled_a_index) -- so that a fragment load is one contiguous kilobyte
+    // instead of sixteen 64-byte row pieces: eight cache lines for the L1 to look up instead of sixty-four, which is what
+    // these short products are bound by (64 x 3072 x 768: 6.6 us row-major, 4.4 us tiled).
+    const bool w_tiled = LPR == 0 && ep.w_tiled, a_tiled = LPR == 0 && ep.a_tiled;
+    const T *wrow = w_tiled ? Wt + (int64_t)(n0 >> 4) * (K >> 5) * 512 + 8 * l : Wt + (int64_t)min(n0 + lr, N - 1) * K + 8 * lg;
+    const T *arow = a_tiled ? A + (int64_t)(m0 >> 4) * 512 + 8 * l : A + (int64_t)min(m0 + lr, M - 1) * lda + 8 * lg;
+    const int wks = w_tiled ? 512 : 32, aks = a_tiled ? 512 * ((M + 15) >> 4) : 32;   // elements from one k-step's piece to the next
     float inv = 1.0f;
     // The partial sums of a row are requested together, before the operands stream, and added up after the product
     // (in the order a loop over them would add them): loaded one at a time inside such a loop they were a chain of
@@ -267,8 +273,8 @@ __global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu
         for (int s = 0; s < kHalf; s++) {
             const int ks = base + s * kGemmWaves;
             // steps past K multiply zeros (every fragment is defined on every path)
-            bf[h][s] = ks < nk ? *reinterpret_cast<const uint4 *>(wrow + 32 * ks) : make_uint4(0, 0, 0, 0);
-            af[h][s] = ks < nk ? *reinterpret_cast<const uint4 *>(arow + 32 * ks) : make_uint4(0, 0, 0, 0);
+            bf[h][s] = ks < nk ? *reinterpret_cast<const uint4 *>(wrow + wks * ks) : make_uint4(0, 0, 0, 0);
+            af[h][s] = ks < nk ? *reinterpret_cast<const uint4 *>(arow + aks * ks) : make_uint4(0, 0, 0, 0);
         }
     };
     constexpr int kStride = kGemmWaves * kHalf;   // k-steps one half-batch covers across the workgroup's waves
@@ -315,7 +321,8 @@ __global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu
                 const float rn = res_old + Store<T>::ld(&orr);
                 ep.residual[(int64_t)row * N + col] = rn;
                 sq = rn * rn;
-                if (ep.next_norm_w) Store<T>::st(reinterpret_cast<T *>(ep.prenorm) + (int64_t)row * N + col, rn * nw);
+                if (ep.next_norm_w)
+                    Store<T>::st(reinterpret_cast<T *>(ep.prenorm) + (ep.prenorm_mt ? tiled_a_index(row, col, ep.prenorm_mt) : (int64_t)row * N + col), rn * nw);
             }
 #pragma unroll
             for (int m = 8; m >= 1; m >>= 1) sq += __shfl_xor(sq, m, kWave);
@@ -341,6 +348,7 @@ __global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu
             }
             const T ur = (T)silu(o);
             reinterpret_cast<T *>(ep.u)[(int64_t)row * ep.di + col] = ur;
+            if (ep.u_tiled) reinterpret_cast<T *>(ep.u_tiled)[tiled_a_index(row, col, ep.u_tiled_mt)] = ur;   // x_proj's operand
             u_out = Store<T>::ld(&ur);
         } else if (EPI == 0 && LPR == 0 && gridDim.z > 1) {
             ep.xpart[((int64_t)blockIdx.z * M + row) * N + col] = s;   // this slice's share, summed by the reader
@@ -518,6 +526,7 @@ static int launch_skinny_t(hipStream_t st, TO *C, int64_t ldc, const T *A, int64
                                                                                : (K % (64 * EPV) == 0 ? 64 : (K % (32 * EPV) == 0 ? 32 : 0));
     const int ksplit = (ep.mode == 0 && ep.ksplit > 1) ? ep.ksplit : 1;
     if (ksplit > 1) lpr = 0;   // a split K runs on the matrix-core route at any row count
+    if (ep.w_tiled || ep.a_tiled) lpr = 0;   // tiled operands are matrix-core operands
     if (sizeof(T) == 4 && lpr == 0) return fail(MRS_E_SHAPE, "skinny gemm: f32 storage runs on the row-wise route only (M <= 4, K %% 128 == 0, no K split)");
     if (ksplit > 1 && (ep.row_scale || !ep.xpart || ksplit > (K >> 5)))
         return fail(MRS_E_SHAPE, "skinny gemm: K split needs the matrix-core route, a plain product, a share buffer and ksplit <= K / 32 (ksplit=%d)", ksplit);

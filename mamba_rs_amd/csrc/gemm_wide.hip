@@ -258,7 +258,9 @@ __global__ __launch_bounds__(kTiledThreads) void tiled_gemm_kernel(void *__restr
                     st[k] = wk;
                 }
             }
-            Store<T>::st(reinterpret_cast<T *>(ep.u) + (int64_t)row * ep.di + col, silu(o));
+            const T ur = (T)silu(o);
+            reinterpret_cast<T *>(ep.u)[(int64_t)row * ep.di + col] = ur;
+            if (ep.u_tiled) reinterpret_cast<T *>(ep.u_tiled)[tiled_a_index(row, col, ep.u_tiled_mt)] = ur;   // x_proj's operand
         } else if (out_f32) {
             Cf[(int64_t)row * ldc + col] = s;
         } else {
@@ -355,5 +357,10 @@ extern "C" int mrs_gemm_tiled(void *stream, int dtype, void *C, int out_f32, int
     if (ldc < N) return fail(MRS_E_SHAPE, "mrs_gemm_tiled: ldc=%lld < N=%d", (long long)ldc, N);
     if (lda < K) return fail(MRS_E_SHAPE, "mrs_gemm_tiled: lda=%lld < K=%d", (long long)lda, K);
     SkinnyEpi ep = {};
-    return launch_tiled_gemm(as_stream(stream), dtype, C, out_f32, ldc, A, lda, Wp, M, N, K, ep);
+    // a weight of 16 MB or more on the column-tile kernel (up to 64 rows), a smaller one on the 16 x 16 tiles of
+    // gemm_skinny.hip reading the same tiled weight (up to 128 rows): the split the decode chain makes
+    if ((int64_t)N * K * 2 >= ((int64_t)16 << 20) && M <= 64) return launch_tiled_gemm(as_stream(stream), dtype, C, out_f32, ldc, A, lda, Wp, M, N, K, ep);
+    if (dtype != MRS_BF16 && dtype != MRS_F16) return fail(MRS_E_DTYPE, "mrs_gemm_tiled: 16-bit storage only");
+    ep.w_tiled = 1;
+    return launch_skinny_gemm(as_stream(stream), dtype, C, out_f32, ldc, A, lda, Wp, M, N, K, ep);
 }

@@ -37,8 +37,10 @@ def test_gemm_skinny_matches_f64_matmul(shape, dtype, out_f32):
 
 # (M, N, K): the 2.8b decode projections at one to four 16-row tiles (whole and partly filled), N not a multiple of 16, a K
 # shorter than the eight waves' ranges, a K that does not divide by them
+# (small weights go to the 16 x 16 tiles reading the same tiled weight: the 130m decode projections, up to 128 rows)
 TILED_SHAPES = [(16, 10240, 2560), (64, 10240, 2560), (5, 2560, 5120), (23, 2560, 5120), (40, 2560, 5120), (64, 2560, 5120),
-                (16, 200, 96), (33, 16, 32), (48, 1000, 1056), (1, 50, 256), (64, 8200, 64)]
+                (16, 200, 96), (33, 16, 32), (48, 1000, 1056), (1, 50, 256), (64, 8200, 64),
+                (64, 3072, 768), (128, 768, 1536), (97, 80, 1536), (3, 3072, 768)]
 
 
 @pytest.mark.parametrize("dtype", [orc.BF16, orc.F16])
@@ -74,8 +76,8 @@ def test_gemm_tiled_matches_f64_matmul(shape, dtype):
 def test_gemm_tiled_rejects_bad_arguments():
     wt = torch.zeros(32, 64, device=DEV, dtype=torch.bfloat16)
     wp, n = ops.tile_weight(wt)
-    with pytest.raises(RuntimeError, match="tiled gemm"):
-        ops.gemm_tiled(torch.zeros(65, 64, device=DEV, dtype=torch.bfloat16), wp, n)      # more than 64 rows
+    with pytest.raises(RuntimeError, match="skinny gemm"):
+        ops.gemm_tiled(torch.zeros(129, 64, device=DEV, dtype=torch.bfloat16), wp, n)      # more than 128 rows
     with pytest.raises(ValueError):
         ops.tile_weight(torch.zeros(32, 48, device=DEV, dtype=torch.bfloat16))              # K % 32 != 0
 
