@@ -33,7 +33,7 @@ __global__ __launch_bounds__(1024) void m3_layer_step_kernel(
     T *__restrict__ gated, const float *__restrict__ proj, int64_t ip, const float *__restrict__ dt_bias,
     const float *__restrict__ bnw, const float *__restrict__ cnw, const float *__restrict__ b_bias,
     const float *__restrict__ c_bias, const float *__restrict__ Dp, const float *__restrict__ ngw, int nh, int hd, int ng,
-    int nr, float a_floor, float eps, int outproj_norm) {
+    int nr, float a_floor, float eps, int outproj_norm, int gated_mt) {
     constexpr int ds = 4 * LG;
     __shared__ float kl[ds], ql[ds], red[16];
     const int b = blockIdx.x / nh, h = blockIdx.x - b * nh;
@@ -130,7 +130,8 @@ __global__ __launch_bounds__(1024) void m3_layer_step_kernel(
     }
     if (g == 0) {
         const float o = outproj_norm ? yv * inv_y * ngv * silu(zi) : yv * silu(zi);
-        Store<T>::st(gated + (int64_t)b * di + h * hd + p, o);
+        // gated_mt != 0: out_proj reads its operand in tile order (tiled_a_index, gated_mt row tiles)
+        Store<T>::st(gated + (gated_mt ? tiled_a_index(b, h * hd + p, gated_mt) : (int64_t)b * di + h * hd + p), o);
         vst[bh * hd + p] = xv;
     }
     // every lane has read the previous k_state (kp) at the top; the full barrier after the rotation orders those reads before this write
@@ -549,13 +550,14 @@ struct Layer3 {
     float *norm_w, *dt_bias, *bnw, *cnw, *b_bias, *c_bias, *D, *ngw;
     void *in_proj, *out_proj;      // [K][N] storage type (library GEMM)
     void *in_proj_t, *out_proj_t;  // [N][K] copies for the skinny GEMM (null: library chain)
+    void *in_proj_p, *out_proj_p;  // tiled copies (launch_tile_weight): the own chain from 5 rows up
 };
 
 }  // namespace
 
 struct mrs_m3_backbone {
     mrs_m3_config cfg;
-    int input_dim, batch, dtype, di, nh, ip, nr, identity_proj, device, skinny;
+    int input_dim, batch, dtype, di, nh, ip, nr, identity_proj, device, skinny, tiled;
     hipStream_t stream;
     rocblas_handle blas;
     GemmTuner *tuner;       // vendor-kernel choice for the prefill projections (off unless asked for)
@@ -622,7 +624,7 @@ int launch_layer_step_t(mrs_m3_backbone *bb, int l) {
     case L:                                                                                                                       \
         hipLaunchKernelGGL((m3_layer_step_kernel<T, L>), grid, block, 0, bb->stream, ssm, kst, vst, ang, (T *)bb->gated, bb->proj,  \
                            (int64_t)bb->ip, lw.dt_bias, lw.bnw, lw.cnw, lw.b_bias, lw.c_bias, lw.D, lw.ngw, nh, hd, c.ngroups,     \
-                           bb->nr, c.a_floor, c.rms_norm_eps, c.is_outproj_norm);                                                   \
+                           bb->nr, c.a_floor, c.rms_norm_eps, c.is_outproj_norm, bb->tiled ? (B + 15) / 16 : 0);                   \
         break
     switch (lg) { MRS_LG(1); MRS_LG(2); MRS_LG(4); MRS_LG(8); MRS_LG(16); MRS_LG(32); MRS_LG(64); default: return fail(MRS_E_SHAPE, "m3 layer step: d_state %d", ds); }
 #undef MRS_LG
@@ -643,6 +645,7 @@ int step_body3(mrs_m3_backbone *bb) {
     }
     const int dm = c.d_model, di = bb->di, B = bb->batch, dt = bb->dtype, L = c.n_layers, ip = bb->ip;
     const int P = (dm + 15) / 16;
+    const int a_mt = bb->tiled ? (B + 15) / 16 : 0;   // the projections' operands in tile order (16-row tiles)
     // residual <- input (identity) or input . W + b
     const float *src = nullptr;
     if (bb->identity_proj) {
@@ -662,10 +665,11 @@ int step_body3(mrs_m3_backbone *bb) {
         if (bb->skinny) {
             if (l == 0)
                 MRS_TRY(launch_prenorm_rows(bb->stream, dt, bb->partials, P, bb->normed, src ? src : bb->residual, src ? bb->residual : nullptr,
-                                            lw.norm_w, B, dm));
+                                            lw.norm_w, B, dm, a_mt));
             SkinnyEpi inp = {};
             inp.row_scale = 1; inp.partials = bb->partials; inp.n_partials = P; inp.eps = c.rms_norm_eps;
-            MRS_TRY(launch_skinny_gemm(bb->stream, dt, bb->proj, 1, ip, bb->normed, dm, lw.in_proj_t, B, ip, dm, inp));
+            inp.a_tiled = inp.w_tiled = a_mt ? 1 : 0;
+            MRS_TRY(launch_skinny_gemm(bb->stream, dt, bb->proj, 1, ip, bb->normed, dm, a_mt ? lw.in_proj_p : lw.in_proj_t, B, ip, dm, inp));
         } else {
             MRS_TRY(launch_add_rmsnorm_any(bb->stream, dt, bb->residual, l == 0 ? nullptr : bb->out, bb->normed, false, nullptr, lw.norm_w,
                                            c.rms_norm_eps, B, dm, dm));
@@ -676,7 +680,8 @@ int step_body3(mrs_m3_backbone *bb) {
             SkinnyEpi outp = {};
             outp.mode = 2; outp.residual = bb->residual; outp.partials = bb->partials; outp.n_partials = P;
             outp.next_norm_w = l + 1 < L ? bb->layers[l + 1].norm_w : nullptr; outp.prenorm = bb->normed;
-            MRS_TRY(launch_skinny_gemm(bb->stream, dt, bb->out, 0, dm, bb->gated, di, lw.out_proj_t, B, dm, di, outp));
+            outp.a_tiled = outp.w_tiled = a_mt ? 1 : 0; outp.prenorm_mt = a_mt;
+            MRS_TRY(launch_skinny_gemm(bb->stream, dt, bb->out, 0, dm, bb->gated, di, a_mt ? lw.out_proj_p : lw.out_proj_t, B, dm, di, outp));
         } else {
             MRS_TRY(gemm3(bb, bb->out, false, bb->gated, lw.out_proj, B, dm, di));
         }
@@ -756,6 +761,8 @@ extern "C" int mrs_m3_backbone_create(mrs_m3_backbone **out, int gpu_ordinal, co
     const int dm = cfg->d_model, di = bb->di, ip = bb->ip, L = cfg->n_layers;
     // (above 64 rows the library chain is the faster one for this layer: 1261 vs 1318 us per step at 128 rows, 768-wide shape)
     bb->skinny = (dtype == MRS_BF16 || dtype == MRS_F16) && batch <= std::min(64, skinny_max_rows()) && dm % 32 == 0 && di % 32 == 0;
+    // from 5 rows up (the matrix-core route) the two projections read tiled weights and tiled activation operands
+    { const char *e = getenv("MRS_DECODE_NO_TILED"); bb->tiled = bb->skinny && batch >= 5 && !(e && atoi(e) != 0); }
     // f32 storage: the row-wise route of the same GEMM, one to four rows
     if (dtype == MRS_F32 && batch <= 4 && dm % 128 == 0 && di % 128 == 0 && (int64_t)di * 16 <= 48 * 1024 && getenv("MRS_DECODE_NO_ROWWISE") == nullptr)
         bb->skinny = 1;
@@ -796,6 +803,14 @@ extern "C" int mrs_m3_backbone_create(mrs_m3_backbone **out, int gpu_ordinal, co
             MRS_CREATE_TRY(launch_transpose(bb->stream, dtype, d.in_proj_t, d.in_proj, dm, ip));
             MRS_CREATE_TRY(launch_transpose(bb->stream, dtype, d.out_proj_t, d.out_proj, di, dm));
         }
+        d.in_proj_p = d.out_proj_p = nullptr;
+        if (bb->tiled) {
+            const size_t es = esize3(dtype);
+            MRS_CREATE_TRY(dev_alloc3(bb, &d.in_proj_p, tiled_weight_elems(ip, dm) * es));
+            MRS_CREATE_TRY(dev_alloc3(bb, &d.out_proj_p, tiled_weight_elems(dm, di) * es));
+            MRS_CREATE_TRY(launch_tile_weight(bb->stream, dtype, d.in_proj_p, d.in_proj_t, ip, dm));
+            MRS_CREATE_TRY(launch_tile_weight(bb->stream, dtype, d.out_proj_p, d.out_proj_t, dm, di));
+        }
     }
     MRS_CREATE_TRY(upload_f32_3(bb, &bb->norm_f, w->norm_f_weight, dm));
     {
@@ -823,8 +838,9 @@ extern "C" int mrs_m3_backbone_create(mrs_m3_backbone **out, int gpu_ordinal, co
     MRS_CREATE_TRY(dev_alloc3(bb, (void **)&bb->residual, B * dm * 4));
     MRS_CREATE_TRY(dev_alloc3(bb, (void **)&bb->proj, B * ip * 4));
     MRS_CREATE_TRY(dev_alloc3(bb, (void **)&bb->partials, B * ((dm + 15) / 16) * 4));
-    MRS_CREATE_TRY(dev_alloc3(bb, &bb->normed, B * dm * es));
-    MRS_CREATE_TRY(dev_alloc3(bb, &bb->gated, B * di * es));
+    const size_t B16 = bb->tiled ? (B + 15) / 16 * 16 : B;   // tiled operands come in 16-row tiles
+    MRS_CREATE_TRY(dev_alloc3(bb, &bb->normed, B16 * dm * es));
+    MRS_CREATE_TRY(dev_alloc3(bb, &bb->gated, B16 * di * es));
     MRS_CREATE_TRY(dev_alloc3(bb, &bb->out, B * dm * es));
     MRS_CREATE_TRY(mrs_m3_backbone_reset(bb));
     { hipError_t e = hipStreamSynchronize(bb->stream);

@@ -120,24 +120,29 @@ def test_batch_rows_are_independent_and_graph_equals_eager():
 
 
 @pytest.mark.parametrize("dtype", [WeightDtype.BF16, WeightDtype.F16])
-@pytest.mark.parametrize("ci", [0, 1])
-def test_16bit_engine_tracks_cpu_path_on_rounded_weights(dtype, ci):
+@pytest.mark.parametrize("ci,B", [(0, 2), (1, 2), (0, 7), (1, 21), (2, 16)])
+def test_16bit_engine_tracks_cpu_path_on_rounded_weights(dtype, ci, B):
     """bf16/f16 storage (own-GEMM decode chain: folded RMSNorm, residual epilogue) vs the CPU route on weights
-    rounded to the storage type: cosine >= 0.999 per step, the reference's mixed-precision bar."""
+    rounded to the storage type: cosine >= 0.999 per step, the reference's mixed-precision bar.  Two rows take the
+    row-wise GEMM route; from five rows up the projections read tiled weights and tiled operands (7 and 21 rows: one and
+    two 16-row tiles, partly filled; 16: a whole one), eager for 24 steps, then replayed."""
     cfg = CONFIGS[ci]
     w = perturbed(cfg, 64, 11 + ci)
     w.input_proj_w = np.zeros(0, np.float32)
     code = orc.BF16 if dtype == WeightDtype.BF16 else orc.F16
     wi = Mamba3Weights(np.eye(64, dtype=np.float32), np.zeros(64, np.float32), w.layers, w.norm_f_weight)
     P = oracle_params(wi, cfg, 64, round_to=code)
-    eng = GpuMamba3Backbone.new_with_dtype(0, w, cfg, 64, 2, dtype)
-    st = [P.zero_state() for _ in range(2)]
+    eng = GpuMamba3Backbone.new_with_dtype(0, w, cfg, 64, B, dtype)
+    rows = sorted({0, B // 2, B - 1})
+    st = {b: P.zero_state() for b in rows}
     rng = np.random.default_rng(3)
-    x = rng.standard_normal((48, 2, 64)).astype(np.float32)
-    print(f"case m3 engine 16-bit dtype={dtype} config={ci}", flush=True)
+    x = rng.standard_normal((48, B, 64)).astype(np.float32)
+    print(f"case m3 engine 16-bit dtype={dtype} config={ci} batch={B}", flush=True)
     for t in range(48):
+        if t == 24:
+            eng.capture_graph()
         got = eng.step(x[t])
-        for b in range(2):
+        for b in rows:
             want = orc.m3_backbone_step(P, x[t, b], st[b])
             assert cosine(got[b], want) >= 0.999, (t, b)
     eng.close()
