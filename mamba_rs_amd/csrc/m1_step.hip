@@ -44,7 +44,7 @@ constexpr int kFoldMaxXd = 256;
 // shares in fold.xpart [tile][row][xd] -- so each workgroup first sums the shares of its batch row, in tile order,
 // rounds them to the storage type as the stored projection would be, and keeps the row in LDS.  A workgroup's 256 / LG
 // channels lie in one batch row (d_inner is a multiple of that).
-template <typename T, int LG, int DT, bool VECBC, bool FOLD = false>
+template <typename T, int LG, int DT, bool VECBC, bool FOLD = false, int PRE = 4>
 __global__ __launch_bounds__(256) void ssm_step_kernel(
     float *__restrict__ h, T *__restrict__ y, const T *__restrict__ delta, const T *__restrict__ u,
     const T *__restrict__ Bbase, const T *__restrict__ Cbase, int64_t bc_stride,
@@ -91,11 +91,23 @@ __global__ __launch_bounds__(256) void ssm_step_kernel(
         ld4<T, VECBC>(Cbase + (int64_t)b * bc_stride + 4 * g, Cv);
     }
     const int kpl = DT == 2 ? dr / LG : 0;
-    float wv0[4][4];   // DT 2: the first 16 terms of this lane's share of the weight row
+    // DT 2: this lane's share of the weight row is requested here, with everything else that waits for nothing -- the
+    // first 16 terms, or the first 48 (16-bit storage, d_state 16: a dt_rank of 160 over four lanes is 40 -- fetched inside
+    // the loop below they were two more round trips behind the sum of the x_proj shares)
+    // PRE = 12 costs 14 registers (a sixth wave per SIMD, which the 130m shape at 64 rows needs to run in one round), so
+    // only a dt_rank that needs it takes that variant
+    constexpr int kPre = PRE;   // groups of four terms
+    struct alignas(4 * sizeof(T)) W4 { T v[4]; };
+    W4 wq[kPre];
     if constexpr (DT == 2) {
         const T *wp = dt_w + (int64_t)d * dr + g * kpl;
 #pragma unroll
-        for (int j = 0; j < 4; j++) ld4<T, true>(wp + (4 * j < kpl ? 4 * j : 0), wv0[j]);
+        for (int cb = 0; cb < kPre / 4; cb++) {
+            if (cb == 0 || 16 * cb < kpl) {   // the same for every lane; a narrow dt_rank asks for its one round only
+#pragma unroll
+                for (int j = 4 * cb; j < 4 * cb + 4; j++) wq[j] = *reinterpret_cast<const W4 *>(wp + (4 * j < kpl ? 4 * j : 0));
+            }
+        }
     }
     if constexpr (FOLD) {
         const int xd = fold.xd;
@@ -129,19 +141,34 @@ __global__ __launch_bounds__(256) void ssm_step_kernel(
         float part = 0.0f;
         if constexpr (DT == 2) {
             const T *xp = xr + g * kpl, *wp = dt_w + (int64_t)d * dr + g * kpl;
-            for (int c0 = 0; c0 < kpl; c0 += 16) {
+            // the prefetched groups, sixteen terms a round (the same order of additions as the loop behind them)
+#pragma unroll
+            for (int cb = 0; cb < kPre / 4; cb++) {
+                const int c0 = 16 * cb;
+                if (c0 < kpl) {
+                    float xv[4][4];
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        const int kk = c0 + 4 * j;
+                        const bool in = kk < kpl;
+                        ld4<T, true>(xp + (in ? kk : 0), xv[j]);      // masked-off chunks read an in-range address
+#pragma unroll
+                        for (int i = 0; i < 4; i++) xv[j][i] = in ? xv[j][i] : 0.0f;
+                    }
+#pragma unroll
+                    for (int j = 0; j < 4; j++)
+#pragma unroll
+                        for (int i = 0; i < 4; i++) part = fmaf(xv[j][i], Store<T>::ld(&wq[4 * cb + j].v[i]), part);
+                }
+            }
+            for (int c0 = 4 * kPre; c0 < kpl; c0 += 16) {
                 float xv[4][4], wv[4][4];
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
                     const int kk = c0 + 4 * j;
                     const bool in = kk < kpl;
-                    ld4<T, true>(xp + (in ? kk : 0), xv[j]);      // masked-off chunks read an in-range address
-                    if (c0 == 0) {
-#pragma unroll
-                        for (int i = 0; i < 4; i++) wv[j][i] = wv0[j][i];
-                    } else {
-                        ld4<T, true>(wp + (in ? kk : 0), wv[j]);
-                    }
+                    ld4<T, true>(xp + (in ? kk : 0), xv[j]);
+                    ld4<T, true>(wp + (in ? kk : 0), wv[j]);
 #pragma unroll
                     for (int i = 0; i < 4; i++) xv[j][i] = in ? xv[j][i] : 0.0f;
                 }
@@ -271,6 +298,12 @@ static int launch_step(hipStream_t st, float *h, void *y, const void *delta, con
             StepFold folded = *fold;
             folded.y_mt = y_mt;
 #define MRS_LGF(L) case L: hipLaunchKernelGGL((ssm_step_kernel<T, L, 2, true, true>), grid, block, 0, st, MRS_ARGS, folded); break
+            if constexpr (sizeof(T) == 2) {
+                if (lg == 4 && dr / lg > 16) {   // a wide dt_rank: the whole weight share requested up front
+                    hipLaunchKernelGGL((ssm_step_kernel<T, 4, 2, true, true, 12>), grid, block, 0, st, MRS_ARGS, folded);
+                    return check_launch("ssm_step_kernel");
+                }
+            }
             switch (lg) { MRS_LGF(1); MRS_LGF(2); MRS_LGF(4); MRS_LGF(8); MRS_LGF(16); MRS_LGF(32); MRS_LGF(64); }
 #undef MRS_LGF
             return check_launch("ssm_step_kernel");
