@@ -275,7 +275,7 @@ typedef struct {            /* MambaWeights, src/weights.rs:51-64 */
 MRS_API int mrs_gemm_skinny(void *stream, int dtype, void *C, int out_f32, int64_t ldc, const void *A, int64_t lda,
                             const void *Wt, int M, int N, int K);
 MRS_API int mrs_transpose(void *stream, int dtype, void *Wt, const void *W, int K, int N);
-/* The same product from a TILED weight (what the decode chain reads from 5 rows up; wide models: in_proj of the 2.8b shape
+/* The same product from a TILED weight (what the decode chain reads from two or three rows up; wide models: in_proj of the 2.8b shape
  * is 52 MB): the 16 columns x 32 k of one matrix-core operand are 1 KB of consecutive memory, so the product is one
  * contiguous stream per wave (call sites src/mamba_ssm/gpu/blas.rs:1138-1163).
  *   mrs_tiled_weight_bytes: bytes of the tiled copy (columns padded to a multiple of 16); 0 for an unsupported dtype / K

@@ -134,7 +134,7 @@ struct SkinnyEpi {
     void *u_tiled;
     int u_tiled_mt;
 };
-// The same products from a TILED weight (gemm_wide.hip): 5..64 rows over a weight of megabytes.  Wp holds the 16 columns x 32 k
+// The same products from a TILED weight (gemm_wide.hip): up to 64 rows over a weight of megabytes.  Wp holds the 16 columns x 32 k
 // of each matrix-core operand as 1 KB in lane order, column tile by column tile (launch_tile_weight builds it from the
 // transposed weight Wt[N][K]; tiled_weight_elems() elements, columns padded to a multiple of 16).  Same epilogues, except
 // the x_proj shares (SkinnyEpi::xw, ksplit).

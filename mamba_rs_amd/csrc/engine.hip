@@ -213,7 +213,7 @@ struct LayerDev {
     void *dt_w_t;  // [d_inner][dt_rank] copy: the fused decode step (when dt_t_step) and the prefill dt_proj+softplus kernel read it
     int dt_t_step;
     void *in_proj_t, *x_proj_t, *out_proj_t;  // [N][K] copies: in / out for every 16-bit engine (own GEMM and vendor GEMM read them), x for the own chain only
-    void *in_proj_p, *out_proj_p, *x_proj_p;  // tiled copies (launch_tile_weight): the own chain from 5 rows up
+    void *in_proj_p, *out_proj_p, *x_proj_p;  // tiled copies (launch_tile_weight): the own chain from two or three rows up
     int s4d;
 };
 
@@ -264,7 +264,7 @@ struct mrs_backbone {
     mrs_m1_config cfg;
     int input_dim, batch, dtype, di, dr, xd, identity_proj, device;
     const float *step_src;  // decode step: where layer 0 reads its input rows (null: the residual buffer itself)
-    int tiled;   // own chain from 5 rows up: the projections read tiled weights and tiled activation operands
+    int tiled;   // own chain from two (narrow models) or three rows up: the projections read tiled weights and tiled activation operands
     int wide;    // ... and in_proj / out_proj run on the column-tile kernel of gemm_wide.hip (wide models, up to 64 rows)
     int skinny;  // decode projections on the library's own GEMM (16-bit storage: batch <= 128 or 64, K % 32 == 0; f32: batch <= 4, K % 128 == 0)
     hipStream_t stream;
@@ -599,13 +599,18 @@ extern "C" int mrs_backbone_create(mrs_backbone **out, int gpu_ordinal, const mr
         // vendor kernels), measured: 128 at the 130m shape (1032 vs 1091 us per step; at 256 rows 1490 vs 1392), 40 at the
         // 2.8b shape (32 rows 5.13 vs 8.35 ms, 40 rows 5.74 vs 5.92, 48 rows 6.13 vs 5.98, 64 rows 7.58 vs 6.19).  "Narrow"
         // as for the x_proj shares.
-        // From 5 rows up (the matrix-core route) the projections of the own chain read TILED operands -- weights tiled at load,
+        // From two (narrow models) or three rows up the projections of the own chain run on the matrix cores and read TILED operands -- weights tiled at load,
         // activation operands written tiled by their producers.  On wide models in_proj / out_proj also run on the
         // column-tile kernel of gemm_wide.hip, which carries the own chain up to 64 rows there.
         static const bool no_tiled = [] { const char *e = getenv("MRS_DECODE_NO_TILED"); return e && atoi(e) != 0; }();
         static const int tiled_max_rows = [] { const char *e = getenv("MRS_DECODE_TILED_MAX_ROWS"); return e ? atoi(e) : 64; }();
         const bool pow2_state = ds == 4 || ds == 8 || ds == 16 || ds == 32 || ds == 64 || ds == 128 || ds == 256;
-        const bool can_tile = !off && !no_tiled && (dtype == MRS_BF16 || dtype == MRS_F16) && batch >= 5 && dm % 32 == 0 && di % 32 == 0 && pow2_state;
+        // Below that the lanes-along-the-row route of the 16 x 16-tile GEMM is the faster one.  Per step, row-wise / tiled
+        // matrix-core route: 130m shape 330 / 356 us at 1 row, 378 / 359 at 2, 420 / 370 at 4; 2.8b shape 1.90 / 2.22 ms at
+        // 1 row, 2.08 / 2.25 at 2, 2.42 / 2.27 at 3, 2.48 / 2.31 at 4.
+        static const int forced_min_rows = [] { const char *e = getenv("MRS_DECODE_TILED_MIN_ROWS"); return e ? atoi(e) : 0; }();
+        const int tiled_min_rows = forced_min_rows > 0 ? forced_min_rows : (narrow_model(di, xd) ? 2 : 3);
+        const bool can_tile = !off && !no_tiled && (dtype == MRS_BF16 || dtype == MRS_F16) && batch >= tiled_min_rows && dm % 32 == 0 && di % 32 == 0 && pow2_state;
         bb->wide = can_tile && batch <= std::min(tiled_max_rows, 64) && (int64_t)dm * 2 * di >= (int64_t)8 << 20 && !narrow_model(di, xd);
         const int max_rows = std::min(skinny_max_rows(), narrow_model(di, xd) ? 128 : (bb->wide ? 64 : 40));
         bb->skinny = !off && (dtype == MRS_BF16 || dtype == MRS_F16) && batch <= max_rows && dm % 32 == 0 && di % 32 == 0;

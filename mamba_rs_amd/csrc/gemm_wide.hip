@@ -1,4 +1,4 @@
-// Decode GEMM for wide models: C[M,N] = A[M,K] . W[K,N] with 5 <= M <= 64 rows (the batch) and a weight of megabytes
+// Decode GEMM for wide models: C[M,N] = A[M,K] . W[K,N] with up to 64 rows (the batch; the decode chain comes here from 3 rows) and a weight of megabytes
 // (in_proj of the 2.8b shape: 2560 x 10240, 52 MB), 16-bit operands, f32 accumulate on the matrix cores.
 //
 // The reference sends these products to the vendor GEMM (cuBLAS call sites src/mamba_ssm/gpu/blas.rs:1138-1163).  At

@@ -550,7 +550,7 @@ struct Layer3 {
     float *norm_w, *dt_bias, *bnw, *cnw, *b_bias, *c_bias, *D, *ngw;
     void *in_proj, *out_proj;      // [K][N] storage type (library GEMM)
     void *in_proj_t, *out_proj_t;  // [N][K] copies for the skinny GEMM (null: library chain)
-    void *in_proj_p, *out_proj_p;  // tiled copies (launch_tile_weight): the own chain from 5 rows up
+    void *in_proj_p, *out_proj_p;  // tiled copies (launch_tile_weight): the own chain from two rows up
 };
 
 }  // namespace
@@ -761,8 +761,10 @@ extern "C" int mrs_m3_backbone_create(mrs_m3_backbone **out, int gpu_ordinal, co
     const int dm = cfg->d_model, di = bb->di, ip = bb->ip, L = cfg->n_layers;
     // (above 64 rows the library chain is the faster one for this layer: 1261 vs 1318 us per step at 128 rows, 768-wide shape)
     bb->skinny = (dtype == MRS_BF16 || dtype == MRS_F16) && batch <= std::min(64, skinny_max_rows()) && dm % 32 == 0 && di % 32 == 0;
-    // from 5 rows up (the matrix-core route) the two projections read tiled weights and tiled activation operands
-    { const char *e = getenv("MRS_DECODE_NO_TILED"); bb->tiled = bb->skinny && batch >= 5 && !(e && atoi(e) != 0); }
+    // from two rows up the two projections run on the matrix cores and read tiled weights and tiled activation operands
+    // (768-wide shape, per step, row-wise / tiled route: 282 / 302 us at 1 row, 326 / 308 at 2, 364 / 308 at 3, 368 / 314 at 4)
+    { const char *e = getenv("MRS_DECODE_NO_TILED"), *m = getenv("MRS_DECODE_TILED_MIN_ROWS");
+      bb->tiled = bb->skinny && (dtype == MRS_BF16 || dtype == MRS_F16) && batch >= (m ? atoi(m) : 2) && !(e && atoi(e) != 0); }
     // f32 storage: the row-wise route of the same GEMM, one to four rows
     if (dtype == MRS_F32 && batch <= 4 && dm % 128 == 0 && di % 128 == 0 && (int64_t)di * 16 <= 48 * 1024 && getenv("MRS_DECODE_NO_ROWWISE") == nullptr)
         bb->skinny = 1;

@@ -203,7 +203,7 @@ def tile_weight(wt):
 
 def gemm_tiled(a, wp, N: int, *, out_f32: bool = False):
     """C[M,N] = A[M,K] . W from the tiled weight of tile_weight (16-bit operands, f32 accumulate; up to 64 rows over a weight
-    of 16 MB or more, up to 128 rows below that): the decode projections from 5 rows up, which the reference sends to cuBLAS
+    of 16 MB or more, up to 128 rows below that): the decode projections from two or three rows up, which the reference sends to cuBLAS
     (src/mamba_ssm/gpu/blas.rs:1138-1163)."""
     _dev(wp)
     if not a.is_cuda or a.dim() != 2 or a.stride(1) != 1:

@@ -123,9 +123,9 @@ def test_batch_rows_are_independent_and_graph_equals_eager():
 @pytest.mark.parametrize("ci,B", [(0, 2), (1, 2), (0, 7), (1, 21), (2, 16)])
 def test_16bit_engine_tracks_cpu_path_on_rounded_weights(dtype, ci, B):
     """bf16/f16 storage (own-GEMM decode chain: folded RMSNorm, residual epilogue) vs the CPU route on weights
-    rounded to the storage type: cosine >= 0.999 per step, the reference's mixed-precision bar.  Two rows take the
-    row-wise GEMM route; from five rows up the projections read tiled weights and tiled operands (7 and 21 rows: one and
-    two 16-row tiles, partly filled; 16: a whole one), eager for 24 steps, then replayed."""
+    rounded to the storage type: cosine >= 0.999 per step, the reference's mixed-precision bar.  From two rows up the
+    projections run on the matrix cores and read tiled weights and tiled operands (2, 7 and 21 rows: one and two 16-row
+    tiles, partly filled; 16: a whole one), eager for 24 steps, then replayed."""
     cfg = CONFIGS[ci]
     w = perturbed(cfg, 64, 11 + ci)
     w.input_proj_w = np.zeros(0, np.float32)
