@@ -286,22 +286,25 @@ def lm_leg(name, cfg_kw, vocab, prefill_bt, decode_b, decode_steps, seed=42, sha
     lm_p = GpuMambaLM(pre, embed)
     toks = rng.integers(0, vocab, (pb, pt)).astype(np.int32)
     lm_p.prefill(toks); pre.sync()                      # warm-up (library kernel selection, scratch)
-    times = []
-    for _ in range(3):
-        pre.reset(); pre.sync()
-        t0 = time.perf_counter(); lm_p.prefill(toks); pre.sync(); times.append(time.perf_counter() - t0)
-    tp = sorted(times)[1]
+
+    def timed_prefill():
+        # untimed passes until the GPU has been under load for 150 ms (its clocks settle within about 50 ms), then three timed
+        t_end = time.perf_counter() + 0.15
+        while time.perf_counter() < t_end:
+            pre.reset(); lm_p.prefill(toks); pre.sync()
+        times = []
+        for _ in range(3):
+            pre.reset(); pre.sync()
+            t0 = time.perf_counter(); lm_p.prefill(toks); pre.sync(); times.append(time.perf_counter() - t0)
+        return sorted(times)[1]
+    tp = timed_prefill()
     out["prefill"] = {"batch": pb, "seq_len": pt, "ms": tp * 1e3, "tok_per_s": pb * pt / tp}
     if gemm_tuning:
         t0 = time.perf_counter()
         pre.set_gemm_tuning(True)
         pre.reset(); lm_p.prefill(toks); pre.sync()     # the projection shapes are timed over the library's kernels here
         tune_s = time.perf_counter() - t0
-        times = []
-        for _ in range(3):
-            pre.reset(); pre.sync()
-            t0 = time.perf_counter(); lm_p.prefill(toks); pre.sync(); times.append(time.perf_counter() - t0)
-        tt = sorted(times)[1]
+        tt = timed_prefill()
         out["prefill"] = {"batch": pb, "seq_len": pt, "ms": tt * 1e3, "tok_per_s": pb * pt / tt, "vendor_gemm_kernels": "timed once, fastest kept",
                           "tuning_s": tune_s, "ms_with_default_vendor_kernels": tp * 1e3}
     out["prefill"]["roofline"] = m1_prefill_roofline(cfg, pb, pt, out["prefill"]["ms"] * 1e-3)
@@ -653,6 +656,9 @@ def m3_engine_leg(steps=512, batches=(1, 16), prefill_bt=(4, 4096)):
     pb, pt = prefill_bt
     pre = GpuMamba3Backbone.new_with_dtype(0, w, cfg, 768, pb, WeightDtype.BF16)
     pre.prefill_sequence((rng.standard_normal((pb, pt, 768)) * 0.5).astype(np.float32))   # warm-up; leaves the input on the device
+    t_end = time.perf_counter() + 0.15      # untimed passes until the clocks have settled under load, as in lm_leg
+    while time.perf_counter() < t_end:
+        pre.reset(); pre.prefill_device(pt); pre.sync()
     times = []
     for _ in range(3):
         pre.reset(); pre.sync()
