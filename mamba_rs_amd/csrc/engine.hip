@@ -49,6 +49,18 @@ static rocblas_datatype blas_type(int dtype) {
 
 // ---- glue kernels -------------------------------------------------------------------
 
+// out[i] = round_T(sum over the K slices of a split x_proj of part[slice][i]), slices added in order (the library chain's
+// x_proj at 65 to 128 rows: a K-split launch of the own GEMM and this sum take 10 us where the vendor kernel for 128 x 192 x
+// 5120 takes 15.7)
+template <typename T>
+__global__ __launch_bounds__(256) void sum_shares_kernel(T *__restrict__ out, const float *__restrict__ part, int slices, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    float s = 0.0f;
+    for (int k = 0; k < slices; k++) s += part[(int64_t)k * n + i];
+    Store<T>::st(out + i, s);
+}
+
 // delta = softplus(raw + bias[d]) in place (dt_proj bias + softplus_forward, kernels/activations.cu:32-52).
 // VEC elements per thread as one 16-byte access (VEC = 16 / sizeof(T), d_inner % VEC == 0), or one by one.
 template <typename T, int VEC>
@@ -264,6 +276,7 @@ struct mrs_backbone {
     mrs_m1_config cfg;
     int input_dim, batch, dtype, di, dr, xd, identity_proj, device;
     const float *step_src;  // decode step: where layer 0 reads its input rows (null: the residual buffer itself)
+    int split_xproj;  // library chain at up to 128 rows of a wide 16-bit model: x_proj as a K-split launch of the own GEMM
     int tiled;   // own chain from two (narrow models) or three rows up: the projections read tiled weights and tiled activation operands
     int wide;    // ... and in_proj / out_proj run on the column-tile kernel of gemm_wide.hip (wide models, up to 64 rows)
     int skinny;  // decode projections on the library's own GEMM (16-bit storage: batch <= 128 or 64, K % 32 == 0; f32: batch <= 4, K % 128 == 0)
@@ -325,6 +338,10 @@ static int alloc_scratch(mrs_backbone *bb, Scratch *s, int64_t rows, int T) {
     MRS_TRY(dev_alloc(bb, &s->y, rows16 * di * es));
     MRS_TRY(dev_alloc(bb, &s->out, rows * dm * es));
     if (T == 1) MRS_TRY(dev_alloc(bb, (void **)&s->partials, rows * (size_t)((dm + 15) / 16) * sizeof(float)));
+    if (T == 1 && !bb->skinny && bb->split_xproj) {
+        s->xpart_floats = (int64_t)kMaxXprojSlices * rows * xd;
+        MRS_TRY(dev_alloc(bb, (void **)&s->xpart, (size_t)s->xpart_floats * sizeof(float)));
+    }
     if (T == 1 && bb->skinny) {
         // shares of the x_proj rows: per 16-column tile of in_proj (few rows), else per K slice of a split x_proj
         int64_t need = (int64_t)kMaxXprojSlices * rows * xd;
@@ -491,7 +508,20 @@ static int run_layers(mrs_backbone *bb, Scratch *s, int T) {
         else MRS_TRY(gemm_rm(bb, dt, s->proj, 2 * di, s->normed, dm, lw.in_proj, (int)rows, 2 * di, dm));
         if (T == 1) {
             MRS_TRY(launch_conv1d_step(bb->stream, dt, s->u, conv, s->proj, 2 * di, lw.conv_w, lw.conv_b, B, di, dc, 1));
-            MRS_TRY(gemm_rm(bb, dt, s->xdbl, xd, s->u, di, lw.x_proj, (int)rows, xd, di));
+            if (bb->split_xproj && lw.x_proj_p && s->xpart) {
+                // few output tiles over a long K: the own GEMM with K cut into slices, then the slices added up
+                const int tiles = ((xd + 15) / 16) * (((int)rows + 15) / 16);
+                const int ksplit = std::max(2, std::min(std::min(kMaxXprojSlices, 768 / tiles), di / 32 / 8));
+                SkinnyEpi xp = {};
+                xp.ksplit = ksplit; xp.xpart = s->xpart; xp.w_tiled = 1;
+                MRS_TRY(launch_skinny_gemm(bb->stream, dt, s->xdbl, 0, xd, s->u, di, lw.x_proj_p, (int)rows, xd, di, xp));
+                const int64_t n = rows * xd;
+                MRS_DISPATCH_DTYPE(dt, T_, hipLaunchKernelGGL((sum_shares_kernel<T_>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, bb->stream,
+                                                              (T_ *)s->xdbl, s->xpart, ksplit, n));
+                MRS_TRY(check_launch("sum_shares_kernel"));
+            } else {
+                MRS_TRY(gemm_rm(bb, dt, s->xdbl, xd, s->u, di, lw.x_proj, (int)rows, xd, di));
+            }
             if ((int64_t)B * dr <= kFuseDtProjLimit) {
                 // dt_proj (K = dt_rank) + bias + softplus + state update + B/C gather + SiLU gate: one kernel
                 MRS_TRY(launch_ssm_step_fused(bb->stream, dt, ssm, s->y, s->delta, lw.dt_b, s->xdbl, lw.dt_t_step ? lw.dt_w_t : lw.dt_w, dr,
@@ -616,6 +646,8 @@ extern "C" int mrs_backbone_create(mrs_backbone **out, int gpu_ordinal, const mr
         bb->skinny = !off && (dtype == MRS_BF16 || dtype == MRS_F16) && batch <= max_rows && dm % 32 == 0 && di % 32 == 0;
         bb->tiled = can_tile && bb->skinny;
         if (!bb->skinny) bb->wide = 0;
+        bb->split_xproj = !off && !bb->skinny && (dtype == MRS_BF16 || dtype == MRS_F16) && batch <= 128 && di % 256 == 0 && xd % 8 == 0 &&
+                          !narrow_model(di, xd);
         // f32 storage: the same chain on the row-wise route of the GEMM (one to four rows, rows of the operand in LDS)
         if (!off && dtype == MRS_F32 && batch <= 4 && dm % 128 == 0 && di % 128 == 0 && (int64_t)di * 16 <= 48 * 1024 &&
             getenv("MRS_DECODE_NO_ROWWISE") == nullptr)
@@ -662,10 +694,10 @@ extern "C" int mrs_backbone_create(mrs_backbone **out, int gpu_ordinal, const mr
             MRS_CREATE_TRY(launch_tile_weight(bb->stream, bb->dtype, d.in_proj_p, d.in_proj_t, 2 * di, dm));
             MRS_CREATE_TRY(launch_tile_weight(bb->stream, bb->dtype, d.out_proj_p, d.out_proj_t, dm, di));
         }
-        if (bb->skinny) {
+        if (bb->skinny || bb->split_xproj) {
             MRS_CREATE_TRY(dev_alloc(bb, &d.x_proj_t, (size_t)di * xd * esize(bb->dtype)));
             MRS_CREATE_TRY(launch_transpose(bb->stream, bb->dtype, d.x_proj_t, d.x_proj, di, xd));
-            if (bb->tiled) {
+            if (bb->tiled || bb->split_xproj) {
                 MRS_CREATE_TRY(dev_alloc(bb, &d.x_proj_p, tiled_weight_elems(xd, di) * esize(bb->dtype)));
                 MRS_CREATE_TRY(launch_tile_weight(bb->stream, bb->dtype, d.x_proj_p, d.x_proj_t, xd, di));
             }
