@@ -8,7 +8,7 @@
 //     A wave's load instruction then fetches one whole kilobyte and a wave streams a contiguous region -- with the
 //     row-major transposed copy the same instruction touches sixteen 64-byte pieces 2 K bytes apart (measured on the
 //     2.8b in_proj at 16 rows: 18.5 us tiled, 21.8 us row-major, the rest of the kernel being equal);
-//   * a workgroup owns 16 NT output columns (NT column tiles) over ALL of K and all rows.  Two or four of its eight
+//   * a workgroup owns 16 NT output columns (NT column tiles, up to three) over ALL of K and all rows.  Two or four of its eight
 //     waves stream the operands, wave w taking k-steps w, w + WS, ..., so every weight byte is requested once, by one
 //     wave, and no sum leaves the workgroup: the partial tiles meet in LDS (splitting K over workgroups instead, with
 //     the slices meeting in memory behind an arrival counter, cost 4-6 us of store / count / reload round trips at the
@@ -26,8 +26,9 @@
 //     costs the L1 sixty-four tag look-ups where a tile costs eight (in_proj at 64 rows: 24 us tiled, 38 us row-major);
 //   * the epilogues are those of gemm_skinny.hip (plain store, in_proj's conv step + SiLU, out_proj's residual add with
 //     the row's sums of squares), one result element per thread and pass: element (row ml, column nl) of a 16 x 16 tile
-//     sits in lane 16 (ml / 4) + nl, register ml % 4 of the accumulator.  With one element per thread its epilogue
-//     operands and the row's partial sums of squares are requested before the operand stream and wait in registers.
+//     sits in lane 16 (ml / 4) + nl, register ml % 4 of the accumulator.  The epilogue operands of all of a thread's
+//     elements are requested together (before the operand stream for up to two elements, right behind it otherwise)
+//     and the row's partial sums of squares before the stream.
 #include "common.hpp"
 #include "mfma_tiles.hpp"
 #include <stdlib.h>
@@ -77,48 +78,35 @@ __global__ __launch_bounds__(kTiledThreads) void tiled_gemm_kernel(void *__restr
         return __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(ares, aoff[mt], so, 0));
     };
     // Epilogue work is spread over all threads: element e = tid + (threads) j of the workgroup's MT NT tiles of 256 -- tile
-    // e / 256, row (e % 256) / 16 and column e % 16 of it -- so sixteen consecutive lanes share a row.  With one element
-    // per thread its epilogue operands (conv window, taps and bias; or residual and next norm weight) are requested
-    // here, ahead of the operand stream, and wait in registers.
+    // e / 256, row (e % 256) / 16 and column e % 16 of it -- so sixteen consecutive lanes share a row.
     constexpr int kTiles = MT * NT;
     constexpr int EP = (kTiles * 256 + kTiledThreads - 1) / kTiledThreads;
-    constexpr bool kPrefetch = EP == 1;
-    const int e_row0 = (tid >> 4) & 15, e_nl = tid & 15;
-    float4 pf_win = make_float4(0.f, 0.f, 0.f, 0.f), pf_tap = pf_win;
-    float pf_x = 0.0f, pf_y = 0.0f;
-    if constexpr (kPrefetch) {
-        const int tile = tid >> 8;
-        const int row = 16 * (tile / NT) + e_row0, col = 16 * ((int)blockIdx.x * NT + tile % NT) + e_nl;
-        if (tile < kTiles && row < M && col < N) {
-            if (ep.mode == 1 && col < ep.di && ep.dc == 4) {
-                pf_win = *reinterpret_cast<const float4 *>(ep.conv_state + ((int64_t)row * ep.di + col) * 4);
-                pf_tap = *reinterpret_cast<const float4 *>(ep.conv_w + (int64_t)col * 4);
-                pf_x = ep.conv_b[col];
-            } else if (ep.mode == 2) {
-                pf_x = ep.residual[(int64_t)row * N + col];
-                if (ep.next_norm_w) pf_y = ep.next_norm_w[col];
+    // The operands of an element's epilogue (conv window, taps and bias; or residual and next norm weight) are requested
+    // for all of a thread's elements at once: ahead of the operand stream where a thread has one or two elements, right
+    // behind the stream otherwise (the registers of the stream are free then) -- inside the element loop they would be
+    // one memory round trip per element, one after the other (the conv windows of a decode step are cold).
+    constexpr bool kEarly = EP <= 2;
+    float4 pf_win[EP], pf_tap[EP];
+    float pf_x[EP], pf_y[EP];
+    auto request_epilogue = [&]() {
+#pragma unroll
+        for (int j = 0; j < EP; j++) {
+            pf_win[j] = make_float4(0.f, 0.f, 0.f, 0.f); pf_tap[j] = pf_win[j]; pf_x[j] = 0.0f; pf_y[j] = 0.0f;
+            const int e = tid + kTiledThreads * j, tile = e >> 8;
+            const int row = 16 * (tile / NT) + ((e >> 4) & 15), col = 16 * ((int)blockIdx.x * NT + tile % NT) + (e & 15);
+            if (tile < kTiles && row < M && col < N) {
+                if (ep.mode == 1 && col < ep.di && ep.dc == 4) {
+                    pf_win[j] = *reinterpret_cast<const float4 *>(ep.conv_state + ((int64_t)row * ep.di + col) * 4);
+                    pf_tap[j] = *reinterpret_cast<const float4 *>(ep.conv_w + (int64_t)col * 4);
+                    pf_x[j] = ep.conv_b[col];
+                } else if (ep.mode == 2) {
+                    pf_x[j] = ep.residual[(int64_t)row * N + col];
+                    if (ep.next_norm_w) pf_y[j] = ep.next_norm_w[col];
+                }
             }
         }
-    }
-    // RMSNorm folded around the product (gemm_skinny.hip): 1/rms of each row from its partial sums of squares.  Sixteen
-    // lanes share a row; its partial sums (up to 256 of them, a multiple of four) are requested here as 16-byte pieces,
-    // all at once and ahead of the operand stream -- summed one load at a time in a loop they were ten L2 round trips in
-    // a row before the first matrix instruction (5.5 us of a 21 us in_proj at d_model 2560).
-    constexpr int kRowsPerPass = kTiledThreads / 16;
-    constexpr int kScalePasses = (16 * MT + kRowsPerPass - 1) / kRowsPerPass;
-    const bool ps_fast = ep.row_scale && ep.n_partials % 4 == 0 && ep.n_partials <= 256;
-    float4 ps[kScalePasses][4];
-    if (ps_fast) {
-#pragma unroll
-        for (int h = 0; h < kScalePasses; h++) {
-            const float *pp = ep.partials + (int64_t)min((tid >> 4) + kRowsPerPass * h, M - 1) * ep.n_partials;
-#pragma unroll
-            for (int q = 0; q < 4; q++) {
-                const int p4 = 4 * ((tid & 15) + 16 * q);
-                ps[h][q] = p4 < ep.n_partials ? *reinterpret_cast<const float4 *>(pp + p4) : make_float4(0.f, 0.f, 0.f, 0.f);
-            }
-        }
-    }
+    };
+    if constexpr (kEarly) request_epilogue();
     // waves 0 .. WS-1 stream the operands (wave w takes k-steps w, w + WS, ...); the others only share the epilogue
     const bool streams = w < WS;
     uint4 wr[R][NT], ar[R][MT];
@@ -132,32 +120,35 @@ __global__ __launch_bounds__(kTiledThreads) void tiled_gemm_kernel(void *__restr
             __builtin_amdgcn_sched_barrier(0);   // requested in the order of use, as in the loop (the wait counts of its first round follow this order)
         }
     }
-    // RMSNorm folded around the product (gemm_skinny.hip), second half: the partial sums requested above are in
-    if (ep.row_scale) {
-        if (ps_fast) {
+    // RMSNorm folded around the product (gemm_skinny.hip): 1/rms of each row from its partial sums of squares, by the
+    // waves that do not stream (the streaming waves entered their loop 1.3 us later when they shared this).  Sixteen
+    // lanes share a row; its partial sums (up to 256 of them, a multiple of four) are fetched as 16-byte pieces, all of a
+    // row's at once -- summed one load at a time in a loop they were ten L2 round trips in a row.
+    static_assert(WS <= 4, "at least four waves beside the streaming ones");
+    if (ep.row_scale && !streams) {
+        constexpr int kHelpers = kTiledThreads - 64 * WS;
+        const int ht = tid - 64 * WS;
+        const bool ps_fast = ep.n_partials % 4 == 0 && ep.n_partials <= 256;
+        for (int r = ht >> 4; r < 16 * MT; r += kHelpers / 16) {
+            const float *pp = ep.partials + (int64_t)min(r, M - 1) * ep.n_partials;
+            float ss = 0.0f;
+            if (ps_fast) {
+                float4 ps[4];
 #pragma unroll
-            for (int h = 0; h < kScalePasses; h++) {
-                float ss = 0.0f;
+                for (int q = 0; q < 4; q++) {
+                    const int p4 = 4 * ((ht & 15) + 16 * q);
+                    ps[q] = p4 < ep.n_partials ? *reinterpret_cast<const float4 *>(pp + p4) : make_float4(0.f, 0.f, 0.f, 0.f);
+                }
 #pragma unroll
-                for (int q = 0; q < 4; q++) ss += (ps[h][q].x + ps[h][q].y) + (ps[h][q].z + ps[h][q].w);
-#pragma unroll
-                for (int m = 8; m >= 1; m >>= 1) ss += __shfl_xor(ss, m, kWave);
-                float rms = sqrtf(ss / (float)K + ep.eps);
-                if (!isfinite(rms) || rms < 1e-20f) rms = 1.0f;
-                const int r = (tid >> 4) + kRowsPerPass * h;
-                if ((tid & 15) == 0 && r < 16 * MT) inv_s[r] = 1.0f / rms;
+                for (int q = 0; q < 4; q++) ss += (ps[q].x + ps[q].y) + (ps[q].z + ps[q].w);
+            } else {
+                for (int p_ = ht & 15; p_ < ep.n_partials; p_ += 16) ss += pp[p_];
             }
-        } else {
-            for (int r = tid >> 4; r < 16 * MT; r += kTiledThreads / 16) {
-                const float *pp = ep.partials + (int64_t)min(r, M - 1) * ep.n_partials;
-                float ss = 0.0f;
-                for (int p = tid & 15; p < ep.n_partials; p += 16) ss += pp[p];
 #pragma unroll
-                for (int m = 8; m >= 1; m >>= 1) ss += __shfl_xor(ss, m, kWave);
-                float rms = sqrtf(ss / (float)K + ep.eps);
-                if (!isfinite(rms) || rms < 1e-20f) rms = 1.0f;
-                if ((tid & 15) == 0) inv_s[r] = 1.0f / rms;
-            }
+            for (int m = 8; m >= 1; m >>= 1) ss += __shfl_xor(ss, m, kWave);
+            float rms = sqrtf(ss / (float)K + ep.eps);
+            if (!isfinite(rms) || rms < 1e-20f) rms = 1.0f;
+            if ((ht & 15) == 0) inv_s[r] = 1.0f / rms;
         }
     }
     v4f acc[MT][NT];
@@ -179,6 +170,7 @@ __global__ __launch_bounds__(kTiledThreads) void tiled_gemm_kernel(void *__restr
             __builtin_amdgcn_sched_barrier(0);   // keep each refill right behind its use: the scheduler would gather the loads at the end of the round
         }
     }
+    if constexpr (!kEarly) request_epilogue();
     // the K ranges meet in LDS: of four or eight streaming waves the upper half parks its tiles, the lower half adds them
     // and parks the sums (one or two streaming waves just park); the thread that owns an element then adds the parked
     // sums in wave order (one fixed order of additions)
@@ -225,8 +217,8 @@ __global__ __launch_bounds__(kTiledThreads) void tiled_gemm_kernel(void *__restr
             float sq = 0.0f;
             if (valid) {
                 const T orr = (T)s;
-                const float res_old = kPrefetch ? pf_x : ep.residual[(int64_t)row * N + col];
-                const float nw = kPrefetch ? pf_y : (ep.next_norm_w ? ep.next_norm_w[col] : 0.0f);
+                const float res_old = pf_x[j];
+                const float nw = pf_y[j];
                 const float rn = res_old + Store<T>::ld(&orr);
                 ep.residual[(int64_t)row * N + col] = rn;
                 sq = rn * rn;
@@ -245,9 +237,9 @@ __global__ __launch_bounds__(kTiledThreads) void tiled_gemm_kernel(void *__restr
             const float *cw = ep.conv_w + (int64_t)col * ep.dc;
             float o;
             if (ep.dc == 4) {   // window and taps are one aligned 16-byte vector each
-                const float4 win = kPrefetch ? pf_win : *reinterpret_cast<const float4 *>(st);
-                const float4 tap = kPrefetch ? pf_tap : *reinterpret_cast<const float4 *>(cw);
-                o = kPrefetch ? pf_x : ep.conv_b[col];
+                const float4 win = pf_win[j];
+                const float4 tap = pf_tap[j];
+                o = pf_x[j];
                 o = fmaf(win.y, tap.x, o); o = fmaf(win.z, tap.y, o); o = fmaf(win.w, tap.z, o); o = fmaf(xnew, tap.w, o);
                 *reinterpret_cast<float4 *>(st) = make_float4(win.y, win.z, win.w, xnew);
             } else {
@@ -286,24 +278,39 @@ int launch_tiled_t(hipStream_t st, void *C, int out_f32, int64_t ldc, const T *A
                    const SkinnyEpi &ep) {
     const int mt = (M + 15) / 16;
     const int ntiles = (N + 15) / 16;
-    // two column tiles per workgroup where the rows are many (a k-step's activation pieces serve both) and the chip stays
-    // full of workgroups
-    const int nt = (ntiles >= 512 && mt >= 2) ? 2 : 1;
-    // Streaming waves per workgroup (they split K): four at up to 16 rows, two above.  In the 2.8b-shape decode chain, per
-    // step with 1 / 2 / 4 / 8 of them: 16 rows 2.85 / 2.75 / 2.65 / 2.72 ms, 32 rows 3.48 / 3.35 / 3.44 / 3.62, 64 rows
-    // 5.29 / 4.77 / 4.81 / 4.92 -- more waves only put more requests in front of the memory system at once (alone, with
-    // a plain store, in_proj at 16 rows takes 13.7 us with one streaming wave and 18.3 us with eight).
+    // Column tiles per workgroup.  A compute unit keeps about 64 KB of requests in flight whatever runs on it (measured
+    // with time stamps per workgroup: two workgroups sharing a unit each take twice as long), so a launch takes as long
+    // as the unit with the most tiles: ceil(workgroups / 256) NT of them.  NT is the count of up to three that makes
+    // this smallest, the larger on a tie (fewer workgroups read the activation operand).  in_proj of the 2.8b shape,
+    // 640 tiles: 214 workgroups of three tiles -- with two tiles 320 workgroups, 64 units run two of them one after the
+    // other while the rest of the chip idles (alone, with a plain store, 64 rows: 22.6 us against 15.4 us; 16 rows, one
+    // tile: 12.9 against 11.4).
+    int nt = 1, worst = 1 << 30;
+    for (int c = 1; c <= 3; c++) {
+        const int wgs = (ntiles + c - 1) / c, load = (wgs + 255) / 256 * c;
+        if (load <= worst) { worst = load; nt = c; }
+    }
+    // Streaming waves WS (they split K) and k-steps R each keeps requested ahead: WS R (NT + MT) KB in flight per
+    // workgroup, 48 to 64 of them -- more only queues in front of the unit's memory pipeline (alone, with a plain
+    // store, in_proj at 16 rows and one tile takes 13.7 us with one streaming wave and 18.3 us with eight).  In the
+    // 2.8b-shape decode chain, per step with 1 / 2 / 4 / 8 streaming waves: 16 rows 2.85 / 2.75 / 2.65 / 2.72 ms,
+    // 32 rows 3.48 / 3.35 / 3.44 / 3.62, 64 rows 5.29 / 4.77 / 4.81 / 4.92.
     const dim3 grid((unsigned)((ntiles + nt - 1) / nt)), block(kTiledThreads);
 #define MRS_TG(MT_, NT_, R_, W_) \
     hipLaunchKernelGGL((tiled_gemm_kernel<T, MT_, NT_, R_, W_>), grid, block, 0, st, C, out_f32, ldc, A, lda, Wp, M, N, K, ep)
     switch (mt * 10 + nt) {
         case 11: MRS_TG(1, 1, 10, 4); break;
+        case 12: MRS_TG(1, 2, 5, 4); break;
+        case 13: MRS_TG(1, 3, 4, 4); break;
         case 21: MRS_TG(2, 1, 8, 2); break;
         case 22: MRS_TG(2, 2, 6, 2); break;
+        case 23: MRS_TG(2, 3, 3, 4); break;
         case 31: MRS_TG(3, 1, 6, 2); break;
         case 32: MRS_TG(3, 2, 5, 2); break;
+        case 33: MRS_TG(3, 3, 5, 2); break;
         case 41: MRS_TG(4, 1, 5, 2); break;
-        default: MRS_TG(4, 2, 4, 2); break;
+        case 42: MRS_TG(4, 2, 4, 2); break;
+        default: MRS_TG(4, 3, 2, 4); break;
     }
 #undef MRS_TG
     return check_launch("tiled_gemm_kernel");

@@ -173,12 +173,13 @@ def test_28b_shape_decode_follows_the_cpu_route(w28, B):
     """d_model 2560 / d_inner 5120 / dt_rank 160 / xdbl 192, two layers: the row-wise route (1 row), the own chain on
     tiled weights and tiled activation operands at 3 to 64 rows -- one to four 16-row tiles, whole (16, 64) and partly
     filled (3, 5, 23, 40); x_proj split over K with the shares summed by the step kernel up to 25 rows, a dt_proj launch of
-    its own above -- and the library chain (128 rows), eager then replayed."""
+    its own above -- and the library chain (81 and 128 rows: x_proj split over K by the own GEMM and summed by a small
+    kernel, the other projections by the GEMM library), eager then replayed."""
     w, P = w28
     print(f"case 2.8b-shape decode batch {B}", flush=True)
     assert CFG_28B.dt_rank() == 160 and CFG_28B.xdbl_dim() == 192
     eng = GpuMambaBackbone.new_with_dtype(0, w, CFG_28B, 2560, B, WeightDtype.BF16)
-    assert eng.decode_route() == (0 if B == 128 else 1), eng.decode_route()   # 0: library chain, 1: own chain
+    assert eng.decode_route() == (0 if B > 64 else 1), eng.decode_route()   # 0: library chain, 1: own chain
     rng = np.random.default_rng(B)
     x = orc.round_to(rng.standard_normal((5, B, 2560)).astype(np.float32), orc.BF16)
     rows = sorted({0, B // 2, B - 1})
