@@ -168,7 +168,7 @@ def w28():
     return w, lm_oracle(CFG_28B, w)
 
 
-@pytest.mark.parametrize("B", [1, 3, 5, 16, 23, 40, 64, 81, 128])
+@pytest.mark.parametrize("B", [1, 2, 3, 5, 16, 23, 40, 64, 81, 128])
 def test_28b_shape_decode_follows_the_cpu_route(w28, B):
     """d_model 2560 / d_inner 5120 / dt_rank 160 / xdbl 192, two layers: the row-wise route (1 row), the own chain on
     tiled weights and tiled activation operands at 3 to 64 rows -- one to four 16-row tiles, whole (16, 64) and partly

@@ -38,7 +38,7 @@ def test_gemm_skinny_matches_f64_matmul(shape, dtype, out_f32):
 # (M, N, K): the 2.8b decode projections at one to four 16-row tiles (whole and partly filled), N not a multiple of 16, a K
 # shorter than the eight waves' ranges, a K that does not divide by them
 # (small weights go to the 16 x 16 tiles reading the same tiled weight: the 130m decode projections, up to 128 rows)
-TILED_SHAPES = [(16, 10240, 2560), (64, 10240, 2560), (5, 2560, 5120), (23, 2560, 5120), (40, 2560, 5120), (64, 2560, 5120),
+TILED_SHAPES = [(16, 4096, 2080), (16, 10240, 2560), (64, 10240, 2560), (5, 2560, 5120), (23, 2560, 5120), (40, 2560, 5120), (64, 2560, 5120),
                 (16, 200, 96), (33, 16, 32), (48, 1000, 1056), (1, 50, 256), (64, 8200, 64),
                 (64, 3072, 768), (128, 768, 1536), (97, 80, 1536), (3, 3072, 768)]
 
