@@ -58,6 +58,20 @@ def scan_algorithmic_bytes(batch, T, di, ds, s, gated=True):
     return 3 * act + (act if gated else 0) + 2 * batch * T * ds * s + 2 * 4 * batch * di * ds + 4 * di * ds + 4 * di
 
 
+def loaded_libraries(names):
+    """Paths of the shared libraries with these name prefixes that are mapped into this process."""
+    found = set()
+    try:
+        with open("/proc/self/maps") as f:
+            for line in f:
+                path = line.rsplit(" ", 1)[-1].strip()
+                if any(os.path.basename(path).startswith(n) for n in names):
+                    found.add(path)
+    except OSError:
+        pass
+    return sorted(found)
+
+
 def make_inputs(batch, T, di, ds, seed=42):
     import numpy as np
     from util import scan_inputs
@@ -699,6 +713,50 @@ def m3_engine_leg(steps=512, batches=(1, 16), prefill_bt=(4, 4096)):
     return {"prefill": prefill, "decode": out}
 
 
+def engine_legs(args, legs, tune):
+    """The legs that drive the engines through the C ABI from numpy buffers: no torch in them."""
+    extras = {}
+    if "c1" in legs:
+        extras["tiny_f32_cpu_config"] = c1_leg()
+        extras["reference_default_configs_f32"] = default_configs_leg()
+    if "lm" in legs:
+        extras["lm_130m_shape_bf16"] = lm_leg("130m-shape", dict(d_model=768, d_state=16, d_conv=4, expand=2, n_layers=24), 50280,
+                                              (8, 2048), [64, 1], 256, cpu_sample=(24, 256), gemm_tuning=tune,
+                                              decode_graph=not args.lm_no_graph)
+    if "published" in legs:
+        extras["reference_published_configs"] = published_configs_leg()
+    if "m3_engine" in legs:
+        extras["mamba3_768_bf16"] = {"backbone": m3_engine_leg()}
+    elif "m3_prefill" in legs:   # the backbone's prefill alone (not a default leg: the command behind its profile)
+        extras["mamba3_768_bf16"] = {"backbone": m3_engine_leg(batches=())}
+    if "lm28" in legs or args.big:
+        extras["lm_2.8b_shape_bf16"] = lm_leg("2.8b-shape", dict(d_model=2560, d_state=16, d_conv=4, expand=2, n_layers=64), 50280,
+                                              (4, 4096), [1, 16, 64, 128], 128, shared_layer=not args.big, cpu_sample=(2, 64),
+                                              with_generate=False, gemm_tuning=tune, decode_graph=not args.lm_no_graph)
+    return extras
+
+
+def run_engine_legs_child(args, tune):
+    """Runs the engine legs in a child process (started before this process has touched the GPU) and returns its JSON line,
+    or {"failure": ...} -- the caller then runs the legs itself."""
+    import subprocess
+    cmd = [sys.executable, os.path.abspath(__file__), "--engine-legs-child", "--legs", args.legs, "--gemm-tune", "on" if tune else "off"]
+    if args.big:
+        cmd.append("--big")
+    if args.lm_no_graph:
+        cmd.append("--lm-no-graph")
+    try:
+        r = subprocess.run(cmd, capture_output=True, text=True, timeout=1500)
+        if r.returncode != 0:
+            return {"failure": f"exit code {r.returncode}: {r.stderr.strip()[-300:]}"}
+        res = json.loads(r.stdout.strip().splitlines()[-1])
+        if res.get("torch_in_process"):
+            return {"failure": "the child process imported torch"}
+        return res
+    except Exception as e:   # noqa: BLE001 - any failure of the child falls back to the in-process legs
+        return {"failure": f"{type(e).__name__}: {e}"}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -712,6 +770,14 @@ def main():
     ap.add_argument("--big", action="store_true", help="the 2.8b-shape LM leg with 64 independently initialised layers (minutes of host-side init) instead of one shared layer")
     ap.add_argument("--gemm-tune", choices=["auto", "on", "off"], default="auto",
                     help="prefill legs of the LM engines pick their vendor GEMM kernels by timing them (auto: in the full default run only)")
+    ap.add_argument("--engine-legs", choices=["auto", "child", "inprocess"], default="auto",
+                    help="where the engine legs (c1, lm, lm28, published, m3_engine) run.  torch bundles its own build of the vendor GEMM "
+                         "library, and a process that imports torch first binds libmamba_hip.so to that copy; a host without torch, such "
+                         "as the Rust binding, runs on the copy under /opt/rocm, whose kernels for the engines' library projections "
+                         "(prefill; decode past the own chain's row limit) are faster.  'child' runs those legs, which need no torch, in "
+                         "a process of their own before this one touches the GPU; 'inprocess' runs them here behind the torch legs; "
+                         "'auto' = child in the full default run, inprocess when --legs, --no-cpu or --lm-no-graph narrows it (profiling)")
+    ap.add_argument("--engine-legs-child", action="store_true", help=argparse.SUPPRESS)
     ap.add_argument("--lm-no-graph", action="store_true",
                     help="the decode steps of the lm / lm28 legs launch kernel by kernel instead of replaying a hipGraph, and the "
                          "generation runs are skipped (for kernel traces of those steps)")
@@ -726,6 +792,18 @@ def main():
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus must be 1 (no multi-GPU path exists)", file=sys.stderr)
         sys.exit(2)
+    tune = args.gemm_tune == "on" or (args.gemm_tune == "auto" and legs == set(DEFAULT_LEGS.split(",")))
+    if args.engine_legs_child:
+        # the engine legs alone, in a process that never imports torch; one JSON line for the parent
+        res = {"extras": engine_legs(args, legs, tune), "torch_in_process": "torch" in sys.modules,
+               "libraries": loaded_libraries(("librocblas", "libhipblaslt", "libamdhip64"))}
+        print(json.dumps(res))
+        return
+    child = None
+    use_child = args.engine_legs == "child" or (args.engine_legs == "auto" and legs == set(DEFAULT_LEGS.split(",")) and not args.no_cpu
+                                                 and not args.lm_no_graph)
+    if use_child and not args.no_extras:
+        child = run_engine_legs_child(args, tune)
     shape = (8, 2048, 1536, 16)
     batch, T, di, ds = shape
     nbytes = scan_algorithmic_bytes(batch, T, di, ds, 2, gated=True)
@@ -776,28 +854,25 @@ def main():
         out["cpu_baseline"] = cpu_leg(inp, shape, nbytes)
     if not args.no_extras:
         extras = {}
-        tune = args.gemm_tune == "on" or (args.gemm_tune == "auto" and legs == set(DEFAULT_LEGS.split(",")))
-        if "c1" in legs:
-            extras["tiny_f32_cpu_config"] = c1_leg()
-            extras["reference_default_configs_f32"] = default_configs_leg()
-        if "lm" in legs:
-            extras["lm_130m_shape_bf16"] = lm_leg("130m-shape", dict(d_model=768, d_state=16, d_conv=4, expand=2, n_layers=24), 50280,
-                                                  (8, 2048), [64, 1], 256, cpu_sample=(24, 256), gemm_tuning=tune,
-                                                  decode_graph=not args.lm_no_graph)
-        if "published" in legs:
-            extras["reference_published_configs"] = published_configs_leg()
         if "m1_kernels" in legs:
             extras["m1_kernels_130m_shape_bf16"] = m1_kernels_leg()
-        if "m3" in legs or "m3_engine" in legs or "m3_prefill" in legs:
-            extras["mamba3_768_bf16"] = m3_leg() if "m3" in legs else {}
-        if "m3_engine" in legs:
-            extras["mamba3_768_bf16"]["backbone"] = m3_engine_leg()
-        elif "m3_prefill" in legs:   # the backbone's prefill alone (not a default leg: the command behind its profile)
-            extras["mamba3_768_bf16"]["backbone"] = m3_engine_leg(batches=())
-        if "lm28" in legs or args.big:
-            extras["lm_2.8b_shape_bf16"] = lm_leg("2.8b-shape", dict(d_model=2560, d_state=16, d_conv=4, expand=2, n_layers=64), 50280,
-                                                  (4, 4096), [1, 16, 64, 128], 128, shared_layer=not args.big, cpu_sample=(2, 64),
-                                                  with_generate=False, gemm_tuning=tune, decode_graph=not args.lm_no_graph)
+        if "m3" in legs:
+            extras["mamba3_768_bf16"] = m3_leg()
+        if child is not None and "extras" in child:
+            eng, where = child["extras"], {"process": "child process without torch", "libraries": child.get("libraries")}
+        else:
+            eng = engine_legs(args, legs, tune)
+            where = {"process": "this process, behind the torch legs", "libraries": loaded_libraries(("librocblas", "libhipblaslt", "libamdhip64"))}
+            if child is not None:
+                where["child_failure"] = child.get("failure")
+        for k, v in eng.items():
+            if k == "mamba3_768_bf16":
+                extras.setdefault(k, {}).update(v)
+            else:
+                extras[k] = v
+        where["note"] = ("the copies of the vendor libraries the engine legs ran on (see --engine-legs): their prefill projections and the "
+                         "128-row decode of the 2.8b shape are the library's kernels; this package's own kernels do not depend on it")
+        extras["engine_legs"] = where
         out["extras"] = extras
     print(json.dumps(out))
 
