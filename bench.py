@@ -58,6 +58,16 @@ def scan_algorithmic_bytes(batch, T, di, ds, s, gated=True):
     return 3 * act + (act if gated else 0) + 2 * batch * T * ds * s + 2 * 4 * batch * di * ds + 4 * di * ds + 4 * di
 
 
+def spin_steps(step, sync, seconds=0.15):
+    """Untimed decode steps until the GPU has been under load for `seconds` (its clocks settle within about 50 ms of
+    sustained work; eight steps of a small model are over before they move), as the kernel and prefill legs do."""
+    t_end = time.perf_counter() + seconds
+    while time.perf_counter() < t_end:
+        for _ in range(16):
+            step()
+        sync()
+
+
 def loaded_libraries(names):
     """Paths of the shared libraries with these name prefixes that are mapped into this process."""
     found = set()
@@ -335,9 +345,7 @@ def lm_leg(name, cfg_kw, vocab, prefill_bt, decode_b, decode_steps, seed=42, sha
             lm_d.set_tokens(rng.integers(0, vocab, db).astype(np.int32))
             if decode_graph:
                 lm_d.capture_graph()
-            for _ in range(8):
-                lm_d.decode_step()
-            dec.sync()
+            spin_steps(lm_d.decode_step, dec.sync)
             t0 = time.perf_counter()
             for _ in range(decode_steps):
                 lm_d.decode_step()
@@ -405,9 +413,7 @@ def c1_leg():
         t0 = time.perf_counter(); orc.m1_backbone_prefill(P, x[0], cs, ss); ctimes.append(time.perf_counter() - t0)
     tc = sorted(ctimes)[2]
     eng.reset(); eng.step(x[0, 0:1]); eng.capture_graph()
-    for _ in range(8):
-        eng.step_gpu_only()
-    eng.sync()
+    spin_steps(eng.step_gpu_only, eng.sync)
     t0 = time.perf_counter()
     for _ in range(256):
         eng.step_gpu_only()
@@ -439,9 +445,7 @@ def default_configs_leg():
 
     def run(eng, x, n=400):
         eng.step(x); eng.capture_graph()
-        for _ in range(10):
-            eng.step_gpu_only()
-        eng.sync()
+        spin_steps(eng.step_gpu_only, eng.sync)
         t0 = time.perf_counter()
         for _ in range(n):
             eng.step_gpu_only()
@@ -499,9 +503,7 @@ def published_configs_leg():
         lm = GpuMambaLM(dec, embed)
         lm.set_tokens(rng.integers(0, vocab, B).astype(np.int32))
         lm.capture_graph()
-        for _ in range(8):
-            lm.decode_step()
-        dec.sync()
+        spin_steps(lm.decode_step, dec.sync)
         t0 = time.perf_counter()
         for _ in range(128):
             lm.decode_step()
@@ -684,9 +686,7 @@ def m3_engine_leg(steps=512, batches=(1, 16), prefill_bt=(4, 4096)):
         eng = GpuMamba3Backbone.new_with_dtype(0, w, cfg, 768, B, WeightDtype.BF16)
         eng.step((rng.standard_normal((B, 768)) * 0.5).astype(np.float32))
         eng.capture_graph()
-        for _ in range(8):
-            eng.step_gpu_only()
-        eng.sync()
+        spin_steps(eng.step_gpu_only, eng.sync)
         t0 = time.perf_counter()
         for _ in range(steps):
             eng.step_gpu_only()
