@@ -24,6 +24,9 @@ DEVICE_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     # MFMA accumulators stay in ordinary VGPRs (no AccVGPR copies around each instruction).
     "-mllvm", "-amdgpu-mfma-vgpr-form",
+    # The first 16 dwords of a kernel's arguments arrive in scalar registers with the wave instead of being loaded by its
+    # first instructions: 0.15 us per launch, which is 3 % of a batch-1 decode step (72 launches of 4.5 us).
+    "-mllvm", "-amdgpu-kernarg-preload-count=16",
     "-Wno-unused-command-line-argument", "-Wno-unused-result", "-Wno-unused-value",
 ]
 
