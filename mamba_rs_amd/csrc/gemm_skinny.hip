@@ -101,44 +101,59 @@ __global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu
     const T *arow = a_tiled ? A + (int64_t)(m0 >> 4) * 512 + 8 * l : A + (int64_t)min(m0 + lr, M - 1) * lda + 8 * lg;
     const int wks = w_tiled ? 512 : 32, aks = a_tiled ? 512 * ((M + 15) >> 4) : 32;   // elements from one k-step's piece to the next
     float inv = 1.0f;
-    // The partial sums of a row are requested together, before the operands stream, and added up after the product
-    // (in the order a loop over them would add them): loaded one at a time inside such a loop they were a chain of
-    // n_partials / 16 round trips to L2 ahead of the first operand request (ten at d_model 2560).
-    constexpr int kScaleAhead = 8;   // partial sums per lane requested ahead (d_model up to 2048; more would spill in_proj's variants); any beyond are loaded late
-    float psum[PRO == 1 ? kScaleAhead : 1];
+    // The partial sums of a row are requested together, right behind the first operand requests, and added up at once in
+    // the order a loop over them would add them (loads come back in the order they were issued, so this waits for nothing
+    // the first products do not wait for as well).  Loaded one at a time inside such a loop they were a chain of
+    // n_partials / 16 round trips to L2 ahead of the first operand request (ten at d_model 2560); requested ahead of the
+    // operands and kept until after the product, three of the eight were spilled under this kernel's register limit, each
+    // behind a wait of its own for its load.
+    // Partial sums per lane requested together; any beyond are loaded late.  Matrix-core route: the 16 lanes of an
+    // epilogue row share them, four each (narrow models: d_model up to 1024 without a late load; no registers to spare
+    // for more under this kernel's limit).  Row-wise route (up to four rows): wave m sums row m, four per lane cover 256
+    // partial sums, and the rows' scales meet the epilogue threads in LDS.
+    constexpr int kScaleAhead = 4;
+    constexpr int kScaleLanes = LPR == 0 ? 16 : 64;
+    __shared__ float inv_rows[4];
+    float ss_ahead;                           // set by row_scale_fold alone (an addition to a preset would be made at the loads)
+    float psum[PRO == 1 ? kScaleAhead : 1];   // no presets, no branch around a load: see prefetch_epilogue
+    const bool scale_thread = PRO == 1 && (LPR == 0 ? tid < 256 : w < MR);   // the same for a whole wave
+    const int scale_row = m0 + (LPR == 0 ? (tid >> 4) : w), scale_lane = LPR == 0 ? (tid & 15) : l;
     auto row_scale_request = [&]() {
-        if (PRO == 1 && tid < 256) {
-            const float *pp = ep.partials + (int64_t)min(m0 + (tid >> 4), M - 1) * ep.n_partials;
+        if (scale_thread) {
+            const float *pp = ep.partials + (int64_t)min(scale_row, M - 1) * ep.n_partials;
 #pragma unroll
-            for (int j = 0; j < kScaleAhead; j++) {
-                const int p = (tid & 15) + 16 * j;
-                psum[j] = p < ep.n_partials ? pp[p] : 0.0f;
-            }
+            for (int j = 0; j < kScaleAhead; j++) psum[j] = pp[min(scale_lane + kScaleLanes * j, ep.n_partials - 1)];
+        }
+    };
+    auto row_scale_fold = [&]() {
+        if (scale_thread) {
+            float a = scale_lane < ep.n_partials ? psum[0] : 0.0f;
+#pragma unroll
+            for (int j = 1; j < kScaleAhead; j++) a += scale_lane + kScaleLanes * j < ep.n_partials ? psum[j] : 0.0f;
+            ss_ahead = a;
         }
     };
     auto row_scale = [&]() {
-        if (PRO == 1 && tid < 256) {
-            // epilogue thread (row tid/16, column tid%16): the 16 lanes of a row share the sum over the partials
-            const float *pp = ep.partials + (int64_t)min(m0 + (tid >> 4), M - 1) * ep.n_partials;
-            float ss = 0.0f;
-#pragma unroll
-            for (int j = 0; j < kScaleAhead; j++) ss += psum[j];
-            if (ep.n_partials > 16 * kScaleAhead) {   // a wider row: the next eight per lane as one more round trip, then one at a time
+        if (scale_thread) {
+            const float *pp = ep.partials + (int64_t)min(scale_row, M - 1) * ep.n_partials;
+            float ss = ss_ahead;
+            if (ep.n_partials > kScaleLanes * kScaleAhead) {   // a wider row: the next eight per lane as one more round trip, then one at a time
                 float late[8];
 #pragma unroll
                 for (int j = 0; j < 8; j++) {
-                    const int p = (tid & 15) + 16 * (kScaleAhead + j);
+                    const int p = scale_lane + kScaleLanes * (kScaleAhead + j);
                     late[j] = p < ep.n_partials ? pp[p] : 0.0f;
                 }
 #pragma unroll
                 for (int j = 0; j < 8; j++) ss += late[j];
-                for (int p = (tid & 15) + 16 * (kScaleAhead + 8); p < ep.n_partials; p += 16) ss += pp[p];
+                for (int p = scale_lane + kScaleLanes * (kScaleAhead + 8); p < ep.n_partials; p += kScaleLanes) ss += pp[p];
             }
 #pragma unroll
-            for (int m = 8; m >= 1; m >>= 1) ss += __shfl_xor(ss, m, kWave);
+            for (int m = kScaleLanes / 2; m >= 1; m >>= 1) ss += __shfl_xor(ss, m, kWave);
             float rms = sqrtf(ss / (float)K + ep.eps);
             if (!isfinite(rms) || rms < 1e-20f) rms = 1.0f;
             inv = 1.0f / rms;
+            if (LPR != 0 && l == 0) inv_rows[w] = inv;   // published by the barrier behind the products
         }
     };
     // Epilogue operands that do not depend on the product -- the conv window / taps / bias (mode 1), the
@@ -147,34 +162,49 @@ __global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu
     const bool e_valid = tid < 256 && e_row < M && e_col < N;
     constexpr bool kConv = EPI == 1 || EPI == 3;
     constexpr int kTaps = EPI == 3 ? kMaxConvTaps : 4;
-    float win[kTaps], cwv[kTaps], cbias = 0.0f, res_old = 0.0f, nw = 0.0f;
+    // No presets and no branch that depends on the lane around a load: a value that is a load on one path and a constant
+    // on another has to be copied into place once the load is back, and the compiler waits for the load right there --
+    // each of these requests then cost a memory round trip of its own in front of the product.  Lanes whose element lies
+    // outside the result load from a clamped (row, column) and never use what they get.
+    float win[kTaps], cwv[kTaps], cbias, res_old, nw;
     auto prefetch_epilogue = [&]() {
-        if (kConv && e_valid && e_col < ep.di) {
-            const float *st = ep.conv_state + ((int64_t)e_row * ep.di + e_col) * ep.dc;
-            const float *cw = ep.conv_w + (int64_t)e_col * ep.dc;
-            if constexpr (EPI == 1) {   // four taps: window and taps are one aligned 16-byte vector each
-                const float4 s4 = *reinterpret_cast<const float4 *>(st), c4 = *reinterpret_cast<const float4 *>(cw);
-                win[0] = s4.y; win[1] = s4.z; win[2] = s4.w;
-                cwv[0] = c4.x; cwv[1] = c4.y; cwv[2] = c4.z; cwv[3] = c4.w;
-            } else {
+        if (tid < 256) {   // the same for a whole wave
+            const int r = min(e_row, M - 1), c = min(e_col, N - 1);
+            if constexpr (kConv) {
+                const int cc = min(c, ep.di - 1);
+                const float *st = ep.conv_state + ((int64_t)r * ep.di + cc) * ep.dc;
+                const float *cw = ep.conv_w + (int64_t)cc * ep.dc;
+                if constexpr (EPI == 1) {   // four taps: window and taps are one aligned 16-byte vector each
+                    const float4 s4 = *reinterpret_cast<const float4 *>(st), c4 = *reinterpret_cast<const float4 *>(cw);
+                    win[0] = s4.y; win[1] = s4.z; win[2] = s4.w; win[3] = 0.0f;
+                    cwv[0] = c4.x; cwv[1] = c4.y; cwv[2] = c4.z; cwv[3] = c4.w;
+                } else {
 #pragma unroll
-                for (int k = 0; k < kTaps; k++) {
-                    win[k] = (k + 1 < ep.dc) ? st[k + 1] : 0.0f;
-                    cwv[k] = (k < ep.dc) ? cw[k] : 0.0f;
+                    for (int k = 0; k < kTaps; k++) {
+                        win[k] = (k + 1 < ep.dc) ? st[k + 1] : 0.0f;
+                        cwv[k] = (k < ep.dc) ? cw[k] : 0.0f;
+                    }
                 }
+                cbias = ep.conv_b[cc];
             }
-            cbias = ep.conv_b[e_col];
+            if constexpr (EPI == 2) {
+                const float *pr = ep.residual + (int64_t)r * N + c;
+                res_old = *pr;
+                nw = *(ep.next_norm_w ? ep.next_norm_w + c : pr);   // used only with a next norm weight
+            }
         }
-        if (EPI == 2 && e_valid) {
-            res_old = ep.residual[(int64_t)e_row * N + e_col];
-            if (ep.next_norm_w) nw = ep.next_norm_w[e_col];
-        }
+    };
+    // every request first, then the first use of any of them (left to itself the scheduler puts the first partial sum's
+    // addition in front of the epilogue's requests, which then start a memory round trip late)
+    auto early_requests = [&]() {
+        row_scale_request();
+        prefetch_epilogue();
+        __builtin_amdgcn_sched_barrier(0);
+        row_scale_fold();
     };
     // Requested up front, but on the matrix-core route behind the first round of operand loads: with several row
     // tiles the conv windows are a megabyte-scale read that would otherwise queue ahead of the operands.
     if constexpr (LPR != 0) {
-        row_scale_request();
-        prefetch_epilogue();
         constexpr int NC = LPR == 64 ? 2 : 1;           // columns a lane works on (with 32 lanes per row each half-wave has its own)
         constexpr int JB = LPR == 64 ? 2 : 4;             // pieces per column requested together
         const int ll = l & (LPR - 1), half = LPR == 64 ? 0 : (l >> 5);
@@ -201,6 +231,10 @@ __global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu
                         av[j] = *reinterpret_cast<const uint4 *>(A + EPV * ll + off);
                     }
                 }
+                // the row's partial sums and the epilogue's operands behind the first weight requests (ahead of them, the
+                // conv sum the compiler starts from window, taps and bias alone waited for the cold conv windows before
+                // any weight was asked for)
+                if (jb == 0) { early_requests(); }
 #pragma unroll
                 for (int j = 0; j < J1; j++) {
                     if (jb + j < per) {
@@ -226,6 +260,7 @@ __global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu
 #pragma unroll
                 for (int t = 0; t < NC; t++) wv[t][j] = *reinterpret_cast<const uint4 *>(wp[t] + EPV * LPR * j);
             }
+        early_requests();
         lds_barrier();   // the rows are in LDS; the weight loads above stay in flight
         for (int jb = 0; jb < per; jb += JB) {
             uint4 nx[NC][JB];
@@ -278,10 +313,9 @@ __global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu
         }
     };
     constexpr int kStride = kGemmWaves * kHalf;   // k-steps one half-batch covers across the workgroup's waves
-    row_scale_request();
     request(0, k_lo + w);
     request(1, k_lo + w + kStride);
-    prefetch_epilogue();
+    early_requests();
     for (int base = k_lo + w; base < nk; base += 2 * kStride) {
 #pragma unroll
         for (int s = 0; s < kHalf; s++) acc = Mma32<T>::mma(af[0][s], bf[0][s], acc);
@@ -309,6 +343,7 @@ __global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu
 #pragma unroll
             for (int ww = 0; ww < kGemmWaves / 2; ww++) s += red[ww][lane][i];
         }
+        if constexpr (LPR != 0 && PRO == 1) inv = inv_rows[ml < MR ? ml : 0];
         s *= inv;
         const int row = m0 + ml, col = n0 + nl;
         const bool valid = row < M && col < N;

@@ -89,24 +89,26 @@ __global__ __launch_bounds__(kTiledThreads) void tiled_gemm_kernel(void *__restr
     float4 pf_win[EP], pf_tap[EP];
     float pf_x[EP], pf_y[EP];
     auto request_epilogue = [&]() {
+        // Four loads per element, issued on every path with no branch around them: the addresses are chosen by selects (a
+        // clamped row / column where the element lies outside the result, the activation operand's first bytes where the
+        // epilogue has no such operand).  A value that is a load on one path and something else on another has to be copied
+        // into place once the load is back, and the wait for that copy sat in front of the operand stream -- a memory round
+        // trip for the cold conv windows before the first weight request.
+        const bool conv4 = ep.mode == 1 && ep.dc == 4, resid = ep.mode == 2;
+        const float4 *dummy4 = reinterpret_cast<const float4 *>(A);
+        const float *dummy = reinterpret_cast<const float *>(A);
 #pragma unroll
         for (int j = 0; j < EP; j++) {
-            pf_win[j] = make_float4(0.f, 0.f, 0.f, 0.f); pf_tap[j] = pf_win[j]; pf_x[j] = 0.0f; pf_y[j] = 0.0f;
-            const int e = tid + kTiledThreads * j, tile = e >> 8;
-            const int row = 16 * (tile / NT) + ((e >> 4) & 15), col = 16 * ((int)blockIdx.x * NT + tile % NT) + (e & 15);
-            if (tile < kTiles && row < M && col < N) {
-                if (ep.mode == 1 && col < ep.di && ep.dc == 4) {
-                    pf_win[j] = *reinterpret_cast<const float4 *>(ep.conv_state + ((int64_t)row * ep.di + col) * 4);
-                    pf_tap[j] = *reinterpret_cast<const float4 *>(ep.conv_w + (int64_t)col * 4);
-                    pf_x[j] = ep.conv_b[col];
-                } else if (ep.mode == 2) {
-                    pf_x[j] = ep.residual[(int64_t)row * N + col];
-                    if (ep.next_norm_w) pf_y[j] = ep.next_norm_w[col];
-                }
-            }
+            const int e = tid + kTiledThreads * j, tile = min(e >> 8, kTiles - 1);
+            const int row = min(16 * (tile / NT) + ((e >> 4) & 15), M - 1), col = min(16 * ((int)blockIdx.x * NT + tile % NT) + (e & 15), N - 1);
+            const int cc = conv4 ? min(col, ep.di - 1) : 0;
+            const float4 *pw = conv4 ? reinterpret_cast<const float4 *>(ep.conv_state + ((int64_t)row * ep.di + cc) * 4) : dummy4;
+            const float4 *pt = conv4 ? reinterpret_cast<const float4 *>(ep.conv_w + (int64_t)cc * 4) : dummy4;
+            const float *px = conv4 ? ep.conv_b + cc : (resid ? ep.residual + (int64_t)row * N + col : dummy);
+            const float *py = (resid && ep.next_norm_w) ? ep.next_norm_w + col : dummy;
+            pf_win[j] = *pw; pf_tap[j] = *pt; pf_x[j] = *px; pf_y[j] = *py;
         }
     };
-    if constexpr (kEarly) request_epilogue();
     // waves 0 .. WS-1 stream the operands (wave w takes k-steps w, w + WS, ...); the others only share the epilogue
     const bool streams = w < WS;
     uint4 wr[R][NT], ar[R][MT];
@@ -120,6 +122,7 @@ __global__ __launch_bounds__(kTiledThreads) void tiled_gemm_kernel(void *__restr
             __builtin_amdgcn_sched_barrier(0);   // requested in the order of use, as in the loop (the wait counts of its first round follow this order)
         }
     }
+    if constexpr (kEarly) request_epilogue();   // behind the first operand requests: loads come back in the order they were issued
     // RMSNorm folded around the product (gemm_skinny.hip): 1/rms of each row from its partial sums of squares, by the
     // waves that do not stream (the streaming waves entered their loop 1.3 us later when they shared this).  Sixteen
     // lanes share a row; its partial sums (up to 256 of them, a multiple of four) are fetched as 16-byte pieces, all of a
@@ -218,7 +221,7 @@ __global__ __launch_bounds__(kTiledThreads) void tiled_gemm_kernel(void *__restr
             if (valid) {
                 const T orr = (T)s;
                 const float res_old = pf_x[j];
-                const float nw = pf_y[j];
+                const float nw = ep.next_norm_w ? pf_y[j] : 0.0f;
                 const float rn = res_old + Store<T>::ld(&orr);
                 ep.residual[(int64_t)row * N + col] = rn;
                 sq = rn * rn;
