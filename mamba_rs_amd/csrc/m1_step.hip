@@ -81,9 +81,14 @@ __global__ __launch_bounds__(256) void ssm_step_kernel(
     const float4 av = *reinterpret_cast<const float4 *>(a_neg + (int64_t)d * ds + 4 * g);
     const float uu = Store<T>::ld(u + r);
     const float Dd = Dp[d];
-    float bias = 0.0f, gz = 0.0f, dl = 0.0f;
-    if (dt_bias) bias = dt_bias[d];
-    if (gate_mode != 0) gz = Store<T>::ld(gate + (int64_t)b * gate_stride + d);
+    // the optional operands are loaded on every path, from an address that is valid either way, and looked at only where
+    // they apply: a value that is a load on one path and a preset on the other is copied into place once the load is
+    // back, and the wait for that copy stood between these requests and the ones below (a round trip of its own)
+    // (the stand-in address is one that nothing else here loads from: a load the compiler finds twice becomes a branch
+    // around the other one again)
+    const float bias = *(dt_bias ? dt_bias + d : Dp + (d + 1 < di ? d + 1 : 0));
+    const float gz = Store<T>::ld(gate_mode != 0 ? gate + (int64_t)b * gate_stride + d : u + (r + 1 < total ? r + 1 : 0));
+    float dl = 0.0f;
     if constexpr (DT == 0) dl = Store<T>::ld(delta + r);
     float Bv[4], Cv[4];
     if constexpr (!FOLD) {
