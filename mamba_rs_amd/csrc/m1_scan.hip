@@ -490,14 +490,17 @@ __device__ __forceinline__ void pass_a_body(
     load_a2<S4D>(a2, a_neg, dd);
 #pragma unroll
     for (int j = 0; j < 16; j++) hs[j] = 0.0f;
-    if (c == 0) {
+    auto load_entering = [&]() {   // chunk 0 alone starts from the caller's state
+        if (c == 0) {
 #pragma unroll
-        for (int j = 0; j < 16; j++) {
-            hs[j] = h[((int64_t)b * di + dd) * 16 + j];
-            if constexpr (FUSED) h_keep[j] = hs[j];
-            else if (live) h0copy[((int64_t)b * 16 + j) * di + dd] = hs[j];
+            for (int j = 0; j < 16; j++) {
+                hs[j] = h[((int64_t)b * di + dd) * 16 + j];
+                if constexpr (FUSED) h_keep[j] = hs[j];
+                else if (live) h0copy[((int64_t)b * 16 + j) * di + dd] = hs[j];
+            }
         }
-    }
+    };
+    if (!S4D) load_entering();   // the forward walk needs it at once
     const int t0 = c * len;
     const int64_t row0 = (int64_t)b * Tlen;
     const int64_t slab = (int64_t)Tlen * di - d0;  // elements from this wave's base to the end of batch row b
@@ -527,13 +530,18 @@ __device__ __forceinline__ void pass_a_body(
         for (int j = 0; j < 16; j++) S16[j] = 0.0f;
         // spans are walked last to first; span s sits in slot s & 1, span s-1 is published while s is computed and
         // the rows of span s-2 requested
+        // everything the first steps need is requested before any of it is used (loads come back in the order they were
+        // issued): the rows of the last span, those of the span before it, the first group of steps, and -- chunk 0 --
+        // the entering state, which the backward walk needs only at its end.  One after the other they were three memory
+        // round trips in front of the first step, for every wave of the launch at the same time.
         {
             RowPiece<T> first;
             piece_ld(first, Bp, bc_stride, t0 + (nspans - 1) * kSpan + prow);
+            piece_ld(nb, Bp, bc_stride, t0 + max(nspans - 2, 0) * kSpan + prow);
+            load_group(rdB, ruB, t0 + (nspans - 1) * kSpan + kGroup);
+            load_entering();
             Bs.publish((nspans - 1) & 1, piece_widen(first, (const T *)nullptr));
         }
-        piece_ld(nb, Bp, bc_stride, t0 + max(nspans - 2, 0) * kSpan + prow);
-        load_group(rdB, ruB, t0 + (nspans - 1) * kSpan + kGroup);
         for (int sp = nspans - 1; sp >= 0; sp--) {
             const int ts = t0 + sp * kSpan, slot = sp & 1;
             set_progress_priority(nspans - 1 - sp, nspans);
@@ -574,12 +582,12 @@ __device__ __forceinline__ void pass_a_body(
 #pragma unroll
         for (int r = 0; r < 16; r++) hr[r] = hs[kStateOfReg(r)];
         {
-            RowPiece<T> first;
+            RowPiece<T> first;   // requested together, as in the backward walk above
             piece_ld(first, Bp, bc_stride, t0 + prow);
+            piece_ld(nb, Bp, bc_stride, t0 + min(1, nspans - 1) * kSpan + prow);
+            load_group(rdA, ruA, t0);
             Bs.publish(0, piece_widen(first, (const T *)nullptr));
         }
-        piece_ld(nb, Bp, bc_stride, t0 + min(1, nspans - 1) * kSpan + prow);
-        load_group(rdA, ruA, t0);
         v4f bv = Bs.read(0, 0);
         for (int sp = 0; sp < nspans; sp++) {
             const int ts = t0 + sp * kSpan, slot = sp & 1;
