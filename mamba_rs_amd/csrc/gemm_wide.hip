@@ -27,8 +27,8 @@
 //   * the epilogues are those of gemm_skinny.hip (plain store, in_proj's conv step + SiLU, out_proj's residual add with
 //     the row's sums of squares), one result element per thread and pass: element (row ml, column nl) of a 16 x 16 tile
 //     sits in lane 16 (ml / 4) + nl, register ml % 4 of the accumulator.  The epilogue operands of all of a thread's
-//     elements are requested together (before the operand stream for up to two elements, right behind it otherwise)
-//     and the row's partial sums of squares before the stream.
+//     elements are requested together behind the first operand requests; the rows' scales are formed by the waves
+//     that do not stream.
 #include "common.hpp"
 #include "mfma_tiles.hpp"
 #include <stdlib.h>
@@ -82,10 +82,9 @@ __global__ __launch_bounds__(kTiledThreads) void tiled_gemm_kernel(void *__restr
     constexpr int kTiles = MT * NT;
     constexpr int EP = (kTiles * 256 + kTiledThreads - 1) / kTiledThreads;
     // The operands of an element's epilogue (conv window, taps and bias; or residual and next norm weight) are requested
-    // for all of a thread's elements at once: ahead of the operand stream where a thread has one or two elements, right
-    // behind the stream otherwise (the registers of the stream are free then) -- inside the element loop they would be
-    // one memory round trip per element, one after the other (the conv windows of a decode step are cold).
-    constexpr bool kEarly = EP <= 2;
+    // for all of a thread's elements at once, right behind the first operand requests (the conv windows of a decode step
+    // are cold: fetched inside the element loop they would be a memory round trip per element, behind the stream one
+    // round trip at the end of the kernel; a workgroup per compute unit has the registers to hold them).
     float4 pf_win[EP], pf_tap[EP];
     float pf_x[EP], pf_y[EP];
     auto request_epilogue = [&]() {
@@ -122,7 +121,7 @@ __global__ __launch_bounds__(kTiledThreads) void tiled_gemm_kernel(void *__restr
             __builtin_amdgcn_sched_barrier(0);   // requested in the order of use, as in the loop (the wait counts of its first round follow this order)
         }
     }
-    if constexpr (kEarly) request_epilogue();   // behind the first operand requests: loads come back in the order they were issued
+    request_epilogue();   // behind the first operand requests: loads come back in the order they were issued
     // RMSNorm folded around the product (gemm_skinny.hip): 1/rms of each row from its partial sums of squares, by the
     // waves that do not stream (the streaming waves entered their loop 1.3 us later when they shared this).  Sixteen
     // lanes share a row; its partial sums (up to 256 of them, a multiple of four) are fetched as 16-byte pieces, all of a
@@ -173,7 +172,6 @@ __global__ __launch_bounds__(kTiledThreads) void tiled_gemm_kernel(void *__restr
             __builtin_amdgcn_sched_barrier(0);   // keep each refill right behind its use: the scheduler would gather the loads at the end of the round
         }
     }
-    if constexpr (!kEarly) request_epilogue();
     // the K ranges meet in LDS: of four or eight streaming waves the upper half parks its tiles, the lower half adds them
     // and parks the sums (one or two streaming waves just park); the thread that owns an element then adds the parked
     // sums in wave order (one fixed order of additions)
