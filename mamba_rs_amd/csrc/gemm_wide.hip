@@ -10,7 +10,7 @@
 //     2.8b in_proj at 16 rows: 18.5 us tiled, 21.8 us row-major, the rest of the kernel being equal);
 //   * a workgroup owns 16 NT output columns (NT column tiles, up to three) over ALL of K and all rows.  Two or four of its eight
 //     waves stream the operands, wave w taking k-steps w, w + WS, ..., so every weight byte is requested once, by one
-//     wave, and no sum leaves the workgroup: the partial tiles meet in LDS (splitting K over workgroups instead, with
+//     wave, and no sum leaves the workgroup: the waves' partial tiles meet in LDS (splitting K over workgroups instead, with
 //     the slices meeting in memory behind an arrival counter, cost 4-6 us of store / count / reload round trips at the
 //     end of a 12 us stream).  The other waves only share the epilogue: more streaming waves put more requests in
 //     front of the memory system at once and the stream gets slower, fewer epilogue threads make the end of the kernel
@@ -42,7 +42,7 @@ constexpr int kTiledThreads = 512;   // eight waves per workgroup: WS of them st
 template <typename T, int MT, int NT, int R, int WS = 8>
 __global__ __launch_bounds__(kTiledThreads) void tiled_gemm_kernel(void *__restrict__ Cv, int out_f32, int64_t ldc, const T *__restrict__ A,
                                                                    int64_t lda, const T *__restrict__ Wp, int M, int N, int K, SkinnyEpi ep) {
-    constexpr int kPark = WS >= 4 ? WS / 2 : WS;   // partial tiles that meet in LDS
+    constexpr int kPark = WS;   // partial tiles that meet in LDS, one per streaming wave
     __shared__ v4f red[kPark][MT * NT][kWave];
     __shared__ float inv_s[16 * MT];
     const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), l = tid & 63, lr = l & 15, lg = l >> 4;
@@ -172,24 +172,9 @@ __global__ __launch_bounds__(kTiledThreads) void tiled_gemm_kernel(void *__restr
             __builtin_amdgcn_sched_barrier(0);   // keep each refill right behind its use: the scheduler would gather the loads at the end of the round
         }
     }
-    // the K ranges meet in LDS: of four or eight streaming waves the upper half parks its tiles, the lower half adds them
-    // and parks the sums (one or two streaming waves just park); the thread that owns an element then adds the parked
-    // sums in wave order (one fixed order of additions)
-    if constexpr (WS >= 4) {
-        if (w >= WS / 2 && w < WS) {
-#pragma unroll
-            for (int mt = 0; mt < MT; mt++)
-#pragma unroll
-                for (int nt = 0; nt < NT; nt++) red[w - WS / 2][mt * NT + nt][l] = acc[mt][nt];
-        }
-        lds_barrier();
-        if (w < WS / 2) {
-#pragma unroll
-            for (int mt = 0; mt < MT; mt++)
-#pragma unroll
-                for (int nt = 0; nt < NT; nt++) red[w][mt * NT + nt][l] += acc[mt][nt];
-        }
-    } else if (streams) {
+    // the K ranges meet in LDS: every streaming wave parks its tiles, and the thread that owns an element adds them in
+    // wave order (one fixed order of additions, one barrier)
+    if (streams) {
 #pragma unroll
         for (int mt = 0; mt < MT; mt++)
 #pragma unroll
