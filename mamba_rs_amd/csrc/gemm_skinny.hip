@@ -80,7 +80,7 @@ template <typename T, typename TO, int EPI, int PRO, int LPR = 0, int MR = 1>
 __global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu(6))) void skinny_gemm_kernel(
     TO *__restrict__ C, int64_t ldc, const T *__restrict__ A, int64_t lda, const T *__restrict__ Wt, int M, int N, int K,
     SkinnyEpi ep) {
-    __shared__ v4f red[LPR ? 1 : kGemmWaves / 2][kWave];
+    __shared__ v4f red[LPR ? 1 : kGemmWaves][kWave];
     __shared__ float gv[4][16];   // LPR != 0: the [row][column] sums of the workgroup
     const int n0 = blockIdx.x * 16, m0 = blockIdx.y * 16;
     const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, lr = l & 15, lg = l >> 4;
@@ -325,11 +325,9 @@ __global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu
         request(1, base + 3 * kStride);
     }
     row_scale();
-    // K-split reduction: upper half of the waves parks its tile in LDS, lower half adds and parks the sums
-    if (w >= kGemmWaves / 2) red[w - kGemmWaves / 2][l] = acc;
+    // K-split reduction: every wave parks its tile in LDS; the thread that owns an element adds them in wave order
+    red[w][l] = acc;
     lds_barrier();   // LDS exchanges only: the epilogue's prefetched operands stay in flight
-    if (w < kGemmWaves / 2) red[w][l] += acc;
-    lds_barrier();
     }
     // element e of the 16x16 tile: row ml = e / 16, column nl = e % 16 lives in lane 16 (ml / 4) + nl, register ml % 4
     float u_out = 0.0f;   // mode 1: this thread's u as stored (0 for gate columns / rows past M)
@@ -341,7 +339,7 @@ __global__ __launch_bounds__(kGemmWaves * 64) __attribute__((amdgpu_waves_per_eu
             s = ml < MR ? gv[ml & 3][nl] : 0.0f;
         } else {
 #pragma unroll
-            for (int ww = 0; ww < kGemmWaves / 2; ww++) s += red[ww][lane][i];
+            for (int ww = 0; ww < kGemmWaves; ww++) s += red[ww][lane][i];
         }
         if constexpr (LPR != 0 && PRO == 1) inv = inv_rows[ml < MR ? ml : 0];
         s *= inv;
