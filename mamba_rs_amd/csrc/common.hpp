@@ -61,15 +61,15 @@ __device__ __forceinline__ float softplus20(float v) {
 // through global memory.
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
-// softplus for a result that is stored in 16 bits (8 or 11 significant bits): one branch of arithmetic instead of two.
-// log(1 + e) on the transcendental unit is off by at most 2^-24 / e relative, i.e. below 2^-12 for e >= 2^-12; under
-// that, log1p(e) = e (1 - e/2) to 2^-25.  Half the issue slots of softplus20.
+// softplus for a result that is stored in 16 bits (8 or 11 significant bits), as max(v, 0) + log(1 + e^-|v|): no overflow,
+// so no clamp, and above 20 the sum 1 + e^-|v| is 1 and the result is v itself, the reference's pass-through
+// (kernels/activations.cu:39).  log(1 + t) on the transcendental unit is off by at most 2^-24 / t relative to itself,
+// i.e. below 2^-12 of the result for t >= 2^-12; under that (v < -12 ln 2) the result is t to 2^-13.  Eight issue slots,
+// two of them transcendental (the clamped form with log1p's second term and two selects took twelve).
 __device__ __forceinline__ float softplus20_16(float v) {
-    const float e = fast_exp2(fminf(v, 20.0f) * kLog2e);
-    const float small = e * fmaf(e, -0.5f, 1.0f);
-    const float vialog = __builtin_amdgcn_logf(1.0f + e) * 0.6931471805599453f;
-    const float r = e < 0.000244140625f ? small : vialog;
-    return v > 20.0f ? v : r;
+    const float t = fast_exp2(-fabsf(v) * kLog2e);
+    const float r = fmaf(__builtin_amdgcn_logf(1.0f + t), 0.6931471805599453f, fmaxf(v, 0.0f));
+    return v < -8.317766f ? t : r;
 }
 
 // ---- host-side error plumbing ---------------------------------------------

@@ -436,96 +436,97 @@ __global__ __launch_bounds__(256) void prenorm_rows_kernel(float *__restrict__ p
 // Prefill dt_proj with its bias and softplus fused: delta[r, d] = softplus(round_T(sum_k dt_in[r, k] dt_w[k, d]) + bias[d]).
 // The reference runs a GEMM with K = dt_rank, then bias add and softplus_forward (src/mamba_ssm/gpu/prefill.rs:846-905,
 // kernels/activations.cu:32-52).  K is tiny (48 at d_model 768), so the op is one write of delta (50 MB per layer at the
-// 130m prefill shape) and nothing else: a workgroup forms a 64 x 64 tile with two v_mfma_f32_16x16x32 steps per 16 x 16 block
-// (K zero-padded to a multiple of 32), applies the epilogue on the accumulators, and transposes through LDS so that the
-// rows leave as 16-byte stores.  dt_in rows have stride xs (they are the head of the x_proj row); wt is [d_inner][dt_rank].
-// KS = 32-wide k-steps held in registers (dt_rank <= 32 KS).  A workgroup owns 64 columns and walks row tiles blockIdx.y,
-// blockIdx.y + gridDim.y, ...: the weight fragments and the bias are loaded once, the next tile's rows are requested
-// while the current tile is in its epilogue, and the transpose through LDS is private to each wave (no workgroup
-// barrier).  Measured at the 130m prefill shape (50 MB of delta per layer): 25.7 us with one tile per workgroup, 22.4 us
-// walking row tiles, 26.5 us walking along the rows instead, 21.2 us with the one-branch softplus20_16.
-// WLDS: the weight fragments live in LDS instead of registers.  From dt_rank 97 up (KS >= 4: the 2.8b shape has dt_rank
-// 160) 16 registers per k-step for them left two waves per SIMD (178 registers at KS = 6); read back from LDS as they are
-// used they cost a 16-byte LDS read per matrix instruction and the kernel keeps four waves per SIMD (2.8b shape, 168 MB of
-// delta: 102 -> 91 us).  What bounds it there is no longer this kernel's shape but its blocking: each of the 80 column
-// blocks re-reads the 6.3 MB of dt_in rows (0.5 GB through L2), which only square tiles of a real GEMM would cut.
-template <typename T, int KS, bool WLDS = (KS >= 4)>
+// 130m prefill shape) and the softplus arithmetic.  dt_in rows have stride xs (they are the head of the x_proj row); wt is
+// [d_inner][dt_rank].  KS = 32-wide k-steps (dt_rank <= 32 KS, K zero-padded), CT = 16-column tiles per workgroup.
+//
+// The product is formed TRANSPOSED: the weight is the matrix instruction's first operand and the 16 rows of a wave its
+// second, so a lane's four results of one instruction are four COLUMNS of one row.  Operand row m of column tile ct stands
+// for column 64 (ct / 4) + 16 (m / 4) + 4 (ct % 4) + m % 4 of the workgroup's block: after the four tiles of a 64-column
+// sub-block a lane holds 16 consecutive columns of its row, which leave as two 16-byte stores -- the four lane groups of a
+// row fill a 128-byte line, with no transpose through LDS (which the row-major product needed: 16 two-byte LDS writes per
+// lane and tile).  A workgroup owns 16 CT columns and walks row tiles blockIdx.y, blockIdx.y + gridDim.y, ...: weight
+// operands and bias are loaded once, the next tile's rows are requested while the current tile is in its epilogue.
+// WLDS: the weight operands live in LDS, in operand order (one conflict-free kilobyte per matrix instruction), instead of
+// registers: from dt_rank 97 up (KS >= 4: the 2.8b shape has dt_rank 160) 16 registers per k-step and sub-block for them
+// would leave two waves per SIMD.  There the workgroup owns 128 columns: every column block re-reads the dt_in rows
+// (6.3 MB at 4 x 4096 rows) through L2, 40 blocks instead of 80.
+// What the kernel costs is its arithmetic: per result ten plain and two transcendental instructions (rounding the
+// projection to the storage type and back, bias, softplus, packing).  Measured per layer, 130m prefill shape (50 MB of
+// delta) / 2.8b shape (168 MB): the row-major product with its LDS transpose and a twelve-slot softplus 21.4 / 94 us; this
+// kernel with the same softplus 21.1 / 93; with softplus20_16 as it is now 20.3 / 84.8; with the row tiles dealt evenly
+// among the workgroups (launch_dt_proj_softplus) 18.7 / 77.2.
+template <typename T, int KS, int CT, bool WLDS>
 __global__ __launch_bounds__(256) void dt_proj_softplus_kernel(T *__restrict__ delta, const T *__restrict__ dt_in, int64_t xs,
                                                                const T *__restrict__ wt, const float *__restrict__ bias, int64_t rows,
                                                                int di, int dr) {
-    __shared__ alignas(16) T tile[4][16][64 + 8];
-    __shared__ alignas(16) T wlds[WLDS ? 64 : 1][WLDS ? KS * 32 + 8 : 8];   // [column][k], k zero-padded to 32 KS
+    static_assert(CT % 4 == 0, "whole 64-column sub-blocks");
+    constexpr int SB = CT / 4;
+    __shared__ uint4 wl[WLDS ? CT * KS * 64 : 1];   // [column tile][k-step][lane]
     const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, lr = l & 15, lg = l >> 4;
-    const int n0 = blockIdx.x * 64;
+    const int n0 = blockIdx.x * (16 * CT);
     const int64_t n_tiles = (rows + 63) / 64;
-    // weight fragments and bias of this workgroup's 64 columns
-    uint4 bf[WLDS ? 1 : KS][4];
-    float bv[4];
-#pragma unroll
-    for (int nt = 0; nt < 4; nt++) {
-        const int col = min(n0 + 16 * nt + lr, di - 1);
-        bv[nt] = bias[col];
-        if constexpr (!WLDS) {
-#pragma unroll
-            for (int ks = 0; ks < KS; ks++) {
-                const int k = 32 * ks + 8 * lg;   // dt_rank % 8 == 0: a lane's 8 values are all inside or all outside
-                bf[ks][nt] = k < dr ? *reinterpret_cast<const uint4 *>(wt + (int64_t)col * dr + k) : make_uint4(0, 0, 0, 0);
-            }
-        }
-    }
-    if constexpr (WLDS) {
-        for (int i = tid; i < 64 * KS * 4; i += 256) {   // 16-byte pieces: column i / (4 KS), k = 8 (i % (4 KS))
-            const int c = i / (KS * 4), k = 8 * (i - c * (KS * 4));
-            const int col = min(n0 + c, di - 1);
-            *reinterpret_cast<uint4 *>(&wlds[c][k]) = k < dr ? *reinterpret_cast<const uint4 *>(wt + (int64_t)col * dr + k) : make_uint4(0, 0, 0, 0);
-        }
-        __syncthreads();
-    }
-    auto load_a = [&](int64_t rt, uint4 (&af)[KS]) {
-        const int64_t arow = min(rt * 64 + 16 * w + lr, rows - 1);
-#pragma unroll
-        for (int ks = 0; ks < KS; ks++) {
-            const int k = 32 * ks + 8 * lg;
-            af[ks] = k < dr ? *reinterpret_cast<const uint4 *>(dt_in + arow * xs + k) : make_uint4(0, 0, 0, 0);
-        }
+    // the weight piece that lane `lane` brings to the instruction of (column tile ct, k-step ks)
+    auto weight_piece = [&](int ct, int ks, int lane) {
+        const int m = lane & 15, k = 32 * ks + 8 * (lane >> 4);   // dt_rank % 8 == 0: a lane's 8 values are all inside or all outside
+        const int col = min(n0 + 64 * (ct >> 2) + 16 * (m >> 2) + 4 * (ct & 3) + (m & 3), di - 1);
+        return k < dr ? *reinterpret_cast<const uint4 *>(wt + (int64_t)col * dr + k) : make_uint4(0, 0, 0, 0);
     };
-    uint4 af[KS], an[KS];
-    int64_t rt = blockIdx.y;
-    if (rt < n_tiles) load_a(rt, af);
-    for (; rt < n_tiles; rt += gridDim.y) {
-        const int64_t nxt = rt + gridDim.y;
-        if (nxt < n_tiles) load_a(nxt, an);
-        v4f acc[4];
+    uint4 wf[WLDS ? 1 : KS][WLDS ? 1 : CT];
+    if constexpr (WLDS) {
+        for (int i = tid; i < CT * KS * 64; i += 256) wl[i] = weight_piece((i >> 6) / KS, (i >> 6) % KS, i & 63);
+        __syncthreads();
+    } else {
 #pragma unroll
-        for (int nt = 0; nt < 4; nt++) {
-            acc[nt] = (v4f){0.f, 0.f, 0.f, 0.f};
+        for (int ct = 0; ct < CT; ct++)
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++) wf[ks][ct] = weight_piece(ct, ks, l);
+    }
+    float bv[SB][16];   // bias of this lane's 16 consecutive columns per sub-block
+#pragma unroll
+    for (int sb = 0; sb < SB; sb++)
+#pragma unroll
+        for (int j = 0; j < 16; j++) bv[sb][j] = bias[min(n0 + 64 * sb + 16 * lg + j, di - 1)];
+    // Rows of tile rt.  Every load and every store is issued on every path -- past the last tile the last one again, past
+    // the last row the last row again (its lanes then hold, and store, the same values), past dt_rank the row's own next
+    // values (B and C of the x_proj row), which meet zero weights.  Behind conditions the compiler waited for the NEXT
+    // tile's rows in front of the current tile's matrix instructions, and for the stores of a tile before the next.
+    auto load_rows = [&](int64_t rt, uint4 (&rf)[KS]) {
+        const int64_t row = min(min(rt, n_tiles - 1) * 64 + 16 * w + lr, rows - 1);
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) rf[ks] = *reinterpret_cast<const uint4 *>(dt_in + row * xs + min(32 * ks + 8 * lg, (int)xs - 8));
+    };
+    uint4 rf[KS];
+    int64_t rt = blockIdx.y;
+    load_rows(rt, rf);
+    for (; rt < n_tiles; rt += gridDim.y) {
+        const int64_t row = min(rt * 64 + 16 * w + lr, rows - 1);
+        // (the weight operands are read from LDS where they are used: hoisted out of this loop they are 128 registers and more)
+        if constexpr (WLDS) asm volatile("" ::: "memory");
+        v4f acc[CT];
+#pragma unroll
+        for (int ct = 0; ct < CT; ct++) {
+            acc[ct] = (v4f){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int ks = 0; ks < KS; ks++) {
-                uint4 b;
-                if constexpr (WLDS) b = *reinterpret_cast<const uint4 *>(&wlds[16 * nt + lr][32 * ks + 8 * lg]);
-                else b = bf[ks][nt];
-                acc[nt] = Mma32<T>::mma(af[ks], b, acc[nt]);
+                uint4 wv;
+                if constexpr (WLDS) wv = wl[(ct * KS + ks) * 64 + l];
+                else wv = wf[ks][ct];
+                acc[ct] = Mma32<T>::mma(wv, rf[ks], acc[ct]);
             }
         }
+        load_rows(rt + gridDim.y, rf);   // the next tile's rows travel during this tile's epilogue
 #pragma unroll
-        for (int nt = 0; nt < 4; nt++) {
+        for (int sb = 0; sb < SB; sb++) {
+            alignas(16) T out[16];
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const T raw = (T)acc[nt][i];   // the projection as the reference stores it, before bias and softplus
-                Store<T>::st(&tile[w][4 * lg + i][16 * nt + lr], softplus20_16(Store<T>::ld(&raw) + bv[nt]));
+            for (int j = 0; j < 16; j++) {
+                const T raw = (T)acc[4 * sb + (j >> 2)][j & 3];   // the projection as the reference stores it, before bias and softplus
+                Store<T>::st(&out[j], softplus20_16(Store<T>::ld(&raw) + bv[sb][j]));
             }
+            T *dst = delta + row * di + n0 + 64 * sb + 16 * lg;
+            *reinterpret_cast<uint4 *>(dst) = *reinterpret_cast<const uint4 *>(&out[0]);
+            *reinterpret_cast<uint4 *>(dst + 8) = *reinterpret_cast<const uint4 *>(&out[8]);
         }
-        __builtin_amdgcn_wave_barrier();   // tile[w] belongs to this wave: its LDS accesses execute in program order
-        const int64_t m0 = rt * 64 + 16 * w;
-#pragma unroll
-        for (int j = 0; j < 2; j++) {
-            const int idx = l + 64 * j, r = idx >> 3, seg = idx & 7;
-            if (m0 + r < rows && n0 + seg * 8 < di)
-                *reinterpret_cast<uint4 *>(delta + (m0 + r) * di + n0 + seg * 8) = *reinterpret_cast<const uint4 *>(&tile[w][r][seg * 8]);
-        }
-        __builtin_amdgcn_wave_barrier();
-#pragma unroll
-        for (int ks = 0; ks < KS; ks++) af[ks] = an[ks];
     }
 }
 
@@ -632,22 +633,35 @@ int launch_prenorm_rows(hipStream_t st, int dtype, float *partials, int n_partia
 }
 
 bool dt_proj_softplus_ok(int dtype, int di, int dr, int64_t xs, const void *delta, const void *dt_in, const void *wt) {
-    return (dtype == MRS_BF16 || dtype == MRS_F16) && di % 8 == 0 && dr >= 8 && dr % 8 == 0 && dr <= 256 && xs % 8 == 0 && aligned(delta, 16) &&
-           aligned(dt_in, 16) && aligned(wt, 16);
+    return (dtype == MRS_BF16 || dtype == MRS_F16) && di % 64 == 0 && dr >= 8 && dr % 8 == 0 && dr <= 256 && xs % 8 == 0 && xs >= dr &&
+           aligned(delta, 16) && aligned(dt_in, 16) && aligned(wt, 16);
 }
 
 int launch_dt_proj_softplus(hipStream_t st, int dtype, void *delta, const void *dt_in, int64_t xs, const void *wt, const float *bias,
                             int64_t rows, int di, int dr) {
     if (!dt_proj_softplus_ok(dtype, di, dr, xs, delta, dt_in, wt))
-        return fail(MRS_E_SHAPE, "dt_proj+softplus: needs 16-bit storage, d_inner, dt_rank and the row stride multiples of 8, 16-byte aligned operands");
+        return fail(MRS_E_SHAPE, "dt_proj+softplus: needs 16-bit storage, d_inner a multiple of 64, dt_rank and the row stride multiples of 8, 16-byte aligned operands");
     if (rows < 1) return fail(MRS_E_SHAPE, "dt_proj+softplus: rows=%lld", (long long)rows);
-    // about eight workgroups per compute unit in flight, each walking several row tiles
-    const int64_t n_tiles = (rows + 63) / 64;
-    const int gx = (di + 63) / 64;
-    const int64_t gy = std::max<int64_t>(1, std::min<int64_t>(n_tiles, (2048 + gx - 1) / gx));
-    const dim3 grid((unsigned)gx, (unsigned)gy), block(256);
+    // About eight workgroups per compute unit, each walking several row tiles -- as many as its neighbours where the tile
+    // count allows: the launch takes as long as the workgroup with the most tiles (2.8b shape, 256 row tiles over 40 column
+    // blocks: 32 workgroups per block with 8 tiles each 78.5 us, 52 with 4 or 5 tiles 85.7 us).
     const int ks = (dr + 31) / 32;
-#define MRS_DTP(T_, KS_) hipLaunchKernelGGL((dt_proj_softplus_kernel<T_, KS_>), grid, block, 0, st, (T_ *)delta, (const T_ *)dt_in, xs, (const T_ *)wt, bias, rows, di, dr)
+    // columns per workgroup (every block is whole: the stores carry no column test): 64 with the weight in registers; with
+    // the weight in LDS 128 where d_inner allows
+    const bool wlds = ks >= 4;
+    const int ct = wlds && di % 128 == 0 ? 8 : 4;
+    const int64_t n_tiles = (rows + 63) / 64;
+    const int gx = (di + 16 * ct - 1) / (16 * ct);
+    int64_t gy = std::max<int64_t>(1, std::min<int64_t>(n_tiles, (2048 + gx - 1) / gx));
+    for (int64_t d = gy; 2 * d > gy; d--)
+        if (n_tiles % d == 0) { gy = d; break; }
+    const dim3 grid((unsigned)gx, (unsigned)gy), block(256);
+#define MRS_DTP_CT(T_, KS_, CT_) hipLaunchKernelGGL((dt_proj_softplus_kernel<T_, KS_, CT_, (KS_ >= 4)>), grid, block, 0, st, (T_ *)delta, (const T_ *)dt_in, xs, (const T_ *)wt, bias, rows, di, dr)
+#define MRS_DTP(T_, KS_)                                                    \
+    do {                                                                    \
+        if constexpr (KS_ >= 4) { if (ct == 8) MRS_DTP_CT(T_, KS_, 8); else MRS_DTP_CT(T_, KS_, 4); } \
+        else MRS_DTP_CT(T_, KS_, 4);                                        \
+    } while (0)
 #define MRS_DTP_KS(T_)                                      \
     switch (ks) {                                           \
         case 1: MRS_DTP(T_, 1); break;                      \
@@ -660,6 +674,7 @@ int launch_dt_proj_softplus(hipStream_t st, int dtype, void *delta, const void *
     if (dtype == MRS_BF16) { MRS_DTP_KS(bf16_t) } else { MRS_DTP_KS(f16_t) }
 #undef MRS_DTP_KS
 #undef MRS_DTP
+#undef MRS_DTP_CT
     return check_launch("dt_proj_softplus_kernel");
 }
 
