@@ -223,6 +223,38 @@ def test_28b_shape_prefill_follows_the_cpu_route(w28, T):
     eng.close()
 
 
+@pytest.mark.parametrize("d_model", [128, 1536, 2048, 4096])
+def test_prefill_delta_kernel_at_every_dt_rank_width(d_model):
+    """One layer, 2 x 80 steps (two and a half 64-row tiles: the last tile's spare lanes repeat the last row) at widths
+    whose dt_rank is 8, 96, 128 and 256: the fused dt_proj + bias + softplus kernel of the 16-bit prefill with one, three,
+    four and eight k-steps -- the weight in registers (64 columns per workgroup) and in LDS (128) -- against the CPU
+    prefill: last output and final state.  (No hand-off step here: with a third of the channels at delta ~ 1e-5 and a
+    seventh at delta ~ 25 the few large channels carry the output, and the decode chain's own rounding points -- f32
+    x_proj shares where the prefill stores a 16-bit row -- show at 0.99 instead of 0.999; the hand-off is held to the
+    CPU route at every width by the tests above, on weights as they come.)"""
+    cfg = MambaConfig(d_model=d_model, d_state=16, d_conv=4, expand=2, n_layers=1)
+    assert cfg.dt_rank() == {128: 8, 1536: 96, 2048: 128, 4096: 256}[d_model]
+    w = MambaWeights.random_lm(cfg, seed=d_model, std=0.02)
+    for lw in w.layers:      # a bias that reaches both sides of the softplus's small-argument branch and its pass-through
+        lw.dt_proj_b[::3] -= 12.0
+        lw.dt_proj_b[1::7] += 25.0
+    P = lm_oracle(cfg, w)
+    B, T = 2, 80
+    print(f"case prefill delta kernel d_model={d_model}", flush=True)
+    eng = GpuMambaBackbone.new_with_dtype(0, w, cfg, d_model, B, WeightDtype.BF16)
+    rng = np.random.default_rng(d_model)
+    x = orc.round_to(rng.standard_normal((B, T, d_model)).astype(np.float32), orc.BF16)
+    last = eng.prefill_sequence(x)
+    state = eng.download_state(0)[1]
+    for b in range(B):
+        conv, ssm = orc.m1_zero_state(P)
+        ref = orc.m1_backbone_prefill(P, x[b], conv, ssm, identity_proj=True)
+        assert cosine(last[b], ref[-1]) >= COS, (b, cosine(last[b], ref[-1]))
+        r = ssm[0].reshape(2 * d_model, 16)
+        assert cosine(state[b], r) >= COS and scaled_err(state[b], r) < 5e-2, (b, cosine(state[b], r), scaled_err(state[b], r))
+    eng.close()
+
+
 # ---- Mamba-3 backbone at 24 heads -----------------------------------------------------------------------------------
 
 CFG_M3 = Mamba3Config(d_model=768, d_state=64, expand=2, headdim=64, ngroups=1, n_layers=2, rope_fraction=0.5)
